@@ -1,0 +1,145 @@
+"""Benchmark of the compressed multiply hot path on one MI355X.
+
+A step = one pass of compressed X %*% v over BASELINE config 2 (10,000,000 x 100,
+single-column DDC groups, 256 values per column, Zipf(1.1) uint8 codes), with the
+compressed block, v and the output resident in HBM. Prints ONE JSON line.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--scale S] [--no-cpu] [--extra]
+"""
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--scale", type=int, default=1, help="divide the number of rows (testing only)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--extra", action="store_true", help="also time X %*% B (100x64) of the same config")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU (the path shards by rows, see DESIGN.md); "
+              f"--gpus {args.gpus} is not supported", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from systemds_amd import capi, synth
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    torch.cuda.set_device(0)
+    capi.init(0)
+
+    t0 = time.time()
+    cfg = synth.config2(scale=args.scale)
+    n_rows, n_cols = cfg["n_rows"], cfg["n_cols"]
+    t_gen = time.time() - t0
+    t0 = time.time()
+    blk = capi.build_block(n_rows, n_cols, cfg["groups"])
+    t_upload = time.time() - t0
+
+    stream = torch.cuda.Stream()
+    blk.set_stream(stream.cuda_stream)
+    dv = torch.from_numpy(cfg["v"].copy()).cuda()
+    dout = torch.empty(n_rows, dtype=torch.float64, device="cuda")
+    torch.cuda.synchronize()
+
+    def step():
+        return blk.rmm_dev(dv.data_ptr(), 1, dout.data_ptr())
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    # whole-job throughput: wall clock over exactly K steps (each step returns nnz,
+    # i.e. includes its own stream synchronisation)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        nnz = step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+
+    # dominant kernel: HIP events on the stream the kernel is launched on
+    blk.profile(True)
+    kms, kbytes, kname = [], 0.0, ""
+    for _ in range(min(args.steps, 20)):
+        step()
+        ks = blk.stats()["kernels"]
+        dom = max(ks, key=lambda k: k["ms"])
+        kms.append(dom["ms"])
+        kbytes, kname = dom["algo_bytes"], dom["name"]
+    blk.profile(False)
+    k_ms = statistics.mean(kms)
+    achieved = kbytes / (k_ms * 1e-3) / 1e9
+
+    result = {
+        "metric": "compressed X%*%v on DDC 10Mx100: rows/s and achieved HBM GB/s vs peak",
+        "value": n_rows / (ms_per_step * 1e-3),
+        "unit": "rows/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f64", "data": "synthetic",
+        "config": {"workload": f"C2 X%*%v: {n_rows}x{n_cols} fp64 as {n_cols} single-column DDC groups, 256 values, "
+                               "Zipf(1.1) uint8 codes, v 100x1; block, v and output resident in HBM",
+                   "nnz": int(nnz), "gen_s": round(t_gen, 2), "upload_s": round(t_upload, 2),
+                   "block_bytes": int(blk.device_bytes())},
+        "roofline": {"bound": "hbm", "kernel": kname, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "kernel_ms": k_ms, "algo_bytes_per_launch": kbytes,
+                     "traffic": None},
+    }
+
+    if args.extra:
+        dB = torch.from_numpy(cfg["B"].copy()).cuda()
+        doutB = torch.empty((n_rows, 64), dtype=torch.float64, device="cuda")
+        for _ in range(2):
+            blk.rmm_dev(dB.data_ptr(), 64, doutB.data_ptr())
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        reps = max(args.steps // 5, 3)
+        for _ in range(reps):
+            blk.rmm_dev(dB.data_ptr(), 64, doutB.data_ptr())
+        torch.cuda.synchronize()
+        msB = (time.perf_counter() - t0) / reps * 1e3
+        bytesB = n_rows * (n_cols + 64 * 8.0)
+        result["extra"] = {"C2 X%*%B(100x64)": {"ms": msB, "rows_per_s": n_rows / (msB * 1e-3),
+                                                "algo_GBs": bytesB / (msB * 1e-3) / 1e9,
+                                                "frac_hbm": bytesB / (msB * 1e-3) / 1e9 / HBM_PEAK_GBS}}
+        del doutB
+
+    if not args.no_cpu:
+        # CPU baseline: the oracle's multithreaded restatement of the reference algorithm
+        # (a port, not the SystemDS JVM) on the same full workload, host cores of this box.
+        from oracle import cla_oracle as ora
+        cores = min(len(os.sched_getaffinity(0)), int(os.environ.get("OMP_NUM_THREADS", "64")))
+        G = ora.Groups(cfg["groups"], n_rows, n_cols)
+        times = []
+        for _ in range(3):
+            t0 = time.perf_counter()
+            ref, rnnz = ora.rmm(G, cfg["v"], cores)
+            times.append(time.perf_counter() - t0)
+        cpu_s = statistics.median(times)
+        got = dout.cpu().numpy()
+        result["cpu_baseline"] = {"value": n_rows / cpu_s, "unit": "rows/s", "cores": cores, "kind": "port",
+                                  "sample": f"the full workload ({n_rows} rows x {n_cols} groups), median of 3 passes, "
+                                            f"{cpu_s:.3f} s per pass",
+                                  "parity_bit_exact": bool(np.array_equal(got, ref[:, 0]) and rnnz == nnz)}
+
+    blk.close()
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

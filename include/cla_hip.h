@@ -1,0 +1,166 @@
+/*
+ * cla_hip.h — C ABI of libclahip.so: the compressed linear algebra (CLA)
+ * multiply path of Apache SystemDS on one AMD MI355X (gfx950), hand-written HIP.
+ *
+ * This is the boundary a SystemDS maintainer binds with JNI or Panama FFM from
+ * org.apache.sysds.runtime.compress. It follows the conventions of the
+ * reference's existing native bridge (utils/NativeHelper.java:361-418,
+ * src/main/cpp/systemds.cpp:64-84): primitive arrays in, the number of
+ * non-zeros (a long) out, a negative value on failure so that the caller falls
+ * back to its Java kernel (R/matrix/data/LibMatrixNative.java:123-135).
+ *
+ * Granularity: one call per CLALib* driver on a whole CompressedMatrixBlock,
+ * so code streams, offset lists, run lists and dictionaries stay resident in
+ * HBM between calls. The per-group virtual methods of AColGroup
+ * (CG/AColGroup.java:353-462) are served by cla_counts / cla_cooc /
+ * cla_preagg / cla_decompress.
+ *
+ * Reference paths: C/ = src/main/java/org/apache/sysds/runtime/compress/,
+ * CG/ = C/colgroup/.
+ *
+ * Conventions
+ *  - All matrices are dense row-major fp64 (Java DenseBlockFP64).
+ *  - Host pointers are borrowed only for the duration of the call.
+ *  - `_dev` variants take device pointers (HBM) and run asynchronously on the
+ *    block's stream up to the final non-zero count read-back.
+ *  - No exceptions cross the boundary; errors are negative return codes and
+ *    cla_last_error() (thread local) explains them.
+ *  - Calls on different blocks are thread safe; calls on one block are
+ *    serialised internally (one HIP stream per block).
+ */
+#ifndef CLA_HIP_H
+#define CLA_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct cla_block* cla_handle;
+
+/* error codes (returned negated) */
+enum {
+	CLA_OK = 0,
+	CLA_ERR_INVALID = 1,     /* bad argument / shape (Java: DMLCompressionException) */
+	CLA_ERR_UNSUPPORTED = 2, /* encoding or combination not handled (Java: NotImplementedException) */
+	CLA_ERR_DEVICE = 3,      /* HIP runtime error, no device, out of memory */
+	CLA_ERR_STATE = 4        /* block not finalized / already finalized */
+};
+
+/* Library bring-up: replaces NativeHelper's load/initialise step
+ * (utils/NativeHelper.java:109-360). Selects the HIP device; fails (negative)
+ * when no gfx950 device is visible — the product never computes on the CPU. */
+int cla_init(int device);
+/* Human readable reason of the last failure on this thread. */
+const char* cla_last_error(void);
+/* Device/library facts as a JSON object (name, CUs, LDS bytes, HBM bytes). */
+int cla_device_info(char* json, size_t cap);
+
+/* ---- CompressedMatrixBlock construction (C/CompressedMatrixBlock.java:119-132) ---- */
+cla_handle cla_block_create(int64_t nRows, int32_t nCols);
+void cla_block_free(cla_handle h);
+
+/* ColGroupDDC (CG/ColGroupDDC.java:79-113): X[r, cols] = dict[codes[r]].
+ * codeWidth 1 = MapToByte/MapToUByte (unsigned, `& 0xFF`), 2 = MapToChar,
+ * 4 = MapToInt (CG/mapping/MapToFactory.java:102-117). codes has nRows entries. */
+int cla_block_add_ddc(cla_handle h, const int32_t* cols, int32_t nColG, const double* dict, int32_t nVals,
+	const void* codes, int32_t codeWidth);
+
+/* ColGroupSDC / ColGroupSDCZeros (CG/ColGroupSDC.java:68-117,
+ * CG/ColGroupSDCZeros.java:76-104) with the raw AOffset arrays
+ * (CG/offset/OffsetByte.java, OffsetChar.java): `deltas` holds nDeltas entries
+ * of deltaWidth bytes (1 or 2), a 0 entry means "+255 (or +65535) and no row".
+ * The list has nOffsets rows from offsetToFirst to offsetToLast; codes has
+ * nOffsets entries. defaultTuple NULL => SDCZeros. nOffsets may be 1 or 2 with
+ * nDeltas 0 / 1 (OffsetSingle / OffsetTwo). */
+int cla_block_add_sdc(cla_handle h, const int32_t* cols, int32_t nColG, const double* dict, int32_t nVals,
+	const double* defaultTuple, const void* codes, int32_t codeWidth, const void* deltas, int32_t deltaWidth,
+	int64_t nDeltas, int32_t offsetToFirst, int32_t offsetToLast, int64_t nOffsets);
+
+/* ColGroupRLE (CG/ColGroupRLE.java:53-91, CG/AColGroupOffset.java:36-55):
+ * ptr[nVals+1] positions into data[]; data = (gap, runLength) char pairs. */
+int cla_block_add_rle(cla_handle h, const int32_t* cols, int32_t nColG, const double* dict, int32_t nVals,
+	const int32_t* ptr, const uint16_t* data, int64_t nData);
+
+/* ColGroupUncompressed (dense MatrixBlock nRows x nColG, row-major). */
+int cla_block_add_uncompressed(cla_handle h, const int32_t* cols, int32_t nColG, const double* values);
+/* ColGroupConst (CG/ColGroupConst.java): every row equals `row`. */
+int cla_block_add_const(cla_handle h, const int32_t* cols, int32_t nColG, const double* row);
+/* ColGroupEmpty. */
+int cla_block_add_empty(cla_handle h, const int32_t* cols, int32_t nColG);
+
+/* Ends construction: validates codes < nVals, builds the device-side
+ * acceleration structures (offset checkpoints and row-tile index — the
+ * device twin of AOffset's skip list, CG/offset/AOffset.java:177-199 — and the
+ * merged run table for RLE) and the pre-filter of CLALibUtils.filterGroups
+ * (C/lib/CLALibUtils.java:188-206: SDC default -> constV, dict - default). */
+int cla_block_finalize(cla_handle h);
+
+/* Use an existing HIP stream (hipStream_t) for all work of this block. */
+int cla_block_set_stream(cla_handle h, void* hipStream);
+int32_t cla_block_num_groups(cla_handle h);
+/* Bytes of HBM held by the block's compressed representation. */
+int64_t cla_block_device_bytes(cla_handle h);
+
+/* ---- multiply drivers ---- */
+
+/* CLALibRightMultBy.rightMultByMatrix with allowOverlap=false (RMM,
+ * C/lib/CLALibRightMultBy.java:51-102, 208-258): out[nRows x nColB] = X %*% B,
+ * B is nCols x nColB. Returns nnz(out) or a negative error. */
+int64_t cla_rmm(cla_handle h, const double* B, int32_t nColB, double* out);
+int64_t cla_rmm_dev(cla_handle h, const double* dB, int32_t nColB, double* dOut);
+
+/* CLALibLeftMultBy.leftMultByMatrix (C/lib/CLALibLeftMultBy.java:126-145,
+ * 286-346): out[nRowY x nCols] = Y %*% X, Y is nRowY x nRows. */
+int64_t cla_lmm(cla_handle h, const double* Y, int32_t nRowY, double* out);
+int64_t cla_lmm_dev(cla_handle h, const double* dY, int32_t nRowY, double* dOut);
+
+/* CLALibTSMM.leftMultByTransposeSelf (C/lib/CLALibTSMM.java:59-94):
+ * out[nCols x nCols] = t(X) %*% X, full symmetric. */
+int64_t cla_tsmm(cla_handle h, double* out);
+int64_t cla_tsmm_dev(cla_handle h, double* dOut);
+
+/* CLALibMMChain.mmChain (C/lib/CLALibMMChain.java:92-148):
+ * out[nCols] = t(X) %*% (w * (X %*% v)); ctype 0 = XtXv (w ignored), 1 = XtwXv. */
+int64_t cla_mmchain(cla_handle h, const double* v, const double* w, int32_t ctype, double* out);
+int64_t cla_mmchain_dev(cla_handle h, const double* dV, const double* dW, int32_t ctype, double* dOut);
+
+/* CLALibDecompress.decompressDense (C/lib/CLALibDecompress.java:310-357):
+ * out[nRows x nCols] = X. */
+int64_t cla_decompress(cla_handle h, double* out);
+int64_t cla_decompress_dev(cla_handle h, double* dOut);
+
+/* ---- per-group pieces (AColGroup surface) ---- */
+
+/* AMapToData.getCounts / ColGroupRLE.getCounts (CG/mapping/AMapToData.java:408-419,
+ * CG/mapping/MapToByte.java:168-187, CG/ColGroupRLE.java:259-265): exact integer
+ * histogram of group `group`'s code stream, nVals entries. */
+int cla_counts(cla_handle h, int32_t group, int32_t* counts);
+
+/* Integer co-occurrence between two groups of the block:
+ * out[a * nVals_B + b] = #{rows r : code_A(r) = a and code_B(r) = b}, rows not
+ * covered by an SDCZeros/RLE group are skipped. This is the exact-integer form
+ * of APreAgg.preAggregateThatIndexStructure (CG/APreAgg.java:87-110,
+ * CG/mapping/AMapToData.java:429-794). */
+int cla_cooc(cla_handle h, int32_t groupA, int32_t groupB, int64_t* out);
+
+/* APreAgg.preAggregateDense (CG/APreAgg.java:137-151; DDC
+ * CG/mapping/AMapToData.java:214-330, SDCZ CG/offset/AOffset.java:288-430, RLE
+ * CG/ColGroupRLE.java:759-796): preAgg[nRowY x nVals] with
+ * preAgg[i, code(r)] += Y[i, r]. */
+int cla_preagg(cla_handle h, int32_t group, const double* Y, int32_t nRowY, double* preAgg);
+
+/* ---- introspection (the twin of the reference's -stats timers,
+ * utils/DMLCompressionStatistics.java:44-125) ---- */
+/* enable != 0: bracket every kernel of this block with HIP events on its stream. */
+int cla_block_profile(cla_handle h, int enable);
+/* JSON with the kernels launched by the last driver call on this block: launch
+ * geometry, algorithmic bytes and (when profiling) milliseconds. */
+int cla_stats(cla_handle h, char* json, size_t cap);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,297 @@
+"""ctypes binding of libclahip.so — the same entry points a JNI/Panama caller binds.
+
+The library is the only compute path: if it is missing or no gfx950 device is
+visible this module raises, it never computes on the CPU.
+"""
+import ctypes as C
+import json
+import os
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libclahip.so")
+
+_i32p = C.POINTER(C.c_int32)
+_f64p = C.POINTER(C.c_double)
+
+
+class ClaError(RuntimeError):
+    """Negative return code of the C ABI (message from cla_last_error)."""
+
+    def __init__(self, code, msg):
+        super().__init__(f"cla error {code}: {msg}")
+        self.code = code
+
+
+# name -> (restype, argtypes); mirrors include/cla_hip.h one to one
+SIGNATURES = {
+    "cla_init": (C.c_int, [C.c_int]),
+    "cla_last_error": (C.c_char_p, []),
+    "cla_device_info": (C.c_int, [C.c_char_p, C.c_size_t]),
+    "cla_block_create": (C.c_void_p, [C.c_int64, C.c_int32]),
+    "cla_block_free": (None, [C.c_void_p]),
+    "cla_block_add_ddc": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p, C.c_int32, C.c_void_p, C.c_int32]),
+    "cla_block_add_sdc": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p,
+                                    C.c_int32, C.c_void_p, C.c_int32, C.c_int64, C.c_int32, C.c_int32, C.c_int64]),
+    "cla_block_add_rle": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p,
+                                    C.c_int64]),
+    "cla_block_add_uncompressed": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
+    "cla_block_add_const": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
+    "cla_block_add_empty": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32]),
+    "cla_block_finalize": (C.c_int, [C.c_void_p]),
+    "cla_block_set_stream": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "cla_block_num_groups": (C.c_int32, [C.c_void_p]),
+    "cla_block_device_bytes": (C.c_int64, [C.c_void_p]),
+    "cla_rmm": (C.c_int64, [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
+    "cla_rmm_dev": (C.c_int64, [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
+    "cla_lmm": (C.c_int64, [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
+    "cla_lmm_dev": (C.c_int64, [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
+    "cla_tsmm": (C.c_int64, [C.c_void_p, C.c_void_p]),
+    "cla_tsmm_dev": (C.c_int64, [C.c_void_p, C.c_void_p]),
+    "cla_mmchain": (C.c_int64, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
+    "cla_mmchain_dev": (C.c_int64, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
+    "cla_decompress": (C.c_int64, [C.c_void_p, C.c_void_p]),
+    "cla_decompress_dev": (C.c_int64, [C.c_void_p, C.c_void_p]),
+    "cla_counts": (C.c_int, [C.c_void_p, C.c_int32, C.c_void_p]),
+    "cla_cooc": (C.c_int, [C.c_void_p, C.c_int32, C.c_int32, C.c_void_p]),
+    "cla_preagg": (C.c_int, [C.c_void_p, C.c_int32, C.c_void_p, C.c_int32, C.c_void_p]),
+    "cla_block_profile": (C.c_int, [C.c_void_p, C.c_int]),
+    "cla_stats": (C.c_int, [C.c_void_p, C.c_char_p, C.c_size_t]),
+}
+
+_lib = None
+_initialised = False
+
+
+def load_library():
+    """dlopen the in-tree library and declare the prototypes. Raises if it is not built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ClaError(-3, f"{LIB_PATH} is not built; run `python -c 'import __graft_entry__ as g; g.build()'`")
+    lib = C.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def last_error():
+    return (load_library().cla_last_error() or b"").decode()
+
+
+def _check(rc):
+    if rc is None or rc < 0:
+        raise ClaError(rc, last_error())
+    return rc
+
+
+def init(device=0):
+    global _initialised
+    _check(load_library().cla_init(device))
+    _initialised = True
+
+
+def device_info():
+    buf = C.create_string_buffer(1024)
+    _check(load_library().cla_device_info(buf, len(buf)))
+    return json.loads(buf.value.decode())
+
+
+def _ptr(a):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+def _arr(a, dtype):
+    if a is None:
+        return None
+    return np.ascontiguousarray(a, dtype=dtype)
+
+
+def _code_arr(codes):
+    a = np.ascontiguousarray(codes)
+    if a.dtype == np.uint8 or a.dtype == np.int8:
+        return a.view(np.uint8), 1
+    if a.dtype == np.uint16:
+        return a, 2
+    if a.dtype == np.int32 or a.dtype == np.uint32:
+        return a.view(np.int32), 4
+    raise ClaError(-2, f"unsupported code dtype {a.dtype}")
+
+
+class ClaBlock:
+    """A device-resident CompressedMatrixBlock (thin handle wrapper)."""
+
+    def __init__(self, n_rows, n_cols):
+        if not _initialised:
+            init(0)
+        self.lib = load_library()
+        self.n_rows, self.n_cols = int(n_rows), int(n_cols)
+        self.h = self.lib.cla_block_create(self.n_rows, self.n_cols)
+        if not self.h:
+            raise ClaError(-1, last_error())
+        self.n_vals = []
+
+    def close(self):
+        if self.h:
+            self.lib.cla_block_free(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    # ---- construction ----
+    def add_ddc(self, cols, dict_, codes):
+        cols = _arr(cols, np.int32)
+        d = _arr(dict_, np.float64).reshape(-1, len(cols))
+        c, w = _code_arr(codes)
+        _check(self.lib.cla_block_add_ddc(self.h, _ptr(cols), len(cols), _ptr(d), d.shape[0], _ptr(c), w))
+        self.n_vals.append(d.shape[0])
+
+    def add_sdc(self, cols, dict_, default, codes, deltas, first, last, n_offsets):
+        cols = _arr(cols, np.int32)
+        d = _arr(dict_, np.float64).reshape(-1, len(cols))
+        de = _arr(default, np.float64)
+        c, w = _code_arr(codes) if codes is not None else (None, 1)
+        dl = np.ascontiguousarray(deltas) if deltas is not None else np.zeros(0, np.uint8)
+        dw = 2 if dl.dtype == np.uint16 else 1
+        _check(self.lib.cla_block_add_sdc(self.h, _ptr(cols), len(cols), _ptr(d), d.shape[0], _ptr(de), _ptr(c), w,
+                                          _ptr(dl), dw, dl.size, int(first), int(last), int(n_offsets)))
+        self.n_vals.append(d.shape[0])
+
+    def add_rle(self, cols, dict_, ptr, data):
+        cols = _arr(cols, np.int32)
+        d = _arr(dict_, np.float64).reshape(-1, len(cols))
+        p = _arr(ptr, np.int32)
+        r = _arr(data, np.uint16)
+        _check(self.lib.cla_block_add_rle(self.h, _ptr(cols), len(cols), _ptr(d), d.shape[0], _ptr(p), _ptr(r), r.size))
+        self.n_vals.append(d.shape[0])
+
+    def add_uncompressed(self, cols, values):
+        cols = _arr(cols, np.int32)
+        v = _arr(values, np.float64)
+        _check(self.lib.cla_block_add_uncompressed(self.h, _ptr(cols), len(cols), _ptr(v)))
+        self.n_vals.append(0)
+
+    def add_const(self, cols, row):
+        cols = _arr(cols, np.int32)
+        _check(self.lib.cla_block_add_const(self.h, _ptr(cols), len(cols), _ptr(_arr(row, np.float64))))
+
+    def add_empty(self, cols):
+        cols = _arr(cols, np.int32)
+        _check(self.lib.cla_block_add_empty(self.h, _ptr(cols), len(cols)))
+
+    def add(self, spec):
+        """Adds a group described by a systemds_amd.synth.GroupSpec."""
+        t = spec.type
+        if t == "ddc":
+            self.add_ddc(spec.cols, spec.dict, spec.codes)
+        elif t == "sdc":
+            self.add_sdc(spec.cols, spec.dict, spec.default, spec.codes, spec.deltas, spec.first, spec.last,
+                         spec.n_offsets)
+        elif t == "rle":
+            self.add_rle(spec.cols, spec.dict, spec.ptr, spec.rle)
+        elif t == "unc":
+            self.add_uncompressed(spec.cols, spec.dense)
+        elif t == "const":
+            self.add_const(spec.cols, spec.dict)
+        elif t == "empty":
+            self.add_empty(spec.cols)
+        else:
+            raise ClaError(-2, f"unknown group type {t}")
+
+    def finalize(self):
+        _check(self.lib.cla_block_finalize(self.h))
+        return self
+
+    def set_stream(self, stream_ptr):
+        _check(self.lib.cla_block_set_stream(self.h, C.c_void_p(stream_ptr)))
+
+    def device_bytes(self):
+        return _check(self.lib.cla_block_device_bytes(self.h))
+
+    # ---- host-pointer drivers (what a JNI caller uses) ----
+    def rmm(self, B):
+        B = _arr(B, np.float64).reshape(self.n_cols, -1)
+        out = np.empty((self.n_rows, B.shape[1]), np.float64)
+        nnz = _check(self.lib.cla_rmm(self.h, _ptr(B), B.shape[1], _ptr(out)))
+        return out, nnz
+
+    def lmm(self, Y):
+        Y = _arr(Y, np.float64).reshape(-1, self.n_rows)
+        out = np.empty((Y.shape[0], self.n_cols), np.float64)
+        nnz = _check(self.lib.cla_lmm(self.h, _ptr(Y), Y.shape[0], _ptr(out)))
+        return out, nnz
+
+    def tsmm(self):
+        out = np.empty((self.n_cols, self.n_cols), np.float64)
+        nnz = _check(self.lib.cla_tsmm(self.h, _ptr(out)))
+        return out, nnz
+
+    def mmchain(self, v, w=None, ctype=0):
+        v = _arr(v, np.float64).reshape(-1)
+        w = None if w is None else _arr(w, np.float64).reshape(-1)
+        out = np.empty((self.n_cols,), np.float64)
+        nnz = _check(self.lib.cla_mmchain(self.h, _ptr(v), _ptr(w), int(ctype), _ptr(out)))
+        return out, nnz
+
+    def decompress(self):
+        out = np.empty((self.n_rows, self.n_cols), np.float64)
+        nnz = _check(self.lib.cla_decompress(self.h, _ptr(out)))
+        return out, nnz
+
+    def counts(self, group):
+        out = np.zeros(self.n_vals[group], np.int32)
+        _check(self.lib.cla_counts(self.h, int(group), _ptr(out)))
+        return out
+
+    def cooc(self, ga, gb):
+        out = np.zeros((self.n_vals[ga], self.n_vals[gb]), np.int64)
+        _check(self.lib.cla_cooc(self.h, int(ga), int(gb), _ptr(out)))
+        return out
+
+    def preagg(self, group, Y):
+        Y = _arr(Y, np.float64).reshape(-1, self.n_rows)
+        out = np.zeros((Y.shape[0], self.n_vals[group]), np.float64)
+        _check(self.lib.cla_preagg(self.h, int(group), _ptr(Y), Y.shape[0], _ptr(out)))
+        return out
+
+    # ---- device-pointer drivers (inputs/outputs already in HBM) ----
+    def rmm_dev(self, dB_ptr, n_col_b, dOut_ptr):
+        return _check(self.lib.cla_rmm_dev(self.h, C.c_void_p(dB_ptr), int(n_col_b), C.c_void_p(dOut_ptr)))
+
+    def lmm_dev(self, dY_ptr, n_row_y, dOut_ptr):
+        return _check(self.lib.cla_lmm_dev(self.h, C.c_void_p(dY_ptr), int(n_row_y), C.c_void_p(dOut_ptr)))
+
+    def tsmm_dev(self, dOut_ptr):
+        return _check(self.lib.cla_tsmm_dev(self.h, C.c_void_p(dOut_ptr)))
+
+    def mmchain_dev(self, dV_ptr, dW_ptr, ctype, dOut_ptr):
+        return _check(self.lib.cla_mmchain_dev(self.h, C.c_void_p(dV_ptr), C.c_void_p(dW_ptr or 0), int(ctype),
+                                               C.c_void_p(dOut_ptr)))
+
+    def decompress_dev(self, dOut_ptr):
+        return _check(self.lib.cla_decompress_dev(self.h, C.c_void_p(dOut_ptr)))
+
+    def profile(self, enable=True):
+        _check(self.lib.cla_block_profile(self.h, 1 if enable else 0))
+
+    def stats(self):
+        buf = C.create_string_buffer(1 << 16)
+        _check(self.lib.cla_stats(self.h, buf, len(buf)))
+        return json.loads(buf.value.decode())
+
+
+def build_block(n_rows, n_cols, specs):
+    """Uploads a list of group specs into a finalized device block."""
+    b = ClaBlock(n_rows, n_cols)
+    for s in specs:
+        b.add(s)
+    return b.finalize()

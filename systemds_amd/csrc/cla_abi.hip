@@ -1,0 +1,674 @@
+// C ABI of libclahip.so (see include/cla_hip.h): block construction, finalize,
+// host/device entry points of the multiply drivers. Host-side logic only; the
+// kernels live in k_*.hip.
+#include "../../include/cla_hip.h"
+#include "cla_internal.hpp"
+#include <algorithm>
+#include <cstdarg>
+#include <cstring>
+#include <map>
+
+namespace cla {
+
+static thread_local char t_err[1024] = "";
+int g_ldsPerBlock = 65536;
+int g_numCU = 256;
+static int g_device = -1;
+static hipDeviceProp_t g_prop;
+static std::mutex g_initMu;
+
+void set_error(const char* fmt, ...) {
+	va_list ap;
+	va_start(ap, fmt);
+	vsnprintf(t_err, sizeof(t_err), fmt, ap);
+	va_end(ap);
+}
+
+Prof::Prof(cla_block* blk, const char* name, long grid, long block, long lds, double algoBytes) : b(blk) {
+	KernelStat k;
+	k.name = name; k.grid = grid; k.block = block; k.lds = lds; k.algoBytes = algoBytes;
+	if(b->profile && hipEventCreate(&k.e0) == hipSuccess && hipEventCreate(&k.e1) == hipSuccess)
+		(void) hipEventRecord(k.e0, b->stream);
+	idx = b->lastStats.size();
+	b->lastStats.push_back(k);
+}
+
+Prof::~Prof() {
+	KernelStat& k = b->lastStats[idx];
+	if(k.e0 && k.e1) (void) hipEventRecord(k.e1, b->stream);
+}
+
+void clear_stats(cla_block* b) {
+	for(auto& k : b->lastStats) {
+		if(k.e0) (void) hipEventDestroy(k.e0);
+		if(k.e1) (void) hipEventDestroy(k.e1);
+	}
+	b->lastStats.clear();
+}
+
+int ensure_tables(cla_block* b, size_t nDoubles) {
+	if(nDoubles <= b->tablesCap) return 0;
+	if(b->dTables) CLA_HIP(hipFree(b->dTables));
+	b->dTables = nullptr; b->tablesCap = 0;
+	CLA_HIP(hipMalloc((void**) &b->dTables, nDoubles * sizeof(double)));
+	b->tablesCap = nDoubles;
+	return 0;
+}
+
+int ensure_scratch(cla_block* b, size_t bytes) {
+	if(bytes <= b->scratchCap) return 0;
+	if(b->dScratch) CLA_HIP(hipFree(b->dScratch));
+	b->dScratch = nullptr; b->scratchCap = 0;
+	CLA_HIP(hipMalloc(&b->dScratch, bytes));
+	b->scratchCap = bytes;
+	return 0;
+}
+
+static int ensure_stage(double** p, size_t* cap, size_t nDoubles) {
+	if(nDoubles <= *cap) return 0;
+	if(*p) CLA_HIP(hipFree(*p));
+	*p = nullptr; *cap = 0;
+	CLA_HIP(hipMalloc((void**) p, std::max<size_t>(nDoubles, 1) * sizeof(double)));
+	*cap = nDoubles;
+	return 0;
+}
+
+static int upload(HostGroup& g, const void* src, size_t bytes, const void** dst) {
+	void* d = nullptr;
+	CLA_HIP(hipMalloc(&d, std::max<size_t>(bytes, 16)));
+	g.owned.push_back(d);
+	if(bytes) CLA_HIP(hipMemcpy(d, src, bytes, hipMemcpyHostToDevice));
+	g.bytes += (int64_t) bytes;
+	*dst = d;
+	return 0;
+}
+
+static void free_group(HostGroup& g) {
+	for(void* p : g.owned) (void) hipFree(p);
+	g.owned.clear();
+}
+
+static int check_ready() {
+	if(g_device < 0) {
+		set_error("cla_init has not been called (or failed): no HIP device selected");
+		return -CLA_ERR_STATE;
+	}
+	hipError_t e = hipSetDevice(g_device);
+	if(e != hipSuccess) {
+		set_error("hipSetDevice(%d) failed: %s", g_device, hipGetErrorString(e));
+		return -CLA_ERR_DEVICE;
+	}
+	return 0;
+}
+
+static int check_cols(cla_block* b, const int32_t* cols, int32_t nColG) {
+	if(!cols || nColG <= 0) { set_error("column group without column indexes"); return -CLA_ERR_INVALID; }
+	for(int j = 0; j < nColG; j++)
+		if(cols[j] < 0 || cols[j] >= b->nCols) {
+			set_error("column index %d outside [0,%d)", cols[j], b->nCols);
+			return -CLA_ERR_INVALID;
+		}
+	return 0;
+}
+
+static int check_open(cla_block* b) {
+	if(!b) { set_error("null block handle"); return -CLA_ERR_INVALID; }
+	if(b->finalized) { set_error("block already finalized"); return -CLA_ERR_STATE; }
+	return check_ready();
+}
+
+static int check_final(cla_block* b) {
+	if(!b) { set_error("null block handle"); return -CLA_ERR_INVALID; }
+	if(!b->finalized) { set_error("block not finalized"); return -CLA_ERR_STATE; }
+	return check_ready();
+}
+
+static int init_group(cla_block* b, HostGroup& g, int type, const int32_t* cols, int nColG, const double* dict,
+	int nVals) {
+	memset(&g.d, 0, sizeof(g.d));
+	g.d.type = type; g.d.nColG = nColG; g.d.nVals = nVals;
+	g.cols.assign(cols, cols + nColG);
+	int rc = upload(g, cols, sizeof(int32_t) * (size_t) nColG, (const void**) &g.d.cols);
+	if(rc) return rc;
+	if(dict) g.dict.assign(dict, dict + (size_t) nVals * nColG);
+	(void) b;
+	return 0;
+}
+
+static int upload_dict(HostGroup& g) {
+	return upload(g, g.dict.data(), sizeof(double) * g.dict.size(), (const void**) &g.d.dict);
+}
+
+} // namespace cla
+
+using namespace cla;
+
+extern "C" {
+
+int cla_init(int device) {
+	std::lock_guard<std::mutex> lk(g_initMu);
+	int n = 0;
+	hipError_t e = hipGetDeviceCount(&n);
+	if(e != hipSuccess || n <= 0) {
+		set_error("no HIP device visible (%s); libclahip computes on the GPU only",
+			e != hipSuccess ? hipGetErrorString(e) : "device count 0");
+		g_device = -1;
+		return -CLA_ERR_DEVICE;
+	}
+	if(device < 0 || device >= n) { set_error("device %d out of range (have %d)", device, n); return -CLA_ERR_INVALID; }
+	CLA_HIP(hipSetDevice(device));
+	CLA_HIP(hipGetDeviceProperties(&g_prop, device));
+	if(strncmp(g_prop.gcnArchName, "gfx950", 6) != 0) {
+		set_error("device %d is %s; this library holds gfx950 (MI355X) code only", device, g_prop.gcnArchName);
+		g_device = -1;
+		return -CLA_ERR_DEVICE;
+	}
+	g_numCU = g_prop.multiProcessorCount;
+	g_ldsPerBlock = (int) g_prop.sharedMemPerBlock;
+	if(g_prop.maxSharedMemoryPerMultiProcessor > (size_t) g_ldsPerBlock)
+		g_ldsPerBlock = (int) g_prop.maxSharedMemoryPerMultiProcessor;
+	g_device = device;
+	return 0;
+}
+
+const char* cla_last_error(void) { return t_err; }
+
+int cla_device_info(char* json, size_t cap) {
+	int rc = check_ready();
+	if(rc) return rc;
+	snprintf(json, cap,
+		"{\"name\":\"%s\",\"arch\":\"%s\",\"cus\":%d,\"lds_per_block\":%zu,\"lds_per_cu\":%zu,\"hbm_bytes\":%zu,"
+		"\"clock_khz\":%d,\"mem_clock_khz\":%d,\"mem_bus_bits\":%d,\"l2_bytes\":%d}",
+		g_prop.name, g_prop.gcnArchName, g_prop.multiProcessorCount, g_prop.sharedMemPerBlock,
+		g_prop.maxSharedMemoryPerMultiProcessor, g_prop.totalGlobalMem, g_prop.clockRate, g_prop.memoryClockRate,
+		g_prop.memoryBusWidth, g_prop.l2CacheSize);
+	return 0;
+}
+
+cla_handle cla_block_create(int64_t nRows, int32_t nCols) {
+	if(check_ready()) return nullptr;
+	if(nRows < 0 || nRows > 0x7fffffffLL || nCols <= 0) {
+		set_error("invalid block shape %lld x %d", (long long) nRows, nCols);
+		return nullptr;
+	}
+	cla_block* b = new cla_block();
+	b->nRows = nRows;
+	b->nCols = nCols;
+	b->constV.assign((size_t) nCols, 0.0);
+	if(hipStreamCreate(&b->stream) != hipSuccess) { set_error("hipStreamCreate failed"); delete b; return nullptr; }
+	b->ownStream = true;
+	if(hipMalloc((void**) &b->dCounters, 8 * sizeof(unsigned long long)) != hipSuccess ||
+		hipHostMalloc((void**) &b->hCounters, 8 * sizeof(unsigned long long)) != hipSuccess) {
+		set_error("allocating counters failed");
+		cla_block_free(b);
+		return nullptr;
+	}
+	return b;
+}
+
+void cla_block_free(cla_handle b) {
+	if(!b) return;
+	if(g_device >= 0) (void) hipSetDevice(g_device);
+	if(b->stream) (void) hipStreamSynchronize(b->stream);
+	clear_stats(b);
+	for(auto& g : b->groups) free_group(g);
+	if(b->dGroups) (void) hipFree(b->dGroups);
+	if(b->dConstV) (void) hipFree(b->dConstV);
+	if(b->dSlabStart) (void) hipFree(b->dSlabStart);
+	if(b->dTables) (void) hipFree(b->dTables);
+	if(b->dStageIn) (void) hipFree(b->dStageIn);
+	if(b->dStageOut) (void) hipFree(b->dStageOut);
+	if(b->dScratch) (void) hipFree(b->dScratch);
+	if(b->dCounters) (void) hipFree(b->dCounters);
+	if(b->hCounters) (void) hipHostFree(b->hCounters);
+	if(b->ownStream && b->stream) (void) hipStreamDestroy(b->stream);
+	delete b;
+}
+
+int cla_block_add_ddc(cla_handle b, const int32_t* cols, int32_t nColG, const double* dict, int32_t nVals,
+	const void* codes, int32_t codeWidth) {
+	int rc = check_open(b);
+	if(rc) return rc;
+	if((rc = check_cols(b, cols, nColG))) return rc;
+	if(!dict || nVals <= 0) { set_error("DDC group needs a dictionary"); return -CLA_ERR_INVALID; }
+	if(codeWidth != 1 && codeWidth != 2 && codeWidth != 4) {
+		set_error("unsupported map width %d (MapToByte/UByte=1, MapToChar=2, MapToInt=4)", codeWidth);
+		return -CLA_ERR_UNSUPPORTED;
+	}
+	if(!codes && b->nRows > 0) { set_error("DDC group without codes"); return -CLA_ERR_INVALID; }
+	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	HostGroup g;
+	if((rc = init_group(b, g, G_DDC, cols, nColG, dict, nVals)) || (rc = upload_dict(g)) ||
+		(rc = upload(g, codes, (size_t) b->nRows * codeWidth, &g.d.codes))) {
+		free_group(g);
+		return rc;
+	}
+	g.d.codeWidth = codeWidth;
+	b->groups.push_back(std::move(g));
+	return 0;
+}
+
+int cla_block_add_sdc(cla_handle b, const int32_t* cols, int32_t nColG, const double* dict, int32_t nVals,
+	const double* defaultTuple, const void* codes, int32_t codeWidth, const void* deltas, int32_t deltaWidth,
+	int64_t nDeltas, int32_t offsetToFirst, int32_t offsetToLast, int64_t nOffsets) {
+	int rc = check_open(b);
+	if(rc) return rc;
+	if((rc = check_cols(b, cols, nColG))) return rc;
+	if(!dict || nVals <= 0) { set_error("SDC group needs a dictionary"); return -CLA_ERR_INVALID; }
+	if(codeWidth != 1 && codeWidth != 2 && codeWidth != 4) {
+		set_error("unsupported map width %d", codeWidth);
+		return -CLA_ERR_UNSUPPORTED;
+	}
+	if(nOffsets < 0 || nOffsets > b->nRows || nDeltas < 0) { set_error("invalid offset list size"); return -CLA_ERR_INVALID; }
+	if(nOffsets > 0 && (offsetToFirst < 0 || offsetToLast < offsetToFirst)) {
+		set_error("Invalid negative offset / first %d last %d", offsetToFirst, offsetToLast);
+		return -CLA_ERR_INVALID;
+	}
+	if(nDeltas > 0 && deltaWidth != 1 && deltaWidth != 2) {
+		set_error("unsupported offset width %d (OffsetByte=1, OffsetChar=2)", deltaWidth);
+		return -CLA_ERR_UNSUPPORTED;
+	}
+	if(nDeltas > 0 && !deltas) { set_error("offset deltas missing"); return -CLA_ERR_INVALID; }
+	if(nOffsets > 0 && nDeltas < nOffsets - 1) { set_error("offset list shorter than its size"); return -CLA_ERR_INVALID; }
+	if(nOffsets > 1 && !codes && nVals > 1) { set_error("SDC group without codes"); return -CLA_ERR_INVALID; }
+	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	HostGroup g;
+	if((rc = init_group(b, g, G_SDCZ, cols, nColG, dict, nVals))) { free_group(g); return rc; }
+	if(defaultTuple) {
+		// ColGroupSDC.extractCommon: dictionary minus the default tuple, default into constV
+		g.def.assign(defaultTuple, defaultTuple + nColG);
+		for(int k = 0; k < nVals; k++)
+			for(int j = 0; j < nColG; j++) g.dict[(size_t) k * nColG + j] -= defaultTuple[j];
+	}
+	std::vector<uint8_t> zeros;
+	const void* codeSrc = codes;
+	if(!codes) { zeros.assign((size_t) std::max<int64_t>(nOffsets, 1) * codeWidth, 0); codeSrc = zeros.data(); }
+	if((rc = upload_dict(g)) || (rc = upload(g, codeSrc, (size_t) nOffsets * codeWidth, &g.d.codes)) ||
+		(rc = upload(g, deltas, (size_t) nDeltas * (nDeltas ? deltaWidth : 1), &g.d.deltas))) {
+		free_group(g);
+		return rc;
+	}
+	g.d.codeWidth = codeWidth;
+	g.d.deltaWidth = nDeltas ? deltaWidth : 1;
+	g.d.nDeltas = nDeltas; g.d.nOffsets = nOffsets;
+	g.d.first = nOffsets ? offsetToFirst : 0;
+	g.d.last = nOffsets ? offsetToLast : -1;
+	b->groups.push_back(std::move(g));
+	return 0;
+}
+
+int cla_block_add_rle(cla_handle b, const int32_t* cols, int32_t nColG, const double* dict, int32_t nVals,
+	const int32_t* ptr, const uint16_t* data, int64_t nData) {
+	int rc = check_open(b);
+	if(rc) return rc;
+	if((rc = check_cols(b, cols, nColG))) return rc;
+	if(!dict || nVals <= 0 || !ptr) { set_error("RLE group needs a dictionary and run pointers"); return -CLA_ERR_INVALID; }
+	if(nData < 0 || (nData & 1) || ptr[0] != 0 || ptr[nVals] != nData) {
+		set_error("RLE run array malformed (nData %lld, ptr[0] %d, ptr[nVals] %d)", (long long) nData, ptr[0], ptr[nVals]);
+		return -CLA_ERR_INVALID;
+	}
+	// Merge the per-value run lists into one table sorted by run start
+	// (rs = re + gap; re = rs + len per value, CG/ColGroupRLE.java:114-117).
+	struct Run { int64_t s, e; int32_t k; };
+	std::vector<Run> runs;
+	runs.reserve((size_t) nData / 2);
+	for(int k = 0; k < nVals; k++) {
+		if(ptr[k + 1] < ptr[k] || ((ptr[k + 1] - ptr[k]) & 1)) { set_error("RLE ptr not monotone/even at value %d", k); return -CLA_ERR_INVALID; }
+		int64_t rs = 0, re = 0;
+		for(int p = ptr[k]; p < ptr[k + 1]; p += 2) {
+			rs = re + data[p];
+			re = rs + data[p + 1];
+			if(re > b->nRows) { set_error("RLE run of value %d ends at %lld beyond %lld rows", k, (long long) re, (long long) b->nRows); return -CLA_ERR_INVALID; }
+			if(re > rs) runs.push_back({rs, re, k});
+		}
+	}
+	std::sort(runs.begin(), runs.end(), [](const Run& a, const Run& c) { return a.s < c.s; });
+	std::vector<int32_t> runStart, runCode;
+	int64_t pos = 0;
+	for(const Run& r : runs) {
+		if(r.s < pos) { set_error("RLE runs overlap at row %lld", (long long) r.s); return -CLA_ERR_INVALID; }
+		if(r.s > pos) { runStart.push_back((int32_t) pos); runCode.push_back(-1); }
+		runStart.push_back((int32_t) r.s);
+		runCode.push_back(r.k);
+		pos = r.e;
+	}
+	if(pos < b->nRows || runStart.empty()) { runStart.push_back((int32_t) pos); runCode.push_back(-1); }
+	const int nRuns = (int) runCode.size();
+	runStart.push_back((int32_t) b->nRows);
+	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	HostGroup g;
+	if((rc = init_group(b, g, G_RLE, cols, nColG, dict, nVals)) || (rc = upload_dict(g)) ||
+		(rc = upload(g, runStart.data(), sizeof(int32_t) * runStart.size(), (const void**) &g.d.runStart)) ||
+		(rc = upload(g, runCode.data(), sizeof(int32_t) * runCode.size(), (const void**) &g.d.runCode))) {
+		free_group(g);
+		return rc;
+	}
+	g.d.nRuns = nRuns;
+	b->groups.push_back(std::move(g));
+	return 0;
+}
+
+int cla_block_add_uncompressed(cla_handle b, const int32_t* cols, int32_t nColG, const double* values) {
+	int rc = check_open(b);
+	if(rc) return rc;
+	if((rc = check_cols(b, cols, nColG))) return rc;
+	if(!values && b->nRows > 0) { set_error("uncompressed group without values"); return -CLA_ERR_INVALID; }
+	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	HostGroup g;
+	if((rc = init_group(b, g, G_UNC, cols, nColG, nullptr, 0)) ||
+		(rc = upload(g, values, sizeof(double) * (size_t) b->nRows * nColG, (const void**) &g.d.dense))) {
+		free_group(g);
+		return rc;
+	}
+	b->groups.push_back(std::move(g));
+	return 0;
+}
+
+int cla_block_add_const(cla_handle b, const int32_t* cols, int32_t nColG, const double* row) {
+	int rc = check_open(b);
+	if(rc) return rc;
+	if((rc = check_cols(b, cols, nColG))) return rc;
+	if(!row) { set_error("const group without values"); return -CLA_ERR_INVALID; }
+	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	// ColGroupConst.addToCommon (CG/ColGroupConst.java:330-362)
+	for(int j = 0; j < nColG; j++) b->constV[cols[j]] += row[j];
+	b->hasConst = true;
+	return 0;
+}
+
+int cla_block_add_empty(cla_handle b, const int32_t* cols, int32_t nColG) {
+	int rc = check_open(b);
+	if(rc) return rc;
+	if((rc = check_cols(b, cols, nColG))) return rc;
+	b->hasConst = true; // CLALibUtils.shouldPreFilter is true for empty groups as well
+	return 0;
+}
+
+int cla_block_finalize(cla_handle b) {
+	int rc = check_open(b);
+	if(rc) return rc;
+	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	int tblOff = 0, colOff = 0, maxVals = 0;
+	for(size_t gi = 0; gi < b->groups.size(); gi++) {
+		HostGroup& g = b->groups[gi];
+		DGroup& G = g.d;
+		G.tblOff = tblOff;
+		G.colOff = colOff;
+		tblOff += G.nVals;
+		colOff += G.nColG;
+		maxVals = std::max(maxVals, G.nVals);
+		if(G.type == G_DDC || G.type == G_SDCZ) {
+			int ok = 1;
+			const int64_t n = G.type == G_DDC ? b->nRows : G.nOffsets;
+			if((rc = launch_validate_codes(b, G.codes, G.codeWidth, n, G.nVals, &ok))) return rc;
+			if(!ok) {
+				set_error("group %zu holds a code >= its number of dictionary entries (%d)", gi, G.nVals);
+				return -CLA_ERR_INVALID;
+			}
+		}
+		if(G.type == G_SDCZ) {
+			if(!g.def.empty()) {
+				for(int j = 0; j < G.nColG; j++) b->constV[g.cols[j]] += g.def[j];
+				b->hasConst = true;
+			}
+			if((rc = launch_sdc_build(b, g))) return rc;
+			b->hasSdc = true;
+		}
+		if(G.type == G_RLE) b->hasRle = true;
+		if(G.type == G_UNC) b->hasUnc = true;
+	}
+	b->totalVals = tblOff;
+	b->totalColsG = colOff;
+	b->maxVals = maxVals;
+
+	const size_t nG = b->groups.size();
+	std::vector<DGroup> flat(nG);
+	for(size_t i = 0; i < nG; i++) flat[i] = b->groups[i].d;
+	CLA_HIP(hipMalloc((void**) &b->dGroups, sizeof(DGroup) * std::max<size_t>(nG, 1)));
+	if(nG) CLA_HIP(hipMemcpy(b->dGroups, flat.data(), sizeof(DGroup) * nG, hipMemcpyHostToDevice));
+	CLA_HIP(hipMalloc((void**) &b->dConstV, sizeof(double) * (size_t) b->nCols));
+	CLA_HIP(hipMemcpy(b->dConstV, b->constV.data(), sizeof(double) * (size_t) b->nCols, hipMemcpyHostToDevice));
+
+	// slabs of groups whose mat-vec tables (nVals doubles each) fit the LDS budget
+	const int budget = std::min(g_ldsPerBlock, 64 * 1024);
+	b->slabStart.clear();
+	b->slabLdsBytes = 0;
+	bool fits = nG > 0;
+	int cur = 0;
+	b->slabStart.push_back(0);
+	for(size_t i = 0; i < nG; i++) {
+		const int bytes = b->groups[i].d.nVals * 8;
+		if(bytes > budget) { fits = false; break; }
+		if(cur + bytes > budget) { b->slabStart.push_back((int) i); cur = 0; }
+		cur += bytes;
+		b->slabLdsBytes = std::max(b->slabLdsBytes, cur);
+	}
+	b->slabStart.push_back((int) nG);
+	if(!fits) b->slabLdsBytes = 0;
+	CLA_HIP(hipMalloc((void**) &b->dSlabStart, sizeof(int32_t) * b->slabStart.size()));
+	CLA_HIP(hipMemcpy(b->dSlabStart, b->slabStart.data(), sizeof(int32_t) * b->slabStart.size(), hipMemcpyHostToDevice));
+	b->finalized = true;
+	return 0;
+}
+
+int cla_block_set_stream(cla_handle b, void* hipStream) {
+	if(!b) { set_error("null block handle"); return -CLA_ERR_INVALID; }
+	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	if(b->ownStream && b->stream) { (void) hipStreamSynchronize(b->stream); (void) hipStreamDestroy(b->stream); }
+	b->stream = (hipStream_t) hipStream;
+	b->ownStream = false;
+	return 0;
+}
+
+int32_t cla_block_num_groups(cla_handle b) { return b ? (int32_t) b->groups.size() : -CLA_ERR_INVALID; }
+
+int64_t cla_block_device_bytes(cla_handle b) {
+	if(!b) return -CLA_ERR_INVALID;
+	int64_t s = 0;
+	for(auto& g : b->groups) s += g.bytes;
+	return s;
+}
+
+// ---- drivers -------------------------------------------------------------
+
+static int64_t finish_nnz(cla_block* b) {
+	CLA_HIP(hipMemcpyAsync(b->hCounters, b->dCounters, sizeof(unsigned long long), hipMemcpyDeviceToHost, b->stream));
+	CLA_HIP(hipStreamSynchronize(b->stream));
+	return (int64_t) b->hCounters[0];
+}
+
+int64_t cla_rmm_dev(cla_handle b, const double* dB, int32_t nColB, double* dOut) {
+	int rc = check_final(b);
+	if(rc) return rc;
+	if(!dB || !dOut || nColB <= 0) { set_error("rmm: invalid right-hand side"); return -CLA_ERR_INVALID; }
+	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	if((rc = launch_rmm(b, dB, nColB, dOut, b->dCounters))) return rc;
+	return finish_nnz(b);
+}
+
+int64_t cla_rmm(cla_handle b, const double* B, int32_t nColB, double* out) {
+	int rc = check_final(b);
+	if(rc) return rc;
+	if(!B || !out || nColB <= 0) { set_error("rmm: invalid right-hand side"); return -CLA_ERR_INVALID; }
+	const size_t nIn = (size_t) b->nCols * nColB, nOut = (size_t) b->nRows * nColB;
+	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	if((rc = ensure_stage(&b->dStageIn, &b->stageInCap, nIn)) || (rc = ensure_stage(&b->dStageOut, &b->stageOutCap, nOut)))
+		return rc;
+	CLA_HIP(hipMemcpyAsync(b->dStageIn, B, nIn * sizeof(double), hipMemcpyHostToDevice, b->stream));
+	const int64_t nnz = cla_rmm_dev(b, b->dStageIn, nColB, b->dStageOut);
+	if(nnz < 0) return nnz;
+	if(nOut) CLA_HIP(hipMemcpy(out, b->dStageOut, nOut * sizeof(double), hipMemcpyDeviceToHost));
+	return nnz;
+}
+
+
+int64_t cla_decompress_dev(cla_handle b, double* dOut) {
+	int rc = check_final(b);
+	if(rc) return rc;
+	if(!dOut) { set_error("decompress: null output"); return -CLA_ERR_INVALID; }
+	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	if((rc = launch_decompress(b, dOut, b->dCounters))) return rc;
+	return finish_nnz(b);
+}
+
+int64_t cla_decompress(cla_handle b, double* out) {
+	int rc = check_final(b);
+	if(rc) return rc;
+	if(!out) { set_error("decompress: null output"); return -CLA_ERR_INVALID; }
+	const size_t nOut = (size_t) b->nRows * b->nCols;
+	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	if((rc = ensure_stage(&b->dStageOut, &b->stageOutCap, nOut))) return rc;
+	const int64_t nnz = cla_decompress_dev(b, b->dStageOut);
+	if(nnz < 0) return nnz;
+	if(nOut) CLA_HIP(hipMemcpy(out, b->dStageOut, nOut * sizeof(double), hipMemcpyDeviceToHost));
+	return nnz;
+}
+
+int64_t cla_lmm_dev(cla_handle b, const double* dY, int32_t nRowY, double* dOut) {
+	int rc = check_final(b);
+	if(rc) return rc;
+	if(!dY || !dOut || nRowY <= 0) { set_error("lmm: invalid left-hand side"); return -CLA_ERR_INVALID; }
+	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	if((rc = launch_lmm(b, dY, nRowY, dOut, b->dCounters))) return rc;
+	return finish_nnz(b);
+}
+
+int64_t cla_lmm(cla_handle b, const double* Y, int32_t nRowY, double* out) {
+	int rc = check_final(b);
+	if(rc) return rc;
+	if(!Y || !out || nRowY <= 0) { set_error("lmm: invalid left-hand side"); return -CLA_ERR_INVALID; }
+	const size_t nIn = (size_t) nRowY * b->nRows, nOut = (size_t) nRowY * b->nCols;
+	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	if((rc = ensure_stage(&b->dStageIn, &b->stageInCap, nIn)) || (rc = ensure_stage(&b->dStageOut, &b->stageOutCap, nOut)))
+		return rc;
+	if(nIn) CLA_HIP(hipMemcpyAsync(b->dStageIn, Y, nIn * sizeof(double), hipMemcpyHostToDevice, b->stream));
+	const int64_t nnz = cla_lmm_dev(b, b->dStageIn, nRowY, b->dStageOut);
+	if(nnz < 0) return nnz;
+	CLA_HIP(hipMemcpy(out, b->dStageOut, nOut * sizeof(double), hipMemcpyDeviceToHost));
+	return nnz;
+}
+
+int64_t cla_tsmm_dev(cla_handle b, double* dOut) {
+	int rc = check_final(b);
+	if(rc) return rc;
+	if(!dOut) { set_error("tsmm: null output"); return -CLA_ERR_INVALID; }
+	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	if((rc = launch_tsmm(b, dOut, b->dCounters))) return rc;
+	return finish_nnz(b);
+}
+
+int64_t cla_tsmm(cla_handle b, double* out) {
+	int rc = check_final(b);
+	if(rc) return rc;
+	if(!out) { set_error("tsmm: null output"); return -CLA_ERR_INVALID; }
+	const size_t nOut = (size_t) b->nCols * b->nCols;
+	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	if((rc = ensure_stage(&b->dStageOut, &b->stageOutCap, nOut))) return rc;
+	const int64_t nnz = cla_tsmm_dev(b, b->dStageOut);
+	if(nnz < 0) return nnz;
+	CLA_HIP(hipMemcpy(out, b->dStageOut, nOut * sizeof(double), hipMemcpyDeviceToHost));
+	return nnz;
+}
+
+int64_t cla_mmchain_dev(cla_handle b, const double* dV, const double* dW, int32_t ctype, double* dOut) {
+	int rc = check_final(b);
+	if(rc) return rc;
+	if(!dV || !dOut) { set_error("mmchain: null vector"); return -CLA_ERR_INVALID; }
+	if(ctype != 0 && ctype != 1) { set_error("mmchain: chain type %d not supported (XtXv=0, XtwXv=1)", ctype); return -CLA_ERR_UNSUPPORTED; }
+	if(ctype == 1 && !dW) { set_error("mmchain: XtwXv needs w"); return -CLA_ERR_INVALID; }
+	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	if((rc = launch_mmchain(b, dV, dW, ctype, dOut, b->dCounters))) return rc;
+	return finish_nnz(b);
+}
+
+int64_t cla_mmchain(cla_handle b, const double* v, const double* w, int32_t ctype, double* out) {
+	int rc = check_final(b);
+	if(rc) return rc;
+	if(!v || !out) { set_error("mmchain: null vector"); return -CLA_ERR_INVALID; }
+	if(ctype == 1 && !w) { set_error("mmchain: XtwXv needs w"); return -CLA_ERR_INVALID; }
+	const size_t nV = (size_t) b->nCols, nW = ctype == 1 ? (size_t) b->nRows : 0;
+	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	if((rc = ensure_stage(&b->dStageIn, &b->stageInCap, nV + nW)) || (rc = ensure_stage(&b->dStageOut, &b->stageOutCap, nV)))
+		return rc;
+	CLA_HIP(hipMemcpyAsync(b->dStageIn, v, nV * sizeof(double), hipMemcpyHostToDevice, b->stream));
+	if(nW) CLA_HIP(hipMemcpyAsync(b->dStageIn + nV, w, nW * sizeof(double), hipMemcpyHostToDevice, b->stream));
+	const int64_t nnz = cla_mmchain_dev(b, b->dStageIn, nW ? b->dStageIn + nV : nullptr, ctype, b->dStageOut);
+	if(nnz < 0) return nnz;
+	CLA_HIP(hipMemcpy(out, b->dStageOut, nV * sizeof(double), hipMemcpyDeviceToHost));
+	return nnz;
+}
+
+int cla_cooc(cla_handle b, int32_t gA, int32_t gB, int64_t* out) {
+	int rc = check_final(b);
+	if(rc) return rc;
+	const int nG = (int) b->groups.size();
+	if(gA < 0 || gA >= nG || gB < 0 || gB >= nG || !out) { set_error("cooc: bad group pair (%d,%d)", gA, gB); return -CLA_ERR_INVALID; }
+	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	const size_t n = (size_t) b->groups[gA].d.nVals * b->groups[gB].d.nVals;
+	if(n == 0) { set_error("cooc: groups without dictionaries"); return -CLA_ERR_UNSUPPORTED; }
+	if((rc = ensure_scratch(b, n * sizeof(unsigned long long)))) return rc;
+	if((rc = launch_cooc(b, gA, gB, (unsigned long long*) b->dScratch))) return rc;
+	CLA_HIP(hipMemcpyAsync(out, b->dScratch, n * sizeof(int64_t), hipMemcpyDeviceToHost, b->stream));
+	CLA_HIP(hipStreamSynchronize(b->stream));
+	return 0;
+}
+
+int cla_preagg(cla_handle b, int32_t group, const double* Y, int32_t nRowY, double* preAgg) {
+	int rc = check_final(b);
+	if(rc) return rc;
+	if(group < 0 || group >= (int) b->groups.size() || !Y || !preAgg || nRowY <= 0) { set_error("preagg: bad arguments"); return -CLA_ERR_INVALID; }
+	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	const int nVals = b->groups[group].d.nVals;
+	if(nVals <= 0) { set_error("preagg: group %d is not pre-aggregable", group); return -CLA_ERR_UNSUPPORTED; }
+	const size_t nIn = (size_t) nRowY * b->nRows, nOut = (size_t) nRowY * nVals;
+	if((rc = ensure_stage(&b->dStageIn, &b->stageInCap, nIn)) || (rc = ensure_stage(&b->dStageOut, &b->stageOutCap, nOut)))
+		return rc;
+	if(nIn) CLA_HIP(hipMemcpyAsync(b->dStageIn, Y, nIn * sizeof(double), hipMemcpyHostToDevice, b->stream));
+	if((rc = launch_preagg(b, group, b->dStageIn, nRowY, b->dStageOut))) return rc;
+	CLA_HIP(hipMemcpyAsync(preAgg, b->dStageOut, nOut * sizeof(double), hipMemcpyDeviceToHost, b->stream));
+	CLA_HIP(hipStreamSynchronize(b->stream));
+	return 0;
+}
+
+int cla_counts(cla_handle b, int32_t group, int32_t* counts) {
+	int rc = check_final(b);
+	if(rc) return rc;
+	if(group < 0 || group >= (int) b->groups.size() || !counts) { set_error("counts: bad group %d", group); return -CLA_ERR_INVALID; }
+	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	const int nVals = b->groups[group].d.nVals;
+	if(nVals <= 0) { set_error("counts: group %d has no dictionary", group); return -CLA_ERR_UNSUPPORTED; }
+	if((rc = ensure_scratch(b, sizeof(int32_t) * (size_t) nVals))) return rc;
+	if((rc = launch_counts(b, group, (int32_t*) b->dScratch))) return rc;
+	CLA_HIP(hipMemcpyAsync(counts, b->dScratch, sizeof(int32_t) * (size_t) nVals, hipMemcpyDeviceToHost, b->stream));
+	CLA_HIP(hipStreamSynchronize(b->stream));
+	return 0;
+}
+
+int cla_block_profile(cla_handle b, int enable) {
+	if(!b) { set_error("null block handle"); return -CLA_ERR_INVALID; }
+	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	b->profile = enable != 0;
+	return 0;
+}
+
+int cla_stats(cla_handle b, char* json, size_t cap) {
+	if(!b || !json || cap < 8) return -CLA_ERR_INVALID;
+	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	if(b->stream) (void) hipStreamSynchronize(b->stream);
+	std::string s = "{\"kernels\":[";
+	for(size_t i = 0; i < b->lastStats.size(); i++) {
+		KernelStat& k = b->lastStats[i];
+		if(k.e0 && k.e1 && k.ms < 0) (void) hipEventElapsedTime(&k.ms, k.e0, k.e1);
+		char buf[320];
+		snprintf(buf, sizeof(buf),
+			"%s{\"name\":\"%s\",\"grid\":%ld,\"block\":%ld,\"lds\":%ld,\"algo_bytes\":%.0f,\"ms\":%.6f}", i ? "," : "",
+			k.name.c_str(), k.grid, k.block, k.lds, k.algoBytes, (double) k.ms);
+		s += buf;
+	}
+	s += "]}";
+	if(s.size() + 1 > cap) return -CLA_ERR_INVALID;
+	memcpy(json, s.c_str(), s.size() + 1);
+	return 0;
+}
+
+} // extern "C"

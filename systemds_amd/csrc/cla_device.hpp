@@ -1,0 +1,81 @@
+// Device-side helpers shared by the kernels (gfx950, wave64).
+#pragma once
+#include "cla_internal.hpp"
+
+namespace cla {
+
+constexpr int WAVE = 64;
+
+// AMapToData.getIndex for the three device code widths (unsigned byte, char, int).
+__device__ __forceinline__ int32_t load_code(const void* codes, int width, int64_t i) {
+	if(width == 1) return ((const uint8_t*) codes)[i];
+	if(width == 2) return ((const uint16_t*) codes)[i];
+	return ((const int32_t*) codes)[i];
+}
+
+__device__ __forceinline__ int wave_sum_i32(int v) {
+#pragma unroll
+	for(int d = 32; d > 0; d >>= 1) v += __shfl_down(v, d, WAVE);
+	return v;
+}
+
+__device__ __forceinline__ double wave_sum_f64(double v) {
+#pragma unroll
+	for(int d = 32; d > 0; d >>= 1) v += __shfl_down(v, d, WAVE);
+	return v;
+}
+
+// Adds a per-thread count into a global 64-bit counter: one atomic per wave.
+__device__ __forceinline__ void count_add(unsigned long long* counter, int local) {
+	const int s = wave_sum_i32(local);
+	if((threadIdx.x & (WAVE - 1)) == 0 && s != 0) atomicAdd(counter, (unsigned long long) s);
+}
+
+// Largest j in [0, nRuns) with runStart[j] <= row (runStart[0] == 0).
+__device__ __forceinline__ int rle_find(const int32_t* __restrict__ runStart, int nRuns, int32_t row) {
+	int lo = 0, hi = nRuns - 1;
+	while(lo < hi) {
+		const int mid = (lo + hi + 1) >> 1;
+		if(runStart[mid] <= row) lo = mid; else hi = mid - 1;
+	}
+	return lo;
+}
+
+// One wave decodes 256 consecutive delta entries of an offset list starting at
+// entry i0 from iterator state (row, emit). Lane l owns entries i0+4l .. i0+4l+3.
+// A 0 entry advances the row by maxV without emitting (OffsetByte / OffsetChar
+// semantics). On return rows[k] / didx[k] hold the absolute row and the data
+// index of entry k when bit k of `mask` is set, and (row, emit) is the state
+// behind the 256 entries.
+template <int W>
+__device__ __forceinline__ void sdc_decode256(const void* __restrict__ deltas, int64_t nDeltas, int64_t i0,
+	int32_t& row, int32_t& emit, int32_t rows[4], int32_t didx[4], unsigned& mask) {
+	const int lane = threadIdx.x & (WAVE - 1);
+	const int maxV = W == 1 ? 255 : 65535;
+	const int64_t i = i0 + (int64_t) lane * 4;
+	int s = 0, c = 0;
+	mask = 0;
+#pragma unroll
+	for(int k = 0; k < 4; k++) {
+		int v = -1;
+		if(i + k < nDeltas) v = W == 1 ? (int) ((const uint8_t*) deltas)[i + k] : (int) ((const uint16_t*) deltas)[i + k];
+		s += v < 0 ? 0 : (v == 0 ? maxV : v);
+		rows[k] = s;
+		didx[k] = c;
+		if(v > 0) { mask |= 1u << k; c++; }
+	}
+	int ps = s, pc = c;
+#pragma unroll
+	for(int d = 1; d < WAVE; d <<= 1) {
+		const int t = __shfl_up(ps, d, WAVE);
+		const int u = __shfl_up(pc, d, WAVE);
+		if(lane >= d) { ps += t; pc += u; }
+	}
+	const int exs = ps - s, exc = pc - c;
+#pragma unroll
+	for(int k = 0; k < 4; k++) { rows[k] += row + exs; didx[k] += emit + exc; }
+	row += __shfl(ps, WAVE - 1, WAVE);
+	emit += __shfl(pc, WAVE - 1, WAVE);
+}
+
+} // namespace cla

@@ -1,0 +1,147 @@
+// Internal declarations shared by the HIP translation units of libclahip.so.
+// Nothing here is part of the exported C ABI (see include/cla_hip.h).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <cstdint>
+#include <cstdio>
+#include <mutex>
+#include <string>
+#include <vector>
+
+namespace cla {
+
+enum : int32_t { G_DDC = 0, G_SDCZ = 1, G_RLE = 2, G_UNC = 3 };
+
+// Offset lists are cut into chunks of SDC_CK delta entries; a checkpoint holds
+// the iterator state in front of each chunk. Row tiles of SDC_TILE rows have an
+// index entry with the iterator state in front of the first entry of the tile.
+constexpr int SDC_CK = 1024;
+constexpr int SDC_TILE = 1024;
+
+// Iterator state of an offset list in front of delta entry `idx`:
+// `row` = rows accumulated so far (last emitted row plus pending 0-entry skips),
+// `emit` = number of rows emitted so far (= data index of the next row).
+struct OffState {
+	int32_t idx;
+	int32_t emit;
+	int32_t row;
+	int32_t pad;
+};
+
+// Device-visible description of one column group (plain data).
+struct DGroup {
+	const void* codes;        // DDC: nRows codes; SDCZ: nOffsets codes
+	const double* dict;       // nVals x nColG, row-major (SDC: dict - default)
+	const int32_t* cols;      // nColG global column ids
+	const void* deltas;       // SDCZ: delta entries (u8 / u16)
+	const OffState* ckpt;     // SDCZ: one per chunk of SDC_CK delta entries
+	const OffState* tileIdx;  // SDCZ: one per row tile of SDC_TILE rows
+	const int32_t* runStart;  // RLE: nRuns+1 run starts of the merged run table (last = nRows)
+	const int32_t* runCode;   // RLE: code per merged run, -1 = uncovered rows
+	const double* dense;      // UNC: nRows x nColG row-major
+	int64_t nDeltas;
+	int64_t nOffsets;
+	int32_t type, codeWidth, nVals, nColG;
+	int32_t deltaWidth, first, last, nRuns;
+	int32_t tblOff;           // first row of this group's table in the concatenated pre-aggregate
+	int32_t colOff;           // first column of this group in "decoded column" order
+	int32_t nCkpt, nTiles;
+};
+
+struct HostGroup {
+	DGroup d;                       // host mirror of the device descriptor
+	std::vector<int32_t> cols;
+	std::vector<double> dict;       // host copy of the (morphed) dictionary
+	std::vector<double> def;        // SDC default tuple (empty => none)
+	std::vector<void*> owned;       // device allocations owned by this group
+	int64_t bytes = 0;              // HBM bytes of the compressed representation
+};
+
+struct KernelStat {
+	std::string name;
+	long grid = 0, block = 0, lds = 0;
+	double algoBytes = 0;     // compulsory bytes of this launch (0 = not a streaming kernel)
+	hipEvent_t e0 = nullptr, e1 = nullptr; // only when profiling is enabled
+	float ms = -1.f;
+};
+
+} // namespace cla
+
+struct cla_block {
+	int64_t nRows = 0;
+	int32_t nCols = 0;
+	bool finalized = false;
+	std::vector<cla::HostGroup> groups;
+	std::vector<double> constV;      // filtered constants (SDC defaults, const groups), nCols
+	bool hasConst = false;
+	bool hasUnc = false, hasSdc = false, hasRle = false;
+	int32_t totalVals = 0;           // sum of nVals over groups (+1 row for constV)
+	int32_t totalColsG = 0;          // sum of nColG over groups
+	int32_t maxVals = 0;
+
+	hipStream_t stream = nullptr;
+	bool ownStream = false;
+	std::recursive_mutex mu;
+
+	cla::DGroup* dGroups = nullptr;  // device array of descriptors
+	double* dConstV = nullptr;       // device copy of constV (nCols)
+
+	// q == 1 gather kernel: groups packed into LDS-sized slabs
+	std::vector<int32_t> slabStart;
+	int32_t* dSlabStart = nullptr;
+	int32_t slabLdsBytes = 0;
+
+	// reusable workspaces
+	double* dTables = nullptr;  size_t tablesCap = 0;
+	double* dStageIn = nullptr; size_t stageInCap = 0;
+	double* dStageOut = nullptr; size_t stageOutCap = 0;
+	void* dScratch = nullptr;   size_t scratchCap = 0;
+	unsigned long long* dCounters = nullptr;   // 8 x u64
+	unsigned long long* hCounters = nullptr;   // pinned
+
+	std::vector<cla::KernelStat> lastStats;
+	bool profile = false;            // bracket every kernel with HIP events on `stream`
+};
+
+namespace cla {
+
+void set_error(const char* fmt, ...);
+extern int g_ldsPerBlock;   // usable LDS bytes per workgroup
+extern int g_numCU;
+
+#define CLA_HIP(expr)                                                                              \
+	do {                                                                                           \
+		hipError_t _e = (expr);                                                                    \
+		if(_e != hipSuccess) {                                                                     \
+			cla::set_error("%s failed: %s (%s:%d)", #expr, hipGetErrorString(_e), __FILE__, __LINE__); \
+			return -CLA_ERR_DEVICE;                                                                \
+		}                                                                                          \
+	} while(0)
+
+// ---- launchers implemented in the kernel translation units ----
+int launch_validate_codes(cla_block* b, const void* codes, int width, int64_t n, int nVals, int* ok);
+int launch_counts(cla_block* b, int group, int32_t* dCounts);
+int launch_sdc_build(cla_block* b, HostGroup& g);
+int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned long long* dNnz);
+int launch_decompress(cla_block* b, double* dOut, unsigned long long* dNnz);
+int launch_lmm(cla_block* b, const double* dY, int p, double* dOut, unsigned long long* dNnz);
+int launch_preagg(cla_block* b, int group, const double* dY, int p, double* dPre);
+int launch_tsmm(cla_block* b, double* dOut, unsigned long long* dNnz);
+int launch_cooc(cla_block* b, int gA, int gB, unsigned long long* dOut);
+int launch_mmchain(cla_block* b, const double* dV, const double* dW, int ctype, double* dOut,
+	unsigned long long* dNnz);
+
+// Scope around one kernel launch: records launch geometry and, when the block is
+// in profiling mode, HIP events on the block's stream in front of and behind it.
+struct Prof {
+	cla_block* b;
+	size_t idx;
+	Prof(cla_block* b, const char* name, long grid, long block, long lds, double algoBytes);
+	~Prof();
+};
+void clear_stats(cla_block* b);
+
+int ensure_tables(cla_block* b, size_t nDoubles);
+int ensure_scratch(cla_block* b, size_t bytes);
+
+} // namespace cla

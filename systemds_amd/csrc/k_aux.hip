@@ -1,0 +1,230 @@
+// Finalize-time and per-group helper kernels: code validation, exact integer
+// counts, offset-list checkpoints and row-tile index.
+#include "../../include/cla_hip.h"
+#include "cla_device.hpp"
+
+namespace cla {
+
+// ---------------------------------------------------------------------------
+// max code of a stream (validation: every code must be < nVals)
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void k_max_code(const void* __restrict__ codes, int width, int64_t n,
+	int* __restrict__ maxOut) {
+	int m = -1;
+	for(int64_t i = (int64_t) blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t) gridDim.x * blockDim.x) {
+		const int c = load_code(codes, width, i);
+		// a negative MapToInt entry is invalid as well: report it as a huge code
+		m = max(m, c < 0 ? 0x7fffffff : c);
+	}
+#pragma unroll
+	for(int d = 32; d > 0; d >>= 1) m = max(m, __shfl_down(m, d, WAVE));
+	if((threadIdx.x & 63) == 0) atomicMax(maxOut, m);
+}
+
+int launch_validate_codes(cla_block* b, const void* codes, int width, int64_t n, int nVals, int* ok) {
+	*ok = 1;
+	if(n == 0) return 0;
+	int rc = ensure_scratch(b, 64);
+	if(rc) return rc;
+	int* dMax = (int*) b->dScratch;
+	int init = -1;
+	CLA_HIP(hipMemcpyAsync(dMax, &init, sizeof(int), hipMemcpyHostToDevice, b->stream));
+	const int64_t blocks = (n + 256 * 16 - 1) / (256 * 16);
+	hipLaunchKernelGGL(k_max_code, dim3((unsigned) (blocks > 4096 ? 4096 : blocks)), dim3(256), 0, b->stream, codes,
+		width, n, dMax);
+	int mx = -1;
+	CLA_HIP(hipMemcpyAsync(&mx, dMax, sizeof(int), hipMemcpyDeviceToHost, b->stream));
+	CLA_HIP(hipStreamSynchronize(b->stream));
+	*ok = mx < nVals;
+	return 0;
+}
+
+// ---------------------------------------------------------------------------
+// K10 counts: exact integer histogram of a code stream. Block-private bins in
+// LDS (u32) when they fit, merged with integer atomics; bit-exact by
+// construction. RLE groups sum their run lengths per value.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void k_counts_lds(const void* __restrict__ codes, int width, int64_t n, int nVals,
+	int32_t* __restrict__ counts) {
+	extern __shared__ unsigned int bins[];
+	for(int i = threadIdx.x; i < nVals; i += blockDim.x) bins[i] = 0;
+	__syncthreads();
+	for(int64_t i = (int64_t) blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t) gridDim.x * blockDim.x)
+		atomicAdd(&bins[load_code(codes, width, i)], 1u);
+	__syncthreads();
+	for(int i = threadIdx.x; i < nVals; i += blockDim.x)
+		if(bins[i]) atomicAdd(&counts[i], (int) bins[i]);
+}
+
+__global__ __launch_bounds__(256) void k_counts_global(const void* __restrict__ codes, int width, int64_t n,
+	int32_t* __restrict__ counts) {
+	for(int64_t i = (int64_t) blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t) gridDim.x * blockDim.x)
+		atomicAdd(&counts[load_code(codes, width, i)], 1);
+}
+
+// merged run table: count[code] += runStart[j+1] - runStart[j]
+__global__ __launch_bounds__(256) void k_counts_rle(const int32_t* __restrict__ runStart,
+	const int32_t* __restrict__ runCode, int nRuns, int32_t* __restrict__ counts) {
+	const int j = blockIdx.x * blockDim.x + threadIdx.x;
+	if(j >= nRuns) return;
+	const int c = runCode[j];
+	if(c >= 0) atomicAdd(&counts[c], runStart[j + 1] - runStart[j]);
+}
+
+int launch_counts(cla_block* b, int group, int32_t* dCounts) {
+	const DGroup& G = b->groups[group].d;
+	hipStream_t st = b->stream;
+	CLA_HIP(hipMemsetAsync(dCounts, 0, sizeof(int32_t) * (size_t) G.nVals, st));
+	if(G.type == G_RLE) {
+		if(G.nRuns > 0)
+			hipLaunchKernelGGL(k_counts_rle, dim3((G.nRuns + 255) / 256), dim3(256), 0, st, G.runStart, G.runCode, G.nRuns,
+				dCounts);
+	}
+	else if(G.type == G_DDC || G.type == G_SDCZ) {
+		const int64_t n = G.type == G_DDC ? b->nRows : G.nOffsets;
+		if(n > 0) {
+			int64_t blocks = (n + 256 * 32 - 1) / (256 * 32);
+			if(blocks > g_numCU * 8) blocks = g_numCU * 8;
+			const size_t lds = (size_t) G.nVals * 4;
+			if(lds <= 48 * 1024)
+				hipLaunchKernelGGL(k_counts_lds, dim3((unsigned) blocks), dim3(256), lds, st, G.codes, G.codeWidth, n, G.nVals,
+					dCounts);
+			else
+				hipLaunchKernelGGL(k_counts_global, dim3((unsigned) blocks), dim3(256), 0, st, G.codes, G.codeWidth, n,
+					dCounts);
+		}
+	}
+	else {
+		set_error("counts: group %d is not a dictionary-coded group", group);
+		return -CLA_ERR_UNSUPPORTED;
+	}
+	CLA_HIP(hipGetLastError());
+	return 0;
+}
+
+// ---------------------------------------------------------------------------
+// Offset-list acceleration structures (device twin of AOffset's skip list).
+// ---------------------------------------------------------------------------
+// per chunk of SDC_CK entries: (sum of row increments, number of emitted rows)
+template <int W>
+__global__ __launch_bounds__(256) void k_sdc_chunk_sums(const void* __restrict__ deltas, int64_t nDeltas,
+	int2* __restrict__ sums) {
+	__shared__ int sInc[4], sNz[4];
+	const int maxV = W == 1 ? 255 : 65535;
+	const int64_t i0 = (int64_t) blockIdx.x * SDC_CK + threadIdx.x * 4;
+	int inc = 0, nz = 0;
+#pragma unroll
+	for(int k = 0; k < 4; k++)
+		if(i0 + k < nDeltas) {
+			const int v = W == 1 ? (int) ((const uint8_t*) deltas)[i0 + k] : (int) ((const uint16_t*) deltas)[i0 + k];
+			inc += v == 0 ? maxV : v;
+			nz += v != 0;
+		}
+	inc = wave_sum_i32(inc);
+	nz = wave_sum_i32(nz);
+	if((threadIdx.x & 63) == 0) { sInc[threadIdx.x >> 6] = inc; sNz[threadIdx.x >> 6] = nz; }
+	__syncthreads();
+	if(threadIdx.x == 0) sums[blockIdx.x] = make_int2(sInc[0] + sInc[1] + sInc[2] + sInc[3], sNz[0] + sNz[1] + sNz[2] + sNz[3]);
+}
+
+// exclusive scan of the chunk sums into iterator states; entry nCkpt = final state
+__global__ void k_sdc_scan(const int2* __restrict__ sums, int nCkpt, int first, OffState* __restrict__ ckpt) {
+	if(threadIdx.x != 0 || blockIdx.x != 0) return;
+	long long row = first;
+	int emit = 1;
+	for(int c = 0; c < nCkpt; c++) {
+		OffState s;
+		s.idx = c * SDC_CK; s.emit = emit; s.row = (int32_t) (row > 0x7fffffffLL ? 0x7fffffffLL : row); s.pad = 0;
+		ckpt[c] = s;
+		row += sums[c].x;
+		emit += sums[c].y;
+	}
+	OffState s;
+	s.idx = -1; s.emit = emit; s.row = (int32_t) (row > 0x7fffffffLL ? 0x7fffffffLL : row); s.pad = 0;
+	ckpt[nCkpt] = s;
+}
+
+// tile t: iterator state in front of the first delta entry whose accumulated row
+// reaches t * SDC_TILE.
+template <int W>
+__global__ __launch_bounds__(256) void k_sdc_tile_index(const void* __restrict__ deltas, int64_t nDeltas,
+	const OffState* __restrict__ ckpt, int nCkpt, int first, int nTiles, OffState* __restrict__ tileIdx) {
+	const int t = blockIdx.x * blockDim.x + threadIdx.x;
+	if(t >= nTiles) return;
+	const int maxV = W == 1 ? 255 : 65535;
+	const int64_t tb = (int64_t) t * SDC_TILE;
+	OffState s;
+	s.idx = 0; s.emit = 1; s.row = first; s.pad = 0;
+	if(nCkpt > 0 && first < tb) {
+		// last chunk whose state row is < tb
+		int lo = 0, hi = nCkpt - 1;
+		while(lo < hi) {
+			const int mid = (lo + hi + 1) >> 1;
+			if(ckpt[mid].row < tb) lo = mid; else hi = mid - 1;
+		}
+		s = ckpt[lo];
+		int64_t i = s.idx;
+		const int64_t end = (i + SDC_CK < nDeltas) ? i + SDC_CK : nDeltas;
+		for(; i < end; i++) {
+			const int v = W == 1 ? (int) ((const uint8_t*) deltas)[i] : (int) ((const uint16_t*) deltas)[i];
+			const int nr = s.row + (v == 0 ? maxV : v);
+			if(nr >= tb) break;
+			s.row = nr;
+			s.emit += v != 0;
+		}
+		s.idx = (int32_t) i;
+	}
+	tileIdx[t] = s;
+}
+
+int launch_sdc_build(cla_block* b, HostGroup& g) {
+	DGroup& G = g.d;
+	hipStream_t st = b->stream;
+	const int nCkpt = (int) ((G.nDeltas + SDC_CK - 1) / SDC_CK);
+	const int nTiles = (int) ((b->nRows + SDC_TILE - 1) / SDC_TILE);
+	OffState* ckpt = nullptr;
+	OffState* tiles = nullptr;
+	int2* sums = nullptr;
+	CLA_HIP(hipMalloc((void**) &ckpt, sizeof(OffState) * (size_t) (nCkpt + 1)));
+	g.owned.push_back(ckpt);
+	CLA_HIP(hipMalloc((void**) &tiles, sizeof(OffState) * (size_t) (nTiles > 0 ? nTiles : 1)));
+	g.owned.push_back(tiles);
+	g.bytes += (int64_t) sizeof(OffState) * (nCkpt + 1 + nTiles);
+	if(nCkpt > 0) {
+		CLA_HIP(hipMalloc((void**) &sums, sizeof(int2) * (size_t) nCkpt));
+		if(G.deltaWidth == 1)
+			hipLaunchKernelGGL(k_sdc_chunk_sums<1>, dim3(nCkpt), dim3(256), 0, st, G.deltas, G.nDeltas, sums);
+		else
+			hipLaunchKernelGGL(k_sdc_chunk_sums<2>, dim3(nCkpt), dim3(256), 0, st, G.deltas, G.nDeltas, sums);
+	}
+	hipLaunchKernelGGL(k_sdc_scan, dim3(1), dim3(1), 0, st, sums, nCkpt, G.first, ckpt);
+	if(nTiles > 0) {
+		if(G.deltaWidth == 1)
+			hipLaunchKernelGGL(k_sdc_tile_index<1>, dim3((nTiles + 255) / 256), dim3(256), 0, st, G.deltas, G.nDeltas, ckpt,
+				nCkpt, G.first, nTiles, tiles);
+		else
+			hipLaunchKernelGGL(k_sdc_tile_index<2>, dim3((nTiles + 255) / 256), dim3(256), 0, st, G.deltas, G.nDeltas, ckpt,
+				nCkpt, G.first, nTiles, tiles);
+	}
+	OffState fin;
+	CLA_HIP(hipMemcpyAsync(&fin, ckpt + nCkpt, sizeof(OffState), hipMemcpyDeviceToHost, st));
+	CLA_HIP(hipStreamSynchronize(st));
+	if(sums) CLA_HIP(hipFree(sums));
+	CLA_HIP(hipGetLastError());
+	if(fin.row != G.last || fin.emit != G.nOffsets) {
+		set_error("SDC offsets inconsistent: decoded last row %d / %d rows, declared offsetToLast %d / %lld rows",
+			fin.row, fin.emit, G.last, (long long) G.nOffsets);
+		return -CLA_ERR_INVALID;
+	}
+	if(G.last >= b->nRows) {
+		set_error("SDC offsetToLast %d is outside the block (%lld rows)", G.last, (long long) b->nRows);
+		return -CLA_ERR_INVALID;
+	}
+	G.ckpt = ckpt;
+	G.tileIdx = tiles;
+	G.nCkpt = nCkpt;
+	G.nTiles = nTiles;
+	return 0;
+}
+
+} // namespace cla

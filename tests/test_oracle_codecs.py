@@ -1,0 +1,189 @@
+"""Pins the oracle's offset / RLE / map-width codecs against the reference's own
+known-answer vectors (src/test/java/org/apache/sysds/test/component/compress/
+offset/OffsetTests.java:78-140, OffsetPreAggTests.java:50-350)."""
+import numpy as np
+import pytest
+
+from conftest import java_random_ints
+
+CMAX = 65535
+
+
+def gen(i, j, seed):
+    """OffsetTests.gen (OffsetTests.java:150-160) on java.util.Random."""
+    nxt = java_random_ints(seed)
+    o = nxt(j)
+    a = [o]
+    for _ in range(1, i):
+        o += nxt(j) + 1
+        a.append(o)
+    return a
+
+
+KNOWN = [
+    [1, 2], [1, 3, 5, 7], [2, 3, 6, 7], [2, 5, 10, 12], [2, 6, 8, 14], [2, 142], [142, 421], [1, 1023], [1023, 1024],
+    [1023], [0, 1, 2, 3, 4, 5], [0], [500], [1442], [CMAX, CMAX + 1], [0, 256], [0, 254], [0, CMAX], [2, CMAX + 2],
+    [0, CMAX + 1], [0, CMAX - 1], [0, 256 * 2], [0, 255 * 2], [0, 254 * 2], [0, 510, 765], [0, 254 * 3],
+    [0, 255, 255 * 2, 255 * 3], [0, 255 * 2, 255 * 3], [0, 255 * 2, 255 * 3, 255 * 10], [0, 255 * 3], [0, 255 * 4],
+    [0, 256 * 3], [0, 100, 200, 300, 400, 500, 600], [0, 200, 400, 600, 800, 1000, 1200], [255 * 3, 255 * 5],
+    [1000000, 1000000 + 255 * 5], [100000000, 100000000 + 255 * 5], [100000000, 100001275, 100001530],
+    [0, 1, 2, 3, 255 * 4, 1500], [2458248, 2458249, 2458253, 2458254, 2458256, 2458257, 2458258, 2458262, 2458264,
+                                  2458266, 2458267, 2458271, 2458272, 2458275, 2458276, 2458281],
+    [CMAX, CMAX * 2], [0, CMAX, CMAX * 2], [1, CMAX * 2 + 3, CMAX * 4 + 4, CMAX * 16 + 4],
+]
+RANDOM = [gen(100, 100, 1)] + [g for i in range(10) for g in (
+    gen(100, 200, i), gen(100, 250, i + 10230), gen(100, 4, i + 120), gen(100, 350, i + 1030),
+    gen(30, 1000, i + 101420), gen(30, 3000, i + 101420))]
+
+
+def test_java_random_matches_documented_sequence():
+    # java.util.Random(42): nextInt(10) starts 0, 3, 8 (the widely quoted sequence)
+    nxt = java_random_ints(42)
+    assert [nxt(10) for _ in range(3)] == [0, 3, 8]
+
+
+@pytest.mark.parametrize("width", [1, 2])
+@pytest.mark.parametrize("rows", KNOWN + RANDOM, ids=lambda r: f"n{len(r)}_{r[0]}_{r[-1]}")
+def test_offset_round_trip_reference_vectors(ora, rows, width):
+    rows = np.array(rows, np.int32)
+    max_v = 255 if width == 1 else CMAX
+    d = ora.offset_encode(rows, width)
+    # structure: entries <= maxV, count = sum(1 + (gap-1)//maxV) (calcSize), zeros only in front of long gaps
+    gaps = np.diff(rows.astype(np.int64))
+    assert d.size == int(np.sum(1 + (gaps - 1) // max_v))
+    assert d.size == 0 or int(d.max()) <= max_v
+    assert int(np.count_nonzero(d)) == rows.size - 1
+    if gaps.size and gaps.max() <= max_v:
+        assert np.array_equal(d.astype(np.int64), gaps)
+    # decode with the C iterator and with an independent plain-Python iterator
+    assert np.array_equal(ora.offset_decode(d, rows[0], rows.size), rows)
+    assert np.array_equal(ora.py_offset_decode(d, rows[0]), rows)
+
+
+def test_offset_boundary_encodings(ora):
+    # the decoder rule "0 means +maxV and no row" fixes these encodings uniquely up to
+    # where the non-zero entry sits; the encoder puts the remainder last.
+    enc = lambda r: ora.offset_encode(np.array(r, np.int32), 1).tolist()
+    assert enc([0, 255]) == [255]
+    assert enc([0, 256]) == [0, 1]
+    assert enc([0, 510]) == [0, 255]
+    assert enc([0, 510, 765]) == [0, 255, 255]
+    assert enc([0, 765]) == [0, 0, 255]
+    assert enc([0, 508]) == [0, 253]
+    enc2 = lambda r: ora.offset_encode(np.array(r, np.int32), 2).tolist()
+    assert enc2([0, CMAX]) == [CMAX]
+    assert enc2([0, CMAX + 1]) == [0, 1]
+    assert enc2([CMAX, CMAX * 2]) == [CMAX]
+
+
+def test_offset_rejects_unsorted_and_negative(ora):
+    with pytest.raises(ora.OracleError):
+        ora.offset_encode(np.array([3, 3], np.int32), 1)
+    with pytest.raises(ora.OracleError):
+        ora.offset_encode(np.array([5, 2], np.int32), 1)
+    with pytest.raises(ora.OracleError):
+        ora.offset_encode(np.array([-1, 2], np.int32), 1)
+
+
+def test_harness_encoder_agrees_with_oracle(ora):
+    from systemds_amd import synth
+    for rows in KNOWN + RANDOM:
+        rows = np.array(rows, np.int32)
+        for width in (1, 2):
+            d, first, last, n = synth.encode_offsets(rows, width)
+            assert (first, last, n) == (rows[0], rows[-1], rows.size)
+            assert np.array_equal(d, ora.offset_encode(rows, width))
+        if rows.size >= 3:
+            assert synth.choose_offset_width(rows) == ora.offset_choose_width(rows)
+
+
+# OffsetPreAggTests: db is 2 x 5 with db[r][i] = i; preAV has one bin (all codes 0).
+PREAGG_CASES = [
+    # (offsets, fill, rl, ru, cl, cu, expected per row)
+    ([0, 1, 2, 3, 4], "ones", 0, 1, 0, 5, [5.0]),
+    ([0, 1, 2, 3, 4], "iota", 0, 1, 0, 5, [10.0]),
+    ([0, 1, 2, 4], "iota", 0, 1, 0, 5, [7.0]),
+    ([0, 1, 2], "iota", 0, 1, 0, 5, [3.0]),
+    ([0, 2], "iota", 0, 1, 0, 5, [2.0]),
+    ([0, 2], "iota", 1, 2, 0, 5, [2.0]),
+    ([1, 2, 3], "iota", 1, 2, 4, 5, [0.0]),
+    ([3], "iota", 1, 2, 0, 2, [0.0]),
+    ([3], "iota", 1, 2, 0, 3, [0.0]),
+    ([3, 4, 5], "iota", 1, 2, 0, 4, [3.0]),
+    ([3], "iota", 0, 2, 0, 5, [3.0, 3.0]),
+    ([2, 3, 4], "iota", 0, 2, 0, 5, [9.0, 9.0]),
+    ([2, 3, 4], "iota", 0, 2, 0, 4, [5.0, 5.0]),
+]
+
+
+@pytest.mark.parametrize("case", PREAGG_CASES, ids=lambda c: f"{c[0]}_{c[2]}{c[3]}{c[4]}{c[5]}")
+def test_offset_preaggregate_known_sums(ora, case):
+    """OffsetPreAggTests.preAggDense* (exact sums). The reference call is
+    off.preAggregateDenseMap(db, preAV, rl, ru, cl, cu, nVal=1, data); here the
+    row range selects rows of Y and the column range is applied by zeroing Y
+    outside [cl,cu) (a column of Y is a row of X)."""
+    from systemds_amd import synth
+    offs, fill, rl, ru, cl, cu, expect = case
+    n_x_rows = 6
+    Y = np.zeros((2, n_x_rows))
+    Y[:, :5] = 1.0 if fill == "ones" else np.arange(5.0)
+    Ysel = np.zeros_like(Y)
+    Ysel[:, cl:cu] = Y[:, cl:cu]
+    Ysel = Ysel[rl:ru]
+    rows = np.array(offs, np.int32)
+    for width in (1, 2):
+        d, first, last, n = synth.encode_offsets(rows, width)
+        g = synth.GroupSpec("sdc", np.array([0], np.int32), np.array([[1.0]]), np.zeros(n, np.uint8), None, d, first,
+                            last, n)
+        G = ora.Groups([g], n_x_rows, 1)
+        pre = ora.preaggregate_dense(G, 0, Ysel)
+        assert pre[:, 0].tolist() == expect
+
+
+def test_rle_round_trip_and_structure(ora):
+    rng = np.random.default_rng(5)
+    cases = [
+        [0], [5], [0, 1, 2, 3], [1, 3, 5], [CMAX], [CMAX + 1], [0, CMAX + 10], [3 * CMAX + 7, 3 * CMAX + 8],
+        list(range(10, 10 + CMAX + 5)),           # a run longer than 65535 is cut
+        [2, 3, 4, 200000, 200001, 500000],
+    ]
+    for _ in range(20):
+        n = int(rng.integers(1, 400))
+        cases.append(np.unique(rng.integers(0, 300000, n)).tolist())
+    for rows in cases:
+        rows = np.array(rows, np.int32)
+        data = ora.rle_encode(rows)
+        assert data.size % 2 == 0
+        assert np.array_equal(ora.rle_decode(data, rows.size), rows)
+        gaps, lens = data[0::2].astype(np.int64), data[1::2].astype(np.int64)
+        assert lens.sum() == rows.size
+        # zero-length filler runs always carry a full 65535 gap
+        assert np.all(gaps[lens == 0] == CMAX)
+        # independent python decode of a one-value group
+        assert np.array_equal(ora.py_rle_rows(np.array([0, data.size]), data, 0), rows)
+
+
+def test_harness_rle_encoder_agrees_with_oracle(ora):
+    from systemds_amd import synth
+    rng = np.random.default_rng(11)
+    for n_rows in (1, 17, 5000, 300000):
+        run_codes = rng.integers(-1, 3, size=max(n_rows // 50, 2))
+        lens = rng.integers(1, 100 if n_rows < 300000 else 150000, size=run_codes.size)
+        codes = np.repeat(run_codes, lens)[:n_rows]
+        if codes.size < n_rows:
+            codes = np.concatenate([codes, np.full(n_rows - codes.size, -1)])
+        ptr, data = synth.encode_rle(codes, 3)
+        for k in range(3):
+            rows = np.flatnonzero(codes == k).astype(np.int32)
+            seg = data[ptr[k]:ptr[k + 1]]
+            if rows.size == 0:
+                assert seg.size == 0
+            else:
+                assert np.array_equal(seg, ora.rle_encode(rows))
+
+
+def test_map_width_table(ora):
+    # MapToFactory.java:102-117
+    L = ora.lib()
+    assert [L.ora_map_width(n) for n in (0, 1, 2, 128, 256, 257, 65536, 65537, 8388607, 8388608)] == \
+        [0, 0, 1, 1, 1, 2, 2, 3, 3, 4]
