@@ -214,7 +214,9 @@ void cla_block_free(cla_handle b) {
 	for(auto& g : b->groups) free_group(g);
 	if(b->dGroups) (void) hipFree(b->dGroups);
 	if(b->dConstV) (void) hipFree(b->dConstV);
-	if(b->dSlabStart) (void) hipFree(b->dSlabStart);
+	if(b->dQ1Slabs) (void) hipFree(b->dQ1Slabs);
+	if(b->dArena) (void) hipFree(b->dArena);
+	if(b->dTblOff) (void) hipFree(b->dTblOff);
 	if(b->dTables) (void) hipFree(b->dTables);
 	if(b->dStageIn) (void) hipFree(b->dStageIn);
 	if(b->dStageOut) (void) hipFree(b->dStageOut);
@@ -429,24 +431,66 @@ int cla_block_finalize(cla_handle b) {
 	CLA_HIP(hipMalloc((void**) &b->dConstV, sizeof(double) * (size_t) b->nCols));
 	CLA_HIP(hipMemcpy(b->dConstV, b->constV.data(), sizeof(double) * (size_t) b->nCols, hipMemcpyHostToDevice));
 
-	// slabs of groups whose mat-vec tables (nVals doubles each) fit the LDS budget
-	const int budget = std::min(g_ldsPerBlock, 64 * 1024);
-	b->slabStart.clear();
-	b->slabLdsBytes = 0;
-	bool fits = nG > 0;
-	int cur = 0;
-	b->slabStart.push_back(0);
-	for(size_t i = 0; i < nG; i++) {
-		const int bytes = b->groups[i].d.nVals * 8;
-		if(bytes > budget) { fits = false; break; }
-		if(cur + bytes > budget) { b->slabStart.push_back((int) i); cur = 0; }
-		cur += bytes;
-		b->slabLdsBytes = std::max(b->slabLdsBytes, cur);
+	// table offsets (prefix sums of nVals) for kernels that stage tables in LDS
+	{
+		std::vector<int32_t> off(nG + 1, 0);
+		for(size_t i = 0; i < nG; i++) off[i + 1] = off[i] + b->groups[i].d.nVals;
+		CLA_HIP(hipMalloc((void**) &b->dTblOff, sizeof(int32_t) * (nG + 1)));
+		CLA_HIP(hipMemcpy(b->dTblOff, off.data(), sizeof(int32_t) * (nG + 1), hipMemcpyHostToDevice));
 	}
-	b->slabStart.push_back((int) nG);
-	if(!fits) b->slabLdsBytes = 0;
-	CLA_HIP(hipMalloc((void**) &b->dSlabStart, sizeof(int32_t) * b->slabStart.size()));
-	CLA_HIP(hipMemcpy(b->dSlabStart, b->slabStart.data(), sizeof(int32_t) * b->slabStart.size(), hipMemcpyHostToDevice));
+
+	// code arena: all groups DDC with one code width -> one allocation, uniform stride
+	bool allDdc = nG > 0 && b->nRows > 0;
+	const int cw = nG ? b->groups[0].d.codeWidth : 0;
+	for(auto& g : b->groups)
+		if(g.d.type != G_DDC || g.d.codeWidth != cw) allDdc = false;
+	if(allDdc) {
+		const size_t stride = (((size_t) b->nRows * cw) + 255) & ~(size_t) 255;
+		CLA_HIP(hipMalloc((void**) &b->dArena, stride * nG));
+		for(size_t i = 0; i < nG; i++) {
+			HostGroup& g = b->groups[i];
+			uint8_t* dst = b->dArena + i * stride;
+			CLA_HIP(hipMemcpyAsync(dst, g.d.codes, (size_t) b->nRows * cw, hipMemcpyDeviceToDevice, b->stream));
+			CLA_HIP(hipStreamSynchronize(b->stream));
+			void* old = const_cast<void*>(g.d.codes);
+			g.owned.erase(std::remove(g.owned.begin(), g.owned.end(), old), g.owned.end());
+			CLA_HIP(hipFree(old));
+			g.d.codes = dst;
+			flat[i].codes = dst;
+		}
+		CLA_HIP(hipMemcpy(b->dGroups, flat.data(), sizeof(DGroup) * nG, hipMemcpyHostToDevice));
+		b->arenaStride = stride;
+		b->arenaWidth = cw;
+	}
+
+	// Slabs of groups whose mat-vec tables fit the LDS budget. Inside a slab every
+	// table gets the same LDS stride (the largest nVals of the block) plus one
+	// all-zero table, so table addresses are pure arithmetic; every slab but the
+	// last holds a multiple of 8 groups (two batches of 4, see k_rmm_q1_ddc).
+	{
+		int budget = 52 * 1024;
+		if(const char* e = getenv("CLA_Q1_LDS_KB")) budget = atoi(e) * 1024;
+		budget = std::min(budget, g_ldsPerBlock);
+		b->q1Slabs.clear();
+		b->q1LdsBytes = 0;
+		const int mx = std::max(maxVals, 1);
+		int per = budget / (mx * 8) - 1;   // groups per slab, one slot kept for the zero table
+		// a thread stages at most 16 table values (Q1_TPT) for the next slab; the smallest block has 256 threads
+		per = std::min(per, 16 * 256 / mx);
+		per = per / 8 * 8;
+		if(nG > 0 && per >= 8) {
+			for(size_t i = 0; i < nG; i += per) {
+				const size_t j = std::min(nG, i + (size_t) per);
+				bool uniform = true;
+				for(size_t g = i; g < j; g++) uniform &= b->groups[g].d.nVals == mx;
+				b->q1Slabs.push_back(make_int4((int) i, (int) j, mx, uniform ? 1 : 0));
+			}
+			const size_t most = std::min(nG, (size_t) per);
+			b->q1LdsBytes = (int32_t) ((most + 1) * mx * 8);
+			CLA_HIP(hipMalloc((void**) &b->dQ1Slabs, sizeof(int4) * b->q1Slabs.size()));
+			CLA_HIP(hipMemcpy(b->dQ1Slabs, b->q1Slabs.data(), sizeof(int4) * b->q1Slabs.size(), hipMemcpyHostToDevice));
+		}
+	}
 	b->finalized = true;
 	return 0;
 }

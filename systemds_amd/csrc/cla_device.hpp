@@ -6,6 +6,11 @@ namespace cla {
 
 constexpr int WAVE = 64;
 
+// clang vector types: the non-temporal load/store builtins want these
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef double f64x2 __attribute__((ext_vector_type(2)));
+
 // AMapToData.getIndex for the three device code widths (unsigned byte, char, int).
 __device__ __forceinline__ int32_t load_code(const void* codes, int width, int64_t i) {
 	if(width == 1) return ((const uint8_t*) codes)[i];

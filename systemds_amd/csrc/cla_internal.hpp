@@ -86,10 +86,17 @@ struct cla_block {
 	cla::DGroup* dGroups = nullptr;  // device array of descriptors
 	double* dConstV = nullptr;       // device copy of constV (nCols)
 
-	// q == 1 gather kernel: groups packed into LDS-sized slabs
-	std::vector<int32_t> slabStart;
-	int32_t* dSlabStart = nullptr;
-	int32_t slabLdsBytes = 0;
+	// All-DDC blocks of one code width keep their code streams in one arena with a
+	// uniform stride, so kernels address stream g as arena + g * arenaStride.
+	uint8_t* dArena = nullptr;
+	size_t arenaStride = 0;
+	int32_t arenaWidth = 0;
+	int32_t* dTblOff = nullptr;      // nGroups+1 table offsets (prefix sum of nVals)
+
+	// mat-vec gather kernel: groups packed into LDS-sized slabs (g0, g1, table stride, 0)
+	std::vector<int4> q1Slabs;
+	int4* dQ1Slabs = nullptr;
+	int32_t q1LdsBytes = 0;
 
 	// reusable workspaces
 	double* dTables = nullptr;  size_t tablesCap = 0;

@@ -190,6 +190,14 @@ int launch_sdc_build(cla_block* b, HostGroup& g) {
 	CLA_HIP(hipMalloc((void**) &tiles, sizeof(OffState) * (size_t) (nTiles > 0 ? nTiles : 1)));
 	g.owned.push_back(tiles);
 	g.bytes += (int64_t) sizeof(OffState) * (nCkpt + 1 + nTiles);
+	if(G.nOffsets == 0) {
+		// empty list: every consumer checks nOffsets before emitting the first row
+		CLA_HIP(hipMemsetAsync(ckpt, 0, sizeof(OffState) * (size_t) (nCkpt + 1), st));
+		CLA_HIP(hipMemsetAsync(tiles, 0, sizeof(OffState) * (size_t) (nTiles > 0 ? nTiles : 1), st));
+		CLA_HIP(hipStreamSynchronize(st));
+		G.ckpt = ckpt; G.tileIdx = tiles; G.nCkpt = 0; G.nTiles = nTiles;
+		return 0;
+	}
 	if(nCkpt > 0) {
 		CLA_HIP(hipMalloc((void**) &sums, sizeof(int2) * (size_t) nCkpt));
 		if(G.deltaWidth == 1)

@@ -43,102 +43,173 @@ __global__ void k_preagg(const DGroup* __restrict__ groups, int nGroups, const d
 }
 
 // ---------------------------------------------------------------------------
-// K2 (mat-vec): all groups DDC with the same code width CW.
-// A thread owns RPT = 16 consecutive rows and keeps their sums in registers;
-// the pre-aggregated tables of a slab of groups are staged in LDS. Code streams
-// are read with 16-byte loads (a wave reads 1 KiB x CW contiguous per group),
-// NB groups in flight per thread. Groups are visited in list order, so every
-// output cell is summed in the same order as the CPU algorithm.
+// K2 (mat-vec): all groups DDC with the same code width CW, code streams in one
+// arena with a uniform stride.
+// A thread owns RPT consecutive rows and keeps their sums in registers; the
+// pre-aggregated tables of a slab of groups are staged in LDS with a uniform
+// stride, so code and table addresses are pure arithmetic (no per-group pointer
+// loads in the hot loop). Code streams are read with 16-byte non-temporal loads,
+// NB groups in flight per thread and the next batch requested before the current
+// one is consumed. Groups are visited in list order, so every output cell is
+// summed in the same order as the CPU algorithm.
 // ---------------------------------------------------------------------------
-template <int CW>
-struct CodeVec;
+template <int BYTES>
+struct RawVec;
 template <>
-struct CodeVec<1> {
-	uint4 v;
-	__device__ __forceinline__ void load(const void* codes, int64_t row0) { v = *(const uint4*) ((const uint8_t*) codes + row0); }
-	__device__ __forceinline__ int get(int i) const {
-		const uint32_t w = i < 4 ? v.x : i < 8 ? v.y : i < 12 ? v.z : v.w;
-		return (w >> (8 * (i & 3))) & 0xffu;
-	}
+struct RawVec<8> {
+	u32x2 v;
+	__device__ __forceinline__ void load(const uint8_t* p) { v = __builtin_nontemporal_load((const u32x2*) p); }
+	__device__ __forceinline__ uint32_t word(int i) const { return i == 0 ? v.x : v.y; }
 };
 template <>
-struct CodeVec<2> {
-	uint4 v[2];
-	__device__ __forceinline__ void load(const void* codes, int64_t row0) {
-		const uint4* p = (const uint4*) ((const uint16_t*) codes + row0);
-		v[0] = p[0]; v[1] = p[1];
-	}
-	__device__ __forceinline__ int get(int i) const {
-		const uint4 q = v[i >> 3];
-		const int j = i & 7;
-		const uint32_t w = j < 2 ? q.x : j < 4 ? q.y : j < 6 ? q.z : q.w;
-		return (w >> (16 * (j & 1))) & 0xffffu;
-	}
+struct RawVec<16> {
+	u32x4 v;
+	__device__ __forceinline__ void load(const uint8_t* p) { v = __builtin_nontemporal_load((const u32x4*) p); }
+	__device__ __forceinline__ uint32_t word(int i) const { return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w; }
 };
 template <>
-struct CodeVec<4> {
-	uint4 v[4];
-	__device__ __forceinline__ void load(const void* codes, int64_t row0) {
-		const uint4* p = (const uint4*) ((const int32_t*) codes + row0);
-		v[0] = p[0]; v[1] = p[1]; v[2] = p[2]; v[3] = p[3];
+struct RawVec<32> {
+	u32x4 v[2];
+	__device__ __forceinline__ void load(const uint8_t* p) {
+		v[0] = __builtin_nontemporal_load((const u32x4*) p);
+		v[1] = __builtin_nontemporal_load((const u32x4*) p + 1);
 	}
-	__device__ __forceinline__ int get(int i) const {
-		const uint4 q = v[i >> 2];
+	__device__ __forceinline__ uint32_t word(int i) const {
+		const u32x4 q = v[i >> 2];
 		const int j = i & 3;
-		return (int) (j == 0 ? q.x : j == 1 ? q.y : j == 2 ? q.z : q.w);
+		return j == 0 ? q.x : j == 1 ? q.y : j == 2 ? q.z : q.w;
+	}
+};
+template <>
+struct RawVec<64> {
+	u32x4 v[4];
+	__device__ __forceinline__ void load(const uint8_t* p) {
+#pragma unroll
+		for(int k = 0; k < 4; k++) v[k] = __builtin_nontemporal_load((const u32x4*) p + k);
+	}
+	__device__ __forceinline__ uint32_t word(int i) const {
+		const u32x4 q = v[i >> 2];
+		const int j = i & 3;
+		return j == 0 ? q.x : j == 1 ? q.y : j == 2 ? q.z : q.w;
 	}
 };
 
-constexpr int Q1_RPT = 16;
+// RPT codes of width CW held in registers
+template <int CW, int RPT>
+struct CodeVec {
+	RawVec<CW * RPT> raw;
+	__device__ __forceinline__ void load(const uint8_t* p) { raw.load(p); }
+	__device__ __forceinline__ int get(int i) const {
+		if(CW == 1) return (raw.word(i >> 2) >> (8 * (i & 3))) & 0xffu;
+		if(CW == 2) return (raw.word(i >> 1) >> (16 * (i & 1))) & 0xffffu;
+		return (int) raw.word(i);
+	}
+};
 
-template <int CW, int THREADS>
-__global__ __launch_bounds__(THREADS) void k_rmm_q1_ddc(const DGroup* __restrict__ groups,
-	const int32_t* __restrict__ slabStart, int nSlabs, const double* __restrict__ T, int constIdx,
-	double* __restrict__ out, int64_t nRows, unsigned long long* __restrict__ nnz) {
-	extern __shared__ double tbl[];
-	constexpr int NB = CW == 1 ? 8 : CW == 2 ? 4 : 2;
-	const int tid = threadIdx.x;
-	const int64_t row0 = ((int64_t) blockIdx.x * THREADS + tid) * Q1_RPT;
-	const bool full = row0 + Q1_RPT <= nRows;
-	const bool any = row0 < nRows;
-	double acc[Q1_RPT];
+template <int CW, int RPT, int NB>
+__device__ __forceinline__ void q1_load(CodeVec<CW, RPT> (&cv)[NB], const uint8_t* myCodes, size_t arenaStride, int g,
+	int gLast) {
 #pragma unroll
-	for(int i = 0; i < Q1_RPT; i++) acc[i] = 0.0;
+	for(int j = 0; j < NB; j++) cv[j].load(myCodes + (size_t) min(g + j, gLast) * arenaStride);
+}
+
+// adds table[code] of NB groups; LDS slot 0 is an all-zero table that serves the
+// padded batch slots beyond the slab, group gRel of the slab sits in slot gRel + 1
+template <int CW, int RPT, int NB>
+__device__ __forceinline__ void q1_consume(const CodeVec<CW, RPT> (&cv)[NB], const double* tbl, int tstride, int gRel,
+	int nInSlab, double (&acc)[RPT]) {
+#pragma unroll
+	for(int j = 0; j < NB; j++) {
+		const double* t = tbl + (size_t) (gRel + j < nInSlab ? gRel + j + 1 : 0) * tstride;
+#pragma unroll
+		for(int i = 0; i < RPT; i++) acc[i] += t[cv[j].get(i)];
+	}
+}
+
+// Every slab but the last holds a multiple of 2 * Q1_NB groups (the host plans
+// it so): batches of Q1_NB groups alternate between two register sets, and the
+// request for the batch after next is always issued before a batch is consumed,
+// also across slab boundaries. The tables of the next slab are fetched into
+// registers (Q1_TPT values per thread) while the current slab is processed.
+constexpr int Q1_NB = 4;
+constexpr int Q1_TPT = 16;
+
+// value f of a slab's padded table image: group f / tstride, entry f % tstride
+__device__ __forceinline__ double q1_table_value(const double* __restrict__ T, const int32_t* __restrict__ tblOff,
+	int4 sl, int f) {
+	const int tstride = sl.z;
+	if(sl.w) return T[tblOff[sl.x] + f]; // uniform nVals == tstride: the image is a plain copy
+	const int g = f / tstride, i = f - g * tstride;
+	const int o = tblOff[sl.x + g], n = tblOff[sl.x + g + 1] - o;
+	return i < n ? T[o + i] : 0.0;
+}
+
+template <int CW, int RPT, int THREADS>
+__global__ __launch_bounds__(THREADS) void k_rmm_q1_ddc(const uint8_t* __restrict__ arena, size_t arenaStride,
+	int nGroups, const int4* __restrict__ slabs, int nSlabs, const int32_t* __restrict__ tblOff,
+	const double* __restrict__ T, int constIdx, double* __restrict__ out, int64_t nRows,
+	unsigned long long* __restrict__ nnz) {
+	extern __shared__ double tbl[];
+	constexpr int NB = Q1_NB;
+	const int tid = threadIdx.x;
+	const int64_t row0 = ((int64_t) blockIdx.x * THREADS + tid) * RPT;
+	const bool full = row0 + RPT <= nRows;
+	const bool any = row0 < nRows;
+	const uint8_t* myCodes = arena + (size_t) row0 * CW;
+	double acc[RPT];
+#pragma unroll
+	for(int i = 0; i < RPT; i++) acc[i] = 0.0;
+	CodeVec<CW, RPT> ping[NB], pong[NB];
+	if(full) q1_load<CW, RPT, NB>(ping, myCodes, arenaStride, 0, nGroups - 1);
+
+	double stage[Q1_TPT];
+	int4 sl = slabs[0];
+	{
+		const int total = (sl.y - sl.x) * sl.z;
+#pragma unroll
+		for(int k = 0; k < Q1_TPT; k++) {
+			const int f = tid + k * THREADS;
+			stage[k] = f < total ? q1_table_value(T, tblOff, sl, f) : 0.0;
+		}
+		for(int i = tid; i < sl.z; i += THREADS) tbl[i] = 0.0; // slot 0: zero table
+	}
 
 	for(int s = 0; s < nSlabs; s++) {
-		const int g0 = slabStart[s], g1 = slabStart[s + 1];
-		const int t0 = groups[g0].tblOff;
-		const int t1 = groups[g1 - 1].tblOff + groups[g1 - 1].nVals;
-		__syncthreads();
-		for(int i = tid; i < t1 - t0; i += THREADS) tbl[i] = T[t0 + i];
-		__syncthreads();
-		if(full) {
-			int g = g0;
-			for(; g + NB <= g1; g += NB) {
-				CodeVec<CW> cv[NB];
+		const int g0 = sl.x, g1 = sl.y, tstride = sl.z;
+		const int nIn = g1 - g0;
+		__syncthreads(); // everyone is done with the previous slab's tables
+		{
+			const int total = nIn * tstride;
 #pragma unroll
-				for(int j = 0; j < NB; j++) cv[j].load(groups[g + j].codes, row0);
-#pragma unroll
-				for(int j = 0; j < NB; j++) {
-					const double* t = tbl + (groups[g + j].tblOff - t0);
-#pragma unroll
-					for(int i = 0; i < Q1_RPT; i++) acc[i] += t[cv[j].get(i)];
-				}
+			for(int k = 0; k < Q1_TPT; k++) {
+				const int f = tid + k * THREADS;
+				if(f < total) tbl[tstride + f] = stage[k];
 			}
-			for(; g < g1; g++) {
-				CodeVec<CW> cv;
-				cv.load(groups[g].codes, row0);
-				const double* t = tbl + (groups[g].tblOff - t0);
+		}
+		__syncthreads();
+		if(s + 1 < nSlabs) {
+			sl = slabs[s + 1];
+			const int total = (sl.y - sl.x) * sl.z;
 #pragma unroll
-				for(int i = 0; i < Q1_RPT; i++) acc[i] += t[cv.get(i)];
+			for(int k = 0; k < Q1_TPT; k++) {
+				const int f = tid + k * THREADS;
+				stage[k] = f < total ? q1_table_value(T, tblOff, sl, f) : 0.0;
+			}
+		}
+		if(full) {
+			for(int g = g0; g < g1; g += 2 * NB) {
+				q1_load<CW, RPT, NB>(pong, myCodes, arenaStride, g + NB, nGroups - 1);
+				q1_consume<CW, RPT, NB>(ping, tbl, tstride, g - g0, nIn, acc);
+				q1_load<CW, RPT, NB>(ping, myCodes, arenaStride, g + 2 * NB, nGroups - 1);
+				q1_consume<CW, RPT, NB>(pong, tbl, tstride, g - g0 + NB, nIn, acc);
 			}
 		}
 		else if(any) {
 			for(int g = g0; g < g1; g++) {
-				const double* t = tbl + (groups[g].tblOff - t0);
-				const void* codes = groups[g].codes;
+				const double* t = tbl + (size_t) (g - g0 + 1) * tstride;
+				const uint8_t* codes = arena + (size_t) g * arenaStride;
 #pragma unroll
-				for(int i = 0; i < Q1_RPT; i++)
+				for(int i = 0; i < RPT; i++)
 					if(row0 + i < nRows) acc[i] += t[load_code(codes, CW, row0 + i)];
 			}
 		}
@@ -146,21 +217,119 @@ __global__ __launch_bounds__(THREADS) void k_rmm_q1_ddc(const DGroup* __restrict
 
 	int cnt = 0;
 	if(any) {
-		const double cadd = constIdx >= 0 ? T[constIdx] : 0.0;
 		if(constIdx >= 0) {
+			const double cadd = T[constIdx];
 #pragma unroll
-			for(int i = 0; i < Q1_RPT; i++) acc[i] += cadd;
+			for(int i = 0; i < RPT; i++) acc[i] += cadd;
 		}
 		if(full) {
 #pragma unroll
-			for(int i = 0; i < Q1_RPT; i += 2) {
+			for(int i = 0; i < RPT; i += 2) {
 				cnt += (acc[i] != 0.0) + (acc[i + 1] != 0.0);
-				*(double2*) (out + row0 + i) = make_double2(acc[i], acc[i + 1]);
+				f64x2 v2;
+				v2.x = acc[i]; v2.y = acc[i + 1];
+				__builtin_nontemporal_store(v2, (f64x2*) (out + row0 + i));
 			}
 		}
 		else {
 #pragma unroll
-			for(int i = 0; i < Q1_RPT; i++)
+			for(int i = 0; i < RPT; i++)
+				if(row0 + i < nRows) { cnt += acc[i] != 0.0; out[row0 + i] = acc[i]; }
+		}
+	}
+	count_add(nnz, cnt);
+}
+
+// ---------------------------------------------------------------------------
+// K2 (mat-vec), byte codes: all groups DDC with uint8 codes (nVals <= 256).
+// Same scheme as k_rmm_q1_ddc, specialised so that the hot loop carries no
+// address arithmetic beyond code*8: every table has the fixed LDS stride of 256
+// doubles, slabs hold U8_PER groups and the loop over the slab is fully unrolled,
+// which turns every table base into an immediate offset of the LDS read.
+// Slots of a short last slab are zero-filled (x + 0.0 leaves the sum unchanged).
+// ---------------------------------------------------------------------------
+constexpr int U8_PER = 16;   // groups (tables) per slab: 16 x 2 KiB = 32 KiB of LDS
+constexpr int U8_NB = 4;     // groups per load batch
+constexpr int U8_RPT = 16;   // rows per thread = one 16-byte load per group
+
+template <int THREADS>
+__global__ __launch_bounds__(THREADS) void k_rmm_q1_u8(const uint8_t* __restrict__ arena, size_t arenaStride,
+	int nGroups, const int32_t* __restrict__ tblOff, const double* __restrict__ T, int constIdx,
+	double* __restrict__ out, int64_t nRows, unsigned long long* __restrict__ nnz) {
+	__shared__ double tbl[U8_PER * 256];
+	const char* tb = (const char*) tbl;
+	constexpr int RPT = U8_RPT, NB = U8_NB;
+	const int tid = threadIdx.x;
+	const int64_t row0 = ((int64_t) blockIdx.x * THREADS + tid) * RPT;
+	const bool full = row0 + RPT <= nRows;
+	const bool any = row0 < nRows;
+	const uint8_t* myCodes = arena + (size_t) row0;
+	double acc[RPT];
+#pragma unroll
+	for(int i = 0; i < RPT; i++) acc[i] = 0.0;
+	CodeVec<1, RPT> ping[NB], pong[NB];
+	if(full) q1_load<1, RPT, NB>(ping, myCodes, arenaStride, 0, nGroups - 1);
+
+	for(int g0 = 0; g0 < nGroups; g0 += U8_PER) {
+		const int nIn = min(U8_PER, nGroups - g0);
+		__syncthreads();
+		for(int f = tid; f < U8_PER * 256; f += THREADS) {
+			const int g = f >> 8, i = f & 255;
+			double v = 0.0;
+			if(g < nIn) {
+				const int o = tblOff[g0 + g], n = tblOff[g0 + g + 1] - o;
+				if(i < n) v = T[o + i];
+			}
+			tbl[f] = v;
+		}
+		__syncthreads();
+		if(full) {
+#pragma unroll
+			for(int s = 0; s < U8_PER; s += 2 * NB) {
+				q1_load<1, RPT, NB>(pong, myCodes, arenaStride, g0 + s + NB, nGroups - 1);
+#pragma unroll
+				for(int j = 0; j < NB; j++) {
+#pragma unroll
+					for(int i = 0; i < RPT; i++) acc[i] += *(const double*) (tb + (s + j) * 2048 + (ping[j].get(i) << 3));
+				}
+				q1_load<1, RPT, NB>(ping, myCodes, arenaStride, g0 + s + 2 * NB, nGroups - 1);
+#pragma unroll
+				for(int j = 0; j < NB; j++) {
+#pragma unroll
+					for(int i = 0; i < RPT; i++)
+						acc[i] += *(const double*) (tb + (s + NB + j) * 2048 + (pong[j].get(i) << 3));
+				}
+			}
+		}
+		else if(any) {
+			for(int g = 0; g < nIn; g++) {
+				const uint8_t* codes = arena + (size_t) (g0 + g) * arenaStride;
+#pragma unroll
+				for(int i = 0; i < RPT; i++)
+					if(row0 + i < nRows) acc[i] += tbl[g * 256 + codes[row0 + i]];
+			}
+		}
+	}
+
+	int cnt = 0;
+	if(any) {
+		if(constIdx >= 0) {
+			const double cadd = T[constIdx];
+#pragma unroll
+			for(int i = 0; i < RPT; i++) acc[i] += cadd;
+		}
+		if(full) {
+#pragma unroll
+			for(int i = 0; i < RPT; i += 2) {
+				cnt += (acc[i] != 0.0) + (acc[i + 1] != 0.0);
+				f64x2 v2;
+				v2.x = acc[i]; v2.y = acc[i + 1];
+				__builtin_nontemporal_store(v2, (f64x2*) (out + row0 + i));
+			}
+		}
+		else {
+#pragma unroll
+			for(int i = 0; i < RPT; i++)
 				if(row0 + i < nRows) { cnt += acc[i] != 0.0; out[row0 + i] = acc[i]; }
 		}
 	}
@@ -265,33 +434,46 @@ int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned lon
 	const int constRow = b->hasConst ? b->totalVals : -1;
 	if(nRows == 0) return 0;
 
-	bool allDdc = nG > 0;
-	int cw = nG > 0 ? b->groups[0].d.codeWidth : 0;
-	for(auto& g : b->groups)
-		if(g.d.type != G_DDC || g.d.codeWidth != cw) allDdc = false;
-
-	if(q == 1 && allDdc && b->slabLdsBytes > 0) {
-		constexpr int THREADS = 256;
-		const int64_t rowsPerBlock = (int64_t) THREADS * Q1_RPT;
+	if(q == 1 && b->dArena && b->arenaWidth == 1 && b->maxVals <= 256 && !getenv("CLA_Q1_GENERIC")) {
+		constexpr int THREADS = 512;
+		const int64_t rowsPerBlock = (int64_t) THREADS * U8_RPT;
 		const unsigned grid = (unsigned) ((nRows + rowsPerBlock - 1) / rowsPerBlock);
-		const int nSlabs = (int) b->slabStart.size() - 1;
-		const size_t lds = (size_t) b->slabLdsBytes;
-		double codeBytes = 0;
-		for(auto& g : b->groups) codeBytes += (double) nRows * g.d.codeWidth;
-		const double bytes = codeBytes + (double) nRows * 8 + (double) b->totalVals * 8;
-#define LAUNCH_Q1(CWV)                                                                                          \
+		const double bytes = (double) nRows * nG + (double) nRows * 8 + (double) b->totalVals * 8;
+		Prof pf(b, "k_rmm_q1_u8", grid, THREADS, U8_PER * 256 * 8, bytes);
+		hipLaunchKernelGGL(k_rmm_q1_u8<THREADS>, dim3(grid), dim3(THREADS), 0, st, b->dArena, b->arenaStride, nG,
+			b->dTblOff, b->dTables, constRow, dOut, nRows, dNnz);
+		CLA_HIP(hipGetLastError());
+		return 0;
+	}
+	if(q == 1 && b->dArena && b->q1LdsBytes > 0) {
+		const int cw = b->arenaWidth;
+		int threads = 256, rpt = cw == 4 ? 8 : 16;
+		if(const char* e = getenv("CLA_Q1_THREADS")) threads = atoi(e);
+		if(const char* e = getenv("CLA_Q1_RPT")) rpt = atoi(e);
+		if(cw == 4 && rpt > 16) rpt = 16;
+		const int64_t rowsPerBlock = (int64_t) threads * rpt;
+		const unsigned grid = (unsigned) ((nRows + rowsPerBlock - 1) / rowsPerBlock);
+		const int nSlabs = (int) b->q1Slabs.size();
+		const size_t lds = (size_t) b->q1LdsBytes;
+		const double bytes = (double) nRows * cw * nG + (double) nRows * 8 + (double) b->totalVals * 8;
+		Prof pf(b, "k_rmm_q1_ddc", grid, threads, (long) lds, bytes);
+#define LAUNCH_Q1(CWV, RPTV, THR)                                                                               \
 	do {                                                                                                        \
-		auto kern = k_rmm_q1_ddc<CWV, THREADS>;                                                                 \
+		auto kern = k_rmm_q1_ddc<CWV, RPTV, THR>;                                                               \
 		CLA_HIP(hipFuncSetAttribute((const void*) kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds)); \
-		hipLaunchKernelGGL(kern, dim3(grid), dim3(THREADS), lds, st, b->dGroups, b->dSlabStart, nSlabs,         \
-			b->dTables, constRow, dOut, nRows, dNnz);                                                           \
+		hipLaunchKernelGGL(kern, dim3(grid), dim3(THR), lds, st, b->dArena, b->arenaStride, nG, b->dQ1Slabs,    \
+			nSlabs, b->dTblOff, b->dTables, constRow, dOut, nRows, dNnz);                                       \
 	} while(0)
-		{
-			Prof pf(b, "k_rmm_q1_ddc", grid, THREADS, (long) lds, bytes);
-			if(cw == 1) LAUNCH_Q1(1);
-			else if(cw == 2) LAUNCH_Q1(2);
-			else LAUNCH_Q1(4);
-		}
+#define LAUNCH_Q1_T(CWV, RPTV)                                                   \
+	do {                                                                         \
+		if(threads == 512) LAUNCH_Q1(CWV, RPTV, 512);                            \
+		else if(threads == 1024) LAUNCH_Q1(CWV, RPTV, 1024);                     \
+		else LAUNCH_Q1(CWV, RPTV, 256);                                          \
+	} while(0)
+		if(cw == 1) { if(rpt == 8) LAUNCH_Q1_T(1, 8); else LAUNCH_Q1_T(1, 16); }
+		else if(cw == 2) { if(rpt == 8) LAUNCH_Q1_T(2, 8); else LAUNCH_Q1_T(2, 16); }
+		else { if(rpt == 8) LAUNCH_Q1_T(4, 8); else LAUNCH_Q1_T(4, 16); }
+#undef LAUNCH_Q1_T
 #undef LAUNCH_Q1
 		CLA_HIP(hipGetLastError());
 		return 0;
