@@ -4,9 +4,6 @@
 namespace cla {
 #define NOT_YET(name) do { set_error(name ": not implemented"); return -CLA_ERR_UNSUPPORTED; } while(0)
 int launch_decompress(cla_block*, double*, unsigned long long*) { NOT_YET("decompress"); }
-int launch_lmm(cla_block*, const double*, int, double*, unsigned long long*) { NOT_YET("lmm"); }
-int launch_preagg(cla_block*, int, const double*, int, double*) { NOT_YET("preagg"); }
 int launch_tsmm(cla_block*, double*, unsigned long long*) { NOT_YET("tsmm"); }
 int launch_cooc(cla_block*, int, int, unsigned long long*) { NOT_YET("cooc"); }
-int launch_mmchain(cla_block*, const double*, const double*, int, double*, unsigned long long*) { NOT_YET("mmchain"); }
 }

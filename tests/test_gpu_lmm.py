@@ -1,0 +1,94 @@
+"""GPU parity of the left multiply (cla_lmm), pre-aggregation (cla_preagg) and the
+mm-chain (cla_mmchain) against the CPU oracle, through the C ABI."""
+import numpy as np
+import pytest
+
+from conftest import mixed_block
+from parity import assert_fp64_close
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("seed,n_rows", [(0, 1), (1, 37), (2, 3000), (3, 20011), (4, 200003)])
+@pytest.mark.parametrize("p", [1, 3])
+def test_mixed_groups_lmm(cla, ora, seed, n_rows, p):
+    specs, n_cols = mixed_block(seed, n_rows)
+    Y = np.random.default_rng(seed + 70).standard_normal((p, n_rows))
+    blk = cla.build_block(n_rows, n_cols, specs)
+    out, nnz = blk.lmm(Y)
+    blk.close()
+    ref, rnnz = ora.lmm(ora.Groups(specs, n_rows, n_cols), Y, 4)
+    D = ora.np_decompress(specs, n_rows, n_cols)
+    assert_fp64_close(out, ref, ora.abs_matmul(Y, D), what=f"lmm p={p}")
+    assert nnz == rnnz
+
+
+def test_c4_scaled_both_products(cla, ora):
+    """BASELINE config 4 at 1/50 scale (200,000 x 200 SDCZeros): t(v) %*% X and X %*% u."""
+    from systemds_amd import synth
+    c = synth.config4(scale=50)
+    n_rows, n_cols = c["n_rows"], c["n_cols"]
+    blk = cla.build_block(n_rows, n_cols, c["groups"])
+    G = ora.Groups(c["groups"], n_rows, n_cols)
+    D = ora.np_decompress(c["groups"], n_rows, n_cols)
+    out, nnz = blk.lmm(c["v"])
+    ref, rnnz = ora.lmm(G, c["v"], 4)
+    assert_fp64_close(out, ref, ora.abs_matmul(c["v"], D), what="C4 t(v)%*%X")
+    assert nnz == rnnz
+    out, nnz = blk.rmm(c["u"])
+    ref, rnnz = ora.rmm(G, c["u"], 4)
+    assert_fp64_close(out, ref, ora.abs_matmul(D, c["u"]), what="C4 X%*%u")
+    assert nnz == rnnz
+    blk.close()
+
+
+def test_c2_scaled_left_vector(cla, ora):
+    from systemds_amd import synth
+    c = synth.config2(scale=100, n_cols=40)
+    n_rows, n_cols = c["n_rows"], c["n_cols"]
+    y = np.random.default_rng(5).standard_normal((1, n_rows))
+    blk = cla.build_block(n_rows, n_cols, c["groups"])
+    out, nnz = blk.lmm(y)
+    blk.close()
+    ref, rnnz = ora.lmm(ora.Groups(c["groups"], n_rows, n_cols), y, 4)
+    D = ora.np_decompress(c["groups"], n_rows, n_cols)
+    assert_fp64_close(out, ref, ora.abs_matmul(y, D), what="C2 t(y)%*%X")
+    assert nnz == rnnz
+
+
+def test_preagg_per_group(cla, ora):
+    specs, n_cols = mixed_block(11, 30011, with_unc=False)
+    Y = np.random.default_rng(12).standard_normal((2, 30011))
+    blk = cla.build_block(30011, n_cols, specs)
+    G = ora.Groups(specs, 30011, n_cols)
+    gi = 0
+    for i, s in enumerate(specs):
+        if s.type in ("ddc", "sdc", "rle"):
+            pre = blk.preagg(gi, Y)
+            ref = ora.preaggregate_dense(G, i, Y)
+            scale = np.zeros_like(ref)
+            refabs = ora.preaggregate_dense(G, i, np.abs(Y))
+            assert_fp64_close(pre, ref, refabs + scale, what=f"preagg {s.type}")
+            # sum over bins = sum of Y over the rows the group covers
+            assert np.allclose(pre.sum(axis=1), ref.sum(axis=1), rtol=0, atol=1e-9)
+        if s.type not in ("const", "empty"):
+            gi += 1
+    blk.close()
+
+
+@pytest.mark.parametrize("ctype", [0, 1])
+def test_mmchain(cla, ora, ctype):
+    specs, n_cols = mixed_block(21, 40009)
+    rng = np.random.default_rng(22)
+    v, w = rng.standard_normal(n_cols), rng.standard_normal(40009)
+    blk = cla.build_block(40009, n_cols, specs)
+    out, nnz = blk.mmchain(v, w if ctype else None, ctype)
+    blk.close()
+    ref, rnnz = ora.mmchain(ora.Groups(specs, 40009, n_cols), v, w if ctype else None, ctype, 4)
+    D = ora.np_decompress(specs, 40009, n_cols)
+    inner = np.abs(D) @ np.abs(v)
+    if ctype:
+        inner = inner * np.abs(w)
+    scale = np.abs(D).T @ inner
+    assert_fp64_close(out, ref, scale, what="mmchain")
+    assert nnz == rnnz
