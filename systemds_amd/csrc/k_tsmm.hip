@@ -1,0 +1,542 @@
+// t(X) %*% X on a compressed block, integer co-occurrence and additive
+// decompression (gfx950).
+//
+//   tile_codes          materialises the per-row codes of one group for a tile of
+//                       SDC_TILE rows in LDS (-1 = row not covered): DDC direct,
+//                       RLE by run walk, SDCZeros from the row-tile index
+//   k_tsmm_pair         P[code_t(r), :] += dict_s[code_s(r), :] in LDS (the reference's
+//                       preAggregateThatIndexStructure), contracted with dict_t per block
+//   k_tsmm_self         counts x dict (x) dict, and column sums for the correction layer
+//   k_tsmm_dense        fallback: decode row tiles and accumulate the Gram matrix
+//   k_tsmm_finish       correction layer, mirror upper -> lower, non-zero count
+//   k_cooc_*            exact integer co-occurrence counts
+//   k_decompress_*      additive decompression into a dense block
+#include "../../include/cla_hip.h"
+#include "cla_device.hpp"
+
+namespace cla {
+
+constexpr int TT = SDC_TILE;      // rows per tile
+constexpr int TSMM_THREADS = 256; // 4 rows per thread per tile
+
+// Fills codes[0..TT) for rows [tile*TT, tile*TT+TT) of group G. All threads of the
+// block must call it; ends with a barrier.
+__device__ void tile_codes(const DGroup& G, int tile, int64_t nRows, int32_t* __restrict__ codes) {
+	const int64_t r0 = (int64_t) tile * TT;
+	const int tid = threadIdx.x;
+	if(G.type == G_DDC) {
+		for(int t = tid; t < TT; t += TSMM_THREADS) codes[t] = r0 + t < nRows ? load_code(G.codes, G.codeWidth, r0 + t) : -1;
+	}
+	else if(G.type == G_RLE) {
+		// each thread expands 4 consecutive rows from the merged run table
+		const int64_t rb = r0 + tid * 4;
+		if(rb < nRows) {
+			int j = rle_find(G.runStart, G.nRuns, (int32_t) rb);
+			for(int t = 0; t < 4; t++) {
+				const int64_t r = rb + t;
+				if(r >= nRows) { codes[tid * 4 + t] = -1; continue; }
+				while(G.runStart[j + 1] <= r) j++;
+				codes[tid * 4 + t] = G.runCode[j];
+			}
+		}
+		else
+			for(int t = 0; t < 4; t++) codes[tid * 4 + t] = -1;
+	}
+	else if(G.type == G_SDCZ) {
+		for(int t = tid; t < TT; t += TSMM_THREADS) codes[t] = -1;
+		__syncthreads();
+		if(G.nOffsets > 0) {
+			const int64_t rEnd = r0 + TT;
+			if(tid == 0 && G.first >= r0 && G.first < rEnd) codes[G.first - r0] = load_code(G.codes, G.codeWidth, 0);
+			// wave 0 walks the list from the tile's iterator state
+			if(tid < 64 && tile < G.nTiles) {
+				const OffState st = G.tileIdx[tile];
+				int32_t row = st.row, emit = st.emit;
+				int64_t i0 = st.idx;
+				while(i0 < G.nDeltas && row < rEnd) {
+					int32_t rows[4], didx[4];
+					unsigned mask;
+					if(G.deltaWidth == 1) sdc_decode256<1>(G.deltas, G.nDeltas, i0, row, emit, rows, didx, mask);
+					else sdc_decode256<2>(G.deltas, G.nDeltas, i0, row, emit, rows, didx, mask);
+#pragma unroll
+					for(int k = 0; k < 4; k++)
+						if((mask & (1u << k)) && rows[k] < rEnd && rows[k] >= r0)
+							codes[rows[k] - r0] = load_code(G.codes, G.codeWidth, didx[k]);
+					i0 += 256;
+				}
+			}
+		}
+	}
+	else {
+		for(int t = tid; t < TT; t += TSMM_THREADS) codes[t] = -1;
+	}
+	__syncthreads();
+}
+
+__device__ __forceinline__ void add_upper_atomic(double* out, int nCols, int row, int col, double v) {
+	// DictLibMatrixMult.addToUpperTriangle: lower-triangle cells are mirrored, a
+	// diagonal cell (only reachable with overlapping groups) receives the value twice
+	if(row == col) unsafeAtomicAdd(&out[(size_t) row * nCols + col], v + v);
+	else if(row > col) unsafeAtomicAdd(&out[(size_t) col * nCols + row], v);
+	else unsafeAtomicAdd(&out[(size_t) row * nCols + col], v);
+}
+
+// ---------------------------------------------------------------------------
+// Pair term. `t` = target group (its codes select the accumulator row), `s` =
+// source group (its dictionary tuples are accumulated). LDS: P[nVals_t x nC_s],
+// optionally a copy of dict_s, and the two code tiles. Each block owns a
+// contiguous range of tiles, then contracts t(dict_t) . P and adds the
+// nC_t x nC_s result into the upper triangle.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(TSMM_THREADS) void k_tsmm_pair(const DGroup* __restrict__ groups,
+	const int4* __restrict__ pairs, int64_t nRows, int tilesPerBlock, double* __restrict__ out, int nCols) {
+	extern __shared__ double smem[];
+	const int4 pr = pairs[blockIdx.y]; // (target, source, dictInLds, 0)
+	const DGroup& Gt = groups[pr.x];
+	const DGroup& Gs = groups[pr.y];
+	const int dictInLds = pr.z;
+	const int nCs = Gs.nColG, nCt = Gt.nColG;
+	double* P = smem;                                             // nVals_t * nCs
+	double* dS = P + (size_t) Gt.nVals * nCs;                      // nVals_s * nCs (optional)
+	int32_t* ca = (int32_t*) (dS + (dictInLds ? (size_t) Gs.nVals * nCs : 0));
+	int32_t* cb = ca + TT;
+	const int tid = threadIdx.x;
+	for(int i = tid; i < Gt.nVals * nCs; i += TSMM_THREADS) P[i] = 0.0;
+	if(dictInLds)
+		for(int i = tid; i < Gs.nVals * nCs; i += TSMM_THREADS) dS[i] = Gs.dict[i];
+	const double* dsrc = dictInLds ? dS : Gs.dict;
+	const int nTiles = (int) ((nRows + TT - 1) / TT);
+	const int t0 = blockIdx.x * tilesPerBlock, t1 = min(t0 + tilesPerBlock, nTiles);
+	__syncthreads();
+	for(int tile = t0; tile < t1; tile++) {
+		tile_codes(Gt, tile, nRows, ca);
+		tile_codes(Gs, tile, nRows, cb);
+		for(int t = tid; t < TT; t += TSMM_THREADS) {
+			const int a = ca[t], c = cb[t];
+			if(a >= 0 && c >= 0) {
+				const double* v = dsrc + (size_t) c * nCs;
+				double* p = P + (size_t) a * nCs;
+				for(int j = 0; j < nCs; j++) unsafeAtomicAdd(&p[j], v[j]);
+			}
+		}
+		__syncthreads();
+	}
+	// contraction: S[i, j] = sum_a dict_t[a, i] * P[a, j]
+	__shared__ double red[4];
+	for(int i = 0; i < nCt; i++)
+		for(int j = 0; j < nCs; j++) {
+			double s = 0.0;
+			for(int a = tid; a < Gt.nVals; a += TSMM_THREADS) s += Gt.dict[(size_t) a * nCt + i] * P[(size_t) a * nCs + j];
+			s = wave_sum_f64(s);
+			if((tid & 63) == 0) red[tid >> 6] = s;
+			__syncthreads();
+			if(tid == 0) add_upper_atomic(out, nCols, Gt.cols[i], Gs.cols[j], red[0] + red[1] + red[2] + red[3]);
+			__syncthreads();
+		}
+}
+
+// Self term (AColGroupCompressed.tsmmDense) + column sums of the group:
+// out[cols[i], cols[j]] += sum_k cnt[k] d[k,i] d[k,j], j >= i; colSum[cols[j]] += sum_k cnt[k] d[k,j]
+__global__ __launch_bounds__(256) void k_tsmm_self(const DGroup* __restrict__ groups, int g, const int32_t* __restrict__ counts,
+	double* __restrict__ out, int nCols, double* __restrict__ colSum) {
+	__shared__ double red[4];
+	const DGroup& G = groups[g];
+	const int nC = G.nColG, tid = threadIdx.x;
+	for(int i = 0; i < nC; i++) {
+		for(int j = i; j <= nC; j++) { // j == nC: column sum of column i
+			double s = 0.0;
+			for(int k = tid; k < G.nVals; k += 256) {
+				const double v = G.dict[(size_t) k * nC + i] * (double) counts[k];
+				s += j < nC ? v * G.dict[(size_t) k * nC + j] : v;
+			}
+			s = wave_sum_f64(s);
+			if((tid & 63) == 0) red[tid >> 6] = s;
+			__syncthreads();
+			if(tid == 0) {
+				const double tot = red[0] + red[1] + red[2] + red[3];
+				if(j < nC) {
+					const int r = G.cols[i], c = G.cols[j];
+					unsafeAtomicAdd(&out[(size_t) min(r, c) * nCols + max(r, c)], tot);
+				}
+				else
+					unsafeAtomicAdd(&colSum[G.cols[i]], tot);
+			}
+			__syncthreads();
+		}
+	}
+}
+
+// ---------------------------------------------------------------------------
+// Dense fallback (any uncompressed group, or at least as many groups as columns):
+// decode DT rows into LDS and accumulate the upper triangle of t(D) %*% D.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void k_tsmm_dense(const DGroup* __restrict__ groups, int nGroups,
+	const double* __restrict__ constV, int64_t nRows, int nCols, int DT, int tilesPerBlock, double* __restrict__ out) {
+	extern __shared__ double D[]; // DT x nCols
+	const int tid = threadIdx.x;
+	const int nPairs = nCols * (nCols + 1) / 2;
+	const int64_t nTiles = (nRows + DT - 1) / DT;
+	const int64_t t0 = (int64_t) blockIdx.x * tilesPerBlock, t1 = min(t0 + tilesPerBlock, nTiles);
+	// pairs owned by this thread (strided), partial sums kept in registers for up to 8 pairs
+	constexpr int MAXP = 24;
+	double acc[MAXP];
+#pragma unroll
+	for(int k = 0; k < MAXP; k++) acc[k] = 0.0;
+	for(int64_t tile = t0; tile < t1; tile++) {
+		const int64_t r0 = tile * DT;
+		const int nr = (int) min((int64_t) DT, nRows - r0);
+		for(int i = tid; i < DT * nCols; i += 256) D[i] = (i / nCols) < nr ? constV[i % nCols] : 0.0;
+		__syncthreads();
+		for(int g = 0; g < nGroups; g++) {
+			const DGroup& G = groups[g];
+			if(G.type == G_DDC || G.type == G_RLE) {
+				for(int t = tid; t < nr; t += 256) {
+					const int64_t r = r0 + t;
+					const int code = G.type == G_DDC ? load_code(G.codes, G.codeWidth, r)
+					                                 : G.runCode[rle_find(G.runStart, G.nRuns, (int32_t) r)];
+					if(code >= 0)
+						for(int j = 0; j < G.nColG; j++) D[t * nCols + G.cols[j]] += G.dict[(size_t) code * G.nColG + j];
+				}
+			}
+			else if(G.type == G_UNC) {
+				for(int t = tid; t < nr * G.nColG; t += 256) {
+					const int rr = t / G.nColG, j = t - rr * G.nColG;
+					D[rr * nCols + G.cols[j]] += G.dense[(size_t) (r0 + rr) * G.nColG + j];
+				}
+			}
+			else if(G.type == G_SDCZ && G.nOffsets > 0) {
+				// thread 0.. walk: rows of the list inside [r0, r0+nr) via the coarse tile index
+				if(tid < 64) {
+					const int64_t rEnd = r0 + nr;
+					if(tid == 0 && G.first >= r0 && G.first < rEnd) {
+						const int code = load_code(G.codes, G.codeWidth, 0);
+						for(int j = 0; j < G.nColG; j++) D[(G.first - r0) * nCols + G.cols[j]] += G.dict[(size_t) code * G.nColG + j];
+					}
+					const int ti = (int) (r0 / SDC_TILE);
+					if(ti < G.nTiles) {
+						const OffState st = G.tileIdx[ti];
+						int32_t row = st.row, emit = st.emit;
+						int64_t i0 = st.idx;
+						while(i0 < G.nDeltas && row < rEnd) {
+							int32_t rows[4], didx[4];
+							unsigned mask;
+							if(G.deltaWidth == 1) sdc_decode256<1>(G.deltas, G.nDeltas, i0, row, emit, rows, didx, mask);
+							else sdc_decode256<2>(G.deltas, G.nDeltas, i0, row, emit, rows, didx, mask);
+#pragma unroll
+							for(int k = 0; k < 4; k++)
+								if((mask & (1u << k)) && rows[k] >= r0 && rows[k] < rEnd) {
+									const int code = load_code(G.codes, G.codeWidth, didx[k]);
+									for(int j = 0; j < G.nColG; j++)
+										D[(rows[k] - r0) * nCols + G.cols[j]] += G.dict[(size_t) code * G.nColG + j];
+								}
+							i0 += 256;
+						}
+					}
+				}
+			}
+			__syncthreads();
+		}
+		int slot = 0;
+		for(int pr = tid; pr < nPairs && slot < MAXP; pr += 256, slot++) {
+			// pair index -> (i, j), j >= i
+			int i = 0, rem = pr;
+			while(rem >= nCols - i) { rem -= nCols - i; i++; }
+			const int j = i + rem;
+			double s = 0.0;
+			for(int t = 0; t < nr; t++) s += D[t * nCols + i] * D[t * nCols + j];
+			acc[slot] += s;
+		}
+		__syncthreads();
+	}
+	int slot = 0;
+	for(int pr = tid; pr < nPairs && slot < MAXP; pr += 256, slot++) {
+		int i = 0, rem = pr;
+		while(rem >= nCols - i) { rem -= nCols - i; i++; }
+		const int j = i + rem;
+		if(acc[slot] != 0.0) unsafeAtomicAdd(&out[(size_t) i * nCols + j], acc[slot]);
+	}
+}
+
+// correction layer (CLALibTSMM.addCorrectionLayer), mirror, nnz; single block
+__global__ __launch_bounds__(256) void k_tsmm_finish(double* __restrict__ out, int nCols, const double* __restrict__ constV,
+	const double* __restrict__ colSum, double nRowsD, int applyCorrection, unsigned long long* __restrict__ nnz) {
+	int cnt = 0;
+	for(int idx = threadIdx.x + blockIdx.x * 256; idx < nCols * nCols; idx += 256 * gridDim.x) {
+		const int i = idx / nCols, j = idx - i * nCols;
+		if(j < i) continue;
+		double v = out[idx];
+		if(applyCorrection) {
+			const double v1l = constV[i];
+			const double v2l = colSum[i] + constV[i] * nRowsD;
+			v += v1l * colSum[j] + v2l * constV[j];
+		}
+		out[idx] = v;
+		out[(size_t) j * nCols + i] = v;
+		cnt += v != 0.0 ? (i == j ? 1 : 2) : 0;
+	}
+	count_add(nnz, cnt);
+}
+
+int launch_tsmm(cla_block* b, double* dOut, unsigned long long* dNnz) {
+	const int nG = (int) b->groups.size();
+	const int nCols = b->nCols;
+	const int64_t nRows = b->nRows;
+	hipStream_t st = b->stream;
+	clear_stats(b);
+	CLA_HIP(hipMemsetAsync(dOut, 0, sizeof(double) * (size_t) nCols * nCols, st));
+	CLA_HIP(hipMemsetAsync(dNnz, 0, sizeof(unsigned long long), st));
+	// overlapping column groups need the diagonal doubling of addToUpperTriangle in
+	// every kernel; reject instead (the caller falls back)
+	{
+		std::vector<char> seen((size_t) nCols, 0);
+		for(auto& g : b->groups)
+			for(int c : g.cols) {
+				if(seen[c]) { set_error("tsmm: overlapping column groups are not supported"); return -CLA_ERR_UNSUPPORTED; }
+				seen[c] = 1;
+			}
+	}
+	int rc;
+	const bool dense = nG >= nCols || b->hasUnc;
+	if(dense) {
+		// t(D) %*% D of the decoded rows, constants included (no correction layer needed)
+		int DT = 256;
+		while(DT > 8 && (size_t) DT * nCols * 8 > (size_t) 96 * 1024) DT /= 2;
+		if((size_t) DT * nCols * 8 > (size_t) 96 * 1024 || (int64_t) nCols * (nCols + 1) / 2 > 24 * 256) {
+			set_error("tsmm: dense fallback supports at most 110 columns (block has %d)", nCols);
+			return -CLA_ERR_UNSUPPORTED;
+		}
+		if(DT > SDC_TILE) DT = SDC_TILE;
+		const int64_t nTiles = (nRows + DT - 1) / DT;
+		int tpb = 1;
+		while(nTiles / tpb > (int64_t) g_numCU * 16) tpb *= 2;
+		const unsigned grid = (unsigned) std::max<int64_t>((nTiles + tpb - 1) / tpb, 1);
+		const size_t lds = (size_t) DT * nCols * 8;
+		if(nRows > 0) {
+			Prof pf(b, "k_tsmm_dense", grid, 256, (long) lds, 0);
+			CLA_HIP(hipFuncSetAttribute((const void*) k_tsmm_dense, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
+			hipLaunchKernelGGL(k_tsmm_dense, dim3(grid), dim3(256), lds, st, b->dGroups, nG, b->dConstV, nRows, nCols, DT,
+				tpb, dOut);
+		}
+		Prof pf(b, "k_tsmm_finish", 1, 256, 0, 0);
+		hipLaunchKernelGGL(k_tsmm_finish, dim3(1), dim3(256), 0, st, dOut, nCols, b->dConstV, b->dConstV, (double) nRows, 0, dNnz);
+		CLA_HIP(hipGetLastError());
+		return 0;
+	}
+
+	// scratch: counts (maxVals int32) | colSum (nCols doubles)
+	const size_t cntBytes = ((size_t) std::max(b->maxVals, 1) * 4 + 255) & ~(size_t) 255;
+	if((rc = ensure_scratch(b, cntBytes + sizeof(double) * (size_t) nCols))) return rc;
+	int32_t* dCounts = (int32_t*) b->dScratch;
+	double* dColSum = (double*) ((char*) b->dScratch + cntBytes);
+	CLA_HIP(hipMemsetAsync(dColSum, 0, sizeof(double) * (size_t) nCols, st));
+	for(int g = 0; g < nG; g++) {
+		if((rc = launch_counts(b, g, dCounts))) return rc;
+		Prof pf(b, "k_tsmm_self", 1, 256, 0, 0);
+		hipLaunchKernelGGL(k_tsmm_self, dim3(1), dim3(256), 0, st, b->dGroups, g, dCounts, dOut, nCols, dColSum);
+	}
+	const int nTiles = (int) ((nRows + TT - 1) / TT);
+	std::vector<int4> pairs;
+	size_t ldsMax = 0;
+	for(int g = 0; g < nG && nRows > 0; g++)
+		for(int h = g + 1; h < nG; h++) {
+			const DGroup& A = b->groups[g].d;
+			const DGroup& B = b->groups[h].d;
+			// target = side with the smaller accumulator nVals_t * nC_s
+			const bool gTarget = (size_t) A.nVals * B.nColG <= (size_t) B.nVals * A.nColG;
+			const int gt = gTarget ? g : h, gs = gTarget ? h : g;
+			const DGroup& T = b->groups[gt].d;
+			const DGroup& S = b->groups[gs].d;
+			const size_t pBytes = (size_t) T.nVals * S.nColG * 8;
+			const size_t dBytes = (size_t) S.nVals * S.nColG * 8;
+			const size_t cBytes = (size_t) 2 * TT * 4;
+			if(pBytes + cBytes > (size_t) 150 * 1024) {
+				set_error("tsmm: pre-aggregate of groups %d,%d needs %zu bytes of LDS", gt, gs, pBytes);
+				return -CLA_ERR_UNSUPPORTED;
+			}
+			const int dictInLds = pBytes + dBytes + cBytes <= (size_t) 150 * 1024;
+			ldsMax = std::max(ldsMax, pBytes + (dictInLds ? dBytes : 0) + cBytes);
+			pairs.push_back(make_int4(gt, gs, dictInLds, 0));
+		}
+	if(!pairs.empty()) {
+		int4* dPairs = nullptr;
+		CLA_HIP(hipMalloc((void**) &dPairs, sizeof(int4) * pairs.size()));
+		CLA_HIP(hipMemcpyAsync(dPairs, pairs.data(), sizeof(int4) * pairs.size(), hipMemcpyHostToDevice, st));
+		// blocks per pair: fill the machine about 8x over all pairs, but keep at least 64 tiles per block
+		const int64_t want = std::max<int64_t>(1, (int64_t) g_numCU * 8 / (int64_t) pairs.size());
+		int bpp = (int) std::min<int64_t>(want, std::max(1, nTiles / 64));
+		const int tpb = (nTiles + bpp - 1) / bpp;
+		bpp = (nTiles + tpb - 1) / tpb;
+		double codeBytes = 0;
+		for(auto& pr : pairs) {
+			const DGroup& T = b->groups[pr.x].d;
+			const DGroup& S = b->groups[pr.y].d;
+			codeBytes += (double) nRows * ((T.type == G_DDC ? T.codeWidth : 0) + (S.type == G_DDC ? S.codeWidth : 0));
+		}
+		{
+			Prof pf(b, "k_tsmm_pair", (long) bpp * (long) pairs.size(), TSMM_THREADS, (long) ldsMax, codeBytes);
+			CLA_HIP(hipFuncSetAttribute((const void*) k_tsmm_pair, hipFuncAttributeMaxDynamicSharedMemorySize, (int) ldsMax));
+			hipLaunchKernelGGL(k_tsmm_pair, dim3(bpp, (unsigned) pairs.size()), dim3(TSMM_THREADS), ldsMax, st, b->dGroups,
+				dPairs, nRows, tpb, dOut, nCols);
+		}
+		CLA_HIP(hipStreamSynchronize(st));
+		CLA_HIP(hipFree(dPairs));
+	}
+	{
+		Prof pf(b, "k_tsmm_finish", 1, 256, 0, 0);
+		hipLaunchKernelGGL(k_tsmm_finish, dim3(1), dim3(256), 0, st, dOut, nCols, b->dConstV, dColSum, (double) nRows,
+			b->hasConst ? 1 : 0, dNnz);
+	}
+	CLA_HIP(hipGetLastError());
+	return 0;
+}
+
+// ---------------------------------------------------------------------------
+// Exact integer co-occurrence N[a, b] = #{r : code_A(r) = a, code_B(r) = b}.
+// 64-bit bins in HBM updated with integer atomics; block-private 32-bit bins in
+// LDS first when the whole table fits.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(TSMM_THREADS) void k_cooc(const DGroup* __restrict__ groups, int ga, int gb, int64_t nRows,
+	int tilesPerBlock, int useLds, unsigned long long* __restrict__ N) {
+	extern __shared__ unsigned int lbins[];
+	__shared__ int32_t ca[TT], cb[TT];
+	const DGroup& A = groups[ga];
+	const DGroup& B = groups[gb];
+	const int tid = threadIdx.x;
+	const int nBins = A.nVals * B.nVals;
+	if(useLds) {
+		for(int i = tid; i < nBins; i += TSMM_THREADS) lbins[i] = 0;
+		__syncthreads();
+	}
+	const int nTiles = (int) ((nRows + TT - 1) / TT);
+	const int t0 = blockIdx.x * tilesPerBlock, t1 = min(t0 + tilesPerBlock, nTiles);
+	for(int tile = t0; tile < t1; tile++) {
+		tile_codes(A, tile, nRows, ca);
+		tile_codes(B, tile, nRows, cb);
+		for(int t = tid; t < TT; t += TSMM_THREADS) {
+			const int a = ca[t], c = cb[t];
+			if(a >= 0 && c >= 0) {
+				if(useLds) atomicAdd(&lbins[a * B.nVals + c], 1u);
+				else atomicAdd(&N[(size_t) a * B.nVals + c], 1ull);
+			}
+		}
+		__syncthreads();
+	}
+	if(useLds)
+		for(int i = tid; i < nBins; i += TSMM_THREADS)
+			if(lbins[i]) atomicAdd(&N[i], (unsigned long long) lbins[i]);
+}
+
+int launch_cooc(cla_block* b, int gA, int gB, unsigned long long* dOut) {
+	const DGroup& A = b->groups[gA].d;
+	const DGroup& B = b->groups[gB].d;
+	if(A.type == G_UNC || B.type == G_UNC) { set_error("cooc: uncompressed groups have no codes"); return -CLA_ERR_UNSUPPORTED; }
+	clear_stats(b);
+	const size_t nBins = (size_t) A.nVals * B.nVals;
+	CLA_HIP(hipMemsetAsync(dOut, 0, nBins * sizeof(unsigned long long), b->stream));
+	if(b->nRows == 0) return 0;
+	const int nTiles = (int) ((b->nRows + TT - 1) / TT);
+	const int useLds = nBins * 4 <= (size_t) 48 * 1024;
+	int tpb = std::max(1, nTiles / (g_numCU * 4));
+	const unsigned grid = (unsigned) ((nTiles + tpb - 1) / tpb);
+	const size_t lds = useLds ? nBins * 4 : 0;
+	Prof pf(b, "k_cooc", grid, TSMM_THREADS, (long) lds, 0);
+	hipLaunchKernelGGL(k_cooc, dim3(grid), dim3(TSMM_THREADS), lds, b->stream, b->dGroups, gA, gB, b->nRows, tpb, useLds,
+		dOut);
+	CLA_HIP(hipGetLastError());
+	return 0;
+}
+
+// ---------------------------------------------------------------------------
+// Additive decompression: out[r, c] = constV[c] + sum over groups covering c.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void k_decompress_fill(double* __restrict__ out, int64_t n, int nCols,
+	const double* __restrict__ constV) {
+	for(int64_t i = (int64_t) blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t) gridDim.x * 256) out[i] = constV[i % nCols];
+}
+
+__global__ __launch_bounds__(256) void k_decompress_rows(const DGroup* __restrict__ groups, int g, int64_t nRows, int nCols,
+	double* __restrict__ out) {
+	const DGroup& G = groups[g];
+	const int64_t idx = (int64_t) blockIdx.x * 256 + threadIdx.x;
+	if(idx >= nRows * G.nColG) return;
+	const int64_t r = idx / G.nColG;
+	const int j = (int) (idx - r * G.nColG);
+	double v;
+	if(G.type == G_UNC) v = G.dense[idx];
+	else {
+		const int code = G.type == G_DDC ? load_code(G.codes, G.codeWidth, r) : G.runCode[rle_find(G.runStart, G.nRuns, (int32_t) r)];
+		if(code < 0) return;
+		v = G.dict[(size_t) code * G.nColG + j];
+	}
+	unsafeAtomicAdd(&out[(size_t) r * nCols + G.cols[j]], v);
+}
+
+template <int W>
+__global__ __launch_bounds__(256) void k_decompress_sdc(const DGroup* __restrict__ groups, int g, int nCols,
+	double* __restrict__ out) {
+	const DGroup& G = groups[g];
+	const int chunk = blockIdx.x, wave = threadIdx.x >> 6;
+	if(chunk == 0 && threadIdx.x == 0 && G.nOffsets > 0) {
+		const int code = load_code(G.codes, G.codeWidth, 0);
+		for(int j = 0; j < G.nColG; j++) unsafeAtomicAdd(&out[(size_t) G.first * nCols + G.cols[j]], G.dict[(size_t) code * G.nColG + j]);
+	}
+	if(chunk >= G.nCkpt) return;
+	const OffState st = G.ckpt[chunk];
+	int32_t row = st.row, emit = st.emit;
+	int32_t rows[4], didx[4];
+	unsigned mask;
+	const int64_t base = (int64_t) chunk * SDC_CK;
+	for(int w = 0; w < wave; w++) sdc_decode256<W>(G.deltas, G.nDeltas, base + w * 256, row, emit, rows, didx, mask);
+	sdc_decode256<W>(G.deltas, G.nDeltas, base + wave * 256, row, emit, rows, didx, mask);
+#pragma unroll
+	for(int k = 0; k < 4; k++)
+		if(mask & (1u << k)) {
+			const int code = load_code(G.codes, G.codeWidth, didx[k]);
+			for(int j = 0; j < G.nColG; j++)
+				unsafeAtomicAdd(&out[(size_t) rows[k] * nCols + G.cols[j]], G.dict[(size_t) code * G.nColG + j]);
+		}
+}
+
+__global__ __launch_bounds__(256) void k_count_nnz2(const double* __restrict__ x, int64_t n, unsigned long long* __restrict__ nnz) {
+	int cnt = 0;
+	for(int64_t i = (int64_t) blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t) gridDim.x * 256) cnt += x[i] != 0.0;
+	count_add(nnz, cnt);
+}
+
+int launch_decompress(cla_block* b, double* dOut, unsigned long long* dNnz) {
+	const int nG = (int) b->groups.size();
+	const int64_t nRows = b->nRows, n = nRows * b->nCols;
+	hipStream_t st = b->stream;
+	clear_stats(b);
+	CLA_HIP(hipMemsetAsync(dNnz, 0, sizeof(unsigned long long), st));
+	if(n == 0) return 0;
+	const unsigned fg = (unsigned) std::min<int64_t>((n + 255) / 256, (int64_t) g_numCU * 64);
+	{
+		Prof pf(b, "k_decompress_fill", fg, 256, 0, 0);
+		hipLaunchKernelGGL(k_decompress_fill, dim3(fg), dim3(256), 0, st, dOut, n, b->nCols, b->dConstV);
+	}
+	for(int g = 0; g < nG; g++) {
+		const DGroup& G = b->groups[g].d;
+		if(G.type == G_SDCZ) {
+			if(G.nOffsets == 0) continue;
+			const unsigned sg = (unsigned) std::max(G.nCkpt, 1);
+			Prof pf(b, "k_decompress_sdc", sg, 256, 0, 0);
+			if(G.deltaWidth == 1) hipLaunchKernelGGL(k_decompress_sdc<1>, dim3(sg), dim3(256), 0, st, b->dGroups, g, b->nCols, dOut);
+			else hipLaunchKernelGGL(k_decompress_sdc<2>, dim3(sg), dim3(256), 0, st, b->dGroups, g, b->nCols, dOut);
+		}
+		else {
+			const int64_t m = nRows * G.nColG;
+			Prof pf(b, "k_decompress_rows", (long) ((m + 255) / 256), 256, 0, 0);
+			hipLaunchKernelGGL(k_decompress_rows, dim3((unsigned) ((m + 255) / 256)), dim3(256), 0, st, b->dGroups, g, nRows,
+				b->nCols, dOut);
+		}
+	}
+	{
+		Prof pf(b, "k_count_nnz", fg, 256, 0, 0);
+		hipLaunchKernelGGL(k_count_nnz2, dim3(fg), dim3(256), 0, st, dOut, n, dNnz);
+	}
+	CLA_HIP(hipGetLastError());
+	return 0;
+}
+
+} // namespace cla

@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 
 from conftest import mixed_block
-from parity import assert_fp64_close
+from parity import assert_fp64_close, assert_matches_truth
 
 pytestmark = pytest.mark.gpu
 
@@ -19,7 +19,8 @@ def test_mixed_groups_lmm(cla, ora, seed, n_rows, p):
     blk.close()
     ref, rnnz = ora.lmm(ora.Groups(specs, n_rows, n_cols), Y, 4)
     D = ora.np_decompress(specs, n_rows, n_cols)
-    assert_fp64_close(out, ref, ora.abs_matmul(Y, D), what=f"lmm p={p}")
+    assert_matches_truth(out, Y, D, what=f"lmm p={p}")
+    assert_fp64_close(out, ref, ora.abs_matmul(Y, D), what=f"lmm p={p}", n_terms=n_rows)
     assert nnz == rnnz
 
 
@@ -33,11 +34,13 @@ def test_c4_scaled_both_products(cla, ora):
     D = ora.np_decompress(c["groups"], n_rows, n_cols)
     out, nnz = blk.lmm(c["v"])
     ref, rnnz = ora.lmm(G, c["v"], 4)
-    assert_fp64_close(out, ref, ora.abs_matmul(c["v"], D), what="C4 t(v)%*%X")
+    assert_matches_truth(out, c["v"], D, what="C4 t(v)%*%X")
+    assert_fp64_close(out, ref, ora.abs_matmul(c["v"], D), what="C4 t(v)%*%X", n_terms=n_rows)
     assert nnz == rnnz
     out, nnz = blk.rmm(c["u"])
     ref, rnnz = ora.rmm(G, c["u"], 4)
-    assert_fp64_close(out, ref, ora.abs_matmul(D, c["u"]), what="C4 X%*%u")
+    assert_matches_truth(out, D, c["u"], what="C4 X%*%u")
+    assert_fp64_close(out, ref, ora.abs_matmul(D, c["u"]), what="C4 X%*%u", n_terms=n_cols)
     assert nnz == rnnz
     blk.close()
 
@@ -52,7 +55,8 @@ def test_c2_scaled_left_vector(cla, ora):
     blk.close()
     ref, rnnz = ora.lmm(ora.Groups(c["groups"], n_rows, n_cols), y, 4)
     D = ora.np_decompress(c["groups"], n_rows, n_cols)
-    assert_fp64_close(out, ref, ora.abs_matmul(y, D), what="C2 t(y)%*%X")
+    assert_matches_truth(out, y, D, what="C2 t(y)%*%X")
+    assert_fp64_close(out, ref, ora.abs_matmul(y, D), what="C2 t(y)%*%X", n_terms=n_rows)
     assert nnz == rnnz
 
 
@@ -68,7 +72,7 @@ def test_preagg_per_group(cla, ora):
             ref = ora.preaggregate_dense(G, i, Y)
             scale = np.zeros_like(ref)
             refabs = ora.preaggregate_dense(G, i, np.abs(Y))
-            assert_fp64_close(pre, ref, refabs + scale, what=f"preagg {s.type}")
+            assert_fp64_close(pre, ref, refabs + scale, what=f"preagg {s.type}", n_terms=30011)
             # sum over bins = sum of Y over the rows the group covers
             assert np.allclose(pre.sum(axis=1), ref.sum(axis=1), rtol=0, atol=1e-9)
         if s.type not in ("const", "empty"):
@@ -90,5 +94,5 @@ def test_mmchain(cla, ora, ctype):
     if ctype:
         inner = inner * np.abs(w)
     scale = np.abs(D).T @ inner
-    assert_fp64_close(out, ref, scale, what="mmchain")
+    assert_fp64_close(out, ref, scale, what="mmchain", n_terms=40009)
     assert nnz == rnnz

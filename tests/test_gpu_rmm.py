@@ -3,7 +3,7 @@ import numpy as np
 import pytest
 
 from conftest import mixed_block
-from parity import assert_fp64_close
+from parity import assert_fp64_close, assert_matches_truth
 
 pytestmark = pytest.mark.gpu
 
@@ -58,7 +58,9 @@ def test_c2_scaled_matvec_and_matmat(cla, ora):
     assert nnz == rnnz
     scale_B = abs_scale(ora, c["groups"], c["n_rows"], c["n_cols"], c["B"])
     out, nnz, ref, rnnz = run_both(cla, ora, c["groups"], c["n_rows"], c["n_cols"], c["B"])
-    assert_fp64_close(out, ref, scale_B, what="C2 X%*%B")
+    assert_fp64_close(out, ref, scale_B, what="C2 X%*%B", n_terms=c["n_cols"])
+    D = ora.np_decompress(c["groups"], c["n_rows"], c["n_cols"])
+    assert_matches_truth(out[:4000], D[:4000], c["B"], what="C2 X%*%B (first 4000 rows)")
     assert nnz == rnnz
 
 
@@ -70,7 +72,9 @@ def test_mixed_groups(cla, ora, seed, n_rows, q):
     specs, n_cols = mixed_block(seed, n_rows)
     B = np.random.default_rng(seed + 50).standard_normal((n_cols, q))
     out, nnz, ref, rnnz = run_both(cla, ora, specs, n_rows, n_cols, B)
-    assert_fp64_close(out, ref, abs_scale(ora, specs, n_rows, n_cols, B), what=f"mixed q={q}")
+    assert_fp64_close(out, ref, abs_scale(ora, specs, n_rows, n_cols, B), what=f"mixed q={q}", n_terms=n_cols)
+    D = ora.np_decompress(specs, n_rows, n_cols)
+    assert_matches_truth(out[:3000], D[:3000], B, what=f"mixed q={q}")
     assert nnz == rnnz
 
 

@@ -1,0 +1,91 @@
+"""GPU parity of t(X) %*% X (cla_tsmm), integer co-occurrence (cla_cooc) and
+decompression (cla_decompress) against the CPU oracle, through the C ABI."""
+import numpy as np
+import pytest
+
+from conftest import mixed_block
+from parity import assert_fp64_close, assert_matches_truth
+
+pytestmark = pytest.mark.gpu
+
+
+def check_tsmm(cla, ora, specs, n_rows, n_cols, what):
+    blk = cla.build_block(n_rows, n_cols, specs)
+    out, nnz = blk.tsmm()
+    blk.close()
+    ref, rnnz = ora.tsmm(ora.Groups(specs, n_rows, n_cols), 4)
+    D = ora.np_decompress(specs, n_rows, n_cols)
+    assert np.array_equal(out, out.T)
+    assert_matches_truth(out, D.T, D, what=what)
+    assert_fp64_close(out, ref, ora.abs_matmul(D.T, D), what=what, n_terms=n_rows)
+    assert nnz == rnnz
+
+
+@pytest.mark.parametrize("seed,n_rows", [(0, 1), (1, 37), (2, 3000), (3, 20011), (4, 150001)])
+@pytest.mark.parametrize("with_unc", [False, True])
+def test_mixed_groups_tsmm(cla, ora, seed, n_rows, with_unc):
+    """Compressed pair path (no uncompressed group) and the decompressing fallback."""
+    specs, n_cols = mixed_block(seed, n_rows, with_unc=with_unc)
+    check_tsmm(cla, ora, specs, n_rows, n_cols, f"tsmm unc={with_unc}")
+
+
+def test_c3_scaled(cla, ora):
+    """BASELINE config 3 at 1/100 scale: 25 co-coded pairs, 4096 tuples, uint16 codes."""
+    from systemds_amd import synth
+    c = synth.config3(scale=100)
+    check_tsmm(cla, ora, c["groups"], c["n_rows"], c["n_cols"], "C3")
+
+
+def test_c5_scaled(cla, ora):
+    """BASELINE config 5 at 1/500 scale (mixed RLE + DDC + SDC + dense): both products."""
+    from systemds_amd import synth
+    c = synth.config5(scale=500)
+    n_rows, n_cols = c["n_rows"], c["n_cols"]
+    check_tsmm(cla, ora, c["groups"], n_rows, n_cols, "C5 tsmm")
+    blk = cla.build_block(n_rows, n_cols, c["groups"])
+    out, nnz = blk.rmm(c["B"])
+    blk.close()
+    ref, rnnz = ora.rmm(ora.Groups(c["groups"], n_rows, n_cols), c["B"], 4)
+    D = ora.np_decompress(c["groups"], n_rows, n_cols)
+    assert_matches_truth(out, D, c["B"], what="C5 X%*%B")
+    assert_fp64_close(out, ref, ora.abs_matmul(D, c["B"]), what="C5 X%*%B", n_terms=n_cols)
+    assert nnz == rnnz
+
+
+def test_single_column_groups_use_dense_path(cla, ora):
+    """As many groups as columns: the reference decompresses (CLALibTSMM.java:73-77)."""
+    from systemds_amd import synth
+    c = synth.config4(scale=200, n_cols=12)
+    check_tsmm(cla, ora, c["groups"], c["n_rows"], c["n_cols"], "C4-like")
+    c = synth.config2(scale=500, n_cols=30)
+    check_tsmm(cla, ora, c["groups"], c["n_rows"], c["n_cols"], "C2-like")
+
+
+def test_cooc_bit_exact(cla, ora):
+    specs, n_cols = mixed_block(31, 60007, with_unc=False)
+    blk = cla.build_block(60007, n_cols, specs)
+    G = ora.Groups(specs, 60007, n_cols)
+    idx = [i for i, s in enumerate(specs) if s.type in ("ddc", "sdc", "rle")]
+    for a, i in enumerate(idx):
+        for b_, j in enumerate(idx):
+            if specs[i].n_vals * specs[j].n_vals > 400000:
+                continue
+            N = blk.cooc(a, b_)
+            assert np.array_equal(N, ora.cooc(G, i, j)), (specs[i].type, specs[j].type)
+    # large code space (70000 x 300 bins -> HBM atomics): marginals must equal the counts
+    N = blk.cooc(2, 1)
+    assert np.array_equal(N.sum(axis=1), blk.counts(2))
+    assert np.array_equal(N.sum(axis=0), blk.counts(1))
+    assert N.sum() == 60007
+    blk.close()
+
+
+@pytest.mark.parametrize("seed,n_rows", [(0, 1), (2, 3000), (4, 70001)])
+def test_decompress(cla, ora, seed, n_rows):
+    specs, n_cols = mixed_block(seed, n_rows)
+    blk = cla.build_block(n_rows, n_cols, specs)
+    out, nnz = blk.decompress()
+    blk.close()
+    ref = ora.decompress(ora.Groups(specs, n_rows, n_cols))
+    assert np.array_equal(out, ref)
+    assert nnz == np.count_nonzero(ref)
