@@ -214,6 +214,7 @@ void cla_block_free(cla_handle b) {
 	for(auto& g : b->groups) free_group(g);
 	if(b->dGroups) (void) hipFree(b->dGroups);
 	if(b->dConstV) (void) hipFree(b->dConstV);
+	if(b->dAllDict) (void) hipFree(b->dAllDict);
 	if(b->dQ1Slabs) (void) hipFree(b->dQ1Slabs);
 	if(b->dArena) (void) hipFree(b->dArena);
 	if(b->dTblOff) (void) hipFree(b->dTblOff);
@@ -424,6 +425,23 @@ int cla_block_finalize(cla_handle b) {
 	b->maxVals = maxVals;
 
 	const size_t nG = b->groups.size();
+	// all dictionaries back to back in one allocation (kernels copy a slab of
+	// consecutive groups' dictionaries into LDS as one contiguous range)
+	{
+		size_t total = 0;
+		for(auto& g : b->groups) total += g.dict.size();
+		CLA_HIP(hipMalloc((void**) &b->dAllDict, sizeof(double) * std::max<size_t>(total, 1)));
+		size_t off = 0;
+		for(auto& g : b->groups) {
+			if(g.dict.empty()) continue;
+			CLA_HIP(hipMemcpy(b->dAllDict + off, g.dict.data(), sizeof(double) * g.dict.size(), hipMemcpyHostToDevice));
+			void* old = const_cast<double*>(g.d.dict);
+			g.owned.erase(std::remove(g.owned.begin(), g.owned.end(), old), g.owned.end());
+			CLA_HIP(hipFree(old));
+			g.d.dict = b->dAllDict + off;
+			off += g.dict.size();
+		}
+	}
 	std::vector<DGroup> flat(nG);
 	for(size_t i = 0; i < nG; i++) flat[i] = b->groups[i].d;
 	CLA_HIP(hipMalloc((void**) &b->dGroups, sizeof(DGroup) * std::max<size_t>(nG, 1)));

@@ -85,6 +85,7 @@ struct cla_block {
 
 	cla::DGroup* dGroups = nullptr;  // device array of descriptors
 	double* dConstV = nullptr;       // device copy of constV (nCols)
+	double* dAllDict = nullptr;      // all (morphed) dictionaries back to back in group order
 
 	// All-DDC blocks of one code width keep their code streams in one arena with a
 	// uniform stride, so kernels address stream g as arena + g * arenaStride.
@@ -130,6 +131,8 @@ int launch_validate_codes(cla_block* b, const void* codes, int width, int64_t n,
 int launch_counts(cla_block* b, int group, int32_t* dCounts);
 int launch_sdc_build(cla_block* b, HostGroup& g);
 int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned long long* dNnz);
+int launch_rmm_mfma(cla_block* b, const double* dB, int q, const double* dConstRow, double* dOut,
+	unsigned long long* dNnz);
 int launch_decompress(cla_block* b, double* dOut, unsigned long long* dNnz);
 int launch_lmm(cla_block* b, const double* dY, int p, double* dOut, unsigned long long* dNnz);
 int launch_preagg(cla_block* b, int group, const double* dY, int p, double* dPre);

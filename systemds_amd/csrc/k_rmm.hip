@@ -479,6 +479,12 @@ int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned lon
 		return 0;
 	}
 
+	// wide B on an all-DDC block: fused decode + fp64 MFMA (K1 above still supplies constV x B)
+	if(q >= 8 && !getenv("CLA_NO_MFMA")) {
+		const int r = launch_rmm_mfma(b, dB, q, constRow >= 0 ? b->dTables + (size_t) constRow * q : nullptr, dOut, dNnz);
+		if(r <= 0) return r;
+	}
+
 	// generic path
 	{
 		const int64_t n = nRows * q;
