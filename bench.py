@@ -19,6 +19,95 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
 
+def timed(blk, fn, reps=5, warm=2):
+    """Median wall time of fn() (each call returns nnz, i.e. is synchronous) and the
+    per-kernel HIP-event times of the last call."""
+    import torch
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    ts = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        fn()
+        ts.append(time.perf_counter() - t0)
+    blk.profile(True)
+    fn()
+    ks = blk.stats()["kernels"]
+    blk.profile(False)
+    agg = {}
+    for k in ks:
+        a = agg.setdefault(k["name"], {"ms": 0.0, "launches": 0, "algo_bytes": 0.0})
+        a["ms"] += k["ms"]
+        a["launches"] += 1
+        a["algo_bytes"] += k["algo_bytes"]
+    return statistics.median(ts) * 1e3, agg
+
+
+def other_configs(scale):
+    """X %*% v of C1, t(X) %*% X of C3, both products of C4, both products of C5."""
+    import numpy as np
+    import torch
+    from systemds_amd import capi, synth
+    out = {}
+
+    def dev(a):
+        return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+    def run(name, cfg, ops):
+        t0 = time.time()
+        blk = capi.build_block(cfg["n_rows"], cfg["n_cols"], cfg["groups"])
+        up = time.time() - t0
+        for op, fn, algo_bytes in ops(blk, cfg):
+            ms, ks = timed(blk, fn)
+            out[f"{name} {op}"] = {"ms": ms, "rows_per_s": cfg["n_rows"] / (ms * 1e-3), "algo_bytes": algo_bytes,
+                                  "algo_GBs": algo_bytes / (ms * 1e-3) / 1e9,
+                                  "frac_hbm": algo_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "kernels": ks,
+                                  "upload_s": round(up, 2)}
+        blk.close()
+        torch.cuda.empty_cache()
+
+    def rmm_ops(vname, q):
+        def ops(blk, cfg):
+            dv = dev(cfg[vname])
+            do = torch.empty((cfg["n_rows"], q), dtype=torch.float64, device="cuda")
+            bytes_in = blk.device_bytes()
+            yield (f"X%*%{vname}", lambda: blk.rmm_dev(dv.data_ptr(), q, do.data_ptr()), bytes_in + cfg["n_rows"] * q * 8.0)
+        return ops
+
+    c = synth.config1()
+    run("C1", c, rmm_ops("v", 1))
+    c = synth.config3(scale=scale)
+
+    def tsmm_ops(blk, cfg):
+        do = torch.empty((cfg["n_cols"], cfg["n_cols"]), dtype=torch.float64, device="cuda")
+        yield ("t(X)%*%X", lambda: blk.tsmm_dev(do.data_ptr()), float(blk.device_bytes()))
+    run("C3", c, tsmm_ops)
+    del c
+    c = synth.config4(scale=scale)
+
+    def c4_ops(blk, cfg):
+        dv, du = dev(cfg["v"]), dev(cfg["u"])
+        do1 = torch.empty((1, cfg["n_cols"]), dtype=torch.float64, device="cuda")
+        do2 = torch.empty((cfg["n_rows"], 1), dtype=torch.float64, device="cuda")
+        comp = float(sum(g.deltas.nbytes + g.codes.nbytes for g in cfg["groups"]))
+        yield ("t(v)%*%X", lambda: blk.lmm_dev(dv.data_ptr(), 1, do1.data_ptr()), comp + cfg["n_rows"] * 8.0)
+        yield ("X%*%u", lambda: blk.rmm_dev(du.data_ptr(), 1, do2.data_ptr()), comp + cfg["n_rows"] * 8.0)
+    run("C4", c, c4_ops)
+    del c
+    c = synth.config5(scale=scale)
+
+    def c5_ops(blk, cfg):
+        dB = dev(cfg["B"])
+        do1 = torch.empty((cfg["n_rows"], 10), dtype=torch.float64, device="cuda")
+        do2 = torch.empty((20, 20), dtype=torch.float64, device="cuda")
+        comp = float(blk.device_bytes())
+        yield ("X%*%B", lambda: blk.rmm_dev(dB.data_ptr(), 10, do1.data_ptr()), comp + cfg["n_rows"] * 80.0)
+        yield ("t(X)%*%X", lambda: blk.tsmm_dev(do2.data_ptr()), comp)
+    run("C5", c, c5_ops)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -27,6 +116,7 @@ def main():
     ap.add_argument("--scale", type=int, default=1, help="divide the number of rows (testing only)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--extra", action="store_true", help="also time X %*% B (100x64) of the same config")
+    ap.add_argument("--all", action="store_true", help="also time the other BASELINE configs (C1, C3, C4, C5)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (the path shards by rows, see DESIGN.md); "
@@ -119,6 +209,10 @@ def main():
                                                 "frac_hbm": bytesB / (msB * 1e-3) / 1e9 / HBM_PEAK_GBS}}
         del doutB
 
+    if args.all:
+        blk.close()
+        result.setdefault("extra", {}).update(other_configs(args.scale))
+
     if not args.no_cpu:
         # CPU baseline: the oracle's multithreaded restatement of the reference algorithm
         # (a port, not the SystemDS JVM) on the same full workload, host cores of this box.
@@ -137,7 +231,8 @@ def main():
                                             f"{cpu_s:.3f} s per pass",
                                   "parity_bit_exact": bool(np.array_equal(got, ref[:, 0]) and rnnz == nnz)}
 
-    blk.close()
+    if not args.all:
+        blk.close()
     print(json.dumps(result))
 
 

@@ -133,6 +133,8 @@ int launch_sdc_build(cla_block* b, HostGroup& g);
 int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned long long* dNnz);
 int launch_rmm_mfma(cla_block* b, const double* dB, int q, const double* dConstRow, double* dOut,
 	unsigned long long* dNnz);
+int launch_lmm_sdc_tiles(cla_block* b, const double* dY, int p, double* dPre, int onlyGroup);
+int launch_rmm_sdc_tiles(cla_block* b, int q, int constRow, int accumulate, double* dOut, unsigned long long* dNnz);
 int launch_decompress(cla_block* b, double* dOut, unsigned long long* dNnz);
 int launch_lmm(cla_block* b, const double* dY, int p, double* dOut, unsigned long long* dNnz);
 int launch_preagg(cla_block* b, int group, const double* dY, int p, double* dPre);

@@ -221,6 +221,13 @@ static int run_preagg(cla_block* b, const double* dY, int p, double* dPre, int o
 		}
 		g = g1;
 	}
+	// SDCZeros groups: all lists walked tile by tile with the Y tile in LDS; the
+	// per-group chunk kernel below only serves dictionaries too large for LDS bins
+	{
+		const int r = nRows > 0 ? launch_lmm_sdc_tiles(b, dY, p, dPre, onlyGroup) : 0;
+		if(r < 0) return r;
+		if(r == 0) { CLA_HIP(hipGetLastError()); return 0; }
+	}
 	for(g = 0; g < nG; g++) {
 		const DGroup& G = b->groups[g].d;
 		if(G.type != G_SDCZ || G.nOffsets == 0 || (onlyGroup >= 0 && onlyGroup != g)) continue;

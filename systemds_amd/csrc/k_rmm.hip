@@ -7,6 +7,7 @@
 //   k_count_nnz       non-zero count of the result
 #include "../../include/cla_hip.h"
 #include "cla_device.hpp"
+#include <algorithm>
 
 namespace cla {
 
@@ -337,39 +338,67 @@ __global__ __launch_bounds__(THREADS) void k_rmm_q1_u8(const uint8_t* __restrict
 }
 
 // ---------------------------------------------------------------------------
-// Generic row-parallel gather: one thread per output cell (r, c), groups in list
-// order; handles DDC, RLE (merged run table) and uncompressed groups. SDCZeros
-// groups are added afterwards by k_rmm_sdc_scatter.
+// Generic row-parallel gather: a block owns 256 consecutive rows, a thread one row
+// and a strip of output columns (blockIdx.y); groups in list order. Handles DDC,
+// RLE (merged run table: one binary search per block and group, then a short
+// walk) and uncompressed groups. SDCZeros groups are added afterwards.
 // ---------------------------------------------------------------------------
+constexpr int ROWS_QS = 8; // output columns per thread
+
 __global__ __launch_bounds__(256) void k_rmm_rows(const DGroup* __restrict__ groups, int nGroups,
 	const double* __restrict__ T, const double* __restrict__ B, int q, int constRow, double* __restrict__ out,
 	int64_t nRows) {
-	const int64_t idx = (int64_t) blockIdx.x * blockDim.x + threadIdx.x;
-	if(idx >= nRows * q) return;
-	const int64_t r = idx / q;
-	const int c = (int) (idx - r * q);
-	double acc = 0.0;
+	__shared__ int runBase;
+	const int64_t r = (int64_t) blockIdx.x * 256 + threadIdx.x;
+	const int c0 = blockIdx.y * ROWS_QS;
+	const int nc = min(ROWS_QS, q - c0);
+	const bool live = r < nRows;
+	double acc[ROWS_QS];
+#pragma unroll
+	for(int c = 0; c < ROWS_QS; c++) acc[c] = 0.0;
 	for(int g = 0; g < nGroups; g++) {
 		const DGroup& G = groups[g];
 		if(G.type == G_DDC) {
-			const int code = load_code(G.codes, G.codeWidth, r);
-			acc += T[(size_t) (G.tblOff + code) * q + c];
+			if(live) {
+				const double* t = T + (size_t) (G.tblOff + load_code(G.codes, G.codeWidth, r)) * q + c0;
+#pragma unroll
+				for(int c = 0; c < ROWS_QS; c++)
+					if(c < nc) acc[c] += t[c];
+			}
 		}
 		else if(G.type == G_RLE) {
-			const int code = G.runCode[rle_find(G.runStart, G.nRuns, (int32_t) r)];
-			if(code >= 0) acc += T[(size_t) (G.tblOff + code) * q + c];
-		}
-		else if(G.type == G_UNC) {
-			double s = 0.0;
-			for(int h = 0; h < G.nColG; h++) {
-				const double a = G.dense[(size_t) r * G.nColG + h];
-				if(a != 0) s = __dadd_rn(s, __dmul_rn(a, B[(size_t) G.cols[h] * q + c]));
+			__syncthreads();
+			if(threadIdx.x == 0) runBase = rle_find(G.runStart, G.nRuns, (int32_t) ((int64_t) blockIdx.x * 256));
+			__syncthreads();
+			if(live) {
+				int j = runBase;
+				while(G.runStart[j + 1] <= r) j++;
+				const int code = G.runCode[j];
+				if(code >= 0) {
+					const double* t = T + (size_t) (G.tblOff + code) * q + c0;
+#pragma unroll
+					for(int c = 0; c < ROWS_QS; c++)
+						if(c < nc) acc[c] += t[c];
+				}
 			}
-			acc += s;
+		}
+		else if(G.type == G_UNC && live) {
+#pragma unroll
+			for(int c = 0; c < ROWS_QS; c++) {
+				if(c >= nc) continue;
+				double s = 0.0;
+				for(int h = 0; h < G.nColG; h++) {
+					const double a = G.dense[(size_t) r * G.nColG + h];
+					if(a != 0) s = __dadd_rn(s, __dmul_rn(a, B[(size_t) G.cols[h] * q + c0 + c]));
+				}
+				acc[c] += s;
+			}
 		}
 	}
-	if(constRow >= 0) acc += T[(size_t) constRow * q + c];
-	out[idx] = acc;
+	if(!live) return;
+#pragma unroll
+	for(int c = 0; c < ROWS_QS; c++)
+		if(c < nc) out[(size_t) r * q + c0 + c] = acc[c] + (constRow >= 0 ? T[(size_t) constRow * q + c0 + c] : 0.0);
 }
 
 // One block per chunk of SDC_CK delta entries of one SDCZeros group: decode the
@@ -485,28 +514,50 @@ int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned lon
 		if(r <= 0) return r;
 	}
 
-	// generic path
+	// generic path: row-parallel gather for DDC / RLE / uncompressed groups, then the
+	// SDCZeros groups tile by tile (or per-entry scatter when their tables do not fit LDS)
 	{
 		const int64_t n = nRows * q;
-		const unsigned grid = (unsigned) ((n + 255) / 256);
-		{
-			Prof pf(b, "k_rmm_rows", grid, 256, 0, 0);
-			hipLaunchKernelGGL(k_rmm_rows, dim3(grid), dim3(256), 0, st, b->dGroups, nG, b->dTables, dB, q, constRow,
-				dOut, nRows);
+		bool anyRowGroup = false, anySdc = false;
+		for(auto& g : b->groups) {
+			if(g.d.type == G_SDCZ) anySdc |= g.d.nOffsets > 0;
+			else anyRowGroup = true;
 		}
-		for(int g = 0; g < nG; g++) {
-			const DGroup& G = b->groups[g].d;
-			if(G.type != G_SDCZ || G.nOffsets == 0) continue;
-			const unsigned sg = (unsigned) (G.nCkpt > 1 ? G.nCkpt : 1);
-			Prof pf(b, "k_rmm_sdc_scatter", sg, 256, 0, 0);
-			if(G.deltaWidth == 1)
-				hipLaunchKernelGGL(k_rmm_sdc_scatter<1>, dim3(sg), dim3(256), 0, st, b->dGroups, g, b->dTables, q, dOut);
-			else
-				hipLaunchKernelGGL(k_rmm_sdc_scatter<2>, dim3(sg), dim3(256), 0, st, b->dGroups, g, b->dTables, q, dOut);
+		bool needNnzPass = true;
+		if(anyRowGroup || !anySdc) {
+			const dim3 grid((unsigned) ((nRows + 255) / 256), (unsigned) ((q + ROWS_QS - 1) / ROWS_QS));
+			Prof pf(b, "k_rmm_rows", (long) grid.x * grid.y, 256, 0, 0);
+			hipLaunchKernelGGL(k_rmm_rows, grid, dim3(256), 0, st, b->dGroups, nG, b->dTables, dB, q, constRow, dOut, nRows);
 		}
-		const unsigned cg = (unsigned) ((n + 256 * 8 - 1) / (256 * 8));
-		Prof pf(b, "k_count_nnz", cg, 256, 0, 0);
-		hipLaunchKernelGGL(k_count_nnz, dim3(cg > 65535 * 16 ? 65535 * 16 : cg), dim3(256), 0, st, dOut, n, dNnz);
+		if(anySdc) {
+			const int r = launch_rmm_sdc_tiles(b, q, constRow, anyRowGroup ? 1 : 0, dOut, dNnz);
+			if(r < 0) return r;
+			if(r == 0) needNnzPass = false;
+			else {
+				if(!anyRowGroup) {
+					// the scatter adds on top of an initialised output
+					const dim3 grid((unsigned) ((nRows + 255) / 256), (unsigned) ((q + ROWS_QS - 1) / ROWS_QS));
+					Prof pf(b, "k_rmm_rows", (long) grid.x * grid.y, 256, 0, 0);
+					hipLaunchKernelGGL(k_rmm_rows, grid, dim3(256), 0, st, b->dGroups, nG, b->dTables, dB, q, constRow, dOut,
+						nRows);
+				}
+				for(int g = 0; g < nG; g++) {
+					const DGroup& G = b->groups[g].d;
+					if(G.type != G_SDCZ || G.nOffsets == 0) continue;
+					const unsigned sg = (unsigned) (G.nCkpt > 1 ? G.nCkpt : 1);
+					Prof pf(b, "k_rmm_sdc_scatter", sg, 256, 0, 0);
+					if(G.deltaWidth == 1)
+						hipLaunchKernelGGL(k_rmm_sdc_scatter<1>, dim3(sg), dim3(256), 0, st, b->dGroups, g, b->dTables, q, dOut);
+					else
+						hipLaunchKernelGGL(k_rmm_sdc_scatter<2>, dim3(sg), dim3(256), 0, st, b->dGroups, g, b->dTables, q, dOut);
+				}
+			}
+		}
+		if(needNnzPass) {
+			const unsigned cg = (unsigned) std::min<int64_t>((n + 256 * 8 - 1) / (256 * 8), (int64_t) g_numCU * 32);
+			Prof pf(b, "k_count_nnz", cg, 256, 0, 0);
+			hipLaunchKernelGGL(k_count_nnz, dim3(cg), dim3(256), 0, st, dOut, n, dNnz);
+		}
 	}
 	CLA_HIP(hipGetLastError());
 	return 0;
