@@ -117,6 +117,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--extra", action="store_true", help="also time X %*% B (100x64) of the same config")
     ap.add_argument("--all", action="store_true", help="also time the other BASELINE configs (C1, C3, C4, C5)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 1 GiB device copy (torch) so that a rocprofv3 --pmc run can scale "
+                         "FETCH_SIZE / WRITE_SIZE against a kernel of known traffic")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (the path shards by rows, see DESIGN.md); "
@@ -190,6 +193,14 @@ def main():
                      "frac": achieved / HBM_PEAK_GBS, "kernel_ms": k_ms, "algo_bytes_per_launch": kbytes,
                      "traffic": None},
     }
+
+    if args.calibrate_copy:
+        src = torch.empty(1 << 27, dtype=torch.float64, device="cuda").fill_(1.0)  # 1 GiB
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     if args.extra:
         dB = torch.from_numpy(cfg["B"].copy()).cuda()

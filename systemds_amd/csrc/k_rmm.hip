@@ -249,11 +249,11 @@ __global__ __launch_bounds__(THREADS) void k_rmm_q1_ddc(const uint8_t* __restric
 // which turns every table base into an immediate offset of the LDS read.
 // Slots of a short last slab are zero-filled (x + 0.0 leaves the sum unchanged).
 // ---------------------------------------------------------------------------
-constexpr int U8_PER = 16;   // groups (tables) per slab: 16 x 2 KiB = 32 KiB of LDS
-constexpr int U8_NB = 4;     // groups per load batch
 constexpr int U8_RPT = 16;   // rows per thread = one 16-byte load per group
 
-template <int THREADS>
+// U8_PER = groups (tables) per slab (2 KiB of LDS each), U8_NB = groups per load batch,
+// U8_PER is a multiple of 2 * U8_NB. The host picks the variant that pads least.
+template <int THREADS, int U8_PER, int U8_NB>
 __global__ __launch_bounds__(THREADS) void k_rmm_q1_u8(const uint8_t* __restrict__ arena, size_t arenaStride,
 	int nGroups, const int32_t* __restrict__ tblOff, const double* __restrict__ T, int constIdx,
 	double* __restrict__ out, int64_t nRows, unsigned long long* __restrict__ nnz) {
@@ -271,19 +271,34 @@ __global__ __launch_bounds__(THREADS) void k_rmm_q1_u8(const uint8_t* __restrict
 	CodeVec<1, RPT> ping[NB], pong[NB];
 	if(full) q1_load<1, RPT, NB>(ping, myCodes, arenaStride, 0, nGroups - 1);
 
-	for(int g0 = 0; g0 < nGroups; g0 += U8_PER) {
+	// the tables of the next slab are fetched into registers while the current slab is processed
+	constexpr int TPT = (U8_PER * 256 + THREADS - 1) / THREADS;
+	double stage[TPT];
+	auto fetch = [&](int g0) {
 		const int nIn = min(U8_PER, nGroups - g0);
-		__syncthreads();
-		for(int f = tid; f < U8_PER * 256; f += THREADS) {
+#pragma unroll
+		for(int k = 0; k < TPT; k++) {
+			const int f = tid + k * THREADS;
 			const int g = f >> 8, i = f & 255;
 			double v = 0.0;
 			if(g < nIn) {
 				const int o = tblOff[g0 + g], n = tblOff[g0 + g + 1] - o;
 				if(i < n) v = T[o + i];
 			}
-			tbl[f] = v;
+			stage[k] = v;
+		}
+	};
+	fetch(0);
+	for(int g0 = 0; g0 < nGroups; g0 += U8_PER) {
+		const int nIn = min(U8_PER, nGroups - g0);
+		__syncthreads();
+#pragma unroll
+		for(int k = 0; k < TPT; k++) {
+			const int f = tid + k * THREADS;
+			if(f < U8_PER * 256) tbl[f] = stage[k];
 		}
 		__syncthreads();
+		if(g0 + U8_PER < nGroups) fetch(g0 + U8_PER);
 		if(full) {
 #pragma unroll
 			for(int s = 0; s < U8_PER; s += 2 * NB) {
@@ -312,27 +327,42 @@ __global__ __launch_bounds__(THREADS) void k_rmm_q1_u8(const uint8_t* __restrict
 		}
 	}
 
+	// Epilogue. A thread holds 16 consecutive rows, so direct stores would touch 64
+	// different lines per instruction with 16 bytes each (measured: 2.9x write
+	// amplification). Full tiles are transposed through LDS in two halves of 8 rows per
+	// thread instead, so that 8 consecutive lanes write one 64-byte segment.
 	int cnt = 0;
-	if(any) {
-		if(constIdx >= 0) {
-			const double cadd = T[constIdx];
+	const double cadd = constIdx >= 0 ? T[constIdx] : 0.0;
+	const bool tileFull = (int64_t) (blockIdx.x + 1) * THREADS * RPT <= nRows;
+	if(tileFull) {
+		const int wave = tid >> 6, lane = tid & 63;
+		double* wbuf = tbl + wave * (64 * 8); // 8 values per lane, XOR-swizzled against bank conflicts
+		double* obase = out + ((int64_t) blockIdx.x * THREADS + wave * 64) * RPT;
 #pragma unroll
-			for(int i = 0; i < RPT; i++) acc[i] += cadd;
-		}
-		if(full) {
+		for(int h = 0; h < 2; h++) {
+			__syncthreads();
 #pragma unroll
-			for(int i = 0; i < RPT; i += 2) {
-				cnt += (acc[i] != 0.0) + (acc[i + 1] != 0.0);
-				f64x2 v2;
-				v2.x = acc[i]; v2.y = acc[i + 1];
-				__builtin_nontemporal_store(v2, (f64x2*) (out + row0 + i));
+			for(int i = 0; i < 8; i++) {
+				const double v = acc[h * 8 + i] + cadd;
+				cnt += v != 0.0;
+				wbuf[lane * 8 + (i ^ ((lane >> 2) & 7))] = v;
+			}
+			__syncthreads();
+#pragma unroll
+			for(int j = 0; j < 8; j++) {
+				const int t = j * 64 + lane, sl = t >> 3, i = t & 7;
+				__builtin_nontemporal_store(wbuf[sl * 8 + (i ^ ((sl >> 2) & 7))], obase + sl * RPT + h * 8 + i);
 			}
 		}
-		else {
+	}
+	else if(any) {
 #pragma unroll
-			for(int i = 0; i < RPT; i++)
-				if(row0 + i < nRows) { cnt += acc[i] != 0.0; out[row0 + i] = acc[i]; }
-		}
+		for(int i = 0; i < RPT; i++)
+			if(row0 + i < nRows) {
+				const double v = acc[i] + cadd;
+				cnt += v != 0.0;
+				out[row0 + i] = v;
+			}
 	}
 	count_add(nnz, cnt);
 }
@@ -468,9 +498,17 @@ int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned lon
 		const int64_t rowsPerBlock = (int64_t) THREADS * U8_RPT;
 		const unsigned grid = (unsigned) ((nRows + rowsPerBlock - 1) / rowsPerBlock);
 		const double bytes = (double) nRows * nG + (double) nRows * 8 + (double) b->totalVals * 8;
-		Prof pf(b, "k_rmm_q1_u8", grid, THREADS, U8_PER * 256 * 8, bytes);
-		hipLaunchKernelGGL(k_rmm_q1_u8<THREADS>, dim3(grid), dim3(THREADS), 0, st, b->dArena, b->arenaStride, nG,
-			b->dTblOff, b->dTables, constRow, dOut, nRows, dNnz);
+		// slab size: 16 or 20 groups, whichever leaves fewer padded table slots
+		const int pad16 = (nG + 15) / 16 * 16 - nG, pad20 = (nG + 19) / 20 * 20 - nG;
+		int per = pad20 < pad16 ? 20 : 16;
+		if(const char* e = getenv("CLA_Q1_PER")) per = atoi(e) == 20 ? 20 : 16;
+		Prof pf(b, "k_rmm_q1_u8", grid, THREADS, per * 256 * 8, bytes);
+		if(per == 20)
+			hipLaunchKernelGGL((k_rmm_q1_u8<THREADS, 20, 5>), dim3(grid), dim3(THREADS), 0, st, b->dArena, b->arenaStride,
+				nG, b->dTblOff, b->dTables, constRow, dOut, nRows, dNnz);
+		else
+			hipLaunchKernelGGL((k_rmm_q1_u8<THREADS, 16, 4>), dim3(grid), dim3(THREADS), 0, st, b->dArena, b->arenaStride,
+				nG, b->dTblOff, b->dTables, constRow, dOut, nRows, dNnz);
 		CLA_HIP(hipGetLastError());
 		return 0;
 	}
