@@ -18,6 +18,12 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs,
+# scaled against a plain 1 GiB copy: 2.0 KiB per FETCH_SIZE unit, 1.0 KiB per WRITE_SIZE
+# unit); figures and commands: profiles/k_rmm_q1_u8_C2_matvec.md. Valid for the full-size
+# C2 workload only.
+MEASURED_TRAFFIC = {"k_rmm_q1_u8": 489701.3 * 2048 + 87130.4 * 1024}
+
 
 def timed(blk, fn, reps=5, warm=2):
     """Median wall time of fn() (each call returns nnz, i.e. is synchronous) and the
@@ -191,7 +197,7 @@ def main():
                    "block_bytes": int(blk.device_bytes())},
         "roofline": {"bound": "hbm", "kernel": kname, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "kernel_ms": k_ms, "algo_bytes_per_launch": kbytes,
-                     "traffic": None},
+                     "traffic": MEASURED_TRAFFIC.get(kname) if args.scale == 1 else None},
     }
 
     if args.calibrate_copy:
