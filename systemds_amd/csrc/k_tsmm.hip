@@ -24,13 +24,15 @@ constexpr int TSMM_THREADS = 256; // 4 rows per thread per tile
 __device__ void tile_codes(const DGroup& G, int tile, int64_t nRows, int32_t* __restrict__ codes) {
 	const int64_t r0 = (int64_t) tile * TT;
 	const int tid = threadIdx.x;
+	const int TSMM_THREADS = blockDim.x; // any multiple of 64, at least 256
 	if(G.type == G_DDC) {
 		for(int t = tid; t < TT; t += TSMM_THREADS) codes[t] = r0 + t < nRows ? load_code(G.codes, G.codeWidth, r0 + t) : -1;
 	}
 	else if(G.type == G_RLE) {
-		// each thread expands 4 consecutive rows from the merged run table
+		// threads 0..255 expand 4 consecutive rows each from the merged run table
 		const int64_t rb = r0 + tid * 4;
-		if(rb < nRows) {
+		if(tid >= TT / 4) {}
+		else if(rb < nRows) {
 			int j = rle_find(G.runStart, G.nRuns, (int32_t) rb);
 			for(int t = 0; t < 4; t++) {
 				const int64_t r = rb + t;
@@ -88,8 +90,24 @@ __device__ __forceinline__ void add_upper_atomic(double* out, int nCols, int row
 // contiguous range of tiles, then contracts t(dict_t) . P and adds the
 // nC_t x nC_s result into the upper triangle.
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(TSMM_THREADS) void k_tsmm_pair(const DGroup* __restrict__ groups,
+constexpr int PAIR_THREADS = 1024;
+
+// one row of a DDC-DDC pair: P[a, :] += dict_s[c, :]
+__device__ __forceinline__ void pair_add(double* __restrict__ P, const double* __restrict__ dsrc, int nCs, int a, int c) {
+	const double* v = dsrc + (size_t) c * nCs;
+	double* p = P + (size_t) a * nCs;
+	if(nCs == 2) {
+		const double2 vv = *(const double2*) v;
+		unsafeAtomicAdd(&p[0], vv.x);
+		unsafeAtomicAdd(&p[1], vv.y);
+	}
+	else
+		for(int j = 0; j < nCs; j++) unsafeAtomicAdd(&p[j], v[j]);
+}
+
+__global__ __launch_bounds__(PAIR_THREADS) void k_tsmm_pair(const DGroup* __restrict__ groups,
 	const int4* __restrict__ pairs, int64_t nRows, int tilesPerBlock, double* __restrict__ out, int nCols) {
+	constexpr int TSMM_THREADS = PAIR_THREADS;
 	extern __shared__ double smem[];
 	const int4 pr = pairs[blockIdx.y]; // (target, source, dictInLds, 0)
 	const DGroup& Gt = groups[pr.x];
@@ -108,21 +126,47 @@ __global__ __launch_bounds__(TSMM_THREADS) void k_tsmm_pair(const DGroup* __rest
 	const int nTiles = (int) ((nRows + TT - 1) / TT);
 	const int t0 = blockIdx.x * tilesPerBlock, t1 = min(t0 + tilesPerBlock, nTiles);
 	__syncthreads();
-	for(int tile = t0; tile < t1; tile++) {
-		tile_codes(Gt, tile, nRows, ca);
-		tile_codes(Gs, tile, nRows, cb);
-		for(int t = tid; t < TT; t += TSMM_THREADS) {
-			const int a = ca[t], c = cb[t];
-			if(a >= 0 && c >= 0) {
-				const double* v = dsrc + (size_t) c * nCs;
-				double* p = P + (size_t) a * nCs;
-				for(int j = 0; j < nCs; j++) unsafeAtomicAdd(&p[j], v[j]);
+	if(Gt.type == G_DDC && Gs.type == G_DDC) {
+		// both code streams are read directly, 8 rows per thread and step
+		const int64_t rb = (int64_t) t0 * TT, re = min((int64_t) t1 * TT, nRows);
+		const int wt = Gt.codeWidth, ws = Gs.codeWidth;
+		for(int64_t r0 = rb + (int64_t) tid * 8; r0 < re; r0 += (int64_t) TSMM_THREADS * 8) {
+			if(r0 + 8 <= re && wt == 2 && ws == 2) {
+				const u32x4 ua = __builtin_nontemporal_load((const u32x4*) ((const uint16_t*) Gt.codes + r0));
+				const u32x4 ub = __builtin_nontemporal_load((const u32x4*) ((const uint16_t*) Gs.codes + r0));
+				const uint32_t wa[4] = {ua.x, ua.y, ua.z, ua.w}, wb[4] = {ub.x, ub.y, ub.z, ub.w};
+#pragma unroll
+				for(int t = 0; t < 8; t++)
+					pair_add(P, dsrc, nCs, (wa[t >> 1] >> (16 * (t & 1))) & 0xffff, (wb[t >> 1] >> (16 * (t & 1))) & 0xffff);
+			}
+			else if(r0 + 8 <= re && wt == 1 && ws == 1) {
+				const uint2 ua = *(const uint2*) ((const uint8_t*) Gt.codes + r0);
+				const uint2 ub = *(const uint2*) ((const uint8_t*) Gs.codes + r0);
+				const uint32_t wa[2] = {ua.x, ua.y}, wb[2] = {ub.x, ub.y};
+#pragma unroll
+				for(int t = 0; t < 8; t++)
+					pair_add(P, dsrc, nCs, (wa[t >> 2] >> (8 * (t & 3))) & 0xff, (wb[t >> 2] >> (8 * (t & 3))) & 0xff);
+			}
+			else {
+				for(int t = 0; t < 8 && r0 + t < re; t++)
+					pair_add(P, dsrc, nCs, load_code(Gt.codes, wt, r0 + t), load_code(Gs.codes, ws, r0 + t));
 			}
 		}
 		__syncthreads();
 	}
+	else {
+		for(int tile = t0; tile < t1; tile++) {
+			tile_codes(Gt, tile, nRows, ca);
+			tile_codes(Gs, tile, nRows, cb);
+			for(int t = tid; t < TT; t += TSMM_THREADS) {
+				const int a = ca[t], c = cb[t];
+				if(a >= 0 && c >= 0) pair_add(P, dsrc, nCs, a, c);
+			}
+			__syncthreads();
+		}
+	}
 	// contraction: S[i, j] = sum_a dict_t[a, i] * P[a, j]
-	__shared__ double red[4];
+	__shared__ double red[PAIR_THREADS / 64];
 	for(int i = 0; i < nCt; i++)
 		for(int j = 0; j < nCs; j++) {
 			double s = 0.0;
@@ -130,7 +174,11 @@ __global__ __launch_bounds__(TSMM_THREADS) void k_tsmm_pair(const DGroup* __rest
 			s = wave_sum_f64(s);
 			if((tid & 63) == 0) red[tid >> 6] = s;
 			__syncthreads();
-			if(tid == 0) add_upper_atomic(out, nCols, Gt.cols[i], Gs.cols[j], red[0] + red[1] + red[2] + red[3]);
+			if(tid == 0) {
+				double tot = 0.0;
+				for(int w = 0; w < TSMM_THREADS / 64; w++) tot += red[w];
+				add_upper_atomic(out, nCols, Gt.cols[i], Gs.cols[j], tot);
+			}
 			__syncthreads();
 		}
 }
@@ -373,9 +421,9 @@ int launch_tsmm(cla_block* b, double* dOut, unsigned long long* dNnz) {
 			codeBytes += (double) nRows * ((T.type == G_DDC ? T.codeWidth : 0) + (S.type == G_DDC ? S.codeWidth : 0));
 		}
 		{
-			Prof pf(b, "k_tsmm_pair", (long) bpp * (long) pairs.size(), TSMM_THREADS, (long) ldsMax, codeBytes);
+			Prof pf(b, "k_tsmm_pair", (long) bpp * (long) pairs.size(), PAIR_THREADS, (long) ldsMax, codeBytes);
 			CLA_HIP(hipFuncSetAttribute((const void*) k_tsmm_pair, hipFuncAttributeMaxDynamicSharedMemorySize, (int) ldsMax));
-			hipLaunchKernelGGL(k_tsmm_pair, dim3(bpp, (unsigned) pairs.size()), dim3(TSMM_THREADS), ldsMax, st, b->dGroups,
+			hipLaunchKernelGGL(k_tsmm_pair, dim3(bpp, (unsigned) pairs.size()), dim3(PAIR_THREADS), ldsMax, st, b->dGroups,
 				dPairs, nRows, tpb, dOut, nCols);
 		}
 		CLA_HIP(hipStreamSynchronize(st));
