@@ -509,6 +509,8 @@ int cla_block_finalize(cla_handle b) {
 			CLA_HIP(hipMemcpy(b->dQ1Slabs, b->q1Slabs.data(), sizeof(int4) * b->q1Slabs.size(), hipMemcpyHostToDevice));
 		}
 	}
+	b->device_bytes_cached = 0;
+	for(auto& g : b->groups) b->device_bytes_cached += g.bytes;
 	b->finalized = true;
 	return 0;
 }

@@ -78,6 +78,7 @@ struct cla_block {
 	int32_t totalVals = 0;           // sum of nVals over groups (+1 row for constV)
 	int32_t totalColsG = 0;          // sum of nColG over groups
 	int32_t maxVals = 0;
+	int64_t device_bytes_cached = 0; // HBM bytes of the compressed representation (set at finalize)
 
 	hipStream_t stream = nullptr;
 	bool ownStream = false;
@@ -135,6 +136,8 @@ int launch_rmm_mfma(cla_block* b, const double* dB, int q, const double* dConstR
 	unsigned long long* dNnz);
 int launch_lmm_sdc_tiles(cla_block* b, const double* dY, int p, double* dPre, int onlyGroup);
 int launch_rmm_sdc_tiles(cla_block* b, int q, int constRow, int accumulate, double* dOut, unsigned long long* dNnz);
+int launch_rmm_decode(cla_block* b, const double* dB, int q, const double* dConstRow, double* dOut,
+	unsigned long long* dNnz);
 int launch_decompress(cla_block* b, double* dOut, unsigned long long* dNnz);
 int launch_lmm(cla_block* b, const double* dY, int p, double* dOut, unsigned long long* dNnz);
 int launch_preagg(cla_block* b, int group, const double* dY, int p, double* dPre);

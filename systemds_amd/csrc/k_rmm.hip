@@ -552,6 +552,12 @@ int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned lon
 		if(r <= 0) return r;
 	}
 
+	// narrow B on any group mix: decode rows from LDS dictionaries, B rows as scalars
+	if(q >= 2 && q <= 16 && !getenv("CLA_NO_DECODE")) {
+		const int r = launch_rmm_decode(b, dB, q, constRow >= 0 ? b->dTables + (size_t) constRow * q : nullptr, dOut, dNnz);
+		if(r <= 0) return r;
+	}
+
 	// generic path: row-parallel gather for DDC / RLE / uncompressed groups, then the
 	// SDCZeros groups tile by tile (or per-entry scatter when their tables do not fit LDS)
 	{
