@@ -1,133 +1,303 @@
-// Right multiply X %*% B for narrow B (2 <= q <= 16) on blocks of any group mix:
-// every thread decodes one row of X group by group (dictionary copies in LDS) and
-// accumulates value x B[col, :] with B rows as scalar operands. Codes, offset lists,
-// runs and dense columns are read once, the output tile is staged in LDS and written
-// with full-line stores. (Wide B on all-DDC blocks uses k_rmm_mfma instead.)
+// Right multiply X %*% B for narrow B (2 <= q <= 16) on blocks of any group mix.
+// A block owns a contiguous range of 1024-row tiles. Per tile every dictionary
+// coded group gets its codes expanded into an LDS code tile (DDC: straight copy,
+// prefetched one tile ahead in registers; SDCZeros: wave-wide offset decode from
+// the tile index; RLE: run expansion with the run cursor carried from tile to
+// tile). Each thread then decodes two rows group by group from dictionary copies
+// in LDS and accumulates value x B[col, :]; B is kept in LDS in decoded column
+// order. The output tile is staged in LDS and written with full-line stores.
+// (Wide B on all-DDC blocks uses k_rmm_mfma instead.)
 #include "../../include/cla_hip.h"
 #include "cla_device.hpp"
 #include <algorithm>
 
 namespace cla {
 
-constexpr int DEC_THREADS = 512;       // rows per half tile, one row per thread
+constexpr int DEC_THREADS = 512;       // one thread per row of a half tile
 constexpr int DEC_TILE = SDC_TILE;     // rows per tile = granularity of the offset tile index
 constexpr int DEC_QMAX = 16;
+constexpr int DEC_PF = 4;              // 16-byte code chunks a thread holds for the next tile
 
-struct DecPlan {
-	int32_t dictOff;   // offset (doubles) of the group's dictionary copy in LDS, -1 = not dictionary coded
-	int32_t sdcSlot;   // SDCZeros: index of the group's code tile in LDS, else -1
+struct DecGroup {
+	int32_t type;
+	int32_t nC;
+	int32_t dictOff;   // doubles, into the LDS dictionary copy (-1: dense group)
+	int32_t slotOff;   // bytes, into the LDS code tiles (-1: dense group)
+	int32_t slotW;     // 1 or 2 bytes per code in the tile; all ones = row has no value
+	int32_t kOff;      // first decoded column of the group (row of the LDS copy of B)
+	int32_t copyIdx;   // DDC with codeWidth == slotW: index in the chunk copy list, else -1
+	int32_t pad;
 };
 
-template <int Q>
-__global__ __launch_bounds__(DEC_THREADS) void k_rmm_decode(const DGroup* __restrict__ groups, int nGroups,
-	const DecPlan* __restrict__ plan, int dictDoubles, int nSdc, const double* __restrict__ B, int q,
-	const double* __restrict__ constRow, double* __restrict__ out, int64_t nRows, unsigned long long* __restrict__ nnz) {
-	extern __shared__ double smem[];
-	double* dictS = smem;                                   // dictDoubles
-	double* otile = dictS + dictDoubles;                    // DEC_THREADS * Q (padded row stride Q + 1 when Q even)
-	int32_t* sdcCodes = (int32_t*) (otile + (size_t) DEC_THREADS * (Q + 1)); // nSdc * DEC_TILE
-	int32_t* runBase = sdcCodes + (size_t) nSdc * DEC_TILE; // nGroups
-	const int tid = threadIdx.x, wave = tid >> 6;
-	constexpr int OS = Q + 1; // LDS row stride of the output tile (odd: conflict-free column access)
+// Chunk copy list: DDC groups whose code tile is a plain copy of 1024 codes.
+struct DecCopy {
+	int32_t group;
+	int32_t chunk0;    // first 16-byte chunk of this group in the flattened chunk numbering
+};
 
-	// dictionary copies, once per block
+struct DecArgs {
+	const DGroup* groups;
+	const DecGroup* plan;
+	const DecCopy* copies;
+	int nGroups, nCopies, nChunks;     // nChunks: 16-byte chunks per tile over all copy-list groups
+	int dictDoubles, slotBytes, K;     // LDS sizes: dictionaries, code tiles, decoded columns
+	const double* B;
+	int q;
+	const double* constRow;
+	double* out;
+	int64_t nRows;
+	unsigned long long* nnz;
+};
+
+__device__ __forceinline__ void dec_store_code(uint8_t* slot, int w, int i, int code) {
+	if(w == 1) slot[i] = (uint8_t) code;
+	else ((uint16_t*) slot)[i] = (uint16_t) code;
+}
+
+template <int Q>
+__global__ __launch_bounds__(DEC_THREADS) void k_rmm_decode(const DecArgs A) {
+	extern __shared__ __align__(16) double smem[];
+	constexpr int OS = Q + 1; // LDS row stride of the output tile (odd: conflict-free column access)
+	double* dictS = smem;                                         // dictDoubles
+	double* Bs = dictS + A.dictDoubles;                           // K * Q, zero padded columns
+	double* otile = Bs + (size_t) A.K * Q;                        // DEC_THREADS * OS
+	uint8_t* slots = (uint8_t*) (smem + (((size_t) A.dictDoubles + (size_t) A.K * Q + (size_t) DEC_THREADS * OS + 1) & ~(size_t) 1)); // slotBytes, 16-byte aligned
+	DecGroup* planS = (DecGroup*) (slots + A.slotBytes);          // nGroups
+	int32_t* runBase = (int32_t*) (planS + A.nGroups);            // nGroups
+	DecCopy* copyS = (DecCopy*) (runBase + A.nGroups);            // nCopies
+	const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+	const DGroup* __restrict__ groups = A.groups;
+	const int nGroups = A.nGroups;
+	const int64_t nRows = A.nRows;
+
+	const int nTiles = (int) ((nRows + DEC_TILE - 1) / DEC_TILE);
+	const int tileBeg = (int) ((int64_t) nTiles * blockIdx.x / gridDim.x);
+	const int tileEnd = (int) ((int64_t) nTiles * (blockIdx.x + 1) / gridDim.x);
+	if(tileBeg >= tileEnd) return;
+
+	// ---- once per block: plan, dictionaries, B in decoded column order, run cursors
+	for(int g = tid; g < nGroups; g += DEC_THREADS) {
+		planS[g] = A.plan[g];
+		runBase[g] = groups[g].type == G_RLE ? rle_find(groups[g].runStart, groups[g].nRuns, (int32_t) ((int64_t) tileBeg * DEC_TILE)) : 0;
+	}
+	for(int i = tid; i < A.nCopies; i += DEC_THREADS) copyS[i] = A.copies[i];
+	for(int i = tid; i < A.dictDoubles; i += DEC_THREADS) dictS[i] = 0.0;
+	__syncthreads();
 	for(int g = 0; g < nGroups; g++) {
-		const int off = plan[g].dictOff;
-		if(off < 0) continue;
+		const DecGroup P = planS[g];
 		const DGroup& G = groups[g];
-		const int n = G.nVals * G.nColG;
-		for(int i = tid; i < n; i += DEC_THREADS) dictS[off + i] = G.dict[i];
+		if(P.dictOff >= 0) {
+			const int n = G.nVals * G.nColG;
+			for(int i = tid; i < n; i += DEC_THREADS) dictS[P.dictOff + i] = G.dict[i];
+		}
+		for(int i = tid; i < P.nC * Q; i += DEC_THREADS) {
+			const int h = i / Q, c = i - h * Q;
+			Bs[(size_t) (P.kOff + h) * Q + c] = c < A.q ? A.B[(size_t) G.cols[h] * A.q + c] : 0.0;
+		}
 	}
 	double cadd[Q];
 #pragma unroll
-	for(int c = 0; c < Q; c++) cadd[c] = (constRow != nullptr && c < q) ? constRow[c] : 0.0;
+	for(int c = 0; c < Q; c++) cadd[c] = (A.constRow != nullptr && c < A.q) ? A.constRow[c] : 0.0;
 
-	const int nTiles = (int) ((nRows + DEC_TILE - 1) / DEC_TILE);
-	int cnt = 0;
-	for(int tile = blockIdx.x; tile < nTiles; tile += gridDim.x) {
-		const int64_t t0 = (int64_t) tile * DEC_TILE;
-		__syncthreads();
-		for(int i = tid; i < nSdc * DEC_TILE; i += DEC_THREADS) sdcCodes[i] = -1;
-		// one binary search per RLE group and tile
-		for(int g = tid; g < nGroups; g += DEC_THREADS)
-			if(groups[g].type == G_RLE) runBase[g] = rle_find(groups[g].runStart, groups[g].nRuns, (int32_t) t0);
-		__syncthreads();
-		// SDCZeros lists of this tile -> per-row codes in LDS (one wave per group)
-		for(int g = wave; g < nGroups; g += DEC_THREADS / 64) {
-			const int slot = plan[g].sdcSlot;
-			if(slot < 0) continue;
-			const DGroup& G = groups[g];
-			if(G.nOffsets <= 0) continue;
-			int32_t* ct = sdcCodes + (size_t) slot * DEC_TILE;
-			const int64_t rEnd = t0 + DEC_TILE;
-			if((tid & 63) == 0 && G.first >= t0 && G.first < rEnd) ct[G.first - t0] = load_code(G.codes, G.codeWidth, 0);
-			if(tile < G.nTiles) {
-				const OffState st = G.tileIdx[tile];
-				int32_t row = st.row, emit = st.emit;
-				int64_t i0 = st.idx;
-				while(i0 < G.nDeltas && row < rEnd) {
-					int32_t rows[4], didx[4];
-					unsigned mask;
-					if(G.deltaWidth == 1) sdc_decode256<1>(G.deltas, G.nDeltas, i0, row, emit, rows, didx, mask);
-					else sdc_decode256<2>(G.deltas, G.nDeltas, i0, row, emit, rows, didx, mask);
+	// DDC code chunks of one tile, flattened over the copy list: chunk i of a thread is
+	// tid + k * DEC_THREADS, so its group and place in the tile never change. Whole
+	// chunks are loaded as 16 bytes one tile ahead; the ragged end of the last tile is
+	// copied element-wise.
+	auto chunk_place = [&](int i, const uint8_t*& src, int& dstOff, int& w, int& row) {
+		int lo = 0, hi = A.nCopies - 1;
+		while(lo < hi) {
+			const int mid = (lo + hi + 1) >> 1;
+			if(copyS[mid].chunk0 <= i) lo = mid; else hi = mid - 1;
+		}
+		const DecCopy C = copyS[lo];
+		const DecGroup P = planS[C.group];
+		w = P.slotW;
+		const int ci = i - C.chunk0;
+		row = ci * (16 / w);
+		src = (const uint8_t*) groups[C.group].codes + (size_t) ci * 16;
+		dstOff = P.slotOff + ci * 16;
+	};
+	auto copy_ragged = [&](const uint8_t* src, int dstOff, int w, int64_t row0) {
+		for(int e = 0; e < 16 / w; e++)
+			if(row0 + e < nRows) {
+				if(w == 1) slots[dstOff + e] = src[e];
+				else ((uint16_t*) (slots + dstOff))[e] = ((const uint16_t*) src)[e];
+			}
+	};
+	const uint8_t* pfSrc[DEC_PF];
+	int pfDst[DEC_PF], pfW[DEC_PF], pfRow[DEC_PF];
+	u32x4 pf[DEC_PF];
 #pragma unroll
-					for(int k = 0; k < 4; k++)
-						if((mask & (1u << k)) && rows[k] < rEnd) ct[rows[k] - t0] = load_code(G.codes, G.codeWidth, didx[k]);
-					i0 += 256;
+	for(int k = 0; k < DEC_PF; k++) {
+		pfSrc[k] = nullptr; pfDst[k] = 0; pfW[k] = 1; pfRow[k] = 0;
+		if(tid + k * DEC_THREADS < A.nChunks) chunk_place(tid + k * DEC_THREADS, pfSrc[k], pfDst[k], pfW[k], pfRow[k]);
+	}
+	auto prefetch = [&](int tile) {
+		const int64_t t0 = (int64_t) tile * DEC_TILE;
+#pragma unroll
+		for(int k = 0; k < DEC_PF; k++) {
+			pf[k] = u32x4{0, 0, 0, 0};
+			if(pfSrc[k] != nullptr && t0 + pfRow[k] + 16 / pfW[k] <= nRows)
+				pf[k] = __builtin_nontemporal_load((const u32x4*) (pfSrc[k] + t0 * pfW[k]));
+		}
+	};
+	prefetch(tileBeg);
+
+	int cnt = 0;
+	for(int tile = tileBeg; tile < tileEnd; tile++) {
+		const int64_t t0 = (int64_t) tile * DEC_TILE;
+		const int64_t rEnd = t0 + DEC_TILE;
+		__syncthreads(); // previous tile's readers are done with the code tiles
+		// ---- DDC tiles: prefetched chunks, then what did not fit the prefetch registers
+#pragma unroll
+		for(int k = 0; k < DEC_PF; k++) {
+			if(pfSrc[k] == nullptr) continue;
+			if(t0 + pfRow[k] + 16 / pfW[k] <= nRows) *(u32x4*) (slots + pfDst[k]) = pf[k];
+			else copy_ragged(pfSrc[k] + t0 * pfW[k], pfDst[k], pfW[k], t0 + pfRow[k]);
+		}
+		for(int i = tid + DEC_PF * DEC_THREADS; i < A.nChunks; i += DEC_THREADS) {
+			const uint8_t* src; int dstOff, w, row;
+			chunk_place(i, src, dstOff, w, row);
+			if(t0 + row + 16 / w <= nRows) *(u32x4*) (slots + dstOff) = __builtin_nontemporal_load((const u32x4*) (src + t0 * w));
+			else copy_ragged(src + t0 * w, dstOff, w, t0 + row);
+		}
+		if(tile + 1 < tileEnd) prefetch(tile + 1);
+
+		// ---- other dictionary coded groups, one wave per group
+		for(int g = wave; g < nGroups; g += DEC_THREADS / 64) {
+			const DecGroup P = planS[g];
+			if(P.slotOff < 0 || P.copyIdx >= 0) continue;
+			const DGroup& G = groups[g];
+			uint8_t* slot = slots + P.slotOff;
+			const int w = P.slotW;
+			if(P.type == G_DDC) { // code width differs from the tile's: convert
+				for(int i = lane; i < DEC_TILE; i += 64)
+					if(t0 + i < nRows) dec_store_code(slot, w, i, load_code(G.codes, G.codeWidth, t0 + i));
+			}
+			else if(P.type == G_RLE) {
+				int j = runBase[g];
+				while(true) {
+					const int jj = j + lane;
+					const bool inTable = jj < G.nRuns;
+					const int32_t s = inTable ? G.runStart[jj] : 0x7fffffff;
+					const int32_t e = inTable ? G.runStart[jj + 1] : 0x7fffffff;
+					const int32_t code = inTable ? G.runCode[jj] : -1;
+					const unsigned long long valid = __ballot(inTable && s < rEnd);
+					const int nv = __popcll(valid);
+					if(nv <= 8) { // long runs: all lanes write each run
+						for(int k = 0; k < nv; k++) {
+							const int sk = max((int) (__shfl(s, k, 64) - t0), 0);
+							const int ek = (int) (min((int64_t) __shfl(e, k, 64), rEnd) - t0);
+							const int ck = __shfl(code, k, 64);
+							for(int i = sk + lane; i < ek; i += 64) dec_store_code(slot, w, i, ck);
+						}
+					}
+					else if(inTable && s < rEnd) { // short runs: one run per lane
+						const int sk = max((int) (s - t0), 0);
+						const int ek = (int) (min((int64_t) e, rEnd) - t0);
+						for(int i = sk; i < ek; i++) dec_store_code(slot, w, i, code);
+					}
+					if(nv < 64) { j += max(nv - 1, 0); break; }      // base: last run starting before the tile end
+					if(__shfl(e, 63, 64) >= rEnd) { j += 63; break; }
+					j += 64;
+				}
+				j = min(j, G.nRuns - 1);
+				if(lane == 0) runBase[g] = j;
+			}
+			else { // SDCZeros: rows without an entry hold the no-value code
+				for(int i = lane; i < DEC_TILE; i += 64) dec_store_code(slot, w, i, 0xffff);
+				if(G.nOffsets <= 0) continue;
+				// same-wave LDS writes are ordered, no barrier needed between fill and scatter
+				if(lane == 0 && G.first >= t0 && G.first < rEnd) dec_store_code(slot, w, (int) (G.first - t0), load_code(G.codes, G.codeWidth, 0));
+				if(tile < G.nTiles) {
+					const OffState st = G.tileIdx[tile];
+					int32_t row = st.row, emit = st.emit;
+					int64_t i0 = st.idx;
+					while(i0 < G.nDeltas && row < rEnd) {
+						int32_t rows[4], didx[4];
+						unsigned mask;
+						if(G.deltaWidth == 1) sdc_decode256<1>(G.deltas, G.nDeltas, i0, row, emit, rows, didx, mask);
+						else sdc_decode256<2>(G.deltas, G.nDeltas, i0, row, emit, rows, didx, mask);
+#pragma unroll
+						for(int k = 0; k < 4; k++)
+							if((mask & (1u << k)) && rows[k] < rEnd)
+								dec_store_code(slot, w, (int) (rows[k] - t0), load_code(G.codes, G.codeWidth, didx[k]));
+						i0 += 256;
+					}
 				}
 			}
 		}
 		__syncthreads();
-		for(int half = 0; half < DEC_TILE / DEC_THREADS; half++) {
-			const int rt = half * DEC_THREADS + tid; // row inside the tile
-			const int64_t r = t0 + rt;
-			double acc[Q];
+
+		// ---- decode two rows per thread
+		double acc0[Q], acc1[Q];
 #pragma unroll
-			for(int c = 0; c < Q; c++) acc[c] = 0.0;
-			if(r < nRows) {
-				for(int g = 0; g < nGroups; g++) {
-					const DGroup& G = groups[g];
-					const int nC = G.nColG;
-					const double* vals = nullptr;
-					if(G.type == G_DDC) vals = dictS + plan[g].dictOff + (size_t) load_code(G.codes, G.codeWidth, r) * nC;
-					else if(G.type == G_RLE) {
-						int j = runBase[g];
-						while(G.runStart[j + 1] <= r) j++;
-						const int code = G.runCode[j];
-						if(code >= 0) vals = dictS + plan[g].dictOff + (size_t) code * nC;
-					}
-					else if(G.type == G_SDCZ) {
-						const int code = sdcCodes[(size_t) plan[g].sdcSlot * DEC_TILE + rt];
-						if(code >= 0) vals = dictS + plan[g].dictOff + (size_t) code * nC;
-					}
-					else
-						vals = G.dense + (size_t) r * nC;
-					if(vals == nullptr) continue;
-					for(int h = 0; h < nC; h++) {
-						const double a = vals[h];
-						const double* brow = B + (size_t) G.cols[h] * q; // uniform: scalar loads
+		for(int c = 0; c < Q; c++) { acc0[c] = 0.0; acc1[c] = 0.0; }
+		const int rt0 = tid, rt1 = tid + DEC_THREADS;
+		const int64_t r0 = t0 + rt0, r1 = t0 + rt1;
+		const bool in0 = r0 < nRows, in1 = r1 < nRows;
+		for(int g = 0; g < nGroups; g++) {
+			const DecGroup P = planS[g];
+			const int nC = P.nC;
+			if(P.slotOff < 0) { // dense columns
+				const double* dense = groups[g].dense;
+				for(int h = 0; h < nC; h++) {
+					const double a0 = in0 ? dense[(size_t) r0 * nC + h] : 0.0;
+					const double a1 = in1 ? dense[(size_t) r1 * nC + h] : 0.0;
+					const double* bq = Bs + (size_t) (P.kOff + h) * Q;
 #pragma unroll
-						for(int c = 0; c < Q; c++)
-							if(c < q) acc[c] += a * brow[c];
-					}
+					for(int c = 0; c < Q; c++) { const double bv = bq[c]; acc0[c] += a0 * bv; acc1[c] += a1 * bv; }
+				}
+				continue;
+			}
+			int c0, c1;
+			bool v0, v1;
+			if(P.slotW == 1) {
+				c0 = slots[P.slotOff + rt0]; c1 = slots[P.slotOff + rt1];
+				v0 = in0 && c0 != 0xff; v1 = in1 && c1 != 0xff;
+			}
+			else {
+				c0 = ((const uint16_t*) (slots + P.slotOff))[rt0]; c1 = ((const uint16_t*) (slots + P.slotOff))[rt1];
+				v0 = in0 && c0 != 0xffff; v1 = in1 && c1 != 0xffff;
+			}
+			const double* p0 = dictS + P.dictOff + (v0 ? c0 * nC : 0);
+			const double* p1 = dictS + P.dictOff + (v1 ? c1 * nC : 0);
+			for(int h = 0; h < nC; h++) {
+				const double a0 = p0[h], a1 = p1[h];
+				const double* bq = Bs + (size_t) (P.kOff + h) * Q;
+				double bv[Q];
+#pragma unroll
+				for(int c = 0; c < Q; c++) bv[c] = bq[c];
+				if(v0) {
+#pragma unroll
+					for(int c = 0; c < Q; c++) acc0[c] += a0 * bv[c];
+				}
+				if(v1) {
+#pragma unroll
+					for(int c = 0; c < Q; c++) acc1[c] += a1 * bv[c];
 				}
 			}
-			__syncthreads(); // previous half's stores have read the tile
+		}
+
+		// ---- output: two half tiles through LDS, full-line stores
+		const int q = A.q;
 #pragma unroll
-			for(int c = 0; c < Q; c++) otile[tid * OS + c] = acc[c] + cadd[c];
+		for(int half = 0; half < 2; half++) {
+			if(half == 1) __syncthreads(); // the first half has been read
+#pragma unroll
+			for(int c = 0; c < Q; c++) otile[tid * OS + c] = (half == 0 ? acc0[c] : acc1[c]) + cadd[c];
 			__syncthreads();
-			// coalesced write of the half tile: rows [t0 + half*DEC_THREADS, +DEC_THREADS) x q
 			const int64_t rowBase = t0 + (int64_t) half * DEC_THREADS;
 			const int nr = (int) max((int64_t) 0, min((int64_t) DEC_THREADS, nRows - rowBase));
 			for(int i = tid; i < nr * q; i += DEC_THREADS) {
 				const int rr = i / q, c = i - rr * q;
 				const double v = otile[rr * OS + c];
 				cnt += v != 0.0;
-				__builtin_nontemporal_store(v, out + (size_t) rowBase * q + i);
+				__builtin_nontemporal_store(v, A.out + (size_t) rowBase * q + i);
 			}
 		}
 	}
-	count_add(nnz, cnt);
+	count_add(A.nnz, cnt);
 }
 
 // Returns 1 when the block/shape is not eligible (caller uses the generic path).
@@ -135,35 +305,56 @@ int launch_rmm_decode(cla_block* b, const double* dB, int q, const double* dCons
 	unsigned long long* dNnz) {
 	const int nG = (int) b->groups.size();
 	if(nG == 0 || b->nRows == 0 || q < 2 || q > DEC_QMAX) return 1;
-	std::vector<DecPlan> plan((size_t) nG);
-	size_t dictD = 0;
-	int nSdc = 0;
+	const int Q = q <= 4 ? 4 : q <= 8 ? 8 : q <= 12 ? 12 : 16;
+	std::vector<DecGroup> plan((size_t) nG);
+	std::vector<DecCopy> copies;
+	size_t dictD = 0, slotB = 0;
+	int K = 0, nChunks = 0;
 	for(int g = 0; g < nG; g++) {
 		const DGroup& G = b->groups[g].d;
-		plan[g].dictOff = -1; plan[g].sdcSlot = -1;
+		DecGroup& P = plan[g];
+		P.type = G.type; P.nC = G.nColG; P.dictOff = -1; P.slotOff = -1; P.slotW = 0; P.copyIdx = -1; P.pad = 0;
+		P.kOff = K;
+		K += G.nColG;
 		if(G.type == G_UNC) continue;
-		plan[g].dictOff = (int32_t) dictD;
+		if(G.nVals > 65535) return 1;
+		P.dictOff = (int32_t) dictD;
 		dictD += (size_t) G.nVals * G.nColG;
-		if(G.type == G_SDCZ) plan[g].sdcSlot = nSdc++;
+		P.slotW = G.nVals <= 255 ? 1 : 2;
+		P.slotOff = (int32_t) slotB;
+		slotB += (size_t) DEC_TILE * P.slotW;
+		if(G.type == G_DDC && G.codeWidth == P.slotW && ((uintptr_t) G.codes & 15) == 0) {
+			P.copyIdx = (int32_t) copies.size();
+			copies.push_back(DecCopy{g, nChunks});
+			nChunks += DEC_TILE * P.slotW / 16;
+		}
 	}
-	const int Q = q <= 4 ? 4 : q <= 8 ? 8 : q <= 12 ? 12 : 16;
-	const size_t lds = dictD * 8 + (size_t) DEC_THREADS * (Q + 1) * 8 + (size_t) nSdc * DEC_TILE * 4 + (size_t) nG * 4 + 64;
+	if(dictD == 0) dictD = 1;
+	const size_t lds = dictD * 8 + (size_t) K * Q * 8 + (size_t) DEC_THREADS * (Q + 1) * 8 + slotB +
+		(size_t) nG * (sizeof(DecGroup) + 4) + copies.size() * sizeof(DecCopy) + 96;
 	if(lds > (size_t) std::min(g_ldsPerBlock, 160 * 1024) - 1024) return 1;
-	int rc = ensure_scratch(b, plan.size() * sizeof(DecPlan) + 64);
+	const size_t planBytes = plan.size() * sizeof(DecGroup), copyBytes = copies.size() * sizeof(DecCopy);
+	int rc = ensure_scratch(b, planBytes + copyBytes + 64);
 	if(rc) return rc;
-	DecPlan* dPlan = (DecPlan*) b->dScratch;
-	CLA_HIP(hipMemcpyAsync(dPlan, plan.data(), plan.size() * sizeof(DecPlan), hipMemcpyHostToDevice, b->stream));
+	DecGroup* dPlan = (DecGroup*) b->dScratch;
+	DecCopy* dCopies = (DecCopy*) ((uint8_t*) b->dScratch + planBytes);
+	CLA_HIP(hipMemcpyAsync(dPlan, plan.data(), planBytes, hipMemcpyHostToDevice, b->stream));
+	if(copyBytes) CLA_HIP(hipMemcpyAsync(dCopies, copies.data(), copyBytes, hipMemcpyHostToDevice, b->stream));
 	CLA_HIP(hipStreamSynchronize(b->stream));
 	const int nTiles = (int) ((b->nRows + DEC_TILE - 1) / DEC_TILE);
 	const int blocksPerCU = lds <= 76 * 1024 ? 2 : 1;
 	const unsigned grid = (unsigned) std::min(nTiles, g_numCU * blocksPerCU);
+	DecArgs A;
+	A.groups = b->dGroups; A.plan = dPlan; A.copies = dCopies;
+	A.nGroups = nG; A.nCopies = (int) copies.size(); A.nChunks = nChunks;
+	A.dictDoubles = (int) dictD; A.slotBytes = (int) ((slotB + 15) & ~(size_t) 15); A.K = K;
+	A.B = dB; A.q = q; A.constRow = dConstRow; A.out = dOut; A.nRows = b->nRows; A.nnz = dNnz;
 	double algo = (double) b->device_bytes_cached + (double) b->nRows * q * 8;
 	Prof pf(b, "k_rmm_decode", grid, DEC_THREADS, (long) lds, algo);
 #define DEC_LAUNCH(QV)                                                                                          \
 	do {                                                                                                        \
 		CLA_HIP(hipFuncSetAttribute((const void*) k_rmm_decode<QV>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds)); \
-		hipLaunchKernelGGL(k_rmm_decode<QV>, dim3(grid), dim3(DEC_THREADS), lds, b->stream, b->dGroups, nG, dPlan, (int) dictD, \
-			nSdc, dB, q, dConstRow, dOut, b->nRows, dNnz);                                                      \
+		hipLaunchKernelGGL(k_rmm_decode<QV>, dim3(grid), dim3(DEC_THREADS), lds, b->stream, A);                 \
 	} while(0)
 	if(Q == 4) DEC_LAUNCH(4);
 	else if(Q == 8) DEC_LAUNCH(8);
