@@ -28,6 +28,26 @@ def build_lib(verbose=True):
     return LIB
 
 
+HOST_DIR = os.path.join(HERE, "host")
+HOST_LIB = os.path.join(HOST_DIR, "_clahost.so")
+
+
+def build_host(verbose=True):
+    """The C++ host layer (host/cla_host.hpp) as a Python module over libclahip.so."""
+    import sysconfig
+    import pybind11
+    cxx = os.environ.get("CXX", "g++")
+    cmd = [cxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden", "-Wall",
+           "-I" + sysconfig.get_paths()["include"], "-I" + pybind11.get_include(),
+           os.path.join(HOST_DIR, "bindings.cpp"), "-o", HOST_LIB,
+           "-L" + HERE, "-lclahip", "-Wl,-rpath,$ORIGIN/.."]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.run(cmd, check=True)
+    return HOST_LIB
+
+
 if __name__ == "__main__":
     build_lib()
+    build_host()
     sys.exit(0)

@@ -80,4 +80,44 @@ def mixed_block(seed, n_rows, with_unc=True, with_const=True, overlap=False):
     if with_const:
         specs.append(synth.GroupSpec("const", cols(1), np.array([[2.5]])))
         specs.append(synth.GroupSpec("empty", cols(1)))
+    if overlap:  # groups over columns that other groups already cover: the values add up
+        specs.append(synth.GroupSpec("ddc", np.array([0, 2], np.int32), rng.standard_normal((9, 2)),
+                                     rng.integers(0, 9, n_rows).astype(np.uint8)))
+        specs.append(synth.sdc_group(rng, n_rows, [1, 4], 3, 0.2, 0.5))
     return specs, c
+
+
+@pytest.fixture(scope="session")
+def H():
+    """The C++ host layer (systemds_amd/host) as a Python module."""
+    from systemds_amd import host
+    return host.load()
+
+
+def host_groups(H, ora, specs, n_rows):
+    """GroupSpec list -> column groups built with the host layer's factories."""
+    out = []
+    for s in specs:
+        cols = np.asarray(s.cols, np.int32)
+        if s.type == "ddc":
+            out.append(H.ColGroupDDC.create(cols, H.Dictionary.create(s.dict),
+                                            H.MapToFactory.create(s.n_vals, s.codes.astype(np.int32))))
+        elif s.type == "sdc":
+            rows = ora.py_offset_decode(s.deltas, s.first) if s.n_offsets else np.zeros(0, np.int64)
+            width = H.OFF_TYPE.BYTE if s.deltas.dtype == np.uint8 else H.OFF_TYPE.CHAR
+            off = H.OffsetFactory.createOffset(rows.astype(np.int32), width)
+            mp = H.MapToFactory.create(s.n_vals, s.codes.astype(np.int32))
+            d = H.Dictionary.create(s.dict)
+            if s.default is None:
+                out.append(H.ColGroupSDCZeros.create(cols, n_rows, d, off, mp))
+            else:
+                out.append(H.ColGroupSDC.create(cols, n_rows, d, s.default, off, mp))
+        elif s.type == "rle":
+            out.append(H.ColGroupRLE.create(cols, n_rows, H.Dictionary.create(s.dict), s.rle.tolist(), s.ptr))
+        elif s.type == "unc":
+            out.append(H.ColGroupUncompressed.create(H.MatrixBlock(s.dense), cols))
+        elif s.type == "const":
+            out.append(H.ColGroupConst.create(cols, s.dict.reshape(-1)))
+        else:
+            out.append(H.ColGroupEmpty(cols))
+    return out
