@@ -19,9 +19,11 @@ namespace cla {
 // grid.y = group index; grid.y == nGroups computes constV x B.
 // ---------------------------------------------------------------------------
 __global__ void k_preagg(const DGroup* __restrict__ groups, int nGroups, const double* __restrict__ B, int q,
-	int nCols, const double* __restrict__ constV, double* __restrict__ T, int totalVals) {
+	int nCols, const double* __restrict__ constV, double* __restrict__ T, int totalVals,
+	unsigned long long* __restrict__ nnz) {
 	const int g = blockIdx.y;
 	const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+	if(g == 0 && idx == 0) *nnz = 0; // the multiply kernels behind this one on the stream count into it
 	if(g == nGroups) {
 		if(constV == nullptr || idx >= q) return;
 		double acc = 0;
@@ -252,33 +254,78 @@ __global__ __launch_bounds__(THREADS) void k_rmm_q1_ddc(const uint8_t* __restric
 constexpr int U8_RPT = 16;   // rows per thread = one 16-byte load per group
 
 // U8_PER = groups (tables) per slab (2 KiB of LDS each), U8_NB = groups per load batch,
+// Adds table[code] for NB groups x RPT rows held in registers. The NB * RPT lookups are
+// issued as batches of LB LDS reads with LN batches in flight: the reads of batch b + LN - 1
+// are issued before the adds of batch b, and scheduling barriers pin that order, so a wave
+// keeps (LN - 1) * LB .. LN * LB reads outstanding instead of the one to three the
+// scheduler chooses on its own under register pressure. Group order per row is kept
+// (batches walk group-major), so the sums are bit-identical to the sequential loop.
+template <int RPT, int NB, int LB, int LN>
+__device__ __forceinline__ void u8_consume(const CodeVec<1, RPT> (&cv)[NB], const char* tb, double (&acc)[RPT]) {
+	static_assert(RPT % LB == 0, "a batch stays inside one group");
+	constexpr int NBATCH = NB * RPT / LB;
+	double t[LN][LB];
+	auto issue = [&](int b) {
+		const int j = (b * LB) / RPT, i0 = (b * LB) % RPT;
+#pragma unroll
+		for(int k = 0; k < LB; k++) t[b % LN][k] = *(const double*) (tb + j * 2048 + (cv[j].get(i0 + k) << 3));
+	};
+#pragma unroll
+	for(int b = 0; b < LN - 1 && b < NBATCH; b++) issue(b);
+	__builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+	for(int b = 0; b < NBATCH; b++) {
+		if(b + LN - 1 < NBATCH) issue(b + LN - 1);
+		__builtin_amdgcn_sched_barrier(0);
+		const int i0 = (b * LB) % RPT;
+#pragma unroll
+		for(int k = 0; k < LB; k++) acc[i0 + k] += t[b % LN][k];
+		__builtin_amdgcn_sched_barrier(0);
+	}
+}
+
 // U8_PER is a multiple of 2 * U8_NB. The host picks the variant that pads least.
-template <int THREADS, int U8_PER, int U8_NB>
-__global__ __launch_bounds__(THREADS) void k_rmm_q1_u8(const uint8_t* __restrict__ arena, size_t arenaStride,
+template <int THREADS, int U8_PER, int U8_NB, int LB, int LN>
+__global__ __launch_bounds__(THREADS, 4) void k_rmm_q1_u8(const uint8_t* __restrict__ arena, size_t arenaStride,
 	int nGroups, const int32_t* __restrict__ tblOff, const double* __restrict__ T, int constIdx,
 	double* __restrict__ out, int64_t nRows, unsigned long long* __restrict__ nnz) {
 	__shared__ double tbl[U8_PER * 256];
+	__shared__ double wbufAll[(THREADS / 64) * 64 * 8]; // per-wave transpose buffers of the epilogue
 	const char* tb = (const char*) tbl;
 	constexpr int RPT = U8_RPT, NB = U8_NB;
 	const int tid = threadIdx.x;
-	const int64_t row0 = ((int64_t) blockIdx.x * THREADS + tid) * RPT;
-	const bool full = row0 + RPT <= nRows;
-	const bool any = row0 < nRows;
-	const uint8_t* myCodes = arena + (size_t) row0;
-	double acc[RPT];
-#pragma unroll
-	for(int i = 0; i < RPT; i++) acc[i] = 0.0;
+	const int off = tid * RPT; // first row of this thread inside a pass
+	const int gLast = nGroups - 1;
+	const int nPad = (nGroups + U8_PER - 1) / U8_PER * U8_PER; // groups incl. the zero-table slots of the last slab
+
+	// The block is persistent: it owns an equal share of the rows (a multiple of 16) and covers
+	// it in nPass equally filled passes of at most THREADS * RPT rows, so all blocks finish
+	// together and the load pipeline (codes two batches ahead, tables one slab ahead) keeps
+	// running from pass to pass. Everything about a pass but `off` is uniform.
+	const int64_t share = ((nRows + gridDim.x - 1) / gridDim.x + RPT - 1) / RPT * RPT;
+	const int64_t blockBeg = (int64_t) blockIdx.x * share;
+	if(blockBeg >= nRows) return;
+	const int blockLen = (int) (min(nRows, blockBeg + share) - blockBeg);
+	const int nPass = (blockLen + THREADS * RPT - 1) / (THREADS * RPT);
+	const int passRows = ((blockLen + nPass - 1) / nPass + RPT - 1) / RPT * RPT;
+
+	int passLen = min(passRows, blockLen);
+	bool full = off + RPT <= passLen;
+	const uint8_t* myCodes = arena + (size_t) blockBeg + (full ? off : 0);
+
 	CodeVec<1, RPT> ping[NB], pong[NB];
-	if(full) q1_load<1, RPT, NB>(ping, myCodes, arenaStride, 0, nGroups - 1);
+	if(full) q1_load<1, RPT, NB>(ping, myCodes, arenaStride, 0, gLast);
 
 	// the tables of the next slab are fetched into registers while the current slab is processed
 	constexpr int TPT = (U8_PER * 256 + THREADS - 1) / THREADS;
 	double stage[TPT];
 	auto fetch = [&](int g0) {
 		const int nIn = min(U8_PER, nGroups - g0);
+		int tidF = tid; // laundered like tidE below: keeps the index arithmetic out of registers between uses
+		asm volatile("" : "+v"(tidF));
 #pragma unroll
 		for(int k = 0; k < TPT; k++) {
-			const int f = tid + k * THREADS;
+			const int f = tidF + k * THREADS;
 			const int g = f >> 8, i = f & 255;
 			double v = 0.0;
 			if(g < nIn) {
@@ -289,80 +336,99 @@ __global__ __launch_bounds__(THREADS) void k_rmm_q1_u8(const uint8_t* __restrict
 		}
 	};
 	fetch(0);
-	for(int g0 = 0; g0 < nGroups; g0 += U8_PER) {
-		const int nIn = min(U8_PER, nGroups - g0);
-		__syncthreads();
+	const double cadd = constIdx >= 0 ? T[constIdx] : 0.0;
+	int cnt = 0;
+	for(int pass = 0; pass < nPass; pass++) {
+		const int64_t passBeg = blockBeg + (int64_t) pass * passRows;
+		// the first batch of the next pass is requested in the last batch slot of this pass; a
+		// thread without a full next pass requests valid but unused bytes instead, so that the
+		// number of loads in flight never depends on a branch
+		const int nextLen = pass + 1 < nPass ? min(passRows, blockLen - (pass + 1) * passRows) : 0;
+		const bool nfull = off + RPT <= nextLen;
+		const uint8_t* nextCodes = nfull ? arena + (size_t) (passBeg + passRows) + off : myCodes;
+		double acc[RPT];
 #pragma unroll
-		for(int k = 0; k < TPT; k++) {
-			const int f = tid + k * THREADS;
-			if(f < U8_PER * 256) tbl[f] = stage[k];
-		}
-		__syncthreads();
-		if(g0 + U8_PER < nGroups) fetch(g0 + U8_PER);
-		if(full) {
+		for(int i = 0; i < RPT; i++) acc[i] = 0.0;
+		for(int g0 = 0; g0 < nGroups; g0 += U8_PER) {
+			const int nIn = min(U8_PER, nGroups - g0);
+			__syncthreads();
+			int tidW = tid;
+			asm volatile("" : "+v"(tidW));
 #pragma unroll
-			for(int s = 0; s < U8_PER; s += 2 * NB) {
-				q1_load<1, RPT, NB>(pong, myCodes, arenaStride, g0 + s + NB, nGroups - 1);
+			for(int k = 0; k < TPT; k++) {
+				const int f = tidW + k * THREADS;
+				if(f < U8_PER * 256) tbl[f] = stage[k];
+			}
+			__syncthreads();
+			fetch(g0 + U8_PER < nGroups ? g0 + U8_PER : 0);
+			if(full) {
 #pragma unroll
-				for(int j = 0; j < NB; j++) {
-#pragma unroll
-					for(int i = 0; i < RPT; i++) acc[i] += *(const double*) (tb + (s + j) * 2048 + (ping[j].get(i) << 3));
+				for(int s = 0; s < U8_PER; s += 2 * NB) {
+					q1_load<1, RPT, NB>(pong, myCodes, arenaStride, g0 + s + NB, gLast);
+					u8_consume<RPT, NB, LB, LN>(ping, tb + s * 2048, acc);
+					const int gn = g0 + s + 2 * NB;
+					const bool wrap = gn >= nPad;
+					q1_load<1, RPT, NB>(ping, wrap ? nextCodes : myCodes, arenaStride, wrap ? 0 : gn, gLast);
+					u8_consume<RPT, NB, LB, LN>(pong, tb + (s + NB) * 2048, acc);
 				}
-				q1_load<1, RPT, NB>(ping, myCodes, arenaStride, g0 + s + 2 * NB, nGroups - 1);
-#pragma unroll
-				for(int j = 0; j < NB; j++) {
+			}
+			else if(off < passLen) {
+				for(int g = 0; g < nIn; g++) {
+					const uint8_t* codes = arena + (size_t) (g0 + g) * arenaStride + passBeg;
 #pragma unroll
 					for(int i = 0; i < RPT; i++)
-						acc[i] += *(const double*) (tb + (s + NB + j) * 2048 + (pong[j].get(i) << 3));
+						if(off + i < passLen) acc[i] += tbl[g * 256 + codes[off + i]];
 				}
 			}
 		}
-		else if(any) {
-			for(int g = 0; g < nIn; g++) {
-				const uint8_t* codes = arena + (size_t) (g0 + g) * arenaStride;
-#pragma unroll
-				for(int i = 0; i < RPT; i++)
-					if(row0 + i < nRows) acc[i] += tbl[g * 256 + codes[row0 + i]];
-			}
-		}
-	}
 
-	// Epilogue. A thread holds 16 consecutive rows, so direct stores would touch 64
-	// different lines per instruction with 16 bytes each (measured: 2.9x write
-	// amplification). Full tiles are transposed through LDS in two halves of 8 rows per
-	// thread instead, so that 8 consecutive lanes write one 64-byte segment.
-	int cnt = 0;
-	const double cadd = constIdx >= 0 ? T[constIdx] : 0.0;
-	const bool tileFull = (int64_t) (blockIdx.x + 1) * THREADS * RPT <= nRows;
-	if(tileFull) {
-		const int wave = tid >> 6, lane = tid & 63;
-		double* wbuf = tbl + wave * (64 * 8); // 8 values per lane, XOR-swizzled against bank conflicts
-		double* obase = out + ((int64_t) blockIdx.x * THREADS + wave * 64) * RPT;
+		// Epilogue. A thread holds 16 consecutive rows, so direct stores would touch 64
+		// different lines per instruction with 16 bytes each (measured: 2.9x write
+		// amplification). Waves whose 64 threads all hold full rows transpose through LDS in
+		// two halves of 8 rows per thread instead, so that 8 consecutive lanes write one
+		// 64-byte segment. The buffer is private to the wave and LDS executes a wave's
+		// accesses in order, so no block barrier is needed.
+		// (the empty asm keeps the epilogue's address arithmetic inside the pass loop: hoisted
+		// out of it, it would occupy registers all through the slab loop)
+		int tidE = tid;
+		asm volatile("" : "+v"(tidE));
+		const int wave = tidE >> 6, lane = tidE & 63;
+		if((wave + 1) * 64 * RPT <= passLen) {
+			double* wbuf = wbufAll + wave * (64 * 8); // 8 values per lane, XOR-swizzled against bank conflicts
+			double* obase = out + passBeg + (int64_t) wave * 64 * RPT;
 #pragma unroll
-		for(int h = 0; h < 2; h++) {
-			__syncthreads();
+			for(int h = 0; h < 2; h++) {
 #pragma unroll
-			for(int i = 0; i < 8; i++) {
-				const double v = acc[h * 8 + i] + cadd;
-				cnt += v != 0.0;
-				wbuf[lane * 8 + (i ^ ((lane >> 2) & 7))] = v;
-			}
-			__syncthreads();
+				for(int i = 0; i < 8; i++) {
+					const double v = acc[h * 8 + i] + cadd;
+					cnt += v != 0.0;
+					wbuf[lane * 8 + (i ^ ((lane >> 2) & 7))] = v;
+				}
+				__builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+				__builtin_amdgcn_wave_barrier();
+				__builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
-			for(int j = 0; j < 8; j++) {
-				const int t = j * 64 + lane, sl = t >> 3, i = t & 7;
-				__builtin_nontemporal_store(wbuf[sl * 8 + (i ^ ((sl >> 2) & 7))], obase + sl * RPT + h * 8 + i);
+				for(int j = 0; j < 8; j++) {
+					const int t = j * 64 + lane, sl = t >> 3, i = t & 7;
+					__builtin_nontemporal_store(wbuf[sl * 8 + (i ^ ((sl >> 2) & 7))], obase + sl * RPT + h * 8 + i);
+				}
+				__builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+				__builtin_amdgcn_wave_barrier();
+				__builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 			}
 		}
-	}
-	else if(any) {
+		else if(off < passLen) {
 #pragma unroll
-		for(int i = 0; i < RPT; i++)
-			if(row0 + i < nRows) {
-				const double v = acc[i] + cadd;
-				cnt += v != 0.0;
-				out[row0 + i] = v;
-			}
+			for(int i = 0; i < RPT; i++)
+				if(off + i < passLen) {
+					const double v = acc[i] + cadd;
+					cnt += v != 0.0;
+					out[passBeg + off + i] = v;
+				}
+		}
+		passLen = nextLen;
+		full = nfull;
+		myCodes = nextCodes;
 	}
 	count_add(nnz, cnt);
 }
@@ -480,15 +546,14 @@ int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned lon
 	clear_stats(b);
 	int rc = ensure_tables(b, (size_t) (b->totalVals + 1) * q);
 	if(rc) return rc;
-	CLA_HIP(hipMemsetAsync(dNnz, 0, sizeof(unsigned long long), st));
 
-	// K1
+	// K1 (also clears the non-zero counter)
 	{
 		const int maxWork = (b->maxVals > 1 ? b->maxVals : 1) * q;
 		dim3 grid((maxWork + 255) / 256 > (q + 255) / 256 ? (maxWork + 255) / 256 : (q + 255) / 256, nG + 1);
 		Prof pf(b, "k_preagg", (long) grid.x * grid.y, 256, 0, 0);
 		hipLaunchKernelGGL(k_preagg, grid, dim3(256), 0, st, b->dGroups, nG, dB, q, b->nCols,
-			b->hasConst ? b->dConstV : nullptr, b->dTables, b->totalVals);
+			b->hasConst ? b->dConstV : nullptr, b->dTables, b->totalVals, dNnz);
 	}
 	const int constRow = b->hasConst ? b->totalVals : -1;
 	if(nRows == 0) return 0;
@@ -496,19 +561,24 @@ int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned lon
 	if(q == 1 && b->dArena && b->arenaWidth == 1 && b->maxVals <= 256 && !getenv("CLA_Q1_GENERIC")) {
 		constexpr int THREADS = 512;
 		const int64_t rowsPerBlock = (int64_t) THREADS * U8_RPT;
-		const unsigned grid = (unsigned) ((nRows + rowsPerBlock - 1) / rowsPerBlock);
+		(void) rowsPerBlock;
+		// persistent blocks: two per CU is what the register and LDS footprint allows; small
+		// inputs get a block per 2048 rows
+		int perCU = 2;
+		if(const char* e = getenv("CLA_Q1_BLOCKS_PER_CU")) perCU = std::max(1, atoi(e));
+		const unsigned grid = (unsigned) std::min<int64_t>((nRows + 2047) / 2048, (int64_t) g_numCU * perCU);
 		const double bytes = (double) nRows * nG + (double) nRows * 8 + (double) b->totalVals * 8;
 		// slab size: 16 or 20 groups, whichever leaves fewer padded table slots
 		const int pad16 = (nG + 15) / 16 * 16 - nG, pad20 = (nG + 19) / 20 * 20 - nG;
 		int per = pad20 < pad16 ? 20 : 16;
 		if(const char* e = getenv("CLA_Q1_PER")) per = atoi(e) == 20 ? 20 : 16;
 		Prof pf(b, "k_rmm_q1_u8", grid, THREADS, per * 256 * 8, bytes);
-		if(per == 20)
-			hipLaunchKernelGGL((k_rmm_q1_u8<THREADS, 20, 5>), dim3(grid), dim3(THREADS), 0, st, b->dArena, b->arenaStride,
-				nG, b->dTblOff, b->dTables, constRow, dOut, nRows, dNnz);
-		else
-			hipLaunchKernelGGL((k_rmm_q1_u8<THREADS, 16, 4>), dim3(grid), dim3(THREADS), 0, st, b->dArena, b->arenaStride,
-				nG, b->dTblOff, b->dTables, constRow, dOut, nRows, dNnz);
+#define U8_LAUNCH(PER, NBV, LB, LN)                                                                             \
+	hipLaunchKernelGGL((k_rmm_q1_u8<THREADS, PER, NBV, LB, LN>), dim3(grid), dim3(THREADS), 0, st, b->dArena,   \
+		b->arenaStride, nG, b->dTblOff, b->dTables, constRow, dOut, nRows, dNnz)
+		if(per == 20) U8_LAUNCH(20, 5, 4, 2);
+		else U8_LAUNCH(16, 4, 8, 2);
+#undef U8_LAUNCH
 		CLA_HIP(hipGetLastError());
 		return 0;
 	}
