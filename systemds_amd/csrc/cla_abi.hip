@@ -222,6 +222,7 @@ void cla_block_free(cla_handle b) {
 	if(b->dStageIn) (void) hipFree(b->dStageIn);
 	if(b->dStageOut) (void) hipFree(b->dStageOut);
 	if(b->dScratch) (void) hipFree(b->dScratch);
+	if(b->dSdcPlan) (void) hipFree(b->dSdcPlan);
 	if(b->dCounters) (void) hipFree(b->dCounters);
 	if(b->hCounters) (void) hipHostFree(b->hCounters);
 	if(b->ownStream && b->stream) (void) hipStreamDestroy(b->stream);

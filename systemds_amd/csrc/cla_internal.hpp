@@ -105,6 +105,11 @@ struct cla_block {
 	double* dStageIn = nullptr; size_t stageInCap = 0;
 	double* dStageOut = nullptr; size_t stageOutCap = 0;
 	void* dScratch = nullptr;   size_t scratchCap = 0;
+	// list of SDCZeros groups + prefix sums of their nVals, as the row-tile kernels read it;
+	// built on first use for all groups (sdcPlanGroup -1) or for one group (its index)
+	int32_t* dSdcPlan = nullptr;
+	int sdcPlanGroup = -2;
+	std::vector<int32_t> sdcList, sdcBinOff;
 	unsigned long long* dCounters = nullptr;   // 8 x u64
 	unsigned long long* hCounters = nullptr;   // pinned
 

@@ -140,36 +140,40 @@ __global__ __launch_bounds__(ST_THREADS) void k_rmm_sdc_tiles(const DGroup* __re
 	count_add(nnz, cnt);
 }
 
-// Host side: list of SDCZeros groups and the prefix sums of their nVals.
-struct SdcPlan {
-	std::vector<int32_t> list, binOff;
-};
-
-static void sdc_plan(cla_block* b, int onlyGroup, SdcPlan& p) {
-	p.list.clear();
-	p.binOff.assign(1, 0);
-	for(int g = 0; g < (int) b->groups.size(); g++) {
-		const DGroup& G = b->groups[g].d;
-		if(G.type != G_SDCZ || G.nOffsets == 0 || (onlyGroup >= 0 && onlyGroup != g)) continue;
-		p.list.push_back(g);
-		p.binOff.push_back(p.binOff.back() + G.nVals);
+// Host side: list of SDCZeros groups and the prefix sums of their nVals, kept on the block
+// (host and device copy) and rebuilt only when the requested group selection changes.
+static int sdc_plan(cla_block* b, int onlyGroup, int32_t** dList, int32_t** dBinOff) {
+	const size_t nG = b->groups.size();
+	if(b->dSdcPlan == nullptr) CLA_HIP(hipMalloc((void**) &b->dSdcPlan, (2 * nG + 2) * sizeof(int32_t)));
+	if(b->sdcPlanGroup != onlyGroup) {
+		b->sdcList.clear();
+		b->sdcBinOff.assign(1, 0);
+		for(int g = 0; g < (int) nG; g++) {
+			const DGroup& G = b->groups[g].d;
+			if(G.type != G_SDCZ || G.nOffsets == 0 || (onlyGroup >= 0 && onlyGroup != g)) continue;
+			b->sdcList.push_back(g);
+			b->sdcBinOff.push_back(b->sdcBinOff.back() + G.nVals);
+		}
+		b->sdcPlanGroup = -2; // invalid until both copies have been issued
+		if(!b->sdcList.empty()) {
+			CLA_HIP(hipMemcpyAsync(b->dSdcPlan, b->sdcList.data(), b->sdcList.size() * 4, hipMemcpyHostToDevice, b->stream));
+			CLA_HIP(hipMemcpyAsync(b->dSdcPlan + nG, b->sdcBinOff.data(), b->sdcBinOff.size() * 4, hipMemcpyHostToDevice, b->stream));
+			// the host vectors are rewritten by the next selection: the copies must have read them
+			CLA_HIP(hipStreamSynchronize(b->stream));
+		}
+		b->sdcPlanGroup = onlyGroup;
 	}
-}
-
-static int upload_plan(cla_block* b, const SdcPlan& p, int32_t** dList, int32_t** dBinOff) {
-	const size_t n1 = p.list.size() * 4, n2 = p.binOff.size() * 4;
-	CLA_HIP(hipMalloc((void**) dList, n1 + n2 + 16));
-	*dBinOff = *dList + p.list.size();
-	CLA_HIP(hipMemcpyAsync(*dList, p.list.data(), n1, hipMemcpyHostToDevice, b->stream));
-	CLA_HIP(hipMemcpyAsync(*dBinOff, p.binOff.data(), n2, hipMemcpyHostToDevice, b->stream));
-	CLA_HIP(hipStreamSynchronize(b->stream));
+	*dList = b->dSdcPlan;
+	*dBinOff = b->dSdcPlan + nG;
 	return 0;
 }
 
 // Returns 1 if some SDC group cannot use the tile kernel (caller falls back), 0 when done.
 int launch_lmm_sdc_tiles(cla_block* b, const double* dY, int p, double* dPre, int onlyGroup) {
-	SdcPlan plan;
-	sdc_plan(b, onlyGroup, plan);
+	int32_t *dList = nullptr, *dBinOff = nullptr;
+	int rc = sdc_plan(b, onlyGroup, &dList, &dBinOff);
+	if(rc) return rc;
+	struct { const std::vector<int32_t>&list, &binOff; } plan{b->sdcList, b->sdcBinOff};
 	if(plan.list.empty()) return 0;
 	const size_t ldsMax = (size_t) std::min(g_ldsPerBlock, 160 * 1024) - 2048;
 	// bins of a slab of groups next to the Y tile; small slabs keep LDS per block low
@@ -182,9 +186,6 @@ int launch_lmm_sdc_tiles(cla_block* b, const double* dY, int p, double* dPre, in
 	binBudget = std::min(binBudget, ldsMax - (size_t) ST * 8);
 	for(size_t l = 0; l < plan.list.size(); l++)
 		if((size_t) (plan.binOff[l + 1] - plan.binOff[l]) * 8 > binBudget) return 1;
-	int32_t *dList = nullptr, *dBinOff = nullptr;
-	int rc = upload_plan(b, plan, &dList, &dBinOff);
-	if(rc) return rc;
 	const int nTiles = (int) ((b->nRows + ST - 1) / ST);
 	// slabs of groups whose bins fit next to the Y tile
 	size_t l0 = 0;
@@ -208,30 +209,33 @@ int launch_lmm_sdc_tiles(cla_block* b, const double* dY, int p, double* dPre, in
 		l0 = l1;
 	}
 	CLA_HIP(hipGetLastError());
-	CLA_HIP(hipStreamSynchronize(b->stream));
-	CLA_HIP(hipFree(dList));
 	return 0;
 }
 
 // Returns 1 if the tile kernel cannot be used (caller falls back), 0 when done.
 int launch_rmm_sdc_tiles(cla_block* b, int q, int constRow, int accumulate, double* dOut, unsigned long long* dNnz) {
-	SdcPlan plan;
-	sdc_plan(b, -1, plan);
+	int32_t *dList = nullptr, *dBinOff = nullptr;
+	int rc = sdc_plan(b, -1, &dList, &dBinOff);
+	if(rc) return rc;
+	struct { const std::vector<int32_t>&list, &binOff; } plan{b->sdcList, b->sdcBinOff};
 	if(plan.list.empty() || b->nRows == 0) return 1;
 	const size_t ldsMax = (size_t) std::min(g_ldsPerBlock, 160 * 1024) - 2048;
 	// rows per tile: a multiple of the tile-index granularity whose output tile takes at most ~half of LDS
 	int tileRows = ST;
 	while(tileRows > SDC_TILE && (size_t) tileRows * q * 8 > ldsMax / 2) tileRows /= 2;
 	if((size_t) tileRows * q * 8 + 4096 > ldsMax) return 1;
-	const size_t tblBudget = ldsMax - (size_t) tileRows * q * 8;
-	// groups per slab: uniform count so that every slab's tables fit
 	size_t maxVals = 1;
 	for(size_t l = 0; l < plan.list.size(); l++) maxVals = std::max(maxVals, (size_t) (plan.binOff[l + 1] - plan.binOff[l]));
+	// Small table slabs keep LDS per block low enough for four blocks per CU: the list walks
+	// are chains of dependent loads and only occupancy hides them (C4: 1.95 ms with one
+	// 100 KB slab, 0.75 ms with 8 KB slabs).
+	size_t tblBudget = 8 * 1024;
+	if(const char* e = getenv("CLA_RMM_SDC_TBL_KB")) tblBudget = (size_t) std::max(1, atoi(e)) * 1024;
+	tblBudget = std::max(tblBudget, maxVals * q * 8);
+	tblBudget = std::min(tblBudget, ldsMax - (size_t) tileRows * q * 8);
+	// groups per slab: uniform count so that every slab's tables fit
 	const size_t slabLen = tblBudget / (maxVals * q * 8);
 	if(slabLen < 1) return 1;
-	int32_t *dList = nullptr, *dBinOff = nullptr;
-	int rc = upload_plan(b, plan, &dList, &dBinOff);
-	if(rc) return rc;
 	const int nTiles = (int) ((b->nRows + tileRows - 1) / tileRows);
 	const int sl = (int) std::min(slabLen, plan.list.size());
 	size_t tblDoubles = 0;
@@ -250,8 +254,6 @@ int launch_rmm_sdc_tiles(cla_block* b, int q, int constRow, int accumulate, doub
 			(int) plan.list.size(), sl, b->dTables, q, constRow, accumulate, tileRows, dOut, b->nRows, dNnz);
 	}
 	CLA_HIP(hipGetLastError());
-	CLA_HIP(hipStreamSynchronize(b->stream));
-	CLA_HIP(hipFree(dList));
 	return 0;
 }
 

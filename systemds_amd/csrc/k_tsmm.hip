@@ -371,11 +371,14 @@ int launch_tsmm(cla_block* b, double* dOut, unsigned long long* dNnz) {
 		return 0;
 	}
 
-	// scratch: counts (maxVals int32) | colSum (nCols doubles)
+	// scratch: counts (maxVals int32) | colSum (nCols doubles) | pair list (one int4 per pair of groups)
 	const size_t cntBytes = ((size_t) std::max(b->maxVals, 1) * 4 + 255) & ~(size_t) 255;
-	if((rc = ensure_scratch(b, cntBytes + sizeof(double) * (size_t) nCols))) return rc;
+	const size_t sumBytes = (sizeof(double) * (size_t) nCols + 255) & ~(size_t) 255;
+	const size_t pairBytes = sizeof(int4) * ((size_t) nG * (nG > 0 ? nG - 1 : 0) / 2 + 1);
+	if((rc = ensure_scratch(b, cntBytes + sumBytes + pairBytes))) return rc;
 	int32_t* dCounts = (int32_t*) b->dScratch;
 	double* dColSum = (double*) ((char*) b->dScratch + cntBytes);
+	int4* dPairs = (int4*) ((char*) b->dScratch + cntBytes + sumBytes);
 	CLA_HIP(hipMemsetAsync(dColSum, 0, sizeof(double) * (size_t) nCols, st));
 	for(int g = 0; g < nG; g++) {
 		if((rc = launch_counts(b, g, dCounts))) return rc;
@@ -406,9 +409,8 @@ int launch_tsmm(cla_block* b, double* dOut, unsigned long long* dNnz) {
 			pairs.push_back(make_int4(gt, gs, dictInLds, 0));
 		}
 	if(!pairs.empty()) {
-		int4* dPairs = nullptr;
-		CLA_HIP(hipMalloc((void**) &dPairs, sizeof(int4) * pairs.size()));
 		CLA_HIP(hipMemcpyAsync(dPairs, pairs.data(), sizeof(int4) * pairs.size(), hipMemcpyHostToDevice, st));
+		CLA_HIP(hipStreamSynchronize(st)); // `pairs` is a local: the copy must have read it
 		// blocks per pair: fill the machine about 8x over all pairs, but keep at least 64 tiles per block
 		const int64_t want = std::max<int64_t>(1, (int64_t) g_numCU * 8 / (int64_t) pairs.size());
 		int bpp = (int) std::min<int64_t>(want, std::max(1, nTiles / 64));
@@ -426,8 +428,6 @@ int launch_tsmm(cla_block* b, double* dOut, unsigned long long* dNnz) {
 			hipLaunchKernelGGL(k_tsmm_pair, dim3(bpp, (unsigned) pairs.size()), dim3(PAIR_THREADS), ldsMax, st, b->dGroups,
 				dPairs, nRows, tpb, dOut, nCols);
 		}
-		CLA_HIP(hipStreamSynchronize(st));
-		CLA_HIP(hipFree(dPairs));
 	}
 	{
 		Prof pf(b, "k_tsmm_finish", 1, 256, 0, 0);
