@@ -20,10 +20,13 @@ namespace cla {
 // ---------------------------------------------------------------------------
 __global__ void k_preagg(const DGroup* __restrict__ groups, int nGroups, const double* __restrict__ B, int q,
 	int nCols, const double* __restrict__ constV, double* __restrict__ T, int totalVals,
-	unsigned long long* __restrict__ nnz) {
+	unsigned long long* __restrict__ nnz, double* __restrict__ Tpad) {
 	const int g = blockIdx.y;
 	const int idx = blockIdx.x * blockDim.x + threadIdx.x;
 	if(g == 0 && idx == 0) *nnz = 0; // the multiply kernels behind this one on the stream count into it
+	// Tpad (mat-vec on byte codes only): the same tables at a fixed stride of 256 entries, zero
+	// beyond nVals, so that the gather kernel copies a slab of tables without looking up offsets
+	if(Tpad != nullptr && g < nGroups && idx < 256 && idx >= groups[g].nVals) Tpad[(size_t) g * 256 + idx] = 0.0;
 	if(g == nGroups) {
 		if(constV == nullptr || idx >= q) return;
 		double acc = 0;
@@ -43,6 +46,7 @@ __global__ void k_preagg(const DGroup* __restrict__ groups, int nGroups, const d
 		if(v != 0) acc = __dadd_rn(acc, __dmul_rn(v, B[(size_t) G.cols[h] * q + c]));
 	}
 	T[(size_t) (G.tblOff + k) * q + c] = acc;
+	if(Tpad != nullptr) Tpad[(size_t) g * 256 + k] = acc;
 }
 
 // ---------------------------------------------------------------------------
@@ -287,7 +291,7 @@ __device__ __forceinline__ void u8_consume(const CodeVec<1, RPT> (&cv)[NB], cons
 // U8_PER is a multiple of 2 * U8_NB. The host picks the variant that pads least.
 template <int THREADS, int U8_PER, int U8_NB, int LB, int LN>
 __global__ __launch_bounds__(THREADS, 4) void k_rmm_q1_u8(const uint8_t* __restrict__ arena, size_t arenaStride,
-	int nGroups, const int32_t* __restrict__ tblOff, const double* __restrict__ T, int constIdx,
+	int nGroups, const double* __restrict__ Tpad, const double* __restrict__ constTerm,
 	double* __restrict__ out, int64_t nRows, unsigned long long* __restrict__ nnz) {
 	__shared__ double tbl[U8_PER * 256];
 	__shared__ double wbufAll[(THREADS / 64) * 64 * 8]; // per-wave transpose buffers of the epilogue
@@ -319,24 +323,19 @@ __global__ __launch_bounds__(THREADS, 4) void k_rmm_q1_u8(const uint8_t* __restr
 	// the tables of the next slab are fetched into registers while the current slab is processed
 	constexpr int TPT = (U8_PER * 256 + THREADS - 1) / THREADS;
 	double stage[TPT];
-	auto fetch = [&](int g0) {
-		const int nIn = min(U8_PER, nGroups - g0);
+	auto fetch = [&](int g0) { // tables g0 .. g0 + U8_PER - 1 of the padded image (zero beyond the last group)
+		const int nIn = min(U8_PER, nGroups - g0) * 256;
+		const double* src = Tpad + (size_t) g0 * 256;
 		int tidF = tid; // laundered like tidE below: keeps the index arithmetic out of registers between uses
 		asm volatile("" : "+v"(tidF));
 #pragma unroll
 		for(int k = 0; k < TPT; k++) {
 			const int f = tidF + k * THREADS;
-			const int g = f >> 8, i = f & 255;
-			double v = 0.0;
-			if(g < nIn) {
-				const int o = tblOff[g0 + g], n = tblOff[g0 + g + 1] - o;
-				if(i < n) v = T[o + i];
-			}
-			stage[k] = v;
+			stage[k] = f < nIn ? src[f] : 0.0;
 		}
 	};
 	fetch(0);
-	const double cadd = constIdx >= 0 ? T[constIdx] : 0.0;
+	const double cadd = constTerm != nullptr ? *constTerm : 0.0;
 	int cnt = 0;
 	for(int pass = 0; pass < nPass; pass++) {
 		const int64_t passBeg = blockBeg + (int64_t) pass * passRows;
@@ -544,21 +543,25 @@ int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned lon
 	const int64_t nRows = b->nRows;
 	hipStream_t st = b->stream;
 	clear_stats(b);
-	int rc = ensure_tables(b, (size_t) (b->totalVals + 1) * q);
+	// mat-vec on byte codes: all groups DDC in one arena, at most 256 values each
+	const bool u8Path = q == 1 && nRows > 0 && b->dArena && b->arenaWidth == 1 && b->maxVals <= 256 && !getenv("CLA_Q1_GENERIC");
+	const size_t nTbl = (size_t) (b->totalVals + 1) * q;
+	int rc = ensure_tables(b, nTbl + (u8Path ? (size_t) nG * 256 + 256 : 0));
 	if(rc) return rc;
+	double* dTpad = u8Path ? b->dTables + ((nTbl + 31) & ~(size_t) 31) : nullptr;
 
 	// K1 (also clears the non-zero counter)
 	{
-		const int maxWork = (b->maxVals > 1 ? b->maxVals : 1) * q;
+		const int maxWork = (u8Path ? 256 : (b->maxVals > 1 ? b->maxVals : 1)) * q;
 		dim3 grid((maxWork + 255) / 256 > (q + 255) / 256 ? (maxWork + 255) / 256 : (q + 255) / 256, nG + 1);
 		Prof pf(b, "k_preagg", (long) grid.x * grid.y, 256, 0, 0);
 		hipLaunchKernelGGL(k_preagg, grid, dim3(256), 0, st, b->dGroups, nG, dB, q, b->nCols,
-			b->hasConst ? b->dConstV : nullptr, b->dTables, b->totalVals, dNnz);
+			b->hasConst ? b->dConstV : nullptr, b->dTables, b->totalVals, dNnz, dTpad);
 	}
 	const int constRow = b->hasConst ? b->totalVals : -1;
 	if(nRows == 0) return 0;
 
-	if(q == 1 && b->dArena && b->arenaWidth == 1 && b->maxVals <= 256 && !getenv("CLA_Q1_GENERIC")) {
+	if(u8Path) {
 		constexpr int THREADS = 512;
 		const int64_t rowsPerBlock = (int64_t) THREADS * U8_RPT;
 		(void) rowsPerBlock;
@@ -575,7 +578,7 @@ int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned lon
 		Prof pf(b, "k_rmm_q1_u8", grid, THREADS, per * 256 * 8, bytes);
 #define U8_LAUNCH(PER, NBV, LB, LN)                                                                             \
 	hipLaunchKernelGGL((k_rmm_q1_u8<THREADS, PER, NBV, LB, LN>), dim3(grid), dim3(THREADS), 0, st, b->dArena,   \
-		b->arenaStride, nG, b->dTblOff, b->dTables, constRow, dOut, nRows, dNnz)
+		b->arenaStride, nG, dTpad, constRow >= 0 ? b->dTables + constRow : nullptr, dOut, nRows, dNnz)
 		if(per == 20) U8_LAUNCH(20, 5, 4, 2);
 		else U8_LAUNCH(16, 4, 8, 2);
 #undef U8_LAUNCH
