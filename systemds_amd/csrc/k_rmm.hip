@@ -289,6 +289,15 @@ __device__ __forceinline__ void u8_consume(const CodeVec<1, RPT> (&cv)[NB], cons
 }
 
 // U8_PER is a multiple of 2 * U8_NB. The host picks the variant that pads least.
+// Batch request with a uniform base and a 32-bit per-thread offset: the address of every load
+// is (scalar base + group * stride) + vector offset, which costs no vector arithmetic.
+template <int RPT, int NB>
+__device__ __forceinline__ void u8_load(CodeVec<1, RPT> (&cv)[NB], const uint8_t* base, uint32_t voff, size_t arenaStride, int g,
+	int gLast) {
+#pragma unroll
+	for(int j = 0; j < NB; j++) cv[j].load(base + (size_t) min(g + j, gLast) * arenaStride + voff);
+}
+
 template <int THREADS, int U8_PER, int U8_NB, int LB, int LN>
 __global__ __launch_bounds__(THREADS, 4) void k_rmm_q1_u8(const uint8_t* __restrict__ arena, size_t arenaStride,
 	int nGroups, const double* __restrict__ Tpad, const double* __restrict__ constTerm,
@@ -315,10 +324,11 @@ __global__ __launch_bounds__(THREADS, 4) void k_rmm_q1_u8(const uint8_t* __restr
 
 	int passLen = min(passRows, blockLen);
 	bool full = off + RPT <= passLen;
-	const uint8_t* myCodes = arena + (size_t) blockBeg + (full ? off : 0);
+	const uint8_t* passBase = arena + (size_t) blockBeg; // uniform; a thread's codes start at passBase + off
+	uint32_t voff = full ? off : 0;
 
 	CodeVec<1, RPT> ping[NB], pong[NB];
-	if(full) q1_load<1, RPT, NB>(ping, myCodes, arenaStride, 0, gLast);
+	if(full) u8_load<RPT, NB>(ping, passBase, voff, arenaStride, 0, gLast);
 
 	// the tables of the next slab are fetched into registers while the current slab is processed
 	constexpr int TPT = (U8_PER * 256 + THREADS - 1) / THREADS;
@@ -344,7 +354,8 @@ __global__ __launch_bounds__(THREADS, 4) void k_rmm_q1_u8(const uint8_t* __restr
 		// number of loads in flight never depends on a branch
 		const int nextLen = pass + 1 < nPass ? min(passRows, blockLen - (pass + 1) * passRows) : 0;
 		const bool nfull = off + RPT <= nextLen;
-		const uint8_t* nextCodes = nfull ? arena + (size_t) (passBeg + passRows) + off : myCodes;
+		const uint8_t* nextBase = nextLen > 0 ? passBase + passRows : passBase; // uniform
+		const uint32_t noff = nextLen > 0 ? (nfull ? off : 0) : voff;
 		double acc[RPT];
 #pragma unroll
 		for(int i = 0; i < RPT; i++) acc[i] = 0.0;
@@ -363,11 +374,11 @@ __global__ __launch_bounds__(THREADS, 4) void k_rmm_q1_u8(const uint8_t* __restr
 			if(full) {
 #pragma unroll
 				for(int s = 0; s < U8_PER; s += 2 * NB) {
-					q1_load<1, RPT, NB>(pong, myCodes, arenaStride, g0 + s + NB, gLast);
+					u8_load<RPT, NB>(pong, passBase, voff, arenaStride, g0 + s + NB, gLast);
 					u8_consume<RPT, NB, LB, LN>(ping, tb + s * 2048, acc);
 					const int gn = g0 + s + 2 * NB;
 					const bool wrap = gn >= nPad;
-					q1_load<1, RPT, NB>(ping, wrap ? nextCodes : myCodes, arenaStride, wrap ? 0 : gn, gLast);
+					u8_load<RPT, NB>(ping, wrap ? nextBase : passBase, wrap ? noff : voff, arenaStride, wrap ? 0 : gn, gLast);
 					u8_consume<RPT, NB, LB, LN>(pong, tb + (s + NB) * 2048, acc);
 				}
 			}
@@ -427,7 +438,8 @@ __global__ __launch_bounds__(THREADS, 4) void k_rmm_q1_u8(const uint8_t* __restr
 		}
 		passLen = nextLen;
 		full = nfull;
-		myCodes = nextCodes;
+		passBase = nextBase;
+		voff = noff;
 	}
 	count_add(nnz, cnt);
 }
