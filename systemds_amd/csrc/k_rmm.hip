@@ -312,7 +312,7 @@ __global__ __launch_bounds__(THREADS, 4) void k_rmm_q1_u8(const uint8_t* __restr
 	const int nPad = (nGroups + U8_PER - 1) / U8_PER * U8_PER; // groups incl. the zero-table slots of the last slab
 
 	// The block is persistent: it owns an equal share of the rows (a multiple of 16) and covers
-	// it in nPass equally filled passes of at most THREADS * RPT rows, so all blocks finish
+	// it in nPass passes of at most THREADS * RPT rows, the same for every block, so all blocks finish
 	// together and the load pipeline (codes two batches ahead, tables one slab ahead) keeps
 	// running from pass to pass. Everything about a pass but `off` is uniform.
 	const int64_t share = ((nRows + gridDim.x - 1) / gridDim.x + RPT - 1) / RPT * RPT;
@@ -320,7 +320,9 @@ __global__ __launch_bounds__(THREADS, 4) void k_rmm_q1_u8(const uint8_t* __restr
 	if(blockBeg >= nRows) return;
 	const int blockLen = (int) (min(nRows, blockBeg + share) - blockBeg);
 	const int nPass = (blockLen + THREADS * RPT - 1) / (THREADS * RPT);
-	const int passRows = ((blockLen + nPass - 1) / nPass + RPT - 1) / RPT * RPT;
+	// whole waves per pass (64 threads x RPT rows), so that only a block's last pass can hold a
+	// partly filled wave, which has to store its rows untransposed
+	const int passRows = ((blockLen + nPass - 1) / nPass + 64 * RPT - 1) / (64 * RPT) * (64 * RPT);
 
 	int passLen = min(passRows, blockLen);
 	bool full = off + RPT <= passLen;
@@ -355,7 +357,7 @@ __global__ __launch_bounds__(THREADS, 4) void k_rmm_q1_u8(const uint8_t* __restr
 		const int nextLen = pass + 1 < nPass ? min(passRows, blockLen - (pass + 1) * passRows) : 0;
 		const bool nfull = off + RPT <= nextLen;
 		const uint8_t* nextBase = nextLen > 0 ? passBase + passRows : passBase; // uniform
-		const uint32_t noff = nextLen > 0 ? (nfull ? off : 0) : voff;
+		const uint32_t noff = nfull ? off : 0; // without a next pass: everybody re-requests the same 16 bytes
 		double acc[RPT];
 #pragma unroll
 		for(int i = 0; i < RPT; i++) acc[i] = 0.0;
