@@ -22,7 +22,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # scaled against a plain 1 GiB copy: 2.0 KiB per FETCH_SIZE unit, 1.0 KiB per WRITE_SIZE
 # unit); figures and commands: profiles/k_rmm_q1_u8_C2_matvec.md. Valid for the full-size
 # C2 workload only.
-MEASURED_TRAFFIC = {"k_rmm_q1_u8": 489701.3 * 2048 + 87130.4 * 1024}
+MEASURED_TRAFFIC = {"k_rmm_q1_u8": 510678.0 * 2048 + 99626.9 * 1024}
 
 
 def timed(blk, fn, reps=5, warm=2):
