@@ -83,6 +83,20 @@ def other_configs(scale):
 
     c = synth.config1()
     run("C1", c, rmm_ops("v", 1))
+    c = synth.config2(scale=scale)
+
+    def c2_ops(blk, cfg):
+        # the left multiply and the chain on the headline block (the adjacent rows of the scope table)
+        n, m = cfg["n_rows"], cfg["n_cols"]
+        dy = dev(np.random.default_rng(3).standard_normal((1, n)))
+        dv = dev(cfg["v"])
+        do1 = torch.empty((1, m), dtype=torch.float64, device="cuda")
+        do2 = torch.empty((m,), dtype=torch.float64, device="cuda")
+        comp = float(blk.device_bytes())
+        yield ("t(y)%*%X", lambda: blk.lmm_dev(dy.data_ptr(), 1, do1.data_ptr()), comp + n * 8.0)
+        yield ("t(X)%*%(X%*%v)", lambda: blk.mmchain_dev(dv.data_ptr(), None, 0, do2.data_ptr()), 2 * comp + 2 * n * 8.0)
+    run("C2", c, c2_ops)
+    del c
     c = synth.config3(scale=scale)
 
     def tsmm_ops(blk, cfg):

@@ -83,4 +83,67 @@ __device__ __forceinline__ void sdc_decode256(const void* __restrict__ deltas, i
 	emit += __shfl(pc, WAVE - 1, WAVE);
 }
 
+// BYTES bytes of a code stream in registers, requested as non-temporal 8/16-byte loads.
+template <int BYTES>
+struct RawVec;
+template <>
+struct RawVec<8> {
+	u32x2 v;
+	__device__ __forceinline__ void load(const uint8_t* p) { v = __builtin_nontemporal_load((const u32x2*) p); }
+	__device__ __forceinline__ uint32_t word(int i) const { return i == 0 ? v.x : v.y; }
+};
+template <>
+struct RawVec<16> {
+	u32x4 v;
+	__device__ __forceinline__ void load(const uint8_t* p) { v = __builtin_nontemporal_load((const u32x4*) p); }
+	__device__ __forceinline__ uint32_t word(int i) const { return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w; }
+};
+template <>
+struct RawVec<32> {
+	u32x4 v[2];
+	__device__ __forceinline__ void load(const uint8_t* p) {
+		v[0] = __builtin_nontemporal_load((const u32x4*) p);
+		v[1] = __builtin_nontemporal_load((const u32x4*) p + 1);
+	}
+	__device__ __forceinline__ uint32_t word(int i) const {
+		const u32x4 q = v[i >> 2];
+		const int j = i & 3;
+		return j == 0 ? q.x : j == 1 ? q.y : j == 2 ? q.z : q.w;
+	}
+};
+template <>
+struct RawVec<64> {
+	u32x4 v[4];
+	__device__ __forceinline__ void load(const uint8_t* p) {
+#pragma unroll
+		for(int k = 0; k < 4; k++) v[k] = __builtin_nontemporal_load((const u32x4*) p + k);
+	}
+	__device__ __forceinline__ uint32_t word(int i) const {
+		const u32x4 q = v[i >> 2];
+		const int j = i & 3;
+		return j == 0 ? q.x : j == 1 ? q.y : j == 2 ? q.z : q.w;
+	}
+};
+
+// RPT codes of width CW held in registers
+template <int CW, int RPT>
+struct CodeVec {
+	RawVec<CW * RPT> raw;
+	__device__ __forceinline__ void load(const uint8_t* p) { raw.load(p); }
+	__device__ __forceinline__ int get(int i) const {
+		if(CW == 1) return (raw.word(i >> 2) >> (8 * (i & 3))) & 0xffu;
+		if(CW == 2) return (raw.word(i >> 1) >> (16 * (i & 1))) & 0xffffu;
+		return (int) raw.word(i);
+	}
+};
+
+// Batch request with a uniform base and a 32-bit per-thread offset: the address of every load
+// is (scalar base + group * stride) + vector offset, which costs no vector arithmetic.
+template <int RPT, int NB>
+__device__ __forceinline__ void u8_load(CodeVec<1, RPT> (&cv)[NB], const uint8_t* base, uint32_t voff, size_t arenaStride, int g,
+	int gLast) {
+#pragma unroll
+	for(int j = 0; j < NB; j++) cv[j].load(base + (size_t) min(g + j, gLast) * arenaStride + voff);
+}
+
 } // namespace cla

@@ -105,6 +105,9 @@ struct cla_block {
 	double* dStageIn = nullptr; size_t stageInCap = 0;
 	double* dStageOut = nullptr; size_t stageOutCap = 0;
 	void* dScratch = nullptr;   size_t scratchCap = 0;
+	// all groups single-column DDC with byte codes: dictionaries at a fixed stride of 256 entries
+	// (zero beyond nVals) followed by the groups' column indexes; built on first use
+	double* dDictPad = nullptr;
 	// list of SDCZeros groups + prefix sums of their nVals, as the row-tile kernels read it;
 	// built on first use for all groups (sdcPlanGroup -1) or for one group (its index)
 	int32_t* dSdcPlan = nullptr;
@@ -139,6 +142,8 @@ int launch_sdc_build(cla_block* b, HostGroup& g);
 int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned long long* dNnz);
 int launch_rmm_mfma(cla_block* b, const double* dB, int q, const double* dConstRow, double* dOut,
 	unsigned long long* dNnz);
+int launch_lmm_u8(cla_block* b, const double* dY, int p, double* dPre);
+int launch_lmm_u8_dot(cla_block* b, const double* dY, int p, double* dOut);
 int launch_lmm_sdc_tiles(cla_block* b, const double* dY, int p, double* dPre, int onlyGroup);
 int launch_rmm_sdc_tiles(cla_block* b, int q, int constRow, int accumulate, double* dOut, unsigned long long* dNnz);
 int launch_rmm_decode(cla_block* b, const double* dB, int q, const double* dConstRow, double* dOut,

@@ -191,6 +191,11 @@ static int run_preagg(cla_block* b, const double* dY, int p, double* dPre, int o
 	const int nG = (int) b->groups.size();
 	const int64_t nRows = b->nRows;
 	hipStream_t st = b->stream;
+	// all groups DDC with byte codes in one arena: one persistent kernel for the whole block
+	if(onlyGroup < 0) {
+		const int r = launch_lmm_u8(b, dY, p, dPre);
+		if(r <= 0) return r;
+	}
 	// row-parallel groups (DDC, RLE) in LDS-sized slabs
 	int64_t rowsPerBlock = 64 * 1024;
 	while(rowsPerBlock > 4096 && (nRows + rowsPerBlock - 1) / rowsPerBlock * p < (int64_t) g_numCU * 2) rowsPerBlock /= 2;
@@ -280,7 +285,10 @@ int launch_lmm(cla_block* b, const double* dY, int p, double* dOut, unsigned lon
 	CLA_HIP(hipMemsetAsync(dPre, 0, sizeof(double) * ((size_t) p * b->totalVals + (size_t) p), st));
 	CLA_HIP(hipMemsetAsync(dOut, 0, sizeof(double) * (size_t) p * b->nCols, st));
 	CLA_HIP(hipMemsetAsync(dNnz, 0, sizeof(unsigned long long), st));
-	if((rc = run_preagg(b, dY, p, dPre, -1))) return rc;
+	// single-column DDC groups on byte codes: contributions go straight into dOut
+	const int dot = nRows > 0 ? launch_lmm_u8_dot(b, dY, p, dOut) : 1;
+	if(dot < 0) return dot;
+	if(dot != 0 && (rc = run_preagg(b, dY, p, dPre, -1))) return rc;
 
 	int64_t rowsPerBlock = 256 * 1024;
 	while(rowsPerBlock > 8192 && (nRows + rowsPerBlock - 1) / rowsPerBlock * p < (int64_t) g_numCU * 2) rowsPerBlock /= 2;
@@ -295,7 +303,7 @@ int launch_lmm(cla_block* b, const double* dY, int p, double* dOut, unsigned lon
 		Prof pf(b, "k_lmm_rowsum", (long) gridRows * p, 256, 0, 0);
 		hipLaunchKernelGGL(k_lmm_rowsum, dim3(gridRows, p), dim3(256), 0, st, dY, nRows, rowsPerBlock, dRs);
 	}
-	if(nG > 0) {
+	if(nG > 0 && dot != 0) {
 		Prof pf(b, "k_lmm_post", (long) nG * p, 256, 0, 0);
 		hipLaunchKernelGGL(k_lmm_post, dim3(nG, p), dim3(256), 0, st, b->dGroups, dPre, b->totalVals, dOut, b->nCols);
 	}

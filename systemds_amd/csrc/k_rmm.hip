@@ -60,59 +60,6 @@ __global__ void k_preagg(const DGroup* __restrict__ groups, int nGroups, const d
 // one is consumed. Groups are visited in list order, so every output cell is
 // summed in the same order as the CPU algorithm.
 // ---------------------------------------------------------------------------
-template <int BYTES>
-struct RawVec;
-template <>
-struct RawVec<8> {
-	u32x2 v;
-	__device__ __forceinline__ void load(const uint8_t* p) { v = __builtin_nontemporal_load((const u32x2*) p); }
-	__device__ __forceinline__ uint32_t word(int i) const { return i == 0 ? v.x : v.y; }
-};
-template <>
-struct RawVec<16> {
-	u32x4 v;
-	__device__ __forceinline__ void load(const uint8_t* p) { v = __builtin_nontemporal_load((const u32x4*) p); }
-	__device__ __forceinline__ uint32_t word(int i) const { return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w; }
-};
-template <>
-struct RawVec<32> {
-	u32x4 v[2];
-	__device__ __forceinline__ void load(const uint8_t* p) {
-		v[0] = __builtin_nontemporal_load((const u32x4*) p);
-		v[1] = __builtin_nontemporal_load((const u32x4*) p + 1);
-	}
-	__device__ __forceinline__ uint32_t word(int i) const {
-		const u32x4 q = v[i >> 2];
-		const int j = i & 3;
-		return j == 0 ? q.x : j == 1 ? q.y : j == 2 ? q.z : q.w;
-	}
-};
-template <>
-struct RawVec<64> {
-	u32x4 v[4];
-	__device__ __forceinline__ void load(const uint8_t* p) {
-#pragma unroll
-		for(int k = 0; k < 4; k++) v[k] = __builtin_nontemporal_load((const u32x4*) p + k);
-	}
-	__device__ __forceinline__ uint32_t word(int i) const {
-		const u32x4 q = v[i >> 2];
-		const int j = i & 3;
-		return j == 0 ? q.x : j == 1 ? q.y : j == 2 ? q.z : q.w;
-	}
-};
-
-// RPT codes of width CW held in registers
-template <int CW, int RPT>
-struct CodeVec {
-	RawVec<CW * RPT> raw;
-	__device__ __forceinline__ void load(const uint8_t* p) { raw.load(p); }
-	__device__ __forceinline__ int get(int i) const {
-		if(CW == 1) return (raw.word(i >> 2) >> (8 * (i & 3))) & 0xffu;
-		if(CW == 2) return (raw.word(i >> 1) >> (16 * (i & 1))) & 0xffffu;
-		return (int) raw.word(i);
-	}
-};
-
 template <int CW, int RPT, int NB>
 __device__ __forceinline__ void q1_load(CodeVec<CW, RPT> (&cv)[NB], const uint8_t* myCodes, size_t arenaStride, int g,
 	int gLast) {
@@ -289,15 +236,6 @@ __device__ __forceinline__ void u8_consume(const CodeVec<1, RPT> (&cv)[NB], cons
 }
 
 // U8_PER is a multiple of 2 * U8_NB. The host picks the variant that pads least.
-// Batch request with a uniform base and a 32-bit per-thread offset: the address of every load
-// is (scalar base + group * stride) + vector offset, which costs no vector arithmetic.
-template <int RPT, int NB>
-__device__ __forceinline__ void u8_load(CodeVec<1, RPT> (&cv)[NB], const uint8_t* base, uint32_t voff, size_t arenaStride, int g,
-	int gLast) {
-#pragma unroll
-	for(int j = 0; j < NB; j++) cv[j].load(base + (size_t) min(g + j, gLast) * arenaStride + voff);
-}
-
 template <int THREADS, int U8_PER, int U8_NB, int LB, int LN>
 __global__ __launch_bounds__(THREADS, 4) void k_rmm_q1_u8(const uint8_t* __restrict__ arena, size_t arenaStride,
 	int nGroups, const double* __restrict__ Tpad, const double* __restrict__ constTerm,

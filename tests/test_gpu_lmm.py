@@ -96,3 +96,32 @@ def test_mmchain(cla, ora, ctype):
     scale = np.abs(D).T @ inner
     assert_fp64_close(out, ref, scale, what="mmchain", n_terms=40009)
     assert nnz == rnnz
+
+
+@pytest.mark.parametrize("n_rows", [1, 15, 16, 1023, 1024, 1025, 40000, 131072 + 17])
+@pytest.mark.parametrize("n_col_g", [1, 2])
+@pytest.mark.parametrize("p", [1, 3])
+def test_byte_code_blocks_left_multiply(cla, ora, n_rows, n_col_g, p):
+    """All groups DDC with byte codes (one code arena): single-column groups take the
+    dot-product kernel, co-coded groups the LDS-bin kernel; group counts that do not fill a
+    slab, ragged row counts, several rows of Y, a constant group on top."""
+    from systemds_amd import synth
+    rng = np.random.default_rng(1000 * n_col_g + n_rows % 977 + p)
+    n_groups = 23
+    specs = []
+    for g in range(n_groups):
+        n_vals = [2, 17, 256, 100][g % 4]
+        cols = np.arange(g * n_col_g, (g + 1) * n_col_g, dtype=np.int32)
+        specs.append(synth.GroupSpec("ddc", cols, rng.standard_normal((n_vals, n_col_g)),
+                                     rng.integers(0, n_vals, n_rows).astype(np.uint8)))
+    n_cols = n_groups * n_col_g + 1
+    specs.append(synth.GroupSpec("const", np.array([n_cols - 1], np.int32), np.array([[1.25]])))
+    Y = rng.standard_normal((p, n_rows))
+    blk = cla.build_block(n_rows, n_cols, specs)
+    out, nnz = blk.lmm(Y)
+    blk.close()
+    D = ora.np_decompress(specs, n_rows, n_cols)
+    assert_matches_truth(out, Y, D, what=f"byte-code lmm nColG={n_col_g} p={p}")
+    ref, rnnz = ora.lmm(ora.Groups(specs, n_rows, n_cols), Y, 4)
+    assert_fp64_close(out, ref, ora.abs_matmul(Y, D), what="byte-code lmm vs oracle", n_terms=n_rows)
+    assert nnz == rnnz
