@@ -183,6 +183,110 @@ __global__ __launch_bounds__(PAIR_THREADS) void k_tsmm_pair(const DGroup* __rest
 		}
 }
 
+// ---------------------------------------------------------------------------
+// Pair term in dot form for two DDC groups whose dictionaries both fit LDS:
+// S[i, j] = sum_r dict_t[code_t(r), i] * dict_s[code_s(r), j], accumulated in registers,
+// no LDS atomics (an LDS fp64 add costs about four LDS reads on this device). Equal to the
+// pre-aggregate form t(dict_t) . P up to rounding. Blocks are ordered row chunk first,
+// pair second, so that the code streams of one chunk of rows are served from the
+// last-level cache for all pairs.
+// ---------------------------------------------------------------------------
+constexpr int PD_THREADS = 1024;
+constexpr int PD_RPT = 8; // rows per thread and step: one 8- or 16-byte load per stream
+constexpr int PD_DEPTH = 4;
+
+template <int CW, int NCT, int NCS>
+__global__ __launch_bounds__(PD_THREADS) void k_tsmm_pair_dot(const DGroup* __restrict__ groups, const int4* __restrict__ pairs,
+	int nPairs, int64_t nRows, int64_t chunkRows, int blocksPerChunkPair, double* __restrict__ out, int nCols) {
+	extern __shared__ double smem[];
+	const int tid = threadIdx.x;
+	// blockIdx.x = (chunk * nPairs + pair) * blocksPerChunkPair + part
+	const int part = blockIdx.x % blocksPerChunkPair;
+	const int cp = blockIdx.x / blocksPerChunkPair;
+	const int pairIdx = cp % nPairs, chunk = cp / nPairs;
+	const int4 pr = pairs[pairIdx];
+	const DGroup& Gt = groups[pr.x];
+	const DGroup& Gs = groups[pr.y];
+	double* dT = smem;                                   // nVals_t * NCT
+	double* dS = smem + (((size_t) Gt.nVals * NCT + 1) & ~(size_t) 1); // nVals_s * NCS, 16-byte aligned
+	for(int i = tid; i < Gt.nVals * NCT; i += PD_THREADS) dT[i] = Gt.dict[i];
+	for(int i = tid; i < Gs.nVals * NCS; i += PD_THREADS) dS[i] = Gs.dict[i];
+	const int64_t cb = (int64_t) chunk * chunkRows, ce = min(cb + chunkRows, nRows);
+	const int64_t per = ((ce - cb + blocksPerChunkPair - 1) / blocksPerChunkPair + PD_RPT - 1) / PD_RPT * PD_RPT;
+	const int64_t rb = cb + (int64_t) part * per, re = min(rb + per, ce);
+	const uint8_t* ct = (const uint8_t*) Gt.codes;
+	const uint8_t* cs = (const uint8_t*) Gs.codes;
+	double acc[NCT][NCS];
+#pragma unroll
+	for(int i = 0; i < NCT; i++)
+#pragma unroll
+		for(int j = 0; j < NCS; j++) acc[i][j] = 0.0;
+	__syncthreads();
+	auto row = [&](int a, int c) {
+		double vt[NCT], vs[NCS];
+#pragma unroll
+		for(int i = 0; i < NCT; i++) vt[i] = dT[a * NCT + i];
+#pragma unroll
+		for(int j = 0; j < NCS; j++) vs[j] = dS[c * NCS + j];
+#pragma unroll
+		for(int i = 0; i < NCT; i++)
+#pragma unroll
+			for(int j = 0; j < NCS; j++) acc[i][j] = __builtin_fma(vt[i], vs[j], acc[i][j]);
+	};
+	// Whole steps (every thread 8 rows) with a ring of PD_DEPTH code requests in flight per
+	// stream, then the rows that do not fill a step.
+	CodeVec<CW, PD_RPT> at[PD_DEPTH], as[PD_DEPTH];
+	const int64_t step = (int64_t) PD_THREADS * PD_RPT;
+	const int nFull = re > rb ? (int) ((re - rb) / step) : 0;
+	const uint8_t* pt = ct + (rb + (int64_t) tid * PD_RPT) * CW;
+	const uint8_t* ps = cs + (rb + (int64_t) tid * PD_RPT) * CW;
+#pragma unroll
+	for(int d = 0; d < PD_DEPTH; d++)
+		if(d < nFull) { at[d].load(pt + (int64_t) d * step * CW); as[d].load(ps + (int64_t) d * step * CW); }
+	for(int it = 0; it < nFull; it += PD_DEPTH) {
+#pragma unroll
+		for(int d = 0; d < PD_DEPTH; d++) {
+			if(it + d >= nFull) break;
+#pragma unroll
+			for(int t = 0; t < PD_RPT; t++) row(at[d].get(t), as[d].get(t));
+			if(it + d + PD_DEPTH < nFull) {
+				at[d].load(pt + (int64_t) (it + d + PD_DEPTH) * step * CW);
+				as[d].load(ps + (int64_t) (it + d + PD_DEPTH) * step * CW);
+			}
+		}
+	}
+	for(int64_t r = rb + (int64_t) nFull * step + tid; r < re; r += PD_THREADS) row(load_code(ct, CW, r), load_code(cs, CW, r));
+	// block reduction, then one add per cell into the upper triangle
+	__shared__ double red[PD_THREADS / 64];
+#pragma unroll
+	for(int i = 0; i < NCT; i++)
+#pragma unroll
+		for(int j = 0; j < NCS; j++) {
+			const double s = wave_sum_f64(acc[i][j]);
+			__syncthreads();
+			if((tid & 63) == 0) red[tid >> 6] = s;
+			__syncthreads();
+			if(tid == 0) {
+				double tot = 0.0;
+				for(int w = 0; w < PD_THREADS / 64; w++) tot += red[w];
+				if(tot != 0.0) add_upper_atomic(out, nCols, Gt.cols[i], Gs.cols[j], tot);
+			}
+		}
+}
+
+template <int CW>
+static void launch_pair_dot_cw(int nct, int ncs, dim3 grid, size_t lds, hipStream_t st, const DGroup* g, const int4* pairs, int nPairs,
+	int64_t nRows, int64_t chunkRows, int bpcp, double* out, int nCols) {
+#define PD_CASE(A, B)                                                                                           \
+	if(nct == A && ncs == B) {                                                                                  \
+		auto kern = k_tsmm_pair_dot<CW, A, B>;                                                                  \
+		(void) hipFuncSetAttribute((const void*) kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds);  \
+		hipLaunchKernelGGL(kern, grid, dim3(PD_THREADS), lds, st, g, pairs, nPairs, nRows, chunkRows, bpcp, out, nCols); \
+	}
+	PD_CASE(1, 1) PD_CASE(1, 2) PD_CASE(2, 1) PD_CASE(2, 2)
+#undef PD_CASE
+}
+
 // Self term (AColGroupCompressed.tsmmDense) + column sums of the group:
 // out[cols[i], cols[j]] += sum_k cnt[k] d[k,i] d[k,j], j >= i; colSum[cols[j]] += sum_k cnt[k] d[k,j]
 __global__ __launch_bounds__(256) void k_tsmm_self(const DGroup* __restrict__ groups, int g, const int32_t* __restrict__ counts,
@@ -386,12 +490,26 @@ int launch_tsmm(cla_block* b, double* dOut, unsigned long long* dNnz) {
 		hipLaunchKernelGGL(k_tsmm_self, dim3(1), dim3(256), 0, st, b->dGroups, g, dCounts, dOut, nCols, dColSum);
 	}
 	const int nTiles = (int) ((nRows + TT - 1) / TT);
+	// Pairs of DDC groups with one or two columns each, equal code width and both dictionaries
+	// in LDS take the dot-form kernel (one launch per shape); the others the pre-aggregate kernel.
+	struct DotShape { int cw, nct, ncs; std::vector<int4> list; };
+	std::vector<DotShape> dots;
 	std::vector<int4> pairs;
-	size_t ldsMax = 0;
+	size_t ldsMax = 0, dotLds = 0;
 	for(int g = 0; g < nG && nRows > 0; g++)
 		for(int h = g + 1; h < nG; h++) {
 			const DGroup& A = b->groups[g].d;
 			const DGroup& B = b->groups[h].d;
+			const size_t bothDicts = ((size_t) A.nVals * A.nColG + (size_t) B.nVals * B.nColG + 2) * 8;
+			if(A.type == G_DDC && B.type == G_DDC && A.codeWidth == B.codeWidth && A.codeWidth <= 2 && A.nColG <= 2 && B.nColG <= 2 &&
+				bothDicts <= (size_t) 150 * 1024 && !getenv("CLA_TSMM_PREAGG")) {
+				size_t k = 0;
+				while(k < dots.size() && !(dots[k].cw == A.codeWidth && dots[k].nct == A.nColG && dots[k].ncs == B.nColG)) k++;
+				if(k == dots.size()) dots.push_back(DotShape{A.codeWidth, A.nColG, B.nColG, {}});
+				dots[k].list.push_back(make_int4(g, h, 0, 0));
+				dotLds = std::max(dotLds, bothDicts);
+				continue;
+			}
 			// target = side with the smaller accumulator nVals_t * nC_s
 			const bool gTarget = (size_t) A.nVals * B.nColG <= (size_t) B.nVals * A.nColG;
 			const int gt = gTarget ? g : h, gs = gTarget ? h : g;
@@ -408,9 +526,41 @@ int launch_tsmm(cla_block* b, double* dOut, unsigned long long* dNnz) {
 			ldsMax = std::max(ldsMax, pBytes + (dictInLds ? dBytes : 0) + cBytes);
 			pairs.push_back(make_int4(gt, gs, dictInLds, 0));
 		}
+	if(!dots.empty()) {
+		// one list on the device: the shapes one after the other, then the remaining pairs
+		std::vector<int4> all;
+		for(auto& d : dots) all.insert(all.end(), d.list.begin(), d.list.end());
+		const size_t nDot = all.size();
+		all.insert(all.end(), pairs.begin(), pairs.end());
+		CLA_HIP(hipMemcpyAsync(dPairs, all.data(), sizeof(int4) * all.size(), hipMemcpyHostToDevice, st));
+		CLA_HIP(hipStreamSynchronize(st)); // `all` is a local: the copy must have read it
+		// rows per chunk: the code streams of one chunk (all DDC groups) stay in the last-level cache
+		double bytesPerRow = 0;
+		for(auto& g : b->groups)
+			if(g.d.type == G_DDC) bytesPerRow += g.d.codeWidth;
+		int64_t chunkRows = (int64_t) (128.0 * 1024 * 1024 / std::max(bytesPerRow, 1.0));
+		chunkRows = std::max<int64_t>(chunkRows / 8192 * 8192, 8192);
+		const int nChunks = (int) ((nRows + chunkRows - 1) / chunkRows);
+		size_t off = 0;
+		for(auto& d : dots) {
+			const int nP = (int) d.list.size();
+			int bpcp = 1;
+			while((int64_t) nChunks * nP * bpcp < (int64_t) g_numCU * 4 && chunkRows / (bpcp * 2) >= 64 * 1024) bpcp *= 2;
+			const dim3 grid((unsigned) ((int64_t) nChunks * nP * bpcp));
+			Prof pf(b, "k_tsmm_pair_dot", (long) grid.x, PD_THREADS, (long) dotLds, (double) nRows * 2 * d.cw * nP);
+			if(d.cw == 1)
+				launch_pair_dot_cw<1>(d.nct, d.ncs, grid, dotLds, st, b->dGroups, dPairs + off, nP, nRows, chunkRows, bpcp, dOut, nCols);
+			else
+				launch_pair_dot_cw<2>(d.nct, d.ncs, grid, dotLds, st, b->dGroups, dPairs + off, nP, nRows, chunkRows, bpcp, dOut, nCols);
+			off += nP;
+		}
+		dPairs += nDot;
+	}
 	if(!pairs.empty()) {
-		CLA_HIP(hipMemcpyAsync(dPairs, pairs.data(), sizeof(int4) * pairs.size(), hipMemcpyHostToDevice, st));
-		CLA_HIP(hipStreamSynchronize(st)); // `pairs` is a local: the copy must have read it
+		if(dots.empty()) {
+			CLA_HIP(hipMemcpyAsync(dPairs, pairs.data(), sizeof(int4) * pairs.size(), hipMemcpyHostToDevice, st));
+			CLA_HIP(hipStreamSynchronize(st)); // `pairs` is a local: the copy must have read it
+		}
 		// blocks per pair: fill the machine about 8x over all pairs, but keep at least 64 tiles per block
 		const int64_t want = std::max<int64_t>(1, (int64_t) g_numCU * 8 / (int64_t) pairs.size());
 		int bpp = (int) std::min<int64_t>(want, std::max(1, nTiles / 64));
