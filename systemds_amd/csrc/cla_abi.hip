@@ -224,6 +224,7 @@ void cla_block_free(cla_handle b) {
 	if(b->dScratch) (void) hipFree(b->dScratch);
 	if(b->dSdcPlan) (void) hipFree(b->dSdcPlan);
 	if(b->dDictPad) (void) hipFree(b->dDictPad);
+	if(b->dCountsAll) (void) hipFree(b->dCountsAll);
 	if(b->dCounters) (void) hipFree(b->dCounters);
 	if(b->hCounters) (void) hipHostFree(b->hCounters);
 	if(b->ownStream && b->stream) (void) hipStreamDestroy(b->stream);

@@ -105,6 +105,10 @@ struct cla_block {
 	double* dStageIn = nullptr; size_t stageInCap = 0;
 	double* dStageOut = nullptr; size_t stageOutCap = 0;
 	void* dScratch = nullptr;   size_t scratchCap = 0;
+	// exact code counts of all dictionary-coded groups (totalVals int32, group g at tblOff[g]),
+	// computed on the first TSMM and kept, like the reference's cached counts
+	// (CG/AColGroupValue.java getCounts)
+	int32_t* dCountsAll = nullptr;
 	// all groups single-column DDC with byte codes: dictionaries at a fixed stride of 256 entries
 	// (zero beyond nVals) followed by the groups' column indexes; built on first use
 	double* dDictPad = nullptr;

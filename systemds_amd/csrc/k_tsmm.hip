@@ -289,10 +289,12 @@ static void launch_pair_dot_cw(int nct, int ncs, dim3 grid, size_t lds, hipStrea
 
 // Self term (AColGroupCompressed.tsmmDense) + column sums of the group:
 // out[cols[i], cols[j]] += sum_k cnt[k] d[k,i] d[k,j], j >= i; colSum[cols[j]] += sum_k cnt[k] d[k,j]
-__global__ __launch_bounds__(256) void k_tsmm_self(const DGroup* __restrict__ groups, int g, const int32_t* __restrict__ counts,
+__global__ __launch_bounds__(256) void k_tsmm_self(const DGroup* __restrict__ groups, const int32_t* __restrict__ countsAll,
 	double* __restrict__ out, int nCols, double* __restrict__ colSum) {
 	__shared__ double red[4];
-	const DGroup& G = groups[g];
+	const DGroup& G = groups[blockIdx.y];
+	if(G.type == G_UNC) return;
+	const int32_t* counts = countsAll + G.tblOff;
 	const int nC = G.nColG, tid = threadIdx.x;
 	for(int i = 0; i < nC; i++) {
 		for(int j = i; j <= nC; j++) { // j == nC: column sum of column i
@@ -475,19 +477,23 @@ int launch_tsmm(cla_block* b, double* dOut, unsigned long long* dNnz) {
 		return 0;
 	}
 
-	// scratch: counts (maxVals int32) | colSum (nCols doubles) | pair list (one int4 per pair of groups)
-	const size_t cntBytes = ((size_t) std::max(b->maxVals, 1) * 4 + 255) & ~(size_t) 255;
+	// scratch: colSum (nCols doubles) | pair list (one int4 per pair of groups)
 	const size_t sumBytes = (sizeof(double) * (size_t) nCols + 255) & ~(size_t) 255;
 	const size_t pairBytes = sizeof(int4) * ((size_t) nG * (nG > 0 ? nG - 1 : 0) / 2 + 1);
-	if((rc = ensure_scratch(b, cntBytes + sumBytes + pairBytes))) return rc;
-	int32_t* dCounts = (int32_t*) b->dScratch;
-	double* dColSum = (double*) ((char*) b->dScratch + cntBytes);
-	int4* dPairs = (int4*) ((char*) b->dScratch + cntBytes + sumBytes);
+	if((rc = ensure_scratch(b, sumBytes + pairBytes))) return rc;
+	double* dColSum = (double*) b->dScratch;
+	int4* dPairs = (int4*) ((char*) b->dScratch + sumBytes);
 	CLA_HIP(hipMemsetAsync(dColSum, 0, sizeof(double) * (size_t) nCols, st));
-	for(int g = 0; g < nG; g++) {
-		if((rc = launch_counts(b, g, dCounts))) return rc;
-		Prof pf(b, "k_tsmm_self", 1, 256, 0, 0);
-		hipLaunchKernelGGL(k_tsmm_self, dim3(1), dim3(256), 0, st, b->dGroups, g, dCounts, dOut, nCols, dColSum);
+	if(b->dCountsAll == nullptr) {
+		int32_t* dc = nullptr;
+		CLA_HIP(hipMalloc((void**) &dc, sizeof(int32_t) * (size_t) std::max(b->totalVals, 1)));
+		for(int g = 0; g < nG; g++)
+			if((rc = launch_counts(b, g, dc + b->groups[g].d.tblOff))) { (void) hipFree(dc); return rc; }
+		b->dCountsAll = dc;
+	}
+	if(nG > 0) {
+		Prof pf(b, "k_tsmm_self", nG, 256, 0, 0);
+		hipLaunchKernelGGL(k_tsmm_self, dim3(1, nG), dim3(256), 0, st, b->dGroups, b->dCountsAll, dOut, nCols, dColSum);
 	}
 	const int nTiles = (int) ((nRows + TT - 1) / TT);
 	// Pairs of DDC groups with one or two columns each, equal code width and both dictionaries
