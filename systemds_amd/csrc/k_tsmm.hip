@@ -453,6 +453,15 @@ int launch_tsmm(cla_block* b, double* dOut, unsigned long long* dNnz) {
 	const bool dense = nG >= nCols || b->hasUnc;
 	if(dense) {
 		// t(D) %*% D of the decoded rows, constants included (no correction layer needed)
+		static const bool noMfma = getenv("CLA_TSMM_NO_MFMA") != nullptr;
+		rc = (noMfma || nRows == 0) ? 1 : launch_tsmm_decode(b, dOut);
+		if(rc < 0) return rc;
+		if(rc == 0) {
+			Prof pf(b, "k_tsmm_finish", 1, 256, 0, 0);
+			hipLaunchKernelGGL(k_tsmm_finish, dim3(1), dim3(256), 0, st, dOut, nCols, b->dConstV, b->dConstV, (double) nRows, 0, dNnz);
+			CLA_HIP(hipGetLastError());
+			return 0;
+		}
 		int DT = 256;
 		while(DT > 8 && (size_t) DT * nCols * 8 > (size_t) 96 * 1024) DT /= 2;
 		if((size_t) DT * nCols * 8 > (size_t) 96 * 1024 || (int64_t) nCols * (nCols + 1) / 2 > 24 * 256) {
