@@ -1,64 +1,78 @@
-// Right multiply X %*% B for narrow B (2 <= q <= 16) on blocks of any group mix.
-// A block owns a contiguous range of 1024-row tiles. Per tile every dictionary
-// coded group gets its codes expanded into an LDS code tile (DDC: straight copy,
-// prefetched one tile ahead in registers; SDCZeros: wave-wide offset decode from
-// the tile index; RLE: run expansion with the run cursor carried from tile to
-// tile). Each thread then decodes two rows group by group from dictionary copies
-// in LDS and accumulates value x B[col, :]; B is kept in LDS in decoded column
-// order. The output tile is staged in LDS and written with full-line stores.
+// Decode-and-multiply on blocks of any group mix, on the matrix cores:
+//   k_rmm_decode      X %*% B for narrow B (2 <= q <= 16)
+//   k_tsmm_decode<NB> upper triangle of t(X) %*% X for blocks of at most 16 * NB <= 64 columns
+// A block owns a contiguous range of 1024-row tiles. Per tile every dictionary coded
+// group gets its codes expanded into an LDS code tile (DDC: straight copy, prefetched one
+// tile ahead in registers together with the rows of uncompressed groups; SDCZeros:
+// wave-wide offset decode from the tile index; RLE: run expansion with the run cursor
+// carried from tile to tile). The waves then look decoded values up (code tile ->
+// dictionary copy in LDS, or the dense tile) straight into v_mfma_f64_16x16x4_f64 operands:
+//   X %*% B:    A operand = 16 rows x 4 decoded columns, B operand = 4 rows of B (padded to
+//               16 outputs); 64 output rows per wave and pass, staged per wave in LDS and
+//               written with full-line stores.
+//   t(X) %*% X: lane l holds column 16 cb + l % 16 of row l / 16, which is both operands; the
+//               NB (NB + 1) / 2 upper 16 x 16 tiles of the Gram matrix stay in registers until
+//               the block has walked all its row tiles.
 // (Wide B on all-DDC blocks uses k_rmm_mfma instead.)
 #include "../../include/cla_hip.h"
 #include "cla_device.hpp"
 #include <algorithm>
+#include <cstring>
 
 namespace cla {
 
-constexpr int DEC_THREADS = 512;       // one thread per row of a half tile
+constexpr int DEC_THREADS = 512;
+constexpr int DEC_WAVES = DEC_THREADS / 64;
 constexpr int DEC_TILE = SDC_TILE;     // rows per tile = granularity of the offset tile index
+constexpr int DEC_WROWS = DEC_TILE / DEC_WAVES; // rows of a tile one wave multiplies
 constexpr int DEC_QMAX = 16;
-constexpr int DEC_PF = 4;              // 16-byte code chunks a thread holds for the next tile
+constexpr int DEC_PF = 4;              // 16-byte chunks a thread holds for the next tile
+constexpr int DEC_SLOT_PAD = 80;       // bytes between code tiles: spreads the columns a wave reads together over the LDS banks
 
 struct DecGroup {
 	int32_t type;
 	int32_t nC;
-	int32_t dictOff;   // doubles, into the LDS dictionary copy (-1: dense group)
-	int32_t slotOff;   // bytes, into the LDS code tiles (-1: dense group)
+	int32_t dictOff;   // doubles from the LDS base: dictionary copy, or the dense tile of an uncompressed group
+	int32_t slotOff;   // bytes, into the LDS code tiles (-1: no code tile)
 	int32_t slotW;     // 1 or 2 bytes per code in the tile; all ones = row has no value
 	int32_t kOff;      // first decoded column of the group (row of the LDS copy of B)
-	int32_t copyIdx;   // DDC with codeWidth == slotW: index in the chunk copy list, else -1
-	int32_t pad;       // t(X) %*% X mode, dense group: offset of its LDS tile (doubles)
+	int32_t copyIdx;   // tile filled by the chunk copy list (index), else -1
+	int32_t pad;
 };
 
-// Chunk copy list: DDC groups whose code tile is a plain copy of 1024 codes.
+// Chunk copy list: what is a plain copy of consecutive global bytes per tile (DDC codes
+// whose width is the tile's, rows of uncompressed groups), in 16-byte chunks.
 struct DecCopy {
-	int32_t group;
-	int32_t chunk0;    // first 16-byte chunk of this group in the flattened chunk numbering
+	const uint8_t* src;   // first byte of row 0
+	int32_t chunk0;       // first chunk of this entry in the flattened chunk numbering
+	int32_t bpr;          // bytes per row
+	int32_t dstOff;       // bytes from the LDS base
+	int32_t pad;
 };
 
-// t(X) %*% X mode: where lane l of a wave finds column 16 * cb + l % 16 of a decoded row
+// One decoded column as the multiply phase sees it (16 bytes, read from LDS per use).
 struct DecCol {
-	int32_t kind;      // 0: no such column, 1: dictionary coded group, 2: dense group, 3: constant only
-	int32_t slotOff;   // kind 1: code tile (bytes); kind 2: offset of the group's dense tile (doubles)
-	int32_t slotW;
-	int32_t dictOff;   // kind 1: dictionary copy (doubles)
-	int32_t nC, h;     // columns of the group, this column's place among them
-	double constV;     // constant part of the column (SDC defaults, const groups)
+	int32_t slotOff;   // dictionary coded: code tile (bytes into the code tiles)
+	int32_t valOff;    // doubles from the LDS base: dictionary copy / dense tile
+	int32_t meta;      // kind (0 none or constant only, 1 dictionary coded, 2 dense) | two-byte codes << 2 | nC << 4 | h << 18
+	int32_t pad;
 };
 
 struct DecArgs {
 	const DGroup* groups;
 	const DecGroup* plan;
 	const DecCopy* copies;
-	int nGroups, nCopies, nChunks;     // nChunks: 16-byte chunks per tile over all copy-list groups
-	int dictDoubles, slotBytes, K;     // LDS sizes: dictionaries, code tiles, decoded columns
-	int auxDoubles, tileDoubles;       // LDS: B copy / dense tiles, output tile / Gram tile
+	const DecCol* cols;
+	const double* colConst;            // t(X) %*% X: constant part per (padded) column
+	int nGroups, nCopies, nChunks;     // nChunks: 16-byte chunks per tile over the copy list
+	int nColD;                         // entries of cols (multiple of 4 / of 16)
+	int valDoubles, bDoubles, stageDoubles, slotBytes; // LDS sizes
 	const double* B;
 	int q;
 	const double* constRow;
 	double* out;
 	int64_t nRows;
 	unsigned long long* nnz;
-	const DecCol* cols;                // t(X) %*% X mode: 16 * NB entries
 	int nCols;
 };
 
@@ -69,23 +83,36 @@ __device__ __forceinline__ void dec_store_code(uint8_t* slot, int w, int i, int 
 	else ((uint16_t*) slot)[i] = (uint16_t) code;
 }
 
-// GRAM == 0: out = X %*% B. GRAM == 1: out += upper triangle of t(X) %*% X (constants
-// included) for blocks of at most 16 * NB columns; the fill phase is the same, then every
-// wave feeds 4 decoded rows at a time to v_mfma_f64_16x16x4_f64 (lane l: row l / 16, column
-// 16 * cb + l % 16 is both the A and the B operand) and keeps the NB (NB + 1) / 2 upper tiles
-// of the Gram matrix in registers until the block has walked all its row tiles.
-template <int Q, int GRAM = 0, int NB = 1>
-__global__ __launch_bounds__(DEC_THREADS) void k_rmm_decode(const DecArgs A) {
+// LDS traffic of one wave is ordered; this keeps the compiler from moving accesses across
+__device__ __forceinline__ void dec_wave_sync() {
+	__builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+	__builtin_amdgcn_wave_barrier();
+	__builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Value of one decoded column at tile row rt (code c from the column's tile); 0 where the row has none.
+__device__ __forceinline__ double dec_value(const double* smem, const DecCol D, int c, int rt) {
+	const int kind = D.meta & 3, nC = (D.meta >> 4) & 0x3fff, h = (int) ((unsigned) D.meta >> 18);
+	const bool two = D.meta & 4;
+	const bool valid = kind == 2 || (kind == 1 && c != (two ? 0xffff : 0xff));
+	const int addr = D.valOff + (kind == 1 ? c : rt) * nC + h;
+	const double v = smem[valid ? addr : 0];
+	return valid ? v : 0.0;
+}
+
+template <int GRAM, int NB>
+__device__ __forceinline__ void decode_body(const DecArgs& A) {
 	extern __shared__ __align__(16) double smem[];
-	constexpr int OS = Q + 1; // LDS row stride of the output tile (odd: conflict-free column access)
-	double* dictS = smem;                                         // dictDoubles
-	double* Bs = dictS + A.dictDoubles;                           // auxDoubles: K * Q zero padded columns of B / dense tiles
-	double* otile = Bs + A.auxDoubles;                            // tileDoubles: DEC_THREADS * OS / Gram tile
-	uint8_t* slots = (uint8_t*) (smem + (((size_t) A.dictDoubles + (size_t) A.auxDoubles + (size_t) A.tileDoubles + 1) & ~(size_t) 1)); // slotBytes, 16-byte aligned
-	DecGroup* planS = (DecGroup*) (slots + A.slotBytes);          // nGroups
-	int32_t* runBase = (int32_t*) (planS + A.nGroups);            // nGroups
-	DecCopy* copyS = (DecCopy*) (runBase + A.nGroups);            // nCopies
+	double* Bs = smem + A.valDoubles;                              // bDoubles: rows of B in decoded column order, 16 outputs each
+	double* stage = Bs + A.bDoubles;                               // stageDoubles: output staging per wave / Gram tile
+	uint8_t* slots = (uint8_t*) (stage + A.stageDoubles);          // slotBytes (multiple of 16)
+	DecCol* colS = (DecCol*) (slots + A.slotBytes);                // nColD
+	double* constS = (double*) (colS + A.nColD);                   // nColD (Gram mode)
+	DecGroup* planS = (DecGroup*) (constS + (GRAM ? A.nColD : 0)); // nGroups
+	DecCopy* copyS = (DecCopy*) (planS + A.nGroups);               // nCopies
+	int32_t* runBase = (int32_t*) (copyS + A.nCopies);             // nGroups
 	const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+	const int i16 = lane & 15, k4 = lane >> 4;
 	const DGroup* __restrict__ groups = A.groups;
 	const int nGroups = A.nGroups;
 	const int64_t nRows = A.nRows;
@@ -95,101 +122,105 @@ __global__ __launch_bounds__(DEC_THREADS) void k_rmm_decode(const DecArgs A) {
 	const int tileEnd = (int) ((int64_t) nTiles * (blockIdx.x + 1) / gridDim.x);
 	if(tileBeg >= tileEnd) return;
 
-	// ---- once per block: plan, dictionaries, B in decoded column order, run cursors
+	// ---- once per block: plan, column descriptors, dictionaries, B, run cursors
 	for(int g = tid; g < nGroups; g += DEC_THREADS) {
 		planS[g] = A.plan[g];
 		runBase[g] = groups[g].type == G_RLE ? rle_find(groups[g].runStart, groups[g].nRuns, (int32_t) ((int64_t) tileBeg * DEC_TILE)) : 0;
 	}
 	for(int i = tid; i < A.nCopies; i += DEC_THREADS) copyS[i] = A.copies[i];
-	for(int i = tid; i < A.dictDoubles; i += DEC_THREADS) dictS[i] = 0.0;
+	for(int i = tid; i < A.nColD; i += DEC_THREADS) {
+		colS[i] = A.cols[i];
+		if(GRAM) constS[i] = A.colConst[i];
+	}
+	for(int i = tid; i < A.valDoubles; i += DEC_THREADS) smem[i] = 0.0;
+	if(!GRAM)
+		for(int i = tid; i < A.bDoubles; i += DEC_THREADS) Bs[i] = 0.0;
 	__syncthreads();
 	for(int g = 0; g < nGroups; g++) {
 		const DecGroup P = planS[g];
 		const DGroup& G = groups[g];
-		if(P.dictOff >= 0) {
+		if(P.slotOff >= 0) {
 			const int n = G.nVals * G.nColG;
-			for(int i = tid; i < n; i += DEC_THREADS) dictS[P.dictOff + i] = G.dict[i];
+			for(int i = tid; i < n; i += DEC_THREADS) smem[P.dictOff + i] = G.dict[i];
 		}
-		if(GRAM == 0)
-			for(int i = tid; i < P.nC * Q; i += DEC_THREADS) {
-				const int h = i / Q, c = i - h * Q;
-				Bs[(size_t) (P.kOff + h) * Q + c] = c < A.q ? A.B[(size_t) G.cols[h] * A.q + c] : 0.0;
+		if(!GRAM)
+			for(int i = tid; i < P.nC * A.q; i += DEC_THREADS) {
+				const int h = i / A.q, c = i - h * A.q;
+				Bs[(size_t) (P.kOff + h) * 16 + c] = A.B[(size_t) G.cols[h] * A.q + c];
 			}
 	}
-	double cadd[Q];
-#pragma unroll
-	for(int c = 0; c < Q; c++) cadd[c] = (GRAM == 0 && A.constRow != nullptr && c < A.q) ? A.constRow[c] : 0.0;
-	// Gram mode: this lane's columns and the accumulator tiles (ib <= jb, row major)
-	DecCol myCol[NB];
-	f64x4 gram[NB * (NB + 1) / 2];
-	if(GRAM) {
-#pragma unroll
-		for(int cb = 0; cb < NB; cb++) myCol[cb] = A.cols[cb * 16 + (lane & 15)];
-#pragma unroll
-		for(int t = 0; t < NB * (NB + 1) / 2; t++) gram[t] = f64x4{0.0, 0.0, 0.0, 0.0};
-	}
 
-	// DDC code chunks of one tile, flattened over the copy list: chunk i of a thread is
-	// tid + k * DEC_THREADS, so its group and place in the tile never change. Whole
-	// chunks are loaded as 16 bytes one tile ahead; the ragged end of the last tile is
-	// copied element-wise.
-	auto chunk_place = [&](int i, const uint8_t*& src, int& dstOff, int& w, int& row) {
+	// Copy list chunks of one tile, flattened: chunk i of a thread is tid + k * DEC_THREADS,
+	// so its entry and place in the tile never change. Whole chunks are loaded as 16 bytes
+	// one tile ahead; the ragged end of the last tile is copied byte-wise.
+	auto chunk_place = [&](int i, const uint8_t*& src, int& dstOff, int& bpr, int& off) {
 		int lo = 0, hi = A.nCopies - 1;
 		while(lo < hi) {
 			const int mid = (lo + hi + 1) >> 1;
 			if(copyS[mid].chunk0 <= i) lo = mid; else hi = mid - 1;
 		}
 		const DecCopy C = copyS[lo];
-		const DecGroup P = planS[C.group];
-		w = P.slotW;
-		const int ci = i - C.chunk0;
-		row = ci * (16 / w);
-		src = (const uint8_t*) groups[C.group].codes + (size_t) ci * 16;
-		dstOff = P.slotOff + ci * 16;
+		off = (i - C.chunk0) * 16;
+		bpr = C.bpr;
+		src = C.src + off;
+		dstOff = C.dstOff + off;
 	};
-	auto copy_ragged = [&](const uint8_t* src, int dstOff, int w, int64_t row0) {
-		for(int e = 0; e < 16 / w; e++)
-			if(row0 + e < nRows) {
-				if(w == 1) slots[dstOff + e] = src[e];
-				else ((uint16_t*) (slots + dstOff))[e] = ((const uint16_t*) src)[e];
-			}
+	uint8_t* const ldsBytes = (uint8_t*) smem;
+	auto copy_ragged = [&](const uint8_t* src, int dstOff, int64_t nValid) {
+		for(int e = 0; e < 16; e++)
+			if(e < nValid) ldsBytes[dstOff + e] = src[e];
 	};
 	const uint8_t* pfSrc[DEC_PF];
-	int pfDst[DEC_PF], pfW[DEC_PF], pfRow[DEC_PF];
+	int pfDst[DEC_PF], pfBpr[DEC_PF], pfOff[DEC_PF];
 	u32x4 pf[DEC_PF];
 #pragma unroll
 	for(int k = 0; k < DEC_PF; k++) {
-		pfSrc[k] = nullptr; pfDst[k] = 0; pfW[k] = 1; pfRow[k] = 0;
-		if(tid + k * DEC_THREADS < A.nChunks) chunk_place(tid + k * DEC_THREADS, pfSrc[k], pfDst[k], pfW[k], pfRow[k]);
+		pfSrc[k] = nullptr; pfDst[k] = 0; pfBpr[k] = 1; pfOff[k] = 0;
+		if(tid + k * DEC_THREADS < A.nChunks) chunk_place(tid + k * DEC_THREADS, pfSrc[k], pfDst[k], pfBpr[k], pfOff[k]);
 	}
+	// bytes of a tile's share of a copy entry that lie inside the matrix
+	auto tile_bytes = [&](int64_t t0, int bpr) { return min((int64_t) DEC_TILE, nRows - t0) * bpr; };
 	auto prefetch = [&](int tile) {
 		const int64_t t0 = (int64_t) tile * DEC_TILE;
 #pragma unroll
 		for(int k = 0; k < DEC_PF; k++) {
 			pf[k] = u32x4{0, 0, 0, 0};
-			if(pfSrc[k] != nullptr && t0 + pfRow[k] + 16 / pfW[k] <= nRows)
-				pf[k] = __builtin_nontemporal_load((const u32x4*) (pfSrc[k] + t0 * pfW[k]));
+			if(pfSrc[k] != nullptr && pfOff[k] + 16 <= tile_bytes(t0, pfBpr[k]))
+				pf[k] = __builtin_nontemporal_load((const u32x4*) (pfSrc[k] + t0 * pfBpr[k]));
 		}
 	};
 	prefetch(tileBeg);
+
+	// multiply phase state
+	f64x4 gram[GRAM ? NB * (NB + 1) / 2 : 1];
+	if(GRAM) {
+#pragma unroll
+		for(int t = 0; t < NB * (NB + 1) / 2; t++) gram[t] = f64x4{0.0, 0.0, 0.0, 0.0};
+	}
+	const int q = A.q;
+	const double cinit = (!GRAM && A.constRow != nullptr && i16 < q) ? A.constRow[i16] : 0.0;
+	double* const wstage = stage + (size_t) wave * 64 * (GRAM ? 0 : q);
+	const int KB = A.nColD >> 2;
 
 	int cnt = 0;
 	for(int tile = tileBeg; tile < tileEnd; tile++) {
 		const int64_t t0 = (int64_t) tile * DEC_TILE;
 		const int64_t rEnd = t0 + DEC_TILE;
-		__syncthreads(); // previous tile's readers are done with the code tiles
-		// ---- DDC tiles: prefetched chunks, then what did not fit the prefetch registers
+		__syncthreads(); // previous tile's readers are done with the code and dense tiles
+		// ---- copy list: prefetched chunks, then what did not fit the prefetch registers
 #pragma unroll
 		for(int k = 0; k < DEC_PF; k++) {
 			if(pfSrc[k] == nullptr) continue;
-			if(t0 + pfRow[k] + 16 / pfW[k] <= nRows) *(u32x4*) (slots + pfDst[k]) = pf[k];
-			else copy_ragged(pfSrc[k] + t0 * pfW[k], pfDst[k], pfW[k], t0 + pfRow[k]);
+			const int64_t tb = tile_bytes(t0, pfBpr[k]);
+			if(pfOff[k] + 16 <= tb) *(u32x4*) (ldsBytes + pfDst[k]) = pf[k];
+			else copy_ragged(pfSrc[k] + t0 * pfBpr[k], pfDst[k], tb - pfOff[k]);
 		}
 		for(int i = tid + DEC_PF * DEC_THREADS; i < A.nChunks; i += DEC_THREADS) {
-			const uint8_t* src; int dstOff, w, row;
-			chunk_place(i, src, dstOff, w, row);
-			if(t0 + row + 16 / w <= nRows) *(u32x4*) (slots + dstOff) = __builtin_nontemporal_load((const u32x4*) (src + t0 * w));
-			else copy_ragged(src + t0 * w, dstOff, w, t0 + row);
+			const uint8_t* src; int dstOff, bpr, off;
+			chunk_place(i, src, dstOff, bpr, off);
+			const int64_t tb = tile_bytes(t0, bpr);
+			if(off + 16 <= tb) *(u32x4*) (ldsBytes + dstOff) = __builtin_nontemporal_load((const u32x4*) (src + t0 * bpr));
+			else copy_ragged(src + t0 * bpr, dstOff, tb - off);
 		}
 		if(tile + 1 < tileEnd) prefetch(tile + 1);
 
@@ -257,112 +288,86 @@ __global__ __launch_bounds__(DEC_THREADS) void k_rmm_decode(const DecArgs A) {
 				}
 			}
 		}
-		if(GRAM) { // dense groups: their rows of the tile, row major per group, zero beyond the matrix
-			for(int g = 0; g < nGroups; g++) {
-				const DecGroup P = planS[g];
-				if(P.type != G_UNC) continue;
-				const double* src = groups[g].dense + (size_t) t0 * P.nC;
-				const int64_t nIn = (min(nRows, rEnd) - t0) * P.nC;
-				for(int i = tid; i < DEC_TILE * P.nC; i += DEC_THREADS) Bs[P.pad + i] = i < nIn ? src[i] : 0.0;
-			}
-		}
 		__syncthreads();
 
 		if(GRAM) {
-			// wave w: rows w * 128 .. + 127 of the tile, four at a time
-			const int kRow = lane >> 4;
-#pragma unroll 2
-			for(int st = 0; st < DEC_TILE / (DEC_THREADS / 64) / 4; st++) {
-				const int rt = wave * (DEC_TILE / (DEC_THREADS / 64)) + st * 4 + kRow;
-				const bool in = t0 + rt < nRows;
-				double x[NB];
+			// wave: 128 rows of the tile; lane (k4, i16): rows k4 * 32 .. + 31, column 16 cb + i16
+#pragma unroll 1
+			for(int half = 0; half < 2; half++) {
+				const int rbase = wave * DEC_WROWS + k4 * 32 + half * 16;
+				DecCol D[NB];
+				double cst[NB];
+				u32x4 cq[NB][2];
 #pragma unroll
 				for(int cb = 0; cb < NB; cb++) {
-					const DecCol C = myCol[cb];
-					double v = 0.0;
-					if(C.kind == 1) {
-						const int code = C.slotW == 1 ? (int) slots[C.slotOff + rt] : (int) ((const uint16_t*) (slots + C.slotOff))[rt];
-						const bool has = in && code != (C.slotW == 1 ? 0xff : 0xffff);
-						v = C.constV + (has ? dictS[C.dictOff + code * C.nC + C.h] : 0.0);
-					}
-					else if(C.kind == 2)
-						v = C.constV + Bs[C.slotOff + rt * C.nC + C.h];
-					else if(C.kind == 3)
-						v = C.constV;
-					x[cb] = in ? v : 0.0;
+					D[cb] = colS[cb * 16 + i16];
+					cst[cb] = constS[cb * 16 + i16];
+					const bool coded = (D[cb].meta & 3) == 1;
+					const u32x4* cp = (const u32x4*) (slots + (coded ? D[cb].slotOff + rbase * ((D[cb].meta & 4) ? 2 : 1) : 0));
+					cq[cb][0] = cp[0];
+					cq[cb][1] = cp[1];
 				}
-				int t = 0;
 #pragma unroll
-				for(int ib = 0; ib < NB; ib++)
+				for(int s = 0; s < 16; s++) {
+					const bool in = t0 + rbase + s < nRows;
+					double x[NB];
 #pragma unroll
-					for(int jb = ib; jb < NB; jb++, t++) gram[t] = __builtin_amdgcn_mfma_f64_16x16x4f64(x[ib], x[jb], gram[t], 0, 0, 0);
+					for(int cb = 0; cb < NB; cb++) {
+						const int c1 = (int) ((cq[cb][0][s >> 2] >> (8 * (s & 3))) & 0xff);
+						const int c2 = (int) ((cq[cb][s >> 3][(s >> 1) & 3] >> (16 * (s & 1))) & 0xffff);
+						const double v = cst[cb] + dec_value(smem, D[cb], (D[cb].meta & 4) ? c2 : c1, rbase + s);
+						x[cb] = in ? v : 0.0;
+					}
+					int t = 0;
+#pragma unroll
+					for(int ib = 0; ib < NB; ib++)
+#pragma unroll
+						for(int jb = ib; jb < NB; jb++, t++) gram[t] = __builtin_amdgcn_mfma_f64_16x16x4f64(x[ib], x[jb], gram[t], 0, 0, 0);
+				}
 			}
 			continue;
 		}
 
-		// ---- decode two rows per thread
-		double acc0[Q], acc1[Q];
-#pragma unroll
-		for(int c = 0; c < Q; c++) { acc0[c] = 0.0; acc1[c] = 0.0; }
-		const int rt0 = tid, rt1 = tid + DEC_THREADS;
-		const int64_t r0 = t0 + rt0, r1 = t0 + rt1;
-		const bool in0 = r0 < nRows, in1 = r1 < nRows;
-		for(int g = 0; g < nGroups; g++) {
-			const DecGroup P = planS[g];
-			const int nC = P.nC;
-			if(P.slotOff < 0) { // dense columns
-				const double* dense = groups[g].dense;
-				for(int h = 0; h < nC; h++) {
-					const double a0 = in0 ? dense[(size_t) r0 * nC + h] : 0.0;
-					const double a1 = in1 ? dense[(size_t) r1 * nC + h] : 0.0;
-					const double* bq = Bs + (size_t) (P.kOff + h) * Q;
-#pragma unroll
-					for(int c = 0; c < Q; c++) { const double bv = bq[c]; acc0[c] += a0 * bv; acc1[c] += a1 * bv; }
-				}
-				continue;
-			}
-			int c0, c1;
-			bool v0, v1;
-			if(P.slotW == 1) {
-				c0 = slots[P.slotOff + rt0]; c1 = slots[P.slotOff + rt1];
-				v0 = in0 && c0 != 0xff; v1 = in1 && c1 != 0xff;
-			}
-			else {
-				c0 = ((const uint16_t*) (slots + P.slotOff))[rt0]; c1 = ((const uint16_t*) (slots + P.slotOff))[rt1];
-				v0 = in0 && c0 != 0xffff; v1 = in1 && c1 != 0xffff;
-			}
-			const double* p0 = dictS + P.dictOff + (v0 ? c0 * nC : 0);
-			const double* p1 = dictS + P.dictOff + (v1 ? c1 * nC : 0);
-			for(int h = 0; h < nC; h++) {
-				const double a0 = p0[h], a1 = p1[h];
-				const double* bq = Bs + (size_t) (P.kOff + h) * Q;
-				double bv[Q];
-#pragma unroll
-				for(int c = 0; c < Q; c++) bv[c] = bq[c];
-				if(v0) {
-#pragma unroll
-					for(int c = 0; c < Q; c++) acc0[c] += a0 * bv[c];
-				}
-				if(v1) {
-#pragma unroll
-					for(int c = 0; c < Q; c++) acc1[c] += a1 * bv[c];
-				}
-			}
-		}
-
-		// ---- output: two half tiles through LDS, full-line stores
-		const int q = A.q;
-#pragma unroll
+		// ---- X %*% B: wave = 128 rows in two passes of 64; lane (k4, i16): rows i16 * 4 .. + 3 of
+		// the pass as the A operand of decoded column 4 kb + k4, B[4 kb + k4, i16] as the B operand
+#pragma unroll 1
 		for(int half = 0; half < 2; half++) {
-			if(half == 1) __syncthreads(); // the first half has been read
+			const int pbase = wave * DEC_WROWS + half * 64;
+			const int rbase = pbase + i16 * 4;
+			f64x4 acc[4];
 #pragma unroll
-			for(int c = 0; c < Q; c++) otile[tid * OS + c] = (half == 0 ? acc0[c] : acc1[c]) + cadd[c];
-			__syncthreads();
-			const int64_t rowBase = t0 + (int64_t) half * DEC_THREADS;
-			const int nr = (int) max((int64_t) 0, min((int64_t) DEC_THREADS, nRows - rowBase));
-			for(int i = tid; i < nr * q; i += DEC_THREADS) {
-				const int rr = i / q, c = i - rr * q;
-				const double v = otile[rr * OS + c];
+			for(int s = 0; s < 4; s++) acc[s] = f64x4{cinit, cinit, cinit, cinit};
+			bool in[4];
+#pragma unroll
+			for(int s = 0; s < 4; s++) in[s] = t0 + rbase + s < nRows;
+#pragma unroll 2
+			for(int kb = 0; kb < KB; kb++) {
+				const DecCol D = colS[kb * 4 + k4];
+				const double bop = Bs[(kb * 4 + k4) * 16 + i16];
+				const bool coded = (D.meta & 3) == 1, two = D.meta & 4;
+				const uint32_t* cp = (const uint32_t*) (slots + (coded ? D.slotOff + rbase * (two ? 2 : 1) : 0));
+				const uint32_t lo = cp[0], hi = cp[1];
+#pragma unroll
+				for(int s = 0; s < 4; s++) {
+					const int c1 = (int) ((lo >> (8 * s)) & 0xff);
+					const int c2 = (int) (((s < 2 ? lo : hi) >> (16 * (s & 1))) & 0xffff);
+					const double v = dec_value(smem, D, two ? c2 : c1, rbase + s);
+					acc[s] = __builtin_amdgcn_mfma_f64_16x16x4f64(in[s] ? v : 0.0, bop, acc[s], 0, 0, 0);
+				}
+			}
+			// accumulator register v of lane l: output row 4 v + l / 16 of the step, output column l % 16
+			dec_wave_sync(); // the previous pass's readers of the staging area are done
+			if(i16 < q) {
+#pragma unroll
+				for(int s = 0; s < 4; s++)
+#pragma unroll
+					for(int v = 0; v < 4; v++) wstage[((4 * v + k4) * 4 + s) * q + i16] = acc[s][v];
+			}
+			dec_wave_sync();
+			const int64_t rowBase = t0 + pbase;
+			const int nr = (int) max((int64_t) 0, min((int64_t) 64, nRows - rowBase));
+			for(int i = lane; i < nr * q; i += 64) {
+				const double v = wstage[i];
 				cnt += v != 0.0;
 				__builtin_nontemporal_store(v, A.out + (size_t) rowBase * q + i);
 			}
@@ -373,7 +378,7 @@ __global__ __launch_bounds__(DEC_THREADS) void k_rmm_decode(const DecArgs A) {
 		// upper triangle. Accumulator register v of lane l is cell (4 v + l / 16, l % 16) of its tile.
 		constexpr int NP = NB * 16;
 		__syncthreads();
-		for(int i = tid; i < NP * NP; i += DEC_THREADS) otile[i] = 0.0;
+		for(int i = tid; i < NP * NP; i += DEC_THREADS) stage[i] = 0.0;
 		__syncthreads();
 		int t = 0;
 #pragma unroll
@@ -382,100 +387,145 @@ __global__ __launch_bounds__(DEC_THREADS) void k_rmm_decode(const DecArgs A) {
 			for(int jb = ib; jb < NB; jb++, t++)
 #pragma unroll
 				for(int v = 0; v < 4; v++)
-					unsafeAtomicAdd(&otile[(ib * 16 + 4 * v + (lane >> 4)) * NP + jb * 16 + (lane & 15)], gram[t][v]);
+					unsafeAtomicAdd(&stage[(ib * 16 + 4 * v + k4) * NP + jb * 16 + i16], gram[t][v]);
 		__syncthreads();
 		for(int i = tid; i < NP * NP; i += DEC_THREADS) {
 			const int r = i / NP, c = i - r * NP;
-			if(r <= c && c < A.nCols && otile[i] != 0.0) unsafeAtomicAdd(&A.out[(size_t) r * A.nCols + c], otile[i]);
+			if(r <= c && c < A.nCols && stage[i] != 0.0) unsafeAtomicAdd(&A.out[(size_t) r * A.nCols + c], stage[i]);
 		}
 		return;
 	}
 	count_add(A.nnz, cnt);
 }
 
-// LDS plan shared by both modes. gram: dense groups get an LDS tile (offset in DecGroup::pad,
-// doubles from the start of the aux region) instead of a share of the B copy, and groups
-// without row data (const, empty) get no code tile. Returns 1 when the block does not fit.
-static int dec_plan(cla_block* b, bool gram, int Q, DecArgs& A, size_t& lds, std::vector<DecGroup>& plan,
-	std::vector<DecCopy>& copies) {
+__global__ __launch_bounds__(DEC_THREADS) void k_rmm_decode(const DecArgs A) { decode_body<0, 1>(A); }
+
+template <int NB>
+__global__ __launch_bounds__(DEC_THREADS) void k_tsmm_decode(const DecArgs A) { decode_body<1, NB>(A); }
+
+// Host side of both kernels: LDS plan, copy list and column descriptors in the block's
+// scratch buffer. Returns 1 when the block does not fit (the caller uses another path).
+struct DecLaunch {
+	DecArgs A;
+	size_t lds = 0;
+	unsigned grid = 0;
+};
+
+static int dec_prepare(cla_block* b, bool gram, int q, DecLaunch& L) {
 	const int nG = (int) b->groups.size();
-	plan.assign((size_t) nG, DecGroup{});
-	copies.clear();
-	size_t dictD = 0, slotB = 0, denseD = 0;
-	int K = 0, nChunks = 0;
+	const int nCols = b->nCols;
+	std::vector<DecGroup> plan((size_t) nG);
+	size_t valD = 0, slotB = 0;
+	int K = 0;
 	for(int g = 0; g < nG; g++) {
 		const DGroup& G = b->groups[g].d;
 		DecGroup& P = plan[g];
 		P.type = G.type; P.nC = G.nColG; P.dictOff = -1; P.slotOff = -1; P.slotW = 0; P.copyIdx = -1; P.pad = 0;
 		P.kOff = K;
 		K += G.nColG;
+		if(G.nColG >= (1 << 14)) return 1;
 		if(G.type == G_UNC) {
-			P.pad = (int32_t) denseD;
-			denseD += (size_t) DEC_TILE * G.nColG;
+			P.dictOff = (int32_t) valD;
+			valD += (size_t) DEC_TILE * G.nColG;
 			continue;
 		}
-		if(gram && G.type != G_DDC && G.type != G_RLE && !(G.type == G_SDCZ && G.nOffsets > 0)) continue;
+		if(G.type != G_DDC && G.type != G_RLE && !(G.type == G_SDCZ && G.nOffsets > 0)) continue; // no row data
 		if(G.nVals > 65535) return 1;
-		P.dictOff = (int32_t) dictD;
-		dictD += (size_t) G.nVals * G.nColG;
+		P.dictOff = (int32_t) valD;
+		valD += (size_t) G.nVals * G.nColG;
 		P.slotW = G.nVals <= 255 ? 1 : 2;
 		P.slotOff = (int32_t) slotB;
-		slotB += (size_t) DEC_TILE * P.slotW;
-		if(G.type == G_DDC && G.codeWidth == P.slotW && ((uintptr_t) G.codes & 15) == 0) {
-			P.copyIdx = (int32_t) copies.size();
-			copies.push_back(DecCopy{g, nChunks});
-			nChunks += DEC_TILE * P.slotW / 16;
+		slotB += (size_t) DEC_TILE * P.slotW + DEC_SLOT_PAD;
+	}
+	if(valD == 0) valD = 2;
+	valD = (valD + 1) & ~(size_t) 1;
+	slotB = (slotB + 16 + 15) & ~(size_t) 15; // the multiply phase may read 16 bytes past the last tile
+	const int nColD = gram ? ((nCols + 15) / 16) * 16 : ((K + 3) / 4) * 4;
+	const size_t bD = gram ? 0 : (size_t) nColD * 16;
+	const size_t stageD = gram ? (size_t) nColD * nColD : (size_t) DEC_WAVES * 64 * q;
+	const size_t slotBase = (valD + bD + stageD) * 8;
+	// copy list
+	std::vector<DecCopy> copies;
+	int nChunks = 0;
+	for(int g = 0; g < nG; g++) {
+		const DGroup& G = b->groups[g].d;
+		DecGroup& P = plan[g];
+		DecCopy C;
+		C.pad = 0;
+		if(G.type == G_UNC) {
+			if(((uintptr_t) G.dense & 15) != 0) return 1;
+			C.src = (const uint8_t*) G.dense; C.bpr = G.nColG * 8; C.dstOff = P.dictOff * 8;
+		}
+		else if(P.slotOff >= 0 && G.type == G_DDC && G.codeWidth == P.slotW && ((uintptr_t) G.codes & 15) == 0) {
+			C.src = (const uint8_t*) G.codes; C.bpr = P.slotW; C.dstOff = (int32_t) (slotBase + P.slotOff);
+		}
+		else continue;
+		C.chunk0 = nChunks;
+		P.copyIdx = (int32_t) copies.size();
+		copies.push_back(C);
+		nChunks += DEC_TILE * C.bpr / 16;
+	}
+	L.lds = slotBase + slotB + (size_t) nColD * (sizeof(DecCol) + (gram ? 8 : 0)) + (size_t) nG * (sizeof(DecGroup) + 4) +
+		copies.size() * sizeof(DecCopy) + 64;
+	if(L.lds > (size_t) std::min(g_ldsPerBlock, 160 * 1024) - 1024) return 1;
+	// column descriptors: decoded column order (X %*% B) or matrix column order (t(X) %*% X)
+	std::vector<DecCol> cols((size_t) nColD, DecCol{0, 0, 0, 0});
+	std::vector<double> colConst((size_t) (gram ? nColD : 0), 0.0);
+	if(gram)
+		for(int c = 0; c < nCols; c++) colConst[c] = b->constV[c];
+	std::vector<char> seen((size_t) nCols, 0);
+	for(int g = 0; g < nG; g++) {
+		const DecGroup& P = plan[g];
+		const auto& hc = b->groups[g].cols;
+		for(int h = 0; h < P.nC; h++) {
+			if(gram && seen[hc[h]]) return 1; // overlapping groups
+			seen[hc[h]] = 1;
+			DecCol& C = cols[gram ? hc[h] : P.kOff + h];
+			const int kind = P.type == G_UNC ? 2 : P.slotOff >= 0 ? 1 : 0;
+			C.slotOff = kind == 1 ? P.slotOff : 0;
+			C.valOff = kind ? P.dictOff : 0;
+			C.meta = (int32_t) ((uint32_t) kind | (P.slotW == 2 ? 4u : 0u) | ((uint32_t) P.nC << 4) | ((uint32_t) h << 18));
 		}
 	}
-	if(dictD == 0) dictD = 1;
-	const size_t aux = gram ? denseD : (size_t) K * Q;
-	const size_t tileD = gram ? (size_t) Q * Q : (size_t) DEC_THREADS * (Q + 1);
-	lds = (dictD + aux + tileD) * 8 + slotB + (size_t) nG * (sizeof(DecGroup) + 4) + copies.size() * sizeof(DecCopy) + 96;
-	if(lds > (size_t) std::min(g_ldsPerBlock, 160 * 1024) - 1024) return 1;
-	A.nGroups = nG; A.nCopies = (int) copies.size(); A.nChunks = nChunks;
-	A.dictDoubles = (int) dictD; A.slotBytes = (int) ((slotB + 15) & ~(size_t) 15); A.K = K;
-	A.auxDoubles = (int) aux; A.tileDoubles = (int) tileD;
-	A.groups = b->dGroups; A.nRows = b->nRows;
-	A.B = nullptr; A.q = 0; A.constRow = nullptr; A.out = nullptr; A.nnz = nullptr; A.cols = nullptr; A.nCols = b->nCols;
+	const size_t planBytes = plan.size() * sizeof(DecGroup), copyBytes = copies.size() * sizeof(DecCopy);
+	const size_t colBytes = cols.size() * sizeof(DecCol), constBytes = colConst.size() * 8;
+	std::vector<uint8_t> img(planBytes + copyBytes + colBytes + constBytes);
+	std::memcpy(img.data(), copies.data(), copyBytes); // pointers first: 8-byte aligned
+	std::memcpy(img.data() + copyBytes, colConst.data(), constBytes);
+	std::memcpy(img.data() + copyBytes + constBytes, cols.data(), colBytes);
+	std::memcpy(img.data() + copyBytes + constBytes + colBytes, plan.data(), planBytes);
+	int rc = ensure_scratch(b, img.size() + 64);
+	if(rc) return rc;
+	uint8_t* d = (uint8_t*) b->dScratch;
+	CLA_HIP(hipMemcpyAsync(d, img.data(), img.size(), hipMemcpyHostToDevice, b->stream));
+	CLA_HIP(hipStreamSynchronize(b->stream));
+	DecArgs& A = L.A;
+	A.groups = b->dGroups;
+	A.copies = (const DecCopy*) d;
+	A.colConst = (const double*) (d + copyBytes);
+	A.cols = (const DecCol*) (d + copyBytes + constBytes);
+	A.plan = (const DecGroup*) (d + copyBytes + constBytes + colBytes);
+	A.nGroups = nG; A.nCopies = (int) copies.size(); A.nChunks = nChunks; A.nColD = nColD;
+	A.valDoubles = (int) valD; A.bDoubles = (int) bD; A.stageDoubles = (int) stageD; A.slotBytes = (int) slotB;
+	A.B = nullptr; A.q = q; A.constRow = nullptr; A.out = nullptr; A.nRows = b->nRows; A.nnz = nullptr; A.nCols = nCols;
+	const int nTiles = (int) ((b->nRows + DEC_TILE - 1) / DEC_TILE);
+	const int blocksPerCU = L.lds <= 76 * 1024 ? 2 : 1;
+	L.grid = (unsigned) std::min(nTiles, g_numCU * blocksPerCU);
 	return 0;
 }
 
 // Returns 1 when the block/shape is not eligible (caller uses the generic path).
 int launch_rmm_decode(cla_block* b, const double* dB, int q, const double* dConstRow, double* dOut,
 	unsigned long long* dNnz) {
-	const int nG = (int) b->groups.size();
-	if(nG == 0 || b->nRows == 0 || q < 2 || q > DEC_QMAX) return 1;
-	const int Q = q <= 4 ? 4 : q <= 8 ? 8 : q <= 12 ? 12 : 16;
-	std::vector<DecGroup> plan;
-	std::vector<DecCopy> copies;
-	DecArgs A;
-	size_t lds;
-	if(dec_plan(b, false, Q, A, lds, plan, copies)) return 1;
-	const size_t planBytes = plan.size() * sizeof(DecGroup), copyBytes = copies.size() * sizeof(DecCopy);
-	int rc = ensure_scratch(b, planBytes + copyBytes + 64);
+	if(b->groups.empty() || b->nRows == 0 || q < 2 || q > DEC_QMAX) return 1;
+	DecLaunch L;
+	int rc = dec_prepare(b, false, q, L);
 	if(rc) return rc;
-	DecGroup* dPlan = (DecGroup*) b->dScratch;
-	DecCopy* dCopies = (DecCopy*) ((uint8_t*) b->dScratch + planBytes);
-	CLA_HIP(hipMemcpyAsync(dPlan, plan.data(), planBytes, hipMemcpyHostToDevice, b->stream));
-	if(copyBytes) CLA_HIP(hipMemcpyAsync(dCopies, copies.data(), copyBytes, hipMemcpyHostToDevice, b->stream));
-	CLA_HIP(hipStreamSynchronize(b->stream));
-	const int nTiles = (int) ((b->nRows + DEC_TILE - 1) / DEC_TILE);
-	const int blocksPerCU = lds <= 76 * 1024 ? 2 : 1;
-	const unsigned grid = (unsigned) std::min(nTiles, g_numCU * blocksPerCU);
-	A.plan = dPlan; A.copies = dCopies;
-	A.B = dB; A.q = q; A.constRow = dConstRow; A.out = dOut; A.nnz = dNnz;
+	L.A.B = dB; L.A.constRow = dConstRow; L.A.out = dOut; L.A.nnz = dNnz;
 	double algo = (double) b->device_bytes_cached + (double) b->nRows * q * 8;
-	Prof pf(b, "k_rmm_decode", grid, DEC_THREADS, (long) lds, algo);
-#define DEC_LAUNCH(QV)                                                                                          \
-	do {                                                                                                        \
-		CLA_HIP(hipFuncSetAttribute((const void*) k_rmm_decode<QV>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds)); \
-		hipLaunchKernelGGL(k_rmm_decode<QV>, dim3(grid), dim3(DEC_THREADS), lds, b->stream, A);                 \
-	} while(0)
-	if(Q == 4) DEC_LAUNCH(4);
-	else if(Q == 8) DEC_LAUNCH(8);
-	else if(Q == 12) DEC_LAUNCH(12);
-	else DEC_LAUNCH(16);
-#undef DEC_LAUNCH
+	Prof pf(b, "k_rmm_decode", L.grid, DEC_THREADS, (long) L.lds, algo);
+	CLA_HIP(hipFuncSetAttribute((const void*) k_rmm_decode, hipFuncAttributeMaxDynamicSharedMemorySize, (int) L.lds));
+	hipLaunchKernelGGL(k_rmm_decode, dim3(L.grid), dim3(DEC_THREADS), L.lds, b->stream, L.A);
 	CLA_HIP(hipGetLastError());
 	return 0;
 }
@@ -483,49 +533,18 @@ int launch_rmm_decode(cla_block* b, const double* dB, int q, const double* dCons
 // dOut (nCols x nCols, zeroed) += upper triangle of t(D) %*% D of the decoded rows, constants
 // included. Returns 1 when the block is not eligible (more than 64 columns, LDS plan too large).
 int launch_tsmm_decode(cla_block* b, double* dOut) {
-	const int nG = (int) b->groups.size();
 	const int nCols = b->nCols;
-	if(nG == 0 || b->nRows == 0 || nCols > 64) return 1;
+	if(b->groups.empty() || b->nRows == 0 || nCols > 64) return 1;
 	const int NB = (nCols + 15) / 16;
-	std::vector<DecGroup> plan;
-	std::vector<DecCopy> copies;
-	DecArgs A;
-	size_t lds;
-	if(dec_plan(b, true, NB * 16, A, lds, plan, copies)) return 1;
-	std::vector<DecCol> cols((size_t) NB * 16);
-	for(auto& c : cols) { c.kind = 0; c.slotOff = 0; c.slotW = 1; c.dictOff = 0; c.nC = 1; c.h = 0; c.constV = 0.0; }
-	for(int c = 0; c < nCols; c++) { cols[c].kind = 3; cols[c].constV = b->constV[c]; }
-	for(int g = 0; g < nG; g++) {
-		const DecGroup& P = plan[g];
-		const auto& hc = b->groups[g].cols;
-		for(int h = 0; h < P.nC; h++) {
-			DecCol& C = cols[hc[h]];
-			if(C.kind != 3) return 1; // overlapping groups
-			C.nC = P.nC; C.h = h;
-			if(P.type == G_UNC) { C.kind = 2; C.slotOff = P.pad; }
-			else if(P.slotOff >= 0) { C.kind = 1; C.slotOff = P.slotOff; C.slotW = P.slotW; C.dictOff = P.dictOff; }
-		}
-	}
-	const size_t planBytes = plan.size() * sizeof(DecGroup), copyBytes = copies.size() * sizeof(DecCopy);
-	const size_t colOff = (planBytes + copyBytes + 15) & ~(size_t) 15, colBytes = cols.size() * sizeof(DecCol);
-	int rc = ensure_scratch(b, colOff + colBytes + 64);
+	DecLaunch L;
+	int rc = dec_prepare(b, true, 0, L);
 	if(rc) return rc;
-	DecGroup* dPlan = (DecGroup*) b->dScratch;
-	DecCopy* dCopies = (DecCopy*) ((uint8_t*) b->dScratch + planBytes);
-	DecCol* dCols = (DecCol*) ((uint8_t*) b->dScratch + colOff);
-	CLA_HIP(hipMemcpyAsync(dPlan, plan.data(), planBytes, hipMemcpyHostToDevice, b->stream));
-	if(copyBytes) CLA_HIP(hipMemcpyAsync(dCopies, copies.data(), copyBytes, hipMemcpyHostToDevice, b->stream));
-	CLA_HIP(hipMemcpyAsync(dCols, cols.data(), colBytes, hipMemcpyHostToDevice, b->stream));
-	CLA_HIP(hipStreamSynchronize(b->stream));
-	const int nTiles = (int) ((b->nRows + DEC_TILE - 1) / DEC_TILE);
-	const int blocksPerCU = lds <= 76 * 1024 ? 2 : 1;
-	const unsigned grid = (unsigned) std::min(nTiles, g_numCU * blocksPerCU);
-	A.plan = dPlan; A.copies = dCopies; A.cols = dCols; A.out = dOut;
-	Prof pf(b, "k_tsmm_decode", grid, DEC_THREADS, (long) lds, (double) b->device_bytes_cached);
+	L.A.out = dOut;
+	Prof pf(b, "k_tsmm_decode", L.grid, DEC_THREADS, (long) L.lds, (double) b->device_bytes_cached);
 #define GRAM_LAUNCH(NBV)                                                                                        \
 	do {                                                                                                        \
-		CLA_HIP(hipFuncSetAttribute((const void*) k_rmm_decode<NBV * 16, 1, NBV>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds)); \
-		hipLaunchKernelGGL((k_rmm_decode<NBV * 16, 1, NBV>), dim3(grid), dim3(DEC_THREADS), lds, b->stream, A); \
+		CLA_HIP(hipFuncSetAttribute((const void*) k_tsmm_decode<NBV>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) L.lds)); \
+		hipLaunchKernelGGL(k_tsmm_decode<NBV>, dim3(L.grid), dim3(DEC_THREADS), L.lds, b->stream, L.A);         \
 	} while(0)
 	if(NB == 1) GRAM_LAUNCH(1);
 	else if(NB == 2) GRAM_LAUNCH(2);
