@@ -11,6 +11,34 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef double f64x2 __attribute__((ext_vector_type(2)));
 
+// A pointer read out of a descriptor in memory is a generic pointer to the compiler, and a
+// generic load also counts on the LDS counter: every wait for LDS data then waits for those
+// loads too. All descriptor pointers point into device global memory; as_global says so
+// (the empty asm keeps the round trip through the global address space from being folded
+// away; the address-space inference then turns every access through the result into a
+// global one).
+template <class T>
+__device__ __forceinline__ T* as_global(T* p) {
+	__attribute__((address_space(1))) T* g = (__attribute__((address_space(1))) T*) p;
+	asm("" : "+v"(g));
+	return (T*) g;
+}
+
+// Descriptor copy whose pointers are known to be global.
+__device__ __forceinline__ DGroup dgroup(const DGroup* p) {
+	DGroup g = *p;
+	g.codes = as_global(g.codes);
+	g.dict = as_global(g.dict);
+	g.cols = as_global(g.cols);
+	g.deltas = as_global(g.deltas);
+	g.ckpt = as_global(g.ckpt);
+	g.tileIdx = as_global(g.tileIdx);
+	g.runStart = as_global(g.runStart);
+	g.runCode = as_global(g.runCode);
+	g.dense = as_global(g.dense);
+	return g;
+}
+
 // AMapToData.getIndex for the three device code widths (unsigned byte, char, int).
 __device__ __forceinline__ int32_t load_code(const void* codes, int width, int64_t i) {
 	if(width == 1) return ((const uint8_t*) codes)[i];

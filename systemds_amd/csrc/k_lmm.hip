@@ -40,7 +40,7 @@ __global__ __launch_bounds__(LMM_THREADS) void k_lmm_preagg_rows(const DGroup* _
 #pragma unroll
 		for(int t = 0; t < LMM_RPT; t++) yv[t] = t < n ? y[r0 + t] : 0.0;
 		for(int g = g0; g < g1; g++) {
-			const DGroup& G = groups[g];
+			const DGroup G = dgroup(groups + (g));
 			double* bg = bins + (G.tblOff - base);
 			if(G.type == G_DDC) {
 				if(n == LMM_RPT && G.codeWidth == 1) {
@@ -83,7 +83,7 @@ template <int W>
 __global__ __launch_bounds__(256) void k_lmm_preagg_sdc(const DGroup* __restrict__ groups, int g, const double* __restrict__ Y,
 	int64_t nRows, int chunksPerBlock, double* __restrict__ pre, int totalVals, int direct) {
 	extern __shared__ double ldsBins[];
-	const DGroup& G = groups[g];
+	const DGroup G = dgroup(groups + (g));
 	const int i = blockIdx.y;
 	const double* y = Y + (size_t) i * nRows;
 	double* bins = direct ? pre + (size_t) i * totalVals + G.tblOff : ldsBins;
@@ -121,7 +121,7 @@ __global__ __launch_bounds__(256) void k_lmm_preagg_sdc(const DGroup* __restrict
 __global__ __launch_bounds__(256) void k_lmm_unc(const DGroup* __restrict__ groups, int g, const double* __restrict__ Y,
 	int64_t nRows, int64_t rowsPerBlock, double* __restrict__ out, int nCols) {
 	__shared__ double red[4];
-	const DGroup& G = groups[g];
+	const DGroup G = dgroup(groups + (g));
 	const int i = blockIdx.y;
 	const double* y = Y + (size_t) i * nRows;
 	const int64_t rb = (int64_t) blockIdx.x * rowsPerBlock, re = min(rb + rowsPerBlock, nRows);
@@ -154,7 +154,7 @@ __global__ __launch_bounds__(256) void k_lmm_rowsum(const double* __restrict__ Y
 __global__ __launch_bounds__(256) void k_lmm_post(const DGroup* __restrict__ groups, const double* __restrict__ pre,
 	int totalVals, double* __restrict__ out, int nCols) {
 	__shared__ double red[4];
-	const DGroup& G = groups[blockIdx.x];
+	const DGroup G = dgroup(groups + (blockIdx.x));
 	if(G.type == G_UNC) return;
 	const int i = blockIdx.y;
 	const double* p = pre + (size_t) i * totalVals + G.tblOff;

@@ -102,7 +102,7 @@ __global__ __launch_bounds__(LU_THREADS) void k_lmm_u8(const DGroup* __restrict_
 		// flush: copies summed, one global add per non-zero bin
 		for(int k = tid; k < nIn * 256; k += THREADS) {
 			const int g = k >> 8, c = k & 255;
-			const DGroup& G = groups[g0 + g];
+			const DGroup G = dgroup(groups + (g0 + g));
 			if(c >= G.nVals) continue;
 			double v = 0.0;
 #pragma unroll

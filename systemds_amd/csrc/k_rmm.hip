@@ -37,7 +37,7 @@ __global__ void k_preagg(const DGroup* __restrict__ groups, int nGroups, const d
 		T[(size_t) totalVals * q + idx] = acc;
 		return;
 	}
-	const DGroup G = groups[g];
+	const DGroup G = dgroup(groups + g);
 	if(G.type == G_UNC || idx >= G.nVals * q) return;
 	const int k = idx / q, c = idx - k * q;
 	double acc = 0;
@@ -404,7 +404,7 @@ __global__ __launch_bounds__(256) void k_rmm_rows(const DGroup* __restrict__ gro
 #pragma unroll
 	for(int c = 0; c < ROWS_QS; c++) acc[c] = 0.0;
 	for(int g = 0; g < nGroups; g++) {
-		const DGroup& G = groups[g];
+		const DGroup G = dgroup(groups + (g));
 		if(G.type == G_DDC) {
 			if(live) {
 				const double* t = T + (size_t) (G.tblOff + load_code(G.codes, G.codeWidth, r)) * q + c0;
@@ -453,7 +453,7 @@ __global__ __launch_bounds__(256) void k_rmm_rows(const DGroup* __restrict__ gro
 template <int W>
 __global__ __launch_bounds__(256) void k_rmm_sdc_scatter(const DGroup* __restrict__ groups, int g,
 	const double* __restrict__ T, int q, double* __restrict__ out) {
-	const DGroup& G = groups[g];
+	const DGroup G = dgroup(groups + (g));
 	const int chunk = blockIdx.x;
 	const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
 	const double* Tg = T + (size_t) G.tblOff * q;

@@ -90,15 +90,26 @@ __device__ __forceinline__ void dec_wave_sync() {
 	__builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-// Value of one decoded column at tile row rt (code c from the column's tile); 0 where the row has none.
-__device__ __forceinline__ double dec_value(const double* smem, const DecCol D, int c, int rt) {
-	const int kind = D.meta & 3, nC = (D.meta >> 4) & 0x3fff, h = (int) ((unsigned) D.meta >> 18);
-	const bool two = D.meta & 4;
-	const bool valid = kind == 2 || (kind == 1 && c != (two ? 0xffff : 0xff));
-	const int addr = D.valOff + (kind == 1 ? c : rt) * nC + h;
-	const double v = smem[valid ? addr : 0];
-	return valid ? v : 0.0;
-}
+// One decoded column, unpacked once per pass; lookups are then branch-free selects.
+struct DecLook {
+	int base;      // valOff + h
+	int nC;
+	int sent;      // no-value code of the column's tile; -1 when the column has no code tile
+	bool coded, dense, two;
+	__device__ __forceinline__ DecLook(const DecCol D) {
+		const int kind = D.meta & 3;
+		coded = kind == 1; dense = kind == 2; two = (D.meta & 4) != 0;
+		nC = (D.meta >> 4) & 0x3fff;
+		base = D.valOff + (int) ((unsigned) D.meta >> 18);
+		sent = coded ? (two ? 0xffff : 0xff) : -1;
+	}
+	// LDS index (doubles) of the value at tile row rt with code c, and whether the row has one
+	__device__ __forceinline__ int addr(int c, int rt, bool& valid) const {
+		valid = dense | (coded & (c != sent));
+		const int a = base + (coded ? c : rt) * nC;
+		return valid ? a : 0;
+	}
+};
 
 template <int GRAM, int NB>
 __device__ __forceinline__ void decode_body(const DecArgs& A) {
@@ -110,7 +121,8 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 	double* constS = (double*) (colS + A.nColD);                   // nColD (Gram mode)
 	DecGroup* planS = (DecGroup*) (constS + (GRAM ? A.nColD : 0)); // nGroups
 	DecCopy* copyS = (DecCopy*) (planS + A.nGroups);               // nCopies
-	int32_t* runBase = (int32_t*) (copyS + A.nCopies);             // nGroups
+	DGroup* groupS = (DGroup*) (copyS + A.nCopies);                // nGroups: descriptors, so that a wave task starts from LDS
+	int32_t* runBase = (int32_t*) (groupS + A.nGroups);            // nGroups
 	const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
 	const int i16 = lane & 15, k4 = lane >> 4;
 	const DGroup* __restrict__ groups = A.groups;
@@ -125,7 +137,8 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 	// ---- once per block: plan, column descriptors, dictionaries, B, run cursors
 	for(int g = tid; g < nGroups; g += DEC_THREADS) {
 		planS[g] = A.plan[g];
-		runBase[g] = groups[g].type == G_RLE ? rle_find(groups[g].runStart, groups[g].nRuns, (int32_t) ((int64_t) tileBeg * DEC_TILE)) : 0;
+		groupS[g] = groups[g];
+		runBase[g] = groups[g].type == G_RLE ? rle_find(as_global(groups[g].runStart), groups[g].nRuns, (int32_t) ((int64_t) tileBeg * DEC_TILE)) : 0;
 	}
 	for(int i = tid; i < A.nCopies; i += DEC_THREADS) copyS[i] = A.copies[i];
 	for(int i = tid; i < A.nColD; i += DEC_THREADS) {
@@ -138,7 +151,7 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 	__syncthreads();
 	for(int g = 0; g < nGroups; g++) {
 		const DecGroup P = planS[g];
-		const DGroup& G = groups[g];
+		const DGroup G = dgroup(groups + (g));
 		if(P.slotOff >= 0) {
 			const int n = G.nVals * G.nColG;
 			for(int i = tid; i < n; i += DEC_THREADS) smem[P.dictOff + i] = G.dict[i];
@@ -162,7 +175,7 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 		const DecCopy C = copyS[lo];
 		off = (i - C.chunk0) * 16;
 		bpr = C.bpr;
-		src = C.src + off;
+		src = as_global(C.src + off);
 		dstOff = C.dstOff + off;
 	};
 	uint8_t* const ldsBytes = (uint8_t*) smem;
@@ -222,13 +235,12 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 			if(off + 16 <= tb) *(u32x4*) (ldsBytes + dstOff) = __builtin_nontemporal_load((const u32x4*) (src + t0 * bpr));
 			else copy_ragged(src + t0 * bpr, dstOff, tb - off);
 		}
-		if(tile + 1 < tileEnd) prefetch(tile + 1);
 
 		// ---- other dictionary coded groups, one wave per group
 		for(int g = wave; g < nGroups; g += DEC_THREADS / 64) {
 			const DecGroup P = planS[g];
 			if(P.slotOff < 0 || P.copyIdx >= 0) continue;
-			const DGroup& G = groups[g];
+			const DGroup G = dgroup(groupS + g);
 			uint8_t* slot = slots + P.slotOff;
 			const int w = P.slotW;
 			if(P.type == G_DDC) { // code width differs from the tile's: convert
@@ -289,40 +301,59 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 			}
 		}
 		__syncthreads();
+		// issued behind the wave tasks: loads return in order, so a task's first load would
+		// otherwise wait for the whole prefetch
+		if(tile + 1 < tileEnd) prefetch(tile + 1);
 
 		if(GRAM) {
 			// wave: 128 rows of the tile; lane (k4, i16): rows k4 * 32 .. + 31, column 16 cb + i16
 #pragma unroll 1
 			for(int half = 0; half < 2; half++) {
 				const int rbase = wave * DEC_WROWS + k4 * 32 + half * 16;
-				DecCol D[NB];
 				double cst[NB];
 				u32x4 cq[NB][2];
+				int lbase[NB], lnC[NB], lsent[NB];
+				bool lcoded[NB], ldense[NB], ltwo[NB];
 #pragma unroll
 				for(int cb = 0; cb < NB; cb++) {
-					D[cb] = colS[cb * 16 + i16];
+					const DecLook L(colS[cb * 16 + i16]);
+					lbase[cb] = L.base; lnC[cb] = L.nC; lsent[cb] = L.sent; lcoded[cb] = L.coded; ldense[cb] = L.dense; ltwo[cb] = L.two;
 					cst[cb] = constS[cb * 16 + i16];
-					const bool coded = (D[cb].meta & 3) == 1;
-					const u32x4* cp = (const u32x4*) (slots + (coded ? D[cb].slotOff + rbase * ((D[cb].meta & 4) ? 2 : 1) : 0));
+					const u32x4* cp = (const u32x4*) (slots + (L.coded ? colS[cb * 16 + i16].slotOff + rbase * (L.two ? 2 : 1) : 0));
 					cq[cb][0] = cp[0];
 					cq[cb][1] = cp[1];
 				}
+				// SB steps of lookups in flight, then their products
+				constexpr int SB = NB <= 2 ? 4 : 2;
 #pragma unroll
-				for(int s = 0; s < 16; s++) {
-					const bool in = t0 + rbase + s < nRows;
-					double x[NB];
+				for(int sb = 0; sb < 16; sb += SB) {
+					double x[SB][NB];
 #pragma unroll
-					for(int cb = 0; cb < NB; cb++) {
-						const int c1 = (int) ((cq[cb][0][s >> 2] >> (8 * (s & 3))) & 0xff);
-						const int c2 = (int) ((cq[cb][s >> 3][(s >> 1) & 3] >> (16 * (s & 1))) & 0xffff);
-						const double v = cst[cb] + dec_value(smem, D[cb], (D[cb].meta & 4) ? c2 : c1, rbase + s);
-						x[cb] = in ? v : 0.0;
+					for(int u = 0; u < SB; u++) {
+						const int s = sb + u;
+#pragma unroll
+						for(int cb = 0; cb < NB; cb++) {
+							const int c1 = (int) ((cq[cb][0][s >> 2] >> (8 * (s & 3))) & 0xff);
+							const int c2 = (int) ((cq[cb][s >> 3][(s >> 1) & 3] >> (16 * (s & 1))) & 0xffff);
+							const int c = ltwo[cb] ? c2 : c1;
+							const bool valid = ldense[cb] | (lcoded[cb] & (c != lsent[cb]));
+							const int ad = lbase[cb] + (lcoded[cb] ? c : rbase + s) * lnC[cb];
+							const double v = smem[valid ? ad : 0];
+							x[u][cb] = valid ? v : 0.0;
+						}
 					}
-					int t = 0;
 #pragma unroll
-					for(int ib = 0; ib < NB; ib++)
+					for(int u = 0; u < SB; u++) {
+						const bool in = t0 + rbase + sb + u < nRows;
 #pragma unroll
-						for(int jb = ib; jb < NB; jb++, t++) gram[t] = __builtin_amdgcn_mfma_f64_16x16x4f64(x[ib], x[jb], gram[t], 0, 0, 0);
+						for(int cb = 0; cb < NB; cb++) x[u][cb] = in ? cst[cb] + x[u][cb] : 0.0;
+						int t = 0;
+#pragma unroll
+						for(int ib = 0; ib < NB; ib++)
+#pragma unroll
+							for(int jb = ib; jb < NB; jb++, t++)
+								gram[t] = __builtin_amdgcn_mfma_f64_16x16x4f64(x[u][ib], x[u][jb], gram[t], 0, 0, 0);
+					}
 				}
 			}
 			continue;
@@ -344,16 +375,21 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 			for(int kb = 0; kb < KB; kb++) {
 				const DecCol D = colS[kb * 4 + k4];
 				const double bop = Bs[(kb * 4 + k4) * 16 + i16];
-				const bool coded = (D.meta & 3) == 1, two = D.meta & 4;
-				const uint32_t* cp = (const uint32_t*) (slots + (coded ? D.slotOff + rbase * (two ? 2 : 1) : 0));
+				const DecLook L(D);
+				const uint32_t* cp = (const uint32_t*) (slots + (L.coded ? D.slotOff + rbase * (L.two ? 2 : 1) : 0));
 				const uint32_t lo = cp[0], hi = cp[1];
+				double x[4];
 #pragma unroll
 				for(int s = 0; s < 4; s++) {
 					const int c1 = (int) ((lo >> (8 * s)) & 0xff);
 					const int c2 = (int) (((s < 2 ? lo : hi) >> (16 * (s & 1))) & 0xffff);
-					const double v = dec_value(smem, D, two ? c2 : c1, rbase + s);
-					acc[s] = __builtin_amdgcn_mfma_f64_16x16x4f64(in[s] ? v : 0.0, bop, acc[s], 0, 0, 0);
+					bool valid;
+					const int ad = L.addr(L.two ? c2 : c1, rbase + s, valid);
+					const double v = smem[ad];
+					x[s] = (valid & in[s]) ? v : 0.0;
 				}
+#pragma unroll
+				for(int s = 0; s < 4; s++) acc[s] = __builtin_amdgcn_mfma_f64_16x16x4f64(x[s], bop, acc[s], 0, 0, 0);
 			}
 			// accumulator register v of lane l: output row 4 v + l / 16 of the step, output column l % 16
 			dec_wave_sync(); // the previous pass's readers of the staging area are done
@@ -465,7 +501,7 @@ static int dec_prepare(cla_block* b, bool gram, int q, DecLaunch& L) {
 		copies.push_back(C);
 		nChunks += DEC_TILE * C.bpr / 16;
 	}
-	L.lds = slotBase + slotB + (size_t) nColD * (sizeof(DecCol) + (gram ? 8 : 0)) + (size_t) nG * (sizeof(DecGroup) + 4) +
+	L.lds = slotBase + slotB + (size_t) nColD * (sizeof(DecCol) + (gram ? 8 : 0)) + (size_t) nG * (sizeof(DecGroup) + sizeof(DGroup) + 4) +
 		copies.size() * sizeof(DecCopy) + 64;
 	if(L.lds > (size_t) std::min(g_ldsPerBlock, 160 * 1024) - 1024) return 1;
 	// column descriptors: decoded column order (X %*% B) or matrix column order (t(X) %*% X)

@@ -82,7 +82,7 @@ __global__ __launch_bounds__(MF_WAVES * 64) void k_rmm_mfma(const DGroup* __rest
 		__syncthreads();
 		if(tid == 0) dictS[0] = 0.0;
 		{
-			const double* src = groups[sl.g0].dict;
+			const double* src = as_global(groups[sl.g0].dict);
 			const int n = sl.dictDoubles - 1;
 			for(int i = tid; i < n; i += MF_THREADS) dictS[1 + i] = src[i];
 		}
@@ -100,7 +100,7 @@ __global__ __launch_bounds__(MF_WAVES * 64) void k_rmm_mfma(const DGroup* __rest
 			src.codes = nullptr; src.dictOff = 0; src.nColG = 0; src.width = 0;
 			if(c < sl.nc) {
 				const MfCol mc = cols[sl.c0 + c];
-				const DGroup& G = groups[mc.group];
+				const DGroup G = dgroup(groups + (mc.group));
 				src.codes = (const uint8_t*) G.codes + (size_t) blockRow0 * G.codeWidth;
 				src.dictOff = mc.dictOff; src.nColG = mc.nColG; src.width = G.codeWidth;
 			}
@@ -113,7 +113,8 @@ __global__ __launch_bounds__(MF_WAVES * 64) void k_rmm_mfma(const DGroup* __rest
 #pragma unroll 4
 			for(int i = tid; i < nQuads; i += MF_THREADS) {
 				const int c = i / (MF_ROWS / 4), r4 = (i - c * (MF_ROWS / 4)) * 4;
-				const MfSrc src = srcS[c];
+				MfSrc src = srcS[c];
+				src.codes = as_global(src.codes);
 				uint32_t o[4] = {0, 0, 0, 0};
 				if(src.width != 0) {
 					int c4[4];

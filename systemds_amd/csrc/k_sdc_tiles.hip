@@ -67,7 +67,7 @@ __global__ __launch_bounds__(ST_THREADS) void k_lmm_sdc_tiles(const DGroup* __re
 		for(int t = tid; t < ST; t += ST_THREADS) ytile[t] = r0 + t < nRows ? y[r0 + t] : 0.0;
 		__syncthreads();
 		for(int l = l0 + wave; l < l1; l += ST_THREADS / 64) {
-			const DGroup& G = groups[sdcList[l]];
+			const DGroup G = dgroup(groups + (sdcList[l]));
 			double* bg = bins + (binOff[l] - b0);
 			const void* codes = G.codes;
 			const int cw = G.codeWidth;
@@ -76,7 +76,7 @@ __global__ __launch_bounds__(ST_THREADS) void k_lmm_sdc_tiles(const DGroup* __re
 	}
 	__syncthreads();
 	for(int l = l0; l < l1; l++) {
-		const DGroup& G = groups[sdcList[l]];
+		const DGroup G = dgroup(groups + (sdcList[l]));
 		const double* bg = bins + (binOff[l] - b0);
 		double* dst = pre + (size_t) i * totalVals + G.tblOff;
 		for(int k = tid; k < G.nVals; k += ST_THREADS) {
@@ -113,14 +113,14 @@ __global__ __launch_bounds__(ST_THREADS) void k_rmm_sdc_tiles(const DGroup* __re
 		const int b0 = binOff[l0];
 		__syncthreads();
 		for(int l = l0; l < l1; l++) {
-			const DGroup& G = groups[sdcList[l]];
+			const DGroup G = dgroup(groups + (sdcList[l]));
 			double* tg = tbl + (size_t) (binOff[l] - b0) * q;
 			const double* src = T + (size_t) G.tblOff * q;
 			for(int k = tid; k < G.nVals * q; k += ST_THREADS) tg[k] = src[k];
 		}
 		__syncthreads();
 		for(int l = l0 + wave; l < l1; l += ST_THREADS / 64) {
-			const DGroup& G = groups[sdcList[l]];
+			const DGroup G = dgroup(groups + (sdcList[l]));
 			const double* tg = tbl + (size_t) (binOff[l] - b0) * q;
 			const void* codes = G.codes;
 			const int cw = G.codeWidth;

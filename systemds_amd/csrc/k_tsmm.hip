@@ -110,8 +110,8 @@ __global__ __launch_bounds__(PAIR_THREADS) void k_tsmm_pair(const DGroup* __rest
 	constexpr int TSMM_THREADS = PAIR_THREADS;
 	extern __shared__ double smem[];
 	const int4 pr = pairs[blockIdx.y]; // (target, source, dictInLds, 0)
-	const DGroup& Gt = groups[pr.x];
-	const DGroup& Gs = groups[pr.y];
+	const DGroup Gt = dgroup(groups + (pr.x));
+	const DGroup Gs = dgroup(groups + (pr.y));
 	const int dictInLds = pr.z;
 	const int nCs = Gs.nColG, nCt = Gt.nColG;
 	double* P = smem;                                             // nVals_t * nCs
@@ -205,8 +205,8 @@ __global__ __launch_bounds__(PD_THREADS) void k_tsmm_pair_dot(const DGroup* __re
 	const int cp = blockIdx.x / blocksPerChunkPair;
 	const int pairIdx = cp % nPairs, chunk = cp / nPairs;
 	const int4 pr = pairs[pairIdx];
-	const DGroup& Gt = groups[pr.x];
-	const DGroup& Gs = groups[pr.y];
+	const DGroup Gt = dgroup(groups + (pr.x));
+	const DGroup Gs = dgroup(groups + (pr.y));
 	double* dT = smem;                                   // nVals_t * NCT
 	double* dS = smem + (((size_t) Gt.nVals * NCT + 1) & ~(size_t) 1); // nVals_s * NCS, 16-byte aligned
 	for(int i = tid; i < Gt.nVals * NCT; i += PD_THREADS) dT[i] = Gt.dict[i];
@@ -292,7 +292,7 @@ static void launch_pair_dot_cw(int nct, int ncs, dim3 grid, size_t lds, hipStrea
 __global__ __launch_bounds__(256) void k_tsmm_self(const DGroup* __restrict__ groups, const int32_t* __restrict__ countsAll,
 	double* __restrict__ out, int nCols, double* __restrict__ colSum) {
 	__shared__ double red[4];
-	const DGroup& G = groups[blockIdx.y];
+	const DGroup G = dgroup(groups + (blockIdx.y));
 	if(G.type == G_UNC) return;
 	const int32_t* counts = countsAll + G.tblOff;
 	const int nC = G.nColG, tid = threadIdx.x;
@@ -342,7 +342,7 @@ __global__ __launch_bounds__(256) void k_tsmm_dense(const DGroup* __restrict__ g
 		for(int i = tid; i < DT * nCols; i += 256) D[i] = (i / nCols) < nr ? constV[i % nCols] : 0.0;
 		__syncthreads();
 		for(int g = 0; g < nGroups; g++) {
-			const DGroup& G = groups[g];
+			const DGroup G = dgroup(groups + (g));
 			if(G.type == G_DDC || G.type == G_RLE) {
 				for(int t = tid; t < nr; t += 256) {
 					const int64_t r = r0 + t;
@@ -612,8 +612,8 @@ __global__ __launch_bounds__(TSMM_THREADS) void k_cooc(const DGroup* __restrict_
 	int tilesPerBlock, int useLds, unsigned long long* __restrict__ N) {
 	extern __shared__ unsigned int lbins[];
 	__shared__ int32_t ca[TT], cb[TT];
-	const DGroup& A = groups[ga];
-	const DGroup& B = groups[gb];
+	const DGroup A = dgroup(groups + (ga));
+	const DGroup B = dgroup(groups + (gb));
 	const int tid = threadIdx.x;
 	const int nBins = A.nVals * B.nVals;
 	if(useLds) {
@@ -669,7 +669,7 @@ __global__ __launch_bounds__(256) void k_decompress_fill(double* __restrict__ ou
 
 __global__ __launch_bounds__(256) void k_decompress_rows(const DGroup* __restrict__ groups, int g, int64_t nRows, int nCols,
 	double* __restrict__ out) {
-	const DGroup& G = groups[g];
+	const DGroup G = dgroup(groups + (g));
 	const int64_t idx = (int64_t) blockIdx.x * 256 + threadIdx.x;
 	if(idx >= nRows * G.nColG) return;
 	const int64_t r = idx / G.nColG;
@@ -687,7 +687,7 @@ __global__ __launch_bounds__(256) void k_decompress_rows(const DGroup* __restric
 template <int W>
 __global__ __launch_bounds__(256) void k_decompress_sdc(const DGroup* __restrict__ groups, int g, int nCols,
 	double* __restrict__ out) {
-	const DGroup& G = groups[g];
+	const DGroup G = dgroup(groups + (g));
 	const int chunk = blockIdx.x, wave = threadIdx.x >> 6;
 	if(chunk == 0 && threadIdx.x == 0 && G.nOffsets > 0) {
 		const int code = load_code(G.codes, G.codeWidth, 0);
