@@ -74,15 +74,28 @@ __device__ __forceinline__ int rle_find(const int32_t* __restrict__ runStart, in
 	return lo;
 }
 
+// Inclusive prefix sum over the 64 lanes of a wave (all lanes active) on the data-parallel
+// primitives: shifts inside each row of 16 lanes, then the row totals broadcast to the rows
+// behind (lane 15 of every row into rows 1 and 3, lane 31 into rows 2 and 3).
+__device__ __forceinline__ int wave_scan_incl(int v) {
+	v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, false); // row_shr:1
+	v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, false); // row_shr:2
+	v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, false); // row_shr:4
+	v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, false); // row_shr:8
+	v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false); // row_bcast:15
+	v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false); // row_bcast:31
+	return v;
+}
+
 // One wave decodes 256 consecutive delta entries of an offset list starting at
 // entry i0 from iterator state (row, emit). Lane l owns entries i0+4l .. i0+4l+3.
 // A 0 entry advances the row by maxV without emitting (OffsetByte / OffsetChar
-// semantics). On return rows[k] / didx[k] hold the absolute row and the data
+// semantics); `deltas` may be a window of the list that starts at entry winBase. On return rows[k] / didx[k] hold the absolute row and the data
 // index of entry k when bit k of `mask` is set, and (row, emit) is the state
 // behind the 256 entries.
 template <int W>
 __device__ __forceinline__ void sdc_decode256(const void* __restrict__ deltas, int64_t nDeltas, int64_t i0,
-	int32_t& row, int32_t& emit, int32_t rows[4], int32_t didx[4], unsigned& mask) {
+	int32_t& row, int32_t& emit, int32_t rows[4], int32_t didx[4], unsigned& mask, int64_t winBase = 0) {
 	const int lane = threadIdx.x & (WAVE - 1);
 	const int maxV = W == 1 ? 255 : 65535;
 	const int64_t i = i0 + (int64_t) lane * 4;
@@ -91,24 +104,18 @@ __device__ __forceinline__ void sdc_decode256(const void* __restrict__ deltas, i
 #pragma unroll
 	for(int k = 0; k < 4; k++) {
 		int v = -1;
-		if(i + k < nDeltas) v = W == 1 ? (int) ((const uint8_t*) deltas)[i + k] : (int) ((const uint16_t*) deltas)[i + k];
+		if(i + k < nDeltas) v = W == 1 ? (int) ((const uint8_t*) deltas)[i + k - winBase] : (int) ((const uint16_t*) deltas)[i + k - winBase];
 		s += v < 0 ? 0 : (v == 0 ? maxV : v);
 		rows[k] = s;
 		didx[k] = c;
 		if(v > 0) { mask |= 1u << k; c++; }
 	}
-	int ps = s, pc = c;
-#pragma unroll
-	for(int d = 1; d < WAVE; d <<= 1) {
-		const int t = __shfl_up(ps, d, WAVE);
-		const int u = __shfl_up(pc, d, WAVE);
-		if(lane >= d) { ps += t; pc += u; }
-	}
+	const int ps = wave_scan_incl(s), pc = wave_scan_incl(c);
 	const int exs = ps - s, exc = pc - c;
 #pragma unroll
 	for(int k = 0; k < 4; k++) { rows[k] += row + exs; didx[k] += emit + exc; }
-	row += __shfl(ps, WAVE - 1, WAVE);
-	emit += __shfl(pc, WAVE - 1, WAVE);
+	row += __builtin_amdgcn_readlane(ps, WAVE - 1);
+	emit += __builtin_amdgcn_readlane(pc, WAVE - 1);
 }
 
 // BYTES bytes of a code stream in registers, requested as non-temporal 8/16-byte loads.

@@ -8,7 +8,7 @@
 // carried from tile to tile). The waves then look decoded values up (code tile ->
 // dictionary copy in LDS, or the dense tile) straight into v_mfma_f64_16x16x4_f64 operands:
 //   X %*% B:    A operand = 16 rows x 4 decoded columns, B operand = 4 rows of B (padded to
-//               16 outputs); 64 output rows per wave and pass, staged per wave in LDS and
+//               16 outputs); 64 (or 32) output rows per wave and pass, staged per wave in LDS and
 //               written with full-line stores.
 //   t(X) %*% X: lane l holds column 16 cb + l % 16 of row l / 16, which is both operands; the
 //               NB (NB + 1) / 2 upper 16 x 16 tiles of the Gram matrix stay in registers until
@@ -27,6 +27,8 @@ constexpr int DEC_TILE = SDC_TILE;     // rows per tile = granularity of the off
 constexpr int DEC_WROWS = DEC_TILE / DEC_WAVES; // rows of a tile one wave multiplies
 constexpr int DEC_QMAX = 16;
 constexpr int DEC_PF = 4;              // 16-byte chunks a thread holds for the next tile
+constexpr int DEC_WIN = 2048;           // bytes of an offset list / of its codes kept in LDS per SDC group
+constexpr int DEC_TWIN = 32;            // tile index entries kept in LDS per SDC group
 constexpr int DEC_SLOT_PAD = 80;       // bytes between code tiles: spreads the columns a wave reads together over the LDS banks
 
 struct DecGroup {
@@ -37,7 +39,7 @@ struct DecGroup {
 	int32_t slotW;     // 1 or 2 bytes per code in the tile; all ones = row has no value
 	int32_t kOff;      // first decoded column of the group (row of the LDS copy of B)
 	int32_t copyIdx;   // tile filled by the chunk copy list (index), else -1
-	int32_t pad;
+	int32_t pad;       // bytes from the LDS base: run window (RLE) / list windows (SDCZeros) of a wave task
 };
 
 // Chunk copy list: what is a plain copy of consecutive global bytes per tile (DDC codes
@@ -111,7 +113,29 @@ struct DecLook {
 	}
 };
 
-template <int GRAM, int NB>
+// 64 runs from run wb of an RLE group into its LDS window (starts | ends | codes)
+__device__ __forceinline__ void dec_load_runs(int32_t* win, const DGroup& G, int wb, int lane) {
+	const int jj = wb + lane;
+	const bool inTable = jj < G.nRuns;
+	win[lane] = inTable ? G.runStart[jj] : 0x7fffffff;
+	win[64 + lane] = inTable ? G.runStart[jj + 1] : 0x7fffffff;
+	win[128 + lane] = inTable ? G.runCode[jj] : -1;
+}
+
+// DEC_WIN bytes of a stream from byte offset off (multiple of 16) into an LDS window; bytes
+// at and beyond `total` are not read.
+__device__ __forceinline__ void dec_load_window(uint8_t* win, const uint8_t* src, int64_t off, int64_t total, int lane) {
+#pragma unroll
+	for(int p = 0; p < DEC_WIN / 1024; p++) {
+		const int o = (p * 64 + lane) * 16;
+		if(off + o + 16 <= total) *(u32x4*) (win + o) = *(const u32x4*) (src + off + o);
+		else
+			for(int e = 0; e < 16; e++)
+				if(off + o + e < total) win[o + e] = src[off + o + e];
+	}
+}
+
+template <int GRAM, int NB, int RPL>
 __device__ __forceinline__ void decode_body(const DecArgs& A) {
 	extern __shared__ __align__(16) double smem[];
 	double* Bs = smem + A.valDoubles;                              // bDoubles: rows of B in decoded column order, 16 outputs each
@@ -163,6 +187,16 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 			}
 	}
 
+	// wave task windows: first 64 runs from the run cursor; list windows start empty
+	for(int g = wave; g < nGroups; g += DEC_WAVES) {
+		const DecGroup P = planS[g];
+		if(P.slotOff < 0 || P.copyIdx >= 0) continue;
+		if(P.type == G_RLE) dec_load_runs((int32_t*) ((uint8_t*) smem + P.pad), dgroup(groupS + g), runBase[g], lane);
+		else if(P.type == G_SDCZ && lane < 3)
+			((int32_t*) ((uint8_t*) smem + P.pad + DEC_TWIN * sizeof(OffState) + 2 * DEC_WIN))[lane] = -(1 << 30);
+	}
+	dec_wave_sync();
+
 	// Copy list chunks of one tile, flattened: chunk i of a thread is tid + k * DEC_THREADS,
 	// so its entry and place in the tile never change. Whole chunks are loaded as 16 bytes
 	// one tile ahead; the ragged end of the last tile is copied byte-wise.
@@ -212,7 +246,7 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 	}
 	const int q = A.q;
 	const double cinit = (!GRAM && A.constRow != nullptr && i16 < q) ? A.constRow[i16] : 0.0;
-	double* const wstage = stage + (size_t) wave * 64 * (GRAM ? 0 : q);
+	double* const wstage = stage + (size_t) wave * 16 * RPL * (GRAM ? 0 : q);
 	const int KB = A.nColD >> 2;
 
 	int cnt = 0;
@@ -248,34 +282,36 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 					if(t0 + i < nRows) dec_store_code(slot, w, i, load_code(G.codes, G.codeWidth, t0 + i));
 			}
 			else if(P.type == G_RLE) {
-				int j = runBase[g];
+				// window of 64 runs in LDS, reloaded when it no longer reaches the end of the tile
+				int32_t* win = (int32_t*) (ldsBytes + P.pad);
+				int wb = runBase[g];
 				while(true) {
-					const int jj = j + lane;
-					const bool inTable = jj < G.nRuns;
-					const int32_t s = inTable ? G.runStart[jj] : 0x7fffffff;
-					const int32_t e = inTable ? G.runStart[jj + 1] : 0x7fffffff;
-					const int32_t code = inTable ? G.runCode[jj] : -1;
-					const unsigned long long valid = __ballot(inTable && s < rEnd);
-					const int nv = __popcll(valid);
-					if(nv <= 8) { // long runs: all lanes write each run
-						for(int k = 0; k < nv; k++) {
+					const bool inTable = wb + lane < G.nRuns;
+					const int32_t s = win[lane], e = win[64 + lane], code = win[128 + lane];
+					const bool ov = inTable && s < rEnd && e > t0;
+					unsigned long long valid = __ballot(ov);
+					if(__popcll(valid) <= 8) { // long runs: all lanes write each run
+						while(valid) {
+							const int k = __ffsll((long long) valid) - 1;
+							valid &= valid - 1;
 							const int sk = max((int) (__shfl(s, k, 64) - t0), 0);
 							const int ek = (int) (min((int64_t) __shfl(e, k, 64), rEnd) - t0);
 							const int ck = __shfl(code, k, 64);
 							for(int i = sk + lane; i < ek; i += 64) dec_store_code(slot, w, i, ck);
 						}
 					}
-					else if(inTable && s < rEnd) { // short runs: one run per lane
+					else if(ov) { // short runs: one run per lane
 						const int sk = max((int) (s - t0), 0);
 						const int ek = (int) (min((int64_t) e, rEnd) - t0);
 						for(int i = sk; i < ek; i++) dec_store_code(slot, w, i, code);
 					}
-					if(nv < 64) { j += max(nv - 1, 0); break; }      // base: last run starting before the tile end
-					if(__shfl(e, 63, 64) >= rEnd) { j += 63; break; }
-					j += 64;
+					if(__ballot(inTable && e >= rEnd) != 0 || wb + 64 >= G.nRuns) break;
+					wb += 64;
+					dec_wave_sync();
+					dec_load_runs(win, G, wb, lane);
+					dec_wave_sync();
 				}
-				j = min(j, G.nRuns - 1);
-				if(lane == 0) runBase[g] = j;
+				if(lane == 0) runBase[g] = wb;
 			}
 			else { // SDCZeros: rows without an entry hold the no-value code
 				for(int i = lane; i < DEC_TILE; i += 64) dec_store_code(slot, w, i, 0xffff);
@@ -283,20 +319,48 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 				// same-wave LDS writes are ordered, no barrier needed between fill and scatter
 				if(lane == 0 && G.first >= t0 && G.first < rEnd) dec_store_code(slot, w, (int) (G.first - t0), load_code(G.codes, G.codeWidth, 0));
 				if(tile < G.nTiles) {
-					const OffState st = G.tileIdx[tile];
+					// windows of the tile index, the delta list and the codes in LDS: a refill every few
+					// tiles instead of three dependent global loads per tile
+					uint8_t* wbase = ldsBytes + P.pad;
+					OffState* tw = (OffState*) wbase;
+					uint8_t* dwin = wbase + DEC_TWIN * sizeof(OffState);
+					uint8_t* cwin = dwin + DEC_WIN;
+					int32_t* wst = (int32_t*) (cwin + DEC_WIN); // dBase, cBase, tBase
+					int dBase = wst[0], cBase = wst[1], tBase = wst[2];
+					if(tile < tBase || tile >= tBase + DEC_TWIN) {
+						tBase = tile;
+						dec_wave_sync();
+						if(lane < DEC_TWIN) tw[lane] = G.tileIdx[min(tile + lane, G.nTiles - 1)];
+						dec_wave_sync();
+					}
+					const OffState st = tw[tile - tBase];
 					int32_t row = st.row, emit = st.emit;
 					int64_t i0 = st.idx;
+					const int dN = DEC_WIN / G.deltaWidth, cN = DEC_WIN / G.codeWidth;
 					while(i0 < G.nDeltas && row < rEnd) {
+						if(i0 < dBase || i0 + 256 > dBase + dN) {
+							dBase = (int) (i0 & ~(int64_t) 15);
+							dec_wave_sync();
+							dec_load_window(dwin, (const uint8_t*) G.deltas, (int64_t) dBase * G.deltaWidth, G.nDeltas * G.deltaWidth, lane);
+							dec_wave_sync();
+						}
+						if(emit < cBase || emit + 256 > cBase + cN) {
+							cBase = emit & ~15;
+							dec_wave_sync();
+							dec_load_window(cwin, (const uint8_t*) G.codes, (int64_t) cBase * G.codeWidth, G.nOffsets * G.codeWidth, lane);
+							dec_wave_sync();
+						}
 						int32_t rows[4], didx[4];
 						unsigned mask;
-						if(G.deltaWidth == 1) sdc_decode256<1>(G.deltas, G.nDeltas, i0, row, emit, rows, didx, mask);
-						else sdc_decode256<2>(G.deltas, G.nDeltas, i0, row, emit, rows, didx, mask);
+						if(G.deltaWidth == 1) sdc_decode256<1>(dwin, G.nDeltas, i0, row, emit, rows, didx, mask, dBase);
+						else sdc_decode256<2>(dwin, G.nDeltas, i0, row, emit, rows, didx, mask, dBase);
 #pragma unroll
 						for(int k = 0; k < 4; k++)
 							if((mask & (1u << k)) && rows[k] < rEnd)
-								dec_store_code(slot, w, (int) (rows[k] - t0), load_code(G.codes, G.codeWidth, didx[k]));
+								dec_store_code(slot, w, (int) (rows[k] - t0), load_code(cwin, G.codeWidth, didx[k] - cBase));
 						i0 += 256;
 					}
+					if(lane == 0) { wst[0] = dBase; wst[1] = cBase; wst[2] = tBase; }
 				}
 			}
 		}
@@ -359,49 +423,52 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 			continue;
 		}
 
-		// ---- X %*% B: wave = 128 rows in two passes of 64; lane (k4, i16): rows i16 * 4 .. + 3 of
+		// ---- X %*% B: wave = 128 rows in passes of 16 * RPL; lane (k4, i16): rows i16 * RPL .. of
 		// the pass as the A operand of decoded column 4 kb + k4, B[4 kb + k4, i16] as the B operand
+		constexpr int PROWS = 16 * RPL;
 #pragma unroll 1
-		for(int half = 0; half < 2; half++) {
-			const int pbase = wave * DEC_WROWS + half * 64;
-			const int rbase = pbase + i16 * 4;
-			f64x4 acc[4];
+		for(int pass = 0; pass < DEC_WROWS / PROWS; pass++) {
+			const int pbase = wave * DEC_WROWS + pass * PROWS;
+			const int rbase = pbase + i16 * RPL;
+			f64x4 acc[RPL];
 #pragma unroll
-			for(int s = 0; s < 4; s++) acc[s] = f64x4{cinit, cinit, cinit, cinit};
-			bool in[4];
+			for(int s = 0; s < RPL; s++) acc[s] = f64x4{cinit, cinit, cinit, cinit};
+			bool in[RPL];
 #pragma unroll
-			for(int s = 0; s < 4; s++) in[s] = t0 + rbase + s < nRows;
+			for(int s = 0; s < RPL; s++) in[s] = t0 + rbase + s < nRows;
 #pragma unroll 2
 			for(int kb = 0; kb < KB; kb++) {
 				const DecCol D = colS[kb * 4 + k4];
 				const double bop = Bs[(kb * 4 + k4) * 16 + i16];
 				const DecLook L(D);
-				const uint32_t* cp = (const uint32_t*) (slots + (L.coded ? D.slotOff + rbase * (L.two ? 2 : 1) : 0));
-				const uint32_t lo = cp[0], hi = cp[1];
-				double x[4];
+				// RPL codes of the column's tile as 16-bit pieces (aligned for either code width)
+				const uint16_t* cp = (const uint16_t*) (slots + (L.coded ? D.slotOff + rbase * (L.two ? 2 : 1) : 0));
+				uint32_t piece[RPL];
 #pragma unroll
-				for(int s = 0; s < 4; s++) {
-					const int c1 = (int) ((lo >> (8 * s)) & 0xff);
-					const int c2 = (int) (((s < 2 ? lo : hi) >> (16 * (s & 1))) & 0xffff);
+				for(int s = 0; s < RPL; s++) piece[s] = cp[s];
+				double x[RPL];
+#pragma unroll
+				for(int s = 0; s < RPL; s++) {
+					const int c1 = (int) ((piece[s >> 1] >> (8 * (s & 1))) & 0xff);
 					bool valid;
-					const int ad = L.addr(L.two ? c2 : c1, rbase + s, valid);
+					const int ad = L.addr(L.two ? (int) piece[s] : c1, rbase + s, valid);
 					const double v = smem[ad];
 					x[s] = (valid & in[s]) ? v : 0.0;
 				}
 #pragma unroll
-				for(int s = 0; s < 4; s++) acc[s] = __builtin_amdgcn_mfma_f64_16x16x4f64(x[s], bop, acc[s], 0, 0, 0);
+				for(int s = 0; s < RPL; s++) acc[s] = __builtin_amdgcn_mfma_f64_16x16x4f64(x[s], bop, acc[s], 0, 0, 0);
 			}
 			// accumulator register v of lane l: output row 4 v + l / 16 of the step, output column l % 16
 			dec_wave_sync(); // the previous pass's readers of the staging area are done
 			if(i16 < q) {
 #pragma unroll
-				for(int s = 0; s < 4; s++)
+				for(int s = 0; s < RPL; s++)
 #pragma unroll
-					for(int v = 0; v < 4; v++) wstage[((4 * v + k4) * 4 + s) * q + i16] = acc[s][v];
+					for(int v = 0; v < 4; v++) wstage[((4 * v + k4) * RPL + s) * q + i16] = acc[s][v];
 			}
 			dec_wave_sync();
 			const int64_t rowBase = t0 + pbase;
-			const int nr = (int) max((int64_t) 0, min((int64_t) 64, nRows - rowBase));
+			const int nr = (int) max((int64_t) 0, min((int64_t) PROWS, nRows - rowBase));
 			for(int i = lane; i < nr * q; i += 64) {
 				const double v = wstage[i];
 				cnt += v != 0.0;
@@ -434,10 +501,11 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 	count_add(A.nnz, cnt);
 }
 
-__global__ __launch_bounds__(DEC_THREADS) void k_rmm_decode(const DecArgs A) { decode_body<0, 1>(A); }
+template <int RPL>
+__global__ __launch_bounds__(DEC_THREADS) void k_rmm_decode(const DecArgs A) { decode_body<0, 1, RPL>(A); }
 
 template <int NB>
-__global__ __launch_bounds__(DEC_THREADS) void k_tsmm_decode(const DecArgs A) { decode_body<1, NB>(A); }
+__global__ __launch_bounds__(DEC_THREADS) void k_tsmm_decode(const DecArgs A) { decode_body<1, NB, 4>(A); }
 
 // Host side of both kernels: LDS plan, copy list and column descriptors in the block's
 // scratch buffer. Returns 1 when the block does not fit (the caller uses another path).
@@ -447,7 +515,7 @@ struct DecLaunch {
 	unsigned grid = 0;
 };
 
-static int dec_prepare(cla_block* b, bool gram, int q, DecLaunch& L) {
+static int dec_prepare(cla_block* b, bool gram, int q, int rpl, DecLaunch& L) {
 	const int nG = (int) b->groups.size();
 	const int nCols = b->nCols;
 	std::vector<DecGroup> plan((size_t) nG);
@@ -478,7 +546,7 @@ static int dec_prepare(cla_block* b, bool gram, int q, DecLaunch& L) {
 	slotB = (slotB + 16 + 15) & ~(size_t) 15; // the multiply phase may read 16 bytes past the last tile
 	const int nColD = gram ? ((nCols + 15) / 16) * 16 : ((K + 3) / 4) * 4;
 	const size_t bD = gram ? 0 : (size_t) nColD * 16;
-	const size_t stageD = gram ? (size_t) nColD * nColD : (size_t) DEC_WAVES * 64 * q;
+	const size_t stageD = gram ? (size_t) nColD * nColD : (size_t) DEC_WAVES * 16 * rpl * q;
 	const size_t slotBase = (valD + bD + stageD) * 8;
 	// copy list
 	std::vector<DecCopy> copies;
@@ -501,8 +569,16 @@ static int dec_prepare(cla_block* b, bool gram, int q, DecLaunch& L) {
 		copies.push_back(C);
 		nChunks += DEC_TILE * C.bpr / 16;
 	}
-	L.lds = slotBase + slotB + (size_t) nColD * (sizeof(DecCol) + (gram ? 8 : 0)) + (size_t) nG * (sizeof(DecGroup) + sizeof(DGroup) + 4) +
-		copies.size() * sizeof(DecCopy) + 64;
+	size_t ldsEnd = slotBase + slotB + (size_t) nColD * (sizeof(DecCol) + (gram ? 8 : 0)) +
+		(size_t) nG * (sizeof(DecGroup) + sizeof(DGroup) + 4) + copies.size() * sizeof(DecCopy);
+	ldsEnd = (ldsEnd + 15) & ~(size_t) 15;
+	for(int g = 0; g < nG; g++) { // windows of the wave tasks
+		DecGroup& P = plan[g];
+		if(P.slotOff < 0 || P.copyIdx >= 0) continue;
+		if(P.type == G_RLE) { P.pad = (int32_t) ldsEnd; ldsEnd += 3 * 64 * 4; }
+		else if(P.type == G_SDCZ) { P.pad = (int32_t) ldsEnd; ldsEnd += DEC_TWIN * sizeof(OffState) + 2 * DEC_WIN + 16; }
+	}
+	L.lds = ldsEnd + 64;
 	if(L.lds > (size_t) std::min(g_ldsPerBlock, 160 * 1024) - 1024) return 1;
 	// column descriptors: decoded column order (X %*% B) or matrix column order (t(X) %*% X)
 	std::vector<DecCol> cols((size_t) nColD, DecCol{0, 0, 0, 0});
@@ -555,13 +631,21 @@ int launch_rmm_decode(cla_block* b, const double* dB, int q, const double* dCons
 	unsigned long long* dNnz) {
 	if(b->groups.empty() || b->nRows == 0 || q < 2 || q > DEC_QMAX) return 1;
 	DecLaunch L;
-	int rc = dec_prepare(b, false, q, L);
+	int rpl = 4; // rows per lane and pass: the smaller output staging area when LDS is short
+	int rc = dec_prepare(b, false, q, rpl, L);
+	if(rc == 1) rc = dec_prepare(b, false, q, rpl = 2, L);
 	if(rc) return rc;
 	L.A.B = dB; L.A.constRow = dConstRow; L.A.out = dOut; L.A.nnz = dNnz;
 	double algo = (double) b->device_bytes_cached + (double) b->nRows * q * 8;
 	Prof pf(b, "k_rmm_decode", L.grid, DEC_THREADS, (long) L.lds, algo);
-	CLA_HIP(hipFuncSetAttribute((const void*) k_rmm_decode, hipFuncAttributeMaxDynamicSharedMemorySize, (int) L.lds));
-	hipLaunchKernelGGL(k_rmm_decode, dim3(L.grid), dim3(DEC_THREADS), L.lds, b->stream, L.A);
+	if(rpl == 4) {
+		CLA_HIP(hipFuncSetAttribute((const void*) k_rmm_decode<4>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) L.lds));
+		hipLaunchKernelGGL(k_rmm_decode<4>, dim3(L.grid), dim3(DEC_THREADS), L.lds, b->stream, L.A);
+	}
+	else {
+		CLA_HIP(hipFuncSetAttribute((const void*) k_rmm_decode<2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) L.lds));
+		hipLaunchKernelGGL(k_rmm_decode<2>, dim3(L.grid), dim3(DEC_THREADS), L.lds, b->stream, L.A);
+	}
 	CLA_HIP(hipGetLastError());
 	return 0;
 }
@@ -573,7 +657,7 @@ int launch_tsmm_decode(cla_block* b, double* dOut) {
 	if(b->groups.empty() || b->nRows == 0 || nCols > 64) return 1;
 	const int NB = (nCols + 15) / 16;
 	DecLaunch L;
-	int rc = dec_prepare(b, true, 0, L);
+	int rc = dec_prepare(b, true, 0, 4, L);
 	if(rc) return rc;
 	L.A.out = dOut;
 	Prof pf(b, "k_tsmm_decode", L.grid, DEC_THREADS, (long) L.lds, (double) b->device_bytes_cached);
