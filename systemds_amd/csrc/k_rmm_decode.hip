@@ -65,6 +65,8 @@ struct DecArgs {
 	const DecGroup* plan;
 	const DecCopy* copies;
 	const DecCol* cols;
+	const int32_t* tasks;              // wave tasks: DEC_WAVES + 1 list offsets, then group ids per wave
+	int nTasks;
 	const double* colConst;            // t(X) %*% X: constant part per (padded) column
 	int nGroups, nCopies, nChunks;     // nChunks: 16-byte chunks per tile over the copy list
 	int nColD;                         // entries of cols (multiple of 4 / of 16)
@@ -147,6 +149,7 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 	DecCopy* copyS = (DecCopy*) (planS + A.nGroups);               // nCopies
 	DGroup* groupS = (DGroup*) (copyS + A.nCopies);                // nGroups: descriptors, so that a wave task starts from LDS
 	int32_t* runBase = (int32_t*) (groupS + A.nGroups);            // nGroups
+	int32_t* taskS = runBase + A.nGroups;                          // DEC_WAVES + 1 + nTasks
 	const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
 	const int i16 = lane & 15, k4 = lane >> 4;
 	const DGroup* __restrict__ groups = A.groups;
@@ -165,6 +168,7 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 		runBase[g] = groups[g].type == G_RLE ? rle_find(as_global(groups[g].runStart), groups[g].nRuns, (int32_t) ((int64_t) tileBeg * DEC_TILE)) : 0;
 	}
 	for(int i = tid; i < A.nCopies; i += DEC_THREADS) copyS[i] = A.copies[i];
+	for(int i = tid; i < DEC_WAVES + 1 + A.nTasks; i += DEC_THREADS) taskS[i] = A.tasks[i];
 	for(int i = tid; i < A.nColD; i += DEC_THREADS) {
 		colS[i] = A.cols[i];
 		if(GRAM) constS[i] = A.colConst[i];
@@ -188,9 +192,9 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 	}
 
 	// wave task windows: first 64 runs from the run cursor; list windows start empty
-	for(int g = wave; g < nGroups; g += DEC_WAVES) {
+	for(int t = taskS[wave]; t < taskS[wave + 1]; t++) {
+		const int g = taskS[DEC_WAVES + 1 + t];
 		const DecGroup P = planS[g];
-		if(P.slotOff < 0 || P.copyIdx >= 0) continue;
 		if(P.type == G_RLE) dec_load_runs((int32_t*) ((uint8_t*) smem + P.pad), dgroup(groupS + g), runBase[g], lane);
 		else if(P.type == G_SDCZ && lane < 3)
 			((int32_t*) ((uint8_t*) smem + P.pad + DEC_TWIN * sizeof(OffState) + 2 * DEC_WIN))[lane] = -(1 << 30);
@@ -270,10 +274,10 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 			else copy_ragged(src + t0 * bpr, dstOff, tb - off);
 		}
 
-		// ---- other dictionary coded groups, one wave per group
-		for(int g = wave; g < nGroups; g += DEC_THREADS / 64) {
+		// ---- other dictionary coded groups: the wave's share of the task list, one group at a time
+		for(int t = taskS[wave]; t < taskS[wave + 1]; t++) {
+			const int g = taskS[DEC_WAVES + 1 + t];
 			const DecGroup P = planS[g];
-			if(P.slotOff < 0 || P.copyIdx >= 0) continue;
 			const DGroup G = dgroup(groupS + g);
 			uint8_t* slot = slots + P.slotOff;
 			const int w = P.slotW;
@@ -569,8 +573,32 @@ static int dec_prepare(cla_block* b, bool gram, int q, int rpl, DecLaunch& L) {
 		copies.push_back(C);
 		nChunks += DEC_TILE * C.bpr / 16;
 	}
+	// wave tasks (groups whose tile needs decoding), longest first onto the least loaded wave
+	std::vector<std::pair<int, int>> taskCost; // (cost, group)
+	for(int g = 0; g < nG; g++) {
+		const DecGroup& P = plan[g];
+		if(P.slotOff < 0 || P.copyIdx >= 0) continue;
+		taskCost.push_back({P.type == G_DDC ? 3 : P.type == G_SDCZ ? 2 : 1, g});
+	}
+	std::stable_sort(taskCost.begin(), taskCost.end(), [](const std::pair<int, int>& a, const std::pair<int, int>& c) { return a.first > c.first; });
+	std::vector<std::vector<int>> waveTasks(DEC_WAVES);
+	{
+		int load[DEC_WAVES] = {0};
+		for(auto& tc : taskCost) {
+			int best = 0;
+			for(int w = 1; w < DEC_WAVES; w++)
+				if(load[w] < load[best]) best = w;
+			load[best] += tc.first;
+			waveTasks[best].push_back(tc.second);
+		}
+	}
+	std::vector<int32_t> tasks(DEC_WAVES + 1, 0);
+	for(int w = 0; w < DEC_WAVES; w++) {
+		tasks[w + 1] = tasks[w] + (int32_t) waveTasks[w].size();
+		for(int g : waveTasks[w]) tasks.push_back(g);
+	}
 	size_t ldsEnd = slotBase + slotB + (size_t) nColD * (sizeof(DecCol) + (gram ? 8 : 0)) +
-		(size_t) nG * (sizeof(DecGroup) + sizeof(DGroup) + 4) + copies.size() * sizeof(DecCopy);
+		(size_t) nG * (sizeof(DecGroup) + sizeof(DGroup) + 4) + copies.size() * sizeof(DecCopy) + tasks.size() * 4;
 	ldsEnd = (ldsEnd + 15) & ~(size_t) 15;
 	for(int g = 0; g < nG; g++) { // windows of the wave tasks
 		DecGroup& P = plan[g];
@@ -601,11 +629,13 @@ static int dec_prepare(cla_block* b, bool gram, int q, int rpl, DecLaunch& L) {
 	}
 	const size_t planBytes = plan.size() * sizeof(DecGroup), copyBytes = copies.size() * sizeof(DecCopy);
 	const size_t colBytes = cols.size() * sizeof(DecCol), constBytes = colConst.size() * 8;
-	std::vector<uint8_t> img(planBytes + copyBytes + colBytes + constBytes);
+	const size_t taskBytes = tasks.size() * 4;
+	std::vector<uint8_t> img(planBytes + copyBytes + colBytes + constBytes + taskBytes);
 	std::memcpy(img.data(), copies.data(), copyBytes); // pointers first: 8-byte aligned
 	std::memcpy(img.data() + copyBytes, colConst.data(), constBytes);
 	std::memcpy(img.data() + copyBytes + constBytes, cols.data(), colBytes);
 	std::memcpy(img.data() + copyBytes + constBytes + colBytes, plan.data(), planBytes);
+	std::memcpy(img.data() + copyBytes + constBytes + colBytes + planBytes, tasks.data(), taskBytes);
 	int rc = ensure_scratch(b, img.size() + 64);
 	if(rc) return rc;
 	uint8_t* d = (uint8_t*) b->dScratch;
@@ -617,6 +647,8 @@ static int dec_prepare(cla_block* b, bool gram, int q, int rpl, DecLaunch& L) {
 	A.colConst = (const double*) (d + copyBytes);
 	A.cols = (const DecCol*) (d + copyBytes + constBytes);
 	A.plan = (const DecGroup*) (d + copyBytes + constBytes + colBytes);
+	A.tasks = (const int32_t*) (d + copyBytes + constBytes + colBytes + planBytes);
+	A.nTasks = (int) taskCost.size();
 	A.nGroups = nG; A.nCopies = (int) copies.size(); A.nChunks = nChunks; A.nColD = nColD;
 	A.valDoubles = (int) valD; A.bDoubles = (int) bD; A.stageDoubles = (int) stageD; A.slotBytes = (int) slotB;
 	A.B = nullptr; A.q = q; A.constRow = nullptr; A.out = nullptr; A.nRows = b->nRows; A.nnz = nullptr; A.nCols = nCols;
