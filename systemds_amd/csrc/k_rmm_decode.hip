@@ -56,8 +56,8 @@ struct DecCopy {
 struct DecCol {
 	int32_t slotOff;   // dictionary coded: code tile (bytes into the code tiles)
 	int32_t valOff;    // doubles from the LDS base: dictionary copy / dense tile
-	int32_t meta;      // kind (0 none or constant only, 1 dictionary coded, 2 dense) | two-byte codes << 2 | nC << 4 | h << 18
-	int32_t pad;
+	int32_t meta;      // kind (0 none or constant only, 1 dictionary coded, 2 dense) | two-byte codes << 2 | dictionary in global memory << 3 | nC << 4 | h << 18
+	int32_t pad;       // group
 };
 
 struct DecArgs {
@@ -107,9 +107,10 @@ struct DecLook {
 		base = D.valOff + (int) ((unsigned) D.meta >> 18);
 		sent = coded ? (two ? 0xffff : 0xff) : -1;
 	}
-	// LDS index (doubles) of the value at tile row rt with code c, and whether the row has one
-	__device__ __forceinline__ int addr(int c, int rt, bool& valid) const {
-		valid = dense | (coded & (c != sent));
+	// LDS index (doubles) of the value at tile row rt with code c, and whether the row has one.
+	// Rows behind the end of the matrix (in == false) hold stale codes: never used as an index.
+	__device__ __forceinline__ int addr(int c, int rt, bool in, bool& valid) const {
+		valid = in & (dense | (coded & (c != sent)));
 		const int a = base + (coded ? c : rt) * nC;
 		return valid ? a : 0;
 	}
@@ -137,7 +138,9 @@ __device__ __forceinline__ void dec_load_window(uint8_t* win, const uint8_t* src
 	}
 }
 
-template <int GRAM, int NB, int RPL>
+// FLAT: dictionaries that do not fit LDS stay in global memory; the lookups then go through
+// generic pointers (LDS or global per lane).
+template <int GRAM, int NB, int RPL, int FLAT>
 __device__ __forceinline__ void decode_body(const DecArgs& A) {
 	extern __shared__ __align__(16) double smem[];
 	double* Bs = smem + A.valDoubles;                              // bDoubles: rows of B in decoded column order, 16 outputs each
@@ -180,7 +183,7 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 	for(int g = 0; g < nGroups; g++) {
 		const DecGroup P = planS[g];
 		const DGroup G = dgroup(groups + (g));
-		if(P.slotOff >= 0) {
+		if(P.slotOff >= 0 && P.dictOff >= 0) {
 			const int n = G.nVals * G.nColG;
 			for(int i = tid; i < n; i += DEC_THREADS) smem[P.dictOff + i] = G.dict[i];
 		}
@@ -382,10 +385,16 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 				u32x4 cq[NB][2];
 				int lbase[NB], lnC[NB], lsent[NB];
 				bool lcoded[NB], ldense[NB], ltwo[NB];
+				const double* lptr[FLAT ? NB : 1];
 #pragma unroll
 				for(int cb = 0; cb < NB; cb++) {
 					const DecLook L(colS[cb * 16 + i16]);
 					lbase[cb] = L.base; lnC[cb] = L.nC; lsent[cb] = L.sent; lcoded[cb] = L.coded; ldense[cb] = L.dense; ltwo[cb] = L.two;
+					if(FLAT) {
+						const DecCol D = colS[cb * 16 + i16];
+						const double* gdict = groupS[D.pad].dict + ((unsigned) D.meta >> 18);
+						lptr[cb] = (D.meta & 8) ? gdict : (const double*) smem + L.base;
+					}
 					cst[cb] = constS[cb * 16 + i16];
 					const u32x4* cp = (const u32x4*) (slots + (L.coded ? colS[cb * 16 + i16].slotOff + rbase * (L.two ? 2 : 1) : 0));
 					cq[cb][0] = cp[0];
@@ -404,9 +413,17 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 							const int c1 = (int) ((cq[cb][0][s >> 2] >> (8 * (s & 3))) & 0xff);
 							const int c2 = (int) ((cq[cb][s >> 3][(s >> 1) & 3] >> (16 * (s & 1))) & 0xffff);
 							const int c = ltwo[cb] ? c2 : c1;
-							const bool valid = ldense[cb] | (lcoded[cb] & (c != lsent[cb]));
-							const int ad = lbase[cb] + (lcoded[cb] ? c : rbase + s) * lnC[cb];
-							const double v = smem[valid ? ad : 0];
+							// rows behind the end of the matrix hold stale codes: never used as an index
+							const bool valid = (t0 + rbase + s < nRows) & (ldense[cb] | (lcoded[cb] & (c != lsent[cb])));
+							double v;
+							if(FLAT) {
+								const double* vp = lptr[cb] + (lcoded[cb] ? c : rbase + s) * lnC[cb];
+								v = *(valid ? vp : (const double*) smem);
+							}
+							else {
+								const int ad = lbase[cb] + (lcoded[cb] ? c : rbase + s) * lnC[cb];
+								v = smem[valid ? ad : 0];
+							}
 							x[u][cb] = valid ? v : 0.0;
 						}
 					}
@@ -455,9 +472,9 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 				for(int s = 0; s < RPL; s++) {
 					const int c1 = (int) ((piece[s >> 1] >> (8 * (s & 1))) & 0xff);
 					bool valid;
-					const int ad = L.addr(L.two ? (int) piece[s] : c1, rbase + s, valid);
+					const int ad = L.addr(L.two ? (int) piece[s] : c1, rbase + s, in[s], valid);
 					const double v = smem[ad];
-					x[s] = (valid & in[s]) ? v : 0.0;
+					x[s] = valid ? v : 0.0;
 				}
 #pragma unroll
 				for(int s = 0; s < RPL; s++) acc[s] = __builtin_amdgcn_mfma_f64_16x16x4f64(x[s], bop, acc[s], 0, 0, 0);
@@ -506,10 +523,10 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 }
 
 template <int RPL>
-__global__ __launch_bounds__(DEC_THREADS) void k_rmm_decode(const DecArgs A) { decode_body<0, 1, RPL>(A); }
+__global__ __launch_bounds__(DEC_THREADS) void k_rmm_decode(const DecArgs A) { decode_body<0, 1, RPL, 0>(A); }
 
-template <int NB>
-__global__ __launch_bounds__(DEC_THREADS) void k_tsmm_decode(const DecArgs A) { decode_body<1, NB, 4>(A); }
+template <int NB, int FLAT>
+__global__ __launch_bounds__(DEC_THREADS) void k_tsmm_decode(const DecArgs A) { decode_body<1, NB, 4, FLAT>(A); }
 
 // Host side of both kernels: LDS plan, copy list and column descriptors in the block's
 // scratch buffer. Returns 1 when the block does not fit (the caller uses another path).
@@ -519,7 +536,8 @@ struct DecLaunch {
 	unsigned grid = 0;
 };
 
-static int dec_prepare(cla_block* b, bool gram, int q, int rpl, DecLaunch& L) {
+// Dictionaries of more than dictLimit doubles stay in global memory (t(X) %*% X only).
+static int dec_prepare(cla_block* b, bool gram, int q, int rpl, DecLaunch& L, size_t dictLimit = (size_t) 1 << 30) {
 	const int nG = (int) b->groups.size();
 	const int nCols = b->nCols;
 	std::vector<DecGroup> plan((size_t) nG);
@@ -539,8 +557,10 @@ static int dec_prepare(cla_block* b, bool gram, int q, int rpl, DecLaunch& L) {
 		}
 		if(G.type != G_DDC && G.type != G_RLE && !(G.type == G_SDCZ && G.nOffsets > 0)) continue; // no row data
 		if(G.nVals > 65535) return 1;
-		P.dictOff = (int32_t) valD;
-		valD += (size_t) G.nVals * G.nColG;
+		if((size_t) G.nVals * G.nColG <= dictLimit) {
+			P.dictOff = (int32_t) valD;
+			valD += (size_t) G.nVals * G.nColG;
+		}
 		P.slotW = G.nVals <= 255 ? 1 : 2;
 		P.slotOff = (int32_t) slotB;
 		slotB += (size_t) DEC_TILE * P.slotW + DEC_SLOT_PAD;
@@ -623,8 +643,9 @@ static int dec_prepare(cla_block* b, bool gram, int q, int rpl, DecLaunch& L) {
 			DecCol& C = cols[gram ? hc[h] : P.kOff + h];
 			const int kind = P.type == G_UNC ? 2 : P.slotOff >= 0 ? 1 : 0;
 			C.slotOff = kind == 1 ? P.slotOff : 0;
-			C.valOff = kind ? P.dictOff : 0;
-			C.meta = (int32_t) ((uint32_t) kind | (P.slotW == 2 ? 4u : 0u) | ((uint32_t) P.nC << 4) | ((uint32_t) h << 18));
+			C.valOff = kind && P.dictOff >= 0 ? P.dictOff : 0;
+			C.pad = g;
+			C.meta = (int32_t) ((uint32_t) kind | (P.slotW == 2 ? 4u : 0u) | (kind == 1 && P.dictOff < 0 ? 8u : 0u) | ((uint32_t) P.nC << 4) | ((uint32_t) h << 18));
 		}
 	}
 	const size_t planBytes = plan.size() * sizeof(DecGroup), copyBytes = copies.size() * sizeof(DecCopy);
@@ -689,19 +710,32 @@ int launch_tsmm_decode(cla_block* b, double* dOut) {
 	if(b->groups.empty() || b->nRows == 0 || nCols > 64) return 1;
 	const int NB = (nCols + 15) / 16;
 	DecLaunch L;
+	bool flat = false;
 	int rc = dec_prepare(b, true, 0, 4, L);
+	if(rc == 1) { // large dictionaries stay in global memory
+		flat = true;
+		rc = dec_prepare(b, true, 0, 4, L, 512);
+	}
 	if(rc) return rc;
 	L.A.out = dOut;
 	Prof pf(b, "k_tsmm_decode", L.grid, DEC_THREADS, (long) L.lds, (double) b->device_bytes_cached);
-#define GRAM_LAUNCH(NBV)                                                                                        \
+#define GRAM_LAUNCH(NBV, FL)                                                                                    \
 	do {                                                                                                        \
-		CLA_HIP(hipFuncSetAttribute((const void*) k_tsmm_decode<NBV>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) L.lds)); \
-		hipLaunchKernelGGL(k_tsmm_decode<NBV>, dim3(L.grid), dim3(DEC_THREADS), L.lds, b->stream, L.A);         \
+		CLA_HIP(hipFuncSetAttribute((const void*) k_tsmm_decode<NBV, FL>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) L.lds)); \
+		hipLaunchKernelGGL((k_tsmm_decode<NBV, FL>), dim3(L.grid), dim3(DEC_THREADS), L.lds, b->stream, L.A);   \
 	} while(0)
-	if(NB == 1) GRAM_LAUNCH(1);
-	else if(NB == 2) GRAM_LAUNCH(2);
-	else if(NB == 3) GRAM_LAUNCH(3);
-	else GRAM_LAUNCH(4);
+	if(!flat) {
+		if(NB == 1) GRAM_LAUNCH(1, 0);
+		else if(NB == 2) GRAM_LAUNCH(2, 0);
+		else if(NB == 3) GRAM_LAUNCH(3, 0);
+		else GRAM_LAUNCH(4, 0);
+	}
+	else {
+		if(NB == 1) GRAM_LAUNCH(1, 1);
+		else if(NB == 2) GRAM_LAUNCH(2, 1);
+		else if(NB == 3) GRAM_LAUNCH(3, 1);
+		else GRAM_LAUNCH(4, 1);
+	}
 #undef GRAM_LAUNCH
 	CLA_HIP(hipGetLastError());
 	return 0;

@@ -450,7 +450,13 @@ int launch_tsmm(cla_block* b, double* dOut, unsigned long long* dNnz) {
 			}
 	}
 	int rc;
-	const bool dense = nG >= nCols || b->hasUnc;
+	// Decoded Gram matrix on the matrix cores (one pass over all groups) against one pass per
+	// pair of groups: the first costs about as much per 16 x 16 tile of the result and row as
+	// the second per eight pairs and row.
+	const bool forceDecode = getenv("CLA_TSMM_DECODE") != nullptr, forcePairs = getenv("CLA_TSMM_PAIRS") != nullptr; // per call: tests switch them
+	const int nb = (nCols + 15) / 16;
+	const bool gramCheaper = nCols <= 64 && (int64_t) nG * (nG - 1) / 2 >= (int64_t) 8 * nb * (nb + 1) / 2;
+	const bool dense = nG >= nCols || b->hasUnc || forceDecode || (gramCheaper && !forcePairs);
 	if(dense) {
 		// t(D) %*% D of the decoded rows, constants included (no correction layer needed)
 		static const bool noMfma = getenv("CLA_TSMM_NO_MFMA") != nullptr;

@@ -29,11 +29,26 @@ def test_mixed_groups_tsmm(cla, ora, seed, n_rows, with_unc):
     check_tsmm(cla, ora, specs, n_rows, n_cols, f"tsmm unc={with_unc}")
 
 
-def test_c3_scaled(cla, ora):
-    """BASELINE config 3 at 1/100 scale: 25 co-coded pairs, 4096 tuples, uint16 codes."""
+@pytest.mark.parametrize("path", ["CLA_TSMM_PAIRS", "CLA_TSMM_DECODE"])
+@pytest.mark.parametrize("seed,n_rows", [(1, 37), (2, 3000), (4, 150001)])
+def test_mixed_groups_tsmm_both_paths(cla, ora, monkeypatch, path, seed, n_rows):
+    """The per-pair path and the decoded Gram matrix on the matrix cores are interchangeable:
+    the library picks by cost, the switches (read per call) force one."""
+    monkeypatch.setenv(path, "1")
+    specs, n_cols = mixed_block(seed, n_rows, with_unc=False)
+    check_tsmm(cla, ora, specs, n_rows, n_cols, f"tsmm {path}")
+
+
+@pytest.mark.parametrize("path", [None, "CLA_TSMM_PAIRS", "CLA_TSMM_DECODE"])
+def test_c3_scaled(cla, ora, monkeypatch, path):
+    """BASELINE config 3 at 1/100 scale: 25 co-coded pairs, 4096 tuples, uint16 codes. The
+    dictionaries do not fit LDS together: the decoded path looks them up in global memory. The
+    row count is no multiple of the tile, so the last tile is ragged."""
     from systemds_amd import synth
+    if path:
+        monkeypatch.setenv(path, "1")
     c = synth.config3(scale=100)
-    check_tsmm(cla, ora, c["groups"], c["n_rows"], c["n_cols"], "C3")
+    check_tsmm(cla, ora, c["groups"], c["n_rows"], c["n_cols"], f"C3 {path}")
 
 
 def test_c5_scaled(cla, ora):
