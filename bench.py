@@ -51,7 +51,7 @@ def timed(blk, fn, reps=5, warm=2):
 
 
 def other_configs(scale):
-    """X %*% v of C1, t(X) %*% X of C3, both products of C4, both products of C5."""
+    """X %*% v of C1, the other products of C2, t(X) %*% X of C3, both products of C4 and of C5."""
     import numpy as np
     import torch
     from systemds_amd import capi, synth
@@ -93,6 +93,10 @@ def other_configs(scale):
         do1 = torch.empty((1, m), dtype=torch.float64, device="cuda")
         do2 = torch.empty((m,), dtype=torch.float64, device="cuda")
         comp = float(blk.device_bytes())
+        dB = dev(cfg["B"])
+        q = cfg["B"].shape[1]
+        do0 = torch.empty((n, q), dtype=torch.float64, device="cuda")
+        yield ("X%*%B", lambda: blk.rmm_dev(dB.data_ptr(), q, do0.data_ptr()), comp + n * q * 8.0)
         yield ("t(y)%*%X", lambda: blk.lmm_dev(dy.data_ptr(), 1, do1.data_ptr()), comp + n * 8.0)
         yield ("t(X)%*%(X%*%v)", lambda: blk.mmchain_dev(dv.data_ptr(), None, 0, do2.data_ptr()), 2 * comp + 2 * n * 8.0)
     run("C2", c, c2_ops)
@@ -136,7 +140,7 @@ def main():
     ap.add_argument("--scale", type=int, default=1, help="divide the number of rows (testing only)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--extra", action="store_true", help="also time X %*% B (100x64) of the same config")
-    ap.add_argument("--all", action="store_true", help="also time the other BASELINE configs (C1, C3, C4, C5)")
+    ap.add_argument("--all", action="store_true", help="also time the other products and BASELINE configs (C1, C2 mat-mat, left multiply and chain, C3, C4, C5)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (torch) so that a rocprofv3 --pmc run can scale "
                          "FETCH_SIZE / WRITE_SIZE against a kernel of known traffic")
