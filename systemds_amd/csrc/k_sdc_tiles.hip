@@ -4,7 +4,7 @@
 // by every group, instead of being gathered from / scattered to HBM per entry.
 //
 //   k_lmm_sdc_tiles   bins[g][code] += Y[i, row] for every listed row (t(v) %*% X)
-//   k_rmm_sdc_tiles   out[row, :] += T_g[code, :] for every listed row (X %*% u)
+//   k_rmm_sdc_tiles   out[row, :] += T_g[code, :] for every listed row (X %*% u); tables from L2
 //
 // A tile is ST = 4 * SDC_TILE rows; the iterator state in front of a tile comes
 // from the row-tile index built at finalize.
@@ -95,7 +95,7 @@ __global__ __launch_bounds__(ST_THREADS) void k_lmm_sdc_tiles(const DGroup* __re
 __global__ __launch_bounds__(ST_THREADS) void k_rmm_sdc_tiles(const DGroup* __restrict__ groups,
 	const int32_t* __restrict__ sdcList, const int32_t* __restrict__ binOff, int nL, int slabLen, const double* __restrict__ T,
 	int q, int constRow, int accumulate, int tileRows, double* __restrict__ out, int64_t nRows,
-	unsigned long long* __restrict__ nnz) {
+	unsigned long long* __restrict__ nnz, int ldsTables) {
 	extern __shared__ double smem[];
 	double* otile = smem;                       // tileRows * q
 	double* tbl = smem + (size_t) tileRows * q; // tables of the current slab, q doubles per tuple
@@ -112,16 +112,18 @@ __global__ __launch_bounds__(ST_THREADS) void k_rmm_sdc_tiles(const DGroup* __re
 		const int l1 = min(l0 + slabLen, nL);
 		const int b0 = binOff[l0];
 		__syncthreads();
-		for(int l = l0; l < l1; l++) {
-			const DGroup G = dgroup(groups + (sdcList[l]));
-			double* tg = tbl + (size_t) (binOff[l] - b0) * q;
-			const double* src = T + (size_t) G.tblOff * q;
-			for(int k = tid; k < G.nVals * q; k += ST_THREADS) tg[k] = src[k];
+		if(ldsTables) {
+			for(int l = l0; l < l1; l++) {
+				const DGroup G = dgroup(groups + (sdcList[l]));
+				double* tg = tbl + (size_t) (binOff[l] - b0) * q;
+				const double* src = T + (size_t) G.tblOff * q;
+				for(int k = tid; k < G.nVals * q; k += ST_THREADS) tg[k] = src[k];
+			}
+			__syncthreads();
 		}
-		__syncthreads();
 		for(int l = l0 + wave; l < l1; l += ST_THREADS / 64) {
 			const DGroup G = dgroup(groups + (sdcList[l]));
-			const double* tg = tbl + (size_t) (binOff[l] - b0) * q;
+			const double* tg = ldsTables ? tbl + (size_t) (binOff[l] - b0) * q : T + (size_t) G.tblOff * q;
 			const void* codes = G.codes;
 			const int cw = G.codeWidth;
 			sdc_walk_tile(G, r0, tileRows, [&](int rr, int di) {
@@ -226,20 +228,25 @@ int launch_rmm_sdc_tiles(cla_block* b, int q, int constRow, int accumulate, doub
 	if((size_t) tileRows * q * 8 + 4096 > ldsMax) return 1;
 	size_t maxVals = 1;
 	for(size_t l = 0; l < plan.list.size(); l++) maxVals = std::max(maxVals, (size_t) (plan.binOff[l + 1] - plan.binOff[l]));
-	// Small table slabs keep LDS per block low enough for four blocks per CU: the list walks
-	// are chains of dependent loads and only occupancy hides them (C4: 1.95 ms with one
-	// 100 KB slab, 0.75 ms with 8 KB slabs).
+	// Tables are read from global memory (they stay in L2): without table slabs in LDS the
+	// waves of a block never meet at a barrier between the list walks, and only the output
+	// tile takes LDS (C4: 1.95 ms with one 100 KB slab in LDS, 0.72 ms with 8 KB slabs,
+	// 0.58 ms with none). CLA_RMM_SDC_TBL_KB > 0 brings the slabs back.
 	size_t tblBudget = 8 * 1024;
-	if(const char* e = getenv("CLA_RMM_SDC_TBL_KB")) tblBudget = (size_t) std::max(1, atoi(e)) * 1024;
+	bool ldsTables = false;
+	if(const char* e = getenv("CLA_RMM_SDC_TBL_KB")) {
+		tblBudget = (size_t) std::max(1, atoi(e)) * 1024;
+		ldsTables = atoi(e) > 0;
+	}
 	tblBudget = std::max(tblBudget, maxVals * q * 8);
 	tblBudget = std::min(tblBudget, ldsMax - (size_t) tileRows * q * 8);
 	// groups per slab: uniform count so that every slab's tables fit
 	const size_t slabLen = tblBudget / (maxVals * q * 8);
 	if(slabLen < 1) return 1;
 	const int nTiles = (int) ((b->nRows + tileRows - 1) / tileRows);
-	const int sl = (int) std::min(slabLen, plan.list.size());
+	const int sl = ldsTables ? (int) std::min(slabLen, plan.list.size()) : (int) plan.list.size();
 	size_t tblDoubles = 0;
-	for(size_t l0 = 0; l0 < plan.list.size(); l0 += sl)
+	for(size_t l0 = 0; ldsTables && l0 < plan.list.size(); l0 += sl)
 		tblDoubles = std::max(tblDoubles, (size_t) (plan.binOff[std::min(l0 + sl, plan.list.size())] - plan.binOff[l0]) * q);
 	const size_t lds = (size_t) tileRows * q * 8 + tblDoubles * 8;
 	double algo = (double) b->nRows * q * 8 * (accumulate ? 2 : 1);
@@ -251,7 +258,7 @@ int launch_rmm_sdc_tiles(cla_block* b, int q, int constRow, int accumulate, doub
 		Prof pf(b, "k_rmm_sdc_tiles", nTiles, ST_THREADS, (long) lds, algo);
 		CLA_HIP(hipFuncSetAttribute((const void*) k_rmm_sdc_tiles, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
 		hipLaunchKernelGGL(k_rmm_sdc_tiles, dim3(nTiles), dim3(ST_THREADS), lds, b->stream, b->dGroups, dList, dBinOff,
-			(int) plan.list.size(), sl, b->dTables, q, constRow, accumulate, tileRows, dOut, b->nRows, dNnz);
+			(int) plan.list.size(), sl, b->dTables, q, constRow, accumulate, tileRows, dOut, b->nRows, dNnz, ldsTables ? 1 : 0);
 	}
 	CLA_HIP(hipGetLastError());
 	return 0;
