@@ -3,6 +3,7 @@
 // component/compress/): build column groups with the factories, put them into a
 // CompressedMatrixBlock, call the CLALib* drivers, compare with the dense product.
 #include "cla_host.hpp"
+#include "cla_wire.hpp"
 
 #include <pybind11/numpy.h>
 #include <pybind11/pybind11.h>
@@ -114,6 +115,7 @@ PYBIND11_MODULE(_clahost, m) {
 		.def("getColIndices", &AColGroup::getColIndices)
 		.def("getNumCols", &AColGroup::getNumCols)
 		.def("getNumValues", &AColGroup::getNumValues)
+		.def("getDictionary", &AColGroup::getDictionary)
 		.def("getCompType", &AColGroup::getCompType);
 	py::class_<ColGroupEmpty, AColGroup, std::shared_ptr<ColGroupEmpty>>(m, "ColGroupEmpty")
 		.def(py::init([](const IArr& c) { return std::make_shared<ColGroupEmpty>(ColIndexFactory::create(to_ivec(c))); }));
@@ -124,6 +126,7 @@ PYBIND11_MODULE(_clahost, m) {
 		.def_static("create", [](const IArr& c, std::shared_ptr<Dictionary> d, std::shared_ptr<AMapToData> map) {
 			return ColGroupDDC::create(ColIndexFactory::create(to_ivec(c)), std::move(d), std::move(map));
 		})
+		.def("getMapToData", &ColGroupDDC::getMapToData)
 		.def("getCounts", &ColGroupDDC::getCounts);
 	py::class_<ColGroupSDCBase, AColGroup, std::shared_ptr<ColGroupSDCBase>>(m, "ColGroupSDCBase")
 		.def("getOffsets", &ColGroupSDCBase::getOffsets)
@@ -154,7 +157,8 @@ PYBIND11_MODULE(_clahost, m) {
 		.def_static("create", [](std::shared_ptr<MatrixBlock> mb, const IArr& c) {
 			return ColGroupUncompressed::create(std::move(mb), ColIndexFactory::create(to_ivec(c)));
 		})
-		.def_static("create", [](std::shared_ptr<MatrixBlock> mb) { return ColGroupUncompressed::create(std::move(mb)); });
+		.def_static("create", [](std::shared_ptr<MatrixBlock> mb) { return ColGroupUncompressed::create(std::move(mb)); })
+		.def("getData", &ColGroupUncompressed::getData);
 
 	py::class_<CompressedMatrixBlock, MatrixBlock, std::shared_ptr<CompressedMatrixBlock>>(m, "CompressedMatrixBlock")
 		.def(py::init([](int rl, int cl) { return std::make_shared<CompressedMatrixBlock>(rl, cl); }))
@@ -187,6 +191,15 @@ PYBIND11_MODULE(_clahost, m) {
 	py::class_<CLALibMatrixMult>(m, "CLALibMatrixMult")
 		.def_static("matrixMultiply", &CLALibMatrixMult::matrixMultiply, py::arg("m1"), py::arg("m2"), py::arg("k") = 1,
 			py::arg("transposeLeft") = false, py::arg("transposeRight") = false);
+	// CompressedMatrixBlock.read / write on byte strings
+	m.def("readCompressedMatrixBlock", [](const py::bytes& b) {
+		const std::string s = b; // copies; the block owns its data afterwards
+		return io::readCompressedMatrixBlock((const uint8_t*) s.data(), s.size());
+	});
+	m.def("writeCompressedMatrixBlock", [](const CompressedMatrixBlock& cmb) {
+		const std::vector<uint8_t> v = io::writeCompressedMatrixBlock(cmb);
+		return py::bytes((const char*) v.data(), v.size());
+	});
 	py::class_<CLALibDecompress>(m, "CLALibDecompress")
 		.def_static("decompress", &CLALibDecompress::decompress, py::arg("cmb"), py::arg("k") = 1);
 }

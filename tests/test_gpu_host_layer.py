@@ -134,3 +134,32 @@ def test_group_list_can_be_replaced(H, ora, cla):
     second = H.CLALibRightMultBy.rightMultByMatrix(cmb, H.MatrixBlock(B)).toArray()
     close(first, D, B, "before", ora)
     close(second, D2, B, "after", ora)
+
+
+@pytest.mark.parametrize("seed,n_rows", [(5, 300), (6, 40000)])
+def test_serialised_block_goes_straight_to_the_device(H, ora, cla, seed, n_rows):
+    """Bytes in the layout of CompressedMatrixBlock.write (C/CompressedMatrixBlock.java:493-523), written by the
+    Python restatement in the type variants the reference's factories pick from, are read into column groups and
+    multiplied on the GPU without a JVM in between."""
+    from oracle import cla_wire
+    specs, n_cols = mixed_block(seed, n_rows, with_unc=True)
+    D = ora.np_decompress(specs, n_rows, n_cols)
+    variants = []
+    for i, s in enumerate(specs):
+        v = {}
+        if s.type == "ddc" and i % 2 == 0:
+            v["dict"] = "MATRIX_BLOCK_DICT"
+            v["block"] = "SPARSE_BLOCK"
+        if s.type == "unc":
+            v["block"] = "SPARSE_BLOCK"
+        if len(s.cols) > 2:
+            v["index"] = "ARRAY"
+        variants.append(v)
+    cmb = H.readCompressedMatrixBlock(cla_wire.compressed_block(n_rows, n_cols, specs, variants=variants))
+    rng = np.random.default_rng(seed)
+    B = rng.standard_normal((n_cols, 5))
+    Y = rng.standard_normal((2, n_rows))
+    mm = H.CLALibMatrixMult.matrixMultiply
+    close(mm(cmb, H.MatrixBlock(B), 4).toArray(), D, B, "X %*% B from bytes", ora)
+    close(mm(H.MatrixBlock(Y), cmb, 4).toArray(), Y, D, "Y %*% X from bytes", ora)
+    close(cmb.transposeSelfMatrixMultOperations(H.MMTSJType.LEFT, 4).toArray(), D.T, D, "t(X) %*% X from bytes", ora)
