@@ -132,6 +132,18 @@ int64_t cla_mmchain_dev(cla_handle h, const double* dV, const double* dW, int32_
 int64_t cla_decompress(cla_handle h, double* out);
 int64_t cla_decompress_dev(cla_handle h, double* dOut);
 
+/* CLALibCompAgg.aggregateUnary (C/lib/CLALibCompAgg.java:78-127) for the operators whose
+ * per-group form is counts x dictionary (AColGroupCompressed.unaryAggregateOperations,
+ * CG/AColGroupCompressed.java:137-205): op = sum, sum of squares, min, max; dir = all cells
+ * (out[1]), per row (out[nRows]), per column (out[nCols]). Returns the number of non-zero
+ * cells of the result. Not on the device path (CLA_ERR_UNSUPPORTED, caller falls back as for
+ * any unsupported combination): row minima / maxima, row sums of squares with an
+ * uncompressed group, anything but plain sums on overlapping groups. */
+enum cla_agg_op { CLA_AGG_SUM = 0, CLA_AGG_SUMSQ = 1, CLA_AGG_MIN = 2, CLA_AGG_MAX = 3 };
+enum cla_agg_dir { CLA_AGG_ALL = 0, CLA_AGG_ROW = 1, CLA_AGG_COL = 2 };
+int64_t cla_aggregate(cla_handle h, int32_t op, int32_t dir, double* out);
+int64_t cla_aggregate_dev(cla_handle h, int32_t op, int32_t dir, double* dOut);
+
 /* ---- per-group pieces (AColGroup surface) ---- */
 
 /* AMapToData.getCounts / ColGroupRLE.getCounts (CG/mapping/AMapToData.java:408-419,

@@ -16,6 +16,10 @@ _i32p = C.POINTER(C.c_int32)
 _f64p = C.POINTER(C.c_double)
 
 
+# negative return codes of the C ABI (include/cla_hip.h, enum cla_error)
+ERR_INVALID, ERR_UNSUPPORTED, ERR_DEVICE, ERR_STATE = -1, -2, -3, -4
+
+
 class ClaError(RuntimeError):
     """Negative return code of the C ABI (message from cla_last_error)."""
 
@@ -51,6 +55,8 @@ SIGNATURES = {
     "cla_tsmm_dev": (C.c_int64, [C.c_void_p, C.c_void_p]),
     "cla_mmchain": (C.c_int64, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
     "cla_mmchain_dev": (C.c_int64, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
+    "cla_aggregate": (C.c_int64, [C.c_void_p, C.c_int32, C.c_int32, C.c_void_p]),
+    "cla_aggregate_dev": (C.c_int64, [C.c_void_p, C.c_int32, C.c_int32, C.c_void_p]),
     "cla_decompress": (C.c_int64, [C.c_void_p, C.c_void_p]),
     "cla_decompress_dev": (C.c_int64, [C.c_void_p, C.c_void_p]),
     "cla_counts": (C.c_int, [C.c_void_p, C.c_int32, C.c_void_p]),
@@ -241,6 +247,19 @@ class ClaBlock:
         out = np.empty((self.n_cols,), np.float64)
         nnz = _check(self.lib.cla_mmchain(self.h, _ptr(v), _ptr(w), int(ctype), _ptr(out)))
         return out, nnz
+
+    AGG_OP = {"sum": 0, "sumsq": 1, "min": 2, "max": 3}
+    AGG_DIR = {"all": 0, "row": 1, "col": 2}
+
+    def aggregate(self, op, direction):
+        """cla_aggregate: op in sum / sumsq / min / max, direction in all / row / col."""
+        n = {"all": 1, "row": self.n_rows, "col": self.n_cols}[direction]
+        out = np.empty((max(n, 1),), np.float64)
+        nnz = _check(self.lib.cla_aggregate(self.h, self.AGG_OP[op], self.AGG_DIR[direction], _ptr(out)))
+        return out[:n], nnz
+
+    def aggregate_dev(self, op, direction, dOut_ptr):
+        return _check(self.lib.cla_aggregate_dev(self.h, self.AGG_OP[op], self.AGG_DIR[direction], C.c_void_p(dOut_ptr)))
 
     def decompress(self):
         out = np.empty((self.n_rows, self.n_cols), np.float64)

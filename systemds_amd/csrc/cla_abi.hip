@@ -225,6 +225,7 @@ void cla_block_free(cla_handle b) {
 	if(b->dSdcPlan) (void) hipFree(b->dSdcPlan);
 	if(b->dDictPad) (void) hipFree(b->dDictPad);
 	if(b->dCountsAll) (void) hipFree(b->dCountsAll);
+	if(b->dOnes) (void) hipFree(b->dOnes);
 	if(b->dCounters) (void) hipFree(b->dCounters);
 	if(b->hCounters) (void) hipHostFree(b->hCounters);
 	if(b->ownStream && b->stream) (void) hipStreamDestroy(b->stream);
@@ -634,6 +635,29 @@ int64_t cla_tsmm(cla_handle b, double* out) {
 	const int64_t nnz = cla_tsmm_dev(b, b->dStageOut);
 	if(nnz < 0) return nnz;
 	CLA_HIP(hipMemcpy(out, b->dStageOut, nOut * sizeof(double), hipMemcpyDeviceToHost));
+	return nnz;
+}
+
+int64_t cla_aggregate_dev(cla_handle b, int32_t op, int32_t dir, double* dOut) {
+	int rc = check_final(b);
+	if(rc) return rc;
+	if(!dOut) { set_error("aggregate: null output"); return -CLA_ERR_INVALID; }
+	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	if((rc = launch_aggregate(b, op, dir, dOut, b->dCounters))) return rc;
+	return finish_nnz(b);
+}
+
+int64_t cla_aggregate(cla_handle b, int32_t op, int32_t dir, double* out) {
+	int rc = check_final(b);
+	if(rc) return rc;
+	if(!out) { set_error("aggregate: null output"); return -CLA_ERR_INVALID; }
+	if(dir < CLA_AGG_ALL || dir > CLA_AGG_COL) { set_error("aggregate: unknown direction %d", dir); return -CLA_ERR_INVALID; }
+	const size_t nOut = dir == CLA_AGG_ALL ? 1 : dir == CLA_AGG_ROW ? (size_t) b->nRows : (size_t) b->nCols;
+	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	if((rc = ensure_stage(&b->dStageOut, &b->stageOutCap, std::max<size_t>(nOut, 1)))) return rc;
+	const int64_t nnz = cla_aggregate_dev(b, op, dir, b->dStageOut);
+	if(nnz < 0) return nnz;
+	if(nOut) CLA_HIP(hipMemcpy(out, b->dStageOut, nOut * sizeof(double), hipMemcpyDeviceToHost));
 	return nnz;
 }
 

@@ -109,6 +109,7 @@ struct cla_block {
 	// computed on the first TSMM and kept, like the reference's cached counts
 	// (CG/AColGroupValue.java getCounts)
 	int32_t* dCountsAll = nullptr;
+	double* dOnes = nullptr;         // nCols ones: rowSums(X) = X %*% 1
 	// all groups single-column DDC with byte codes: dictionaries at a fixed stride of 256 entries
 	// (zero beyond nVals) followed by the groups' column indexes; built on first use
 	double* dDictPad = nullptr;
@@ -143,7 +144,9 @@ extern int g_numCU;
 int launch_validate_codes(cla_block* b, const void* codes, int width, int64_t n, int nVals, int* ok);
 int launch_counts(cla_block* b, int group, int32_t* dCounts);
 int launch_sdc_build(cla_block* b, HostGroup& g);
-int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned long long* dNnz);
+int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned long long* dNnz, int squares = 0);
+int launch_aggregate(cla_block* b, int op, int dir, double* dOut, unsigned long long* dNnz);
+int ensure_counts(cla_block* b);
 int launch_rmm_mfma(cla_block* b, const double* dB, int q, const double* dConstRow, double* dOut,
 	unsigned long long* dNnz);
 int launch_lmm_u8(cla_block* b, const double* dY, int p, double* dPre);

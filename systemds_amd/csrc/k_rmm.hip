@@ -20,7 +20,7 @@ namespace cla {
 // ---------------------------------------------------------------------------
 __global__ void k_preagg(const DGroup* __restrict__ groups, int nGroups, const double* __restrict__ B, int q,
 	int nCols, const double* __restrict__ constV, double* __restrict__ T, int totalVals,
-	unsigned long long* __restrict__ nnz, double* __restrict__ Tpad) {
+	unsigned long long* __restrict__ nnz, double* __restrict__ Tpad, int squares) {
 	const int g = blockIdx.y;
 	const int idx = blockIdx.x * blockDim.x + threadIdx.x;
 	if(g == 0 && idx == 0) *nnz = 0; // the multiply kernels behind this one on the stream count into it
@@ -32,7 +32,8 @@ __global__ void k_preagg(const DGroup* __restrict__ groups, int nGroups, const d
 		double acc = 0;
 		for(int c0 = 0; c0 < nCols; c0++) {
 			const double a = constV[c0];
-			if(a != 0) acc = __dadd_rn(acc, __dmul_rn(a, B[(size_t) c0 * q + idx]));
+			if(squares) acc += a * a;
+			else if(a != 0) acc = __dadd_rn(acc, __dmul_rn(a, B[(size_t) c0 * q + idx]));
 		}
 		T[(size_t) totalVals * q + idx] = acc;
 		return;
@@ -43,7 +44,11 @@ __global__ void k_preagg(const DGroup* __restrict__ groups, int nGroups, const d
 	double acc = 0;
 	for(int h = 0; h < G.nColG; h++) {
 		const double v = G.dict[(size_t) k * G.nColG + h];
-		if(v != 0) acc = __dadd_rn(acc, __dmul_rn(v, B[(size_t) G.cols[h] * q + c]));
+		if(squares) { // row sums of squares: the tuple's part beyond the constants' (q == 1)
+			const double cc = constV != nullptr ? constV[G.cols[h]] : 0.0;
+			acc += (v + cc) * (v + cc) - cc * cc;
+		}
+		else if(v != 0) acc = __dadd_rn(acc, __dmul_rn(v, B[(size_t) G.cols[h] * q + c]));
 	}
 	T[(size_t) (G.tblOff + k) * q + c] = acc;
 	if(Tpad != nullptr) Tpad[(size_t) g * 256 + k] = acc;
@@ -490,7 +495,9 @@ __global__ __launch_bounds__(256) void k_count_nnz(const double* __restrict__ x,
 	count_add(nnz, cnt);
 }
 
-int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned long long* dNnz) {
+// squares != 0 (q == 1, no uncompressed group): the tables hold the sum of squares of each tuple
+// instead of dict x B, so that the gather yields rowSums(X^2).
+int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned long long* dNnz, int squares) {
 	const int nG = (int) b->groups.size();
 	const int64_t nRows = b->nRows;
 	hipStream_t st = b->stream;
@@ -508,7 +515,7 @@ int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned lon
 		dim3 grid((maxWork + 255) / 256 > (q + 255) / 256 ? (maxWork + 255) / 256 : (q + 255) / 256, nG + 1);
 		Prof pf(b, "k_preagg", (long) grid.x * grid.y, 256, 0, 0);
 		hipLaunchKernelGGL(k_preagg, grid, dim3(256), 0, st, b->dGroups, nG, dB, q, b->nCols,
-			b->hasConst ? b->dConstV : nullptr, b->dTables, b->totalVals, dNnz, dTpad);
+			b->hasConst ? b->dConstV : nullptr, b->dTables, b->totalVals, dNnz, dTpad, squares);
 	}
 	const int constRow = b->hasConst ? b->totalVals : -1;
 	if(nRows == 0) return 0;

@@ -499,13 +499,7 @@ int launch_tsmm(cla_block* b, double* dOut, unsigned long long* dNnz) {
 	double* dColSum = (double*) b->dScratch;
 	int4* dPairs = (int4*) ((char*) b->dScratch + sumBytes);
 	CLA_HIP(hipMemsetAsync(dColSum, 0, sizeof(double) * (size_t) nCols, st));
-	if(b->dCountsAll == nullptr) {
-		int32_t* dc = nullptr;
-		CLA_HIP(hipMalloc((void**) &dc, sizeof(int32_t) * (size_t) std::max(b->totalVals, 1)));
-		for(int g = 0; g < nG; g++)
-			if((rc = launch_counts(b, g, dc + b->groups[g].d.tblOff))) { (void) hipFree(dc); return rc; }
-		b->dCountsAll = dc;
-	}
+	if((rc = ensure_counts(b))) return rc;
 	if(nG > 0) {
 		Prof pf(b, "k_tsmm_self", nG, 256, 0, 0);
 		hipLaunchKernelGGL(k_tsmm_self, dim3(1, nG), dim3(256), 0, st, b->dGroups, b->dCountsAll, dOut, nCols, dColSum);

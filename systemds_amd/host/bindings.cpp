@@ -184,6 +184,10 @@ PYBIND11_MODULE(_clahost, m) {
 		.def_static("leftMultByMatrixTransposed", &CLALibLeftMultBy::leftMultByMatrixTransposed, py::arg("right"), py::arg("left"), py::arg("k") = 1);
 	py::class_<CLALibTSMM>(m, "CLALibTSMM")
 		.def_static("leftMultByTransposeSelf", &CLALibTSMM::leftMultByTransposeSelf, py::arg("cmb"), py::arg("k") = 1);
+	py::enum_<AggOp>(m, "AggOp").value("SUM", AggOp::SUM).value("SUMSQ", AggOp::SUMSQ).value("MIN", AggOp::MIN).value("MAX", AggOp::MAX);
+	py::enum_<AggDir>(m, "AggDir").value("ReduceAll", AggDir::ReduceAll).value("ReduceCol", AggDir::ReduceCol).value("ReduceRow", AggDir::ReduceRow);
+	py::class_<CLALibCompAgg>(m, "CLALibCompAgg")
+		.def_static("aggregateUnary", &CLALibCompAgg::aggregateUnary, py::arg("m"), py::arg("op"), py::arg("dir"), py::arg("k") = 1);
 	py::class_<CLALibMMChain>(m, "CLALibMMChain")
 		.def_static("mmChain", [](CompressedMatrixBlock& x, const MatrixBlock& v, const MatrixBlock* w, ChainType ct, int k) {
 			return CLALibMMChain::mmChain(x, v, w, ct, k);

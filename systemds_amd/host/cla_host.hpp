@@ -630,6 +630,26 @@ struct CLALibDecompress {
 	}
 };
 
+// CLALibCompAgg.aggregateUnary (C/lib/CLALibCompAgg.java:78-127) for sum, sumSq, min, max in the
+// three directions of the reference's index functions (ReduceAll, ReduceCol = per row,
+// ReduceRow = per column). Combinations the device path does not take raise
+// NotImplementedException, where the reference's caller would decompress and aggregate.
+enum class AggOp { SUM = CLA_AGG_SUM, SUMSQ = CLA_AGG_SUMSQ, MIN = CLA_AGG_MIN, MAX = CLA_AGG_MAX };
+enum class AggDir { ReduceAll = CLA_AGG_ALL, ReduceCol = CLA_AGG_ROW, ReduceRow = CLA_AGG_COL };
+
+struct CLALibCompAgg {
+	static MatrixBlock aggregateUnary(CompressedMatrixBlock& m, AggOp op, AggDir dir, int /*k*/) {
+		const int rr = dir == AggDir::ReduceCol ? m.getNumRows() : 1;
+		const int rc = dir == AggDir::ReduceRow ? m.getNumColumns() : 1;
+		MatrixBlock ret(rr, rc);
+		if(m.getNumRows() == 0 || m.getNumColumns() == 0) return ret;
+		const int64_t nnz = cla_aggregate(m.hipHandle(), (int32_t) op, (int32_t) dir, ret.getDenseBlockValues());
+		if(nnz == -CLA_ERR_UNSUPPORTED) throw NotImplementedException(std::string("aggregateUnary: ") + cla_last_error());
+		ret.setNonZeros(checkNative(nnz, "aggregateUnary"));
+		return ret;
+	}
+};
+
 struct CLALibRightMultBy {
 	// ret = m1 %*% m2 (dense result; the overlapping compressed result of the reference's
 	// allowOverlap = true branch is not produced here).

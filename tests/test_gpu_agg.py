@@ -1,0 +1,105 @@
+"""GPU parity of the unary aggregates on compressed blocks (cla_aggregate), against the
+aggregate of the decompressed matrix: sum / sumSq by long-double accumulation at the 1e-12
+bar of the multiply path (scale = sum of |terms|), min / max up to the rounding of the SDC
+default morph ((dict - default) + default), which the reference's decompression has as well.
+Mirrors the aggregate cases of the reference's CompressedTestBase (T/CompressedTestBase.java
+unaryAggregate tests: the compressed result against the uncompressed operator)."""
+import numpy as np
+import pytest
+
+from conftest import host_groups, mixed_block
+from parity import assert_fp64_close
+
+pytestmark = pytest.mark.gpu
+
+OPS = ["sum", "sumsq", "min", "max"]
+DIRS = ["all", "row", "col"]
+
+
+def truth(D, op, direction):
+    L = D.astype(np.longdouble)
+    axis = {"all": None, "row": 1, "col": 0}[direction]
+    if op == "sum":
+        return np.asarray(L.sum(axis=axis), np.longdouble).astype(np.float64).reshape(-1), np.abs(D).sum(axis=axis).reshape(-1)
+    if op == "sumsq":
+        return np.asarray((L * L).sum(axis=axis), np.longdouble).astype(np.float64).reshape(-1), (D * D).sum(axis=axis).reshape(-1)
+    f = np.min if op == "min" else np.max
+    return np.asarray(f(D, axis=axis)).reshape(-1), np.asarray(np.abs(D).max(axis=axis)).reshape(-1) + 2.0
+
+
+def check(cla, specs, D, n_rows, n_cols, op, direction, what):
+    blk = cla.build_block(n_rows, n_cols, specs)
+    try:
+        out, nnz = blk.aggregate(op, direction)
+    finally:
+        blk.close()
+    ref, scale = truth(D, op, direction)
+    assert_fp64_close(out, ref, scale, what=f"{what} {op}/{direction}")
+    assert nnz == np.count_nonzero(out)
+
+
+@pytest.mark.parametrize("op", OPS)
+@pytest.mark.parametrize("direction", DIRS)
+@pytest.mark.parametrize("seed,n_rows,with_unc", [(1, 37, False), (2, 3000, True), (3, 150001, False), (4, 70000, True)])
+def test_mixed_groups(cla, ora, op, direction, seed, n_rows, with_unc):
+    specs, n_cols = mixed_block(seed, n_rows, with_unc=with_unc)
+    D = ora.np_decompress(specs, n_rows, n_cols)
+    if direction == "row" and (op in ("min", "max") or (op == "sumsq" and with_unc)):
+        blk = cla.build_block(n_rows, n_cols, specs)
+        with pytest.raises(cla.ClaError) as e:
+            blk.aggregate(op, direction)
+        blk.close()
+        assert e.value.code == cla.ERR_UNSUPPORTED
+        return
+    check(cla, specs, D, n_rows, n_cols, op, direction, "mixed")
+
+
+@pytest.mark.parametrize("direction", DIRS)
+def test_overlapping_groups_sum_only(cla, ora, direction):
+    """Sums are linear in the groups (CLALibCompAgg.java: overlapping blocks aggregate per group for sum-like
+    operators and decompress otherwise); everything else is refused on overlapping blocks."""
+    n_rows = 5000
+    specs, n_cols = mixed_block(5, n_rows, with_unc=False, overlap=True)
+    D = ora.np_decompress(specs, n_rows, n_cols)
+    check(cla, specs, D, n_rows, n_cols, "sum", direction, "overlap")
+    blk = cla.build_block(n_rows, n_cols, specs)
+    with pytest.raises(cla.ClaError) as e:
+        blk.aggregate("max", "col")
+    blk.close()
+    assert e.value.code == cla.ERR_UNSUPPORTED
+
+
+@pytest.mark.parametrize("cfg,scale", [("config2", 200), ("config3", 200), ("config4", 200), ("config5", 500)])
+def test_baseline_configs_scaled(cla, ora, cfg, scale):
+    from systemds_amd import synth
+    c = getattr(synth, cfg)(scale=scale)
+    n_rows, n_cols = c["n_rows"], c["n_cols"]
+    D = ora.np_decompress(c["groups"], n_rows, n_cols)
+    for op in OPS:
+        for direction in DIRS:
+            if direction == "row" and (op in ("min", "max") or (op == "sumsq" and cfg == "config5")):
+                continue
+            check(cla, c["groups"], D, n_rows, n_cols, op, direction, cfg)
+
+
+def test_host_layer_driver(H, ora, cla):
+    """CLALibCompAgg.aggregateUnary with the reference's direction names (ReduceCol = one value per row)."""
+    n_rows = 20000
+    specs, n_cols = mixed_block(6, n_rows, with_unc=True)
+    D = ora.np_decompress(specs, n_rows, n_cols)
+    cmb = H.CompressedMatrixBlock(n_rows, n_cols)
+    cmb.allocateColGroupList(host_groups(H, ora, specs, n_rows))
+    agg = H.CLALibCompAgg.aggregateUnary
+    r = agg(cmb, H.AggOp.SUM, H.AggDir.ReduceCol, 4)
+    assert (r.getNumRows(), r.getNumColumns()) == (n_rows, 1)
+    ref, scale = truth(D, "sum", "row")
+    assert_fp64_close(r.toArray().reshape(-1), ref, scale, what="rowSums")
+    c = agg(cmb, H.AggOp.MAX, H.AggDir.ReduceRow, 4)
+    assert (c.getNumRows(), c.getNumColumns()) == (1, n_cols)
+    ref, scale = truth(D, "max", "col")
+    assert_fp64_close(c.toArray().reshape(-1), ref, scale, what="colMaxs")
+    a = agg(cmb, H.AggOp.SUMSQ, H.AggDir.ReduceAll, 4)
+    ref, scale = truth(D, "sumsq", "all")
+    assert_fp64_close(a.toArray().reshape(-1), ref, scale, what="sumSq")
+    with pytest.raises(H.NotImplementedException):
+        agg(cmb, H.AggOp.MIN, H.AggDir.ReduceCol, 4)
