@@ -122,6 +122,18 @@ int64_t cla_lmm_dev(cla_handle h, const double* dY, int32_t nRowY, double* dOut)
 int64_t cla_tsmm(cla_handle h, double* out);
 int64_t cla_tsmm_dev(cla_handle h, double* dOut);
 
+/* CLALibRightMultBy.rightMultByMatrix with allowOverlap (RMMOverlapping,
+ * C/lib/CLALibRightMultBy.java:157-201): X %*% B kept compressed. Every group with row data
+ * returns a group over all nColB output columns that shares its index structure (codes,
+ * offsets, runs) with the source group and holds the dictionary dict_g x B[cols_g, :]
+ * (ADictBasedColGroup.rightMultByMatrix, CG/ADictBasedColGroup.java:246-275); constants go
+ * through B into the new block's constants. Only the small dictionary products are computed;
+ * the returned block (nRows x nColB, overlapping groups) takes every entry point that is
+ * linear in the groups (cla_rmm, cla_lmm, cla_mmchain, cla_decompress, sums) and borrows the
+ * device copies of the source block, which stays alive until both handles are freed.
+ * NULL on failure (cla_last_error); blocks with uncompressed groups are not supported. */
+cla_handle cla_rmm_overlapping(cla_handle h, const double* B, int32_t nColB);
+
 /* CLALibMMChain.mmChain (C/lib/CLALibMMChain.java:92-148):
  * out[nCols] = t(X) %*% (w * (X %*% v)); ctype 0 = XtXv (w ignored), 1 = XtwXv. */
 int64_t cla_mmchain(cla_handle h, const double* v, const double* w, int32_t ctype, double* out);

@@ -55,6 +55,7 @@ SIGNATURES = {
     "cla_tsmm_dev": (C.c_int64, [C.c_void_p, C.c_void_p]),
     "cla_mmchain": (C.c_int64, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
     "cla_mmchain_dev": (C.c_int64, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
+    "cla_rmm_overlapping": (C.c_void_p, [C.c_void_p, C.c_void_p, C.c_int32]),
     "cla_aggregate": (C.c_int64, [C.c_void_p, C.c_int32, C.c_int32, C.c_void_p]),
     "cla_aggregate_dev": (C.c_int64, [C.c_void_p, C.c_int32, C.c_int32, C.c_void_p]),
     "cla_decompress": (C.c_int64, [C.c_void_p, C.c_void_p]),
@@ -247,6 +248,18 @@ class ClaBlock:
         out = np.empty((self.n_cols,), np.float64)
         nnz = _check(self.lib.cla_mmchain(self.h, _ptr(v), _ptr(w), int(ctype), _ptr(out)))
         return out, nnz
+
+    def rmm_overlapping(self, B):
+        """cla_rmm_overlapping: X %*% B kept compressed (a new block that borrows this block's index structures)."""
+        B = _arr(B, np.float64)
+        B = B.reshape(self.n_cols, -1)
+        h = self.lib.cla_rmm_overlapping(self.h, _ptr(B), B.shape[1])
+        if not h:
+            raise ClaError(-1, last_error())
+        child = ClaBlock.__new__(ClaBlock)
+        child.lib, child.n_rows, child.n_cols, child.h = self.lib, self.n_rows, B.shape[1], h
+        child.n_vals = list(self.n_vals)
+        return child
 
     AGG_OP = {"sum": 0, "sumsq": 1, "min": 2, "max": 3}
     AGG_DIR = {"all": 0, "row": 1, "col": 2}

@@ -139,6 +139,8 @@ static int upload_dict(HostGroup& g) {
 	return upload(g, g.dict.data(), sizeof(double) * g.dict.size(), (const void**) &g.d.dict);
 }
 
+int finish_finalize(cla_block* b, cla_block* arenaFrom);
+
 } // namespace cla
 
 using namespace cla;
@@ -208,6 +210,8 @@ cla_handle cla_block_create(int64_t nRows, int32_t nCols) {
 
 void cla_block_free(cla_handle b) {
 	if(!b) return;
+	if(b->refs.fetch_sub(1) > 1) return; // blocks made from this one still use its streams
+	cla_block* parent = b->parent;
 	if(g_device >= 0) (void) hipSetDevice(g_device);
 	if(b->stream) (void) hipStreamSynchronize(b->stream);
 	clear_stats(b);
@@ -216,7 +220,7 @@ void cla_block_free(cla_handle b) {
 	if(b->dConstV) (void) hipFree(b->dConstV);
 	if(b->dAllDict) (void) hipFree(b->dAllDict);
 	if(b->dQ1Slabs) (void) hipFree(b->dQ1Slabs);
-	if(b->dArena) (void) hipFree(b->dArena);
+	if(b->dArena && !b->arenaShared) (void) hipFree(b->dArena);
 	if(b->dTblOff) (void) hipFree(b->dTblOff);
 	if(b->dTables) (void) hipFree(b->dTables);
 	if(b->dStageIn) (void) hipFree(b->dStageIn);
@@ -230,6 +234,7 @@ void cla_block_free(cla_handle b) {
 	if(b->hCounters) (void) hipHostFree(b->hCounters);
 	if(b->ownStream && b->stream) (void) hipStreamDestroy(b->stream);
 	delete b;
+	if(parent) cla_block_free(parent);
 }
 
 int cla_block_add_ddc(cla_handle b, const int32_t* cols, int32_t nColG, const double* dict, int32_t nVals,
@@ -427,7 +432,18 @@ int cla_block_finalize(cla_handle b) {
 	b->totalVals = tblOff;
 	b->totalColsG = colOff;
 	b->maxVals = maxVals;
+	return finish_finalize(b, nullptr);
+}
 
+} // extern "C"
+
+namespace cla {
+
+// Block-level part of finalize: dictionaries back to back, descriptor array, constants, table
+// offsets, code arena (built, or borrowed from arenaFrom whose groups this block mirrors one to
+// one), mat-vec slabs.
+int finish_finalize(cla_block* b, cla_block* arenaFrom) {
+	const int maxVals = b->maxVals;
 	const size_t nG = b->groups.size();
 	// all dictionaries back to back in one allocation (kernels copy a slab of
 	// consecutive groups' dictionaries into LDS as one contiguous range)
@@ -466,7 +482,13 @@ int cla_block_finalize(cla_handle b) {
 	const int cw = nG ? b->groups[0].d.codeWidth : 0;
 	for(auto& g : b->groups)
 		if(g.d.type != G_DDC || g.d.codeWidth != cw) allDdc = false;
-	if(allDdc) {
+	if(allDdc && arenaFrom != nullptr && arenaFrom->dArena != nullptr && arenaFrom->groups.size() == nG) {
+		b->dArena = arenaFrom->dArena; // the descriptors already point into it
+		b->arenaShared = true;
+		b->arenaStride = arenaFrom->arenaStride;
+		b->arenaWidth = arenaFrom->arenaWidth;
+	}
+	else if(allDdc) {
 		const size_t stride = (((size_t) b->nRows * cw) + 255) & ~(size_t) 255;
 		CLA_HIP(hipMalloc((void**) &b->dArena, stride * nG));
 		for(size_t i = 0; i < nG; i++) {
@@ -518,6 +540,10 @@ int cla_block_finalize(cla_handle b) {
 	b->finalized = true;
 	return 0;
 }
+
+} // namespace cla
+
+extern "C" {
 
 int cla_block_set_stream(cla_handle b, void* hipStream) {
 	if(!b) { set_error("null block handle"); return -CLA_ERR_INVALID; }
@@ -636,6 +662,68 @@ int64_t cla_tsmm(cla_handle b, double* out) {
 	if(nnz < 0) return nnz;
 	CLA_HIP(hipMemcpy(out, b->dStageOut, nOut * sizeof(double), hipMemcpyDeviceToHost));
 	return nnz;
+}
+
+cla_handle cla_rmm_overlapping(cla_handle b, const double* B, int32_t nColB) {
+	if(check_final(b)) return nullptr;
+	if(!B || nColB <= 0) { set_error("rmm: invalid right-hand side"); return nullptr; }
+	if(b->hasUnc) { set_error("overlapping right multiply: uncompressed groups are not supported"); return nullptr; }
+	const int q = nColB;
+	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	const size_t nIn = (size_t) b->nCols * q, nT = (size_t) (b->totalVals + 1) * q;
+	if(ensure_stage(&b->dStageIn, &b->stageInCap, nIn)) return nullptr;
+	if(hipMemcpyAsync(b->dStageIn, B, nIn * sizeof(double), hipMemcpyHostToDevice, b->stream) != hipSuccess) {
+		set_error("overlapping right multiply: copying B failed");
+		return nullptr;
+	}
+	if(launch_tables(b, b->dStageIn, q)) return nullptr;
+	std::vector<double> T(nT);
+	if(hipMemcpyAsync(T.data(), b->dTables, nT * sizeof(double), hipMemcpyDeviceToHost, b->stream) != hipSuccess ||
+		hipStreamSynchronize(b->stream) != hipSuccess) {
+		set_error("overlapping right multiply: reading the tables failed");
+		return nullptr;
+	}
+	cla_block* c = cla_block_create(b->nRows, q);
+	if(!c) return nullptr;
+	std::vector<int32_t> cols((size_t) q);
+	for(int j = 0; j < q; j++) cols[j] = j;
+	int tblOff = 0, colOff = 0, maxVals = 0;
+	for(auto& pg : b->groups) {
+		const DGroup& P = pg.d;
+		// groups without row data (const, empty, SDC without entries) live on in the constants only;
+		// the group list stays one to one with the source block otherwise, so the arena can be shared
+		if(P.type != G_DDC && P.type != G_SDCZ && P.type != G_RLE) {
+			if(b->dArena) { set_error("overlapping right multiply: unexpected group in an arena block"); cla_block_free(c); return nullptr; }
+			continue;
+		}
+		c->groups.emplace_back();
+		HostGroup& g = c->groups.back();
+		g.d = P; // codes, offsets, checkpoints, tile index, run table: borrowed
+		g.cols = cols;
+		g.d.nColG = q;
+		g.dict.assign(T.begin() + (size_t) P.tblOff * q, T.begin() + (size_t) (P.tblOff + P.nVals) * q);
+		g.bytes = 0;
+		if(upload(g, cols.data(), sizeof(int32_t) * (size_t) q, (const void**) &g.d.cols) || upload_dict(g)) { cla_block_free(c); return nullptr; }
+		g.bytes = pg.bytes; // what a kernel streams for this group
+		g.d.tblOff = tblOff;
+		g.d.colOff = colOff;
+		tblOff += P.nVals;
+		colOff += q;
+		maxVals = std::max(maxVals, P.nVals);
+		if(P.type == G_SDCZ) c->hasSdc = true;
+		if(P.type == G_RLE) c->hasRle = true;
+	}
+	if(b->hasConst) {
+		for(int j = 0; j < q; j++) c->constV[j] = T[(size_t) b->totalVals * q + j];
+		c->hasConst = true;
+	}
+	c->totalVals = tblOff;
+	c->totalColsG = colOff;
+	c->maxVals = maxVals;
+	c->parent = b;
+	b->refs.fetch_add(1);
+	if(finish_finalize(c, b)) { cla_block_free(c); return nullptr; }
+	return c;
 }
 
 int64_t cla_aggregate_dev(cla_handle b, int32_t op, int32_t dir, double* dOut) {

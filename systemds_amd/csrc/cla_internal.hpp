@@ -5,6 +5,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <mutex>
+#include <atomic>
 #include <string>
 #include <vector>
 
@@ -71,6 +72,12 @@ struct cla_block {
 	int64_t nRows = 0;
 	int32_t nCols = 0;
 	bool finalized = false;
+	// A block made by cla_rmm_overlapping borrows the code streams, offset lists, run tables
+	// and the code arena of the block it came from: it holds a reference on that block, which
+	// is only torn down when the last reference goes.
+	cla_block* parent = nullptr;
+	std::atomic<int> refs{1};
+	bool arenaShared = false;
 	std::vector<cla::HostGroup> groups;
 	std::vector<double> constV;      // filtered constants (SDC defaults, const groups), nCols
 	bool hasConst = false;
@@ -145,6 +152,7 @@ int launch_validate_codes(cla_block* b, const void* codes, int width, int64_t n,
 int launch_counts(cla_block* b, int group, int32_t* dCounts);
 int launch_sdc_build(cla_block* b, HostGroup& g);
 int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned long long* dNnz, int squares = 0);
+int launch_tables(cla_block* b, const double* dB, int q); // dict x B of every group (+ constV x B) into b->dTables
 int launch_aggregate(cla_block* b, int op, int dir, double* dOut, unsigned long long* dNnz);
 int ensure_counts(cla_block* b);
 int launch_rmm_mfma(cla_block* b, const double* dB, int q, const double* dConstRow, double* dOut,

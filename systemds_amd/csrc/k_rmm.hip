@@ -495,6 +495,21 @@ __global__ __launch_bounds__(256) void k_count_nnz(const double* __restrict__ x,
 	count_add(nnz, cnt);
 }
 
+// K1 alone: T_g = dict_g x B[cols_g, :] for every group, constV x B in row totalVals.
+int launch_tables(cla_block* b, const double* dB, int q) {
+	const int nG = (int) b->groups.size();
+	clear_stats(b);
+	int rc = ensure_tables(b, (size_t) (b->totalVals + 1) * q);
+	if(rc) return rc;
+	const int maxWork = (b->maxVals > 1 ? b->maxVals : 1) * q;
+	dim3 grid((maxWork + 255) / 256 > (q + 255) / 256 ? (maxWork + 255) / 256 : (q + 255) / 256, nG + 1);
+	Prof pf(b, "k_preagg", (long) grid.x * grid.y, 256, 0, 0);
+	hipLaunchKernelGGL(k_preagg, grid, dim3(256), 0, b->stream, b->dGroups, nG, dB, q, b->nCols,
+		b->hasConst ? b->dConstV : nullptr, b->dTables, b->totalVals, b->dCounters, nullptr, 0);
+	CLA_HIP(hipGetLastError());
+	return 0;
+}
+
 // squares != 0 (q == 1, no uncompressed group): the tables hold the sum of squares of each tuple
 // instead of dict x B, so that the gather yields rowSums(X^2).
 int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned long long* dNnz, int squares) {

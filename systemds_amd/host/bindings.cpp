@@ -168,6 +168,7 @@ PYBIND11_MODULE(_clahost, m) {
 		.def("isOverlapping", &CompressedMatrixBlock::isOverlapping)
 		.def("setOverlapping", &CompressedMatrixBlock::setOverlapping)
 		.def("releaseDevice", &CompressedMatrixBlock::releaseDevice)
+		.def("isDeviceOnly", &CompressedMatrixBlock::isDeviceOnly)
 		.def("decompress", &CompressedMatrixBlock::decompress, py::arg("k") = 1)
 		.def("aggregateBinaryOperations", &CompressedMatrixBlock::aggregateBinaryOperations, py::arg("m1"), py::arg("m2"), py::arg("k") = 1,
 			py::arg("transposeLeft") = false, py::arg("transposeRight") = false)
@@ -179,6 +180,7 @@ PYBIND11_MODULE(_clahost, m) {
 	py::class_<CLALibRightMultBy>(m, "CLALibRightMultBy")
 		.def_static("rightMultByMatrix", &CLALibRightMultBy::rightMultByMatrix, py::arg("m1"), py::arg("m2"), py::arg("k") = 1,
 			py::arg("allowOverlap") = false);
+	m.def("rightMultByMatrixOverlapping", &rightMultByMatrixOverlapping, py::arg("m1"), py::arg("m2"), py::arg("k") = 1);
 	py::class_<CLALibLeftMultBy>(m, "CLALibLeftMultBy")
 		.def_static("leftMultByMatrix", &CLALibLeftMultBy::leftMultByMatrix, py::arg("right"), py::arg("left"), py::arg("k") = 1)
 		.def_static("leftMultByMatrixTransposed", &CLALibLeftMultBy::leftMultByMatrixTransposed, py::arg("right"), py::arg("left"), py::arg("k") = 1);

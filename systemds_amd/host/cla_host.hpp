@@ -565,8 +565,19 @@ public:
 	bool isCompressed() const override { return true; }
 
 	// CompressedMatrixBlock.allocateColGroupList / allocateColGroup
+	// A block that lives on the device only: the overlapping result of a right multiply. It has
+	// no host-side column groups; every linear operation of this class works on it.
+	static std::shared_ptr<CompressedMatrixBlock> adoptDevice(int rl, int cl, cla_handle h) {
+		auto r = std::make_shared<CompressedMatrixBlock>(rl, cl);
+		r->handle = h;
+		r->deviceOnly = true;
+		r->overlappingColGroups = true;
+		return r;
+	}
+	bool isDeviceOnly() const { return deviceOnly; }
 	void allocateColGroupList(std::vector<AColGroupPtr> groups) {
 		releaseDevice();
+		deviceOnly = false;
 		for(const auto& g : groups) {
 			if(g == nullptr) throw DMLCompressionException("Invalid null column group");
 			for(int c : g->getColIndices())
@@ -576,9 +587,10 @@ public:
 	}
 	void allocateColGroup(AColGroupPtr g) { allocateColGroupList({std::move(g)}); }
 	const std::vector<AColGroupPtr>& getColGroups() const { return colGroups; }
-	bool isOverlapping() const { return colGroups.size() != 1 && overlappingColGroups; }
+	bool isOverlapping() const { return (deviceOnly || colGroups.size() != 1) && overlappingColGroups; }
 	void setOverlapping(bool o) { overlappingColGroups = o; }
 	bool isEmpty() const override {
+		if(deviceOnly) return rlen == 0 || clen == 0;
 		if(rlen == 0 || clen == 0 || colGroups.empty()) return true;
 		for(const auto& g : colGroups)
 			if(g->getCompType() != CompressionType::EMPTY) return false;
@@ -615,6 +627,7 @@ public:
 private:
 	std::vector<AColGroupPtr> colGroups;
 	bool overlappingColGroups = false;
+	bool deviceOnly = false;
 	cla_handle handle = nullptr;
 };
 
@@ -660,7 +673,7 @@ struct CLALibRightMultBy {
 				throw DMLRuntimeException("Dimensions do not match for matrix multiplication (" + std::to_string(m1.getNumColumns()) +
 					"!=" + std::to_string(m2.getNumRows()) + ").");
 			if(m1.isEmpty() || m2.isEmpty()) return MatrixBlock(rr, rc);
-			if(allowOverlap) throw NotImplementedException("Overlapping compressed output of the right multiply");
+			if(allowOverlap) throw NotImplementedException("a compressed result cannot be returned by value: use rightMultByMatrixOverlapping");
 			MatrixBlock dense2;
 			MatrixBlock* rhs = &m2;
 			if(m2.isCompressed()) {
@@ -677,6 +690,23 @@ struct CLALibRightMultBy {
 		}
 	}
 };
+
+// The allowOverlap = true branch of rightMultByMatrix (RMMOverlapping, CLALibRightMultBy.java:157-201):
+// the product stays compressed, its groups share the index structures of m1's groups.
+inline std::shared_ptr<CompressedMatrixBlock> rightMultByMatrixOverlapping(CompressedMatrixBlock& m1, MatrixBlock& m2, int k) {
+	if(m1.getNumColumns() != m2.getNumRows())
+		throw DMLRuntimeException("Dimensions do not match for matrix multiplication (" + std::to_string(m1.getNumColumns()) + "!=" +
+			std::to_string(m2.getNumRows()) + ").");
+	MatrixBlock dense2;
+	MatrixBlock* rhs = &m2;
+	if(m2.isCompressed()) {
+		dense2 = CLALibDecompress::decompress(static_cast<CompressedMatrixBlock&>(m2), k);
+		rhs = &dense2;
+	}
+	cla_handle h = cla_rmm_overlapping(m1.hipHandle(), rhs->getDenseBlockValues(), m2.getNumColumns());
+	if(h == nullptr) throw NotImplementedException(std::string("RMMOverlapping: ") + cla_last_error());
+	return CompressedMatrixBlock::adoptDevice(m1.getNumRows(), m2.getNumColumns(), h);
+}
 
 struct CLALibLeftMultBy {
 	// ret = left %*% right

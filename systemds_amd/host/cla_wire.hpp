@@ -502,6 +502,7 @@ inline std::shared_ptr<CompressedMatrixBlock> readCompressedMatrixBlock(const ui
 }
 
 inline std::vector<uint8_t> writeCompressedMatrixBlock(const CompressedMatrixBlock& cmb) {
+	if(cmb.isDeviceOnly()) throw NotImplementedException("a device-only block has no host-side column groups to serialise");
 	DataOutput out;
 	out.writeInt(cmb.getNumRows());
 	out.writeInt(cmb.getNumColumns());

@@ -163,3 +163,29 @@ def test_serialised_block_goes_straight_to_the_device(H, ora, cla, seed, n_rows)
     close(mm(cmb, H.MatrixBlock(B), 4).toArray(), D, B, "X %*% B from bytes", ora)
     close(mm(H.MatrixBlock(Y), cmb, 4).toArray(), Y, D, "Y %*% X from bytes", ora)
     close(cmb.transposeSelfMatrixMultOperations(H.MMTSJType.LEFT, 4).toArray(), D.T, D, "t(X) %*% X from bytes", ora)
+
+
+def test_overlapping_right_multiply_stays_compressed(H, ora, cla):
+    """rightMultByMatrix with allowOverlap (RMMOverlapping, CLALibRightMultBy.java:157-201): the product is a
+    compressed block again and feeds the next multiplies without ever being decompressed."""
+    n_rows = 30000
+    cmb, D, _ = build(H, ora, 8, n_rows, with_unc=False)
+    rng = np.random.default_rng(8)
+    B = rng.standard_normal((D.shape[1], 4))
+    xb = H.rightMultByMatrixOverlapping(cmb, H.MatrixBlock(B), 4)
+    assert xb.isCompressed() and xb.isOverlapping() and xb.isDeviceOnly()
+    assert (xb.getNumRows(), xb.getNumColumns()) == (n_rows, 4)
+    P = ora.longdouble_matmul(D, B)
+    absP = np.abs(D) @ np.abs(B)
+    assert_fp64_close(xb.decompress(4).toArray(), P, absP, what="decompress(XB)")
+    C = rng.standard_normal((4, 3))
+    mm = H.CLALibMatrixMult.matrixMultiply
+    assert_fp64_close(mm(xb, H.MatrixBlock(C), 4).toArray(), ora.longdouble_matmul(P, C), absP @ np.abs(C), what="(XB) %*% C")
+    Y = rng.standard_normal((2, n_rows))
+    assert_fp64_close(mm(H.MatrixBlock(Y), xb, 4).toArray(), ora.longdouble_matmul(Y, P), np.abs(Y) @ absP, what="Y %*% (XB)")
+    with pytest.raises(H.NotImplementedException):
+        xb.transposeSelfMatrixMultOperations(H.MMTSJType.LEFT, 4)
+    with pytest.raises(H.NotImplementedException):
+        H.writeCompressedMatrixBlock(xb)
+    with pytest.raises(H.NotImplementedException):   # by-value result cannot be compressed
+        H.CLALibRightMultBy.rightMultByMatrix(cmb, H.MatrixBlock(B), 4, True)

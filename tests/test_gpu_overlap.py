@@ -1,0 +1,79 @@
+"""GPU parity of the overlapping right multiply (cla_rmm_overlapping): X %*% B kept compressed
+with shared index structures, as RMMOverlapping does (C/lib/CLALibRightMultBy.java:157-201).
+The returned block must behave like the dense product D %*% B under every linear entry point."""
+import numpy as np
+import pytest
+
+from conftest import mixed_block
+from parity import assert_fp64_close
+
+pytestmark = pytest.mark.gpu
+
+
+def check_child(ora, child, P, absP, rng, what):
+    n_rows, q = P.shape
+    out, nnz = child.decompress()
+    assert_fp64_close(out, P, absP, what=f"{what}: decompress")
+    C = rng.standard_normal((q, 3))
+    out, _ = child.rmm(C)
+    assert_fp64_close(out, ora.longdouble_matmul(P, C), absP @ np.abs(C), what=f"{what}: (XB) %*% C")
+    v = rng.standard_normal((q, 1))
+    out, _ = child.rmm(v)
+    assert_fp64_close(out, ora.longdouble_matmul(P, v), absP @ np.abs(v), what=f"{what}: (XB) %*% v")
+    Y = rng.standard_normal((2, n_rows))
+    out, _ = child.lmm(Y)
+    assert_fp64_close(out, ora.longdouble_matmul(Y, P), np.abs(Y) @ absP, what=f"{what}: Y %*% (XB)")
+    out, _ = child.aggregate("sum", "col")
+    assert_fp64_close(out, P.astype(np.longdouble).sum(axis=0).astype(np.float64), absP.sum(axis=0), what=f"{what}: colSums")
+    out, _ = child.aggregate("sum", "row")
+    assert_fp64_close(out, P.astype(np.longdouble).sum(axis=1).astype(np.float64), absP.sum(axis=1), what=f"{what}: rowSums")
+
+
+@pytest.mark.parametrize("seed,n_rows,q", [(1, 37, 1), (2, 3000, 4), (3, 70001, 7)])
+def test_mixed_groups(cla, ora, seed, n_rows, q):
+    specs, n_cols = mixed_block(seed, n_rows, with_unc=False)
+    D = ora.np_decompress(specs, n_rows, n_cols)
+    rng = np.random.default_rng(seed)
+    B = rng.standard_normal((n_cols, q))
+    blk = cla.build_block(n_rows, n_cols, specs)
+    child = blk.rmm_overlapping(B)
+    blk.close()   # the child keeps the borrowed device copies alive
+    P = ora.longdouble_matmul(D, B)
+    check_child(ora, child, P, np.abs(D) @ np.abs(B), rng, "mixed")
+    with pytest.raises(cla.ClaError) as e:   # not linear in the groups
+        child.tsmm()
+    assert e.value.code == cla.ERR_UNSUPPORTED
+    with pytest.raises(cla.ClaError) as e:
+        child.aggregate("max", "col")
+    assert e.value.code == cla.ERR_UNSUPPORTED
+    grand = child.rmm_overlapping(rng.standard_normal((q, 2)))   # and again, from the overlapping block
+    child.close()
+    out, _ = grand.decompress()
+    assert out.shape == (n_rows, 2)
+    grand.close()
+
+
+def test_arena_block_shares_the_arena(cla, ora):
+    """All-DDC byte-code block (C2-shaped): the result keeps using the source block's code arena."""
+    from systemds_amd import synth
+    c = synth.config2(scale=200)
+    n_rows, n_cols = c["n_rows"], c["n_cols"]
+    D = ora.np_decompress(c["groups"], n_rows, n_cols)
+    rng = np.random.default_rng(0)
+    B = rng.standard_normal((n_cols, 5))
+    blk = cla.build_block(n_rows, n_cols, c["groups"])
+    child = blk.rmm_overlapping(B)
+    P = ora.longdouble_matmul(D, B)
+    check_child(ora, child, P, np.abs(D) @ np.abs(B), rng, "C2")
+    out, _ = blk.rmm(B)                       # the source block is untouched
+    assert_fp64_close(out, P, np.abs(D) @ np.abs(B), what="source block after")
+    child.close()
+    blk.close()
+
+
+def test_uncompressed_groups_are_refused(cla, ora):
+    specs, n_cols = mixed_block(4, 500, with_unc=True)
+    blk = cla.build_block(500, n_cols, specs)
+    with pytest.raises(cla.ClaError):
+        blk.rmm_overlapping(np.ones((n_cols, 2)))
+    blk.close()
