@@ -123,6 +123,7 @@ struct cla_block {
 	// list of SDCZeros groups + prefix sums of their nVals, as the row-tile kernels read it;
 	// built on first use for all groups (sdcPlanGroup -1) or for one group (its index)
 	int32_t* dSdcPlan = nullptr;
+	void* dSdcDesc = nullptr;        // one compact descriptor per listed group (k_rmm_sdc_pipe)
 	int sdcPlanGroup = -2;
 	std::vector<int32_t> sdcList, sdcBinOff;
 	unsigned long long* dCounters = nullptr;   // 8 x u64

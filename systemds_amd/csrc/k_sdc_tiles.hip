@@ -142,11 +142,212 @@ __global__ __launch_bounds__(ST_THREADS) void k_rmm_sdc_tiles(const DGroup* __re
 	count_add(nnz, cnt);
 }
 
+// What a list walk needs of a group, in one 48-byte read.
+struct SdcDesc {
+	const void* deltas;
+	const void* codes;
+	const OffState* tileIdx;
+	int32_t nDeltas, nOffsets, first, tblOff, nTiles;
+	int32_t widths; // delta width | code width << 8
+	int32_t nVals, pad;
+};
+
+// Bytes p[i .. i + 3] of a byte array of n entries as one word (bytes at and beyond n read as
+// 0): two aligned word loads and a byte alignment instead of four byte loads. The array starts
+// on a word boundary (device allocations do); words are read only where they lie inside it.
+__device__ __forceinline__ uint32_t sdc_load4(const uint8_t* p, int i, int n) {
+	if(i >= n) return 0;
+	const int a = i & ~3;
+	const uint32_t* w = (const uint32_t*) (p + a);
+	uint32_t lo, hi = 0;
+	if(a + 4 <= n) lo = w[0];
+	else {
+		lo = 0;
+		for(int k = 0; a + k < n; k++) lo |= (uint32_t) p[a + k] << (8 * k);
+	}
+	if((i & 3) != 0 && a + 4 < n) {
+		if(a + 8 <= n) hi = w[1];
+		else
+			for(int k = 0; a + 4 + k < n; k++) hi |= (uint32_t) p[a + 4 + k] << (8 * k);
+	}
+	return __builtin_amdgcn_alignbyte(hi, lo, i & 3);
+}
+
+template <class T>
+__device__ __forceinline__ T bcast_lane(T v, int l) {
+	static_assert(sizeof(T) == 4 || sizeof(T) == 8, "readlane moves 32-bit pieces");
+	if(sizeof(T) == 4) {
+		int x;
+		__builtin_memcpy(&x, &v, 4);
+		x = __builtin_amdgcn_readlane(x, l);
+		__builtin_memcpy(&v, &x, 4);
+	}
+	else {
+		int x[2];
+		__builtin_memcpy(x, &v, 8);
+		x[0] = __builtin_amdgcn_readlane(x[0], l);
+		x[1] = __builtin_amdgcn_readlane(x[1], l);
+		__builtin_memcpy(&v, x, 8);
+	}
+	return v;
+}
+
+// ---------------------------------------------------------------------------
+// Right multiply with one output column, software-pipelined list walks. A wave owns the
+// groups l = wave, wave + 8, ... of the list; lane t keeps the descriptor and the tile state
+// of the wave's task t, so one round of loads per tile serves all tasks. The task loop then
+// runs three stages on consecutive tasks: (A) request the 256 delta entries and, at the same
+// positions, the 256 codes behind the tile state of task t; (B) decode task t - 1 from
+// registers and request its table values; (C) add task t - 2 into the output tile. Every wait
+// is for loads issued one iteration earlier, which the other waves of the CU cover. Codes sit
+// at the positions of their entries as long as the 256 entries hold no skip entry (a 0); a
+// task with one, or with more than 256 entries in the tile, takes the plain walk.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(ST_THREADS) void k_rmm_sdc_pipe(const SdcDesc* __restrict__ desc, int nL,
+	const double* __restrict__ T, int constRow, int accumulate, double* __restrict__ out, int64_t nRows,
+	unsigned long long* __restrict__ nnz) {
+	extern __shared__ double otile[]; // ST
+	const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+	const int64_t r0 = (int64_t) blockIdx.x * ST, rEnd = r0 + ST;
+	const int nr = (int) min((int64_t) ST, nRows - r0);
+	for(int t = tid; t < ST; t += ST_THREADS) {
+		double v = 0.0;
+		if(t < nr) v = accumulate ? out[r0 + t] : (constRow >= 0 ? T[constRow] : 0.0);
+		otile[t] = v;
+	}
+	__syncthreads();
+	const int nT = wave < nL ? (nL - wave + ST_THREADS / 64 - 1) / (ST_THREADS / 64) : 0;
+	const int ti = (int) (r0 / SDC_TILE);
+	for(int t0 = 0; t0 < nT; t0 += 64) {
+		const int nHere = min(64, nT - t0);
+		// lane t: descriptor and tile state of task t0 + t
+		SdcDesc D;
+		D.deltas = nullptr; D.codes = nullptr; D.tileIdx = nullptr;
+		D.nDeltas = 0; D.nOffsets = 0; D.first = -1; D.tblOff = 0; D.nTiles = 0; D.widths = 0x101; D.nVals = 0; D.pad = 0;
+		OffState st;
+		st.idx = 0; st.emit = 0; st.row = 0; st.pad = 0;
+		if(lane < nHere) {
+			D = desc[wave + (ST_THREADS / 64) * (t0 + lane)];
+			if(ti < D.nTiles) st = as_global(D.tileIdx)[ti];
+			else st.idx = D.nDeltas; // no entries behind this tile
+		}
+		// pipeline registers
+		int dvA[4] = {-1, -1, -1, -1}, cvA[4] = {0, 0, 0, 0};     // stage A -> B
+		double tblA = 0.0;                                        // table entry `lane` of the group (groups of at most 64 tuples)
+		int rowsC[4] = {0, 0, 0, 0};                              // stage B -> C
+		double tvC[4] = {0.0, 0.0, 0.0, 0.0};
+		unsigned maskC = 0;
+		for(int t = 0; t < nHere + 2; t++) {
+			// ---- stage B inputs are last iteration's A outputs
+			int dvB[4], cvB[4];
+#pragma unroll
+			for(int k = 0; k < 4; k++) { dvB[k] = dvA[k]; cvB[k] = cvA[k]; }
+			const double tblB = tblA;
+			// ---- stage A: task t
+			if(t < nHere) {
+				const uint8_t* dptr = (const uint8_t*) as_global(bcast_lane(D.deltas, t));
+				const uint8_t* cptr = (const uint8_t*) as_global(bcast_lane(D.codes, t));
+				const int nDel = bcast_lane(D.nDeltas, t), nOff = bcast_lane(D.nOffsets, t), w = bcast_lane(D.widths, t);
+				const int i = bcast_lane(st.idx, t) + lane * 4, e = bcast_lane(st.emit, t) + lane * 4;
+				const int dw = w & 0xff, cw = w >> 8;
+				const int nv = bcast_lane(D.nVals, t);
+				tblA = nv <= 64 && lane < nv ? T[bcast_lane(D.tblOff, t) + lane] : 0.0;
+				if(dw == 1 && cw == 1) {
+					// byte lists: the lane's four entries as the two aligned words around them
+					uint32_t dq = sdc_load4(dptr, i, nDel), cq = sdc_load4(cptr, e, nOff);
+#pragma unroll
+					for(int k = 0; k < 4; k++) {
+						dvA[k] = i + k < nDel ? (int) ((dq >> (8 * k)) & 0xff) : -1;
+						cvA[k] = (int) ((cq >> (8 * k)) & 0xff);
+					}
+				}
+				else {
+#pragma unroll
+					for(int k = 0; k < 4; k++) {
+						dvA[k] = i + k < nDel ? (dw == 1 ? (int) dptr[i + k] : (int) ((const uint16_t*) dptr)[i + k]) : -1;
+						cvA[k] = e + k < nOff ? load_code(cptr, cw, e + k) : 0;
+					}
+				}
+			}
+			// ---- stage C: task t - 2
+			if(t >= 2) {
+#pragma unroll
+				for(int k = 0; k < 4; k++)
+					if(maskC & (1u << k)) unsafeAtomicAdd(&otile[rowsC[k]], tvC[k]);
+			}
+			maskC = 0;
+			// ---- stage B: task t - 1
+			if(t >= 1 && t - 1 < nHere) {
+				const int tb = t - 1;
+				const int w = bcast_lane(D.widths, tb), tblOff = bcast_lane(D.tblOff, tb), nDel = bcast_lane(D.nDeltas, tb);
+				const int dw = w & 0xff, cw = w >> 8, maxV = dw == 1 ? 255 : 65535;
+				const int i0 = bcast_lane(st.idx, tb);
+				int row = bcast_lane(st.row, tb), emit = bcast_lane(st.emit, tb);
+				const int first = bcast_lane(D.first, tb);
+				const uint8_t* cptr = (const uint8_t*) as_global(bcast_lane(D.codes, tb));
+				const double* tg = T + tblOff;
+				const bool inRegs = bcast_lane(D.nVals, tb) <= 64; // table in registers: lookups by lane permute
+				if(lane == 0 && first >= r0 && first < rEnd) unsafeAtomicAdd(&otile[first - r0], tg[load_code(cptr, cw, 0)]);
+				// decode the 256 entries from registers (the arithmetic of sdc_decode256)
+				int s = 0, c = 0, rows[4], didx[4];
+				unsigned mask = 0;
+				bool zero = false;
+#pragma unroll
+				for(int k = 0; k < 4; k++) {
+					const int v = dvB[k];
+					zero |= v == 0;
+					s += v < 0 ? 0 : (v == 0 ? maxV : v);
+					rows[k] = s;
+					didx[k] = c;
+					if(v > 0) { mask |= 1u << k; c++; }
+				}
+				const int ps = wave_scan_incl(s), pc = wave_scan_incl(c);
+#pragma unroll
+				for(int k = 0; k < 4; k++) { rows[k] += row + ps - s; didx[k] += emit + pc - c; }
+				row += __builtin_amdgcn_readlane(ps, 63);
+				emit += __builtin_amdgcn_readlane(pc, 63);
+				const bool plain = __ballot(zero) != 0; // a skip entry shifts the codes against the entries
+#pragma unroll
+				for(int k = 0; k < 4; k++) {
+					const bool on = (mask & (1u << k)) && rows[k] < rEnd;
+					const int code = plain ? (on ? load_code(cptr, cw, didx[k]) : 0) : cvB[k];
+					rowsC[k] = (int) (rows[k] - r0);
+					const double tv = inRegs ? __shfl(tblB, code & 63, 64) : (on ? tg[code] : 0.0);
+					tvC[k] = on ? tv : 0.0;
+					if(on) maskC |= 1u << k;
+				}
+				// more than 256 entries of this group in the tile: the plain walk finishes it
+				int64_t j0 = (int64_t) i0 + 256;
+				const void* dptr = as_global(bcast_lane(D.deltas, tb));
+				while(j0 < nDel && row < rEnd) {
+					int32_t rws[4], dix[4];
+					unsigned m;
+					if(dw == 1) sdc_decode256<1>(dptr, nDel, j0, row, emit, rws, dix, m);
+					else sdc_decode256<2>(dptr, nDel, j0, row, emit, rws, dix, m);
+#pragma unroll
+					for(int k = 0; k < 4; k++)
+						if((m & (1u << k)) && rws[k] < rEnd) unsafeAtomicAdd(&otile[rws[k] - r0], tg[load_code(cptr, cw, dix[k])]);
+					j0 += 256;
+				}
+			}
+		}
+	}
+	__syncthreads();
+	int cnt = 0;
+	for(int t = tid; t < nr; t += ST_THREADS) {
+		const double v = otile[t];
+		cnt += v != 0.0;
+		out[r0 + t] = v;
+	}
+	count_add(nnz, cnt);
+}
+
 // Host side: list of SDCZeros groups and the prefix sums of their nVals, kept on the block
 // (host and device copy) and rebuilt only when the requested group selection changes.
 static int sdc_plan(cla_block* b, int onlyGroup, int32_t** dList, int32_t** dBinOff) {
 	const size_t nG = b->groups.size();
 	if(b->dSdcPlan == nullptr) CLA_HIP(hipMalloc((void**) &b->dSdcPlan, (2 * nG + 2) * sizeof(int32_t)));
+	if(b->dSdcDesc == nullptr) CLA_HIP(hipMalloc(&b->dSdcDesc, std::max<size_t>(nG, 1) * sizeof(SdcDesc)));
 	if(b->sdcPlanGroup != onlyGroup) {
 		b->sdcList.clear();
 		b->sdcBinOff.assign(1, 0);
@@ -157,7 +358,18 @@ static int sdc_plan(cla_block* b, int onlyGroup, int32_t** dList, int32_t** dBin
 			b->sdcBinOff.push_back(b->sdcBinOff.back() + G.nVals);
 		}
 		b->sdcPlanGroup = -2; // invalid until both copies have been issued
+		std::vector<SdcDesc> descs;
+		for(int g : b->sdcList) {
+			const DGroup& G = b->groups[g].d;
+			SdcDesc d;
+			d.deltas = G.deltas; d.codes = G.codes; d.tileIdx = G.tileIdx;
+			d.nDeltas = (int32_t) G.nDeltas; d.nOffsets = (int32_t) G.nOffsets; d.first = G.first; d.tblOff = G.tblOff; d.nTiles = G.nTiles;
+			d.widths = G.deltaWidth | (G.codeWidth << 8);
+			d.nVals = G.nVals; d.pad = 0;
+			descs.push_back(d);
+		}
 		if(!b->sdcList.empty()) {
+			CLA_HIP(hipMemcpyAsync(b->dSdcDesc, descs.data(), descs.size() * sizeof(SdcDesc), hipMemcpyHostToDevice, b->stream));
 			CLA_HIP(hipMemcpyAsync(b->dSdcPlan, b->sdcList.data(), b->sdcList.size() * 4, hipMemcpyHostToDevice, b->stream));
 			CLA_HIP(hipMemcpyAsync(b->dSdcPlan + nG, b->sdcBinOff.data(), b->sdcBinOff.size() * 4, hipMemcpyHostToDevice, b->stream));
 			// the host vectors are rewritten by the next selection: the copies must have read them
@@ -254,7 +466,15 @@ int launch_rmm_sdc_tiles(cla_block* b, int q, int constRow, int accumulate, doub
 		const DGroup& G = b->groups[g].d;
 		algo += (double) G.nDeltas * G.deltaWidth + (double) G.nOffsets * G.codeWidth;
 	}
-	{
+	static const bool noPipe = getenv("CLA_RMM_SDC_NO_PIPE") != nullptr;
+	if(q == 1 && !ldsTables && tileRows == ST && !noPipe) {
+		const size_t ldsP = (size_t) ST * 8;
+		Prof pf(b, "k_rmm_sdc_pipe", nTiles, ST_THREADS, (long) ldsP, algo);
+		CLA_HIP(hipFuncSetAttribute((const void*) k_rmm_sdc_pipe, hipFuncAttributeMaxDynamicSharedMemorySize, (int) ldsP));
+		hipLaunchKernelGGL(k_rmm_sdc_pipe, dim3(nTiles), dim3(ST_THREADS), ldsP, b->stream, (const SdcDesc*) b->dSdcDesc,
+			(int) plan.list.size(), b->dTables, constRow, accumulate, dOut, b->nRows, dNnz);
+	}
+	else {
 		Prof pf(b, "k_rmm_sdc_tiles", nTiles, ST_THREADS, (long) lds, algo);
 		CLA_HIP(hipFuncSetAttribute((const void*) k_rmm_sdc_tiles, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
 		hipLaunchKernelGGL(k_rmm_sdc_tiles, dim3(nTiles), dim3(ST_THREADS), lds, b->stream, b->dGroups, dList, dBinOff,
