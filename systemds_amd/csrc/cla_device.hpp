@@ -1,6 +1,7 @@
 // Device-side helpers shared by the kernels (gfx950, wave64).
 #pragma once
 #include "cla_internal.hpp"
+#include <type_traits>
 
 namespace cla {
 
@@ -84,6 +85,34 @@ __device__ __forceinline__ int wave_scan_incl(int v) {
 	v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, false); // row_shr:8
 	v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false); // row_bcast:15
 	v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false); // row_bcast:31
+	return v;
+}
+
+// Sum over the 64 lanes of a wave (all lanes active), the same value in every lane: the scan
+// above on the two halves of a double, total read from the last lane.
+__device__ __forceinline__ double wave_sum_f64_all(double v) {
+	auto dpp = [](double x, auto ctrlTag, auto rowTag) {
+		constexpr int ctrl = decltype(ctrlTag)::value, rowMask = decltype(rowTag)::value;
+		int p[2];
+		__builtin_memcpy(p, &x, 8);
+		p[0] = __builtin_amdgcn_update_dpp(0, p[0], ctrl, rowMask, 0xf, false);
+		p[1] = __builtin_amdgcn_update_dpp(0, p[1], ctrl, rowMask, 0xf, false);
+		double r;
+		__builtin_memcpy(&r, p, 8);
+		return r;
+	};
+	using std::integral_constant;
+	v += dpp(v, integral_constant<int, 0x111>(), integral_constant<int, 0xf>());
+	v += dpp(v, integral_constant<int, 0x112>(), integral_constant<int, 0xf>());
+	v += dpp(v, integral_constant<int, 0x114>(), integral_constant<int, 0xf>());
+	v += dpp(v, integral_constant<int, 0x118>(), integral_constant<int, 0xf>());
+	v += dpp(v, integral_constant<int, 0x142>(), integral_constant<int, 0xa>());
+	v += dpp(v, integral_constant<int, 0x143>(), integral_constant<int, 0xc>());
+	int p[2];
+	__builtin_memcpy(p, &v, 8);
+	p[0] = __builtin_amdgcn_readlane(p[0], WAVE - 1);
+	p[1] = __builtin_amdgcn_readlane(p[1], WAVE - 1);
+	__builtin_memcpy(&v, p, 8);
 	return v;
 }
 

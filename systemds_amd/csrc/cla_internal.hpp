@@ -160,7 +160,7 @@ int launch_rmm_mfma(cla_block* b, const double* dB, int q, const double* dConstR
 	unsigned long long* dNnz);
 int launch_lmm_u8(cla_block* b, const double* dY, int p, double* dPre);
 int launch_lmm_u8_dot(cla_block* b, const double* dY, int p, double* dOut);
-int launch_lmm_sdc_tiles(cla_block* b, const double* dY, int p, double* dPre, int onlyGroup);
+int launch_lmm_sdc_tiles(cla_block* b, const double* dY, int p, double* dPre, int onlyGroup, double* dOut);
 int launch_rmm_sdc_tiles(cla_block* b, int q, int constRow, int accumulate, double* dOut, unsigned long long* dNnz);
 int launch_tsmm_decode(cla_block* b, double* dOut);
 int launch_rmm_decode(cla_block* b, const double* dB, int q, const double* dConstRow, double* dOut,

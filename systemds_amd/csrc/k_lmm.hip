@@ -187,7 +187,9 @@ __global__ __launch_bounds__(256) void k_lmm_finish(double* __restrict__ out, in
 	count_add(nnz, cnt);
 }
 
-static int run_preagg(cla_block* b, const double* dY, int p, double* dPre, int onlyGroup) {
+// dOut != nullptr (whole-block calls): groups whose products can be summed directly write into dOut
+// and leave their part of dPre zero.
+static int run_preagg(cla_block* b, const double* dY, int p, double* dPre, int onlyGroup, double* dOut) {
 	const int nG = (int) b->groups.size();
 	const int64_t nRows = b->nRows;
 	hipStream_t st = b->stream;
@@ -229,7 +231,7 @@ static int run_preagg(cla_block* b, const double* dY, int p, double* dPre, int o
 	// SDCZeros groups: all lists walked tile by tile with the Y tile in LDS; the
 	// per-group chunk kernel below only serves dictionaries too large for LDS bins
 	{
-		const int r = nRows > 0 ? launch_lmm_sdc_tiles(b, dY, p, dPre, onlyGroup) : 0;
+		const int r = nRows > 0 ? launch_lmm_sdc_tiles(b, dY, p, dPre, onlyGroup, dOut) : 0;
 		if(r < 0) return r;
 		if(r == 0) { CLA_HIP(hipGetLastError()); return 0; }
 	}
@@ -266,7 +268,7 @@ int launch_preagg(cla_block* b, int group, const double* dY, int p, double* dPre
 	int rc = ensure_tables(b, (size_t) p * b->totalVals);
 	if(rc) return rc;
 	CLA_HIP(hipMemsetAsync(b->dTables, 0, sizeof(double) * (size_t) p * b->totalVals, b->stream));
-	if((rc = run_preagg(b, dY, p, b->dTables, group))) return rc;
+	if((rc = run_preagg(b, dY, p, b->dTables, group, nullptr))) return rc;
 	CLA_HIP(hipMemcpy2DAsync(dPre, sizeof(double) * (size_t) G.nVals, b->dTables + G.tblOff,
 		sizeof(double) * (size_t) b->totalVals, sizeof(double) * (size_t) G.nVals, (size_t) p, hipMemcpyDeviceToDevice,
 		b->stream));
@@ -288,7 +290,7 @@ int launch_lmm(cla_block* b, const double* dY, int p, double* dOut, unsigned lon
 	// single-column DDC groups on byte codes: contributions go straight into dOut
 	const int dot = nRows > 0 ? launch_lmm_u8_dot(b, dY, p, dOut) : 1;
 	if(dot < 0) return dot;
-	if(dot != 0 && (rc = run_preagg(b, dY, p, dPre, -1))) return rc;
+	if(dot != 0 && (rc = run_preagg(b, dY, p, dPre, -1, dOut))) return rc;
 
 	int64_t rowsPerBlock = 256 * 1024;
 	while(rowsPerBlock > 8192 && (nRows + rowsPerBlock - 1) / rowsPerBlock * p < (int64_t) g_numCU * 2) rowsPerBlock /= 2;

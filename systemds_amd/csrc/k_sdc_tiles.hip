@@ -149,7 +149,8 @@ struct SdcDesc {
 	const OffState* tileIdx;
 	int32_t nDeltas, nOffsets, first, tblOff, nTiles;
 	int32_t widths; // delta width | code width << 8
-	int32_t nVals, pad;
+	int32_t nVals, col0; // col0: the column of a single-column group
+	const double* dict;
 };
 
 // Bytes p[i .. i + 3] of a byte array of n entries as one word (bytes at and beyond n read as
@@ -223,7 +224,7 @@ __global__ __launch_bounds__(ST_THREADS) void k_rmm_sdc_pipe(const SdcDesc* __re
 		// lane t: descriptor and tile state of task t0 + t
 		SdcDesc D;
 		D.deltas = nullptr; D.codes = nullptr; D.tileIdx = nullptr;
-		D.nDeltas = 0; D.nOffsets = 0; D.first = -1; D.tblOff = 0; D.nTiles = 0; D.widths = 0x101; D.nVals = 0; D.pad = 0;
+		D.nDeltas = 0; D.nOffsets = 0; D.first = -1; D.tblOff = 0; D.nTiles = 0; D.widths = 0x101; D.nVals = 0; D.col0 = 0; D.dict = nullptr;
 		OffState st;
 		st.idx = 0; st.emit = 0; st.row = 0; st.pad = 0;
 		if(lane < nHere) {
@@ -342,6 +343,141 @@ __global__ __launch_bounds__(ST_THREADS) void k_rmm_sdc_pipe(const SdcDesc* __re
 	count_add(nnz, cnt);
 }
 
+// ---------------------------------------------------------------------------
+// Left multiply for lists of single-column groups with at most 64 tuples, in the same
+// pipeline: the group's dictionary sits in registers (entry `lane`), every entry contributes
+// Y[row] * dict[code] (row from the Y tile in LDS, dictionary value by lane permute), the wave
+// sums the products and lane t keeps the total of task t. No bins, no atomics in LDS, one
+// launch for all groups; the totals go straight into the output (no pre-aggregate).
+// block = (range of tiles, row i of Y).
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(ST_THREADS) void k_lmm_sdc_pipe(const SdcDesc* __restrict__ desc, int nL,
+	const double* __restrict__ Y, int64_t nRows, int tilesPerBlock,
+	double* __restrict__ out, int nCols) {
+	extern __shared__ double ytile[]; // ST
+	const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+	const int irow = blockIdx.y;
+	const double* y = Y + (size_t) irow * nRows;
+	const int nTilesAll = (int) ((nRows + ST - 1) / ST);
+	const int tile0 = blockIdx.x * tilesPerBlock, tile1 = min(tile0 + tilesPerBlock, nTilesAll);
+	const int nT = wave < nL ? (nL - wave + ST_THREADS / 64 - 1) / (ST_THREADS / 64) : 0;
+	const int nTmax = (nL + ST_THREADS / 64 - 1) / (ST_THREADS / 64); // the same trip count for every wave: barriers inside
+	for(int t0 = 0; t0 < max(nTmax, 1); t0 += 64) { // (at most 512 groups per pass over the tiles: one pass for C4)
+		const int nHere = max(0, min(64, nT - t0));
+		SdcDesc D;
+		D.deltas = nullptr; D.codes = nullptr; D.tileIdx = nullptr;
+		D.nDeltas = 0; D.nOffsets = 0; D.first = -1; D.tblOff = 0; D.nTiles = 0; D.widths = 0x101; D.nVals = 0; D.col0 = 0; D.dict = nullptr;
+		if(lane < nHere) D = desc[wave + (ST_THREADS / 64) * (t0 + lane)];
+		double accT = 0.0; // lane t: total of task t over the block's tiles
+		for(int tile = tile0; tile < tile1; tile++) {
+			const int64_t r0 = (int64_t) tile * ST, rEnd = r0 + ST;
+			__syncthreads(); // the previous tile's readers are done
+			for(int t = tid; t < ST; t += ST_THREADS) ytile[t] = r0 + t < nRows ? y[r0 + t] : 0.0;
+			__syncthreads();
+			const int ti = (int) (r0 / SDC_TILE);
+			OffState st;
+			st.idx = 0; st.emit = 0; st.row = 0; st.pad = 0;
+			if(lane < nHere) {
+				if(ti < D.nTiles) st = as_global(D.tileIdx)[ti];
+				else st.idx = D.nDeltas;
+			}
+			int dvA[4] = {-1, -1, -1, -1}, cvA[4] = {0, 0, 0, 0};
+			double dictA = 0.0;
+			for(int t = 0; t < nHere + 1; t++) {
+				int dvB[4], cvB[4];
+#pragma unroll
+				for(int k = 0; k < 4; k++) { dvB[k] = dvA[k]; cvB[k] = cvA[k]; }
+				const double dictB = dictA;
+				// ---- stage A: task t
+				if(t < nHere) {
+					const uint8_t* dptr = (const uint8_t*) as_global(bcast_lane(D.deltas, t));
+					const uint8_t* cptr = (const uint8_t*) as_global(bcast_lane(D.codes, t));
+					const int nDel = bcast_lane(D.nDeltas, t), nOff = bcast_lane(D.nOffsets, t), w = bcast_lane(D.widths, t);
+					const int i = bcast_lane(st.idx, t) + lane * 4, e = bcast_lane(st.emit, t) + lane * 4;
+					const int dw = w & 0xff, cw = w >> 8;
+					dictA = lane < bcast_lane(D.nVals, t) ? as_global(bcast_lane(D.dict, t))[lane] : 0.0;
+					if(dw == 1 && cw == 1) {
+						const uint32_t dq = sdc_load4(dptr, i, nDel), cq = sdc_load4(cptr, e, nOff);
+#pragma unroll
+						for(int k = 0; k < 4; k++) {
+							dvA[k] = i + k < nDel ? (int) ((dq >> (8 * k)) & 0xff) : -1;
+							cvA[k] = (int) ((cq >> (8 * k)) & 0xff);
+						}
+					}
+					else {
+#pragma unroll
+						for(int k = 0; k < 4; k++) {
+							dvA[k] = i + k < nDel ? (dw == 1 ? (int) dptr[i + k] : (int) ((const uint16_t*) dptr)[i + k]) : -1;
+							cvA[k] = e + k < nOff ? load_code(cptr, cw, e + k) : 0;
+						}
+					}
+				}
+				// ---- stage B: task t - 1
+				if(t >= 1) {
+					const int tb = t - 1;
+					const int w = bcast_lane(D.widths, tb), nDel = bcast_lane(D.nDeltas, tb);
+					const int dw = w & 0xff, cw = w >> 8, maxV = dw == 1 ? 255 : 65535;
+					const int i0 = bcast_lane(st.idx, tb);
+					int row = bcast_lane(st.row, tb), emit = bcast_lane(st.emit, tb);
+					const int first = bcast_lane(D.first, tb);
+					const uint8_t* cptr = (const uint8_t*) as_global(bcast_lane(D.codes, tb));
+					double part = 0.0;
+					{ // the list's first row is not among the delta entries
+						const bool has = first >= r0 && first < rEnd;
+						const int code0 = has ? load_code(cptr, cw, 0) : 0;
+						const double d0 = __shfl(dictB, code0 & 63, 64);
+						if(has && lane == 0) part = ytile[first - r0] * d0;
+					}
+					int s = 0, c = 0, rows[4], didx[4];
+					unsigned mask = 0;
+					bool zero = false;
+#pragma unroll
+					for(int k = 0; k < 4; k++) {
+						const int v = dvB[k];
+						zero |= v == 0;
+						s += v < 0 ? 0 : (v == 0 ? maxV : v);
+						rows[k] = s;
+						didx[k] = c;
+						if(v > 0) { mask |= 1u << k; c++; }
+					}
+					const int ps = wave_scan_incl(s), pc = wave_scan_incl(c);
+#pragma unroll
+					for(int k = 0; k < 4; k++) { rows[k] += row + ps - s; didx[k] += emit + pc - c; }
+					row += __builtin_amdgcn_readlane(ps, 63);
+					emit += __builtin_amdgcn_readlane(pc, 63);
+					const bool plain = __ballot(zero) != 0;
+#pragma unroll
+					for(int k = 0; k < 4; k++) {
+						const bool on = (mask & (1u << k)) && rows[k] < rEnd;
+						const int code = plain ? (on ? load_code(cptr, cw, didx[k]) : 0) : cvB[k];
+						const double d = __shfl(dictB, code & 63, 64);
+						if(on) part += ytile[rows[k] - r0] * d;
+					}
+					int64_t j0 = (int64_t) i0 + 256;
+					const void* dptr = as_global(bcast_lane(D.deltas, tb));
+					while(j0 < nDel && row < rEnd) { // more than 256 entries of this group in the tile
+						int32_t rws[4], dix[4];
+						unsigned m;
+						if(dw == 1) sdc_decode256<1>(dptr, nDel, j0, row, emit, rws, dix, m);
+						else sdc_decode256<2>(dptr, nDel, j0, row, emit, rws, dix, m);
+#pragma unroll
+						for(int k = 0; k < 4; k++) {
+							const bool on = (m & (1u << k)) && rws[k] < rEnd;
+							const int code = on ? load_code(cptr, cw, dix[k]) : 0;
+							const double d = __shfl(dictB, code & 63, 64);
+							if(on) part += ytile[rws[k] - r0] * d;
+						}
+						j0 += 256;
+					}
+					const double total = wave_sum_f64_all(part);
+					if(lane == tb) accT += total;
+				}
+			}
+		}
+		if(lane < nHere && accT != 0.0) unsafeAtomicAdd(&out[(size_t) irow * nCols + D.col0], accT);
+	}
+}
+
 // Host side: list of SDCZeros groups and the prefix sums of their nVals, kept on the block
 // (host and device copy) and rebuilt only when the requested group selection changes.
 static int sdc_plan(cla_block* b, int onlyGroup, int32_t** dList, int32_t** dBinOff) {
@@ -365,7 +501,7 @@ static int sdc_plan(cla_block* b, int onlyGroup, int32_t** dList, int32_t** dBin
 			d.deltas = G.deltas; d.codes = G.codes; d.tileIdx = G.tileIdx;
 			d.nDeltas = (int32_t) G.nDeltas; d.nOffsets = (int32_t) G.nOffsets; d.first = G.first; d.tblOff = G.tblOff; d.nTiles = G.nTiles;
 			d.widths = G.deltaWidth | (G.codeWidth << 8);
-			d.nVals = G.nVals; d.pad = 0;
+			d.nVals = G.nVals; d.col0 = b->groups[g].cols[0]; d.dict = G.dict;
 			descs.push_back(d);
 		}
 		if(!b->sdcList.empty()) {
@@ -383,12 +519,32 @@ static int sdc_plan(cla_block* b, int onlyGroup, int32_t** dList, int32_t** dBin
 }
 
 // Returns 1 if some SDC group cannot use the tile kernel (caller falls back), 0 when done.
-int launch_lmm_sdc_tiles(cla_block* b, const double* dY, int p, double* dPre, int onlyGroup) {
+int launch_lmm_sdc_tiles(cla_block* b, const double* dY, int p, double* dPre, int onlyGroup, double* dOut) {
 	int32_t *dList = nullptr, *dBinOff = nullptr;
 	int rc = sdc_plan(b, onlyGroup, &dList, &dBinOff);
 	if(rc) return rc;
 	struct { const std::vector<int32_t>&list, &binOff; } plan{b->sdcList, b->sdcBinOff};
 	if(plan.list.empty()) return 0;
+	// all listed groups single-column with at most 64 tuples, whole-block call: products straight
+	// into dOut, the groups' part of dPre stays zero
+	static const bool noPipe = getenv("CLA_LMM_SDC_NO_PIPE") != nullptr;
+	bool pipe = dOut != nullptr && onlyGroup < 0 && !noPipe;
+	for(int g : plan.list) pipe &= b->groups[g].d.nColG == 1 && b->groups[g].d.nVals <= 64;
+	if(pipe) {
+		const int nTiles = (int) ((b->nRows + ST - 1) / ST);
+		int tpb = std::max(1, (nTiles * p + 4 * g_numCU - 1) / (4 * g_numCU));
+		tpb = std::min(tpb, std::max(1, nTiles));
+		const unsigned grid = (unsigned) ((nTiles + tpb - 1) / tpb);
+		double algo = (double) b->nRows * 8 * p;
+		for(int g : plan.list) algo += (double) p * ((double) b->groups[g].d.nDeltas * b->groups[g].d.deltaWidth + (double) b->groups[g].d.nOffsets * b->groups[g].d.codeWidth);
+		const size_t lds = (size_t) ST * 8;
+		Prof pf(b, "k_lmm_sdc_pipe", (long) grid * p, ST_THREADS, (long) lds, algo);
+		CLA_HIP(hipFuncSetAttribute((const void*) k_lmm_sdc_pipe, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
+		hipLaunchKernelGGL(k_lmm_sdc_pipe, dim3(grid, p), dim3(ST_THREADS), lds, b->stream, (const SdcDesc*) b->dSdcDesc,
+			(int) plan.list.size(), dY, b->nRows, tpb, dOut, b->nCols);
+		CLA_HIP(hipGetLastError());
+		return 0;
+	}
 	const size_t ldsMax = (size_t) std::min(g_ldsPerBlock, 160 * 1024) - 2048;
 	// bins of a slab of groups next to the Y tile; small slabs keep LDS per block low
 	// enough for three blocks per CU, which hides the latency of the list walks
