@@ -146,7 +146,7 @@ def main():
                          "FETCH_SIZE / WRITE_SIZE against a kernel of known traffic")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py: this build runs on exactly one GPU (the path shards by rows, see DESIGN.md); "
+        print("bench.py: this build runs on exactly one GPU (the path shards by rows, each GPU taking a row range of every group); "
               f"--gpus {args.gpus} is not supported", file=sys.stderr)
         sys.exit(2)
 

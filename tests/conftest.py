@@ -10,7 +10,7 @@ if ROOT not in sys.path:
 
 
 def pytest_configure(config):
-    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with gpurun)")
+    config.addinivalue_line("markers", "gpu: needs a real MI355X")
 
 
 @pytest.fixture(scope="session")
