@@ -228,6 +228,7 @@ void cla_block_free(cla_handle b) {
 	if(b->dScratch) (void) hipFree(b->dScratch);
 	if(b->dSdcPlan) (void) hipFree(b->dSdcPlan);
 	if(b->dSdcDesc) (void) hipFree(b->dSdcDesc);
+	if(b->dSdcPacked) (void) hipFree(b->dSdcPacked);
 	if(b->dDictPad) (void) hipFree(b->dDictPad);
 	if(b->dCountsAll) (void) hipFree(b->dCountsAll);
 	if(b->dOnes) (void) hipFree(b->dOnes);

@@ -123,7 +123,8 @@ struct cla_block {
 	// list of SDCZeros groups + prefix sums of their nVals, as the row-tile kernels read it;
 	// built on first use for all groups (sdcPlanGroup -1) or for one group (its index)
 	int32_t* dSdcPlan = nullptr;
-	void* dSdcDesc = nullptr;        // one compact descriptor per listed group (k_rmm_sdc_pipe)
+	void* dSdcDesc = nullptr;        // one compact descriptor per listed group (k_*_sdc_packed)
+	uint32_t* dSdcPacked = nullptr;  // all listed groups' entries as (code << 16 | row inside its 4096-row tile), built on first use
 	int sdcPlanGroup = -2;
 	std::vector<int32_t> sdcList, sdcBinOff;
 	unsigned long long* dCounters = nullptr;   // 8 x u64

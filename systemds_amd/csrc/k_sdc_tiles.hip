@@ -5,6 +5,9 @@
 //
 //   k_lmm_sdc_tiles   bins[g][code] += Y[i, row] for every listed row (t(v) %*% X)
 //   k_rmm_sdc_tiles   out[row, :] += T_g[code, :] for every listed row (X %*% u); tables from L2
+//   k_sdc_pack        one-time rewrite of the lists into one word per entry (code, row in tile)
+//   k_rmm_sdc_packed  X %*% u on the packed lists, software-pipelined over a wave's groups
+//   k_lmm_sdc_packed  t(v) %*% X on the packed lists for single-column groups of <= 64 tuples
 //
 // A tile is ST = 4 * SDC_TILE rows; the iterator state in front of a tile comes
 // from the row-tile index built at finalize.
@@ -151,28 +154,8 @@ struct SdcDesc {
 	int32_t widths; // delta width | code width << 8
 	int32_t nVals, col0; // col0: the column of a single-column group
 	const double* dict;
+	const uint32_t* packed; // the group's entries as (code << 16 | row & 4095), in list order
 };
-
-// Bytes p[i .. i + 3] of a byte array of n entries as one word (bytes at and beyond n read as
-// 0): two aligned word loads and a byte alignment instead of four byte loads. The array starts
-// on a word boundary (device allocations do); words are read only where they lie inside it.
-__device__ __forceinline__ uint32_t sdc_load4(const uint8_t* p, int i, int n) {
-	if(i >= n) return 0;
-	const int a = i & ~3;
-	const uint32_t* w = (const uint32_t*) (p + a);
-	uint32_t lo, hi = 0;
-	if(a + 4 <= n) lo = w[0];
-	else {
-		lo = 0;
-		for(int k = 0; a + k < n; k++) lo |= (uint32_t) p[a + k] << (8 * k);
-	}
-	if((i & 3) != 0 && a + 4 < n) {
-		if(a + 8 <= n) hi = w[1];
-		else
-			for(int k = 0; a + 4 + k < n; k++) hi |= (uint32_t) p[a + 4 + k] << (8 * k);
-	}
-	return __builtin_amdgcn_alignbyte(hi, lo, i & 3);
-}
 
 template <class T>
 __device__ __forceinline__ T bcast_lane(T v, int l) {
@@ -194,22 +177,47 @@ __device__ __forceinline__ T bcast_lane(T v, int l) {
 }
 
 // ---------------------------------------------------------------------------
-// Right multiply with one output column, software-pipelined list walks. A wave owns the
-// groups l = wave, wave + 8, ... of the list; lane t keeps the descriptor and the tile state
-// of the wave's task t, so one round of loads per tile serves all tasks. The task loop then
-// runs three stages on consecutive tasks: (A) request the 256 delta entries and, at the same
-// positions, the 256 codes behind the tile state of task t; (B) decode task t - 1 from
-// registers and request its table values; (C) add task t - 2 into the output tile. Every wait
-// is for loads issued one iteration earlier, which the other waves of the CU cover. Codes sit
-// at the positions of their entries as long as the 256 entries hold no skip entry (a 0); a
-// task with one, or with more than 256 entries in the tile, takes the plain walk.
+// Packed entry lists: at first use every listed group's offsets and codes are rewritten once
+// into one word per entry, code << 16 | row inside its 4096-row tile, in list order. A tile's
+// entries are then the range [entries before the tile, entries before the next tile) (both from
+// the row-tile index) and need no decoding: no prefix sums, no skip entries, no special first
+// row. Costs 4 bytes per entry in HBM next to the 2 of the reference's own form.
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(ST_THREADS) void k_rmm_sdc_pipe(const SdcDesc* __restrict__ desc, int nL,
+static_assert(ST == 4096, "packed entries hold 12-bit rows");
+
+__global__ __launch_bounds__(256) void k_sdc_pack(const DGroup* __restrict__ groups, int g, int64_t nRows,
+	uint32_t* __restrict__ packed) {
+	const DGroup G = dgroup(groups + g);
+	const int tile = blockIdx.x * 4 + (threadIdx.x >> 6);
+	const int64_t r0 = (int64_t) tile * SDC_TILE;
+	if(r0 >= nRows) return; // whole waves leave
+	const void* codes = G.codes;
+	const int cw = G.codeWidth;
+	sdc_walk_tile(G, r0, SDC_TILE, [&](int rr, int di) { packed[di] = ((uint32_t) load_code(codes, cw, di) << 16) | (uint32_t) ((r0 + rr) & (ST - 1)); });
+}
+
+// lane t of a wave: entry range of task t's group inside the tile [r0, r0 + ST)
+__device__ __forceinline__ void sdc_tile_range(const SdcDesc& D, int64_t r0, int& start, int& cnt) {
+	const int ti = (int) (r0 / SDC_TILE);
+	const OffState* idx = as_global(D.tileIdx);
+	const int s0 = D.first < r0 ? (ti < D.nTiles ? idx[ti].emit : D.nOffsets) : 0;
+	const int s1 = D.first < r0 + ST ? (ti + ST / SDC_TILE < D.nTiles ? idx[ti + ST / SDC_TILE].emit : D.nOffsets) : 0;
+	start = s0;
+	cnt = s1 - s0;
+}
+
+// Right multiply with one output column on packed lists. A wave owns the groups l = wave,
+// wave + 8, ...; lane t keeps descriptor and entry range of the wave's task t. The task loop
+// runs three stages on consecutive tasks: (A) request four packed entries per lane and the
+// group's table entry `lane`; (B) look the table values up (by lane permute for groups of at
+// most 64 tuples, from L2 otherwise); (C) add into the output tile in LDS. Every wait is for
+// loads issued one iteration earlier, which the other waves of the CU cover.
+__global__ __launch_bounds__(ST_THREADS) void k_rmm_sdc_packed(const SdcDesc* __restrict__ desc, int nL,
 	const double* __restrict__ T, int constRow, int accumulate, double* __restrict__ out, int64_t nRows,
 	unsigned long long* __restrict__ nnz) {
 	extern __shared__ double otile[]; // ST
 	const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-	const int64_t r0 = (int64_t) blockIdx.x * ST, rEnd = r0 + ST;
+	const int64_t r0 = (int64_t) blockIdx.x * ST;
 	const int nr = (int) min((int64_t) ST, nRows - r0);
 	for(int t = tid; t < ST; t += ST_THREADS) {
 		double v = 0.0;
@@ -218,142 +226,77 @@ __global__ __launch_bounds__(ST_THREADS) void k_rmm_sdc_pipe(const SdcDesc* __re
 	}
 	__syncthreads();
 	const int nT = wave < nL ? (nL - wave + ST_THREADS / 64 - 1) / (ST_THREADS / 64) : 0;
-	const int ti = (int) (r0 / SDC_TILE);
 	for(int t0 = 0; t0 < nT; t0 += 64) {
 		const int nHere = min(64, nT - t0);
-		// lane t: descriptor and tile state of task t0 + t
 		SdcDesc D;
 		D.deltas = nullptr; D.codes = nullptr; D.tileIdx = nullptr;
-		D.nDeltas = 0; D.nOffsets = 0; D.first = -1; D.tblOff = 0; D.nTiles = 0; D.widths = 0x101; D.nVals = 0; D.col0 = 0; D.dict = nullptr;
-		OffState st;
-		st.idx = 0; st.emit = 0; st.row = 0; st.pad = 0;
+		D.nDeltas = 0; D.nOffsets = 0; D.first = -1; D.tblOff = 0; D.nTiles = 0; D.widths = 0x101; D.nVals = 0; D.col0 = 0; D.dict = nullptr; D.packed = nullptr;
+		int start = 0, cnt = 0;
 		if(lane < nHere) {
 			D = desc[wave + (ST_THREADS / 64) * (t0 + lane)];
-			if(ti < D.nTiles) st = as_global(D.tileIdx)[ti];
-			else st.idx = D.nDeltas; // no entries behind this tile
+			sdc_tile_range(D, r0, start, cnt);
 		}
-		// pipeline registers
-		int dvA[4] = {-1, -1, -1, -1}, cvA[4] = {0, 0, 0, 0};     // stage A -> B
-		double tblA = 0.0;                                        // table entry `lane` of the group (groups of at most 64 tuples)
-		int rowsC[4] = {0, 0, 0, 0};                              // stage B -> C
+		u32x4 eA = {0, 0, 0, 0};
+		double tblA = 0.0;
+		int rowsC[4] = {0, 0, 0, 0};
 		double tvC[4] = {0.0, 0.0, 0.0, 0.0};
 		unsigned maskC = 0;
 		for(int t = 0; t < nHere + 2; t++) {
-			// ---- stage B inputs are last iteration's A outputs
-			int dvB[4], cvB[4];
-#pragma unroll
-			for(int k = 0; k < 4; k++) { dvB[k] = dvA[k]; cvB[k] = cvA[k]; }
+			const u32x4 eB = eA;
 			const double tblB = tblA;
-			// ---- stage A: task t
-			if(t < nHere) {
-				const uint8_t* dptr = (const uint8_t*) as_global(bcast_lane(D.deltas, t));
-				const uint8_t* cptr = (const uint8_t*) as_global(bcast_lane(D.codes, t));
-				const int nDel = bcast_lane(D.nDeltas, t), nOff = bcast_lane(D.nOffsets, t), w = bcast_lane(D.widths, t);
-				const int i = bcast_lane(st.idx, t) + lane * 4, e = bcast_lane(st.emit, t) + lane * 4;
-				const int dw = w & 0xff, cw = w >> 8;
+			if(t < nHere) { // ---- stage A: task t
+				const uint32_t* pk = as_global(bcast_lane(D.packed, t)) + bcast_lane(start, t);
 				const int nv = bcast_lane(D.nVals, t);
+				eA = *(const u32x4*) (pk + lane * 4); // dword aligned; entries beyond the task's count are masked in stage B
 				tblA = nv <= 64 && lane < nv ? T[bcast_lane(D.tblOff, t) + lane] : 0.0;
-				if(dw == 1 && cw == 1) {
-					// byte lists: the lane's four entries as the two aligned words around them
-					uint32_t dq = sdc_load4(dptr, i, nDel), cq = sdc_load4(cptr, e, nOff);
-#pragma unroll
-					for(int k = 0; k < 4; k++) {
-						dvA[k] = i + k < nDel ? (int) ((dq >> (8 * k)) & 0xff) : -1;
-						cvA[k] = (int) ((cq >> (8 * k)) & 0xff);
-					}
-				}
-				else {
-#pragma unroll
-					for(int k = 0; k < 4; k++) {
-						dvA[k] = i + k < nDel ? (dw == 1 ? (int) dptr[i + k] : (int) ((const uint16_t*) dptr)[i + k]) : -1;
-						cvA[k] = e + k < nOff ? load_code(cptr, cw, e + k) : 0;
-					}
-				}
 			}
-			// ---- stage C: task t - 2
-			if(t >= 2) {
+			if(t >= 2) { // ---- stage C: task t - 2
 #pragma unroll
 				for(int k = 0; k < 4; k++)
 					if(maskC & (1u << k)) unsafeAtomicAdd(&otile[rowsC[k]], tvC[k]);
 			}
 			maskC = 0;
-			// ---- stage B: task t - 1
-			if(t >= 1 && t - 1 < nHere) {
+			if(t >= 1 && t - 1 < nHere) { // ---- stage B: task t - 1
 				const int tb = t - 1;
-				const int w = bcast_lane(D.widths, tb), tblOff = bcast_lane(D.tblOff, tb), nDel = bcast_lane(D.nDeltas, tb);
-				const int dw = w & 0xff, cw = w >> 8, maxV = dw == 1 ? 255 : 65535;
-				const int i0 = bcast_lane(st.idx, tb);
-				int row = bcast_lane(st.row, tb), emit = bcast_lane(st.emit, tb);
-				const int first = bcast_lane(D.first, tb);
-				const uint8_t* cptr = (const uint8_t*) as_global(bcast_lane(D.codes, tb));
-				const double* tg = T + tblOff;
-				const bool inRegs = bcast_lane(D.nVals, tb) <= 64; // table in registers: lookups by lane permute
-				if(lane == 0 && first >= r0 && first < rEnd) unsafeAtomicAdd(&otile[first - r0], tg[load_code(cptr, cw, 0)]);
-				// decode the 256 entries from registers (the arithmetic of sdc_decode256)
-				int s = 0, c = 0, rows[4], didx[4];
-				unsigned mask = 0;
-				bool zero = false;
+				const int n = bcast_lane(cnt, tb);
+				const double* tg = T + bcast_lane(D.tblOff, tb);
+				const bool inRegs = bcast_lane(D.nVals, tb) <= 64;
 #pragma unroll
 				for(int k = 0; k < 4; k++) {
-					const int v = dvB[k];
-					zero |= v == 0;
-					s += v < 0 ? 0 : (v == 0 ? maxV : v);
-					rows[k] = s;
-					didx[k] = c;
-					if(v > 0) { mask |= 1u << k; c++; }
-				}
-				const int ps = wave_scan_incl(s), pc = wave_scan_incl(c);
-#pragma unroll
-				for(int k = 0; k < 4; k++) { rows[k] += row + ps - s; didx[k] += emit + pc - c; }
-				row += __builtin_amdgcn_readlane(ps, 63);
-				emit += __builtin_amdgcn_readlane(pc, 63);
-				const bool plain = __ballot(zero) != 0; // a skip entry shifts the codes against the entries
-#pragma unroll
-				for(int k = 0; k < 4; k++) {
-					const bool on = (mask & (1u << k)) && rows[k] < rEnd;
-					const int code = plain ? (on ? load_code(cptr, cw, didx[k]) : 0) : cvB[k];
-					rowsC[k] = (int) (rows[k] - r0);
+					const bool on = lane * 4 + k < n;
+					const int code = (int) (eB[k] >> 16);
 					const double tv = inRegs ? __shfl(tblB, code & 63, 64) : (on ? tg[code] : 0.0);
-					tvC[k] = on ? tv : 0.0;
+					rowsC[k] = (int) (eB[k] & (ST - 1));
+					tvC[k] = tv;
 					if(on) maskC |= 1u << k;
 				}
-				// more than 256 entries of this group in the tile: the plain walk finishes it
-				int64_t j0 = (int64_t) i0 + 256;
-				const void* dptr = as_global(bcast_lane(D.deltas, tb));
-				while(j0 < nDel && row < rEnd) {
-					int32_t rws[4], dix[4];
-					unsigned m;
-					if(dw == 1) sdc_decode256<1>(dptr, nDel, j0, row, emit, rws, dix, m);
-					else sdc_decode256<2>(dptr, nDel, j0, row, emit, rws, dix, m);
-#pragma unroll
-					for(int k = 0; k < 4; k++)
-						if((m & (1u << k)) && rws[k] < rEnd) unsafeAtomicAdd(&otile[rws[k] - r0], tg[load_code(cptr, cw, dix[k])]);
-					j0 += 256;
+				if(n > 256) { // dense lists: the rest of the tile's entries, straight
+					const uint32_t* pk = as_global(bcast_lane(D.packed, tb)) + bcast_lane(start, tb);
+					for(int j = 256 + lane; j < n; j += 64) {
+						const uint32_t e = pk[j];
+						unsafeAtomicAdd(&otile[e & (ST - 1)], tg[e >> 16]);
+					}
 				}
 			}
 		}
 	}
 	__syncthreads();
-	int cnt = 0;
+	int cntNz = 0;
 	for(int t = tid; t < nr; t += ST_THREADS) {
 		const double v = otile[t];
-		cnt += v != 0.0;
+		cntNz += v != 0.0;
 		out[r0 + t] = v;
 	}
-	count_add(nnz, cnt);
+	count_add(nnz, cntNz);
 }
 
-// ---------------------------------------------------------------------------
-// Left multiply for lists of single-column groups with at most 64 tuples, in the same
-// pipeline: the group's dictionary sits in registers (entry `lane`), every entry contributes
-// Y[row] * dict[code] (row from the Y tile in LDS, dictionary value by lane permute), the wave
-// sums the products and lane t keeps the total of task t. No bins, no atomics in LDS, one
-// launch for all groups; the totals go straight into the output (no pre-aggregate).
-// block = (range of tiles, row i of Y).
-// ---------------------------------------------------------------------------
-__global__ __launch_bounds__(ST_THREADS) void k_lmm_sdc_pipe(const SdcDesc* __restrict__ desc, int nL,
-	const double* __restrict__ Y, int64_t nRows, int tilesPerBlock,
-	double* __restrict__ out, int nCols) {
+// Left multiply on packed lists for single-column groups with at most 64 tuples: the group's
+// dictionary sits in registers (entry `lane`), every entry contributes Y[row] * dict[code] (row
+// from the Y tile in LDS, dictionary value by lane permute), the wave sums the products (DPP) and
+// lane t keeps the total of task t. No bins, no LDS atomics, one launch for all groups; the
+// totals go straight into the output. block = (range of tiles, row i of Y).
+__global__ __launch_bounds__(ST_THREADS) void k_lmm_sdc_packed(const SdcDesc* __restrict__ desc, int nL,
+	const double* __restrict__ Y, int64_t nRows, int tilesPerBlock, double* __restrict__ out, int nCols) {
 	extern __shared__ double ytile[]; // ST
 	const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
 	const int irow = blockIdx.y;
@@ -362,112 +305,46 @@ __global__ __launch_bounds__(ST_THREADS) void k_lmm_sdc_pipe(const SdcDesc* __re
 	const int tile0 = blockIdx.x * tilesPerBlock, tile1 = min(tile0 + tilesPerBlock, nTilesAll);
 	const int nT = wave < nL ? (nL - wave + ST_THREADS / 64 - 1) / (ST_THREADS / 64) : 0;
 	const int nTmax = (nL + ST_THREADS / 64 - 1) / (ST_THREADS / 64); // the same trip count for every wave: barriers inside
-	for(int t0 = 0; t0 < max(nTmax, 1); t0 += 64) { // (at most 512 groups per pass over the tiles: one pass for C4)
+	for(int t0 = 0; t0 < max(nTmax, 1); t0 += 64) {
 		const int nHere = max(0, min(64, nT - t0));
 		SdcDesc D;
 		D.deltas = nullptr; D.codes = nullptr; D.tileIdx = nullptr;
-		D.nDeltas = 0; D.nOffsets = 0; D.first = -1; D.tblOff = 0; D.nTiles = 0; D.widths = 0x101; D.nVals = 0; D.col0 = 0; D.dict = nullptr;
+		D.nDeltas = 0; D.nOffsets = 0; D.first = -1; D.tblOff = 0; D.nTiles = 0; D.widths = 0x101; D.nVals = 0; D.col0 = 0; D.dict = nullptr; D.packed = nullptr;
 		if(lane < nHere) D = desc[wave + (ST_THREADS / 64) * (t0 + lane)];
 		double accT = 0.0; // lane t: total of task t over the block's tiles
 		for(int tile = tile0; tile < tile1; tile++) {
-			const int64_t r0 = (int64_t) tile * ST, rEnd = r0 + ST;
+			const int64_t r0 = (int64_t) tile * ST;
 			__syncthreads(); // the previous tile's readers are done
 			for(int t = tid; t < ST; t += ST_THREADS) ytile[t] = r0 + t < nRows ? y[r0 + t] : 0.0;
 			__syncthreads();
-			const int ti = (int) (r0 / SDC_TILE);
-			OffState st;
-			st.idx = 0; st.emit = 0; st.row = 0; st.pad = 0;
-			if(lane < nHere) {
-				if(ti < D.nTiles) st = as_global(D.tileIdx)[ti];
-				else st.idx = D.nDeltas;
-			}
-			int dvA[4] = {-1, -1, -1, -1}, cvA[4] = {0, 0, 0, 0};
+			int start = 0, cnt = 0;
+			if(lane < nHere) sdc_tile_range(D, r0, start, cnt);
+			u32x4 eA = {0, 0, 0, 0};
 			double dictA = 0.0;
 			for(int t = 0; t < nHere + 1; t++) {
-				int dvB[4], cvB[4];
-#pragma unroll
-				for(int k = 0; k < 4; k++) { dvB[k] = dvA[k]; cvB[k] = cvA[k]; }
+				const u32x4 eB = eA;
 				const double dictB = dictA;
-				// ---- stage A: task t
-				if(t < nHere) {
-					const uint8_t* dptr = (const uint8_t*) as_global(bcast_lane(D.deltas, t));
-					const uint8_t* cptr = (const uint8_t*) as_global(bcast_lane(D.codes, t));
-					const int nDel = bcast_lane(D.nDeltas, t), nOff = bcast_lane(D.nOffsets, t), w = bcast_lane(D.widths, t);
-					const int i = bcast_lane(st.idx, t) + lane * 4, e = bcast_lane(st.emit, t) + lane * 4;
-					const int dw = w & 0xff, cw = w >> 8;
+				if(t < nHere) { // ---- stage A: task t
+					const uint32_t* pk = as_global(bcast_lane(D.packed, t)) + bcast_lane(start, t);
+					eA = *(const u32x4*) (pk + lane * 4);
 					dictA = lane < bcast_lane(D.nVals, t) ? as_global(bcast_lane(D.dict, t))[lane] : 0.0;
-					if(dw == 1 && cw == 1) {
-						const uint32_t dq = sdc_load4(dptr, i, nDel), cq = sdc_load4(cptr, e, nOff);
-#pragma unroll
-						for(int k = 0; k < 4; k++) {
-							dvA[k] = i + k < nDel ? (int) ((dq >> (8 * k)) & 0xff) : -1;
-							cvA[k] = (int) ((cq >> (8 * k)) & 0xff);
-						}
-					}
-					else {
-#pragma unroll
-						for(int k = 0; k < 4; k++) {
-							dvA[k] = i + k < nDel ? (dw == 1 ? (int) dptr[i + k] : (int) ((const uint16_t*) dptr)[i + k]) : -1;
-							cvA[k] = e + k < nOff ? load_code(cptr, cw, e + k) : 0;
-						}
-					}
 				}
-				// ---- stage B: task t - 1
-				if(t >= 1) {
+				if(t >= 1) { // ---- stage B: task t - 1
 					const int tb = t - 1;
-					const int w = bcast_lane(D.widths, tb), nDel = bcast_lane(D.nDeltas, tb);
-					const int dw = w & 0xff, cw = w >> 8, maxV = dw == 1 ? 255 : 65535;
-					const int i0 = bcast_lane(st.idx, tb);
-					int row = bcast_lane(st.row, tb), emit = bcast_lane(st.emit, tb);
-					const int first = bcast_lane(D.first, tb);
-					const uint8_t* cptr = (const uint8_t*) as_global(bcast_lane(D.codes, tb));
+					const int n = bcast_lane(cnt, tb);
 					double part = 0.0;
-					{ // the list's first row is not among the delta entries
-						const bool has = first >= r0 && first < rEnd;
-						const int code0 = has ? load_code(cptr, cw, 0) : 0;
-						const double d0 = __shfl(dictB, code0 & 63, 64);
-						if(has && lane == 0) part = ytile[first - r0] * d0;
-					}
-					int s = 0, c = 0, rows[4], didx[4];
-					unsigned mask = 0;
-					bool zero = false;
 #pragma unroll
 					for(int k = 0; k < 4; k++) {
-						const int v = dvB[k];
-						zero |= v == 0;
-						s += v < 0 ? 0 : (v == 0 ? maxV : v);
-						rows[k] = s;
-						didx[k] = c;
-						if(v > 0) { mask |= 1u << k; c++; }
+						const double d = __shfl(dictB, (int) (eB[k] >> 16) & 63, 64);
+						if(lane * 4 + k < n) part += ytile[eB[k] & (ST - 1)] * d;
 					}
-					const int ps = wave_scan_incl(s), pc = wave_scan_incl(c);
-#pragma unroll
-					for(int k = 0; k < 4; k++) { rows[k] += row + ps - s; didx[k] += emit + pc - c; }
-					row += __builtin_amdgcn_readlane(ps, 63);
-					emit += __builtin_amdgcn_readlane(pc, 63);
-					const bool plain = __ballot(zero) != 0;
-#pragma unroll
-					for(int k = 0; k < 4; k++) {
-						const bool on = (mask & (1u << k)) && rows[k] < rEnd;
-						const int code = plain ? (on ? load_code(cptr, cw, didx[k]) : 0) : cvB[k];
-						const double d = __shfl(dictB, code & 63, 64);
-						if(on) part += ytile[rows[k] - r0] * d;
-					}
-					int64_t j0 = (int64_t) i0 + 256;
-					const void* dptr = as_global(bcast_lane(D.deltas, tb));
-					while(j0 < nDel && row < rEnd) { // more than 256 entries of this group in the tile
-						int32_t rws[4], dix[4];
-						unsigned m;
-						if(dw == 1) sdc_decode256<1>(dptr, nDel, j0, row, emit, rws, dix, m);
-						else sdc_decode256<2>(dptr, nDel, j0, row, emit, rws, dix, m);
-#pragma unroll
-						for(int k = 0; k < 4; k++) {
-							const bool on = (m & (1u << k)) && rws[k] < rEnd;
-							const int code = on ? load_code(cptr, cw, dix[k]) : 0;
-							const double d = __shfl(dictB, code & 63, 64);
-							if(on) part += ytile[rws[k] - r0] * d;
+					if(n > 256) {
+						const uint32_t* pk = as_global(bcast_lane(D.packed, tb)) + bcast_lane(start, tb);
+						for(int j0 = 256; j0 < n; j0 += 64) { // uniform trip count: the permute needs every lane
+							const uint32_t e = j0 + lane < n ? pk[j0 + lane] : 0u;
+							const double d = __shfl(dictB, (int) (e >> 16) & 63, 64);
+							if(j0 + lane < n) part += ytile[e & (ST - 1)] * d;
 						}
-						j0 += 256;
 					}
 					const double total = wave_sum_f64_all(part);
 					if(lane == tb) accT += total;
@@ -494,7 +371,26 @@ static int sdc_plan(cla_block* b, int onlyGroup, int32_t** dList, int32_t** dBin
 			b->sdcBinOff.push_back(b->sdcBinOff.back() + G.nVals);
 		}
 		b->sdcPlanGroup = -2; // invalid until both copies have been issued
+		// packed entries of all listed groups (whole-block plans only), 256 entries of slack behind the last
+		std::vector<int64_t> packedOff;
+		bool packable = onlyGroup < 0 && !b->sdcList.empty();
+		int64_t totalEntries = 0;
+		for(int g : b->sdcList) {
+			packedOff.push_back(totalEntries);
+			totalEntries += b->groups[g].d.nOffsets;
+			packable &= b->groups[g].d.nVals <= 65536;
+		}
+		if(packable && b->dSdcPacked == nullptr) {
+			CLA_HIP(hipMalloc((void**) &b->dSdcPacked, sizeof(uint32_t) * (size_t) (totalEntries + 256)));
+			CLA_HIP(hipMemsetAsync(b->dSdcPacked + totalEntries, 0, sizeof(uint32_t) * 256, b->stream));
+			const int nT1 = (int) ((b->nRows + SDC_TILE - 1) / SDC_TILE);
+			for(size_t l = 0; l < b->sdcList.size(); l++)
+				hipLaunchKernelGGL(k_sdc_pack, dim3((unsigned) ((nT1 + 3) / 4)), dim3(256), 0, b->stream, b->dGroups, b->sdcList[l], b->nRows,
+					b->dSdcPacked + packedOff[l]);
+			CLA_HIP(hipGetLastError());
+		}
 		std::vector<SdcDesc> descs;
+		size_t li = 0;
 		for(int g : b->sdcList) {
 			const DGroup& G = b->groups[g].d;
 			SdcDesc d;
@@ -502,6 +398,8 @@ static int sdc_plan(cla_block* b, int onlyGroup, int32_t** dList, int32_t** dBin
 			d.nDeltas = (int32_t) G.nDeltas; d.nOffsets = (int32_t) G.nOffsets; d.first = G.first; d.tblOff = G.tblOff; d.nTiles = G.nTiles;
 			d.widths = G.deltaWidth | (G.codeWidth << 8);
 			d.nVals = G.nVals; d.col0 = b->groups[g].cols[0]; d.dict = G.dict;
+			d.packed = packable && b->dSdcPacked ? b->dSdcPacked + packedOff[li] : nullptr;
+			li++;
 			descs.push_back(d);
 		}
 		if(!b->sdcList.empty()) {
@@ -527,10 +425,10 @@ int launch_lmm_sdc_tiles(cla_block* b, const double* dY, int p, double* dPre, in
 	if(plan.list.empty()) return 0;
 	// all listed groups single-column with at most 64 tuples, whole-block call: products straight
 	// into dOut, the groups' part of dPre stays zero
-	static const bool noPipe = getenv("CLA_LMM_SDC_NO_PIPE") != nullptr;
-	bool pipe = dOut != nullptr && onlyGroup < 0 && !noPipe;
-	for(int g : plan.list) pipe &= b->groups[g].d.nColG == 1 && b->groups[g].d.nVals <= 64;
-	if(pipe) {
+	static const bool noPacked = getenv("CLA_SDC_NO_PACKED") != nullptr;
+	bool packed = dOut != nullptr && onlyGroup < 0 && !noPacked && b->dSdcPacked != nullptr;
+	for(int g : plan.list) packed &= b->groups[g].d.nColG == 1 && b->groups[g].d.nVals <= 64;
+	if(packed) {
 		const int nTiles = (int) ((b->nRows + ST - 1) / ST);
 		int tpb = std::max(1, (nTiles * p + 4 * g_numCU - 1) / (4 * g_numCU));
 		tpb = std::min(tpb, std::max(1, nTiles));
@@ -538,9 +436,9 @@ int launch_lmm_sdc_tiles(cla_block* b, const double* dY, int p, double* dPre, in
 		double algo = (double) b->nRows * 8 * p;
 		for(int g : plan.list) algo += (double) p * ((double) b->groups[g].d.nDeltas * b->groups[g].d.deltaWidth + (double) b->groups[g].d.nOffsets * b->groups[g].d.codeWidth);
 		const size_t lds = (size_t) ST * 8;
-		Prof pf(b, "k_lmm_sdc_pipe", (long) grid * p, ST_THREADS, (long) lds, algo);
-		CLA_HIP(hipFuncSetAttribute((const void*) k_lmm_sdc_pipe, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
-		hipLaunchKernelGGL(k_lmm_sdc_pipe, dim3(grid, p), dim3(ST_THREADS), lds, b->stream, (const SdcDesc*) b->dSdcDesc,
+		Prof pf(b, "k_lmm_sdc_packed", (long) grid * p, ST_THREADS, (long) lds, algo);
+		CLA_HIP(hipFuncSetAttribute((const void*) k_lmm_sdc_packed, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
+		hipLaunchKernelGGL(k_lmm_sdc_packed, dim3(grid, p), dim3(ST_THREADS), lds, b->stream, (const SdcDesc*) b->dSdcDesc,
 			(int) plan.list.size(), dY, b->nRows, tpb, dOut, b->nCols);
 		CLA_HIP(hipGetLastError());
 		return 0;
@@ -622,12 +520,12 @@ int launch_rmm_sdc_tiles(cla_block* b, int q, int constRow, int accumulate, doub
 		const DGroup& G = b->groups[g].d;
 		algo += (double) G.nDeltas * G.deltaWidth + (double) G.nOffsets * G.codeWidth;
 	}
-	static const bool noPipe = getenv("CLA_RMM_SDC_NO_PIPE") != nullptr;
-	if(q == 1 && !ldsTables && tileRows == ST && !noPipe) {
+	static const bool noPacked = getenv("CLA_SDC_NO_PACKED") != nullptr;
+	if(q == 1 && !ldsTables && tileRows == ST && !noPacked && b->dSdcPacked != nullptr) {
 		const size_t ldsP = (size_t) ST * 8;
-		Prof pf(b, "k_rmm_sdc_pipe", nTiles, ST_THREADS, (long) ldsP, algo);
-		CLA_HIP(hipFuncSetAttribute((const void*) k_rmm_sdc_pipe, hipFuncAttributeMaxDynamicSharedMemorySize, (int) ldsP));
-		hipLaunchKernelGGL(k_rmm_sdc_pipe, dim3(nTiles), dim3(ST_THREADS), ldsP, b->stream, (const SdcDesc*) b->dSdcDesc,
+		Prof pf(b, "k_rmm_sdc_packed", nTiles, ST_THREADS, (long) ldsP, algo);
+		CLA_HIP(hipFuncSetAttribute((const void*) k_rmm_sdc_packed, hipFuncAttributeMaxDynamicSharedMemorySize, (int) ldsP));
+		hipLaunchKernelGGL(k_rmm_sdc_packed, dim3(nTiles), dim3(ST_THREADS), ldsP, b->stream, (const SdcDesc*) b->dSdcDesc,
 			(int) plan.list.size(), b->dTables, constRow, accumulate, dOut, b->nRows, dNnz);
 	}
 	else {
