@@ -232,6 +232,8 @@ void cla_block_free(cla_handle b) {
 	if(b->dDictPad) (void) hipFree(b->dDictPad);
 	if(b->dCountsAll) (void) hipFree(b->dCountsAll);
 	if(b->dOnes) (void) hipFree(b->dOnes);
+	for(uint8_t* p : b->expCodes)
+		if(p) (void) hipFree(p);
 	if(b->dCounters) (void) hipFree(b->dCounters);
 	if(b->hCounters) (void) hipHostFree(b->hCounters);
 	if(b->ownStream && b->stream) (void) hipStreamDestroy(b->stream);

@@ -147,6 +147,32 @@ __device__ __forceinline__ void sdc_decode256(const void* __restrict__ deltas, i
 	emit += __builtin_amdgcn_readlane(pc, WAVE - 1);
 }
 
+// Walks the entries of group G with rows in [r0, r0 + tileRows) and calls f(row - r0, dataIdx)
+// on the owning lane. Must be called by all 64 lanes of a wave.
+template <typename F>
+__device__ __forceinline__ void sdc_walk_tile(const DGroup& G, int64_t r0, int tileRows, F f) {
+	// r0 and tileRows are multiples of SDC_TILE
+	if(G.nOffsets <= 0) return;
+	const int lane = threadIdx.x & 63;
+	const int64_t rEnd = r0 + tileRows;
+	if(lane == 0 && G.first >= r0 && G.first < rEnd) f((int) (G.first - r0), 0);
+	const int ti = (int) (r0 / SDC_TILE);
+	if(ti >= G.nTiles) return;
+	const OffState st = G.tileIdx[ti];
+	int32_t row = st.row, emit = st.emit;
+	int64_t i0 = st.idx;
+	while(i0 < G.nDeltas && row < rEnd) {
+		int32_t rows[4], didx[4];
+		unsigned mask;
+		if(G.deltaWidth == 1) sdc_decode256<1>(G.deltas, G.nDeltas, i0, row, emit, rows, didx, mask);
+		else sdc_decode256<2>(G.deltas, G.nDeltas, i0, row, emit, rows, didx, mask);
+#pragma unroll
+		for(int k = 0; k < 4; k++)
+			if((mask & (1u << k)) && rows[k] < rEnd) f((int) (rows[k] - r0), didx[k]);
+		i0 += 256;
+	}
+}
+
 // BYTES bytes of a code stream in registers, requested as non-temporal 8/16-byte loads.
 template <int BYTES>
 struct RawVec;

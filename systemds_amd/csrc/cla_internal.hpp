@@ -117,6 +117,10 @@ struct cla_block {
 	// (CG/AColGroupValue.java getCounts)
 	int32_t* dCountsAll = nullptr;
 	double* dOnes = nullptr;         // nCols ones: rowSums(X) = X %*% 1
+	// one code per row (0xff = row without a value) of RLE / SDCZeros groups with at most 255 tuples,
+	// expanded once for the decode kernels when that costs at most half the block's own bytes
+	std::vector<uint8_t*> expCodes;
+	bool expTried = false;
 	// all groups single-column DDC with byte codes: dictionaries at a fixed stride of 256 entries
 	// (zero beyond nVals) followed by the groups' column indexes; built on first use
 	double* dDictPad = nullptr;

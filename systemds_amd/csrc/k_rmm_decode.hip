@@ -26,7 +26,7 @@ constexpr int DEC_WAVES = DEC_THREADS / 64;
 constexpr int DEC_TILE = SDC_TILE;     // rows per tile = granularity of the offset tile index
 constexpr int DEC_WROWS = DEC_TILE / DEC_WAVES; // rows of a tile one wave multiplies
 constexpr int DEC_QMAX = 16;
-constexpr int DEC_PF = 4;              // 16-byte chunks a thread holds for the next tile
+constexpr int DEC_PF = 6;              // 16-byte chunks a thread holds for the next tile
 constexpr int DEC_WIN = 2048;           // bytes of an offset list / of its codes kept in LDS per SDC group
 constexpr int DEC_TWIN = 32;            // tile index entries kept in LDS per SDC group
 constexpr int DEC_SLOT_PAD = 80;       // bytes between code tiles: spreads the columns a wave reads together over the LDS banks
@@ -528,6 +528,59 @@ __global__ __launch_bounds__(DEC_THREADS) void k_rmm_decode(const DecArgs A) { d
 template <int NB, int FLAT>
 __global__ __launch_bounds__(DEC_THREADS) void k_tsmm_decode(const DecArgs A) { decode_body<1, NB, 4, FLAT>(A); }
 
+// One code per row for an RLE group (0xff where no run covers the row): thread = 4 rows.
+__global__ __launch_bounds__(256) void k_expand_rle(const DGroup* __restrict__ groups, int g, int64_t nRows, uint8_t* __restrict__ codes) {
+	const DGroup G = dgroup(groups + g);
+	const int64_t rb = ((int64_t) blockIdx.x * 256 + threadIdx.x) * 4;
+	if(rb >= nRows) return;
+	int j = rle_find(G.runStart, G.nRuns, (int32_t) rb);
+	for(int t = 0; t < 4 && rb + t < nRows; t++) {
+		while(G.runStart[j + 1] <= rb + t) j++;
+		codes[rb + t] = (uint8_t) G.runCode[j]; // -1 (uncovered) becomes 0xff
+	}
+}
+
+// One code per listed row of an SDCZeros group into a stream preset to 0xff: wave = one tile of the row-tile index.
+__global__ __launch_bounds__(256) void k_expand_sdc(const DGroup* __restrict__ groups, int g, int64_t nRows, uint8_t* __restrict__ codes) {
+	const DGroup G = dgroup(groups + g);
+	const int64_t r0 = ((int64_t) blockIdx.x * 4 + (threadIdx.x >> 6)) * SDC_TILE;
+	if(r0 >= nRows) return; // whole waves leave
+	const void* src = G.codes;
+	const int cw = G.codeWidth;
+	sdc_walk_tile(G, r0, SDC_TILE, [&](int rr, int di) { codes[r0 + rr] = (uint8_t) load_code(src, cw, di); });
+}
+
+// Expanded code streams make every dictionary-coded group of a block a plain copy in the tile
+// fill. Built once, when they cost at most half of what the block itself takes in HBM.
+static int ensure_expanded(cla_block* b) {
+	if(b->expTried) return 0;
+	b->expTried = true;
+	const int nG = (int) b->groups.size();
+	b->expCodes.assign((size_t) nG, nullptr);
+	if(getenv("CLA_DEC_NO_EXPAND") != nullptr || b->nRows == 0) return 0;
+	std::vector<int> cand;
+	for(int g = 0; g < nG; g++) {
+		const DGroup& G = b->groups[g].d;
+		if((G.type == G_RLE || (G.type == G_SDCZ && G.nOffsets > 0)) && G.nVals <= 255) cand.push_back(g);
+	}
+	if(cand.empty() || (int64_t) cand.size() * b->nRows > b->device_bytes_cached / 2) return 0;
+	for(int g : cand) {
+		const DGroup& G = b->groups[g].d;
+		uint8_t* p = nullptr;
+		CLA_HIP(hipMalloc((void**) &p, (size_t) b->nRows + 16));
+		b->expCodes[g] = p;
+		if(G.type == G_RLE)
+			hipLaunchKernelGGL(k_expand_rle, dim3((unsigned) ((b->nRows + 1023) / 1024)), dim3(256), 0, b->stream, b->dGroups, g, b->nRows, p);
+		else {
+			CLA_HIP(hipMemsetAsync(p, 0xff, (size_t) b->nRows + 16, b->stream));
+			const int64_t nT1 = (b->nRows + SDC_TILE - 1) / SDC_TILE;
+			hipLaunchKernelGGL(k_expand_sdc, dim3((unsigned) ((nT1 + 3) / 4)), dim3(256), 0, b->stream, b->dGroups, g, b->nRows, p);
+		}
+	}
+	CLA_HIP(hipGetLastError());
+	return 0;
+}
+
 // Host side of both kernels: LDS plan, copy list and column descriptors in the block's
 // scratch buffer. Returns 1 when the block does not fit (the caller uses another path).
 struct DecLaunch {
@@ -540,6 +593,10 @@ struct DecLaunch {
 static int dec_prepare(cla_block* b, bool gram, int q, int rpl, DecLaunch& L, size_t dictLimit = (size_t) 1 << 30) {
 	const int nG = (int) b->groups.size();
 	const int nCols = b->nCols;
+	{
+		const int rc = ensure_expanded(b);
+		if(rc) return rc;
+	}
 	std::vector<DecGroup> plan((size_t) nG);
 	size_t valD = 0, slotB = 0;
 	int K = 0;
@@ -586,6 +643,9 @@ static int dec_prepare(cla_block* b, bool gram, int q, int rpl, DecLaunch& L, si
 		}
 		else if(P.slotOff >= 0 && G.type == G_DDC && G.codeWidth == P.slotW && ((uintptr_t) G.codes & 15) == 0) {
 			C.src = (const uint8_t*) G.codes; C.bpr = P.slotW; C.dstOff = (int32_t) (slotBase + P.slotOff);
+		}
+		else if(P.slotOff >= 0 && b->expCodes[g] != nullptr) { // RLE / SDCZeros with an expanded byte stream
+			C.src = b->expCodes[g]; C.bpr = 1; C.dstOff = (int32_t) (slotBase + P.slotOff);
 		}
 		else continue;
 		C.chunk0 = nChunks;

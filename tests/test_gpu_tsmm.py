@@ -51,9 +51,14 @@ def test_c3_scaled(cla, ora, monkeypatch, path):
     check_tsmm(cla, ora, c["groups"], c["n_rows"], c["n_cols"], f"C3 {path}")
 
 
-def test_c5_scaled(cla, ora):
-    """BASELINE config 5 at 1/500 scale (mixed RLE + DDC + SDC + dense): both products."""
+@pytest.mark.parametrize("expand", [True, False])
+def test_c5_scaled(cla, ora, monkeypatch, expand):
+    """BASELINE config 5 at 1/500 scale (mixed RLE + DDC + SDC + dense): both products, with the RLE / SDC
+    groups' codes expanded to byte streams for the decode kernels (the default when that is cheap) and with the
+    per-tile run and offset-list decoding."""
     from systemds_amd import synth
+    if not expand:
+        monkeypatch.setenv("CLA_DEC_NO_EXPAND", "1")
     c = synth.config5(scale=500)
     n_rows, n_cols = c["n_rows"], c["n_cols"]
     check_tsmm(cla, ora, c["groups"], n_rows, n_cols, "C5 tsmm")
