@@ -106,6 +106,10 @@ def other_configs(scale):
     def tsmm_ops(blk, cfg):
         do = torch.empty((cfg["n_cols"], cfg["n_cols"]), dtype=torch.float64, device="cuda")
         yield ("t(X)%*%X", lambda: blk.tsmm_dev(do.data_ptr()), float(blk.device_bytes()))
+        # both operands compressed (here the block with itself, 100 columns over the two sides: every group of the
+        # left side meets every group of the right side, 625 pairs)
+        yield ("t(X)%*%X as compressed x compressed", lambda: blk.lmm_compressed_dev(blk, do.data_ptr()),
+               2 * float(blk.device_bytes()))
     run("C3", c, tsmm_ops)
     del c
     c = synth.config4(scale=scale)
@@ -128,6 +132,8 @@ def other_configs(scale):
         comp = float(blk.device_bytes())
         yield ("X%*%B", lambda: blk.rmm_dev(dB.data_ptr(), 10, do1.data_ptr()), comp + cfg["n_rows"] * 80.0)
         yield ("t(X)%*%X", lambda: blk.tsmm_dev(do2.data_ptr()), comp)
+        # 40 columns over the two sides: the joint rows are decoded once and multiplied on the matrix cores
+        yield ("t(X)%*%X as compressed x compressed", lambda: blk.lmm_compressed_dev(blk, do2.data_ptr()), 2 * comp)
     run("C5", c, c5_ops)
     return out
 

@@ -122,6 +122,16 @@ int64_t cla_lmm_dev(cla_handle h, const double* dY, int32_t nRowY, double* dOut)
 int64_t cla_tsmm(cla_handle h, double* out);
 int64_t cla_tsmm_dev(cla_handle h, double* dOut);
 
+/* CLALibLeftMultBy.leftMultByMatrixTransposed for two compressed blocks
+ * (C/lib/CLALibLeftMultBy.java:100-112, 170-284): out[nColsLeft x nColsRight] = t(left) %*% right,
+ * both blocks with the same number of rows. Every group of `left` meets every group of `right`
+ * once (AColGroup.leftMultByAColGroup), the filtered constants of both sides enter through the
+ * outer products with the column sums. Returns nnz(out) or a negative error; blocks with
+ * overlapping groups are not supported, and uncompressed groups only while both blocks together
+ * have at most 64 columns. The first call on a pair of handles builds a small joint descriptor. */
+int64_t cla_lmm_compressed(cla_handle right, cla_handle left, double* out);
+int64_t cla_lmm_compressed_dev(cla_handle right, cla_handle left, double* dOut);
+
 /* CLALibRightMultBy.rightMultByMatrix with allowOverlap (RMMOverlapping,
  * C/lib/CLALibRightMultBy.java:157-201): X %*% B kept compressed. Every group with row data
  * returns a group over all nColB output columns that shares its index structure (codes,

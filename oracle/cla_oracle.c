@@ -924,6 +924,138 @@ int64_t ora_tsmm(const ora_group* groups, int nG, int64_t nRows, int nCols, doub
 }
 
 /* ------------------------------------------------------------------------- */
+/* Compressed x compressed: CLALibLeftMultBy.leftMultByMatrixTransposed for    */
+/* two compressed blocks, single-threaded form                                 */
+/* (C/lib/CLALibLeftMultBy.java:100-112, 249-284): out = t(left) %*% right.    */
+/* ------------------------------------------------------------------------- */
+/* DictLibMatrixMult.MMDictsDenseDense (CG/dictionary/DictLibMatrixMult.java:195-215);
+ * scale != NULL: MMDictsScalingDenseDense (:217-237) */
+static void mm_dicts(const double* left, int lSize, const int32_t* rowsLeft, const double* right, int rSize,
+	const int32_t* colsRight, int commonDim, const int32_t* scale, double* res, int resCols) {
+	for(int k = 0; k < commonDim; k++)
+		for(int i = 0; i < lSize; i++) {
+			const double vl = scale ? left[(size_t) k * lSize + i] * scale[k] : left[(size_t) k * lSize + i];
+			if(vl != 0)
+				for(int j = 0; j < rSize; j++)
+					res[(size_t) rowsLeft[i] * resCols + colsRight[j]] += vl * right[(size_t) k * rSize + j];
+		}
+}
+
+/* pre-aggregate of a dense column block over a group's index structure, rows in ascending order:
+ * P[code(r), i] += D[r, i]  (APreAgg.preAggregate on the transposed uncompressed data,
+ * CG/APreAgg.java:234-249, CG/ColGroupUncompressed.java:741-783) */
+static double* preagg_dense_cols(const ora_group* g, const double* D, int nC, int64_t nRows) {
+	double* P = (double*) calloc((size_t) imax(g->nVals, 1) * nC, sizeof(double));
+	int32_t* c = row_codes(g, nRows);
+	for(int64_t r = 0; r < nRows; r++)
+		if(c[r] >= 0)
+			for(int i = 0; i < nC; i++) P[(size_t) c[r] * nC + i] += D[(size_t) r * nC + i];
+	free(c);
+	return P;
+}
+
+/* rhs.leftMultByAColGroup(lhs, ret, nRows): APreAgg.java:70-79, 211-249; ColGroupUncompressed.java:732-825 */
+static void left_mult_by_group(const ora_group* rhs, const double* dr, const ora_group* lhs, const double* dl,
+	int64_t nRows, double* res, int resCols) {
+	const int lc = lhs->nColG, rc = rhs->nColG;
+	if(lhs->type == ORA_UNC && rhs->type == ORA_UNC) {
+		/* t(lhs data) %*% rhs data, rows in ascending order */
+		for(int64_t r = 0; r < nRows; r++)
+			for(int i = 0; i < lc; i++) {
+				const double a = lhs->dense[(size_t) r * lc + i];
+				if(a != 0)
+					for(int j = 0; j < rc; j++)
+						res[(size_t) lhs->cols[i] * resCols + rhs->cols[j]] += a * rhs->dense[(size_t) r * rc + j];
+			}
+	}
+	else if(lhs->type == ORA_UNC) {
+		/* rhs pre-aggregates the transposed left data, then times its dictionary (APreAgg.java:234-249) */
+		double* P = preagg_dense_cols(rhs, lhs->dense, lc, nRows); /* nVals_r x lc */
+		mm_dicts(P, lc, lhs->cols, dr, rc, rhs->cols, rhs->nVals, NULL, res, resCols);
+		free(P);
+	}
+	else if(rhs->type == ORA_UNC) {
+		/* lhs pre-aggregates the transposed right data one column at a time (ColGroupUncompressed.java:741-783) */
+		double* P = preagg_dense_cols(lhs, rhs->dense, rc, nRows); /* nVals_l x rc */
+		mm_dicts(dl, lc, lhs->cols, P, rc, rhs->cols, lhs->nVals, NULL, res, resCols);
+		free(P);
+	}
+	else if(lhs->codes == rhs->codes && lhs->type == rhs->type && lhs->deltas == rhs->deltas && lhs->rle == rhs->rle) {
+		/* same index structure: the dictionaries meet directly, scaled by the counts (:216-220) */
+		int32_t* counts = (int32_t*) malloc(sizeof(int32_t) * (size_t) imax(rhs->nVals, 1));
+		ora_counts(rhs, nRows, counts);
+		mm_dicts(dl, lc, lhs->cols, dr, rc, rhs->cols, rhs->nVals, counts, res, resCols);
+		free(counts);
+	}
+	else if((double) rhs->nVals * rc < (double) lhs->nVals * lc) { /* shouldPreAggregateLeft (:302-310) */
+		double* lpa = preagg_that(lhs, rhs, dr, nRows); /* nVals_l x rc */
+		mm_dicts(dl, lc, lhs->cols, lpa, rc, rhs->cols, lhs->nVals, NULL, res, resCols);
+		free(lpa);
+	}
+	else {
+		double* rpa = preagg_that(rhs, lhs, dl, nRows); /* nVals_r x lc */
+		mm_dicts(rpa, lc, lhs->cols, dr, rc, rhs->cols, rhs->nVals, NULL, res, resCols);
+		free(rpa);
+	}
+}
+
+/* AColGroup.colSum of the filtered groups (CLALibUtils.getColSum, C/lib/CLALibUtils.java:267-269) */
+static double* filtered_col_sum(const filtered* f, int nCols, int64_t nRows) {
+	double* cs = (double*) calloc((size_t) imax(nCols, 1), sizeof(double));
+	for(int i = 0; i < f->n; i++) {
+		const ora_group* g = f->g[i];
+		if(g->type == ORA_UNC) {
+			for(int64_t r = 0; r < nRows; r++)
+				for(int j = 0; j < g->nColG; j++) cs[g->cols[j]] += g->dense[(size_t) r * g->nColG + j];
+			continue;
+		}
+		int32_t* counts = (int32_t*) malloc(sizeof(int32_t) * (size_t) imax(g->nVals, 1));
+		ora_counts(g, nRows, counts);
+		for(int kk = 0; kk < g->nVals; kk++)
+			for(int j = 0; j < g->nColG; j++) cs[g->cols[j]] += f->dict[i][(size_t) kk * g->nColG + j] * counts[kk];
+		free(counts);
+	}
+	return cs;
+}
+
+int64_t ora_lmm_compressed(const ora_group* right, int nGR, int nColsR, const ora_group* left, int nGL, int nColsL,
+	int64_t nRows, double* out) {
+	if(nRows < 0 || nColsR <= 0 || nColsL <= 0) FAIL(-1, "lmm_compressed: bad dims");
+	memset(out, 0, sizeof(double) * (size_t) nColsL * nColsR);
+	filtered fR, fL;
+	filter_groups(right, nGR, nColsR, &fR);
+	filter_groups(left, nGL, nColsL, &fL);
+	for(int j = 0; j < fL.n; j++)
+		for(int i = 0; i < fR.n; i++)
+			left_mult_by_group(fR.g[i], fR.dict[i], fL.g[j], fL.dict[j], nRows, out, nColsR);
+	const double* cL = fL.constV;
+	const double* cR = fR.constV;
+	if(cL && cR) /* outerProductWithScaling (:639-648) */
+		for(int row = 0; row < nColsL; row++) {
+			const double v = cL[row] * (double) (int) nRows;
+			for(int col = 0; col < nColsR; col++) out[(size_t) row * nColsR + col] += v * cR[col];
+		}
+	if(cL) { /* left constants x column sums of the right groups (:558-569) */
+		double* cs = filtered_col_sum(&fR, nColsR, nRows);
+		for(int row = 0; row < nColsL; row++)
+			if(cL[row] != 0)
+				for(int col = 0; col < nColsR; col++) out[(size_t) row * nColsR + col] += cL[row] * cs[col];
+		free(cs);
+	}
+	if(cR) { /* column sums of the left groups x right constants */
+		double* cs = filtered_col_sum(&fL, nColsL, nRows);
+		for(int row = 0; row < nColsL; row++)
+			if(cs[row] != 0)
+				for(int col = 0; col < nColsR; col++) out[(size_t) row * nColsR + col] += cs[row] * cR[col];
+		free(cs);
+	}
+	filtered_free(&fR); filtered_free(&fL);
+	int64_t nnz = 0;
+	for(size_t z = 0; z < (size_t) nColsL * nColsR; z++) nnz += out[z] != 0;
+	return nnz;
+}
+
+/* ------------------------------------------------------------------------- */
 /* MMChain: CLALibMMChain.mmChain (C/lib/CLALibMMChain.java:92-148):           */
 /* t(X) %*% (w * (X %*% v)) ; ctype 0 = XtXv, 1 = XtwXv.                       */
 /* ------------------------------------------------------------------------- */

@@ -21,6 +21,9 @@
  *                       checked against math.fsum truth; the reference's own
  *                       tests are differential in exactly this way
  *                       (CompressedTestBase.java:609-626, 666-685, 865-884)
+ *   lmm_compressed    : equal t(D_left) @ D_right of the two brute-force decompressed
+ *                       blocks, checked against math.fsum truth (the reference's test is
+ *                       differential the same way, CompressedTestBase.java:726-760)
  *   counts / cooc     : numpy.bincount / np.add.at brute force (exact integers)
  */
 #ifndef CLA_ORACLE_H
@@ -81,6 +84,9 @@ int ora_preaggregate_dense(const ora_group* g, int64_t nRows, const double* Y, i
 int64_t ora_rmm(const ora_group* groups, int nG, int64_t nRows, int nCols, const double* B, int q, double* out, int k);
 int64_t ora_lmm(const ora_group* groups, int nG, int64_t nRows, int nCols, const double* Y, int p, double* out, int k);
 int64_t ora_tsmm(const ora_group* groups, int nG, int64_t nRows, int nCols, double* out, int k);
+/* t(left) %*% right for two compressed blocks of nRows rows each; out is nColsL x nColsR row-major */
+int64_t ora_lmm_compressed(const ora_group* right, int nGR, int nColsR, const ora_group* left, int nGL, int nColsL,
+	int64_t nRows, double* out);
 int64_t ora_mmchain(const ora_group* groups, int nG, int64_t nRows, int nCols, const double* v, const double* w,
 	int ctype, double* out, int k);
 

@@ -73,6 +73,8 @@ def lib():
         L.ora_lmm.argtypes = [vp, i32, i64, i32, vp, i32, vp, i32]
         L.ora_tsmm.restype = i64
         L.ora_tsmm.argtypes = [vp, i32, i64, i32, vp, i32]
+        L.ora_lmm_compressed.restype = i64
+        L.ora_lmm_compressed.argtypes = [vp, i32, i32, vp, i32, i32, i64, vp]
         L.ora_mmchain.restype = i64
         L.ora_mmchain.argtypes = [vp, i32, i64, i32, vp, vp, i32, vp, i32]
         L.ora_last_error.restype = C.c_char_p
@@ -249,6 +251,16 @@ def lmm(groups, Y, k=1):
 def tsmm(groups, k=1):
     out = np.zeros((groups.n_cols, groups.n_cols))
     nnz = _chk(lib().ora_tsmm(groups.ptr, groups.n, groups.n_rows, groups.n_cols, _p(out), k))
+    return out, nnz
+
+
+def lmm_compressed(right, left):
+    """t(left) %*% right for two compressed blocks (CLALibLeftMultBy.java:100-112, 249-284)."""
+    if left.n_rows != right.n_rows:
+        raise OracleError("row counts differ")
+    out = np.zeros((left.n_cols, right.n_cols))
+    nnz = _chk(lib().ora_lmm_compressed(right.ptr, right.n, right.n_cols, left.ptr, left.n, left.n_cols,
+                                        right.n_rows, _p(out)))
     return out, nnz
 
 

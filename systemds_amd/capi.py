@@ -55,6 +55,8 @@ SIGNATURES = {
     "cla_tsmm_dev": (C.c_int64, [C.c_void_p, C.c_void_p]),
     "cla_mmchain": (C.c_int64, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
     "cla_mmchain_dev": (C.c_int64, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
+    "cla_lmm_compressed": (C.c_int64, [C.c_void_p, C.c_void_p, C.c_void_p]),
+    "cla_lmm_compressed_dev": (C.c_int64, [C.c_void_p, C.c_void_p, C.c_void_p]),
     "cla_rmm_overlapping": (C.c_void_p, [C.c_void_p, C.c_void_p, C.c_int32]),
     "cla_aggregate": (C.c_int64, [C.c_void_p, C.c_int32, C.c_int32, C.c_void_p]),
     "cla_aggregate_dev": (C.c_int64, [C.c_void_p, C.c_int32, C.c_int32, C.c_void_p]),
@@ -248,6 +250,15 @@ class ClaBlock:
         out = np.empty((self.n_cols,), np.float64)
         nnz = _check(self.lib.cla_mmchain(self.h, _ptr(v), _ptr(w), int(ctype), _ptr(out)))
         return out, nnz
+
+    def lmm_compressed(self, left):
+        """cla_lmm_compressed: t(left) %*% self for a compressed `left` with the same number of rows."""
+        out = np.empty((left.n_cols, self.n_cols), np.float64)
+        nnz = _check(self.lib.cla_lmm_compressed(self.h, left.h, _ptr(out)))
+        return out, nnz
+
+    def lmm_compressed_dev(self, left, dOut_ptr):
+        return _check(self.lib.cla_lmm_compressed_dev(self.h, left.h, C.c_void_p(dOut_ptr)))
 
     def rmm_overlapping(self, B):
         """cla_rmm_overlapping: X %*% B kept compressed (a new block that borrows this block's index structures)."""

@@ -139,7 +139,7 @@ static int upload_dict(HostGroup& g) {
 	return upload(g, g.dict.data(), sizeof(double) * g.dict.size(), (const void**) &g.d.dict);
 }
 
-int finish_finalize(cla_block* b, cla_block* arenaFrom);
+int finish_finalize(cla_block* b, cla_block* arenaFrom, bool buildArena = true);
 
 } // namespace cla
 
@@ -193,7 +193,9 @@ cla_handle cla_block_create(int64_t nRows, int32_t nCols) {
 		set_error("invalid block shape %lld x %d", (long long) nRows, nCols);
 		return nullptr;
 	}
+	static std::atomic<uint64_t> nextSerial{1};
 	cla_block* b = new cla_block();
+	b->serial = nextSerial.fetch_add(1);
 	b->nRows = nRows;
 	b->nCols = nCols;
 	b->constV.assign((size_t) nCols, 0.0);
@@ -212,6 +214,7 @@ void cla_block_free(cla_handle b) {
 	if(!b) return;
 	if(b->refs.fetch_sub(1) > 1) return; // blocks made from this one still use its streams
 	cla_block* parent = b->parent;
+	if(b->joint) { cla_block_free(b->joint); b->joint = nullptr; }
 	if(g_device >= 0) (void) hipSetDevice(g_device);
 	if(b->stream) (void) hipStreamSynchronize(b->stream);
 	clear_stats(b);
@@ -445,8 +448,8 @@ namespace cla {
 
 // Block-level part of finalize: dictionaries back to back, descriptor array, constants, table
 // offsets, code arena (built, or borrowed from arenaFrom whose groups this block mirrors one to
-// one), mat-vec slabs.
-int finish_finalize(cla_block* b, cla_block* arenaFrom) {
+// one; never built for a block whose code streams are borrowed, buildArena false), mat-vec slabs.
+int finish_finalize(cla_block* b, cla_block* arenaFrom, bool buildArena) {
 	const int maxVals = b->maxVals;
 	const size_t nG = b->groups.size();
 	// all dictionaries back to back in one allocation (kernels copy a slab of
@@ -492,7 +495,7 @@ int finish_finalize(cla_block* b, cla_block* arenaFrom) {
 		b->arenaStride = arenaFrom->arenaStride;
 		b->arenaWidth = arenaFrom->arenaWidth;
 	}
-	else if(allDdc) {
+	else if(allDdc && buildArena) {
 		const size_t stride = (((size_t) b->nRows * cw) + 255) & ~(size_t) 255;
 		CLA_HIP(hipMalloc((void**) &b->dArena, stride * nG));
 		for(size_t i = 0; i < nG; i++) {
@@ -665,6 +668,120 @@ int64_t cla_tsmm(cla_handle b, double* out) {
 	const int64_t nnz = cla_tsmm_dev(b, b->dStageOut);
 	if(nnz < 0) return nnz;
 	CLA_HIP(hipMemcpy(out, b->dStageOut, nOut * sizeof(double), hipMemcpyDeviceToHost));
+	return nnz;
+}
+
+namespace cla {
+
+__global__ __launch_bounds__(256) void k_take_block(const double* __restrict__ G, int n, int r0, int c0, int nr, int nc,
+	double* __restrict__ out, unsigned long long* __restrict__ nnz) {
+	int cnt = 0;
+	for(int idx = threadIdx.x + blockIdx.x * 256; idx < nr * nc; idx += 256 * gridDim.x) {
+		const int i = idx / nc, j = idx - i * nc;
+		const double v = G[(size_t) (r0 + i) * n + c0 + j];
+		out[idx] = v;
+		cnt += v != 0.0;
+	}
+	if(cnt) atomicAdd(nnz, (unsigned long long) cnt);
+}
+
+// cbind(left, right) as a block of its own: the groups of `left` first, then those of `right` with
+// their columns shifted by left->nCols. Row data (codes, offsets, runs, dense values) is borrowed
+// from the two blocks, which must outlive it; column lists and dictionaries are its own copies.
+static cla_block* make_joint(cla_block* left, cla_block* right) {
+	cla_block* c = cla_block_create(left->nRows, left->nCols + right->nCols);
+	if(!c) return nullptr;
+	int tblOff = 0, colOff = 0, maxVals = 0;
+	for(int side = 0; side < 2; side++) {
+		cla_block* src = side ? right : left;
+		const int shift = side ? left->nCols : 0;
+		for(auto& pg : src->groups) {
+			c->groups.emplace_back();
+			HostGroup& g = c->groups.back();
+			g.d = pg.d; // row data: borrowed
+			g.cols = pg.cols;
+			for(int& col : g.cols) col += shift;
+			g.dict = pg.dict;
+			g.bytes = 0;
+			if(upload(g, g.cols.data(), sizeof(int32_t) * g.cols.size(), (const void**) &g.d.cols) ||
+				(!g.dict.empty() && upload_dict(g))) {
+				cla_block_free(c);
+				return nullptr;
+			}
+			g.bytes = pg.bytes;
+			g.d.tblOff = tblOff;
+			g.d.colOff = colOff;
+			tblOff += g.d.nVals;
+			colOff += g.d.nColG;
+			maxVals = std::max(maxVals, g.d.nVals);
+		}
+		for(int j = 0; j < src->nCols; j++) c->constV[(size_t) shift + j] = src->constV[j];
+		c->hasConst |= src->hasConst;
+		c->hasSdc |= src->hasSdc;
+		c->hasRle |= src->hasRle;
+		c->hasUnc |= src->hasUnc;
+	}
+	c->crossSplit = (int32_t) left->groups.size();
+	c->totalVals = tblOff;
+	c->totalColsG = colOff;
+	c->maxVals = maxVals;
+	if(finish_finalize(c, nullptr, false)) { cla_block_free(c); return nullptr; }
+	return c;
+}
+
+} // namespace cla
+
+int64_t cla_lmm_compressed_dev(cla_handle right, cla_handle left, double* dOut) {
+	int rc = check_final(right);
+	if(rc || (rc = check_final(left))) return rc;
+	if(!dOut) { set_error("compressed left multiply: null output"); return -CLA_ERR_INVALID; }
+	if(left->nRows != right->nRows) {
+		set_error("compressed left multiply: %lld rows on the left, %lld on the right", (long long) left->nRows, (long long) right->nRows);
+		return -CLA_ERR_INVALID;
+	}
+	std::lock_guard<std::recursive_mutex> lk(right->mu);
+	std::unique_lock<std::recursive_mutex> lk2(left->mu, std::defer_lock);
+	if(left != right) lk2.lock();
+	if(!right->joint || right->jointSerial != left->serial) {
+		if(right->joint) { cla_block_free(right->joint); right->joint = nullptr; }
+		right->joint = make_joint(left, right);
+		if(!right->joint) return -CLA_ERR_DEVICE;
+		right->jointSerial = left->serial;
+	}
+	cla_block* c = right->joint;
+	c->profile = right->profile;
+	// the joint block works on the right block's stream
+	if(c->stream != right->stream) {
+		if(c->ownStream && c->stream) { (void) hipStreamSynchronize(c->stream); (void) hipStreamDestroy(c->stream); }
+		c->stream = right->stream;
+		c->ownStream = false;
+	}
+	const size_t n = (size_t) c->nCols;
+	if((rc = ensure_stage(&c->dStageOut, &c->stageOutCap, n * n))) return rc;
+	if((rc = launch_tsmm(c, c->dStageOut, c->dCounters))) return rc;
+	CLA_HIP(hipMemsetAsync(right->dCounters, 0, sizeof(unsigned long long), right->stream));
+	const int nOut = left->nCols * right->nCols;
+	{
+		Prof pf(c, "k_take_block", (nOut + 255) / 256, 256, 0, 0);
+		hipLaunchKernelGGL(k_take_block, dim3((unsigned) std::min((nOut + 255) / 256, 1024)), dim3(256), 0, right->stream,
+			c->dStageOut, (int) n, 0, left->nCols, left->nCols, right->nCols, dOut, right->dCounters);
+	}
+	CLA_HIP(hipGetLastError());
+	clear_stats(right);
+	right->lastStats.swap(c->lastStats); // what the kernel statistics of `right` report
+	return finish_nnz(right);
+}
+
+int64_t cla_lmm_compressed(cla_handle right, cla_handle left, double* out) {
+	int rc = check_final(right);
+	if(rc || (rc = check_final(left))) return rc;
+	if(!out) { set_error("compressed left multiply: null output"); return -CLA_ERR_INVALID; }
+	const size_t nOut = (size_t) left->nCols * right->nCols;
+	std::lock_guard<std::recursive_mutex> lk(right->mu);
+	if((rc = ensure_stage(&right->dStageOut, &right->stageOutCap, nOut))) return rc;
+	const int64_t nnz = cla_lmm_compressed_dev(right, left, right->dStageOut);
+	if(nnz < 0) return nnz;
+	CLA_HIP(hipMemcpy(out, right->dStageOut, nOut * sizeof(double), hipMemcpyDeviceToHost));
 	return nnz;
 }
 

@@ -78,6 +78,13 @@ struct cla_block {
 	cla_block* parent = nullptr;
 	std::atomic<int> refs{1};
 	bool arenaShared = false;
+	// cbind(left, this) made by cla_lmm_compressed for the last `left` it saw (told apart by
+	// serial, which is never reused); it borrows both blocks' row data and holds no reference:
+	// it is rebuilt when another left block comes and freed with this block.
+	uint64_t serial = 0;
+	cla_block* joint = nullptr;
+	uint64_t jointSerial = 0;
+	int32_t crossSplit = 0;          // > 0: joint block, groups [0, crossSplit) are the left side's
 	std::vector<cla::HostGroup> groups;
 	std::vector<double> constV;      // filtered constants (SDC defaults, const groups), nCols
 	bool hasConst = false;

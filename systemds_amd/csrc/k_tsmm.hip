@@ -455,8 +455,29 @@ int launch_tsmm(cla_block* b, double* dOut, unsigned long long* dNnz) {
 	// the second per eight pairs and row.
 	const bool forceDecode = getenv("CLA_TSMM_DECODE") != nullptr, forcePairs = getenv("CLA_TSMM_PAIRS") != nullptr; // per call: tests switch them
 	const int nb = (nCols + 15) / 16;
-	const bool gramCheaper = nCols <= 64 && (int64_t) nG * (nG - 1) / 2 >= (int64_t) 8 * nb * (nb + 1) / 2;
-	const bool dense = nG >= nCols || b->hasUnc || forceDecode || (gramCheaper && !forcePairs);
+	// a joint block (cbind of two blocks, only the cross product wanted) pairs left groups with right groups only
+	const int split = b->crossSplit;
+	const int64_t nPairs = split > 0 ? (int64_t) split * (nG - split) : (int64_t) nG * (nG - 1) / 2;
+	const bool gramCheaper = nCols <= 64 && nPairs >= (int64_t) 8 * nb * (nb + 1) / 2;
+	// the per-pair path keeps the smaller accumulator nVals_t x nCol_s of a pair in LDS; where that cannot fit
+	// (two very large dictionaries meet) the block is decoded instead when it is narrow enough
+	bool pairsFit = true;
+	for(int g = 0; g < nG && pairsFit; g++)
+		for(int h = g + 1; h < nG; h++) {
+			if(split > 0 && (g < split) == (h < split)) continue;
+			const DGroup& A = b->groups[g].d;
+			const DGroup& B = b->groups[h].d;
+			if(A.type == G_UNC || B.type == G_UNC) continue;
+			const size_t acc = std::min((size_t) A.nVals * B.nColG, (size_t) B.nVals * A.nColG) * 8;
+			if(acc + (size_t) 2 * TT * 4 > (size_t) 150 * 1024) { pairsFit = false; break; }
+		}
+	const bool mustDecode = b->hasUnc || forceDecode || (!pairsFit && nCols <= 64);
+	const bool dense = split > 0 ? mustDecode || (nCols <= 64 && (nG >= nCols || gramCheaper) && !forcePairs)
+	                             : nG >= nCols || mustDecode || (gramCheaper && !forcePairs);
+	if(dense && split > 0 && nCols > 64) {
+		set_error("compressed left multiply: uncompressed groups need at most 64 columns over both blocks (have %d)", nCols);
+		return -CLA_ERR_UNSUPPORTED;
+	}
 	if(dense) {
 		// t(D) %*% D of the decoded rows, constants included (no correction layer needed)
 		static const bool noMfma = getenv("CLA_TSMM_NO_MFMA") != nullptr;
@@ -513,6 +534,7 @@ int launch_tsmm(cla_block* b, double* dOut, unsigned long long* dNnz) {
 	size_t ldsMax = 0, dotLds = 0;
 	for(int g = 0; g < nG && nRows > 0; g++)
 		for(int h = g + 1; h < nG; h++) {
+			if(split > 0 && (g < split) == (h < split)) continue;
 			const DGroup& A = b->groups[g].d;
 			const DGroup& B = b->groups[h].d;
 			const size_t bothDicts = ((size_t) A.nVals * A.nColG + (size_t) B.nVals * B.nColG + 2) * 8;

@@ -739,7 +739,21 @@ struct CLALibLeftMultBy {
 		MatrixBlock denseL;
 		const MatrixBlock* src = &left;
 		if(left.isCompressed()) {
-			denseL = CLALibDecompress::decompress(static_cast<CompressedMatrixBlock&>(left), k);
+			// both sides compressed (CLALibLeftMultBy.java:100-112): every left group meets every right group on
+			// the device; shapes that path does not take decompress the left side, as the non-compressed overload does
+			CompressedMatrixBlock& cl = static_cast<CompressedMatrixBlock&>(left);
+			MatrixBlock ret(left.getNumColumns(), right.getNumColumns());
+			const int64_t nnz = cla_lmm_compressed(right.hipHandle(), cl.hipHandle(), ret.getDenseBlockValues());
+			if(nnz != -CLA_ERR_UNSUPPORTED) {
+				try {
+					ret.setNonZeros(checkNative(nnz, "Compressed Transposed LMM"));
+				}
+				catch(const std::exception& e) {
+					throw DMLCompressionException(std::string("Failed CLA Compressed Transposed LMM: ") + e.what());
+				}
+				return ret;
+			}
+			denseL = CLALibDecompress::decompress(cl, k);
 			src = &denseL;
 		}
 		MatrixBlock t = src->transpose();
@@ -790,12 +804,15 @@ struct CLALibMatrixMult {
 		MatrixBlock* a = &m1;
 		MatrixBlock* b = &m2;
 		if(a->isCompressed() && b->isCompressed()) {
-			// both compressed: the side that is not transposed stays compressed, the other is decompressed
+			// doubleCompressedMatrixMultiply (CLALibMatrixMult.java:95-124): t(m1) %*% m2 stays compressed on both
+			// sides (the wider block takes the right-hand role, the result is transposed back); the other
+			// combinations decompress the right-hand side
 			auto& ca = static_cast<CompressedMatrixBlock&>(*a);
 			auto& cb = static_cast<CompressedMatrixBlock&>(*b);
 			if(transposeLeft && !transposeRight) { // t(m1) %*% m2
-				MatrixBlock d = CLALibDecompress::decompress(ca, k);
-				return CLALibLeftMultBy::leftMultByMatrixTransposed(cb, d, k);
+				if(ca.getNumColumns() > cb.getNumColumns())
+					return CLALibLeftMultBy::leftMultByMatrixTransposed(ca, cb, k).transpose();
+				return CLALibLeftMultBy::leftMultByMatrixTransposed(cb, ca, k);
 			}
 			MatrixBlock d = CLALibDecompress::decompress(cb, k);
 			return matrixMultiply(m1, d, k, transposeLeft, transposeRight);

@@ -49,7 +49,7 @@ def java_random_ints(seed):
     return next_int
 
 
-def mixed_block(seed, n_rows, with_unc=True, with_const=True, overlap=False):
+def mixed_block(seed, n_rows, with_unc=True, with_const=True, overlap=False, big_dict=True):
     """A small block with every group type, used by several tests."""
     from systemds_amd import synth
     rng = np.random.default_rng(seed)
@@ -64,8 +64,9 @@ def mixed_block(seed, n_rows, with_unc=True, with_const=True, overlap=False):
     specs.append(synth.GroupSpec("ddc", cols(1), rng.standard_normal((7, 1)), rng.integers(0, 7, n_rows).astype(np.uint8)))
     specs.append(synth.GroupSpec("ddc", cols(2), rng.standard_normal((300, 2)),
                                  rng.integers(0, 300, n_rows).astype(np.uint16)))
-    specs.append(synth.GroupSpec("ddc", cols(1), rng.standard_normal((70000, 1)),
-                                 rng.integers(0, 70000, n_rows).astype(np.int32)))
+    nv = 70000 if big_dict else 700
+    specs.append(synth.GroupSpec("ddc", cols(1), rng.standard_normal((nv, 1)),
+                                 rng.integers(0, nv, n_rows).astype(np.int32)))
     specs.append(synth.sdc_group(rng, n_rows, cols(1), 5, 0.1, None))
     specs.append(synth.sdc_group(rng, n_rows, cols(2), 6, 0.004, 1.5))
     run_codes = rng.integers(-1, 4, size=n_rows // 20 + 2)

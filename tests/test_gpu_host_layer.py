@@ -79,6 +79,15 @@ def test_both_sides_compressed(H, ora, cla):
     b, DB, _ = build(H, ora, 8, 300)
     mm = H.CLALibMatrixMult.matrixMultiply
     close(mm(a, b, 1, True, False).toArray(), DA.T, DB, "t(A) %*% B compressed-compressed", ora)
+    # the wider block takes the right-hand role and the result is transposed back (CLALibMatrixMult.java:104-111)
+    w, DW, _ = build(H, ora, 9, 300, with_unc=False)
+    assert DW.shape[1] != DA.shape[1]
+    close(mm(a, w, 1, True, False).toArray(), DA.T, DW, "t(A) %*% W", ora)
+    close(mm(w, a, 1, True, False).toArray(), DW.T, DA, "t(W) %*% A", ora)
+    close(H.CLALibLeftMultBy.leftMultByMatrixTransposed(w, a, 2).toArray(), DA.T, DW, "leftMultByMatrixTransposed(cmb, cmb)", ora)
+    short, _, _ = build(H, ora, 10, 200)
+    with pytest.raises(H.DMLCompressionException):
+        H.CLALibLeftMultBy.leftMultByMatrixTransposed(a, short, 1)
     c = H.CompressedMatrixBlock(DA.shape[1], 2)
     c.allocateColGroupList([H.ColGroupUncompressed.create(H.MatrixBlock(np.random.default_rng(1).standard_normal((DA.shape[1], 2))))])
     close(mm(a, c, 1).toArray(), DA, c.decompress().toArray(), "A %*% C compressed-compressed", ora)

@@ -1,0 +1,118 @@
+"""GPU parity of the compressed x compressed left multiply (cla_lmm_compressed): t(left) %*% right
+for two compressed blocks, as CLALibLeftMultBy.leftMultByMatrixTransposed does
+(C/lib/CLALibLeftMultBy.java:100-112, 170-284), against the CPU oracle and the decompressed truth."""
+import numpy as np
+import pytest
+
+from conftest import mixed_block
+from parity import assert_fp64_close, assert_matches_truth
+
+pytestmark = pytest.mark.gpu
+
+
+def check(cla, ora, specsL, nL, specsR, nR, n_rows, what, keep=False):
+    left = cla.build_block(n_rows, nL, specsL)
+    right = cla.build_block(n_rows, nR, specsR)
+    out, nnz = right.lmm_compressed(left)
+    ref, rnnz = ora.lmm_compressed(ora.Groups(specsR, n_rows, nR), ora.Groups(specsL, n_rows, nL))
+    DL = ora.np_decompress(specsL, n_rows, nL)
+    DR = ora.np_decompress(specsR, n_rows, nR)
+    assert out.shape == (nL, nR)
+    assert_matches_truth(out, DL.T, DR, what=what)
+    assert_fp64_close(out, ref, ora.abs_matmul(DL.T, DR), what=what, n_terms=n_rows)
+    assert nnz == rnnz
+    if keep:
+        return left, right, out
+    left.close()
+    right.close()
+
+
+@pytest.mark.parametrize("path", [None, "CLA_TSMM_PAIRS", "CLA_TSMM_DECODE"])
+@pytest.mark.parametrize("seed,n_rows", [(0, 1), (1, 37), (2, 3000), (4, 150001)])
+def test_mixed_groups(cla, ora, monkeypatch, path, seed, n_rows):
+    """Every pairing of DDC / SDC / SDCZeros / RLE / const / empty groups, on the per-pair path and on the
+    decoded path (the library picks by cost; the switches force one)."""
+    if path:
+        monkeypatch.setenv(path, "1")
+    specsL, nL = mixed_block(seed, n_rows, with_unc=False)
+    # two 70000-tuple dictionaries cannot meet on the per-pair path (the accumulator of either side exceeds LDS):
+    # the library then decodes; the forced per-pair run keeps one of them small
+    specsR, nR = mixed_block(seed + 50, n_rows, with_unc=False, with_const=seed % 2 == 0,
+                             big_dict=path != "CLA_TSMM_PAIRS")
+    check(cla, ora, specsL, nL, specsR, nR, n_rows, f"t(L) %*% R {path}")
+
+
+@pytest.mark.parametrize("unc_l,unc_r", [(True, False), (False, True), (True, True)])
+def test_uncompressed_groups(cla, ora, unc_l, unc_r):
+    specsL, nL = mixed_block(5, 20011, with_unc=unc_l)
+    specsR, nR = mixed_block(6, 20011, with_unc=unc_r)
+    check(cla, ora, specsL, nL, specsR, nR, 20011, f"t(L) %*% R unc={unc_l},{unc_r}")
+
+
+def test_not_transposed_and_cached(cla, ora):
+    """Different column counts on the two sides; a second call reuses the joint descriptor, another left block
+    replaces it, and swapping the operands gives the transpose."""
+    n_rows = 70001
+    specsL, nL = mixed_block(7, n_rows, with_unc=False, with_const=False)
+    specsR, nR = mixed_block(8, n_rows, with_unc=False)
+    assert nL != nR
+    left, right, out = check(cla, ora, specsL, nL, specsR, nR, n_rows, "first", keep=True)
+    again, _ = right.lmm_compressed(left)
+    DL = ora.np_decompress(specsL, n_rows, nL)
+    DR = ora.np_decompress(specsR, n_rows, nR)
+    # (floating-point atomics: the order of the partial sums differs from call to call)
+    assert_fp64_close(again, out, ora.abs_matmul(DL.T, DR), what="second call", n_terms=n_rows)
+    swapped, _ = left.lmm_compressed(right)
+    assert_fp64_close(swapped, out.T, ora.abs_matmul(DR.T, DL), what="swapped", n_terms=n_rows)
+    specsO, nO = mixed_block(9, n_rows, with_unc=False)
+    other = cla.build_block(n_rows, nO, specsO)
+    left.close()   # the cached joint descriptor of (left, right) is stale now and must not be used
+    out2, _ = right.lmm_compressed(other)
+    assert_matches_truth(out2, ora.np_decompress(specsO, n_rows, nO).T, DR, what="other left")
+    # the blocks still serve their own entry points
+    ts, _ = right.tsmm()
+    assert_matches_truth(ts, DR.T, DR, what="right tsmm after")
+    other.close()
+    right.close()
+
+
+def test_same_block_is_tsmm(cla, ora):
+    specs, n = mixed_block(10, 30000, with_unc=False)
+    blk = cla.build_block(30000, n, specs)
+    out, _ = blk.lmm_compressed(blk)
+    ts, _ = blk.tsmm()
+    D = ora.np_decompress(specs, 30000, n)
+    assert_fp64_close(out, ts, 2 * ora.abs_matmul(D.T, D), what="t(X) %*% X", n_terms=30000)
+    blk.close()
+
+
+def test_wide_blocks_take_the_pair_path(cla, ora):
+    """More than 64 columns over both blocks: only the per-pair path applies (C2- and C3-shaped blocks)."""
+    from systemds_amd import synth
+    a = synth.config2(scale=500, n_cols=60)
+    b = synth.config3(scale=500)
+    assert a["n_rows"] == b["n_rows"]
+    check(cla, ora, a["groups"], a["n_cols"], b["groups"], b["n_cols"], a["n_rows"], "C2 x C3")
+
+
+def test_errors(cla):
+    specsL, nL = mixed_block(1, 100, with_unc=False)
+    specsR, nR = mixed_block(2, 101, with_unc=False)
+    left = cla.build_block(100, nL, specsL)
+    right = cla.build_block(101, nR, specsR)
+    with pytest.raises(cla.ClaError) as e:
+        right.lmm_compressed(left)
+    assert e.value.code == cla.ERR_INVALID
+    left.close()
+    right.close()
+    # uncompressed groups with more than 64 columns over both blocks: no per-pair form, not supported
+    from systemds_amd import synth
+    a = synth.config2(scale=1000, n_cols=70)
+    specsU, nU = mixed_block(3, a["n_rows"], with_unc=True)
+    wide = cla.build_block(a["n_rows"], a["n_cols"], a["groups"])
+    unc = cla.build_block(a["n_rows"], nU, specsU)
+    with pytest.raises(cla.ClaError) as e:
+        wide.lmm_compressed(unc)
+    assert e.value.code == cla.ERR_UNSUPPORTED
+    wide.close()
+    unc.close()

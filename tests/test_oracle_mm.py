@@ -190,3 +190,69 @@ def test_edge_sdc_lists(ora):
             Y = rng.standard_normal((2, n_rows))
             out, _ = ora.lmm(G, Y, 1)
             assert np.allclose(out, Y @ D, rtol=1e-12, atol=1e-11)
+
+
+# ---------------------------------------------------------------------------
+# compressed x compressed: t(left) %*% right (CLALibLeftMultBy.java:100-112, 249-284)
+# ---------------------------------------------------------------------------
+def _cc_truth(ora, specsL, nL, specsR, nR, n_rows):
+    DL = ora.np_decompress(specsL, n_rows, nL)
+    DR = ora.np_decompress(specsR, n_rows, nR)
+    return DL, DR
+
+
+@pytest.mark.parametrize("seed,n_rows", [(0, 1), (1, 37), (2, 3000), (3, 20011)])
+@pytest.mark.parametrize("unc_l,unc_r", [(False, False), (True, False), (False, True), (True, True)])
+def test_lmm_compressed_equals_decompressed_product(ora, seed, n_rows, unc_l, unc_r):
+    specsL, nL = mixed_block(seed, n_rows, with_unc=unc_l)
+    specsR, nR = mixed_block(seed + 50, n_rows, with_unc=unc_r, with_const=seed % 2 == 0)
+    DL, DR = _cc_truth(ora, specsL, nL, specsR, nR, n_rows)
+    out, nnz = ora.lmm_compressed(ora.Groups(specsR, n_rows, nR), ora.Groups(specsL, n_rows, nL))
+    assert out.shape == (nL, nR)
+    assert_close(out, ora.longdouble_matmul(DL.T, DR), ora.abs_matmul(DL.T, DR))
+    assert nnz == np.count_nonzero(out)
+
+
+def test_lmm_compressed_tiny_fsum_truth(ora):
+    specsL, nL = mixed_block(11, 50)
+    specsR, nR = mixed_block(12, 50)
+    DL, DR = _cc_truth(ora, specsL, nL, specsR, nR, 50)
+    out, _ = ora.lmm_compressed(ora.Groups(specsR, 50, nR), ora.Groups(specsL, 50, nL))
+    assert_close(out, ora.fsum_matmul(DL.T, DR), ora.abs_matmul(DL.T, DR))
+
+
+def test_lmm_compressed_is_not_its_transpose(ora):
+    # a transposed operand (t(right) %*% left) or swapped output strides must fail: nL != nR and asymmetric data
+    specsL, nL = mixed_block(21, 400, with_unc=False, with_const=False)
+    specsR, nR = mixed_block(22, 400, with_unc=True)
+    assert nL != nR
+    DL, DR = _cc_truth(ora, specsL, nL, specsR, nR, 400)
+    out, _ = ora.lmm_compressed(ora.Groups(specsR, 400, nR), ora.Groups(specsL, 400, nL))
+    assert_close(out, ora.longdouble_matmul(DL.T, DR), ora.abs_matmul(DL.T, DR))
+    other, _ = ora.lmm_compressed(ora.Groups(specsL, 400, nL), ora.Groups(specsR, 400, nR))
+    assert_close(other, out.T, ora.abs_matmul(DR.T, DL))
+
+
+def test_lmm_compressed_same_block_is_tsmm(ora):
+    # left is right (same index structures, the dictionaries meet scaled by the counts): equals the TSMM
+    specs, n = mixed_block(31, 5000, with_unc=False)
+    G = ora.Groups(specs, 5000, n)
+    out, _ = ora.lmm_compressed(G, G)
+    D = ora.np_decompress(specs, 5000, n)
+    assert_close(out, ora.longdouble_matmul(D.T, D), ora.abs_matmul(D.T, D))
+    ts, _ = ora.tsmm(G)
+    assert_close(out, ts, 2 * ora.abs_matmul(D.T, D))
+
+
+def test_lmm_compressed_constants_only(ora):
+    # const x const: n * cL (x) cR exactly; const x DDC: cL (x) colSums(right)
+    from systemds_amd import synth
+    n = 1000
+    cl = synth.GroupSpec("const", np.array([0, 1], np.int32), np.array([[2.0, -3.0]]))
+    cr = synth.GroupSpec("const", np.array([0], np.int32), np.array([[0.5]]))
+    out, _ = ora.lmm_compressed(ora.Groups([cr], n, 1), ora.Groups([cl], n, 2))
+    assert np.array_equal(out, np.array([[1000.0], [-1500.0]]))
+    codes = (np.arange(n) % 4).astype(np.uint8)
+    dd = synth.GroupSpec("ddc", np.array([0], np.int32), np.array([[1.0], [2.0], [4.0], [8.0]]), codes)
+    out, _ = ora.lmm_compressed(ora.Groups([dd], n, 1), ora.Groups([cl], n, 2))
+    assert np.array_equal(out, np.array([[2.0 * 250 * 15], [-3.0 * 250 * 15]]))
