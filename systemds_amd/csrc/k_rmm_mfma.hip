@@ -284,8 +284,10 @@ __global__ __launch_bounds__(WAVES * 64) void k_rmm_mfma(const MfSlab* __restric
 		// writes one whole output row; + constV x B, count non-zeros.
 		// acc[m][n] of lane l is output row 16 m + 4 b + i (b = (l / 4) % 4, i = l / 16), column 4 n + l % 4.
 		__syncthreads();
-		const int col = n0 + lane;
-		const double cadd = (constRow != nullptr && col < q) ? constRow[col] : 0.0;
+		// (two columns per lane and two rows per store instruction: 1 KB per instruction)
+		const int col = n0 + 2 * (lane & 31), rsel = lane >> 5;
+		const double cadd0 = (constRow != nullptr && col < q) ? constRow[col] : 0.0;
+		const double cadd1 = (constRow != nullptr && col + 1 < q) ? constRow[col + 1] : 0.0;
 		double* st = stageS + (size_t) wave * 8 * MF_SS;
 #pragma unroll
 		for(int m = 0; m < MF_MT; m++) {
@@ -297,13 +299,21 @@ __global__ __launch_bounds__(WAVES * 64) void k_rmm_mfma(const MfSlab* __restric
 					for(int n = 0; n < MF_NJ; n++) p[4 * n] = acc[m][n];
 				}
 				__builtin_amdgcn_wave_barrier(); // same-wave LDS accesses complete in order
-				const int64_t row0 = blockRow0 + wave * (MF_MT * 16) + m * 16 + h * 8;
+				const int64_t row0 = blockRow0 + wave * (MF_MT * 16) + m * 16 + h * 8 + rsel;
 #pragma unroll
-				for(int r = 0; r < 8; r++) {
-					const double val = st[(size_t) r * MF_SS + lane] + cadd;
-					if(row0 + r < nRows && col < q) {
-						cnt += val != 0.0;
-						__builtin_nontemporal_store(val, &out[(size_t) (row0 + r) * q + col]);
+				for(int r = 0; r < 8; r += 2) {
+					f64x2 v = *(const f64x2*) (st + (size_t) (r + rsel) * MF_SS + 2 * (lane & 31));
+					v[0] += cadd0; v[1] += cadd1;
+					if(row0 + r < nRows) {
+						double* o = &out[(size_t) (row0 + r) * q + col];
+						if(col + 1 < q) {
+							cnt += (v[0] != 0.0) + (v[1] != 0.0);
+							__builtin_nontemporal_store(v, (f64x2*) o);
+						}
+						else if(col < q) {
+							cnt += v[0] != 0.0;
+							__builtin_nontemporal_store(v[0], o);
+						}
 					}
 				}
 				__builtin_amdgcn_wave_barrier();
