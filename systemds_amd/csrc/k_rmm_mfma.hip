@@ -31,14 +31,6 @@ constexpr int MF_BJ = 18;
 constexpr int MF_BK = 4 * MF_BJ;
 constexpr int MF_SS = 68;                    // row stride (doubles) of the output staging: 8 rows on distinct banks
 
-// decoded column c of a slab: where its values come from
-struct MfCol {
-	int32_t dictOff;   // offset (doubles) of the group's dictionary copy in the LDS slab, + j
-	int32_t nColG;     // tuple width of the group
-	int32_t group;     // group index
-	int32_t pad;
-};
-
 // code stream of a decoded column (device array: at row 0; LDS copy: at the block's first row)
 struct MfSrc {
 	const uint8_t* codes;
@@ -65,153 +57,101 @@ __global__ __launch_bounds__(128) void k_mfma_blayout(const double* __restrict__
 	Bl[(size_t) r * MF_BK + t] = (jg < 16 && gc >= 0 && col < q) ? B[(size_t) gc * q + col] : 0.0;
 }
 
-// LDS layout:
-//   dictS   the slab's dictionaries back to back behind two zero doubles
+// LDS layout: two slab buffers, then the code streams of all decoded columns (srcS) and the slab
+// descriptors (slabS), read once per block. A slab buffer holds
+//   dict    the slab's dictionaries back to back behind two zero doubles
 //   Bs      B rows of the slab's decoded columns (layout above)
-//   infoS   per decoded column of the slab dictOff | nColG << 16 (0 for padding columns: they read a zero)
-//   srcS    code streams of all decoded columns (row 0), slabS the slab descriptors: read once per block
-//   codeS   per decoded column of the slab the codes of the tile's rows, W bytes each: plain copies of
+//   info    per decoded column of the slab dictOff | nColG << 16 (0 for padding columns: they read a zero)
+//   codes   per decoded column of the slab the codes of the tile's rows, W bytes each: plain copies of
 //           the code streams (narrower codes are widened); rows behind the end hold 0
-// A block is persistent and walks (row tile, slab) pairs. The global loads of the next pair's fill (its
-// first pieces per thread; all addresses come from LDS or kernel arguments) are issued before the
-// multiply loop of the current pair and stored to LDS behind it, so the memory latency of a fill is
-// hidden under the matrix instructions. The decode of an A operand is two dependent LDS reads (code,
-// value) and one multiply-add, also under the matrix instructions.
+// A block is persistent and walks (row tile, slab) pairs, pair p in buffer p % 2. The fill of pair p + 1
+// is issued in front of the multiply loop of pair p as global -> LDS loads that bypass the registers
+// (global_load_lds_dwordx4: every lane fetches 16 bytes from its own address, the wave's 1 KB lands
+// contiguously in LDS), in pieces of 1 KB spread over the waves; one barrier per pair. The memory latency
+// of a fill is hidden under the matrix instructions, and so is the decode of an A operand (two dependent
+// LDS reads: code, value; one multiply-add).
+#define MF_GPTR(p) ((const __attribute__((address_space(1))) void*) (p))
+#define MF_LPTR(p) ((__attribute__((address_space(3))) void*) (p))
+
 template <int WAVES, int W>
 __global__ __launch_bounds__(WAVES * 64) void k_rmm_mfma(const MfSlab* __restrict__ slabs, int nSlabs,
-	const MfCol* __restrict__ cols, const MfSrc* __restrict__ colSrc, int nColsAll, const double* __restrict__ Bl, int q, int n0,
-	const double* __restrict__ constRow, double* __restrict__ out, int64_t nRows, int ldsDictDoubles, int ldsKc,
-	unsigned long long* __restrict__ nnz, int stagger) {
+	const uint32_t* __restrict__ infoG, const MfSrc* __restrict__ colSrc, int nColsAll, const double* __restrict__ Bl, int q, int n0,
+	const double* __restrict__ constRow, double* __restrict__ out, int64_t nRows, int ldsDictDoubles, int ldsKc, int bufBytes,
+	unsigned long long* __restrict__ nnz) {
 	constexpr int THREADS = WAVES * 64;
 	constexpr int ROWS = WAVES * MF_MT * 16; // rows per tile
 	extern __shared__ __align__(16) double smem[];
-	double* dictS = smem;                                   // ldsDictDoubles (even)
-	double* Bs = dictS + ldsDictDoubles;                    // ldsKc rows of MF_BK doubles
-	uint32_t* infoS = (uint32_t*) (Bs + (size_t) ldsKc * MF_BK); // ldsKc (multiple of 4)
-	MfSrc* srcS = (MfSrc*) (infoS + ldsKc);                 // nColsAll
+	uint8_t* const lds = (uint8_t*) smem;
+	// offsets inside a slab buffer
+	const int oB = ldsDictDoubles * 8, oInfo = oB + ldsKc * MF_BK * 8, oCodes = oInfo + ldsKc * 4;
+	MfSrc* srcS = (MfSrc*) (lds + 2 * (size_t) bufBytes);   // nColsAll
 	MfSlab* slabS = (MfSlab*) (srcS + nColsAll);            // nSlabs
-	uint8_t* codeS = (uint8_t*) (slabS + ((nSlabs + 1) & ~1)); // ldsKc tiles of ROWS codes (an even count keeps them 16-byte aligned)
-	double* stageS = smem;                                  // epilogue: WAVES x 8 rows x MF_SS, over the slab
 
-	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+	const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 	const int li = lane & 15, lk = lane >> 4, lj = lane & 3, lb = (lane >> 2) & 3;
 	const int nTiles = (int) ((nRows + ROWS - 1) / ROWS);
 
 	for(int c = tid; c < nColsAll; c += THREADS) srcS[c] = colSrc[c];
 	for(int i = tid; i < nSlabs; i += THREADS) slabS[i] = slabs[i];
+	if(tid < 4) *(double*) (lds + (size_t) (tid >> 1) * bufBytes + (tid & 1) * 8) = 0.0; // the zero doubles of both buffers
 	int cnt = 0;
-	// The blocks all have the same work per tile and would write their output tiles at the same moments;
-	// a start delay of 0-3 quarters of a tile's time spreads the output bursts over the other blocks'
-	// multiply phases.
-	if(stagger > 0 && nTiles > 4 * (int) gridDim.x) {
-		const long long until = __builtin_readcyclecounter() + (long long) (blockIdx.x & 3) * stagger;
-		while((long long) __builtin_readcyclecounter() < until) __builtin_amdgcn_s_sleep(32);
-	}
 	__syncthreads();
 
-	// ---- fill of (tile, slab): issue() loads the first pieces per thread into registers, commit() stores
-	// them and copies what did not fit (large slabs) directly
-	constexpr int NC_ = 2, NB_ = 3, ND_ = WAVES == 8 ? 3 : 8; // 16-byte pieces per thread in flight: codes, B, dictionaries
-	constexpr int perCol = ROWS * W / 16;
-	u32x4 tC[NC_];
-	f64x2 tB[NB_], tD[ND_];
-	uint32_t tI = 0;
-	// piece i of the code tiles: bytes [off, off + 16) of column c's tile
-	auto code_piece = [&](const MfSlab& sl, int64_t row0, int rowsHere, int i, bool& fast, const uint8_t*& src, int& gw, int& r0, int& dst) {
-		const int c = i / perCol, off = (i - c * perCol) * 16;
-		const MfSrc ms = srcS[sl.c0 + c];
-		gw = ms.width;
-		src = as_global(ms.codes) + (size_t) row0 * gw;
-		r0 = off / W;
-		dst = c * ROWS * W + off;
-		fast = gw == W && r0 + 16 / W <= rowsHere;
-		if(fast) src += off;
-	};
-	auto code_slow = [&](const uint8_t* src, int gw, int r0, int rowsHere) { // widened or ragged piece
-		uint32_t e[4] = {0, 0, 0, 0};
-		for(int t = 0; t < 16 / W; t++) {
-			const uint32_t code = r0 + t < rowsHere ? (uint32_t) load_code(src, gw, r0 + t) : 0u;
-			e[(t * W) >> 2] |= code << (8 * ((t * W) & 3));
-		}
-		return u32x4{e[0], e[1], e[2], e[3]};
-	};
-	auto issue = [&](int tile, int s) {
+	// ---- fill of (tile, slab) into buffer `buf`: pieces of 1 KB, piece pc by wave pc % WAVES
+	auto fill = [&](int tile, int s, int buf) {
 		const MfSlab sl = slabS[s];
 		const int64_t row0 = (int64_t) tile * ROWS;
 		const int rowsHere = (int) min((int64_t) ROWS, nRows - row0);
 		const int kc = (sl.nc + 3) & ~3;
-		tI = 0;
-		if(tid < sl.nc) {
-			const MfCol mc = cols[sl.c0 + tid];
-			tI = (uint32_t) mc.dictOff | ((uint32_t) mc.nColG << 16);
-		}
-#pragma unroll
-		for(int k = 0; k < NC_; k++) {
-			const int i = tid + k * THREADS;
-			if(i < sl.nc * perCol) {
-				bool fast; const uint8_t* src; int gw, r0, dst;
-				code_piece(sl, row0, rowsHere, i, fast, src, gw, r0, dst);
-				tC[k] = fast ? __builtin_nontemporal_load((const u32x4*) src) : code_slow(src, gw, r0, rowsHere);
+		uint8_t* const base = lds + (size_t) buf * bufBytes;
+		const int dictBytes = (sl.dictDoubles - 2) * 8, bBytes = kc * MF_BK * 8, infoBytes = kc * 4;
+		constexpr int colsPerPiece = 1024 / (ROWS * W) > 0 ? 1024 / (ROWS * W) : 1; // (ROWS * W is 256, 512 or 1024)
+		constexpr int piecesPerCol = ROWS * W / 1024 > 0 ? ROWS * W / 1024 : 1;
+		const int pDict = (dictBytes + 1023) >> 10, pB = (bBytes + 1023) >> 10, pInfo = (infoBytes + 1023) >> 10;
+		const int pCodes = (sl.nc + colsPerPiece - 1) / colsPerPiece * piecesPerCol;
+		const int nPieces = pDict + pB + pInfo + pCodes;
+		for(int pc = wave; pc < nPieces; pc += WAVES) {
+			if(pc < pDict) { // (an odd number of doubles: the last lane reads 8 bytes more; the allocation is padded)
+				const int off = pc * 1024 + lane * 16;
+				if(off < dictBytes)
+					__builtin_amdgcn_global_load_lds(MF_GPTR((const uint8_t*) as_global(sl.dictSrc) + off), MF_LPTR(base + 16 + pc * 1024), 16, 0, 0);
 			}
-		}
-		const f64x2* srcB = (const f64x2*) (Bl + (size_t) sl.kOff * MF_BK);
-#pragma unroll
-		for(int k = 0; k < NB_; k++)
-			if(tid + k * THREADS < kc * (MF_BK / 2)) tB[k] = srcB[tid + k * THREADS];
-		const double* srcD = as_global(sl.dictSrc);
-		const int nD = sl.dictDoubles - 2;
-#pragma unroll
-		for(int k = 0; k < ND_; k++) {
-			const int i = tid + k * THREADS;
-			if(2 * i + 1 < nD) tD[k] = *(const f64x2*) (srcD + 2 * i);
-			else if(2 * i < nD) tD[k] = f64x2{srcD[2 * i], 0.0};
-		}
-	};
-	auto commit = [&](int tile, int s) {
-		const MfSlab sl = slabS[s];
-		const int64_t row0 = (int64_t) tile * ROWS;
-		const int rowsHere = (int) min((int64_t) ROWS, nRows - row0);
-		const int kc = (sl.nc + 3) & ~3;
-		const int nChunksC = sl.nc * perCol, nChunksB = kc * (MF_BK / 2), nD = sl.dictDoubles - 2;
-		if(tid < 2) dictS[tid] = 0.0; // (the epilogue's staging lies over it)
-		if(tid < kc) infoS[tid] = tI;
-		for(int c = tid + THREADS; c < kc; c += THREADS) { // (more columns in a slab than threads: never with these tiles)
-			uint32_t info = 0;
-			if(c < sl.nc) info = (uint32_t) cols[sl.c0 + c].dictOff | ((uint32_t) cols[sl.c0 + c].nColG << 16);
-			infoS[c] = info;
-		}
-#pragma unroll
-		for(int k = 0; k < NC_; k++) {
-			const int i = tid + k * THREADS;
-			if(i < nChunksC) {
-				const int c = i / perCol, off = (i - c * perCol) * 16;
-				*(u32x4*) (codeS + c * ROWS * W + off) = tC[k];
+			else if(pc < pDict + pB) {
+				const int j = pc - pDict, off = j * 1024 + lane * 16;
+				if(off < bBytes)
+					__builtin_amdgcn_global_load_lds(MF_GPTR((const uint8_t*) (Bl + (size_t) sl.kOff * MF_BK) + off), MF_LPTR(base + oB + j * 1024), 16, 0, 0);
 			}
-		}
-#pragma unroll
-		for(int k = 0; k < NB_; k++)
-			if(tid + k * THREADS < nChunksB) ((f64x2*) Bs)[tid + k * THREADS] = tB[k];
-#pragma unroll
-		for(int k = 0; k < ND_; k++) {
-			const int i = tid + k * THREADS;
-			if(2 * i < nD) *(f64x2*) (dictS + 2 + 2 * i) = tD[k]; // (an odd end writes one zero behind the dictionaries)
-		}
-		for(int i = tid + NC_ * THREADS; i < nChunksC; i += THREADS) {
-			bool fast; const uint8_t* src; int gw, r0, dst;
-			code_piece(sl, row0, rowsHere, i, fast, src, gw, r0, dst);
-			*(u32x4*) (codeS + dst) = fast ? __builtin_nontemporal_load((const u32x4*) src) : code_slow(src, gw, r0, rowsHere);
-		}
-		const f64x2* srcB = (const f64x2*) (Bl + (size_t) sl.kOff * MF_BK);
-		for(int i = tid + NB_ * THREADS; i < nChunksB; i += THREADS) ((f64x2*) Bs)[i] = srcB[i];
-		const double* srcD = as_global(sl.dictSrc);
-		for(int i = tid + ND_ * THREADS; 2 * i < nD; i += THREADS) {
-			if(2 * i + 1 < nD) *(f64x2*) (dictS + 2 + 2 * i) = *(const f64x2*) (srcD + 2 * i);
-			else dictS[2 + 2 * i] = srcD[2 * i];
+			else if(pc < pDict + pB + pInfo) {
+				const int j = pc - pDict - pB, off = j * 1024 + lane * 16;
+				if(off < infoBytes)
+					__builtin_amdgcn_global_load_lds(MF_GPTR((const uint8_t*) (infoG + sl.kOff) + off), MF_LPTR(base + oInfo + j * 1024), 16, 0, 0);
+			}
+			else { // code tiles: lane -> (column, 16 bytes of its tile)
+				const int j = pc - pDict - pB - pInfo;
+				const int byte = j * 1024 + lane * 16; // inside the slab's code tiles
+				const int c = byte / (ROWS * W), off = byte - c * (ROWS * W);
+				if(c < sl.nc) {
+					const MfSrc ms = srcS[sl.c0 + c];
+					const uint8_t* src = as_global(ms.codes) + (size_t) row0 * ms.width;
+					const int r0 = off / W;
+					if(ms.width == W && r0 + 16 / W <= rowsHere)
+						__builtin_amdgcn_global_load_lds(MF_GPTR(src + off), MF_LPTR(base + oCodes + j * 1024), 16, 0, 0);
+					else { // widened or ragged piece: through registers
+						uint32_t e[4] = {0, 0, 0, 0};
+						for(int t = 0; t < 16 / W; t++) {
+							const uint32_t code = r0 + t < rowsHere ? (uint32_t) load_code(src, ms.width, r0 + t) : 0u;
+							e[(t * W) >> 2] |= code << (8 * ((t * W) & 3));
+						}
+						*(u32x4*) (base + oCodes + byte) = u32x4{e[0], e[1], e[2], e[3]};
+					}
+				}
+			}
 		}
 	};
 
 	// persistent block: row tiles blockIdx.x, + gridDim.x, ...
-	if((int) blockIdx.x < nTiles) issue(blockIdx.x, 0);
+	int buf = 0;
+	if((int) blockIdx.x < nTiles) fill(blockIdx.x, 0, 0);
 	for(int tile = blockIdx.x; tile < nTiles; tile += gridDim.x) {
 		const int64_t blockRow0 = (int64_t) tile * ROWS;
 		double acc[MF_MT][MF_NJ];
@@ -220,19 +160,23 @@ __global__ __launch_bounds__(WAVES * 64) void k_rmm_mfma(const MfSlab* __restric
 #pragma unroll
 			for(int n = 0; n < MF_NJ; n++) acc[m][n] = 0.0;
 
-		for(int s = 0; s < nSlabs; s++) {
+		for(int s = 0; s < nSlabs; s++, buf ^= 1) {
 			const int kc = (slabS[s].nc + 3) & ~3;
-			__syncthreads(); // the previous pair's readers (multiply loop, epilogue) are done
-			commit(tile, s);
+			// this wave's pieces of the pair's fill have landed; behind the barrier all of them have, and
+			// the other buffer's readers (the pair before) are done
+			__builtin_amdgcn_s_waitcnt(0x0f70); // vmcnt(0)
 			__syncthreads();
-			if(s + 1 < nSlabs) issue(tile, s + 1);
-			else if(tile + (int) gridDim.x < nTiles) issue(tile + gridDim.x, 0);
+			if(s + 1 < nSlabs) fill(tile, s + 1, buf ^ 1);
+			else if(tile + (int) gridDim.x < nTiles) fill(tile + gridDim.x, 0, buf ^ 1);
 
+			const uint8_t* const base = lds + (size_t) buf * bufBytes;
+			const double* dictS = (const double*) base;
+			const uint32_t* infoS = (const uint32_t*) (base + oInfo);
 			// software pipeline over k-steps of 4 decoded columns: codes and column info two steps ahead,
-			// values one step ahead; the B fragments in two halves, each loaded while the other is multiplied
-			const uint8_t* myCode = codeS + ((size_t) lk * ROWS + wave * (MF_MT * 16) + li) * W;
+			// values one step ahead; the B fragments in quarters, each loaded while the one before is multiplied
+			const uint8_t* myCode = base + oCodes + ((size_t) lk * ROWS + wave * (MF_MT * 16) + li) * W;
 			constexpr size_t codeStep = (size_t) 4 * ROWS * W;
-			const double* myB = Bs + (size_t) lk * MF_BK + lj * MF_BJ;
+			const double* myB = (const double*) (base + oB) + (size_t) lk * MF_BK + lj * MF_BJ;
 			auto codes_at = [&](int kt, int (&c)[MF_MT], uint32_t& info) {
 				const uint8_t* p = myCode + (size_t) (kt >> 2) * codeStep;
 				info = infoS[kt + lk];
@@ -266,7 +210,6 @@ __global__ __launch_bounds__(WAVES * 64) void k_rmm_mfma(const MfSlab* __restric
 				const int k2 = min(kt + 8, kc - 4), k1 = min(kt + 4, kc - 4);
 				codes_at(k2, c2, i2);
 				values_at(c1, i1, a1);
-				// the B fragments in quarters, each loaded while the one before is multiplied
 #define MF_QUARTER(QI, CUR, NXT, NKT, NQ)                                                                          \
 				b_quarter(NKT, NQ, NXT);                                                                             \
 				_Pragma("unroll") for(int m = 0; m < MF_MT; m++)                                                      \
@@ -280,10 +223,12 @@ __global__ __launch_bounds__(WAVES * 64) void k_rmm_mfma(const MfSlab* __restric
 			}
 		}
 
-		// epilogue: eight rows of a 16-row tile at a time through LDS, so that every store instruction
-		// writes one whole output row; + constV x B, count non-zeros.
+		// epilogue: eight rows of a 16-row tile at a time through LDS (over the buffer of the tile's last
+		// slab; the next pair's fill goes to the other one), so that every store instruction writes whole
+		// output rows; + constV x B, count non-zeros.
 		// acc[m][n] of lane l is output row 16 m + 4 b + i (b = (l / 4) % 4, i = l / 16), column 4 n + l % 4.
 		__syncthreads();
+		double* const stageS = (double*) (lds + (size_t) (buf ^ 1) * bufBytes); // (buf has moved on to the next pair's)
 		// (two columns per lane and two rows per store instruction: 1 KB per instruction)
 		const int col = n0 + 2 * (lane & 31), rsel = lane >> 5;
 		const double cadd0 = (constRow != nullptr && col < q) ? constRow[col] : 0.0;
@@ -319,17 +264,15 @@ __global__ __launch_bounds__(WAVES * 64) void k_rmm_mfma(const MfSlab* __restric
 				__builtin_amdgcn_wave_barrier();
 			}
 		}
+		if(tid < 2) stageS[tid] = 0.0; // the staging (of wave 0) lay over that buffer's zero doubles
 	} // tiles
 	count_add(nnz, cnt);
 }
 
-// LDS bytes: dictionaries (even count, so that the B slab is 16-byte aligned), B slab, column info,
-// code streams of all columns, code tiles
-static size_t mf_lds_bytes(size_t dictDoubles, int kc, int width, int rows, int nColsAll, int nSlabs) {
-	// (kc is a multiple of 4, the column sources are 16 bytes each, the slab descriptors 40: room for an even
-	// number of them keeps the code tiles 16-byte aligned)
-	return ((dictDoubles + 1) & ~(size_t) 1) * 8 + (size_t) kc * MF_BK * 8 + (size_t) kc * 4 + (size_t) nColsAll * sizeof(MfSrc) +
-		(size_t) ((nSlabs + 1) & ~1) * sizeof(MfSlab) + (size_t) kc * rows * width;
+// bytes of a slab buffer: dictionaries (even count, so that the B slab is 16-byte aligned), B slab, column
+// info (kc is a multiple of 4), code tiles
+static size_t mf_buf_bytes(size_t dictDoubles, int kc, int width, int rows) {
+	return ((dictDoubles + 1) & ~(size_t) 1) * 8 + (size_t) kc * MF_BK * 8 + (size_t) kc * 4 + (size_t) kc * rows * width;
 }
 
 // Host-side plan + launch. Returns 1 when the block/shape is not eligible (caller
@@ -344,98 +287,103 @@ int launch_rmm_mfma(cla_block* b, const double* dB, int q, const double* dConstR
 		nColsAll += g.d.nColG;
 		blockWidth = std::max(blockWidth, g.d.codeWidth);
 	}
-	// waves per block and LDS budget per slab: 8 waves (512-row tiles, two waves per SIMD) with 100 KiB measured
-	// best on the 10M x 100 DDC block (3.4 ms against 5.7 ms with 4 waves and two blocks per CU)
-	int waves = 8, budgetKb = 100;
+	// 8 waves per block (512-row tiles, two waves per SIMD), one block per CU with two slab buffers
+	int waves = 8;
 	if(const char* e = getenv("CLA_MFMA_WAVES")) waves = atoi(e) == 4 ? 4 : 8;
-	if(waves == 4) budgetKb = 76;
-	if(const char* e = getenv("CLA_MFMA_LDS_KB")) budgetKb = atoi(e);
 	const int rows = waves * MF_MT * 16;
-	const size_t budget = (size_t) std::min(g_ldsPerBlock - 1024, budgetKb * 1024);
+	const size_t stageBytes = (size_t) waves * 8 * MF_SS * 8;
+	int ldsKb = 156;
+	if(const char* e = getenv("CLA_MFMA_LDS_KB")) ldsKb = atoi(e);
+	const size_t fixedBytes = (size_t) nColsAll * sizeof(MfSrc) + 32 * sizeof(MfSlab);
+	const size_t ldsTotal = (size_t) std::min(g_ldsPerBlock - 1024, ldsKb * 1024);
+	if(ldsTotal < fixedBytes + 2 * stageBytes) return 1;
+	const size_t budget = (ldsTotal - fixedBytes) / 2 & ~(size_t) 15; // per slab buffer
+
 	std::vector<MfSlab> slabs;
-	std::vector<MfCol> cols;
+	std::vector<uint32_t> info;  // per slab row dictOff | nColG << 16, 0 = padding
 	std::vector<MfSrc> colSrc;
 	std::vector<int32_t> rowCol; // B row list: global column per slab row, -1 = padding
 	size_t maxDict = 0;
-	int maxKc = 0, maxWidth = 1;
-	int g = 0;
-	while(g < nG) {
-		MfSlab sl;
-		memset(&sl, 0, sizeof(sl));
-		sl.g0 = g; sl.c0 = (int) cols.size(); sl.kOff = (int) rowCol.size();
-		sl.dictSrc = b->groups[g].d.dict; // the block's dictionaries lie back to back in group order
-		size_t dictD = 2, goodDict = 2; // the leading zero doubles
-		int nc = 0, width = blockWidth, goodG = g, goodNc = 0, goodWidth = blockWidth;
+	int maxKc = 0;
+	// first pass: how many slabs the budget needs; second pass: the columns spread evenly over them
+	// (in multiples of four, the k-step), so that every fill has a whole multiply loop to hide under
+	int colCap = 1 << 30;
+	for(int pass = 0; pass < 2; pass++) {
+		slabs.clear(); info.clear(); colSrc.clear(); rowCol.clear();
+		maxDict = 0; maxKc = 0;
+		int g = 0;
 		while(g < nG) {
-			const DGroup& G = b->groups[g].d;
-			const size_t d2 = dictD + (size_t) G.nVals * G.nColG;
-			const int nc2 = nc + G.nColG;
-			const int kc2 = (nc2 + 3) & ~3;
-			const int w2 = blockWidth;
-			const size_t need = mf_lds_bytes(d2, kc2, w2, rows, nColsAll, 32);
-			if(need > budget || d2 > 65535 || G.nColG > 0x7fff) break; // dictionary offsets are 16 bit
-			for(int j = 0; j < G.nColG; j++) {
-				MfCol c;
-				c.dictOff = (int32_t) dictD + j; c.nColG = G.nColG; c.group = g; c.pad = 0;
-				cols.push_back(c);
-				MfSrc src;
-				src.codes = (const uint8_t*) G.codes; src.width = G.codeWidth; src.pad = 0;
-				colSrc.push_back(src);
-				rowCol.push_back(b->groups[g].cols[j]);
+			MfSlab sl;
+			memset(&sl, 0, sizeof(sl));
+			sl.g0 = g; sl.c0 = (int) colSrc.size(); sl.kOff = (int) rowCol.size();
+			sl.dictSrc = b->groups[g].d.dict; // the block's dictionaries lie back to back in group order
+			size_t dictD = 2, goodDict = 2; // the leading zero doubles
+			int nc = 0, goodG = g, goodNc = 0;
+			while(g < nG) {
+				const DGroup& G = b->groups[g].d;
+				const size_t d2 = dictD + (size_t) G.nVals * G.nColG;
+				const int nc2 = nc + G.nColG;
+				const size_t need = mf_buf_bytes(d2, (nc2 + 3) & ~3, blockWidth, rows);
+				if(need > budget || d2 > 65535 || G.nColG > 0x7fff) break; // dictionary offsets are 16 bit
+				if(nc > 0 && nc2 > colCap) break;
+				for(int j = 0; j < G.nColG; j++) {
+					info.push_back((uint32_t) (dictD + j) | ((uint32_t) G.nColG << 16));
+					MfSrc src;
+					src.codes = (const uint8_t*) G.codes; src.width = G.codeWidth; src.pad = 0;
+					colSrc.push_back(src);
+					rowCol.push_back(b->groups[g].cols[j]);
+				}
+				dictD = d2; nc = nc2;
+				g++;
+				if(nc % 4 == 0) { goodG = g; goodNc = nc; goodDict = dictD; }
 			}
-			dictD = d2; nc = nc2; width = w2;
-			g++;
-			if(nc % 4 == 0) { goodG = g; goodNc = nc; goodDict = dictD; goodWidth = width; }
+			if(g == sl.g0) return 1; // a single group does not fit LDS
+			// a slab that is not the last ends on a multiple of four columns if it can
+			if(g < nG && nc % 4 != 0 && goodG > sl.g0) {
+				info.resize(info.size() - (size_t) (nc - goodNc));
+				colSrc.resize(colSrc.size() - (size_t) (nc - goodNc));
+				rowCol.resize(rowCol.size() - (size_t) (nc - goodNc));
+				g = goodG; nc = goodNc; dictD = goodDict;
+			}
+			sl.g1 = g; sl.nc = nc; sl.dictDoubles = (int32_t) dictD; sl.width = blockWidth;
+			while(rowCol.size() % 4) { rowCol.push_back(-1); info.push_back(0); }
+			maxDict = std::max(maxDict, (dictD + 1) & ~(size_t) 1);
+			maxKc = std::max(maxKc, (nc + 3) & ~3);
+			slabs.push_back(sl);
 		}
-		if(g == sl.g0) return 1; // a single group does not fit LDS
-		// k-steps take four decoded columns: a slab that is not the last ends on a multiple of four if it can
-		if(g < nG && nc % 4 != 0 && goodG > sl.g0) {
-			cols.resize(cols.size() - (size_t) (nc - goodNc));
-			colSrc.resize(colSrc.size() - (size_t) (nc - goodNc));
-			rowCol.resize(rowCol.size() - (size_t) (nc - goodNc));
-			g = goodG; nc = goodNc; dictD = goodDict; width = goodWidth;
-		}
-		sl.g1 = g; sl.nc = nc; sl.dictDoubles = (int32_t) dictD; sl.width = width;
-		while(rowCol.size() % 4) rowCol.push_back(-1);
-		maxDict = std::max(maxDict, (dictD + 1) & ~(size_t) 1);
-		maxKc = std::max(maxKc, (nc + 3) & ~3);
-		maxWidth = std::max(maxWidth, width);
-		slabs.push_back(sl);
+		if(slabs.size() > 32) return 1;
+		if(pass == 0) colCap = std::max(4, (int) ((nColsAll + slabs.size() - 1) / slabs.size() + 3) / 4 * 4);
 	}
+	// (colSrc is indexed by decoded column, info and rowCol by slab row: they differ by the padding rows)
 	hipStream_t st = b->stream;
 	auto up16 = [](size_t n) { return (n + 15) & ~(size_t) 15; };
-	const size_t oSlabs = 0, oCols = up16(oSlabs + slabs.size() * sizeof(MfSlab)), oSrc = up16(oCols + cols.size() * sizeof(MfCol)),
+	const size_t oSlabs = 0, oInfo = up16(oSlabs + slabs.size() * sizeof(MfSlab)), oSrc = up16(oInfo + info.size() * 4 + 16),
 		oRowCol = up16(oSrc + colSrc.size() * sizeof(MfSrc)), oBl = up16(oRowCol + rowCol.size() * 4),
 		total = oBl + rowCol.size() * MF_BK * 8;
 	int rc = ensure_scratch(b, total + 256);
 	if(rc) return rc;
 	char* base = (char*) b->dScratch;
 	MfSlab* dSlabs = (MfSlab*) (base + oSlabs);
-	MfCol* dCols = (MfCol*) (base + oCols);
+	uint32_t* dInfo = (uint32_t*) (base + oInfo);
 	MfSrc* dSrc = (MfSrc*) (base + oSrc);
 	int32_t* dRowCol = (int32_t*) (base + oRowCol);
 	double* dBl = (double*) (base + oBl);
 	CLA_HIP(hipMemcpyAsync(dSlabs, slabs.data(), slabs.size() * sizeof(MfSlab), hipMemcpyHostToDevice, st));
-	CLA_HIP(hipMemcpyAsync(dCols, cols.data(), cols.size() * sizeof(MfCol), hipMemcpyHostToDevice, st));
+	CLA_HIP(hipMemcpyAsync(dInfo, info.data(), info.size() * 4, hipMemcpyHostToDevice, st));
 	CLA_HIP(hipMemcpyAsync(dSrc, colSrc.data(), colSrc.size() * sizeof(MfSrc), hipMemcpyHostToDevice, st));
 	CLA_HIP(hipMemcpyAsync(dRowCol, rowCol.data(), rowCol.size() * 4, hipMemcpyHostToDevice, st));
 	CLA_HIP(hipStreamSynchronize(st)); // the host vectors go out of scope
 
-	if(slabs.size() > 32) return 1; // (the plan above reserves LDS for 32 descriptors)
-	const size_t lds = std::max(mf_lds_bytes(maxDict, maxKc, maxWidth, rows, nColsAll, (int) slabs.size()), (size_t) waves * 8 * MF_SS * 8);
+	const size_t bufBytes = up16(std::max(mf_buf_bytes(maxDict, maxKc, blockWidth, rows), stageBytes));
+	const size_t lds = 2 * bufBytes + (size_t) nColsAll * sizeof(MfSrc) + slabs.size() * sizeof(MfSlab);
 	CLA_HIP(hipFuncSetAttribute((const void*) k_rmm_mfma<4, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
 	CLA_HIP(hipFuncSetAttribute((const void*) k_rmm_mfma<8, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
 	CLA_HIP(hipFuncSetAttribute((const void*) k_rmm_mfma<4, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
 	CLA_HIP(hipFuncSetAttribute((const void*) k_rmm_mfma<8, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
-	// persistent blocks: as many as fit the device at once (LDS bound), each walks its row tiles
-	const int perCU = std::max(1, std::min(2, (int) ((size_t) 160 * 1024 / (lds + 512))));
-	const unsigned grid = (unsigned) std::min<int64_t>((b->nRows + rows - 1) / rows, (int64_t) g_numCU * perCU);
+	// persistent blocks: one per CU, each walks its row tiles
+	const unsigned grid = (unsigned) std::min<int64_t>((b->nRows + rows - 1) / rows, (int64_t) g_numCU);
 	double codeBytes = 0;
 	for(auto& gr : b->groups) codeBytes += (double) b->nRows * gr.d.codeWidth;
-	// cycles between the starts of blocks: a quarter of a tile's multiply time (64 matrix instructions of about
-	// 17 cycles per k-step and wave, two waves per SIMD)
-	int stagger = (int) (rowCol.size() / 4) * 64 * 17 * 2 / 4;
-	if(const char* e = getenv("CLA_MFMA_STAGGER")) stagger = atoi(e);
 	for(int n0 = 0; n0 < q; n0 += 64) {
 		const int qq = std::min(64, q - n0);
 		{
@@ -444,8 +392,8 @@ int launch_rmm_mfma(cla_block* b, const double* dB, int q, const double* dConstR
 		}
 		Prof pf(b, "k_rmm_mfma", grid, waves * 64, (long) lds, codeBytes + (double) b->nRows * qq * 8);
 #define MF_LAUNCH(WV, CW)                                                                                            \
-	hipLaunchKernelGGL((k_rmm_mfma<WV, CW>), dim3(grid), dim3(WV * 64), lds, st, dSlabs, (int) slabs.size(), dCols, dSrc, \
-		nColsAll, dBl, q, n0, dConstRow, dOut, b->nRows, (int) maxDict, maxKc, dNnz, stagger)
+	hipLaunchKernelGGL((k_rmm_mfma<WV, CW>), dim3(grid), dim3(WV * 64), lds, st, dSlabs, (int) slabs.size(), dInfo, dSrc, \
+		nColsAll, dBl, q, n0, dConstRow, dOut, b->nRows, (int) maxDict, maxKc, (int) bufBytes, dNnz)
 		if(waves == 8) { if(blockWidth == 1) MF_LAUNCH(8, 1); else MF_LAUNCH(8, 2); }
 		else { if(blockWidth == 1) MF_LAUNCH(4, 1); else MF_LAUNCH(4, 2); }
 #undef MF_LAUNCH
