@@ -672,6 +672,8 @@ int64_t cla_tsmm(cla_handle b, double* out) {
 	return nnz;
 }
 
+} // extern "C"
+
 namespace cla {
 
 __global__ __launch_bounds__(256) void k_take_block(const double* __restrict__ G, int n, int r0, int c0, int nr, int nc,
@@ -731,6 +733,8 @@ static cla_block* make_joint(cla_block* left, cla_block* right) {
 }
 
 } // namespace cla
+
+extern "C" {
 
 int64_t cla_lmm_compressed_dev(cla_handle right, cla_handle left, double* dOut) {
 	int rc = check_final(right);
