@@ -490,10 +490,21 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 			dec_wave_sync();
 			const int64_t rowBase = t0 + pbase;
 			const int nr = (int) max((int64_t) 0, min((int64_t) PROWS, nRows - rowBase));
-			for(int i = lane; i < nr * q; i += 64) {
-				const double v = wstage[i];
-				cnt += v != 0.0;
-				__builtin_nontemporal_store(v, A.out + (size_t) rowBase * q + i);
+			// the pass's rows are one contiguous range of the output: 16 bytes per lane (the range starts on a
+			// multiple of 16 bytes: rowBase is a multiple of 16 rows), a single double at an odd end
+			{
+				const int n = nr * q;
+				double* o = A.out + (size_t) rowBase * q;
+				for(int i = 2 * lane; i + 1 < n; i += 128) {
+					const f64x2 v = *(const f64x2*) (wstage + i);
+					cnt += (v[0] != 0.0) + (v[1] != 0.0);
+					__builtin_nontemporal_store(v, (f64x2*) (o + i));
+				}
+				if((n & 1) && lane == 0) {
+					const double v = wstage[n - 1];
+					cnt += v != 0.0;
+					__builtin_nontemporal_store(v, o + n - 1);
+				}
 			}
 		}
 	}
