@@ -116,3 +116,34 @@ def test_errors(cla):
     assert e.value.code == cla.ERR_UNSUPPORTED
     wide.close()
     unc.close()
+
+
+def test_overlapping_operand_is_refused(cla, ora):
+    """An overlapping block (the result of cla_rmm_overlapping) is not linear per cell pair: refused like in TSMM."""
+    n_rows = 5000
+    specs, n = mixed_block(11, n_rows, with_unc=False)
+    blk = cla.build_block(n_rows, n, specs)
+    child = blk.rmm_overlapping(np.random.default_rng(1).standard_normal((n, 3)))
+    with pytest.raises(cla.ClaError) as e:
+        blk.lmm_compressed(child)
+    assert e.value.code == cla.ERR_UNSUPPORTED
+    with pytest.raises(cla.ClaError) as e:
+        child.lmm_compressed(blk)
+    assert e.value.code == cla.ERR_UNSUPPORTED
+    # the refusal leaves both blocks usable
+    out, _ = blk.lmm_compressed(blk)
+    D = ora.np_decompress(specs, n_rows, n)
+    assert_matches_truth(out, D.T, D, what="after refusal")
+    child.close()
+    blk.close()
+
+
+def test_constants_only_on_one_side(cla, ora):
+    """A block of const / empty groups only against a mixed block: the outer products with the column sums."""
+    from systemds_amd import synth
+    n_rows = 3000
+    consts = [synth.GroupSpec("const", np.array([0, 2], np.int32), np.array([[1.5, -2.0]])),
+              synth.GroupSpec("empty", np.array([1], np.int32))]
+    specs, n = mixed_block(12, n_rows, with_unc=False)
+    check(cla, ora, consts, 3, specs, n, n_rows, "const %*% mixed")
+    check(cla, ora, specs, n, consts, 3, n_rows, "mixed %*% const")
