@@ -744,9 +744,12 @@ int64_t cla_lmm_compressed_dev(cla_handle right, cla_handle left, double* dOut) 
 		set_error("compressed left multiply: %lld rows on the left, %lld on the right", (long long) left->nRows, (long long) right->nRows);
 		return -CLA_ERR_INVALID;
 	}
-	std::lock_guard<std::recursive_mutex> lk(right->mu);
-	std::unique_lock<std::recursive_mutex> lk2(left->mu, std::defer_lock);
-	if(left != right) lk2.lock();
+	// both blocks' locks, in address order (two threads may call with the roles swapped)
+	cla_block* const first = left < right ? left : right;
+	cla_block* const second = left < right ? right : left;
+	std::lock_guard<std::recursive_mutex> lk(first->mu);
+	std::unique_lock<std::recursive_mutex> lk2(second->mu, std::defer_lock);
+	if(second != first) lk2.lock();
 	if(!right->joint || right->jointSerial != left->serial) {
 		if(right->joint) { cla_block_free(right->joint); right->joint = nullptr; }
 		right->joint = make_joint(left, right);
@@ -782,7 +785,11 @@ int64_t cla_lmm_compressed(cla_handle right, cla_handle left, double* out) {
 	if(rc || (rc = check_final(left))) return rc;
 	if(!out) { set_error("compressed left multiply: null output"); return -CLA_ERR_INVALID; }
 	const size_t nOut = (size_t) left->nCols * right->nCols;
-	std::lock_guard<std::recursive_mutex> lk(right->mu);
+	cla_block* const first = left < right ? left : right;
+	cla_block* const second = left < right ? right : left;
+	std::lock_guard<std::recursive_mutex> lk(first->mu);
+	std::unique_lock<std::recursive_mutex> lk2(second->mu, std::defer_lock);
+	if(second != first) lk2.lock();
 	if((rc = ensure_stage(&right->dStageOut, &right->stageOutCap, nOut))) return rc;
 	const int64_t nnz = cla_lmm_compressed_dev(right, left, right->dStageOut);
 	if(nnz < 0) return nnz;
