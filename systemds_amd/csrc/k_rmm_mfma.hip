@@ -297,7 +297,8 @@ int launch_rmm_mfma(cla_block* b, const double* dB, int q, const double* dConstR
 	const size_t fixedBytes = (size_t) nColsAll * sizeof(MfSrc) + 32 * sizeof(MfSlab);
 	const size_t ldsTotal = (size_t) std::min(g_ldsPerBlock - 1024, ldsKb * 1024);
 	if(ldsTotal < fixedBytes + 2 * stageBytes) return 1;
-	const size_t budget = (ldsTotal - fixedBytes) / 2 & ~(size_t) 15; // per slab buffer
+	size_t budget = (ldsTotal - fixedBytes) / 2 & ~(size_t) 15; // per slab buffer
+	auto up16 = [](size_t n) { return (n + 15) & ~(size_t) 15; };
 
 	std::vector<MfSlab> slabs;
 	std::vector<uint32_t> info;  // per slab row dictOff | nColG << 16, 0 = padding
@@ -307,6 +308,9 @@ int launch_rmm_mfma(cla_block* b, const double* dB, int q, const double* dConstR
 	int maxKc = 0;
 	// first pass: how many slabs the budget needs; second pass: the columns spread evenly over them
 	// (in multiples of four, the k-step), so that every fill has a whole multiply loop to hide under
+	// The kernel lays a buffer out for the largest dictionary range and the largest column count of any slab,
+	// which need not be the same slab: when two such buffers exceed LDS, the plan is redone on a smaller budget.
+	for(int attempt = 0;; attempt++) {
 	int colCap = 1 << 30;
 	for(int pass = 0; pass < 2; pass++) {
 		slabs.clear(); info.clear(); colSrc.clear(); rowCol.clear();
@@ -354,9 +358,12 @@ int launch_rmm_mfma(cla_block* b, const double* dB, int q, const double* dConstR
 		if(slabs.size() > 32) return 1;
 		if(pass == 0) colCap = std::max(4, (int) ((nColsAll + slabs.size() - 1) / slabs.size() + 3) / 4 * 4);
 	}
+	if(2 * up16(std::max(mf_buf_bytes(maxDict, maxKc, blockWidth, rows), stageBytes)) + fixedBytes <= ldsTotal) break;
+	if(attempt == 8) return 1;
+	budget = (budget * 3 / 4) & ~(size_t) 15;
+	}
 	// (colSrc is indexed by decoded column, info and rowCol by slab row: they differ by the padding rows)
 	hipStream_t st = b->stream;
-	auto up16 = [](size_t n) { return (n + 15) & ~(size_t) 15; };
 	const size_t oSlabs = 0, oInfo = up16(oSlabs + slabs.size() * sizeof(MfSlab)), oSrc = up16(oInfo + info.size() * 4 + 16),
 		oRowCol = up16(oSrc + colSrc.size() * sizeof(MfSrc)), oBl = up16(oRowCol + rowCol.size() * 4),
 		total = oBl + rowCol.size() * MF_BK * 8;

@@ -137,3 +137,31 @@ def test_error_behaviour(cla):
         blk.add_sdc([0], np.ones((1, 1)), None, np.zeros(3, np.uint8), np.array([5, 7], np.uint8), 1, 99, 3)
         blk.finalize()
     blk.close()
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_wide_right_multiply_on_uneven_ddc_blocks(cla, ora, seed):
+    """All-DDC blocks with dictionaries of very different sizes, tuple widths 1-3, both code widths and wide B:
+    the matrix-core right multiply cuts them into LDS slabs. Seed 1 (512 rows, 38 groups, 55 columns) has its
+    largest dictionary range and its largest column count in different slabs."""
+    from systemds_amd import synth
+    rng = np.random.default_rng(2024)
+    for _ in range(seed + 1):   # the seed-th block of one random sequence
+        n_rows = int(rng.choice([1, 15, 511, 512, 513, 1000, 4097, 20000, 70001]))
+        specs, c = [], 0
+        for _g in range(int(rng.integers(1, 40))):
+            nc = int(rng.choice([1, 1, 1, 2, 3]))
+            nv = int(rng.choice([2, 16, 200, 256, 300, 1000, 3000]))
+            codes = rng.integers(0, nv, n_rows).astype(np.uint8 if nv <= 256 else np.uint16)
+            specs.append(synth.GroupSpec("ddc", np.arange(c, c + nc, dtype=np.int32), rng.standard_normal((nv, nc)), codes))
+            c += nc
+        if rng.random() < 0.3:
+            specs.append(synth.GroupSpec("const", np.array([c], np.int32), np.array([[1.25]])))
+            c += 1
+        q = int(rng.choice([8, 9, 16, 33, 64, 65, 100]))
+        B = rng.standard_normal((c, q))
+    out, nnz, ref, rnnz = run_both(cla, ora, specs, n_rows, c, B)
+    D = ora.np_decompress(specs, n_rows, c)
+    assert_matches_truth(out, D, B, what=f"uneven DDC block {seed}")
+    assert_fp64_close(out, ref, abs_scale(ora, specs, n_rows, c, B), what=f"uneven DDC block {seed}", n_terms=c)
+    assert nnz == rnnz
