@@ -472,8 +472,12 @@ int launch_tsmm(cla_block* b, double* dOut, unsigned long long* dNnz) {
 			if(acc + (size_t) 2 * TT * 4 > (size_t) 150 * 1024) { pairsFit = false; break; }
 		}
 	const bool mustDecode = b->hasUnc || forceDecode || (!pairsFit && nCols <= 64);
+	// As many groups as columns: the reference decompresses (CLALibTSMM.java:73-77); here that is the decoded
+	// Gram matrix up to 64 columns. Wider blocks without uncompressed groups go per pair (the scalar
+	// decompressing fallback is slower and ends at 110 columns) unless CLA_TSMM_WIDE_DENSE asks for it.
+	const bool wideDense = nCols > 64 && nG >= nCols && (!pairsFit || getenv("CLA_TSMM_WIDE_DENSE") != nullptr);
 	const bool dense = split > 0 ? mustDecode || (nCols <= 64 && (nG >= nCols || gramCheaper) && !forcePairs)
-	                             : nG >= nCols || mustDecode || (gramCheaper && !forcePairs);
+	                             : mustDecode || wideDense || (nCols <= 64 && (nG >= nCols || gramCheaper) && !forcePairs);
 	if(dense && split > 0 && nCols > 64) {
 		set_error("compressed left multiply: uncompressed groups need at most 64 columns over both blocks (have %d)", nCols);
 		return -CLA_ERR_UNSUPPORTED;

@@ -81,6 +81,20 @@ def test_single_column_groups_use_dense_path(cla, ora):
     check_tsmm(cla, ora, c["groups"], c["n_rows"], c["n_cols"], "C2-like")
 
 
+@pytest.mark.parametrize("wide_dense", [False, True])
+def test_wide_blocks_of_single_column_groups(cla, ora, monkeypatch, wide_dense):
+    """More than 64 columns, as many groups as columns: per pair of groups (the default), or the scalar
+    decompressing fallback up to 110 columns on request; beyond that only the per-pair path exists."""
+    from systemds_amd import synth
+    if wide_dense:
+        monkeypatch.setenv("CLA_TSMM_WIDE_DENSE", "1")
+    c = synth.config2(scale=500, n_cols=100)
+    check_tsmm(cla, ora, c["groups"], c["n_rows"], c["n_cols"], f"C2 100 columns dense={wide_dense}")
+    if not wide_dense:
+        c = synth.config4(scale=500, n_cols=130)
+        check_tsmm(cla, ora, c["groups"], c["n_rows"], c["n_cols"], "C4-like 130 columns")
+
+
 def test_cooc_bit_exact(cla, ora):
     specs, n_cols = mixed_block(31, 60007, with_unc=False)
     blk = cla.build_block(60007, n_cols, specs)
