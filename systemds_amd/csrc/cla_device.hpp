@@ -225,6 +225,18 @@ struct CodeVec {
 		if(CW == 2) return (raw.word(i >> 1) >> (16 * (i & 1))) & 0xffffu;
 		return (int) raw.word(i);
 	}
+	// code i times 8 (the byte offset of an fp64 table entry). The compiler turns bytes 1-3 of a word into one
+	// shift with a byte-select operand but byte 0 into a shift and a mask; written out, byte 0 is one
+	// instruction as well (two vector instructions per table lookup are the floor of the gather kernels).
+	__device__ __forceinline__ uint32_t off8(int i) const {
+		if(CW == 1 && (i & 3) == 0) {
+			uint32_t r;
+			asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_0"
+				: "=v"(r) : "v"(3u), "v"(raw.word(i >> 2)));
+			return r;
+		}
+		return (uint32_t) get(i) << 3;
+	}
 };
 
 // Batch request with a uniform base and a 32-bit per-thread offset: the address of every load

@@ -224,7 +224,7 @@ __device__ __forceinline__ void u8_consume(const CodeVec<1, RPT> (&cv)[NB], cons
 	auto issue = [&](int b) {
 		const int j = (b * LB) / RPT, i0 = (b * LB) % RPT;
 #pragma unroll
-		for(int k = 0; k < LB; k++) t[b % LN][k] = *(const double*) (tb + j * 2048 + (cv[j].get(i0 + k) << 3));
+		for(int k = 0; k < LB; k++) t[b % LN][k] = *(const double*) (tb + j * 2048 + cv[j].off8(i0 + k));
 	};
 #pragma unroll
 	for(int b = 0; b < LN - 1 && b < NBATCH; b++) issue(b);
