@@ -227,7 +227,7 @@ struct CodeVec {
 	}
 	// code i times 8 (the byte offset of an fp64 table entry). The compiler turns bytes 1-3 of a word into one
 	// shift with a byte-select operand but byte 0 into a shift and a mask; written out, byte 0 is one
-	// instruction as well (two vector instructions per table lookup are the floor of the gather kernels).
+	// instruction as well, so that a table lookup costs two vector instructions (offset, add).
 	__device__ __forceinline__ uint32_t off8(int i) const {
 		if(CW == 1 && (i & 3) == 0) {
 			uint32_t r;
