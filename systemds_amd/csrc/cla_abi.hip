@@ -140,6 +140,7 @@ static int upload_dict(HostGroup& g) {
 }
 
 int finish_finalize(cla_block* b, cla_block* arenaFrom, bool buildArena = true);
+static void free_subs(cla_block* b);
 
 } // namespace cla
 
@@ -215,6 +216,7 @@ void cla_block_free(cla_handle b) {
 	if(b->refs.fetch_sub(1) > 1) return; // blocks made from this one still use its streams
 	cla_block* parent = b->parent;
 	if(b->joint) { cla_block_free(b->joint); b->joint = nullptr; }
+	free_subs(b);
 	if(g_device >= 0) (void) hipSetDevice(g_device);
 	if(b->stream) (void) hipStreamSynchronize(b->stream);
 	clear_stats(b);
@@ -730,6 +732,180 @@ static cla_block* make_joint(cla_block* left, cla_block* right) {
 	c->maxVals = maxVals;
 	if(finish_finalize(c, nullptr, false)) { cla_block_free(c); return nullptr; }
 	return c;
+}
+
+// ---------------------------------------------------------------------------
+// t(X) %*% X of a block with more than 64 columns through the decoded Gram matrix: the columns are cut
+// into chunks of at most 32 (groups stay whole; columns that only carry a constant go along), every
+// pair of chunks becomes a block of its own of at most 64 columns that borrows the row data of `b`
+// (built once, kept with `b`), and its Gram matrix is scattered into the result. For a joint block
+// (crossSplit > 0) only chunks of the left side meet chunks of the right side.
+// ---------------------------------------------------------------------------
+struct SubBlock {
+	cla_block* blk;
+	int32_t* dColMap;   // column of `b` per column of blk
+	int nA, nB;         // columns of the first / second chunk
+	bool writeA, writeB, crossOnly;
+};
+
+__global__ __launch_bounds__(256) void k_scatter_gram(const double* __restrict__ S, int k, const int32_t* __restrict__ colMap, int nA,
+	int writeA, int writeB, int crossOnly, double* __restrict__ out, int n) {
+	for(int idx = threadIdx.x + blockIdx.x * 256; idx < k * k; idx += 256 * gridDim.x) {
+		const int r = idx / k, c = idx - r * k;
+		const bool rA = r < nA, cA = c < nA;
+		bool take;
+		if(rA && cA) take = writeA && !crossOnly;
+		else if(!rA && !cA) take = writeB && !crossOnly;
+		else take = crossOnly ? rA : true; // joint block: the (left, right) block only, the caller takes it from the upper half
+		if(take) out[(size_t) colMap[r] * n + colMap[c]] = S[idx];
+	}
+}
+
+static void free_subs(cla_block* b) {
+	for(void* p : b->subs) {
+		SubBlock* sb = (SubBlock*) p;
+		if(sb->dColMap) (void) hipFree(sb->dColMap);
+		if(sb->blk) cla_block_free(sb->blk);
+		delete sb;
+	}
+	b->subs.clear();
+}
+
+// chunk = groups and constant-only columns of b
+struct Chunk { std::vector<int> groups, constCols; int nCols = 0; };
+
+static cla_block* make_sub(cla_block* b, const Chunk& A, const Chunk& B, bool cross, std::vector<int32_t>& colMap) {
+	cla_block* c = cla_block_create(b->nRows, A.nCols + B.nCols);
+	if(!c) return nullptr;
+	colMap.clear();
+	int tblOff = 0, colOff = 0, maxVals = 0;
+	for(int side = 0; side < 2; side++) {
+		const Chunk& ch = side ? B : A;
+		for(int gi : ch.groups) {
+			const HostGroup& pg = b->groups[gi];
+			c->groups.emplace_back();
+			HostGroup& g = c->groups.back();
+			g.d = pg.d; // row data: borrowed
+			g.cols.resize(pg.cols.size());
+			for(size_t j = 0; j < pg.cols.size(); j++) {
+				g.cols[j] = (int32_t) colMap.size();
+				c->constV[colMap.size()] = b->constV[pg.cols[j]];
+				colMap.push_back(pg.cols[j]);
+			}
+			g.dict = pg.dict;
+			g.bytes = 0;
+			if(upload(g, g.cols.data(), sizeof(int32_t) * g.cols.size(), (const void**) &g.d.cols) ||
+				(!g.dict.empty() && upload_dict(g))) {
+				cla_block_free(c);
+				return nullptr;
+			}
+			g.bytes = pg.bytes;
+			g.d.tblOff = tblOff;
+			g.d.colOff = colOff;
+			tblOff += g.d.nVals;
+			colOff += g.d.nColG;
+			maxVals = std::max(maxVals, g.d.nVals);
+			if(g.d.type == G_SDCZ) c->hasSdc = true;
+			if(g.d.type == G_RLE) c->hasRle = true;
+			if(g.d.type == G_UNC) c->hasUnc = true;
+		}
+		for(int col : ch.constCols) {
+			c->constV[colMap.size()] = b->constV[col];
+			colMap.push_back(col);
+		}
+		if(side == 0 && cross) c->crossSplit = (int32_t) c->groups.size();
+	}
+	c->hasConst = b->hasConst;
+	c->totalVals = tblOff;
+	c->totalColsG = colOff;
+	c->maxVals = maxVals;
+	if(finish_finalize(c, nullptr, false)) { cla_block_free(c); return nullptr; }
+	return c;
+}
+
+// Returns 1 when the block cannot be cut that way (a group of more than 32 columns), 0 when dOut (n x n,
+// zeroed by the caller) holds the result: full symmetric, or for a joint block its (left, right) part.
+int launch_tsmm_chunked(cla_block* b, double* dOut) {
+	const int n = b->nCols, nG = (int) b->groups.size(), split = b->crossSplit;
+	if(b->subs.empty()) {
+		// chunks per side (one side when the block is no joint block); joint blocks: left columns are those of
+		// the first `split` groups and, of the constant-only ones, those in front of the right side's first column
+		std::vector<char> covered((size_t) n, 0);
+		for(auto& g : b->groups)
+			for(int c : g.cols) covered[c] = 1;
+		int firstRight = n;
+		if(split > 0)
+			for(int g = split; g < nG; g++)
+				for(int c : b->groups[g].cols) firstRight = std::min(firstRight, c);
+		std::vector<Chunk> chunks[2];
+		auto add_item = [&](int side, int group, int col, int width) -> bool {
+			if(width > 32) return false;
+			auto& v = chunks[side];
+			if(v.empty() || v.back().nCols + width > 32) v.emplace_back();
+			if(group >= 0) v.back().groups.push_back(group); else v.back().constCols.push_back(col);
+			v.back().nCols += width;
+			return true;
+		};
+		for(int g = 0; g < nG; g++)
+			if(!add_item(split > 0 && g >= split ? 1 : 0, g, -1, b->groups[g].d.nColG)) return 1;
+		for(int c = 0; c < n; c++)
+			if(!covered[c] && !add_item(split > 0 && c >= firstRight ? 1 : 0, -1, c, 1)) return 1;
+		std::vector<std::pair<int, int>> pairs; // (chunk of side 0, chunk of side 0 or 1)
+		const int m0 = (int) chunks[0].size(), m1 = (int) chunks[1].size();
+		if(split > 0) {
+			for(int i = 0; i < m0; i++)
+				for(int j = 0; j < m1; j++) pairs.emplace_back(i, j);
+		}
+		else {
+			if(m0 < 2) return 1;
+			for(int i = 0; i < m0; i++)
+				for(int j = i + 1; j < m0; j++) pairs.emplace_back(i, j);
+		}
+		for(auto& pr : pairs) {
+			const Chunk& A = chunks[0][pr.first];
+			const Chunk& B = split > 0 ? chunks[1][pr.second] : chunks[0][pr.second];
+			SubBlock* sb = new SubBlock();
+			sb->blk = nullptr; sb->dColMap = nullptr;
+			b->subs.push_back(sb);
+			std::vector<int32_t> colMap;
+			sb->blk = make_sub(b, A, B, split > 0, colMap);
+			if(!sb->blk) { free_subs(b); return -CLA_ERR_DEVICE; }
+			sb->nA = A.nCols; sb->nB = B.nCols;
+			sb->crossOnly = split > 0;
+			// every diagonal block once: chunk i with its successor, the last chunk with its predecessor
+			sb->writeA = split == 0 && pr.second == pr.first + 1;
+			sb->writeB = split == 0 && pr.first == m0 - 2 && pr.second == m0 - 1;
+			if(hipMalloc((void**) &sb->dColMap, sizeof(int32_t) * colMap.size()) != hipSuccess ||
+				hipMemcpy(sb->dColMap, colMap.data(), sizeof(int32_t) * colMap.size(), hipMemcpyHostToDevice) != hipSuccess) {
+				set_error("tsmm: column map of a chunk pair could not be uploaded");
+				free_subs(b);
+				return -CLA_ERR_DEVICE;
+			}
+		}
+	}
+	for(void* p : b->subs) {
+		SubBlock* sb = (SubBlock*) p;
+		cla_block* c = sb->blk;
+		c->profile = b->profile;
+		if(c->stream != b->stream) {
+			if(c->ownStream && c->stream) { (void) hipStreamSynchronize(c->stream); (void) hipStreamDestroy(c->stream); }
+			c->stream = b->stream;
+			c->ownStream = false;
+		}
+		const int k = c->nCols;
+		int rc = ensure_stage(&c->dStageOut, &c->stageOutCap, (size_t) k * k);
+		if(rc) return rc;
+		if((rc = launch_tsmm(c, c->dStageOut, c->dCounters))) return rc;
+		{
+			Prof pf(c, "k_scatter_gram", (k * k + 255) / 256, 256, 0, 0);
+			hipLaunchKernelGGL(k_scatter_gram, dim3((unsigned) ((k * k + 255) / 256)), dim3(256), 0, b->stream, c->dStageOut, k, sb->dColMap,
+				sb->nA, sb->writeA ? 1 : 0, sb->writeB ? 1 : 0, sb->crossOnly ? 1 : 0, dOut, n);
+		}
+		CLA_HIP(hipGetLastError());
+		b->lastStats.insert(b->lastStats.end(), c->lastStats.begin(), c->lastStats.end());
+		c->lastStats.clear(); // (the events moved along)
+	}
+	return 0;
 }
 
 } // namespace cla

@@ -85,6 +85,9 @@ struct cla_block {
 	cla_block* joint = nullptr;
 	uint64_t jointSerial = 0;
 	int32_t crossSplit = 0;          // > 0: joint block, groups [0, crossSplit) are the left side's
+	// blocks of pairs of column chunks for t(X) %*% X on more than 64 columns (launch_tsmm_chunked): built on
+	// first use, they borrow this block's row data and are freed with it
+	std::vector<void*> subs;
 	std::vector<cla::HostGroup> groups;
 	std::vector<double> constV;      // filtered constants (SDC defaults, const groups), nCols
 	bool hasConst = false;
@@ -181,6 +184,7 @@ int launch_decompress(cla_block* b, double* dOut, unsigned long long* dNnz);
 int launch_lmm(cla_block* b, const double* dY, int p, double* dOut, unsigned long long* dNnz);
 int launch_preagg(cla_block* b, int group, const double* dY, int p, double* dPre);
 int launch_tsmm(cla_block* b, double* dOut, unsigned long long* dNnz);
+int launch_tsmm_chunked(cla_block* b, double* dOut);
 int launch_cooc(cla_block* b, int gA, int gB, unsigned long long* dOut);
 int launch_mmchain(cla_block* b, const double* dV, const double* dW, int ctype, double* dOut,
 	unsigned long long* dNnz);

@@ -56,7 +56,7 @@ struct DecCopy {
 struct DecCol {
 	int32_t slotOff;   // dictionary coded: code tile (bytes into the code tiles)
 	int32_t valOff;    // doubles from the LDS base: dictionary copy / dense tile
-	int32_t meta;      // kind (0 none or constant only, 1 dictionary coded, 2 dense) | two-byte codes << 2 | dictionary in global memory << 3 | nC << 4 | h << 18
+	int32_t meta;      // kind (0 none or constant only, 1 dictionary coded with a no-value code, 2 dense, 3 dictionary coded on every row) | two-byte codes << 2 | dictionary in global memory << 3 | nC << 4 | h << 18
 	int32_t pad;       // group
 };
 
@@ -102,10 +102,10 @@ struct DecLook {
 	bool coded, dense, two;
 	__device__ __forceinline__ DecLook(const DecCol D) {
 		const int kind = D.meta & 3;
-		coded = kind == 1; dense = kind == 2; two = (D.meta & 4) != 0;
+		coded = kind == 1 || kind == 3; dense = kind == 2; two = (D.meta & 4) != 0;
 		nC = (D.meta >> 4) & 0x3fff;
 		base = D.valOff + (int) ((unsigned) D.meta >> 18);
-		sent = coded ? (two ? 0xffff : 0xff) : -1;
+		sent = kind == 1 ? (two ? 0xffff : 0xff) : -1; // (kind 3: every row has a code, all code values are valid)
 	}
 	// LDS index (doubles) of the value at tile row rt with code c, and whether the row has one.
 	// Rows behind the end of the matrix (in == false) hold stale codes: never used as an index.
@@ -629,7 +629,9 @@ static int dec_prepare(cla_block* b, bool gram, int q, int rpl, DecLaunch& L, si
 			P.dictOff = (int32_t) valD;
 			valD += (size_t) G.nVals * G.nColG;
 		}
-		P.slotW = G.nVals <= 255 ? 1 : 2;
+		// DDC codes of one or two bytes keep their width (plain copies; no value is set aside for rows without a
+		// code); the others are stored with 0xff / 0xffff for such rows
+		P.slotW = G.type == G_DDC && G.codeWidth <= 2 ? G.codeWidth : G.nVals <= 255 ? 1 : 2;
 		P.slotOff = (int32_t) slotB;
 		slotB += (size_t) DEC_TILE * P.slotW + DEC_SLOT_PAD;
 	}
@@ -712,11 +714,11 @@ static int dec_prepare(cla_block* b, bool gram, int q, int rpl, DecLaunch& L, si
 			if(gram && seen[hc[h]]) return 1; // overlapping groups
 			seen[hc[h]] = 1;
 			DecCol& C = cols[gram ? hc[h] : P.kOff + h];
-			const int kind = P.type == G_UNC ? 2 : P.slotOff >= 0 ? 1 : 0;
-			C.slotOff = kind == 1 ? P.slotOff : 0;
+			const int kind = P.type == G_UNC ? 2 : P.slotOff >= 0 ? (P.type == G_DDC ? 3 : 1) : 0;
+			C.slotOff = kind == 1 || kind == 3 ? P.slotOff : 0;
 			C.valOff = kind && P.dictOff >= 0 ? P.dictOff : 0;
 			C.pad = g;
-			C.meta = (int32_t) ((uint32_t) kind | (P.slotW == 2 ? 4u : 0u) | (kind == 1 && P.dictOff < 0 ? 8u : 0u) | ((uint32_t) P.nC << 4) | ((uint32_t) h << 18));
+			C.meta = (int32_t) ((uint32_t) kind | (P.slotW == 2 ? 4u : 0u) | ((kind == 1 || kind == 3) && P.dictOff < 0 ? 8u : 0u) | ((uint32_t) P.nC << 4) | ((uint32_t) h << 18));
 		}
 	}
 	const size_t planBytes = plan.size() * sizeof(DecGroup), copyBytes = copies.size() * sizeof(DecCopy);
@@ -787,6 +789,7 @@ int launch_tsmm_decode(cla_block* b, double* dOut) {
 		flat = true;
 		rc = dec_prepare(b, true, 0, 4, L, 512);
 	}
+	if(rc == 1) rc = dec_prepare(b, true, 0, 4, L, 64); // many mid-sized dictionaries: only the small ones in LDS
 	if(rc) return rc;
 	L.A.out = dOut;
 	Prof pf(b, "k_tsmm_decode", L.grid, DEC_THREADS, (long) L.lds, (double) b->device_bytes_cached);

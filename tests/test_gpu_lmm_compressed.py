@@ -105,17 +105,16 @@ def test_errors(cla):
     assert e.value.code == cla.ERR_INVALID
     left.close()
     right.close()
-    # uncompressed groups with more than 64 columns over both blocks: no per-pair form, not supported
+
+
+def test_uncompressed_groups_on_wide_blocks(cla, ora):
+    """More than 64 columns over both blocks and an uncompressed group: chunks of the left side meet chunks of the
+    right side as decoded blocks of at most 64 columns."""
     from systemds_amd import synth
     a = synth.config2(scale=1000, n_cols=70)
     specsU, nU = mixed_block(3, a["n_rows"], with_unc=True)
-    wide = cla.build_block(a["n_rows"], a["n_cols"], a["groups"])
-    unc = cla.build_block(a["n_rows"], nU, specsU)
-    with pytest.raises(cla.ClaError) as e:
-        wide.lmm_compressed(unc)
-    assert e.value.code == cla.ERR_UNSUPPORTED
-    wide.close()
-    unc.close()
+    check(cla, ora, specsU, nU, a["groups"], a["n_cols"], a["n_rows"], "t(unc) %*% wide")
+    check(cla, ora, a["groups"], a["n_cols"], specsU, nU, a["n_rows"], "t(wide) %*% unc")
 
 
 def test_overlapping_operand_is_refused(cla, ora):

@@ -81,18 +81,41 @@ def test_single_column_groups_use_dense_path(cla, ora):
     check_tsmm(cla, ora, c["groups"], c["n_rows"], c["n_cols"], "C2-like")
 
 
-@pytest.mark.parametrize("wide_dense", [False, True])
-def test_wide_blocks_of_single_column_groups(cla, ora, monkeypatch, wide_dense):
-    """More than 64 columns, as many groups as columns: per pair of groups (the default), or the scalar
-    decompressing fallback up to 110 columns on request; beyond that only the per-pair path exists."""
+@pytest.mark.parametrize("path", [None, "CLA_TSMM_PAIRS", "CLA_TSMM_NO_CHUNKS"])
+def test_wide_blocks_of_single_column_groups(cla, ora, monkeypatch, path):
+    """More than 64 columns, as many groups as columns: the decoded Gram matrices of pairs of 32-column chunks
+    (the default with that many pairs of groups), or one pass per pair of groups (forced, or chunks switched off)."""
     from systemds_amd import synth
-    if wide_dense:
-        monkeypatch.setenv("CLA_TSMM_WIDE_DENSE", "1")
+    if path:
+        monkeypatch.setenv(path, "1")
     c = synth.config2(scale=500, n_cols=100)
-    check_tsmm(cla, ora, c["groups"], c["n_rows"], c["n_cols"], f"C2 100 columns dense={wide_dense}")
-    if not wide_dense:
-        c = synth.config4(scale=500, n_cols=130)
-        check_tsmm(cla, ora, c["groups"], c["n_rows"], c["n_cols"], "C4-like 130 columns")
+    check_tsmm(cla, ora, c["groups"], c["n_rows"], c["n_cols"], f"C2 100 columns {path}")
+    c = synth.config4(scale=500, n_cols=130)
+    check_tsmm(cla, ora, c["groups"], c["n_rows"], c["n_cols"], f"C4-like 130 columns {path}")
+
+
+def wide_mixed_block(seed, n_rows, extra_cols=70):
+    """mixed_block (every group type, uncompressed and constant columns included) plus single- and two-column
+    DDC groups up to more than 64 columns."""
+    from systemds_amd import synth
+    specs, c = mixed_block(seed, n_rows, with_unc=True)
+    rng = np.random.default_rng(seed + 900)
+    while c < 11 + extra_cols:
+        nc = int(rng.choice([1, 2]))
+        nv = int(rng.choice([5, 200, 700]))
+        codes = rng.integers(0, nv, n_rows).astype(np.uint8 if nv <= 256 else np.uint16)
+        specs.append(synth.GroupSpec("ddc", np.arange(c, c + nc, dtype=np.int32), rng.standard_normal((nv, nc)), codes))
+        c += nc
+    return specs, c
+
+
+@pytest.mark.parametrize("seed,n_rows", [(1, 37), (2, 3000), (3, 70001)])
+def test_wide_block_with_uncompressed_group(cla, ora, seed, n_rows):
+    """More than 64 columns with an uncompressed group: no per-pair form exists, the block is cut into column
+    chunks whose pairwise decoded Gram matrices are scattered into the result."""
+    specs, n_cols = wide_mixed_block(seed, n_rows)
+    assert n_cols > 64
+    check_tsmm(cla, ora, specs, n_rows, n_cols, "wide block with an uncompressed group")
 
 
 def test_cooc_bit_exact(cla, ora):
