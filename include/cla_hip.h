@@ -127,8 +127,9 @@ int64_t cla_tsmm_dev(cla_handle h, double* dOut);
  * both blocks with the same number of rows. Every group of `left` meets every group of `right`
  * once (AColGroup.leftMultByAColGroup), the filtered constants of both sides enter through the
  * outer products with the column sums. Returns nnz(out) or a negative error; blocks with
- * overlapping groups are not supported, and uncompressed groups only while both blocks together
- * have at most 64 columns. The first call on a pair of handles builds a small joint descriptor. */
+ * overlapping groups are not supported, and beyond 64 columns of both blocks together an
+ * uncompressed group may span at most 32 columns. The first call on a pair of handles builds a
+ * small joint descriptor (and, on more than 64 joint columns, descriptors of column chunks). */
 int64_t cla_lmm_compressed(cla_handle right, cla_handle left, double* out);
 int64_t cla_lmm_compressed_dev(cla_handle right, cla_handle left, double* dOut);
 
