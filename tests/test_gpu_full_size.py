@@ -135,6 +135,38 @@ def test_c2_counts_exact(c2):
         assert int(got.sum()) == c["n_rows"]
 
 
+def test_c2_gram_of_100_single_column_groups(c2):
+    """t(X) %*% X of the 100-column block (column chunks, decoded Gram matrix per pair of chunks): the gram
+    identity on all cells, diagonal cells from the counts and cells of two pairs of groups (inside one chunk
+    and across chunks) from the integer co-occurrence table."""
+    c, blk, _ = c2
+    n, m = c["n_rows"], c["n_cols"]
+    T, nnz = blk.tsmm()
+    assert T.shape == (m, m)
+    assert np.array_equal(T, T.T)
+    assert nnz == np.count_nonzero(T)
+    v = np.random.default_rng(10).standard_normal((m, 1))
+    Xv, _ = blk.rmm(v)
+    lhs = float((v.T.astype(np.longdouble) @ T.astype(np.longdouble) @ v.astype(np.longdouble))[0, 0])
+    assert_scalar_close(lhs, ld_dot(Xv, Xv), float((np.abs(v).T @ np.abs(T) @ np.abs(v))[0, 0]), "C2 v'(X'X)v == |Xv|^2")
+    for g in (0, 31, 32, 64, 99):
+        s = c["groups"][g]
+        cl = np.bincount(s.codes, minlength=s.n_vals).astype(np.longdouble)
+        d = s.dict[:, 0].astype(np.longdouble)
+        a = int(s.cols[0])
+        assert abs(T[a, a] - float(np.sum(cl * d * d))) <= 1e-12 * float(np.sum(cl * d * d)), (g, T[a, a])
+    for ga, gb in ((3, 20), (5, 70), (40, 99)):
+        sa, sb = c["groups"][ga], c["groups"][gb]
+        co = np.bincount(sa.codes.astype(np.int64) * sb.n_vals + sb.codes, minlength=sa.n_vals * sb.n_vals)
+        co = co.reshape(sa.n_vals, sb.n_vals)
+        assert np.array_equal(blk.cooc(ga, gb), co)
+        da, db = sa.dict[:, 0].astype(np.longdouble), sb.dict[:, 0].astype(np.longdouble)
+        want = float(da @ co.astype(np.longdouble) @ db)
+        sc = float(np.abs(da) @ co.astype(np.longdouble) @ np.abs(db))
+        i, j = int(sa.cols[0]), int(sb.cols[0])
+        assert abs(T[i, j] - want) <= 1e-12 * sc, (ga, gb, T[i, j], want)
+
+
 # --------------------------------------------------------------------------- C3
 @pytest.fixture(scope="module")
 def c3(cla):
@@ -183,6 +215,23 @@ def test_c3_tsmm_properties(c3):
                 sc = float(np.abs(da) @ col @ np.abs(db))
                 i, j = int(sa.cols[p]), int(sb.cols[q])
                 assert abs(T[i, j] - want) <= 1e-12 * sc, (ga, gb, i, j, T[i, j], want)
+
+
+def test_c3_with_itself_as_two_compressed_operands(c3, cla):
+    """t(L) %*% R with a second, separately built copy of the block on the left (100 joint columns: column
+    chunks) equals the block's own Gram matrix."""
+    c, blk = c3
+    n, m = c["n_rows"], c["n_cols"]
+    T, nnz = blk.tsmm()
+    left = cla.build_block(n, m, c["groups"])
+    try:
+        out, onnz = blk.lmm_compressed(left)
+    finally:
+        left.close()
+    assert out.shape == (m, m)
+    cm = col_max(c["groups"], m)
+    assert_fp64_close(out, T, n * np.outer(cm, cm), what="C3 t(X)%*%X as compressed x compressed", n_terms=int(np.sqrt(n)))
+    assert onnz == np.count_nonzero(out)
 
 
 # --------------------------------------------------------------------------- C4
