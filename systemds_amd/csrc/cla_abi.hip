@@ -691,15 +691,21 @@ __global__ __launch_bounds__(256) void k_take_block(const double* __restrict__ G
 }
 
 // cbind(left, right) as a block of its own: the groups of `left` first, then those of `right` with
-// their columns shifted by left->nCols. Row data (codes, offsets, runs, dense values) is borrowed
-// from the two blocks, which must outlive it; column lists and dictionaries are its own copies.
+// their columns shifted by left->nCols (rounded up to a multiple of 16 with empty columns between while the whole
+// stays within 64 columns: the decoded Gram kernel then computes the left x right tiles only). Row data (codes,
+// offsets, runs, dense values) is borrowed from the two blocks, which must outlive it; column lists and
+// dictionaries are its own copies. The right side's columns are the last right->nCols ones.
 static cla_block* make_joint(cla_block* left, cla_block* right) {
-	cla_block* c = cla_block_create(left->nRows, left->nCols + right->nCols);
+	const int padL = (left->nCols + 15) / 16 * 16;
+	const bool padded = padL + right->nCols <= 64;
+	const int rightStart = padded ? padL : left->nCols;
+	cla_block* c = cla_block_create(left->nRows, rightStart + right->nCols);
 	if(!c) return nullptr;
+	if(padded) c->crossBlocks = padL / 16;
 	int tblOff = 0, colOff = 0, maxVals = 0;
 	for(int side = 0; side < 2; side++) {
 		cla_block* src = side ? right : left;
-		const int shift = side ? left->nCols : 0;
+		const int shift = side ? rightStart : 0;
 		for(auto& pg : src->groups) {
 			c->groups.emplace_back();
 			HostGroup& g = c->groups.back();
@@ -743,8 +749,8 @@ static cla_block* make_joint(cla_block* left, cla_block* right) {
 // ---------------------------------------------------------------------------
 struct SubBlock {
 	cla_block* blk;
-	int32_t* dColMap;   // column of `b` per column of blk
-	int nA, nB;         // columns of the first / second chunk
+	int32_t* dColMap;   // column of `b` per column of blk (-1: padding behind the first chunk)
+	int nA, nB;         // columns of the first (padding included) / second chunk
 	bool writeA, writeB, crossOnly;
 };
 
@@ -757,7 +763,7 @@ __global__ __launch_bounds__(256) void k_scatter_gram(const double* __restrict__
 		if(rA && cA) take = writeA && !crossOnly;
 		else if(!rA && !cA) take = writeB && !crossOnly;
 		else take = crossOnly ? rA : true; // joint block: the (left, right) block only, the caller takes it from the upper half
-		if(take) out[(size_t) colMap[r] * n + colMap[c]] = S[idx];
+		if(take && colMap[r] >= 0 && colMap[c] >= 0) out[(size_t) colMap[r] * n + colMap[c]] = S[idx];
 	}
 }
 
@@ -774,8 +780,12 @@ static void free_subs(cla_block* b) {
 // chunk = groups and constant-only columns of b
 struct Chunk { std::vector<int> groups, constCols; int nCols = 0; };
 
+// cross: only the product of chunk A with chunk B will be read. A's columns are then padded with empty columns to
+// a multiple of 16, so that the decoded Gram kernel can leave out the tiles inside A and inside B, and the
+// per-pair form leaves out the pairs of groups of one chunk.
 static cla_block* make_sub(cla_block* b, const Chunk& A, const Chunk& B, bool cross, std::vector<int32_t>& colMap) {
-	cla_block* c = cla_block_create(b->nRows, A.nCols + B.nCols);
+	const int padA = cross ? (A.nCols + 15) / 16 * 16 : A.nCols;
+	cla_block* c = cla_block_create(b->nRows, padA + B.nCols);
 	if(!c) return nullptr;
 	colMap.clear();
 	int tblOff = 0, colOff = 0, maxVals = 0;
@@ -813,7 +823,11 @@ static cla_block* make_sub(cla_block* b, const Chunk& A, const Chunk& B, bool cr
 			c->constV[colMap.size()] = b->constV[col];
 			colMap.push_back(col);
 		}
-		if(side == 0 && cross) c->crossSplit = (int32_t) c->groups.size();
+		if(side == 0 && cross) {
+			c->crossSplit = (int32_t) c->groups.size();
+			c->crossBlocks = padA / 16;
+			while((int) colMap.size() < padA) { c->constV[colMap.size()] = 0.0; colMap.push_back(-1); }
+		}
 	}
 	c->hasConst = b->hasConst;
 	c->totalVals = tblOff;
@@ -867,14 +881,14 @@ int launch_tsmm_chunked(cla_block* b, double* dOut) {
 			SubBlock* sb = new SubBlock();
 			sb->blk = nullptr; sb->dColMap = nullptr;
 			b->subs.push_back(sb);
-			std::vector<int32_t> colMap;
-			sb->blk = make_sub(b, A, B, split > 0, colMap);
-			if(!sb->blk) { free_subs(b); return -CLA_ERR_DEVICE; }
-			sb->nA = A.nCols; sb->nB = B.nCols;
-			sb->crossOnly = split > 0;
 			// every diagonal block once: chunk i with its successor, the last chunk with its predecessor
 			sb->writeA = split == 0 && pr.second == pr.first + 1;
 			sb->writeB = split == 0 && pr.first == m0 - 2 && pr.second == m0 - 1;
+			sb->crossOnly = split > 0;
+			std::vector<int32_t> colMap;
+			sb->blk = make_sub(b, A, B, split > 0 || (!sb->writeA && !sb->writeB), colMap);
+			if(!sb->blk) { free_subs(b); return -CLA_ERR_DEVICE; }
+			sb->nA = (int) colMap.size() - B.nCols; sb->nB = B.nCols;
 			if(hipMalloc((void**) &sb->dColMap, sizeof(int32_t) * colMap.size()) != hipSuccess ||
 				hipMemcpy(sb->dColMap, colMap.data(), sizeof(int32_t) * colMap.size(), hipMemcpyHostToDevice) != hipSuccess) {
 				set_error("tsmm: column map of a chunk pair could not be uploaded");
@@ -948,7 +962,7 @@ int64_t cla_lmm_compressed_dev(cla_handle right, cla_handle left, double* dOut) 
 	{
 		Prof pf(c, "k_take_block", (nOut + 255) / 256, 256, 0, 0);
 		hipLaunchKernelGGL(k_take_block, dim3((unsigned) std::min((nOut + 255) / 256, 1024)), dim3(256), 0, right->stream,
-			c->dStageOut, (int) n, 0, left->nCols, left->nCols, right->nCols, dOut, right->dCounters);
+			c->dStageOut, (int) n, 0, c->nCols - right->nCols, left->nCols, right->nCols, dOut, right->dCounters);
 	}
 	CLA_HIP(hipGetLastError());
 	clear_stats(right);

@@ -1,6 +1,7 @@
 // Decode-and-multiply on blocks of any group mix, on the matrix cores:
 //   k_rmm_decode      X %*% B for narrow B (2 <= q <= 16)
-//   k_tsmm_decode<NB> upper triangle of t(X) %*% X for blocks of at most 16 * NB <= 64 columns
+//   k_tsmm_decode<NB> upper triangle of t(X) %*% X for blocks of at most 16 * NB <= 64 columns (or, for a pair of
+//               column chunks, only the tiles of the first chunk's column blocks with the second's)
 // A block owns a contiguous range of 1024-row tiles. Per tile every dictionary coded
 // group gets its codes expanded into an LDS code tile (DDC: straight copy, prefetched one
 // tile ahead in registers together with the rows of uncompressed groups; SDCZeros:
@@ -140,7 +141,7 @@ __device__ __forceinline__ void dec_load_window(uint8_t* win, const uint8_t* src
 
 // FLAT: dictionaries that do not fit LDS stay in global memory; the lookups then go through
 // generic pointers (LDS or global per lane).
-template <int GRAM, int NB, int RPL, int FLAT>
+template <int GRAM, int NB, int RPL, int FLAT, int XB = 0>
 __device__ __forceinline__ void decode_body(const DecArgs& A) {
 	extern __shared__ __align__(16) double smem[];
 	double* Bs = smem + A.valDoubles;                              // bDoubles: rows of B in decoded column order, 16 outputs each
@@ -246,10 +247,13 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 	prefetch(tileBeg);
 
 	// multiply phase state
-	f64x4 gram[GRAM ? NB * (NB + 1) / 2 : 1];
+	// tiles of the Gram matrix held by a wave: the upper triangle, or with XB > 0 (only the product of the first
+	// XB column blocks with the others is wanted) those XB x (NB - XB) tiles
+	constexpr int NTILES = !GRAM ? 1 : XB > 0 ? XB * (NB - XB) : NB * (NB + 1) / 2;
+	f64x4 gram[NTILES];
 	if(GRAM) {
 #pragma unroll
-		for(int t = 0; t < NB * (NB + 1) / 2; t++) gram[t] = f64x4{0.0, 0.0, 0.0, 0.0};
+		for(int t = 0; t < NTILES; t++) gram[t] = f64x4{0.0, 0.0, 0.0, 0.0};
 	}
 	const int q = A.q;
 	const double cinit = (!GRAM && A.constRow != nullptr && i16 < q) ? A.constRow[i16] : 0.0;
@@ -434,9 +438,9 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 						for(int cb = 0; cb < NB; cb++) x[u][cb] = in ? cst[cb] + x[u][cb] : 0.0;
 						int t = 0;
 #pragma unroll
-						for(int ib = 0; ib < NB; ib++)
+						for(int ib = 0; ib < (XB > 0 ? XB : NB); ib++)
 #pragma unroll
-							for(int jb = ib; jb < NB; jb++, t++)
+							for(int jb = (XB > 0 ? XB : ib); jb < NB; jb++, t++)
 								gram[t] = __builtin_amdgcn_mfma_f64_16x16x4f64(x[u][ib], x[u][jb], gram[t], 0, 0, 0);
 					}
 				}
@@ -517,9 +521,9 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 		__syncthreads();
 		int t = 0;
 #pragma unroll
-		for(int ib = 0; ib < NB; ib++)
+		for(int ib = 0; ib < (XB > 0 ? XB : NB); ib++)
 #pragma unroll
-			for(int jb = ib; jb < NB; jb++, t++)
+			for(int jb = (XB > 0 ? XB : ib); jb < NB; jb++, t++)
 #pragma unroll
 				for(int v = 0; v < 4; v++)
 					unsafeAtomicAdd(&stage[(ib * 16 + 4 * v + k4) * NP + jb * 16 + i16], gram[t][v]);
@@ -536,8 +540,8 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 template <int RPL>
 __global__ __launch_bounds__(DEC_THREADS) void k_rmm_decode(const DecArgs A) { decode_body<0, 1, RPL, 0>(A); }
 
-template <int NB, int FLAT>
-__global__ __launch_bounds__(DEC_THREADS) void k_tsmm_decode(const DecArgs A) { decode_body<1, NB, 4, FLAT>(A); }
+template <int NB, int FLAT, int XB>
+__global__ __launch_bounds__(DEC_THREADS) void k_tsmm_decode(const DecArgs A) { decode_body<1, NB, 4, FLAT, XB>(A); }
 
 // One code per row for an RLE group (0xff where no run covers the row): thread = 4 rows.
 __global__ __launch_bounds__(256) void k_expand_rle(const DGroup* __restrict__ groups, int g, int64_t nRows, uint8_t* __restrict__ codes) {
@@ -782,6 +786,10 @@ int launch_tsmm_decode(cla_block* b, double* dOut) {
 	const int nCols = b->nCols;
 	if(b->groups.empty() || b->nRows == 0 || nCols > 64) return 1;
 	const int NB = (nCols + 15) / 16;
+	// only the product of the first crossBlocks column blocks with the others is wanted (a pair of column chunks
+	// whose own Gram matrices nobody reads): shapes 1 x 1, 1 x 2, 2 x 1, 2 x 2 blocks, anything else in full
+	int XB = b->crossBlocks;
+	if(XB < 1 || XB > 2 || NB - XB < 1 || NB - XB > 2) XB = 0;
 	DecLaunch L;
 	bool flat = false;
 	int rc = dec_prepare(b, true, 0, 4, L);
@@ -793,23 +801,27 @@ int launch_tsmm_decode(cla_block* b, double* dOut) {
 	if(rc) return rc;
 	L.A.out = dOut;
 	Prof pf(b, "k_tsmm_decode", L.grid, DEC_THREADS, (long) L.lds, (double) b->device_bytes_cached);
-#define GRAM_LAUNCH(NBV, FL)                                                                                    \
+#define GRAM_LAUNCH(NBV, FL, XBV)                                                                               \
 	do {                                                                                                        \
-		CLA_HIP(hipFuncSetAttribute((const void*) k_tsmm_decode<NBV, FL>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) L.lds)); \
-		hipLaunchKernelGGL((k_tsmm_decode<NBV, FL>), dim3(L.grid), dim3(DEC_THREADS), L.lds, b->stream, L.A);   \
+		CLA_HIP(hipFuncSetAttribute((const void*) k_tsmm_decode<NBV, FL, XBV>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) L.lds)); \
+		hipLaunchKernelGGL((k_tsmm_decode<NBV, FL, XBV>), dim3(L.grid), dim3(DEC_THREADS), L.lds, b->stream, L.A); \
 	} while(0)
-	if(!flat) {
-		if(NB == 1) GRAM_LAUNCH(1, 0);
-		else if(NB == 2) GRAM_LAUNCH(2, 0);
-		else if(NB == 3) GRAM_LAUNCH(3, 0);
-		else GRAM_LAUNCH(4, 0);
-	}
-	else {
-		if(NB == 1) GRAM_LAUNCH(1, 1);
-		else if(NB == 2) GRAM_LAUNCH(2, 1);
-		else if(NB == 3) GRAM_LAUNCH(3, 1);
-		else GRAM_LAUNCH(4, 1);
-	}
+#define GRAM_SHAPES(FL)                                        \
+	do {                                                       \
+		if(XB == 0) {                                          \
+			if(NB == 1) GRAM_LAUNCH(1, FL, 0);                 \
+			else if(NB == 2) GRAM_LAUNCH(2, FL, 0);            \
+			else if(NB == 3) GRAM_LAUNCH(3, FL, 0);            \
+			else GRAM_LAUNCH(4, FL, 0);                        \
+		}                                                      \
+		else if(NB == 2) GRAM_LAUNCH(2, FL, 1);                \
+		else if(NB == 3 && XB == 1) GRAM_LAUNCH(3, FL, 1);     \
+		else if(NB == 3) GRAM_LAUNCH(3, FL, 2);                \
+		else GRAM_LAUNCH(4, FL, 2);                            \
+	} while(0)
+	if(!flat) GRAM_SHAPES(0);
+	else GRAM_SHAPES(1);
+#undef GRAM_SHAPES
 #undef GRAM_LAUNCH
 	CLA_HIP(hipGetLastError());
 	return 0;
