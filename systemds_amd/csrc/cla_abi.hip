@@ -702,6 +702,7 @@ static cla_block* make_joint(cla_block* left, cla_block* right) {
 	cla_block* c = cla_block_create(left->nRows, rightStart + right->nCols);
 	if(!c) return nullptr;
 	if(padded) c->crossBlocks = padL / 16;
+	c->crossCol = rightStart;
 	int tblOff = 0, colOff = 0, maxVals = 0;
 	for(int side = 0; side < 2; side++) {
 		cla_block* src = side ? right : left;
@@ -843,14 +844,12 @@ int launch_tsmm_chunked(cla_block* b, double* dOut) {
 	const int n = b->nCols, nG = (int) b->groups.size(), split = b->crossSplit;
 	if(b->subs.empty()) {
 		// chunks per side (one side when the block is no joint block); joint blocks: left columns are those of
-		// the first `split` groups and, of the constant-only ones, those in front of the right side's first column
+		// the first `split` groups and, of the constant-only ones, those in front of the right side's first
+		// column (which may itself be a constant-only one)
 		std::vector<char> covered((size_t) n, 0);
 		for(auto& g : b->groups)
 			for(int c : g.cols) covered[c] = 1;
-		int firstRight = n;
-		if(split > 0)
-			for(int g = split; g < nG; g++)
-				for(int c : b->groups[g].cols) firstRight = std::min(firstRight, c);
+		const int firstRight = split > 0 ? b->crossCol : n;
 		std::vector<Chunk> chunks[2];
 		auto add_item = [&](int side, int group, int col, int width) -> bool {
 			if(width > 32) return false;

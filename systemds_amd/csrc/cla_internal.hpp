@@ -86,6 +86,7 @@ struct cla_block {
 	uint64_t jointSerial = 0;
 	int32_t crossSplit = 0;          // > 0: joint block, groups [0, crossSplit) are the left side's
 	int32_t crossBlocks = 0;         // > 0: the left side's columns fill the first crossBlocks blocks of 16 columns (padded) and only left x right is read
+	int32_t crossCol = 0;            // joint block: first column of the right side
 	// blocks of pairs of column chunks for t(X) %*% X on more than 64 columns (launch_tsmm_chunked): built on
 	// first use, they borrow this block's row data and are freed with it
 	std::vector<void*> subs;

@@ -146,3 +146,36 @@ def test_constants_only_on_one_side(cla, ora):
     specs, n = mixed_block(12, n_rows, with_unc=False)
     check(cla, ora, consts, 3, specs, n, n_rows, "const %*% mixed")
     check(cla, ora, specs, n, consts, 3, n_rows, "mixed %*% const")
+
+
+@pytest.mark.parametrize("with_unc", [False, True])
+def test_constant_columns_at_the_seam_of_wide_blocks(cla, ora, with_unc):
+    """More than 64 columns over both blocks (column chunks), the right block starting and the left block ending
+    with columns that only carry a constant: those belong to their own side, whichever group comes next."""
+    from systemds_amd import synth
+    n_rows = 1025
+    rng = np.random.default_rng(77)
+
+    def block(lead_const, trail_const, n_ddc):
+        specs, c = [], 0
+        if lead_const:
+            specs.append(synth.GroupSpec("const", np.arange(c, c + 2, dtype=np.int32), rng.standard_normal((1, 2))))
+            c += 2
+        for _ in range(n_ddc):
+            nv = int(rng.choice([3, 40, 300]))
+            codes = rng.integers(0, nv, n_rows).astype(np.uint8 if nv <= 256 else np.uint16)
+            specs.append(synth.GroupSpec("ddc", np.arange(c, c + 2, dtype=np.int32), rng.standard_normal((nv, 2)), codes))
+            c += 2
+        if with_unc:
+            specs.append(synth.GroupSpec("unc", np.arange(c, c + 3, dtype=np.int32), dense=rng.standard_normal((n_rows, 3))))
+            c += 3
+        if trail_const:
+            specs.append(synth.GroupSpec("const", np.arange(c, c + 3, dtype=np.int32), rng.standard_normal((1, 3))))
+            c += 3
+        return specs, c
+
+    specsL, nL = block(True, True, 9)
+    specsR, nR = block(True, True, 30)
+    assert nL + nR > 64
+    check(cla, ora, specsL, nL, specsR, nR, n_rows, "constants at the seam")
+    check(cla, ora, specsR, nR, specsL, nL, n_rows, "constants at the seam, roles swapped")
