@@ -502,7 +502,7 @@ int launch_tsmm(cla_block* b, double* dOut, unsigned long long* dNnz) {
 		}
 	}
 	if(dense && split > 0 && nCols > 64) {
-		set_error("compressed left multiply: uncompressed groups need at most 64 columns over both blocks (have %d)", nCols);
+		set_error("compressed left multiply: an uncompressed group among more than 64 columns over both blocks (have %d) needs every group to span at most 32 columns", nCols);
 		return -CLA_ERR_UNSUPPORTED;
 	}
 	if(dense) {
@@ -625,9 +625,14 @@ int launch_tsmm(cla_block* b, double* dOut, unsigned long long* dNnz) {
 			CLA_HIP(hipMemcpyAsync(dPairs, pairs.data(), sizeof(int4) * pairs.size(), hipMemcpyHostToDevice, st));
 			CLA_HIP(hipStreamSynchronize(st)); // `pairs` is a local: the copy must have read it
 		}
-		// blocks per pair: fill the machine about 8x over all pairs, but keep at least 64 tiles per block
+		// blocks per pair: fill the machine about 8x over all pairs, but keep at least 64 tiles per block.
+		// A target dictionary of a handful of tuples sums most rows of a block into the same few cells, one
+		// after the other, and such a sum of like values drifts with its length (about n / 2 units in the last
+		// place): those pairs get blocks of 8 tiles, whose partial results add up with independent roundings.
 		const int64_t want = std::max<int64_t>(1, (int64_t) g_numCU * 8 / (int64_t) pairs.size());
-		int bpp = (int) std::min<int64_t>(want, std::max(1, nTiles / 64));
+		bool fewCells = false;
+		for(auto& pr : pairs) fewCells |= b->groups[pr.x].d.nVals <= 8;
+		int bpp = fewCells ? std::max(1, nTiles / 8) : (int) std::min<int64_t>(want, std::max(1, nTiles / 64));
 		const int tpb = (nTiles + bpp - 1) / bpp;
 		bpp = (nTiles + tpb - 1) / tpb;
 		double codeBytes = 0;

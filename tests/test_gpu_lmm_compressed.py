@@ -179,3 +179,29 @@ def test_constant_columns_at_the_seam_of_wide_blocks(cla, ora, with_unc):
     assert nL + nR > 64
     check(cla, ora, specsL, nL, specsR, nR, n_rows, "constants at the seam")
     check(cla, ora, specsR, nR, specsL, nL, n_rows, "constants at the seam, roles swapped")
+
+
+def test_one_tuple_dictionary_against_many_rows(cla, ora):
+    """A group with a single tuple (an SDC group of one value, 17 columns) against a DDC group of three tuples over
+    100003 rows on the per-pair path: nearly every row adds one of three values into the same accumulator cells.
+    Such a sum drifts with its length, so the row range per accumulator is kept short; the result stays within
+    the 1e-12 bar of the exact product."""
+    from systemds_amd import synth
+    n_rows = 100003
+    rng = np.random.default_rng(201)
+    left = [synth.sdc_group(rng, n_rows, np.arange(0, 17, dtype=np.int32), 1, 0.6, 0.75)]
+    right = [synth.GroupSpec("ddc", np.arange(0, 33, dtype=np.int32), rng.standard_normal((3, 33)),
+                             rng.integers(0, 3, n_rows).astype(np.uint8)),
+             synth.sdc_group(rng, n_rows, np.arange(33, 38, dtype=np.int32), 300, 0.1, 0.75),
+             synth.GroupSpec("const", np.arange(38, 70, dtype=np.int32), rng.standard_normal((1, 32)))]
+    L = cla.build_block(n_rows, 17, left)
+    R = cla.build_block(n_rows, 70, right)
+    try:
+        out, _ = R.lmm_compressed(L)
+        DL, DR = ora.np_decompress(left, n_rows, 17), ora.np_decompress(right, n_rows, 70)
+        assert_matches_truth(out, DL.T, DR, what="one tuple x three tuples")
+        out, _ = R.tsmm()
+        assert_matches_truth(out, DR.T, DR, what="tsmm with a three-tuple dictionary")
+    finally:
+        L.close()
+        R.close()
