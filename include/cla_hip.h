@@ -146,7 +146,8 @@ int64_t cla_lmm_compressed_dev(cla_handle right, cla_handle left, double* dOut);
 cla_handle cla_rmm_overlapping(cla_handle h, const double* B, int32_t nColB);
 
 /* CLALibMMChain.mmChain (C/lib/CLALibMMChain.java:92-148):
- * out[nCols] = t(X) %*% (w * (X %*% v)); ctype 0 = XtXv (w ignored), 1 = XtwXv. */
+ * out[nCols] = t(X) %*% (w * (X %*% v)); ctype 0 = XtXv (w ignored), 1 = XtwXv,
+ * 2 = XtXvy: t(X) %*% ((X %*% v) - w) (C/lib/CLALibMMChain.java:52). */
 int64_t cla_mmchain(cla_handle h, const double* v, const double* w, int32_t ctype, double* out);
 int64_t cla_mmchain_dev(cla_handle h, const double* dV, const double* dW, int32_t ctype, double* dOut);
 

@@ -1075,8 +1075,8 @@ int64_t cla_mmchain_dev(cla_handle b, const double* dV, const double* dW, int32_
 	int rc = check_final(b);
 	if(rc) return rc;
 	if(!dV || !dOut) { set_error("mmchain: null vector"); return -CLA_ERR_INVALID; }
-	if(ctype != 0 && ctype != 1) { set_error("mmchain: chain type %d not supported (XtXv=0, XtwXv=1)", ctype); return -CLA_ERR_UNSUPPORTED; }
-	if(ctype == 1 && !dW) { set_error("mmchain: XtwXv needs w"); return -CLA_ERR_INVALID; }
+	if(ctype < 0 || ctype > 2) { set_error("mmchain: chain type %d not supported (XtXv=0, XtwXv=1, XtXvy=2)", ctype); return -CLA_ERR_UNSUPPORTED; }
+	if(ctype != 0 && !dW) { set_error("mmchain: XtwXv and XtXvy need w"); return -CLA_ERR_INVALID; }
 	std::lock_guard<std::recursive_mutex> lk(b->mu);
 	if((rc = launch_mmchain(b, dV, dW, ctype, dOut, b->dCounters))) return rc;
 	return finish_nnz(b);
@@ -1086,8 +1086,8 @@ int64_t cla_mmchain(cla_handle b, const double* v, const double* w, int32_t ctyp
 	int rc = check_final(b);
 	if(rc) return rc;
 	if(!v || !out) { set_error("mmchain: null vector"); return -CLA_ERR_INVALID; }
-	if(ctype == 1 && !w) { set_error("mmchain: XtwXv needs w"); return -CLA_ERR_INVALID; }
-	const size_t nV = (size_t) b->nCols, nW = ctype == 1 ? (size_t) b->nRows : 0;
+	if((ctype == 1 || ctype == 2) && !w) { set_error("mmchain: XtwXv and XtXvy need w"); return -CLA_ERR_INVALID; }
+	const size_t nV = (size_t) b->nCols, nW = ctype == 1 || ctype == 2 ? (size_t) b->nRows : 0;
 	std::lock_guard<std::recursive_mutex> lk(b->mu);
 	if((rc = ensure_stage(&b->dStageIn, &b->stageInCap, nV + nW)) || (rc = ensure_stage(&b->dStageOut, &b->stageOutCap, nV)))
 		return rc;

@@ -319,10 +319,15 @@ int launch_lmm(cla_block* b, const double* dY, int p, double* dOut, unsigned lon
 	return 0;
 }
 
-// CLALibMMChain.mmChain: tmp = X %*% v ; tmp *= w (XtwXv) ; out = t(tmp) %*% X.
+// CLALibMMChain.mmChain: tmp = X %*% v ; tmp *= w (XtwXv) or tmp -= w (XtXvy) ; out = t(tmp) %*% X.
 __global__ __launch_bounds__(256) void k_mul_inplace(double* __restrict__ x, const double* __restrict__ w, int64_t n) {
 	const int64_t i = (int64_t) blockIdx.x * 256 + threadIdx.x;
 	if(i < n) x[i] *= w[i];
+}
+
+__global__ __launch_bounds__(256) void k_sub_inplace(double* __restrict__ x, const double* __restrict__ y, int64_t n) {
+	const int64_t i = (int64_t) blockIdx.x * 256 + threadIdx.x;
+	if(i < n) x[i] -= y[i];
 }
 
 int launch_mmchain(cla_block* b, const double* dV, const double* dW, int ctype, double* dOut, unsigned long long* dNnz) {
@@ -335,6 +340,8 @@ int launch_mmchain(cla_block* b, const double* dV, const double* dW, int ctype, 
 	first.swap(b->lastStats);
 	if(ctype == 1 && nRows > 0)
 		hipLaunchKernelGGL(k_mul_inplace, dim3((unsigned) ((nRows + 255) / 256)), dim3(256), 0, b->stream, tmp, dW, nRows);
+	if(ctype == 2 && nRows > 0)
+		hipLaunchKernelGGL(k_sub_inplace, dim3((unsigned) ((nRows + 255) / 256)), dim3(256), 0, b->stream, tmp, dW, nRows);
 	rc = launch_lmm(b, tmp, 1, dOut, dNnz);
 	b->lastStats.insert(b->lastStats.begin(), first.begin(), first.end());
 	return rc;

@@ -782,16 +782,10 @@ struct CLALibMMChain {
 			throw DMLRuntimeException("Dimensions mismatch on mmchain operation (w is not a vector of the number of rows of x)");
 		MatrixBlock out(x.getNumColumns(), 1);
 		if(x.isEmpty()) return out;
-		if(ctype == ChainType::XtXvy) { // subtraction of y between the two multiplies: composed from the two drivers
-			MatrixBlock vv = v;
-			MatrixBlock tmp = CLALibRightMultBy::rightMultByMatrix(x, vv, k);
-			for(int r = 0; r < tmp.getNumRows(); r++) tmp.set(r, 0, tmp.get(r, 0) - w->get(r, 0));
-			tmp.recomputeNonZeros();
-			return CLALibLeftMultBy::leftMultByMatrixTransposed(x, tmp, k).transpose();
-		}
-		const double* wp = ctype == ChainType::XtwXv ? w->getDenseBlockValues() : nullptr;
-		out.setNonZeros(checkNative(cla_mmchain(x.hipHandle(), v.getDenseBlockValues(), wp, ctype == ChainType::XtwXv ? 1 : 0,
-			out.getDenseBlockValues()), "MMChain"));
+		// all three chain types run on the device: X %*% v, then * w (XtwXv) or - w (XtXvy), then t(.) %*% X
+		const double* wp = ctype == ChainType::XtXv ? nullptr : w->getDenseBlockValues();
+		const int ct = ctype == ChainType::XtXv ? 0 : ctype == ChainType::XtwXv ? 1 : 2;
+		out.setNonZeros(checkNative(cla_mmchain(x.hipHandle(), v.getDenseBlockValues(), wp, ct, out.getDenseBlockValues()), "MMChain"));
 		return out;
 	}
 };

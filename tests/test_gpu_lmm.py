@@ -125,3 +125,25 @@ def test_byte_code_blocks_left_multiply(cla, ora, n_rows, n_col_g, p):
     ref, rnnz = ora.lmm(ora.Groups(specs, n_rows, n_cols), Y, 4)
     assert_fp64_close(out, ref, ora.abs_matmul(Y, D), what="byte-code lmm vs oracle", n_terms=n_rows)
     assert nnz == rnnz
+
+
+def test_mmchain_minus_y(cla, ora):
+    """Chain type XtXvy, t(X) %*% ((X %*% v) - y) (CLALibMMChain.java:52), against the exactly accumulated product
+    of the decompressed matrix and against the composition of the two multiplies."""
+    from parity import assert_matches_truth
+    specs, n_cols = mixed_block(23, 40009)
+    rng = np.random.default_rng(24)
+    v, y = rng.standard_normal(n_cols), rng.standard_normal(40009)
+    blk = cla.build_block(40009, n_cols, specs)
+    try:
+        out, nnz = blk.mmchain(v, y, 2)
+        Xv, _ = blk.rmm(v.reshape(-1, 1))
+        D = ora.np_decompress(specs, 40009, n_cols)
+        assert_matches_truth(out.reshape(-1, 1), D.T, Xv - y.reshape(-1, 1), what="mmchain XtXvy")
+        assert nnz == np.count_nonzero(out)
+        with pytest.raises(cla.ClaError):
+            blk.mmchain(v, None, 2)
+        with pytest.raises(cla.ClaError):
+            blk.mmchain(v, y, 3)
+    finally:
+        blk.close()
