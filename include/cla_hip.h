@@ -22,9 +22,12 @@
  *  - All matrices are dense row-major fp64 (Java DenseBlockFP64).
  *  - Host pointers are borrowed only for the duration of the call.
  *  - `_dev` variants take device pointers (HBM) and run asynchronously on the
- *    block's stream up to the final non-zero count read-back.
- *  - No exceptions cross the boundary; errors are negative return codes and
- *    cla_last_error() (thread local) explains them.
+ *    block's stream up to the final non-zero count read-back; `_dev_async`
+ *    variants leave that count in a device counter (cla_block_nnz reads it on
+ *    request) and return without waiting for the stream.
+ *  - No exceptions cross the boundary (every entry point catches what the host
+ *    code below it may throw, std::bad_alloc included); errors are negative
+ *    return codes and cla_last_error() (thread local) explains them.
  *  - Calls on different blocks are thread safe; calls on one block are
  *    serialised internally (one HIP stream per block).
  */
@@ -100,9 +103,26 @@ int cla_block_finalize(cla_handle h);
 
 /* Use an existing HIP stream (hipStream_t) for all work of this block. */
 int cla_block_set_stream(cla_handle h, void* hipStream);
+/* Per-block switch between the alternative kernels of a driver (each a complete implementation of the
+ * same product: the reference likewise holds several variants per product, e.g. the pre-aggregating and
+ * the decompressing right multiply, CG/ColGroupDDC.java:647-692). The defaults are the tuned dispatch.
+ *   tsmm_route      0 cost model, 1 one pass per pair of groups, 2 decoded Gram matrix
+ *   tsmm_chunks     1 / 0: more than 64 columns as pairs of column chunks
+ *   tsmm_wide_dense 0 / 1, tsmm_mfma 1 / 0, tsmm_pair_dot 1 / 0
+ *   expand_streams  1 / 0: one code per row for small RLE / SDCZeros groups (set before the first multiply)
+ *   rmm_disable     bit 0 byte-code mat-vec kernel, 1 its fused tables, 2 matrix-core kernel, 3 decode kernel
+ *   lmm_disable     bit 0 dot form on byte codes, bit 1 byte-code bin kernel
+ *   sdc_packed      1 / 0: packed SDCZeros lists for the mat-vecs
+ * Blocks derived from this one (overlapping results, joint blocks) inherit the values at the time of the call
+ * that uses them. Returns 0, or -CLA_ERR_INVALID for an unknown key or value. */
+int cla_block_set_option(cla_handle h, const char* key, int32_t value);
 int32_t cla_block_num_groups(cla_handle h);
 /* Bytes of HBM held by the block's compressed representation. */
 int64_t cla_block_device_bytes(cla_handle h);
+/* Bytes of HBM held by the formats the library has derived from that representation so far (padded
+ * dictionary image at finalize; packed SDCZeros lists, one-code-per-row streams and cached counts on the
+ * first call of the driver that uses them). */
+int64_t cla_block_derived_bytes(cla_handle h);
 
 /* ---- multiply drivers ---- */
 
@@ -111,16 +131,24 @@ int64_t cla_block_device_bytes(cla_handle h);
  * B is nCols x nColB. Returns nnz(out) or a negative error. */
 int64_t cla_rmm(cla_handle h, const double* B, int32_t nColB, double* out);
 int64_t cla_rmm_dev(cla_handle h, const double* dB, int32_t nColB, double* dOut);
+/* The same without the wait: returns 0 once the kernels are queued on the block's stream (or a negative
+ * error); the non-zero count stays in a device counter until cla_block_nnz asks for it. */
+int cla_rmm_dev_async(cla_handle h, const double* dB, int32_t nColB, double* dOut);
+/* nnz of the result of the last driver call on this block (MatrixBlock.recomputeNonZeros of the reference
+ * drivers, C/lib/CLALibRightMultBy.java:98); waits for the block's stream. */
+int64_t cla_block_nnz(cla_handle h);
 
 /* CLALibLeftMultBy.leftMultByMatrix (C/lib/CLALibLeftMultBy.java:126-145,
  * 286-346): out[nRowY x nCols] = Y %*% X, Y is nRowY x nRows. */
 int64_t cla_lmm(cla_handle h, const double* Y, int32_t nRowY, double* out);
 int64_t cla_lmm_dev(cla_handle h, const double* dY, int32_t nRowY, double* dOut);
+int cla_lmm_dev_async(cla_handle h, const double* dY, int32_t nRowY, double* dOut);
 
 /* CLALibTSMM.leftMultByTransposeSelf (C/lib/CLALibTSMM.java:59-94):
  * out[nCols x nCols] = t(X) %*% X, full symmetric. */
 int64_t cla_tsmm(cla_handle h, double* out);
 int64_t cla_tsmm_dev(cla_handle h, double* dOut);
+int cla_tsmm_dev_async(cla_handle h, double* dOut);
 
 /* CLALibLeftMultBy.leftMultByMatrixTransposed for two compressed blocks
  * (C/lib/CLALibLeftMultBy.java:100-112, 170-284): out[nColsLeft x nColsRight] = t(left) %*% right,
@@ -150,6 +178,7 @@ cla_handle cla_rmm_overlapping(cla_handle h, const double* B, int32_t nColB);
  * 2 = XtXvy: t(X) %*% ((X %*% v) - w) (C/lib/CLALibMMChain.java:52). */
 int64_t cla_mmchain(cla_handle h, const double* v, const double* w, int32_t ctype, double* out);
 int64_t cla_mmchain_dev(cla_handle h, const double* dV, const double* dW, int32_t ctype, double* dOut);
+int cla_mmchain_dev_async(cla_handle h, const double* dV, const double* dW, int32_t ctype, double* dOut);
 
 /* CLALibDecompress.decompressDense (C/lib/CLALibDecompress.java:310-357):
  * out[nRows x nCols] = X. */
@@ -195,6 +224,13 @@ int cla_block_profile(cla_handle h, int enable);
 /* JSON with the kernels launched by the last driver call on this block: launch
  * geometry, algorithmic bytes and (when profiling) milliseconds. */
 int cla_stats(cla_handle h, char* json, size_t cap);
+
+/* Diagnostic: throws inside the library (kind 0 std::bad_alloc, 1 std::length_error, 2 a non-standard
+ * exception, 3 an over-long std::vector reservation) and returns what an entry point returns for it:
+ * -CLA_ERR_DEVICE for a failed allocation, -CLA_ERR_INVALID otherwise, 0 for an unknown kind. Needs no
+ * device. It is how a binding checks that nothing unwinds into the JVM (JNI code must not let C++
+ * exceptions escape, src/main/cpp/systemds.cpp has none to begin with). */
+int cla_selftest_exception(int kind);
 
 #ifdef __cplusplus
 }

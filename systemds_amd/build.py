@@ -1,14 +1,23 @@
-"""Builds libclahip.so (HIP kernels + C ABI) for gfx950 with hipcc, in-tree."""
+"""Builds libclahip.so (HIP kernels + C ABI) for gfx950 with hipcc, in-tree.
+
+Every .hip file under csrc/ is compiled to an object of its own (in parallel) and the
+objects are linked into one shared library. `python -m systemds_amd.build --incremental`
+recompiles only the files that are newer than their object (development); the default
+and `__graft_entry__.build()` compile everything.
+"""
 import os
 import subprocess
 import sys
+from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
+OBJ = os.path.join(CSRC, "obj")
 LIB = os.path.join(HERE, "libclahip.so")
+INCLUDE = os.path.join(os.path.dirname(HERE), "include")
 
 HIPCC_FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-ffp-contract=off", "-munsafe-fp-atomics",
     "-Wall", "-Wno-unused-function", "-Wno-unknown-warning-option", "-Wno-unused-command-line-argument",
@@ -19,9 +28,31 @@ def sources():
     return sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip"))
 
 
-def build_lib(verbose=True):
+def _headers():
+    hs = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hpp")]
+    hs += [os.path.join(INCLUDE, f) for f in os.listdir(INCLUDE) if f.endswith(".h")]
+    return hs
+
+
+def build_lib(verbose=True, incremental=False, jobs=None):
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc] + HIPCC_FLAGS + ["-o", LIB] + sources()
+    os.makedirs(OBJ, exist_ok=True)
+    newest_header = max(os.path.getmtime(h) for h in _headers())
+    jobs = jobs or min(8, os.cpu_count() or 1)
+
+    def compile_one(src):
+        obj = os.path.join(OBJ, os.path.basename(src)[:-4] + ".o")
+        if incremental and os.path.exists(obj) and os.path.getmtime(obj) > max(os.path.getmtime(src), newest_header):
+            return obj
+        cmd = [hipcc] + HIPCC_FLAGS + ["-c", src, "-o", obj]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        subprocess.run(cmd, check=True)
+        return obj
+
+    with ThreadPoolExecutor(max_workers=jobs) as ex:
+        objs = list(ex.map(compile_one, sources()))
+    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.run(cmd, check=True)
@@ -48,6 +79,7 @@ def build_host(verbose=True):
 
 
 if __name__ == "__main__":
-    build_lib()
-    build_host()
+    build_lib(incremental="--incremental" in sys.argv)
+    if "--no-host" not in sys.argv:
+        build_host()
     sys.exit(0)

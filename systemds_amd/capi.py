@@ -45,16 +45,23 @@ SIGNATURES = {
     "cla_block_add_empty": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32]),
     "cla_block_finalize": (C.c_int, [C.c_void_p]),
     "cla_block_set_stream": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "cla_block_set_option": (C.c_int, [C.c_void_p, C.c_char_p, C.c_int32]),
     "cla_block_num_groups": (C.c_int32, [C.c_void_p]),
     "cla_block_device_bytes": (C.c_int64, [C.c_void_p]),
+    "cla_block_derived_bytes": (C.c_int64, [C.c_void_p]),
     "cla_rmm": (C.c_int64, [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
     "cla_rmm_dev": (C.c_int64, [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
+    "cla_rmm_dev_async": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
+    "cla_block_nnz": (C.c_int64, [C.c_void_p]),
     "cla_lmm": (C.c_int64, [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
     "cla_lmm_dev": (C.c_int64, [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
+    "cla_lmm_dev_async": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
     "cla_tsmm": (C.c_int64, [C.c_void_p, C.c_void_p]),
     "cla_tsmm_dev": (C.c_int64, [C.c_void_p, C.c_void_p]),
+    "cla_tsmm_dev_async": (C.c_int, [C.c_void_p, C.c_void_p]),
     "cla_mmchain": (C.c_int64, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
     "cla_mmchain_dev": (C.c_int64, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
+    "cla_mmchain_dev_async": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
     "cla_lmm_compressed": (C.c_int64, [C.c_void_p, C.c_void_p, C.c_void_p]),
     "cla_lmm_compressed_dev": (C.c_int64, [C.c_void_p, C.c_void_p, C.c_void_p]),
     "cla_rmm_overlapping": (C.c_void_p, [C.c_void_p, C.c_void_p, C.c_int32]),
@@ -67,6 +74,7 @@ SIGNATURES = {
     "cla_preagg": (C.c_int, [C.c_void_p, C.c_int32, C.c_void_p, C.c_int32, C.c_void_p]),
     "cla_block_profile": (C.c_int, [C.c_void_p, C.c_int]),
     "cla_stats": (C.c_int, [C.c_void_p, C.c_char_p, C.c_size_t]),
+    "cla_selftest_exception": (C.c_int, [C.c_int]),
 }
 
 _lib = None
@@ -223,8 +231,16 @@ class ClaBlock:
     def set_stream(self, stream_ptr):
         _check(self.lib.cla_block_set_stream(self.h, C.c_void_p(stream_ptr)))
 
+    def set_option(self, key, value):
+        """cla_block_set_option: forces one of the alternative kernels of a driver (see include/cla_hip.h)."""
+        _check(self.lib.cla_block_set_option(self.h, key.encode(), int(value)))
+        return self
+
     def device_bytes(self):
         return _check(self.lib.cla_block_device_bytes(self.h))
+
+    def derived_bytes(self):
+        return _check(self.lib.cla_block_derived_bytes(self.h))
 
     # ---- host-pointer drivers (what a JNI caller uses) ----
     def rmm(self, B):
@@ -309,6 +325,23 @@ class ClaBlock:
     # ---- device-pointer drivers (inputs/outputs already in HBM) ----
     def rmm_dev(self, dB_ptr, n_col_b, dOut_ptr):
         return _check(self.lib.cla_rmm_dev(self.h, C.c_void_p(dB_ptr), int(n_col_b), C.c_void_p(dOut_ptr)))
+
+    def rmm_dev_async(self, dB_ptr, n_col_b, dOut_ptr):
+        return _check(self.lib.cla_rmm_dev_async(self.h, C.c_void_p(dB_ptr), int(n_col_b), C.c_void_p(dOut_ptr)))
+
+    def nnz(self):
+        """cla_block_nnz: non-zero count of the last driver call's result (waits for the block's stream)."""
+        return _check(self.lib.cla_block_nnz(self.h))
+
+    def lmm_dev_async(self, dY_ptr, n_row_y, dOut_ptr):
+        return _check(self.lib.cla_lmm_dev_async(self.h, C.c_void_p(dY_ptr), int(n_row_y), C.c_void_p(dOut_ptr)))
+
+    def tsmm_dev_async(self, dOut_ptr):
+        return _check(self.lib.cla_tsmm_dev_async(self.h, C.c_void_p(dOut_ptr)))
+
+    def mmchain_dev_async(self, dV_ptr, dW_ptr, ctype, dOut_ptr):
+        return _check(self.lib.cla_mmchain_dev_async(self.h, C.c_void_p(dV_ptr), C.c_void_p(dW_ptr or 0), int(ctype),
+                                                     C.c_void_p(dOut_ptr)))
 
     def lmm_dev(self, dY_ptr, n_row_y, dOut_ptr):
         return _check(self.lib.cla_lmm_dev(self.h, C.c_void_p(dY_ptr), int(n_row_y), C.c_void_p(dOut_ptr)))

@@ -7,6 +7,20 @@
 #include <cstdarg>
 #include <cstring>
 #include <map>
+#include <new>
+#include <stdexcept>
+
+// No exception may cross the C ABI (a JNI or FFM caller would abort the JVM instead of falling
+// back): every exported function runs its body between these two.
+#define CLA_TRY try {
+#define CLA_CATCH_BODY(onAlloc, onOther)                                                          \
+	}                                                                                             \
+	catch(const std::bad_alloc&) { cla::set_error("host memory allocation failed"); onAlloc; }   \
+	catch(const std::exception& e) { cla::set_error("unexpected exception: %s", e.what()); onOther; } \
+	catch(...) { cla::set_error("unexpected exception"); onOther; }
+#define CLA_CATCH_CODE(T) CLA_CATCH_BODY(return (T) -CLA_ERR_DEVICE, return (T) -CLA_ERR_INVALID)
+#define CLA_CATCH_NULL CLA_CATCH_BODY(return nullptr, return nullptr)
+#define CLA_CATCH_VOID CLA_CATCH_BODY(return, return)
 
 namespace cla {
 
@@ -113,6 +127,7 @@ static int check_cols(cla_block* b, const int32_t* cols, int32_t nColG) {
 
 static int check_open(cla_block* b) {
 	if(!b) { set_error("null block handle"); return -CLA_ERR_INVALID; }
+	if(b->poisoned) { set_error("an earlier cla_block_finalize on this block failed; free it"); return -CLA_ERR_STATE; }
 	if(b->finalized) { set_error("block already finalized"); return -CLA_ERR_STATE; }
 	return check_ready();
 }
@@ -139,6 +154,15 @@ static int upload_dict(HostGroup& g) {
 	return upload(g, g.dict.data(), sizeof(double) * g.dict.size(), (const void**) &g.d.dict);
 }
 
+// One pair of column chunks of a block with more than 64 columns (launch_tsmm_chunked): a block of its own
+// that borrows the row data.
+struct SubBlock {
+	cla_block* blk;
+	int32_t* dColMap;   // column of `b` per column of blk (-1: padding behind the first chunk)
+	int nA, nB;         // columns of the first (padding included) / second chunk
+	bool writeA, writeB, crossOnly;
+};
+
 int finish_finalize(cla_block* b, cla_block* arenaFrom, bool buildArena = true);
 static void free_subs(cla_block* b);
 
@@ -149,6 +173,7 @@ using namespace cla;
 extern "C" {
 
 int cla_init(int device) {
+	CLA_TRY
 	std::lock_guard<std::mutex> lk(g_initMu);
 	int n = 0;
 	hipError_t e = hipGetDeviceCount(&n);
@@ -172,11 +197,13 @@ int cla_init(int device) {
 		g_ldsPerBlock = (int) g_prop.maxSharedMemoryPerMultiProcessor;
 	g_device = device;
 	return 0;
+	CLA_CATCH_CODE(int)
 }
 
 const char* cla_last_error(void) { return t_err; }
 
 int cla_device_info(char* json, size_t cap) {
+	CLA_TRY
 	int rc = check_ready();
 	if(rc) return rc;
 	snprintf(json, cap,
@@ -186,9 +213,11 @@ int cla_device_info(char* json, size_t cap) {
 		g_prop.maxSharedMemoryPerMultiProcessor, g_prop.totalGlobalMem, g_prop.clockRate, g_prop.memoryClockRate,
 		g_prop.memoryBusWidth, g_prop.l2CacheSize);
 	return 0;
+	CLA_CATCH_CODE(int)
 }
 
 cla_handle cla_block_create(int64_t nRows, int32_t nCols) {
+	CLA_TRY
 	if(check_ready()) return nullptr;
 	if(nRows < 0 || nRows > 0x7fffffffLL || nCols <= 0) {
 		set_error("invalid block shape %lld x %d", (long long) nRows, nCols);
@@ -208,10 +237,17 @@ cla_handle cla_block_create(int64_t nRows, int32_t nCols) {
 		cla_block_free(b);
 		return nullptr;
 	}
+	if(hipMemset(b->dCounters, 0, 8 * sizeof(unsigned long long)) != hipSuccess) {
+		set_error("clearing counters failed");
+		cla_block_free(b);
+		return nullptr;
+	}
 	return b;
+	CLA_CATCH_NULL
 }
 
 void cla_block_free(cla_handle b) {
+	CLA_TRY
 	if(!b) return;
 	if(b->refs.fetch_sub(1) > 1) return; // blocks made from this one still use its streams
 	cla_block* parent = b->parent;
@@ -231,6 +267,7 @@ void cla_block_free(cla_handle b) {
 	if(b->dStageIn) (void) hipFree(b->dStageIn);
 	if(b->dStageOut) (void) hipFree(b->dStageOut);
 	if(b->dScratch) (void) hipFree(b->dScratch);
+	if(b->dChain) (void) hipFree(b->dChain);
 	if(b->dSdcPlan) (void) hipFree(b->dSdcPlan);
 	if(b->dSdcDesc) (void) hipFree(b->dSdcDesc);
 	if(b->dSdcPacked) (void) hipFree(b->dSdcPacked);
@@ -244,10 +281,12 @@ void cla_block_free(cla_handle b) {
 	if(b->ownStream && b->stream) (void) hipStreamDestroy(b->stream);
 	delete b;
 	if(parent) cla_block_free(parent);
+	CLA_CATCH_VOID
 }
 
 int cla_block_add_ddc(cla_handle b, const int32_t* cols, int32_t nColG, const double* dict, int32_t nVals,
 	const void* codes, int32_t codeWidth) {
+	CLA_TRY
 	int rc = check_open(b);
 	if(rc) return rc;
 	if((rc = check_cols(b, cols, nColG))) return rc;
@@ -267,11 +306,13 @@ int cla_block_add_ddc(cla_handle b, const int32_t* cols, int32_t nColG, const do
 	g.d.codeWidth = codeWidth;
 	b->groups.push_back(std::move(g));
 	return 0;
+	CLA_CATCH_CODE(int)
 }
 
 int cla_block_add_sdc(cla_handle b, const int32_t* cols, int32_t nColG, const double* dict, int32_t nVals,
 	const double* defaultTuple, const void* codes, int32_t codeWidth, const void* deltas, int32_t deltaWidth,
 	int64_t nDeltas, int32_t offsetToFirst, int32_t offsetToLast, int64_t nOffsets) {
+	CLA_TRY
 	int rc = check_open(b);
 	if(rc) return rc;
 	if((rc = check_cols(b, cols, nColG))) return rc;
@@ -316,10 +357,12 @@ int cla_block_add_sdc(cla_handle b, const int32_t* cols, int32_t nColG, const do
 	g.d.last = nOffsets ? offsetToLast : -1;
 	b->groups.push_back(std::move(g));
 	return 0;
+	CLA_CATCH_CODE(int)
 }
 
 int cla_block_add_rle(cla_handle b, const int32_t* cols, int32_t nColG, const double* dict, int32_t nVals,
 	const int32_t* ptr, const uint16_t* data, int64_t nData) {
+	CLA_TRY
 	int rc = check_open(b);
 	if(rc) return rc;
 	if((rc = check_cols(b, cols, nColG))) return rc;
@@ -367,9 +410,11 @@ int cla_block_add_rle(cla_handle b, const int32_t* cols, int32_t nColG, const do
 	g.d.nRuns = nRuns;
 	b->groups.push_back(std::move(g));
 	return 0;
+	CLA_CATCH_CODE(int)
 }
 
 int cla_block_add_uncompressed(cla_handle b, const int32_t* cols, int32_t nColG, const double* values) {
+	CLA_TRY
 	int rc = check_open(b);
 	if(rc) return rc;
 	if((rc = check_cols(b, cols, nColG))) return rc;
@@ -383,9 +428,11 @@ int cla_block_add_uncompressed(cla_handle b, const int32_t* cols, int32_t nColG,
 	}
 	b->groups.push_back(std::move(g));
 	return 0;
+	CLA_CATCH_CODE(int)
 }
 
 int cla_block_add_const(cla_handle b, const int32_t* cols, int32_t nColG, const double* row) {
+	CLA_TRY
 	int rc = check_open(b);
 	if(rc) return rc;
 	if((rc = check_cols(b, cols, nColG))) return rc;
@@ -395,20 +442,24 @@ int cla_block_add_const(cla_handle b, const int32_t* cols, int32_t nColG, const 
 	for(int j = 0; j < nColG; j++) b->constV[cols[j]] += row[j];
 	b->hasConst = true;
 	return 0;
+	CLA_CATCH_CODE(int)
 }
 
 int cla_block_add_empty(cla_handle b, const int32_t* cols, int32_t nColG) {
+	CLA_TRY
 	int rc = check_open(b);
 	if(rc) return rc;
 	if((rc = check_cols(b, cols, nColG))) return rc;
+	std::lock_guard<std::recursive_mutex> lk(b->mu);
 	b->hasConst = true; // CLALibUtils.shouldPreFilter is true for empty groups as well
 	return 0;
+	CLA_CATCH_CODE(int)
 }
 
-int cla_block_finalize(cla_handle b) {
-	int rc = check_open(b);
-	if(rc) return rc;
-	std::lock_guard<std::recursive_mutex> lk(b->mu);
+// Finalize changes the block as it goes (SDC defaults into the constants, acceleration structures group by
+// group): a failure half way leaves it unusable, so the block is then marked and only cla_block_free takes it.
+static int finalize_groups(cla_block* b) {
+	int rc;
 	int tblOff = 0, colOff = 0, maxVals = 0;
 	for(size_t gi = 0; gi < b->groups.size(); gi++) {
 		HostGroup& g = b->groups[gi];
@@ -442,6 +493,18 @@ int cla_block_finalize(cla_handle b) {
 	b->totalColsG = colOff;
 	b->maxVals = maxVals;
 	return finish_finalize(b, nullptr);
+}
+
+int cla_block_finalize(cla_handle b) {
+	CLA_TRY
+	int rc = check_open(b);
+	if(rc) return rc;
+	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	b->poisoned = true; // until every step has succeeded (also when a step throws)
+	if((rc = finalize_groups(b))) return rc;
+	b->poisoned = false;
+	return 0;
+	CLA_CATCH_CODE(int)
 }
 
 } // extern "C"
@@ -523,7 +586,6 @@ int finish_finalize(cla_block* b, cla_block* arenaFrom, bool buildArena) {
 	// last holds a multiple of 8 groups (two batches of 4, see k_rmm_q1_ddc).
 	{
 		int budget = 52 * 1024;
-		if(const char* e = getenv("CLA_Q1_LDS_KB")) budget = atoi(e) * 1024;
 		budget = std::min(budget, g_ldsPerBlock);
 		b->q1Slabs.clear();
 		b->q1LdsBytes = 0;
@@ -547,6 +609,10 @@ int finish_finalize(cla_block* b, cla_block* arenaFrom, bool buildArena) {
 	}
 	b->device_bytes_cached = 0;
 	for(auto& g : b->groups) b->device_bytes_cached += g.bytes;
+	{
+		const int rc = ensure_dict_pad(b);
+		if(rc) return rc;
+	}
 	b->finalized = true;
 	return 0;
 }
@@ -556,41 +622,113 @@ int finish_finalize(cla_block* b, cla_block* arenaFrom, bool buildArena) {
 extern "C" {
 
 int cla_block_set_stream(cla_handle b, void* hipStream) {
+	CLA_TRY
 	if(!b) { set_error("null block handle"); return -CLA_ERR_INVALID; }
 	std::lock_guard<std::recursive_mutex> lk(b->mu);
 	if(b->ownStream && b->stream) { (void) hipStreamSynchronize(b->stream); (void) hipStreamDestroy(b->stream); }
 	b->stream = (hipStream_t) hipStream;
 	b->ownStream = false;
 	return 0;
+	CLA_CATCH_CODE(int)
+}
+
+int cla_block_set_option(cla_handle b, const char* key, int32_t value) {
+	CLA_TRY
+	if(!b || !key) { set_error("set_option: null handle or key"); return -CLA_ERR_INVALID; }
+	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	struct Entry { const char* name; int Options::*field; int lo, hi; };
+	static const Entry table[] = {
+		{"tsmm_route", &Options::tsmmRoute, 0, 2},         {"tsmm_chunks", &Options::tsmmChunks, 0, 1},
+		{"tsmm_wide_dense", &Options::tsmmWideDense, 0, 1}, {"tsmm_mfma", &Options::tsmmMfma, 0, 1},
+		{"tsmm_pair_dot", &Options::tsmmPairDot, 0, 1},     {"expand_streams", &Options::expandStreams, 0, 1},
+		{"rmm_disable", &Options::rmmDisable, 0, 15},       {"lmm_disable", &Options::lmmDisable, 0, 3},
+		{"sdc_packed", &Options::sdcPacked, 0, 1},
+	};
+	for(const Entry& e : table)
+		if(strcmp(e.name, key) == 0) {
+			if(value < e.lo || value > e.hi) { set_error("set_option: %s takes %d..%d (got %d)", key, e.lo, e.hi, value); return -CLA_ERR_INVALID; }
+			b->opt.*(e.field) = value;
+			return 0;
+		}
+	set_error("set_option: unknown option '%s'", key);
+	return -CLA_ERR_INVALID;
+	CLA_CATCH_CODE(int)
+}
+
+int cla_selftest_exception(int kind) {
+	CLA_TRY
+	if(kind == 0) throw std::bad_alloc();
+	if(kind == 1) throw std::length_error("selftest");
+	if(kind == 2) throw 42;
+	if(kind == 3) { std::vector<double> v; v.reserve(v.max_size() + 1); } // what an absurd size argument does
+	return 0;
+	CLA_CATCH_CODE(int)
 }
 
 int32_t cla_block_num_groups(cla_handle b) { return b ? (int32_t) b->groups.size() : -CLA_ERR_INVALID; }
 
 int64_t cla_block_device_bytes(cla_handle b) {
+	CLA_TRY
 	if(!b) return -CLA_ERR_INVALID;
 	int64_t s = 0;
 	for(auto& g : b->groups) s += g.bytes;
+	return s;
+	CLA_CATCH_CODE(int64_t)
+}
+
+int64_t cla_block_derived_bytes(cla_handle b) {
+	if(!b) return -CLA_ERR_INVALID;
+	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	int64_t s = b->derivedBytes;
+	if(b->joint) s += b->joint->derivedBytes;
+	for(void* p : b->subs) s += ((SubBlock*) p)->blk ? ((SubBlock*) p)->blk->derivedBytes : 0;
 	return s;
 }
 
 // ---- drivers -------------------------------------------------------------
 
-static int64_t finish_nnz(cla_block* b) {
-	CLA_HIP(hipMemcpyAsync(b->hCounters, b->dCounters, sizeof(unsigned long long), hipMemcpyDeviceToHost, b->stream));
+// sync: wait for the driver's kernels and return its non-zero count; otherwise leave the count in the
+// device counter (cla_block_nnz reads it on request) and return at once
+static int64_t finish_nnz(cla_block* b, bool sync = true) {
+	if(!sync) return 0;
+	CLA_HIP(hipMemcpyAsync(b->hCounters, b->dCounters + b->nnzSlot, sizeof(unsigned long long), hipMemcpyDeviceToHost, b->stream));
 	CLA_HIP(hipStreamSynchronize(b->stream));
 	return (int64_t) b->hCounters[0];
 }
 
-int64_t cla_rmm_dev(cla_handle b, const double* dB, int32_t nColB, double* dOut) {
+static int64_t rmm_dev(cla_handle b, const double* dB, int32_t nColB, double* dOut, bool sync) {
 	int rc = check_final(b);
 	if(rc) return rc;
 	if(!dB || !dOut || nColB <= 0) { set_error("rmm: invalid right-hand side"); return -CLA_ERR_INVALID; }
 	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	b->nnzSlot = 0;
 	if((rc = launch_rmm(b, dB, nColB, dOut, b->dCounters))) return rc;
-	return finish_nnz(b);
+	return finish_nnz(b, sync);
+}
+
+int64_t cla_rmm_dev(cla_handle b, const double* dB, int32_t nColB, double* dOut) {
+	CLA_TRY
+	return rmm_dev(b, dB, nColB, dOut, true);
+	CLA_CATCH_CODE(int64_t)
+}
+
+int cla_rmm_dev_async(cla_handle b, const double* dB, int32_t nColB, double* dOut) {
+	CLA_TRY
+	return (int) rmm_dev(b, dB, nColB, dOut, false);
+	CLA_CATCH_CODE(int)
+}
+
+int64_t cla_block_nnz(cla_handle b) {
+	CLA_TRY
+	int rc = check_final(b);
+	if(rc) return rc;
+	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	return finish_nnz(b, true);
+	CLA_CATCH_CODE(int64_t)
 }
 
 int64_t cla_rmm(cla_handle b, const double* B, int32_t nColB, double* out) {
+	CLA_TRY
 	int rc = check_final(b);
 	if(rc) return rc;
 	if(!B || !out || nColB <= 0) { set_error("rmm: invalid right-hand side"); return -CLA_ERR_INVALID; }
@@ -603,19 +741,24 @@ int64_t cla_rmm(cla_handle b, const double* B, int32_t nColB, double* out) {
 	if(nnz < 0) return nnz;
 	if(nOut) CLA_HIP(hipMemcpy(out, b->dStageOut, nOut * sizeof(double), hipMemcpyDeviceToHost));
 	return nnz;
+	CLA_CATCH_CODE(int64_t)
 }
 
 
 int64_t cla_decompress_dev(cla_handle b, double* dOut) {
+	CLA_TRY
 	int rc = check_final(b);
 	if(rc) return rc;
 	if(!dOut) { set_error("decompress: null output"); return -CLA_ERR_INVALID; }
 	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	b->nnzSlot = 0;
 	if((rc = launch_decompress(b, dOut, b->dCounters))) return rc;
 	return finish_nnz(b);
+	CLA_CATCH_CODE(int64_t)
 }
 
 int64_t cla_decompress(cla_handle b, double* out) {
+	CLA_TRY
 	int rc = check_final(b);
 	if(rc) return rc;
 	if(!out) { set_error("decompress: null output"); return -CLA_ERR_INVALID; }
@@ -626,18 +769,33 @@ int64_t cla_decompress(cla_handle b, double* out) {
 	if(nnz < 0) return nnz;
 	if(nOut) CLA_HIP(hipMemcpy(out, b->dStageOut, nOut * sizeof(double), hipMemcpyDeviceToHost));
 	return nnz;
+	CLA_CATCH_CODE(int64_t)
 }
 
-int64_t cla_lmm_dev(cla_handle b, const double* dY, int32_t nRowY, double* dOut) {
+static int64_t lmm_dev(cla_handle b, const double* dY, int32_t nRowY, double* dOut, bool sync) {
 	int rc = check_final(b);
 	if(rc) return rc;
 	if(!dY || !dOut || nRowY <= 0) { set_error("lmm: invalid left-hand side"); return -CLA_ERR_INVALID; }
 	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	b->nnzSlot = 0;
 	if((rc = launch_lmm(b, dY, nRowY, dOut, b->dCounters))) return rc;
-	return finish_nnz(b);
+	return finish_nnz(b, sync);
+}
+
+int64_t cla_lmm_dev(cla_handle b, const double* dY, int32_t nRowY, double* dOut) {
+	CLA_TRY
+	return lmm_dev(b, dY, nRowY, dOut, true);
+	CLA_CATCH_CODE(int64_t)
+}
+
+int cla_lmm_dev_async(cla_handle b, const double* dY, int32_t nRowY, double* dOut) {
+	CLA_TRY
+	return (int) lmm_dev(b, dY, nRowY, dOut, false);
+	CLA_CATCH_CODE(int)
 }
 
 int64_t cla_lmm(cla_handle b, const double* Y, int32_t nRowY, double* out) {
+	CLA_TRY
 	int rc = check_final(b);
 	if(rc) return rc;
 	if(!Y || !out || nRowY <= 0) { set_error("lmm: invalid left-hand side"); return -CLA_ERR_INVALID; }
@@ -650,18 +808,33 @@ int64_t cla_lmm(cla_handle b, const double* Y, int32_t nRowY, double* out) {
 	if(nnz < 0) return nnz;
 	CLA_HIP(hipMemcpy(out, b->dStageOut, nOut * sizeof(double), hipMemcpyDeviceToHost));
 	return nnz;
+	CLA_CATCH_CODE(int64_t)
 }
 
-int64_t cla_tsmm_dev(cla_handle b, double* dOut) {
+static int64_t tsmm_dev(cla_handle b, double* dOut, bool sync) {
 	int rc = check_final(b);
 	if(rc) return rc;
 	if(!dOut) { set_error("tsmm: null output"); return -CLA_ERR_INVALID; }
 	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	b->nnzSlot = 0;
 	if((rc = launch_tsmm(b, dOut, b->dCounters))) return rc;
-	return finish_nnz(b);
+	return finish_nnz(b, sync);
+}
+
+int64_t cla_tsmm_dev(cla_handle b, double* dOut) {
+	CLA_TRY
+	return tsmm_dev(b, dOut, true);
+	CLA_CATCH_CODE(int64_t)
+}
+
+int cla_tsmm_dev_async(cla_handle b, double* dOut) {
+	CLA_TRY
+	return (int) tsmm_dev(b, dOut, false);
+	CLA_CATCH_CODE(int)
 }
 
 int64_t cla_tsmm(cla_handle b, double* out) {
+	CLA_TRY
 	int rc = check_final(b);
 	if(rc) return rc;
 	if(!out) { set_error("tsmm: null output"); return -CLA_ERR_INVALID; }
@@ -672,6 +845,7 @@ int64_t cla_tsmm(cla_handle b, double* out) {
 	if(nnz < 0) return nnz;
 	CLA_HIP(hipMemcpy(out, b->dStageOut, nOut * sizeof(double), hipMemcpyDeviceToHost));
 	return nnz;
+	CLA_CATCH_CODE(int64_t)
 }
 
 } // extern "C"
@@ -748,12 +922,6 @@ static cla_block* make_joint(cla_block* left, cla_block* right) {
 // (built once, kept with `b`), and its Gram matrix is scattered into the result. For a joint block
 // (crossSplit > 0) only chunks of the left side meet chunks of the right side.
 // ---------------------------------------------------------------------------
-struct SubBlock {
-	cla_block* blk;
-	int32_t* dColMap;   // column of `b` per column of blk (-1: padding behind the first chunk)
-	int nA, nB;         // columns of the first (padding included) / second chunk
-	bool writeA, writeB, crossOnly;
-};
 
 __global__ __launch_bounds__(256) void k_scatter_gram(const double* __restrict__ S, int k, const int32_t* __restrict__ colMap, int nA,
 	int writeA, int writeB, int crossOnly, double* __restrict__ out, int n) {
@@ -900,6 +1068,7 @@ int launch_tsmm_chunked(cla_block* b, double* dOut) {
 		SubBlock* sb = (SubBlock*) p;
 		cla_block* c = sb->blk;
 		c->profile = b->profile;
+		c->opt = b->opt;
 		if(c->stream != b->stream) {
 			if(c->ownStream && c->stream) { (void) hipStreamSynchronize(c->stream); (void) hipStreamDestroy(c->stream); }
 			c->stream = b->stream;
@@ -926,6 +1095,7 @@ int launch_tsmm_chunked(cla_block* b, double* dOut) {
 extern "C" {
 
 int64_t cla_lmm_compressed_dev(cla_handle right, cla_handle left, double* dOut) {
+	CLA_TRY
 	int rc = check_final(right);
 	if(rc || (rc = check_final(left))) return rc;
 	if(!dOut) { set_error("compressed left multiply: null output"); return -CLA_ERR_INVALID; }
@@ -947,6 +1117,7 @@ int64_t cla_lmm_compressed_dev(cla_handle right, cla_handle left, double* dOut) 
 	}
 	cla_block* c = right->joint;
 	c->profile = right->profile;
+	c->opt = right->opt;
 	// the joint block works on the right block's stream
 	if(c->stream != right->stream) {
 		if(c->ownStream && c->stream) { (void) hipStreamSynchronize(c->stream); (void) hipStreamDestroy(c->stream); }
@@ -956,6 +1127,7 @@ int64_t cla_lmm_compressed_dev(cla_handle right, cla_handle left, double* dOut) 
 	const size_t n = (size_t) c->nCols;
 	if((rc = ensure_stage(&c->dStageOut, &c->stageOutCap, n * n))) return rc;
 	if((rc = launch_tsmm(c, c->dStageOut, c->dCounters))) return rc;
+	right->nnzSlot = 0;
 	CLA_HIP(hipMemsetAsync(right->dCounters, 0, sizeof(unsigned long long), right->stream));
 	const int nOut = left->nCols * right->nCols;
 	{
@@ -967,9 +1139,11 @@ int64_t cla_lmm_compressed_dev(cla_handle right, cla_handle left, double* dOut) 
 	clear_stats(right);
 	right->lastStats.swap(c->lastStats); // what the kernel statistics of `right` report
 	return finish_nnz(right);
+	CLA_CATCH_CODE(int64_t)
 }
 
 int64_t cla_lmm_compressed(cla_handle right, cla_handle left, double* out) {
+	CLA_TRY
 	int rc = check_final(right);
 	if(rc || (rc = check_final(left))) return rc;
 	if(!out) { set_error("compressed left multiply: null output"); return -CLA_ERR_INVALID; }
@@ -984,9 +1158,11 @@ int64_t cla_lmm_compressed(cla_handle right, cla_handle left, double* out) {
 	if(nnz < 0) return nnz;
 	CLA_HIP(hipMemcpy(out, right->dStageOut, nOut * sizeof(double), hipMemcpyDeviceToHost));
 	return nnz;
+	CLA_CATCH_CODE(int64_t)
 }
 
 cla_handle cla_rmm_overlapping(cla_handle b, const double* B, int32_t nColB) {
+	CLA_TRY
 	if(check_final(b)) return nullptr;
 	if(!B || nColB <= 0) { set_error("rmm: invalid right-hand side"); return nullptr; }
 	if(b->hasUnc) { set_error("overlapping right multiply: uncompressed groups are not supported"); return nullptr; }
@@ -1046,18 +1222,23 @@ cla_handle cla_rmm_overlapping(cla_handle b, const double* B, int32_t nColB) {
 	b->refs.fetch_add(1);
 	if(finish_finalize(c, b)) { cla_block_free(c); return nullptr; }
 	return c;
+	CLA_CATCH_NULL
 }
 
 int64_t cla_aggregate_dev(cla_handle b, int32_t op, int32_t dir, double* dOut) {
+	CLA_TRY
 	int rc = check_final(b);
 	if(rc) return rc;
 	if(!dOut) { set_error("aggregate: null output"); return -CLA_ERR_INVALID; }
 	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	b->nnzSlot = 0;
 	if((rc = launch_aggregate(b, op, dir, dOut, b->dCounters))) return rc;
 	return finish_nnz(b);
+	CLA_CATCH_CODE(int64_t)
 }
 
 int64_t cla_aggregate(cla_handle b, int32_t op, int32_t dir, double* out) {
+	CLA_TRY
 	int rc = check_final(b);
 	if(rc) return rc;
 	if(!out) { set_error("aggregate: null output"); return -CLA_ERR_INVALID; }
@@ -1069,20 +1250,35 @@ int64_t cla_aggregate(cla_handle b, int32_t op, int32_t dir, double* out) {
 	if(nnz < 0) return nnz;
 	if(nOut) CLA_HIP(hipMemcpy(out, b->dStageOut, nOut * sizeof(double), hipMemcpyDeviceToHost));
 	return nnz;
+	CLA_CATCH_CODE(int64_t)
 }
 
-int64_t cla_mmchain_dev(cla_handle b, const double* dV, const double* dW, int32_t ctype, double* dOut) {
+static int64_t mmchain_dev(cla_handle b, const double* dV, const double* dW, int32_t ctype, double* dOut, bool sync) {
 	int rc = check_final(b);
 	if(rc) return rc;
 	if(!dV || !dOut) { set_error("mmchain: null vector"); return -CLA_ERR_INVALID; }
 	if(ctype < 0 || ctype > 2) { set_error("mmchain: chain type %d not supported (XtXv=0, XtwXv=1, XtXvy=2)", ctype); return -CLA_ERR_UNSUPPORTED; }
 	if(ctype != 0 && !dW) { set_error("mmchain: XtwXv and XtXvy need w"); return -CLA_ERR_INVALID; }
 	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	b->nnzSlot = 0;
 	if((rc = launch_mmchain(b, dV, dW, ctype, dOut, b->dCounters))) return rc;
-	return finish_nnz(b);
+	return finish_nnz(b, sync);
+}
+
+int64_t cla_mmchain_dev(cla_handle b, const double* dV, const double* dW, int32_t ctype, double* dOut) {
+	CLA_TRY
+	return mmchain_dev(b, dV, dW, ctype, dOut, true);
+	CLA_CATCH_CODE(int64_t)
+}
+
+int cla_mmchain_dev_async(cla_handle b, const double* dV, const double* dW, int32_t ctype, double* dOut) {
+	CLA_TRY
+	return (int) mmchain_dev(b, dV, dW, ctype, dOut, false);
+	CLA_CATCH_CODE(int)
 }
 
 int64_t cla_mmchain(cla_handle b, const double* v, const double* w, int32_t ctype, double* out) {
+	CLA_TRY
 	int rc = check_final(b);
 	if(rc) return rc;
 	if(!v || !out) { set_error("mmchain: null vector"); return -CLA_ERR_INVALID; }
@@ -1097,9 +1293,11 @@ int64_t cla_mmchain(cla_handle b, const double* v, const double* w, int32_t ctyp
 	if(nnz < 0) return nnz;
 	CLA_HIP(hipMemcpy(out, b->dStageOut, nV * sizeof(double), hipMemcpyDeviceToHost));
 	return nnz;
+	CLA_CATCH_CODE(int64_t)
 }
 
 int cla_cooc(cla_handle b, int32_t gA, int32_t gB, int64_t* out) {
+	CLA_TRY
 	int rc = check_final(b);
 	if(rc) return rc;
 	const int nG = (int) b->groups.size();
@@ -1112,9 +1310,11 @@ int cla_cooc(cla_handle b, int32_t gA, int32_t gB, int64_t* out) {
 	CLA_HIP(hipMemcpyAsync(out, b->dScratch, n * sizeof(int64_t), hipMemcpyDeviceToHost, b->stream));
 	CLA_HIP(hipStreamSynchronize(b->stream));
 	return 0;
+	CLA_CATCH_CODE(int)
 }
 
 int cla_preagg(cla_handle b, int32_t group, const double* Y, int32_t nRowY, double* preAgg) {
+	CLA_TRY
 	int rc = check_final(b);
 	if(rc) return rc;
 	if(group < 0 || group >= (int) b->groups.size() || !Y || !preAgg || nRowY <= 0) { set_error("preagg: bad arguments"); return -CLA_ERR_INVALID; }
@@ -1129,9 +1329,11 @@ int cla_preagg(cla_handle b, int32_t group, const double* Y, int32_t nRowY, doub
 	CLA_HIP(hipMemcpyAsync(preAgg, b->dStageOut, nOut * sizeof(double), hipMemcpyDeviceToHost, b->stream));
 	CLA_HIP(hipStreamSynchronize(b->stream));
 	return 0;
+	CLA_CATCH_CODE(int)
 }
 
 int cla_counts(cla_handle b, int32_t group, int32_t* counts) {
+	CLA_TRY
 	int rc = check_final(b);
 	if(rc) return rc;
 	if(group < 0 || group >= (int) b->groups.size() || !counts) { set_error("counts: bad group %d", group); return -CLA_ERR_INVALID; }
@@ -1143,16 +1345,20 @@ int cla_counts(cla_handle b, int32_t group, int32_t* counts) {
 	CLA_HIP(hipMemcpyAsync(counts, b->dScratch, sizeof(int32_t) * (size_t) nVals, hipMemcpyDeviceToHost, b->stream));
 	CLA_HIP(hipStreamSynchronize(b->stream));
 	return 0;
+	CLA_CATCH_CODE(int)
 }
 
 int cla_block_profile(cla_handle b, int enable) {
+	CLA_TRY
 	if(!b) { set_error("null block handle"); return -CLA_ERR_INVALID; }
 	std::lock_guard<std::recursive_mutex> lk(b->mu);
 	b->profile = enable != 0;
 	return 0;
+	CLA_CATCH_CODE(int)
 }
 
 int cla_stats(cla_handle b, char* json, size_t cap) {
+	CLA_TRY
 	if(!b || !json || cap < 8) return -CLA_ERR_INVALID;
 	std::lock_guard<std::recursive_mutex> lk(b->mu);
 	if(b->stream) (void) hipStreamSynchronize(b->stream);
@@ -1170,6 +1376,7 @@ int cla_stats(cla_handle b, char* json, size_t cap) {
 	if(s.size() + 1 > cap) return -CLA_ERR_INVALID;
 	memcpy(json, s.c_str(), s.size() + 1);
 	return 0;
+	CLA_CATCH_CODE(int)
 }
 
 } // extern "C"

@@ -58,6 +58,21 @@ struct HostGroup {
 	int64_t bytes = 0;              // HBM bytes of the compressed representation
 };
 
+// Per-block switches set through cla_block_set_option. The defaults are the tuned dispatch; the
+// other values force one of the alternative kernels of a driver (each is a complete
+// implementation of the same product, so forcing one is how the tests cover it).
+struct Options {
+	int tsmmRoute = 0;      // 0 cost model, 1 one kernel pass per pair of groups, 2 decoded Gram matrix
+	int tsmmChunks = 1;     // more than 64 columns: decoded Gram matrices of pairs of column chunks
+	int tsmmWideDense = 0;  // more than 64 columns and as many groups as columns: scalar decompressing form
+	int tsmmMfma = 1;       // decoded Gram matrix on the matrix cores (0: scalar form)
+	int tsmmPairDot = 1;    // DDC x DDC pairs in dot form (0: pre-aggregate form with LDS bins)
+	int expandStreams = 1;  // one code per row for small RLE / SDCZeros groups in the decode kernels
+	int rmmDisable = 0;     // bit 0 byte-code mat-vec, 1 fused tables of the byte-code mat-vec, 2 matrix-core kernel, 3 decode kernel
+	int lmmDisable = 0;     // bit 0 dot form on byte codes, 1 byte-code bin kernel
+	int sdcPacked = 1;      // packed SDCZeros lists for the mat-vecs
+};
+
 struct KernelStat {
 	std::string name;
 	long grid = 0, block = 0, lds = 0;
@@ -98,6 +113,7 @@ struct cla_block {
 	int32_t totalColsG = 0;          // sum of nColG over groups
 	int32_t maxVals = 0;
 	int64_t device_bytes_cached = 0; // HBM bytes of the compressed representation (set at finalize)
+	int64_t derivedBytes = 0;        // HBM bytes of the formats derived from it so far (packed lists, expanded streams, padded dictionaries, counts)
 
 	hipStream_t stream = nullptr;
 	bool ownStream = false;
@@ -124,6 +140,7 @@ struct cla_block {
 	double* dStageIn = nullptr; size_t stageInCap = 0;
 	double* dStageOut = nullptr; size_t stageOutCap = 0;
 	void* dScratch = nullptr;   size_t scratchCap = 0;
+	double* dChain = nullptr;   size_t chainCap = 0;   // X %*% v inside the multiply chain
 	// exact code counts of all dictionary-coded groups (totalVals int32, group g at tblOff[g]),
 	// computed on the first TSMM and kept, like the reference's cached counts
 	// (CG/AColGroupValue.java getCounts)
@@ -148,6 +165,13 @@ struct cla_block {
 
 	std::vector<cla::KernelStat> lastStats;
 	bool profile = false;            // bracket every kernel with HIP events on `stream`
+	cla::Options opt;
+	// Non-zero counter of the last driver call: index into dCounters. Slot 0 is cleared by the first
+	// kernel of a driver; the fused mat-vec kernel rotates over slots 1-3 instead (it counts into one
+	// and clears the next, so that no separate clearing step runs between two calls).
+	int nnzSlot = 0;
+	int nnzRot = 1;
+	bool poisoned = false;           // a failed finalize left the block half built: only free is allowed
 };
 
 namespace cla {
@@ -202,6 +226,7 @@ struct Prof {
 void clear_stats(cla_block* b);
 
 int ensure_tables(cla_block* b, size_t nDoubles);
+int ensure_dict_pad(cla_block* b); // padded dictionary image of byte-code blocks with one column per group (no-op otherwise)
 int ensure_scratch(cla_block* b, size_t bytes);
 
 } // namespace cla

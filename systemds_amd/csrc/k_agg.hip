@@ -67,15 +67,17 @@ __global__ __launch_bounds__(256) void k_agg_cols_dict(const DGroup* __restrict_
 }
 
 // grid (row chunks, columns of the group): partial[chunk * nC + j]
+// (sum of squares: the column's filtered constant c enters as (v + c)^2 - c^2, like the dictionary form; n c^2 is added at the end)
 __global__ __launch_bounds__(256) void k_agg_cols_dense(const double* __restrict__ dense, int64_t nRows, int nC, int64_t rowsPerBlock,
-	int op, double* __restrict__ partial) {
+	int op, const int32_t* __restrict__ cols, const double* __restrict__ constV, double* __restrict__ partial) {
 	__shared__ double red[4];
 	const int j = blockIdx.y;
+	const double c = op == CLA_AGG_SUMSQ ? constV[cols[j]] : 0.0;
 	const int64_t r0 = (int64_t) blockIdx.x * rowsPerBlock, r1 = min(nRows, r0 + rowsPerBlock);
 	double a = agg_identity(op);
 	for(int64_t r = r0 + threadIdx.x; r < r1; r += 256) {
 		const double v = dense[(size_t) r * nC + j];
-		a = op == CLA_AGG_SUMSQ ? a + v * v : agg_combine(op, a, v);
+		a = op == CLA_AGG_SUMSQ ? a + ((v + c) * (v + c) - c * c) : agg_combine(op, a, v);
 	}
 	a = block_reduce(op, a, red);
 	if(threadIdx.x == 0) partial[(size_t) blockIdx.x * nC + j] = a;
@@ -130,6 +132,7 @@ int ensure_counts(cla_block* b) {
 	if(b->dCountsAll != nullptr) return 0;
 	int32_t* dc = nullptr;
 	CLA_HIP(hipMalloc((void**) &dc, sizeof(int32_t) * (size_t) std::max(b->totalVals, 1)));
+	b->derivedBytes += (int64_t) sizeof(int32_t) * std::max(b->totalVals, 1);
 	CLA_HIP(hipMemsetAsync(dc, 0, sizeof(int32_t) * (size_t) std::max(b->totalVals, 1), b->stream));
 	for(int g = 0; g < (int) b->groups.size(); g++) {
 		const int type = b->groups[g].d.type;
@@ -206,7 +209,7 @@ int launch_aggregate(cla_block* b, int op, int dir, double* dOut, unsigned long 
 		const DGroup& G = b->groups[g].d;
 		if(G.type != G_UNC) continue;
 		Prof pf(b, "k_agg_cols_dense", (long) nChunks * G.nColG, 256, 0, (double) nRows * G.nColG * 8);
-		hipLaunchKernelGGL(k_agg_cols_dense, dim3(nChunks, G.nColG), dim3(256), 0, st, G.dense, nRows, G.nColG, rowsPerBlock, op, dPartial);
+		hipLaunchKernelGGL(k_agg_cols_dense, dim3(nChunks, G.nColG), dim3(256), 0, st, G.dense, nRows, G.nColG, rowsPerBlock, op, G.cols, b->dConstV, dPartial);
 		hipLaunchKernelGGL(k_agg_cols_dense_fold, dim3(1), dim3(256), 0, st, dPartial, nChunks, G.nColG, G.cols, op, dAgg);
 	}
 	{

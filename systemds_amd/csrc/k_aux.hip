@@ -185,6 +185,7 @@ int launch_sdc_build(cla_block* b, HostGroup& g) {
 	OffState* ckpt = nullptr;
 	OffState* tiles = nullptr;
 	int2* sums = nullptr;
+	struct FreeSums { int2*& p; ~FreeSums() { if(p) (void) hipFree(p); } } freeSums{sums}; // on every way out
 	CLA_HIP(hipMalloc((void**) &ckpt, sizeof(OffState) * (size_t) (nCkpt + 1)));
 	g.owned.push_back(ckpt);
 	CLA_HIP(hipMalloc((void**) &tiles, sizeof(OffState) * (size_t) (nTiles > 0 ? nTiles : 1)));
@@ -217,7 +218,6 @@ int launch_sdc_build(cla_block* b, HostGroup& g) {
 	OffState fin;
 	CLA_HIP(hipMemcpyAsync(&fin, ckpt + nCkpt, sizeof(OffState), hipMemcpyDeviceToHost, st));
 	CLA_HIP(hipStreamSynchronize(st));
-	if(sums) CLA_HIP(hipFree(sums));
 	CLA_HIP(hipGetLastError());
 	if(fin.row != G.last || fin.emit != G.nOffsets) {
 		set_error("SDC offsets inconsistent: decoded last row %d / %d rows, declared offsetToLast %d / %lld rows",

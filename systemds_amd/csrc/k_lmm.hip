@@ -332,10 +332,18 @@ __global__ __launch_bounds__(256) void k_sub_inplace(double* __restrict__ x, con
 
 int launch_mmchain(cla_block* b, const double* dV, const double* dW, int ctype, double* dOut, unsigned long long* dNnz) {
 	const int64_t nRows = b->nRows;
-	int rc = ensure_scratch(b, sizeof(double) * (size_t) std::max<int64_t>(nRows, 1));
-	if(rc) return rc;
-	double* tmp = (double*) b->dScratch;
+	// the intermediate vector has a workspace of its own: the multiplies below may resize the shared scratch
+	const size_t need = (size_t) std::max<int64_t>(nRows, 1);
+	if(need > b->chainCap) {
+		if(b->dChain) CLA_HIP(hipFree(b->dChain));
+		b->dChain = nullptr; b->chainCap = 0;
+		CLA_HIP(hipMalloc((void**) &b->dChain, need * sizeof(double)));
+		b->chainCap = need;
+	}
+	double* tmp = b->dChain;
+	int rc;
 	if((rc = launch_rmm(b, dV, 1, tmp, dNnz))) return rc;
+	b->nnzSlot = 0; // the left multiply below counts the result's non-zeros into dNnz
 	std::vector<KernelStat> first;
 	first.swap(b->lastStats);
 	if(ctype == 1 && nRows > 0)

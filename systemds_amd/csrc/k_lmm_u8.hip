@@ -116,7 +116,7 @@ __global__ __launch_bounds__(LU_THREADS) void k_lmm_u8(const DGroup* __restrict_
 int launch_lmm_u8(cla_block* b, const double* dY, int p, double* dPre) {
 	const int nG = (int) b->groups.size();
 	if(!(b->dArena && b->arenaWidth == 1 && b->maxVals <= 256 && nG > 0 && b->nRows > 0)) return 1;
-	if(getenv("CLA_LMM_GENERIC")) return 1;
+	if(b->opt.lmmDisable & 2) return 1;
 	// one persistent block per CU and row of Y; small inputs get a block per 4096 rows
 	const unsigned grid = (unsigned) std::min<int64_t>((b->nRows + 4095) / 4096, std::max(1, g_numCU / std::min(p, g_numCU)));
 	const double algo = (double) p * ((double) b->nRows * nG + (double) b->nRows * 8);
@@ -284,28 +284,39 @@ __global__ __launch_bounds__(LD_THREADS, 4) void k_lmm_u8_dot(const uint8_t* __r
 	}
 }
 
+// All groups DDC with byte codes in one arena and one column each: the dictionaries at a fixed stride of
+// 256 entries (zero beyond nVals), followed by the groups' column indexes. Built once at finalize (200 KB
+// for 100 groups); the byte-code mat-vec and the dot-form left multiply read their slabs from it.
+int ensure_dict_pad(cla_block* b) {
+	const int nG = (int) b->groups.size();
+	if(b->dDictPad != nullptr || !(b->dArena && b->arenaWidth == 1 && b->maxVals <= 256 && nG > 0 && b->nRows > 0)) return 0;
+	for(int g = 0; g < nG; g++)
+		if(b->groups[g].d.nColG != 1) return 0;
+	std::vector<double> img((size_t) nG * 256 + (size_t) (nG + 1) / 2 + 1, 0.0);
+	int32_t* cols = (int32_t*) (img.data() + (size_t) nG * 256);
+	for(int g = 0; g < nG; g++) {
+		const HostGroup& H = b->groups[g];
+		std::copy(H.dict.begin(), H.dict.begin() + H.d.nVals, img.begin() + (size_t) g * 256);
+		cols[g] = H.cols[0];
+	}
+	CLA_HIP(hipMalloc((void**) &b->dDictPad, img.size() * sizeof(double)));
+	b->derivedBytes += (int64_t) (img.size() * sizeof(double));
+	CLA_HIP(hipMemcpy(b->dDictPad, img.data(), img.size() * sizeof(double), hipMemcpyHostToDevice));
+	return 0;
+}
+
 // Returns 1 when the block is not eligible, 0 when the groups' contributions have been added to dOut.
 int launch_lmm_u8_dot(cla_block* b, const double* dY, int p, double* dOut) {
 	const int nG = (int) b->groups.size();
 	if(!(b->dArena && b->arenaWidth == 1 && b->maxVals <= 256 && nG > 0 && b->nRows > 0)) return 1;
-	if(getenv("CLA_LMM_GENERIC") || getenv("CLA_LMM_BINS")) return 1;
+	if(b->opt.lmmDisable & 1) return 1;
 	for(int g = 0; g < nG; g++)
 		if(b->groups[g].d.nColG != 1) return 1;
 	constexpr int PER = 20;
 	const int nPad = (nG + PER - 1) / PER * PER;
 	const size_t lds = (size_t) PER * 256 * 8 + (size_t) nPad * LD_SLOTS * 8;
 	if(lds > (size_t) 78 * 1024) return 1; // two blocks per CU
-	if(b->dDictPad == nullptr) {
-		std::vector<double> img((size_t) nG * 256 + (size_t) (nG + 1) / 2 + 1, 0.0);
-		int32_t* cols = (int32_t*) (img.data() + (size_t) nG * 256);
-		for(int g = 0; g < nG; g++) {
-			const HostGroup& H = b->groups[g];
-			std::copy(H.dict.begin(), H.dict.begin() + H.d.nVals, img.begin() + (size_t) g * 256);
-			cols[g] = H.cols[0];
-		}
-		CLA_HIP(hipMalloc((void**) &b->dDictPad, img.size() * sizeof(double)));
-		CLA_HIP(hipMemcpy(b->dDictPad, img.data(), img.size() * sizeof(double), hipMemcpyHostToDevice));
-	}
+	if(b->dDictPad == nullptr) return 1;
 	const int32_t* dCol0 = (const int32_t*) (b->dDictPad + (size_t) nG * 256);
 	const int perCU = 2;
 	const unsigned grid = (unsigned) std::min<int64_t>((b->nRows + 2047) / 2048, std::max(1, g_numCU * perCU / std::min(p, g_numCU * perCU)));

@@ -241,10 +241,18 @@ __device__ __forceinline__ void u8_consume(const CodeVec<1, RPT> (&cv)[NB], cons
 }
 
 // U8_PER is a multiple of 2 * U8_NB. The host picks the variant that pads least.
-template <int THREADS, int U8_PER, int U8_NB, int LB, int LN>
+//
+// FUSED (every group has one column): the tables are not read from a pre-aggregated image but made
+// on the way into LDS, table_g[k] = dict_g[k] * v[col_g] (Dictionary.preaggValuesFromDense for one
+// column: a zero dictionary cell stays zero whatever v holds, and 0 + d * v rounds once, so the
+// entries are bit-identical to the pre-aggregation kernel's). `Tpad` is then the padded dictionary
+// image (256 entries per group, zero beyond nVals), `col0` the groups' columns. Block 0 clears
+// *nnzNext, the counter of the next call, so that no clearing step runs between two calls.
+template <int THREADS, int U8_PER, int U8_NB, int LB, int LN, bool FUSED>
 __global__ __launch_bounds__(THREADS, 4) void k_rmm_q1_u8(const uint8_t* __restrict__ arena, size_t arenaStride,
 	int nGroups, const double* __restrict__ Tpad, const double* __restrict__ constTerm,
-	double* __restrict__ out, int64_t nRows, unsigned long long* __restrict__ nnz) {
+	double* __restrict__ out, int64_t nRows, unsigned long long* __restrict__ nnz,
+	const int32_t* __restrict__ col0, const double* __restrict__ v, unsigned long long* __restrict__ nnzNext) {
 	__shared__ double tbl[U8_PER * 256];
 	__shared__ double wbufAll[(THREADS / 64) * 64 * 8]; // per-wave transpose buffers of the epilogue
 	const char* tb = (const char*) tbl;
@@ -278,6 +286,15 @@ __global__ __launch_bounds__(THREADS, 4) void k_rmm_q1_u8(const uint8_t* __restr
 	// the tables of the next slab are fetched into registers while the current slab is processed
 	constexpr int TPT = (U8_PER * 256 + THREADS - 1) / THREADS;
 	double stage[TPT];
+	// FUSED: a non-finite v[col] must not meet a zero dictionary cell (0 * inf); the plain product serves otherwise
+	bool careful = false;
+	if(FUSED) {
+		static_assert(!FUSED || THREADS % 256 == 0, "a wave's table entries belong to one group");
+		if(blockIdx.x == 0 && tid == 0) *nnzNext = 0;
+		int bad = 0;
+		for(int g = tid; g < nGroups; g += THREADS) bad |= !isfinite(v[col0[g]]);
+		careful = __syncthreads_or(bad) != 0;
+	}
 	auto fetch = [&](int g0) { // tables g0 .. g0 + U8_PER - 1 of the padded image (zero beyond the last group)
 		const int nIn = min(U8_PER, nGroups - g0) * 256;
 		const double* src = Tpad + (size_t) g0 * 256;
@@ -286,7 +303,14 @@ __global__ __launch_bounds__(THREADS, 4) void k_rmm_q1_u8(const uint8_t* __restr
 #pragma unroll
 		for(int k = 0; k < TPT; k++) {
 			const int f = tidF + k * THREADS;
-			stage[k] = f < nIn ? src[f] : 0.0;
+			if(FUSED) {
+				// entry f belongs to group g0 + f / 256, the same for the whole wave: v comes through scalar loads
+				const int gs = __builtin_amdgcn_readfirstlane(g0 + (tid >> 8) + k * (THREADS / 256));
+				const double vv = gs < nGroups ? v[col0[gs]] : 0.0;
+				const double d = f < nIn ? src[f] : 0.0;
+				stage[k] = careful ? (d != 0.0 ? d * vv : 0.0) : d * vv;
+			}
+			else stage[k] = f < nIn ? src[f] : 0.0;
 		}
 	};
 	fetch(0);
@@ -518,53 +542,59 @@ int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned lon
 	hipStream_t st = b->stream;
 	clear_stats(b);
 	// mat-vec on byte codes: all groups DDC in one arena, at most 256 values each
-	const bool u8Path = q == 1 && nRows > 0 && b->dArena && b->arenaWidth == 1 && b->maxVals <= 256 && !getenv("CLA_Q1_GENERIC");
+	const bool u8Path = q == 1 && nRows > 0 && b->dArena && b->arenaWidth == 1 && b->maxVals <= 256 && !(b->opt.rmmDisable & 1);
 	const size_t nTbl = (size_t) (b->totalVals + 1) * q;
 	int rc = ensure_tables(b, nTbl + (u8Path ? (size_t) nG * 256 + 256 : 0));
 	if(rc) return rc;
 	double* dTpad = u8Path ? b->dTables + ((nTbl + 31) & ~(size_t) 31) : nullptr;
 
+	// Byte-code mat-vec with one column per group: the gather kernel makes its tables itself from the
+	// padded dictionary image (built at finalize) and counts into a counter of its own that the call
+	// before has cleared, so it is the only launch (K1 only runs for the constants' term, if any).
+	const bool fused = u8Path && !squares && b->dDictPad != nullptr && !(b->opt.rmmDisable & 2);
+	const int32_t* dCol0 = fused ? (const int32_t*) (b->dDictPad + (size_t) nG * 256) : nullptr;
+	if(fused) {
+		b->nnzSlot = b->nnzRot;
+		dNnz = b->dCounters + b->nnzSlot;
+	}
 	// K1 (also clears the non-zero counter)
-	{
-		const int maxWork = (u8Path ? 256 : (b->maxVals > 1 ? b->maxVals : 1)) * q;
-		dim3 grid((maxWork + 255) / 256 > (q + 255) / 256 ? (maxWork + 255) / 256 : (q + 255) / 256, nG + 1);
+	if(!fused || b->hasConst) {
+		const int nK1 = fused ? 0 : nG; // fused: the constants' row only
+		const int maxWork = (u8Path && !fused ? 256 : (b->maxVals > 1 ? b->maxVals : 1)) * q;
+		dim3 grid(fused ? 1 : ((maxWork + 255) / 256 > (q + 255) / 256 ? (maxWork + 255) / 256 : (q + 255) / 256), nK1 + 1);
 		Prof pf(b, "k_preagg", (long) grid.x * grid.y, 256, 0, 0);
-		hipLaunchKernelGGL(k_preagg, grid, dim3(256), 0, st, b->dGroups, nG, dB, q, b->nCols,
-			b->hasConst ? b->dConstV : nullptr, b->dTables, b->totalVals, dNnz, dTpad, squares);
+		hipLaunchKernelGGL(k_preagg, grid, dim3(256), 0, st, b->dGroups, nK1, dB, q, b->nCols,
+			b->hasConst ? b->dConstV : nullptr, b->dTables, b->totalVals, dNnz, fused ? nullptr : dTpad, squares);
 	}
 	const int constRow = b->hasConst ? b->totalVals : -1;
 	if(nRows == 0) return 0;
 
 	if(u8Path) {
 		constexpr int THREADS = 512;
-		const int64_t rowsPerBlock = (int64_t) THREADS * U8_RPT;
-		(void) rowsPerBlock;
 		// persistent blocks: two per CU is what the register and LDS footprint allows; small
 		// inputs get a block per 2048 rows
-		int perCU = 2;
-		if(const char* e = getenv("CLA_Q1_BLOCKS_PER_CU")) perCU = std::max(1, atoi(e));
+		const int perCU = 2;
 		const unsigned grid = (unsigned) std::min<int64_t>((nRows + 2047) / 2048, (int64_t) g_numCU * perCU);
 		const double bytes = (double) nRows * nG + (double) nRows * 8 + (double) b->totalVals * 8;
 		// slab size: 16 or 20 groups, whichever leaves fewer padded table slots
 		const int pad16 = (nG + 15) / 16 * 16 - nG, pad20 = (nG + 19) / 20 * 20 - nG;
-		int per = pad20 < pad16 ? 20 : 16;
-		if(const char* e = getenv("CLA_Q1_PER")) per = atoi(e) == 20 ? 20 : 16;
+		const int per = pad20 < pad16 ? 20 : 16;
+		const double* constTerm = constRow >= 0 ? b->dTables + constRow : nullptr;
+		unsigned long long* nnzNext = fused ? b->dCounters + (b->nnzRot % 3 + 1) : nullptr;
 		Prof pf(b, "k_rmm_q1_u8", grid, THREADS, per * 256 * 8, bytes);
-#define U8_LAUNCH(PER, NBV, LB, LN)                                                                             \
-	hipLaunchKernelGGL((k_rmm_q1_u8<THREADS, PER, NBV, LB, LN>), dim3(grid), dim3(THREADS), 0, st, b->dArena,   \
-		b->arenaStride, nG, dTpad, constRow >= 0 ? b->dTables + constRow : nullptr, dOut, nRows, dNnz)
-		if(per == 20) U8_LAUNCH(20, 5, 4, 2);
-		else U8_LAUNCH(16, 4, 8, 2);
+#define U8_LAUNCH(PER, NBV, LB, LN, F)                                                                          \
+	hipLaunchKernelGGL((k_rmm_q1_u8<THREADS, PER, NBV, LB, LN, F>), dim3(grid), dim3(THREADS), 0, st, b->dArena, \
+		b->arenaStride, nG, F ? b->dDictPad : dTpad, constTerm, dOut, nRows, dNnz, dCol0, dB, nnzNext)
+		if(per == 20) { if(fused) U8_LAUNCH(20, 5, 4, 2, true); else U8_LAUNCH(20, 5, 4, 2, false); }
+		else { if(fused) U8_LAUNCH(16, 4, 8, 2, true); else U8_LAUNCH(16, 4, 8, 2, false); }
 #undef U8_LAUNCH
 		CLA_HIP(hipGetLastError());
+		if(fused) b->nnzRot = b->nnzRot % 3 + 1;
 		return 0;
 	}
 	if(q == 1 && b->dArena && b->q1LdsBytes > 0) {
 		const int cw = b->arenaWidth;
-		int threads = 256, rpt = cw == 4 ? 8 : 16;
-		if(const char* e = getenv("CLA_Q1_THREADS")) threads = atoi(e);
-		if(const char* e = getenv("CLA_Q1_RPT")) rpt = atoi(e);
-		if(cw == 4 && rpt > 16) rpt = 16;
+		const int threads = 256, rpt = cw == 4 ? 8 : 16;
 		const int64_t rowsPerBlock = (int64_t) threads * rpt;
 		const unsigned grid = (unsigned) ((nRows + rowsPerBlock - 1) / rowsPerBlock);
 		const int nSlabs = (int) b->q1Slabs.size();
@@ -594,13 +624,13 @@ int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned lon
 	}
 
 	// wide B on an all-DDC block: fused decode + fp64 MFMA (K1 above still supplies constV x B)
-	if(q >= 8 && !getenv("CLA_NO_MFMA")) {
+	if(q >= 8 && !(b->opt.rmmDisable & 4)) {
 		const int r = launch_rmm_mfma(b, dB, q, constRow >= 0 ? b->dTables + (size_t) constRow * q : nullptr, dOut, dNnz);
 		if(r <= 0) return r;
 	}
 
 	// narrow B on any group mix: decode rows from LDS dictionaries, B rows as scalars
-	if(q >= 2 && q <= 16 && !getenv("CLA_NO_DECODE")) {
+	if(q >= 2 && q <= 16 && !(b->opt.rmmDisable & 8)) {
 		const int r = launch_rmm_decode(b, dB, q, constRow >= 0 ? b->dTables + (size_t) constRow * q : nullptr, dOut, dNnz);
 		if(r <= 0) return r;
 	}

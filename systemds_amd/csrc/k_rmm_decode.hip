@@ -572,7 +572,7 @@ static int ensure_expanded(cla_block* b) {
 	b->expTried = true;
 	const int nG = (int) b->groups.size();
 	b->expCodes.assign((size_t) nG, nullptr);
-	if(getenv("CLA_DEC_NO_EXPAND") != nullptr || b->nRows == 0) return 0;
+	if(!b->opt.expandStreams || b->nRows == 0) return 0;
 	std::vector<int> cand;
 	for(int g = 0; g < nG; g++) {
 		const DGroup& G = b->groups[g].d;
@@ -583,6 +583,7 @@ static int ensure_expanded(cla_block* b) {
 		const DGroup& G = b->groups[g].d;
 		uint8_t* p = nullptr;
 		CLA_HIP(hipMalloc((void**) &p, (size_t) b->nRows + 16));
+		b->derivedBytes += b->nRows + 16;
 		b->expCodes[g] = p;
 		if(G.type == G_RLE)
 			hipLaunchKernelGGL(k_expand_rle, dim3((unsigned) ((b->nRows + 1023) / 1024)), dim3(256), 0, b->stream, b->dGroups, g, b->nRows, p);

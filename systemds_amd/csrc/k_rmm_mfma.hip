@@ -288,12 +288,10 @@ int launch_rmm_mfma(cla_block* b, const double* dB, int q, const double* dConstR
 		blockWidth = std::max(blockWidth, g.d.codeWidth);
 	}
 	// 8 waves per block (512-row tiles, two waves per SIMD), one block per CU with two slab buffers
-	int waves = 8;
-	if(const char* e = getenv("CLA_MFMA_WAVES")) waves = atoi(e) == 4 ? 4 : 8;
+	const int waves = 8;
 	const int rows = waves * MF_MT * 16;
 	const size_t stageBytes = (size_t) waves * 8 * MF_SS * 8;
-	int ldsKb = 156;
-	if(const char* e = getenv("CLA_MFMA_LDS_KB")) ldsKb = atoi(e);
+	const int ldsKb = 156;
 	const size_t fixedBytes = (size_t) nColsAll * sizeof(MfSrc) + 32 * sizeof(MfSlab);
 	const size_t ldsTotal = (size_t) std::min(g_ldsPerBlock - 1024, ldsKb * 1024);
 	if(ldsTotal < fixedBytes + 2 * stageBytes) return 1;

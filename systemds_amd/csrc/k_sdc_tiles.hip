@@ -356,6 +356,7 @@ static int sdc_plan(cla_block* b, int onlyGroup, int32_t** dList, int32_t** dBin
 		}
 		if(packable && b->dSdcPacked == nullptr) {
 			CLA_HIP(hipMalloc((void**) &b->dSdcPacked, sizeof(uint32_t) * (size_t) (totalEntries + 256)));
+			b->derivedBytes += (int64_t) sizeof(uint32_t) * (totalEntries + 256);
 			CLA_HIP(hipMemsetAsync(b->dSdcPacked + totalEntries, 0, sizeof(uint32_t) * 256, b->stream));
 			const int nT1 = (int) ((b->nRows + SDC_TILE - 1) / SDC_TILE);
 			for(size_t l = 0; l < b->sdcList.size(); l++)
@@ -399,7 +400,7 @@ int launch_lmm_sdc_tiles(cla_block* b, const double* dY, int p, double* dPre, in
 	if(plan.list.empty()) return 0;
 	// all listed groups single-column with at most 64 tuples, whole-block call: products straight
 	// into dOut, the groups' part of dPre stays zero
-	static const bool noPacked = getenv("CLA_SDC_NO_PACKED") != nullptr;
+	const bool noPacked = !b->opt.sdcPacked;
 	bool packed = dOut != nullptr && onlyGroup < 0 && !noPacked && b->dSdcPacked != nullptr;
 	for(int g : plan.list) packed &= b->groups[g].d.nColG == 1 && b->groups[g].d.nVals <= 64;
 	if(packed) {
@@ -421,7 +422,6 @@ int launch_lmm_sdc_tiles(cla_block* b, const double* dY, int p, double* dPre, in
 	// bins of a slab of groups next to the Y tile; small slabs keep LDS per block low
 	// enough for three blocks per CU, which hides the latency of the list walks
 	size_t binBudget = 18 * 1024;
-	if(const char* e = getenv("CLA_LMM_SDC_BIN_KB")) binBudget = (size_t) atoi(e) * 1024;
 	binBudget = std::min(binBudget, ldsMax - (size_t) ST * 8);
 	for(size_t l = 0; l < plan.list.size(); l++)
 		binBudget = std::max(binBudget, (size_t) (plan.binOff[l + 1] - plan.binOff[l]) * 8);
@@ -471,13 +471,9 @@ int launch_rmm_sdc_tiles(cla_block* b, int q, int constRow, int accumulate, doub
 	// Tables are read from global memory (they stay in L2): without table slabs in LDS the
 	// waves of a block never meet at a barrier between the list walks, and only the output
 	// tile takes LDS (C4: 1.95 ms with one 100 KB slab in LDS, 0.72 ms with 8 KB slabs,
-	// 0.58 ms with none). CLA_RMM_SDC_TBL_KB > 0 brings the slabs back.
+	// 0.58 ms with none).
 	size_t tblBudget = 8 * 1024;
-	bool ldsTables = false;
-	if(const char* e = getenv("CLA_RMM_SDC_TBL_KB")) {
-		tblBudget = (size_t) std::max(1, atoi(e)) * 1024;
-		ldsTables = atoi(e) > 0;
-	}
+	const bool ldsTables = false;
 	tblBudget = std::max(tblBudget, maxVals * q * 8);
 	tblBudget = std::min(tblBudget, ldsMax - (size_t) tileRows * q * 8);
 	// groups per slab: uniform count so that every slab's tables fit
@@ -494,7 +490,7 @@ int launch_rmm_sdc_tiles(cla_block* b, int q, int constRow, int accumulate, doub
 		const DGroup& G = b->groups[g].d;
 		algo += (double) G.nDeltas * G.deltaWidth + (double) G.nOffsets * G.codeWidth;
 	}
-	static const bool noPacked = getenv("CLA_SDC_NO_PACKED") != nullptr;
+	const bool noPacked = !b->opt.sdcPacked;
 	if(q == 1 && !ldsTables && tileRows == ST && !noPacked && b->dSdcPacked != nullptr) {
 		const size_t ldsP = (size_t) ST * 8;
 		Prof pf(b, "k_rmm_sdc_packed", nTiles, ST_THREADS, (long) ldsP, algo);

@@ -455,7 +455,7 @@ int launch_tsmm(cla_block* b, double* dOut, unsigned long long* dNnz) {
 	// Decoded Gram matrix on the matrix cores (one pass over all groups) against one pass per
 	// pair of groups: the first costs about as much per 16 x 16 tile of the result and row as
 	// the second per eight pairs and row.
-	const bool forceDecode = getenv("CLA_TSMM_DECODE") != nullptr, forcePairs = getenv("CLA_TSMM_PAIRS") != nullptr; // per call: tests switch them
+	const bool forceDecode = b->opt.tsmmRoute == 2, forcePairs = b->opt.tsmmRoute == 1;
 	const int nb = (nCols + 15) / 16;
 	// a joint block (cbind of two blocks, only the cross product wanted) pairs left groups with right groups only
 	const int split = b->crossSplit;
@@ -476,8 +476,8 @@ int launch_tsmm(cla_block* b, double* dOut, unsigned long long* dNnz) {
 	const bool mustDecode = b->hasUnc || forceDecode || (!pairsFit && nCols <= 64);
 	// As many groups as columns: the reference decompresses (CLALibTSMM.java:73-77); here that is the decoded
 	// Gram matrix up to 64 columns. Wider blocks without uncompressed groups go per pair (the scalar
-	// decompressing fallback is slower and ends at 110 columns) unless CLA_TSMM_WIDE_DENSE asks for it.
-	const bool wideDense = nCols > 64 && nG >= nCols && (!pairsFit || getenv("CLA_TSMM_WIDE_DENSE") != nullptr);
+	// decompressing fallback is slower and ends at 110 columns) unless the option tsmm_wide_dense asks for it.
+	const bool wideDense = nCols > 64 && nG >= nCols && (!pairsFit || b->opt.tsmmWideDense);
 	const bool dense = split > 0 ? mustDecode || (nCols <= 64 && (nG >= nCols || gramCheaper) && !forcePairs)
 	                             : mustDecode || wideDense || (nCols <= 64 && (nG >= nCols || gramCheaper) && !forcePairs);
 	// More than 64 columns: the decoded Gram matrices of pairs of 32-column chunks (about 1.4 ms per pair of
@@ -486,7 +486,7 @@ int launch_tsmm(cla_block* b, double* dOut, unsigned long long* dNnz) {
 	const int64_t mAll = (nCols + 31) / 32, mLeft = split > 0 ? std::max<int64_t>(1, mAll / 2) : 0;
 	const int64_t nJoints = split > 0 ? mLeft * std::max<int64_t>(1, mAll - mLeft) : mAll * (mAll - 1) / 2;
 	const bool chunkCheaper = !forcePairs && pairsFit && nPairs >= 100 * nJoints;
-	if((dense || chunkCheaper) && nCols > 64 && nRows > 0 && !getenv("CLA_TSMM_NO_CHUNKS")) {
+	if((dense || chunkCheaper) && nCols > 64 && nRows > 0 && b->opt.tsmmChunks) {
 		// decoded Gram matrices of pairs of column chunks
 		rc = launch_tsmm_chunked(b, dOut);
 		if(rc < 0) return rc;
@@ -507,7 +507,7 @@ int launch_tsmm(cla_block* b, double* dOut, unsigned long long* dNnz) {
 	}
 	if(dense) {
 		// t(D) %*% D of the decoded rows, constants included (no correction layer needed)
-		static const bool noMfma = getenv("CLA_TSMM_NO_MFMA") != nullptr;
+		const bool noMfma = !b->opt.tsmmMfma;
 		rc = (noMfma || nRows == 0) ? 1 : launch_tsmm_decode(b, dOut);
 		if(rc < 0) return rc;
 		if(rc == 0) {
@@ -566,7 +566,7 @@ int launch_tsmm(cla_block* b, double* dOut, unsigned long long* dNnz) {
 			const DGroup& B = b->groups[h].d;
 			const size_t bothDicts = ((size_t) A.nVals * A.nColG + (size_t) B.nVals * B.nColG + 2) * 8;
 			if(A.type == G_DDC && B.type == G_DDC && A.codeWidth == B.codeWidth && A.codeWidth <= 2 && A.nColG <= 2 && B.nColG <= 2 &&
-				bothDicts <= (size_t) 150 * 1024 && !getenv("CLA_TSMM_PREAGG")) {
+				bothDicts <= (size_t) 150 * 1024 && b->opt.tsmmPairDot) {
 				size_t k = 0;
 				while(k < dots.size() && !(dots[k].cw == A.codeWidth && dots[k].nct == A.nColG && dots[k].ncs == B.nColG)) k++;
 				if(k == dots.size()) dots.push_back(DotShape{A.codeWidth, A.nColG, B.nColG, {}});

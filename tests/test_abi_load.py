@@ -39,3 +39,17 @@ def test_product_fails_loudly_without_gpu_or_init():
     assert lib.cla_init(0) < 0
     assert b"GPU only" in lib.cla_last_error()
     assert not lib.cla_block_create(10, 2)
+
+
+def test_no_exception_crosses_the_boundary():
+    """Host code below the entry points may throw (std::bad_alloc from a vector, std::length_error from an
+    absurd size): every entry point turns that into a negative code and a message. Needs no device."""
+    from systemds_amd import capi
+    lib = capi.load_library()
+    assert lib.cla_selftest_exception(0) == capi.ERR_DEVICE
+    assert b"allocation" in lib.cla_last_error()
+    assert lib.cla_selftest_exception(1) == capi.ERR_INVALID
+    assert b"selftest" in lib.cla_last_error()
+    assert lib.cla_selftest_exception(2) == capi.ERR_INVALID
+    assert lib.cla_selftest_exception(3) == capi.ERR_INVALID
+    assert lib.cla_selftest_exception(99) == 0

@@ -103,3 +103,18 @@ def test_host_layer_driver(H, ora, cla):
     assert_fp64_close(a.toArray().reshape(-1), ref, scale, what="sumSq")
     with pytest.raises(H.NotImplementedException):
         agg(cmb, H.AggOp.MIN, H.AggDir.ReduceCol, 4)
+
+
+@pytest.mark.parametrize("direction", ["all", "col"])
+def test_sum_of_squares_of_a_dense_column_under_a_constant(cla, ora, direction):
+    """A const group on the columns of an uncompressed group (an overlapping block as the overlapping right
+    multiply returns it): sum((v + c)^2) needs the cross term 2 c sum(v), not sum(v^2) + n c^2."""
+    from systemds_amd import synth
+    rng = np.random.default_rng(12)
+    n_rows = 30000
+    specs = [synth.GroupSpec("unc", np.array([0, 1], np.int32), dense=rng.standard_normal((n_rows, 2)) + 0.5),
+             synth.GroupSpec("const", np.array([1, 2], np.int32), np.array([[3.0, -2.0]])),
+             synth.GroupSpec("ddc", np.array([3], np.int32), rng.standard_normal((9, 1)), rng.integers(0, 9, n_rows).astype(np.uint8))]
+    D = ora.np_decompress(specs, n_rows, 4)
+    check(cla, specs, D, n_rows, 4, "sumsq", direction, "dense + const")
+    check(cla, specs, D, n_rows, 4, "sum", direction, "dense + const")

@@ -10,9 +10,9 @@ from parity import assert_fp64_close, assert_matches_truth
 pytestmark = pytest.mark.gpu
 
 
-def check(cla, ora, specsL, nL, specsR, nR, n_rows, what, keep=False):
+def check(cla, ora, specsL, nL, specsR, nR, n_rows, what, keep=False, route=0):
     left = cla.build_block(n_rows, nL, specsL)
-    right = cla.build_block(n_rows, nR, specsR)
+    right = cla.build_block(n_rows, nR, specsR).set_option("tsmm_route", route)
     out, nnz = right.lmm_compressed(left)
     ref, rnnz = ora.lmm_compressed(ora.Groups(specsR, n_rows, nR), ora.Groups(specsL, n_rows, nL))
     DL = ora.np_decompress(specsL, n_rows, nL)
@@ -27,19 +27,17 @@ def check(cla, ora, specsL, nL, specsR, nR, n_rows, what, keep=False):
     right.close()
 
 
-@pytest.mark.parametrize("path", [None, "CLA_TSMM_PAIRS", "CLA_TSMM_DECODE"])
+@pytest.mark.parametrize("path", [0, 1, 2], ids=["auto", "pairs", "decode"])
 @pytest.mark.parametrize("seed,n_rows", [(0, 1), (1, 37), (2, 3000), (4, 150001)])
-def test_mixed_groups(cla, ora, monkeypatch, path, seed, n_rows):
+def test_mixed_groups(cla, ora, path, seed, n_rows):
     """Every pairing of DDC / SDC / SDCZeros / RLE / const / empty groups, on the per-pair path and on the
-    decoded path (the library picks by cost; the switches force one)."""
-    if path:
-        monkeypatch.setenv(path, "1")
+    decoded path (the library picks by cost; the option tsmm_route of the right block forces one)."""
     specsL, nL = mixed_block(seed, n_rows, with_unc=False)
     # two 70000-tuple dictionaries cannot meet on the per-pair path (the accumulator of either side exceeds LDS):
     # the library then decodes; the forced per-pair run keeps one of them small
     specsR, nR = mixed_block(seed + 50, n_rows, with_unc=False, with_const=seed % 2 == 0,
-                             big_dict=path != "CLA_TSMM_PAIRS")
-    check(cla, ora, specsL, nL, specsR, nR, n_rows, f"t(L) %*% R {path}")
+                             big_dict=path != 1)
+    check(cla, ora, specsL, nL, specsR, nR, n_rows, f"t(L) %*% R route {path}", route=path)
 
 
 @pytest.mark.parametrize("unc_l,unc_r", [(True, False), (False, True), (True, True)])

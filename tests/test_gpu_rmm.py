@@ -165,3 +165,128 @@ def test_wide_right_multiply_on_uneven_ddc_blocks(cla, ora, seed):
     assert_matches_truth(out, D, B, what=f"uneven DDC block {seed}")
     assert_fp64_close(out, ref, abs_scale(ora, specs, n_rows, c, B), what=f"uneven DDC block {seed}", n_terms=c)
     assert nnz == rnnz
+
+
+def _u8_block(rng, n_rows, n_cols, n_vals=200, zero_cells=False):
+    from systemds_amd import synth
+    specs = []
+    for c in range(n_cols):
+        d = rng.standard_normal((n_vals, 1))
+        if zero_cells:
+            d[rng.integers(0, n_vals, 5)] = 0.0
+        specs.append(synth.GroupSpec("ddc", np.array([c], np.int32), d, rng.integers(0, n_vals, n_rows).astype(np.uint8)))
+    return specs
+
+
+@pytest.mark.parametrize("n_rows,n_cols", [(1, 3), (2047, 20), (70001, 37), (300000, 100)])
+@pytest.mark.parametrize("with_const", [False, True])
+def test_matvec_fused_tables_equal_preaggregated_tables(cla, ora, n_rows, n_cols, with_const):
+    """Byte-code blocks with one column per group: the gather kernel that makes its tables on the way into
+    LDS (the default) against the one that reads tables pre-aggregated by a kernel of their own
+    (rmm_disable bit 1) and against the oracle, bit for bit; non-zero counts through the rotating counters
+    over several calls."""
+    from systemds_amd import synth
+    rng = np.random.default_rng(n_rows + n_cols)
+    specs = _u8_block(rng, n_rows, n_cols, zero_cells=True)
+    nc = n_cols
+    if with_const:
+        specs.append(synth.GroupSpec("const", np.array([nc], np.int32), np.array([[0.75]])))
+        nc += 1
+    blk = cla.build_block(n_rows, nc, specs)
+    G = ora.Groups(specs, n_rows, nc)
+    for rep in range(5):
+        v = rng.standard_normal((nc, 1))
+        if rep == 3:
+            v[:] = 0.0  # every result cell is the constants' term (or zero): the count must follow
+        ref, rnnz = ora.rmm(G, v, 4)
+        out, nnz = blk.rmm(v)
+        assert np.array_equal(out, ref) and nnz == rnnz
+        blk.set_option("rmm_disable", 2)
+        out2, nnz2 = blk.rmm(v)
+        blk.set_option("rmm_disable", 0)
+        assert np.array_equal(out2, ref) and nnz2 == rnnz
+    blk.close()
+
+
+def test_matvec_fused_tables_non_finite_vector(cla, ora):
+    """Dictionary.preaggValuesFromDense skips zero dictionary cells (Dictionary.java:893-908), so an infinite
+    entry of v must not turn a zero cell into NaN; infinite and NaN entries meet non-zero cells as usual."""
+    rng = np.random.default_rng(5)
+    n_rows, n_cols = 50000, 24
+    specs = _u8_block(rng, n_rows, n_cols, zero_cells=True)
+    blk = cla.build_block(n_rows, n_cols, specs)
+    G = ora.Groups(specs, n_rows, n_cols)
+    v = rng.standard_normal((n_cols, 1))
+    v[3] = np.inf
+    v[7] = -np.inf
+    ref, rnnz = ora.rmm(G, v, 4)
+    out, nnz = blk.rmm(v)
+    assert np.array_equal(out, ref, equal_nan=True) and nnz == rnnz
+    assert np.isfinite(out).any() and not np.isfinite(out).all()
+    v[11] = np.nan
+    ref, rnnz = ora.rmm(G, v, 4)
+    out, nnz = blk.rmm(v)
+    assert np.array_equal(out, ref, equal_nan=True) and nnz == rnnz
+    blk.close()
+
+
+def test_async_calls_leave_the_count_on_the_device(cla, ora):
+    """cla_*_dev_async queue the kernels and return; cla_block_nnz reads the count of the last call."""
+    from devmem import DevBuf
+    from systemds_amd import synth
+    c = synth.config2(scale=200)
+    n, m = c["n_rows"], c["n_cols"]
+    blk = cla.build_block(n, m, c["groups"])
+    G = ora.Groups(c["groups"], n, m)
+    dv = DevBuf.from_numpy(c["v"])
+    dz = DevBuf.from_numpy(np.zeros_like(c["v"]))
+    dout = DevBuf(n * 8)
+    ref, rnnz = ora.rmm(G, c["v"], 4)
+    for _ in range(7):  # more calls than counters in the rotation
+        assert blk.rmm_dev_async(dv.ptr, 1, dout.ptr) == 0
+    assert blk.nnz() == rnnz
+    assert np.array_equal(dout.to_numpy(n), ref[:, 0])
+    assert blk.rmm_dev_async(dz.ptr, 1, dout.ptr) == 0
+    assert blk.nnz() == 0
+    assert blk.rmm_dev(dv.ptr, 1, dout.ptr) == rnnz
+    # the other drivers: same results as their synchronous forms
+    dB = DevBuf.from_numpy(c["B"])
+    doB = DevBuf(n * 64 * 8)
+    want = blk.rmm_dev(dB.ptr, 64, doB.ptr)
+    keep = doB.to_numpy((n, 64))
+    doB.zero()
+    assert blk.rmm_dev_async(dB.ptr, 64, doB.ptr) == 0 and blk.nnz() == want
+    assert np.array_equal(keep, doB.to_numpy((n, 64)))
+    dy = DevBuf.from_numpy(np.random.default_rng(1).standard_normal((1, n)))
+    do1 = DevBuf(m * 8)
+    want = blk.lmm_dev(dy.ptr, 1, do1.ptr)
+    keep = do1.to_numpy(m)
+    assert blk.lmm_dev_async(dy.ptr, 1, do1.ptr) == 0 and blk.nnz() == want
+    np.testing.assert_allclose(do1.to_numpy(m), keep, rtol=1e-12)
+    do2 = DevBuf(m * 8)
+    want = blk.mmchain_dev(dv.ptr, None, 0, do2.ptr)
+    assert blk.mmchain_dev_async(dv.ptr, None, 0, do2.ptr) == 0 and blk.nnz() == want
+    blk.close()
+    c3 = synth.config3(scale=500)
+    blk = cla.build_block(c3["n_rows"], c3["n_cols"], c3["groups"])
+    do3 = DevBuf(c3["n_cols"] ** 2 * 8)
+    want = blk.tsmm_dev(do3.ptr)
+    assert blk.tsmm_dev_async(do3.ptr) == 0 and blk.nnz() == want
+    blk.close()
+
+
+def test_options_and_failed_finalize(cla):
+    blk = cla.ClaBlock(100, 2)
+    with pytest.raises(cla.ClaError, match="unknown option"):
+        blk.set_option("no_such_switch", 1)
+    with pytest.raises(cla.ClaError, match="takes 0..2"):
+        blk.set_option("tsmm_route", 3)
+    # a failed finalize leaves the block unusable: every further add or finalize is refused
+    blk.add_ddc([0], np.zeros((2, 1)), np.full(100, 5, np.uint8))
+    with pytest.raises(cla.ClaError, match="code >="):
+        blk.finalize()
+    with pytest.raises(cla.ClaError, match="earlier cla_block_finalize"):
+        blk.finalize()
+    with pytest.raises(cla.ClaError, match="earlier cla_block_finalize"):
+        blk.add_const([1], np.ones((1, 1)))
+    blk.close()

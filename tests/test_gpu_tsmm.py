@@ -9,8 +9,14 @@ from parity import assert_fp64_close, assert_matches_truth
 pytestmark = pytest.mark.gpu
 
 
-def check_tsmm(cla, ora, specs, n_rows, n_cols, what):
+# option values of cla_block_set_option that force one of the interchangeable t(X) %*% X forms
+PAIRS, DECODE, NO_CHUNKS = {"tsmm_route": 1}, {"tsmm_route": 2}, {"tsmm_chunks": 0}
+
+
+def check_tsmm(cla, ora, specs, n_rows, n_cols, what, options=None):
     blk = cla.build_block(n_rows, n_cols, specs)
+    for key, value in (options or {}).items():
+        blk.set_option(key, value)
     out, nnz = blk.tsmm()
     blk.close()
     ref, rnnz = ora.tsmm(ora.Groups(specs, n_rows, n_cols), 4)
@@ -29,40 +35,36 @@ def test_mixed_groups_tsmm(cla, ora, seed, n_rows, with_unc):
     check_tsmm(cla, ora, specs, n_rows, n_cols, f"tsmm unc={with_unc}")
 
 
-@pytest.mark.parametrize("path", ["CLA_TSMM_PAIRS", "CLA_TSMM_DECODE"])
+@pytest.mark.parametrize("path", [PAIRS, DECODE], ids=["pairs", "decode"])
 @pytest.mark.parametrize("seed,n_rows", [(1, 37), (2, 3000), (4, 150001)])
-def test_mixed_groups_tsmm_both_paths(cla, ora, monkeypatch, path, seed, n_rows):
+def test_mixed_groups_tsmm_both_paths(cla, ora, path, seed, n_rows):
     """The per-pair path and the decoded Gram matrix on the matrix cores are interchangeable:
-    the library picks by cost, the switches (read per call) force one."""
-    monkeypatch.setenv(path, "1")
+    the library picks by cost, the block option tsmm_route forces one."""
     specs, n_cols = mixed_block(seed, n_rows, with_unc=False)
-    check_tsmm(cla, ora, specs, n_rows, n_cols, f"tsmm {path}")
+    check_tsmm(cla, ora, specs, n_rows, n_cols, f"tsmm {path}", path)
 
 
-@pytest.mark.parametrize("path", [None, "CLA_TSMM_PAIRS", "CLA_TSMM_DECODE"])
-def test_c3_scaled(cla, ora, monkeypatch, path):
+@pytest.mark.parametrize("path", [None, PAIRS, DECODE], ids=["auto", "pairs", "decode"])
+def test_c3_scaled(cla, ora, path):
     """BASELINE config 3 at 1/100 scale: 25 co-coded pairs, 4096 tuples, uint16 codes. The
     dictionaries do not fit LDS together: the decoded path looks them up in global memory. The
     row count is no multiple of the tile, so the last tile is ragged."""
     from systemds_amd import synth
-    if path:
-        monkeypatch.setenv(path, "1")
     c = synth.config3(scale=100)
-    check_tsmm(cla, ora, c["groups"], c["n_rows"], c["n_cols"], f"C3 {path}")
+    check_tsmm(cla, ora, c["groups"], c["n_rows"], c["n_cols"], f"C3 {path}", path)
 
 
 @pytest.mark.parametrize("expand", [True, False])
-def test_c5_scaled(cla, ora, monkeypatch, expand):
+def test_c5_scaled(cla, ora, expand):
     """BASELINE config 5 at 1/500 scale (mixed RLE + DDC + SDC + dense): both products, with the RLE / SDC
     groups' codes expanded to byte streams for the decode kernels (the default when that is cheap) and with the
     per-tile run and offset-list decoding."""
     from systemds_amd import synth
-    if not expand:
-        monkeypatch.setenv("CLA_DEC_NO_EXPAND", "1")
+    opts = {"expand_streams": 1 if expand else 0}
     c = synth.config5(scale=500)
     n_rows, n_cols = c["n_rows"], c["n_cols"]
-    check_tsmm(cla, ora, c["groups"], n_rows, n_cols, "C5 tsmm")
-    blk = cla.build_block(n_rows, n_cols, c["groups"])
+    check_tsmm(cla, ora, c["groups"], n_rows, n_cols, "C5 tsmm", opts)
+    blk = cla.build_block(n_rows, n_cols, c["groups"]).set_option("expand_streams", opts["expand_streams"])
     out, nnz = blk.rmm(c["B"])
     blk.close()
     ref, rnnz = ora.rmm(ora.Groups(c["groups"], n_rows, n_cols), c["B"], 4)
@@ -81,17 +83,15 @@ def test_single_column_groups_use_dense_path(cla, ora):
     check_tsmm(cla, ora, c["groups"], c["n_rows"], c["n_cols"], "C2-like")
 
 
-@pytest.mark.parametrize("path", [None, "CLA_TSMM_PAIRS", "CLA_TSMM_NO_CHUNKS"])
-def test_wide_blocks_of_single_column_groups(cla, ora, monkeypatch, path):
+@pytest.mark.parametrize("path", [None, PAIRS, NO_CHUNKS], ids=["auto", "pairs", "no_chunks"])
+def test_wide_blocks_of_single_column_groups(cla, ora, path):
     """More than 64 columns, as many groups as columns: the decoded Gram matrices of pairs of 32-column chunks
     (the default with that many pairs of groups), or one pass per pair of groups (forced, or chunks switched off)."""
     from systemds_amd import synth
-    if path:
-        monkeypatch.setenv(path, "1")
     c = synth.config2(scale=500, n_cols=100)
-    check_tsmm(cla, ora, c["groups"], c["n_rows"], c["n_cols"], f"C2 100 columns {path}")
+    check_tsmm(cla, ora, c["groups"], c["n_rows"], c["n_cols"], f"C2 100 columns {path}", path)
     c = synth.config4(scale=500, n_cols=130)
-    check_tsmm(cla, ora, c["groups"], c["n_rows"], c["n_cols"], f"C4-like 130 columns {path}")
+    check_tsmm(cla, ora, c["groups"], c["n_rows"], c["n_cols"], f"C4-like 130 columns {path}", path)
 
 
 def wide_mixed_block(seed, n_rows, extra_cols=70):
