@@ -32,10 +32,14 @@ __global__ __launch_bounds__(LU_THREADS) void k_lmm_u8(const DGroup* __restrict_
 	const double* y = Y + (size_t) blockIdx.y * nRows;
 	double* dst = pre + (size_t) blockIdx.y * totalVals;
 
-	const int64_t share = ((nRows + gridDim.x - 1) / gridDim.x + RPT - 1) / RPT * RPT;
-	const int64_t blockBeg = (int64_t) blockIdx.x * share;
-	if(blockBeg >= nRows) return;
-	const int blockLen = (int) (min(nRows, blockBeg + share) - blockBeg);
+	// shares of whole units of 64 * RPT rows that differ by at most one unit between blocks (see k_rmm_q1_u8)
+	constexpr int UNIT = 64 * RPT;
+	const int64_t nUnits = (nRows + UNIT - 1) / UNIT;
+	const int64_t unitsLo = nUnits / gridDim.x, unitsRem = nUnits % gridDim.x;
+	const int64_t myUnits = unitsLo + ((int64_t) blockIdx.x < unitsRem ? 1 : 0);
+	const int64_t blockBeg = ((int64_t) blockIdx.x * unitsLo + min((int64_t) blockIdx.x, unitsRem)) * UNIT;
+	if(myUnits == 0 || blockBeg >= nRows) return;
+	const int blockLen = (int) (min(nRows, blockBeg + myUnits * UNIT) - blockBeg);
 	const int nPass = (blockLen + THREADS * RPT - 1) / (THREADS * RPT);
 	const int passRows = ((blockLen + nPass - 1) / nPass + 64 * RPT - 1) / (64 * RPT) * (64 * RPT);
 	auto pass_len = [&](int pass) { return pass < nPass ? min(passRows, blockLen - pass * passRows) : 0; };
@@ -193,10 +197,14 @@ __global__ __launch_bounds__(LD_THREADS, 4) void k_lmm_u8_dot(const uint8_t* __r
 	const int nPad = (nGroups + PER - 1) / PER * PER;
 	const double* y = Y + (size_t) blockIdx.y * nRows;
 
-	const int64_t share = ((nRows + gridDim.x - 1) / gridDim.x + RPT - 1) / RPT * RPT;
-	const int64_t blockBeg = (int64_t) blockIdx.x * share;
-	if(blockBeg >= nRows) return;
-	const int blockLen = (int) (min(nRows, blockBeg + share) - blockBeg);
+	// shares of whole units of 64 * RPT rows that differ by at most one unit between blocks (see k_rmm_q1_u8)
+	constexpr int UNIT = 64 * RPT;
+	const int64_t nUnits = (nRows + UNIT - 1) / UNIT;
+	const int64_t unitsLo = nUnits / gridDim.x, unitsRem = nUnits % gridDim.x;
+	const int64_t myUnits = unitsLo + ((int64_t) blockIdx.x < unitsRem ? 1 : 0);
+	const int64_t blockBeg = ((int64_t) blockIdx.x * unitsLo + min((int64_t) blockIdx.x, unitsRem)) * UNIT;
+	if(myUnits == 0 || blockBeg >= nRows) return;
+	const int blockLen = (int) (min(nRows, blockBeg + myUnits * UNIT) - blockBeg);
 	const int nPass = (blockLen + THREADS * RPT - 1) / (THREADS * RPT);
 	const int passRows = ((blockLen + nPass - 1) / nPass + 64 * RPT - 1) / (64 * RPT) * (64 * RPT);
 

@@ -262,14 +262,20 @@ __global__ __launch_bounds__(THREADS, 4) void k_rmm_q1_u8(const uint8_t* __restr
 	const int gLast = nGroups - 1;
 	const int nPad = (nGroups + U8_PER - 1) / U8_PER * U8_PER; // groups incl. the zero-table slots of the last slab
 
-	// The block is persistent: it owns an equal share of the rows (a multiple of 16) and covers
-	// it in nPass passes of at most THREADS * RPT rows, the same for every block, so all blocks finish
-	// together and the load pipeline (codes two batches ahead, tables one slab ahead) keeps
-	// running from pass to pass. Everything about a pass but `off` is uniform.
-	const int64_t share = ((nRows + gridDim.x - 1) / gridDim.x + RPT - 1) / RPT * RPT;
-	const int64_t blockBeg = (int64_t) blockIdx.x * share;
-	if(blockBeg >= nRows) return;
-	const int blockLen = (int) (min(nRows, blockBeg + share) - blockBeg);
+	// The block is persistent: it owns a share of the rows and covers it in nPass passes of at most
+	// THREADS * RPT rows, so all blocks finish together and the load pipeline (codes two batches
+	// ahead, tables one slab ahead) keeps running from pass to pass. Shares are whole units of
+	// 64 * RPT rows (the rows of one wave in one pass) and differ by at most one unit between
+	// blocks: a share that ends inside a unit leaves a wave with a few live lanes that costs as
+	// much as a full one (measured on 10M rows: 0.2233 ms with equal shares of 19536 rows,
+	// 0.2157 ms with shares of whole units). Everything about a pass but `off` is uniform.
+	constexpr int UNIT = 64 * RPT;
+	const int64_t nUnits = (nRows + UNIT - 1) / UNIT;
+	const int64_t unitsLo = nUnits / gridDim.x, unitsRem = nUnits % gridDim.x;
+	const int64_t myUnits = unitsLo + ((int64_t) blockIdx.x < unitsRem ? 1 : 0);
+	const int64_t blockBeg = ((int64_t) blockIdx.x * unitsLo + min((int64_t) blockIdx.x, unitsRem)) * UNIT;
+	if(myUnits == 0 || blockBeg >= nRows) return;
+	const int blockLen = (int) (min(nRows, blockBeg + myUnits * UNIT) - blockBeg);
 	const int nPass = (blockLen + THREADS * RPT - 1) / (THREADS * RPT);
 	// whole waves per pass (64 threads x RPT rows), so that only a block's last pass can hold a
 	// partly filled wave, which has to store its rows untransposed
