@@ -134,6 +134,16 @@ int64_t cla_rmm_dev(cla_handle h, const double* dB, int32_t nColB, double* dOut)
 /* The same without the wait: returns 0 once the kernels are queued on the block's stream (or a negative
  * error); the non-zero count stays in a device counter until cla_block_nnz asks for it. */
 int cla_rmm_dev_async(cla_handle h, const double* dB, int32_t nColB, double* dOut);
+/* cla_rmm_dev for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc). It has no counterpart in the reference. The pre-aggregated tables
+ * dict_g x B and the non-zero counter live in a static device array of 4 MiB that the library holds per GPU
+ * until the process ends; the call makes no hipMalloc / hipFree and builds no derived format, so it always
+ * takes the table-reading kernels (never the matrix-core or decode kernels). -CLA_ERR_UNSUPPORTED when the
+ * tables ((sum of dictionary sizes + 1) x nColB doubles, plus 256 per group for byte-code mat-vecs) exceed
+ * the array, or when the block holds SDC groups with entries (their row-tile plan is an allocation). All calls
+ * on one GPU share the array: calls that overlap in time on one GPU (two blocks, two threads) race. The
+ * count returned by cla_block_nnz is not updated by this entry point. */
+int64_t cla_rmm_dev_noalloc(cla_handle h, const double* dB, int32_t nColB, double* dOut);
 /* nnz of the result of the last driver call on this block (MatrixBlock.recomputeNonZeros of the reference
  * drivers, C/lib/CLALibRightMultBy.java:98); waits for the block's stream. */
 int64_t cla_block_nnz(cla_handle h);

@@ -52,6 +52,7 @@ SIGNATURES = {
     "cla_rmm": (C.c_int64, [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
     "cla_rmm_dev": (C.c_int64, [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
     "cla_rmm_dev_async": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
+    "cla_rmm_dev_noalloc": (C.c_int64, [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
     "cla_block_nnz": (C.c_int64, [C.c_void_p]),
     "cla_lmm": (C.c_int64, [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
     "cla_lmm_dev": (C.c_int64, [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
@@ -328,6 +329,10 @@ class ClaBlock:
 
     def rmm_dev_async(self, dB_ptr, n_col_b, dOut_ptr):
         return _check(self.lib.cla_rmm_dev_async(self.h, C.c_void_p(dB_ptr), int(n_col_b), C.c_void_p(dOut_ptr)))
+
+    def rmm_dev_noalloc(self, dB_ptr, n_col_b, dOut_ptr):
+        """cla_rmm_dev_noalloc: X %*% B with the tables in the library's static workspace, no allocation."""
+        return _check(self.lib.cla_rmm_dev_noalloc(self.h, C.c_void_p(dB_ptr), int(n_col_b), C.c_void_p(dOut_ptr)))
 
     def nnz(self):
         """cla_block_nnz: non-zero count of the last driver call's result (waits for the block's stream)."""

@@ -22,7 +22,16 @@
 #define CLA_CATCH_NULL CLA_CATCH_BODY(return nullptr, return nullptr)
 #define CLA_CATCH_VOID CLA_CATCH_BODY(return, return)
 
+// Workspace of the entry point that allocates nothing (cla_rmm_dev_noalloc): the non-zero counter in the
+// first 256 bytes, then the pre-aggregated tables. One copy per GPU, held until the process ends. In host
+// code the name is only a handle for hipGetSymbolAddress: kernels get the address looked up at cla_init.
+constexpr size_t CLA_SCRATCH_BYTES = (size_t) 4 << 20;
+static __device__ __align__(256) unsigned char scratch[CLA_SCRATCH_BYTES];
+
 namespace cla {
+
+constexpr int MAX_DEVICES = 64;
+static unsigned char* g_scratchPtr[MAX_DEVICES] = {}; // device address of `scratch` per device (set at cla_init)
 
 static thread_local char t_err[1024] = "";
 int g_ldsPerBlock = 65536;
@@ -195,6 +204,12 @@ int cla_init(int device) {
 	g_ldsPerBlock = (int) g_prop.sharedMemPerBlock;
 	if(g_prop.maxSharedMemoryPerMultiProcessor > (size_t) g_ldsPerBlock)
 		g_ldsPerBlock = (int) g_prop.maxSharedMemoryPerMultiProcessor;
+	if(device < MAX_DEVICES && g_scratchPtr[device] == nullptr) {
+		// this device's copy of the static workspace (every GPU holds its own at its own address)
+		unsigned char* p = nullptr;
+		CLA_HIP(hipGetSymbolAddress((void**) &p, HIP_SYMBOL(scratch)));
+		g_scratchPtr[device] = p;
+	}
 	g_device = device;
 	return 0;
 	CLA_CATCH_CODE(int)
@@ -716,6 +731,28 @@ int cla_rmm_dev_async(cla_handle b, const double* dB, int32_t nColB, double* dOu
 	CLA_TRY
 	return (int) rmm_dev(b, dB, nColB, dOut, false);
 	CLA_CATCH_CODE(int)
+}
+
+int64_t cla_rmm_dev_noalloc(cla_handle b, const double* dB, int32_t nColB, double* dOut) {
+	CLA_TRY
+	int rc = check_final(b);
+	if(rc) return rc;
+	if(!dB || !dOut || nColB <= 0) { set_error("rmm: invalid right-hand side"); return -CLA_ERR_INVALID; }
+	unsigned char* ws = g_device < MAX_DEVICES ? g_scratchPtr[g_device] : nullptr;
+	if(!ws) { set_error("rmm without allocation: no static workspace on device %d", g_device); return -CLA_ERR_STATE; }
+	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	// the counter and the tables live in the static workspace (the pre-aggregation kernel clears the counter
+	// and rewrites every table entry that is read); event pairs of the profiling mode would be allocations
+	unsigned long long* dNnz = (unsigned long long*) ws;
+	const bool profile = b->profile;
+	b->profile = false;
+	rc = launch_rmm(b, dB, nColB, dOut, dNnz, 0, (double*) (ws + 256), (CLA_SCRATCH_BYTES - 256) / sizeof(double));
+	b->profile = profile;
+	if(rc) return rc;
+	CLA_HIP(hipMemcpyAsync(b->hCounters, dNnz, sizeof(unsigned long long), hipMemcpyDeviceToHost, b->stream));
+	CLA_HIP(hipStreamSynchronize(b->stream));
+	return (int64_t) b->hCounters[0];
+	CLA_CATCH_CODE(int64_t)
 }
 
 int64_t cla_block_nnz(cla_handle b) {

@@ -193,7 +193,8 @@ extern int g_numCU;
 int launch_validate_codes(cla_block* b, const void* codes, int width, int64_t n, int nVals, int* ok);
 int launch_counts(cla_block* b, int group, int32_t* dCounts);
 int launch_sdc_build(cla_block* b, HostGroup& g);
-int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned long long* dNnz, int squares = 0);
+int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned long long* dNnz, int squares = 0,
+	double* ws = nullptr, size_t wsDoubles = 0);
 int launch_tables(cla_block* b, const double* dB, int q); // dict x B of every group (+ constV x B) into b->dTables
 int launch_aggregate(cla_block* b, int op, int dir, double* dOut, unsigned long long* dNnz);
 int ensure_counts(cla_block* b);

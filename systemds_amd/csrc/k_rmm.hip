@@ -542,22 +542,38 @@ int launch_tables(cla_block* b, const double* dB, int q) {
 
 // squares != 0 (q == 1, no uncompressed group): the tables hold the sum of squares of each tuple
 // instead of dict x B, so that the gather yields rowSums(X^2).
-int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned long long* dNnz, int squares) {
+// ws != nullptr: a workspace of wsDoubles doubles that the caller owns takes the place of the block's table
+// buffer and nothing is allocated: kernels that need a derived format or a buffer of their own are left
+// out (the tables then always come from the pre-aggregation kernel), and a block that needs them is refused.
+int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned long long* dNnz, int squares, double* ws,
+	size_t wsDoubles) {
 	const int nG = (int) b->groups.size();
 	const int64_t nRows = b->nRows;
 	hipStream_t st = b->stream;
 	clear_stats(b);
+	const bool noAlloc = ws != nullptr;
 	// mat-vec on byte codes: all groups DDC in one arena, at most 256 values each
 	const bool u8Path = q == 1 && nRows > 0 && b->dArena && b->arenaWidth == 1 && b->maxVals <= 256 && !(b->opt.rmmDisable & 1);
 	const size_t nTbl = (size_t) (b->totalVals + 1) * q;
-	int rc = ensure_tables(b, nTbl + (u8Path ? (size_t) nG * 256 + 256 : 0));
-	if(rc) return rc;
-	double* dTpad = u8Path ? b->dTables + ((nTbl + 31) & ~(size_t) 31) : nullptr;
+	const size_t nTblPad = (nTbl + 31) & ~(size_t) 31;
+	const size_t need = u8Path ? nTblPad + (size_t) nG * 256 + 256 : nTbl;
+	if(noAlloc) {
+		if(need > wsDoubles) {
+			set_error("rmm without allocation: the pre-aggregated tables need %zu bytes, the static workspace holds %zu", need * 8, wsDoubles * 8);
+			return -CLA_ERR_UNSUPPORTED;
+		}
+	}
+	else {
+		const int rc = ensure_tables(b, need);
+		if(rc) return rc;
+	}
+	double* const tables = noAlloc ? ws : b->dTables;
+	double* dTpad = u8Path ? tables + nTblPad : nullptr;
 
 	// Byte-code mat-vec with one column per group: the gather kernel makes its tables itself from the
 	// padded dictionary image (built at finalize) and counts into a counter of its own that the call
 	// before has cleared, so it is the only launch (K1 only runs for the constants' term, if any).
-	const bool fused = u8Path && !squares && b->dDictPad != nullptr && !(b->opt.rmmDisable & 2);
+	const bool fused = u8Path && !squares && !noAlloc && b->dDictPad != nullptr && !(b->opt.rmmDisable & 2);
 	const int32_t* dCol0 = fused ? (const int32_t*) (b->dDictPad + (size_t) nG * 256) : nullptr;
 	if(fused) {
 		b->nnzSlot = b->nnzRot;
@@ -570,7 +586,7 @@ int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned lon
 		dim3 grid(fused ? 1 : ((maxWork + 255) / 256 > (q + 255) / 256 ? (maxWork + 255) / 256 : (q + 255) / 256), nK1 + 1);
 		Prof pf(b, "k_preagg", (long) grid.x * grid.y, 256, 0, 0);
 		hipLaunchKernelGGL(k_preagg, grid, dim3(256), 0, st, b->dGroups, nK1, dB, q, b->nCols,
-			b->hasConst ? b->dConstV : nullptr, b->dTables, b->totalVals, dNnz, fused ? nullptr : dTpad, squares);
+			b->hasConst ? b->dConstV : nullptr, tables, b->totalVals, dNnz, fused ? nullptr : dTpad, squares);
 	}
 	const int constRow = b->hasConst ? b->totalVals : -1;
 	if(nRows == 0) return 0;
@@ -585,7 +601,7 @@ int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned lon
 		// slab size: 16 or 20 groups, whichever leaves fewer padded table slots
 		const int pad16 = (nG + 15) / 16 * 16 - nG, pad20 = (nG + 19) / 20 * 20 - nG;
 		const int per = pad20 < pad16 ? 20 : 16;
-		const double* constTerm = constRow >= 0 ? b->dTables + constRow : nullptr;
+		const double* constTerm = constRow >= 0 ? tables + constRow : nullptr;
 		unsigned long long* nnzNext = fused ? b->dCounters + (b->nnzRot % 3 + 1) : nullptr;
 		Prof pf(b, "k_rmm_q1_u8", grid, THREADS, per * 256 * 8, bytes);
 #define U8_LAUNCH(PER, NBV, LB, LN, F)                                                                          \
@@ -612,7 +628,7 @@ int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned lon
 		auto kern = k_rmm_q1_ddc<CWV, RPTV, THR>;                                                               \
 		CLA_HIP(hipFuncSetAttribute((const void*) kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds)); \
 		hipLaunchKernelGGL(kern, dim3(grid), dim3(THR), lds, st, b->dArena, b->arenaStride, nG, b->dQ1Slabs,    \
-			nSlabs, b->dTblOff, b->dTables, constRow, dOut, nRows, dNnz);                                       \
+			nSlabs, b->dTblOff, tables, constRow, dOut, nRows, dNnz);                                       \
 	} while(0)
 #define LAUNCH_Q1_T(CWV, RPTV)                                                   \
 	do {                                                                         \
@@ -630,14 +646,14 @@ int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned lon
 	}
 
 	// wide B on an all-DDC block: fused decode + fp64 MFMA (K1 above still supplies constV x B)
-	if(q >= 8 && !(b->opt.rmmDisable & 4)) {
-		const int r = launch_rmm_mfma(b, dB, q, constRow >= 0 ? b->dTables + (size_t) constRow * q : nullptr, dOut, dNnz);
+	if(q >= 8 && !noAlloc && !(b->opt.rmmDisable & 4)) {
+		const int r = launch_rmm_mfma(b, dB, q, constRow >= 0 ? tables + (size_t) constRow * q : nullptr, dOut, dNnz);
 		if(r <= 0) return r;
 	}
 
 	// narrow B on any group mix: decode rows from LDS dictionaries, B rows as scalars
-	if(q >= 2 && q <= 16 && !(b->opt.rmmDisable & 8)) {
-		const int r = launch_rmm_decode(b, dB, q, constRow >= 0 ? b->dTables + (size_t) constRow * q : nullptr, dOut, dNnz);
+	if(q >= 2 && q <= 16 && !noAlloc && !(b->opt.rmmDisable & 8)) {
+		const int r = launch_rmm_decode(b, dB, q, constRow >= 0 ? tables + (size_t) constRow * q : nullptr, dOut, dNnz);
 		if(r <= 0) return r;
 	}
 
@@ -650,11 +666,15 @@ int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned lon
 			if(g.d.type == G_SDCZ) anySdc |= g.d.nOffsets > 0;
 			else anyRowGroup = true;
 		}
+		if(anySdc && noAlloc) {
+			set_error("rmm without allocation: SDC groups with entries need the row-tile plan, which this entry point cannot build");
+			return -CLA_ERR_UNSUPPORTED;
+		}
 		bool needNnzPass = true;
 		if(anyRowGroup || !anySdc) {
 			const dim3 grid((unsigned) ((nRows + 255) / 256), (unsigned) ((q + ROWS_QS - 1) / ROWS_QS));
 			Prof pf(b, "k_rmm_rows", (long) grid.x * grid.y, 256, 0, 0);
-			hipLaunchKernelGGL(k_rmm_rows, grid, dim3(256), 0, st, b->dGroups, nG, b->dTables, dB, q, constRow, dOut, nRows);
+			hipLaunchKernelGGL(k_rmm_rows, grid, dim3(256), 0, st, b->dGroups, nG, tables, dB, q, constRow, dOut, nRows);
 		}
 		if(anySdc) {
 			const int r = launch_rmm_sdc_tiles(b, q, constRow, anyRowGroup ? 1 : 0, dOut, dNnz);
@@ -665,7 +685,7 @@ int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned lon
 					// the scatter adds on top of an initialised output
 					const dim3 grid((unsigned) ((nRows + 255) / 256), (unsigned) ((q + ROWS_QS - 1) / ROWS_QS));
 					Prof pf(b, "k_rmm_rows", (long) grid.x * grid.y, 256, 0, 0);
-					hipLaunchKernelGGL(k_rmm_rows, grid, dim3(256), 0, st, b->dGroups, nG, b->dTables, dB, q, constRow, dOut,
+					hipLaunchKernelGGL(k_rmm_rows, grid, dim3(256), 0, st, b->dGroups, nG, tables, dB, q, constRow, dOut,
 						nRows);
 				}
 				for(int g = 0; g < nG; g++) {
@@ -674,9 +694,9 @@ int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned lon
 					const unsigned sg = (unsigned) (G.nCkpt > 1 ? G.nCkpt : 1);
 					Prof pf(b, "k_rmm_sdc_scatter", sg, 256, 0, 0);
 					if(G.deltaWidth == 1)
-						hipLaunchKernelGGL(k_rmm_sdc_scatter<1>, dim3(sg), dim3(256), 0, st, b->dGroups, g, b->dTables, q, dOut);
+						hipLaunchKernelGGL(k_rmm_sdc_scatter<1>, dim3(sg), dim3(256), 0, st, b->dGroups, g, tables, q, dOut);
 					else
-						hipLaunchKernelGGL(k_rmm_sdc_scatter<2>, dim3(sg), dim3(256), 0, st, b->dGroups, g, b->dTables, q, dOut);
+						hipLaunchKernelGGL(k_rmm_sdc_scatter<2>, dim3(sg), dim3(256), 0, st, b->dGroups, g, tables, q, dOut);
 				}
 			}
 		}
