@@ -131,6 +131,9 @@ struct SdcDesc {
 	const uint32_t* packed; // the group's entries as (code << 16 | row & 4095), in list order
 };
 
+// Tasks (list segments) whose loads a wave keeps in flight in the packed-list kernels.
+constexpr int SDC_P = 4;
+
 template <class T>
 __device__ __forceinline__ T bcast_lane(T v, int l) {
 	static_assert(sizeof(T) == 4 || sizeof(T) == 8, "readlane moves 32-bit pieces");
@@ -210,48 +213,86 @@ __global__ __launch_bounds__(ST_THREADS) void k_rmm_sdc_packed(const SdcDesc* __
 			D = desc[wave + (ST_THREADS / 64) * (t0 + lane)];
 			sdc_tile_range(D, r0, start, cnt);
 		}
-		u32x4 eA = {0, 0, 0, 0};
-		double tblA = 0.0;
-		int rowsC[4] = {0, 0, 0, 0};
-		double tvC[4] = {0.0, 0.0, 0.0, 0.0};
-		unsigned maskC = 0;
-		for(int t = 0; t < nHere + 2; t++) {
-			const u32x4 eB = eA;
-			const double tblB = tblA;
-			if(t < nHere) { // ---- stage A: task t
+		// Common case, every task of the batch a segment of at most 256 entries of a group with at most 64
+		// tuples: the loads (list segment, table entry `lane`) of SDC_P tasks are kept in flight. Every load
+		// of this loop is unconditional (tasks past the end repeat the last one with no entries, lanes past
+		// a table's end read its last entry): a load under a branch makes the compiler wait for all
+		// outstanding loads at the join, which is what limited the one-task-ahead form to a memory latency
+		// per task.
+		const bool simple = __builtin_amdgcn_ballot_w64(lane < nHere && (cnt > 256 || D.nVals > 64 || D.nVals < 1)) == 0;
+		if(simple) {
+			const int last = nHere - 1;
+			u32x4 eR[SDC_P];
+			double tblR[SDC_P];
+			auto issue = [&](int slot, int t) {
 				const uint32_t* pk = as_global(bcast_lane(D.packed, t)) + bcast_lane(start, t);
 				const int nv = bcast_lane(D.nVals, t);
-				eA = *(const u32x4*) (pk + lane * 4); // dword aligned; entries beyond the task's count are masked in stage B
-				tblA = nv <= 64 && lane < nv ? T[bcast_lane(D.tblOff, t) + lane] : 0.0;
-			}
-			if(t >= 2) { // ---- stage C: task t - 2
+				eR[slot] = *(const u32x4*) (pk + lane * 4); // (256 entries of slack behind the last list)
+				tblR[slot] = T[bcast_lane(D.tblOff, t) + min(lane, nv - 1)];
+			};
 #pragma unroll
-				for(int k = 0; k < 4; k++)
-					if(maskC & (1u << k)) unsafeAtomicAdd(&otile[rowsC[k]], tvC[k]);
-			}
-			maskC = 0;
-			if(t >= 1 && t - 1 < nHere) { // ---- stage B: task t - 1
-				const int tb = t - 1;
-				const int n = bcast_lane(cnt, tb);
-				const double* tg = T + bcast_lane(D.tblOff, tb);
-				const bool inRegs = bcast_lane(D.nVals, tb) <= 64;
+			for(int j = 0; j < SDC_P; j++) issue(j, min(j, last));
+			for(int t = 0; t < nHere; t += SDC_P) {
 #pragma unroll
-				for(int k = 0; k < 4; k++) {
-					const bool on = lane * 4 + k < n;
-					const int code = (int) (eB[k] >> 16);
-					const double tv = inRegs ? __shfl(tblB, code & 63, 64) : (on ? tg[code] : 0.0);
-					rowsC[k] = (int) (eB[k] & (ST - 1));
-					tvC[k] = tv;
-					if(on) maskC |= 1u << k;
-				}
-				if(n > 256) { // dense lists: the rest of the tile's entries, straight
-					const uint32_t* pk = as_global(bcast_lane(D.packed, tb)) + bcast_lane(start, tb);
-					for(int j = 256 + lane; j < n; j += 64) {
-						const uint32_t e = pk[j];
-						unsafeAtomicAdd(&otile[e & (ST - 1)], tg[e >> 16]);
+				for(int j = 0; j < SDC_P; j++) {
+					const int tb = t + j;
+					const u32x4 eB = eR[j];
+					const double tblB = tblR[j];
+					issue(j, min(tb + SDC_P, last));
+					const int n = tb < nHere ? bcast_lane(cnt, min(tb, last)) : 0;
+#pragma unroll
+					for(int k = 0; k < 4; k++) {
+						const double tv = __shfl(tblB, (int) (eB[k] >> 16) & 63, 64);
+						if(lane * 4 + k < n) unsafeAtomicAdd(&otile[eB[k] & (ST - 1)], tv);
 					}
 				}
 			}
+		}
+		else {
+			u32x4 eA = {0, 0, 0, 0};
+			double tblA = 0.0;
+			int rowsC[4] = {0, 0, 0, 0};
+			double tvC[4] = {0.0, 0.0, 0.0, 0.0};
+			unsigned maskC = 0;
+			for(int t = 0; t < nHere + 2; t++) {
+				const u32x4 eB = eA;
+				const double tblB = tblA;
+				if(t < nHere) { // ---- stage A: task t
+					const uint32_t* pk = as_global(bcast_lane(D.packed, t)) + bcast_lane(start, t);
+					const int nv = bcast_lane(D.nVals, t);
+					eA = *(const u32x4*) (pk + lane * 4); // dword aligned; entries beyond the task's count are masked in stage B
+					tblA = nv <= 64 && lane < nv ? T[bcast_lane(D.tblOff, t) + lane] : 0.0;
+				}
+				if(t >= 2) { // ---- stage C: task t - 2
+	#pragma unroll
+					for(int k = 0; k < 4; k++)
+						if(maskC & (1u << k)) unsafeAtomicAdd(&otile[rowsC[k]], tvC[k]);
+				}
+				maskC = 0;
+				if(t >= 1 && t - 1 < nHere) { // ---- stage B: task t - 1
+					const int tb = t - 1;
+					const int n = bcast_lane(cnt, tb);
+					const double* tg = T + bcast_lane(D.tblOff, tb);
+					const bool inRegs = bcast_lane(D.nVals, tb) <= 64;
+	#pragma unroll
+					for(int k = 0; k < 4; k++) {
+						const bool on = lane * 4 + k < n;
+						const int code = (int) (eB[k] >> 16);
+						const double tv = inRegs ? __shfl(tblB, code & 63, 64) : (on ? tg[code] : 0.0);
+						rowsC[k] = (int) (eB[k] & (ST - 1));
+						tvC[k] = tv;
+						if(on) maskC |= 1u << k;
+					}
+					if(n > 256) { // dense lists: the rest of the tile's entries, straight
+						const uint32_t* pk = as_global(bcast_lane(D.packed, tb)) + bcast_lane(start, tb);
+						for(int j = 256 + lane; j < n; j += 64) {
+							const uint32_t e = pk[j];
+							unsafeAtomicAdd(&otile[e & (ST - 1)], tg[e >> 16]);
+						}
+					}
+				}
+			}
+	
 		}
 	}
 	__syncthreads();
@@ -293,36 +334,72 @@ __global__ __launch_bounds__(ST_THREADS) void k_lmm_sdc_packed(const SdcDesc* __
 			__syncthreads();
 			int start = 0, cnt = 0;
 			if(lane < nHere) sdc_tile_range(D, r0, start, cnt);
-			u32x4 eA = {0, 0, 0, 0};
-			double dictA = 0.0;
-			for(int t = 0; t < nHere + 1; t++) {
-				const u32x4 eB = eA;
-				const double dictB = dictA;
-				if(t < nHere) { // ---- stage A: task t
+			// (see k_rmm_sdc_packed: unconditional loads, SDC_P tasks in flight)
+			const bool simple = nHere > 0 && __builtin_amdgcn_ballot_w64(lane < nHere && (cnt > 256 || D.nVals < 1)) == 0;
+			if(simple) {
+				const int last = nHere - 1;
+				u32x4 eR[SDC_P];
+				double dictR[SDC_P];
+				auto issue = [&](int slot, int t) {
 					const uint32_t* pk = as_global(bcast_lane(D.packed, t)) + bcast_lane(start, t);
-					eA = *(const u32x4*) (pk + lane * 4);
-					dictA = lane < bcast_lane(D.nVals, t) ? as_global(bcast_lane(D.dict, t))[lane] : 0.0;
-				}
-				if(t >= 1) { // ---- stage B: task t - 1
-					const int tb = t - 1;
-					const int n = bcast_lane(cnt, tb);
-					double part = 0.0;
+					eR[slot] = *(const u32x4*) (pk + lane * 4);
+					dictR[slot] = as_global(bcast_lane(D.dict, t))[min(lane, bcast_lane(D.nVals, t) - 1)];
+				};
 #pragma unroll
-					for(int k = 0; k < 4; k++) {
-						const double d = __shfl(dictB, (int) (eB[k] >> 16) & 63, 64);
-						if(lane * 4 + k < n) part += ytile[eB[k] & (ST - 1)] * d;
-					}
-					if(n > 256) {
-						const uint32_t* pk = as_global(bcast_lane(D.packed, tb)) + bcast_lane(start, tb);
-						for(int j0 = 256; j0 < n; j0 += 64) { // uniform trip count: the permute needs every lane
-							const uint32_t e = j0 + lane < n ? pk[j0 + lane] : 0u;
-							const double d = __shfl(dictB, (int) (e >> 16) & 63, 64);
-							if(j0 + lane < n) part += ytile[e & (ST - 1)] * d;
+				for(int j = 0; j < SDC_P; j++) issue(j, min(j, last));
+				for(int t = 0; t < nHere; t += SDC_P) {
+#pragma unroll
+					for(int j = 0; j < SDC_P; j++) {
+						const int tb = t + j;
+						const u32x4 eB = eR[j];
+						const double dictB = dictR[j];
+						issue(j, min(tb + SDC_P, last));
+						const int n = tb < nHere ? bcast_lane(cnt, min(tb, last)) : 0;
+						double part = 0.0;
+#pragma unroll
+						for(int k = 0; k < 4; k++) {
+							const double d = __shfl(dictB, (int) (eB[k] >> 16) & 63, 64);
+							const double yv = ytile[eB[k] & (ST - 1)];
+							part += lane * 4 + k < n ? yv * d : 0.0;
 						}
+						const double total = wave_sum_f64_all(part);
+						if(lane == tb) accT += total;
 					}
-					const double total = wave_sum_f64_all(part);
-					if(lane == tb) accT += total;
 				}
+			}
+			else {
+				u32x4 eA = {0, 0, 0, 0};
+				double dictA = 0.0;
+				for(int t = 0; t < nHere + 1; t++) {
+					const u32x4 eB = eA;
+					const double dictB = dictA;
+					if(t < nHere) { // ---- stage A: task t
+						const uint32_t* pk = as_global(bcast_lane(D.packed, t)) + bcast_lane(start, t);
+						eA = *(const u32x4*) (pk + lane * 4);
+						dictA = lane < bcast_lane(D.nVals, t) ? as_global(bcast_lane(D.dict, t))[lane] : 0.0;
+					}
+					if(t >= 1) { // ---- stage B: task t - 1
+						const int tb = t - 1;
+						const int n = bcast_lane(cnt, tb);
+						double part = 0.0;
+	#pragma unroll
+						for(int k = 0; k < 4; k++) {
+							const double d = __shfl(dictB, (int) (eB[k] >> 16) & 63, 64);
+							if(lane * 4 + k < n) part += ytile[eB[k] & (ST - 1)] * d;
+						}
+						if(n > 256) {
+							const uint32_t* pk = as_global(bcast_lane(D.packed, tb)) + bcast_lane(start, tb);
+							for(int j0 = 256; j0 < n; j0 += 64) { // uniform trip count: the permute needs every lane
+								const uint32_t e = j0 + lane < n ? pk[j0 + lane] : 0u;
+								const double d = __shfl(dictB, (int) (e >> 16) & 63, 64);
+								if(j0 + lane < n) part += ytile[e & (ST - 1)] * d;
+							}
+						}
+						const double total = wave_sum_f64_all(part);
+						if(lane == tb) accT += total;
+					}
+				}
+		
 			}
 		}
 		if(lane < nHere && accT != 0.0) unsafeAtomicAdd(&out[(size_t) irow * nCols + D.col0], accT);
