@@ -187,3 +187,29 @@ def test_map_width_table(ora):
     L = ora.lib()
     assert [L.ora_map_width(n) for n in (0, 1, 2, 128, 256, 257, 65536, 65537, 8388607, 8388608)] == \
         [0, 0, 1, 1, 1, 2, 2, 3, 3, 4]
+
+
+def test_offset_width_choice_hand_derived(ora):
+    """OffsetFactory.createOffset (OffsetFactory.java:105-139) takes the byte form when
+    OffsetByte.estimateInMemorySize(n - 1 + correctionByte) < OffsetChar.estimateInMemorySize(n - 1 + correctionChar)
+    with correctionX = max(range - (n - 1) * X, 0) / X for X = 256 and 65535 (:229-235), the estimates being
+    36 + byteArrayCost and 32 + charArrayCost (OffsetByte.java:100-104, OffsetChar.java:88-92;
+    MemoryEstimates.java:68-105: 32 for up to 4 bytes / 2 chars, else 28 + bytes padded to 4 mod 8). The
+    expected widths below were worked out by hand from those formulas:
+      [0,10,20]            2 entries: 36+32=68 vs 32+32=64                                   -> char
+      [0,1,2,3]            3 entries: 36+32=68 vs 32+(28+6+6)=72                             -> byte
+      0..9                 9 entries: 36+28+9+3=76 vs 32+28+18+2=80                          -> byte
+      [0,1e5,2e5]          corrections 779 and 1: byte 781 entries = 852 vs char 3 entries = 72 -> char
+      300*i, i<1000        correction 171: 64+1170+2=1236 vs 60+1998+6=2064                  -> byte
+      600*i, i<1000        correction 1342: 64+2341+7=2412 vs 2064                           -> char
+      511*i, i<1000        correction 995: 64+1994+2=2060 vs 2064                            -> byte
+      512*i, i<1000        correction 999: 64+1998+6=2068 vs 2064                            -> char"""
+    from systemds_amd import synth
+    table = [([0, 10, 20], 2), ([0, 1, 2, 3], 1), (list(range(10)), 1), ([0, 100000, 200000], 2),
+             ([300 * i for i in range(1000)], 1), ([600 * i for i in range(1000)], 2),
+             ([511 * i for i in range(1000)], 1), ([512 * i for i in range(1000)], 2)]
+    for rows, width in table:
+        rows = np.array(rows, np.int32)
+        assert ora.offset_choose_width(rows) == width, rows[:4]
+        if rows.size >= 3:
+            assert synth.choose_offset_width(rows) == width, rows[:4]

@@ -161,15 +161,21 @@ def test_counts_and_cooc_bit_exact(ora):
 
 
 def test_mmchain(ora):
+    """XtXv and XtwXv against the chain accumulated in long double, at the 1e-12 bar of the path: relative to
+    the magnitude of the terms summed into each cell, |D|' (|w| * (|D| |v|))."""
     specs, n_cols = mixed_block(12, 2500)
     G = ora.Groups(specs, 2500, n_cols)
     D = ora.np_decompress(specs, 2500, n_cols)
+    L = D.astype(np.longdouble)
     rng = np.random.default_rng(13)
     v, w = rng.standard_normal(n_cols), rng.standard_normal(2500)
+    inner_scale = np.abs(D) @ np.abs(v)
     out, _ = ora.mmchain(G, v, None, 0)
-    assert np.allclose(out, D.T @ (D @ v), rtol=1e-11, atol=1e-9)
+    truth = (L.T @ (L @ v.astype(np.longdouble))).astype(np.float64)
+    assert_close(out.reshape(-1), truth, np.abs(D).T @ inner_scale)
     out, _ = ora.mmchain(G, v, w, 1)
-    assert np.allclose(out, D.T @ (w * (D @ v)), rtol=1e-11, atol=1e-9)
+    truth = (L.T @ (w.astype(np.longdouble) * (L @ v.astype(np.longdouble)))).astype(np.float64)
+    assert_close(out.reshape(-1), truth, np.abs(D).T @ (np.abs(w) * inner_scale))
 
 
 def test_edge_sdc_lists(ora):
