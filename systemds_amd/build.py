@@ -78,8 +78,40 @@ def build_host(verbose=True):
     return HOST_LIB
 
 
+ROOT = os.path.dirname(HERE)
+C_DRIVER = os.path.join(ROOT, "tests", "cla_c_driver")
+
+
+def build_c_driver(verbose=True):
+    """The plain-C test driver of the C ABI (tests/cla_c_driver.c), linked against libclahip.so."""
+    cc = os.environ.get("CC", "gcc")
+    cmd = [cc, "-O2", "-std=gnu11", "-Wall", "-Wextra", "-I" + INCLUDE, C_DRIVER + ".c", "-o", C_DRIVER,
+           "-L" + HERE, "-lclahip", "-Wl,-rpath,$ORIGIN/../systemds_amd", "-lm"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.run(cmd, check=True)
+    return C_DRIVER
+
+
+def build_jni(verbose=True):
+    """The JNI shim (jni/cla_jni.c) when a JDK is present ($JAVA_HOME/include/jni.h); returns None otherwise."""
+    jh = os.environ.get("JAVA_HOME")
+    if not jh or not os.path.exists(os.path.join(jh, "include", "jni.h")):
+        return None
+    out = os.path.join(HERE, "libclahip_jni.so")
+    cmd = [os.environ.get("CC", "gcc"), "-O2", "-fPIC", "-shared", "-I" + os.path.join(jh, "include"),
+           "-I" + os.path.join(jh, "include", "linux"), "-I" + INCLUDE, os.path.join(HERE, "jni", "cla_jni.c"), "-o", out,
+           "-L" + HERE, "-lclahip", "-Wl,-rpath,$ORIGIN"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.run(cmd, check=True)
+    return out
+
+
 if __name__ == "__main__":
     build_lib(incremental="--incremental" in sys.argv)
     if "--no-host" not in sys.argv:
         build_host()
+        build_c_driver()
+        build_jni()
     sys.exit(0)

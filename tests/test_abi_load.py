@@ -53,3 +53,19 @@ def test_no_exception_crosses_the_boundary():
     assert lib.cla_selftest_exception(2) == capi.ERR_INVALID
     assert lib.cla_selftest_exception(3) == capi.ERR_INVALID
     assert lib.cla_selftest_exception(99) == 0
+
+
+def test_jni_shim_covers_the_java_natives():
+    """systemds_amd/jni: every `static native` of ClaHipNative.java has a shim function in cla_jni.c, and the
+    shim only calls symbols that include/cla_hip.h declares (neither file can be compiled without a JDK)."""
+    jni = os.path.join(ROOT, "systemds_amd", "jni")
+    java = open(os.path.join(jni, "ClaHipNative.java")).read()
+    shim = open(os.path.join(jni, "cla_jni.c")).read()
+    natives = re.findall(r"public static native \S+\s+(\w+)\(", java)
+    assert len(natives) >= 20
+    shims = set(re.findall(r"FN\((\w+)\)\(", shim)) | set(re.findall(r"ADD_COLS_VALUES\((\w+),", shim))
+    shims -= {"name"}  # the macro's own parameter
+    assert sorted(natives) == sorted(shims)
+    called = set(re.findall(r"\b(cla_[a-z_0-9]+)\s*\(", re.sub(r"/\*.*?\*/", "", shim, flags=re.S)))
+    called |= set(re.findall(r"ADD_COLS_VALUES\(\w+, (cla_\w+)\)", shim))
+    assert called and called <= set(declared_symbols()), called - set(declared_symbols())
