@@ -155,7 +155,11 @@ int64_t cla_lmm_dev(cla_handle h, const double* dY, int32_t nRowY, double* dOut)
 int cla_lmm_dev_async(cla_handle h, const double* dY, int32_t nRowY, double* dOut);
 
 /* CLALibTSMM.leftMultByTransposeSelf (C/lib/CLALibTSMM.java:59-94):
- * out[nCols x nCols] = t(X) %*% X, full symmetric. */
+ * out[nCols x nCols] = t(X) %*% X, full symmetric. Blocks no compressed form takes (overlapping
+ * groups, more than 110 columns holding an uncompressed group of more than 32, a pair of groups whose
+ * pre-aggregate exceeds LDS) are decompressed into a temporary dense copy and multiplied on the matrix
+ * cores, as the reference's own fallback does (:73-77); -CLA_ERR_UNSUPPORTED only when that copy does
+ * not fit the free device memory. */
 int64_t cla_tsmm(cla_handle h, double* out);
 int64_t cla_tsmm_dev(cla_handle h, double* dOut);
 int cla_tsmm_dev_async(cla_handle h, double* dOut);
@@ -164,9 +168,10 @@ int cla_tsmm_dev_async(cla_handle h, double* dOut);
  * (C/lib/CLALibLeftMultBy.java:100-112, 170-284): out[nColsLeft x nColsRight] = t(left) %*% right,
  * both blocks with the same number of rows. Every group of `left` meets every group of `right`
  * once (AColGroup.leftMultByAColGroup), the filtered constants of both sides enter through the
- * outer products with the column sums. Returns nnz(out) or a negative error; blocks with
- * overlapping groups are not supported, and beyond 64 columns of both blocks together an
- * uncompressed group may span at most 32 columns. The first call on a pair of handles builds a
+ * outer products with the column sums. Returns nnz(out) or a negative error. Shapes no compressed
+ * form takes (overlapping groups; beyond 64 columns of both blocks together an uncompressed group
+ * of more than 32 columns) go through the decompressed joint rows, as the reference's decompressing
+ * fallback does. The first call on a pair of handles builds a
  * small joint descriptor (and, on more than 64 joint columns, descriptors of column chunks). */
 int64_t cla_lmm_compressed(cla_handle right, cla_handle left, double* out);
 int64_t cla_lmm_compressed_dev(cla_handle right, cla_handle left, double* dOut);
@@ -179,8 +184,10 @@ int64_t cla_lmm_compressed_dev(cla_handle right, cla_handle left, double* dOut);
  * through B into the new block's constants. Only the small dictionary products are computed;
  * the returned block (nRows x nColB, overlapping groups) takes every entry point that is
  * linear in the groups (cla_rmm, cla_lmm, cla_mmchain, cla_decompress, sums) and borrows the
- * device copies of the source block, which stays alive until both handles are freed.
- * NULL on failure (cla_last_error); blocks with uncompressed groups are not supported. */
+ * device copies of the source block, which stays alive until both handles are freed. An
+ * uncompressed group returns an uncompressed group over all output columns that holds its rows times
+ * B[cols_g, :] (CG/ColGroupUncompressed.java:888-927), owned by the new block.
+ * NULL on failure (cla_last_error). */
 cla_handle cla_rmm_overlapping(cla_handle h, const double* B, int32_t nColB);
 
 /* CLALibMMChain.mmChain (C/lib/CLALibMMChain.java:92-148):

@@ -889,6 +889,19 @@ int64_t cla_tsmm(cla_handle b, double* out) {
 
 namespace cla {
 
+// Uncompressed group times B[cols, :] (ColGroupUncompressed.rightMultByMatrix, CG/ColGroupUncompressed.java:888-927):
+// out[r, j] = sum_h U[r, h] * B[cols[h], j]; thread = one output cell.
+__global__ __launch_bounds__(256) void k_unc_times_b(const double* __restrict__ U, int64_t nRows, int nC, const int32_t* __restrict__ cols,
+	const double* __restrict__ B, int q, double* __restrict__ out) {
+	const int64_t idx = (int64_t) blockIdx.x * 256 + threadIdx.x;
+	if(idx >= nRows * q) return;
+	const int64_t r = idx / q;
+	const int j = (int) (idx - r * q);
+	double s = 0.0;
+	for(int h = 0; h < nC; h++) s += U[(size_t) r * nC + h] * B[(size_t) cols[h] * q + j];
+	out[idx] = s;
+}
+
 __global__ __launch_bounds__(256) void k_take_block(const double* __restrict__ G, int n, int r0, int c0, int nr, int nc,
 	double* __restrict__ out, unsigned long long* __restrict__ nnz) {
 	int cnt = 0;
@@ -1202,7 +1215,6 @@ cla_handle cla_rmm_overlapping(cla_handle b, const double* B, int32_t nColB) {
 	CLA_TRY
 	if(check_final(b)) return nullptr;
 	if(!B || nColB <= 0) { set_error("rmm: invalid right-hand side"); return nullptr; }
-	if(b->hasUnc) { set_error("overlapping right multiply: uncompressed groups are not supported"); return nullptr; }
 	const int q = nColB;
 	std::lock_guard<std::recursive_mutex> lk(b->mu);
 	const size_t nIn = (size_t) b->nCols * q, nT = (size_t) (b->totalVals + 1) * q;
@@ -1225,6 +1237,34 @@ cla_handle cla_rmm_overlapping(cla_handle b, const double* B, int32_t nColB) {
 	int tblOff = 0, colOff = 0, maxVals = 0;
 	for(auto& pg : b->groups) {
 		const DGroup& P = pg.d;
+		if(P.type == G_UNC) {
+			// an uncompressed group returns an uncompressed group over all output columns that holds U x B[cols, :]
+			// (CG/ColGroupUncompressed.java:888-927); the new block owns it
+			c->groups.emplace_back();
+			HostGroup& g = c->groups.back();
+			memset(&g.d, 0, sizeof(g.d));
+			g.d.type = G_UNC; g.d.nColG = q;
+			g.cols = cols;
+			double* dense = nullptr;
+			const size_t nOut = (size_t) std::max<int64_t>(b->nRows, 1) * q;
+			if(upload(g, cols.data(), sizeof(int32_t) * (size_t) q, (const void**) &g.d.cols) ||
+				hipMalloc((void**) &dense, nOut * sizeof(double)) != hipSuccess) {
+				set_error("overlapping right multiply: allocating the product of an uncompressed group failed");
+				cla_block_free(c);
+				return nullptr;
+			}
+			g.owned.push_back(dense);
+			g.d.dense = dense;
+			g.bytes = (int64_t) (nOut * sizeof(double));
+			if(b->nRows > 0)
+				hipLaunchKernelGGL(k_unc_times_b, dim3((unsigned) ((b->nRows * q + 255) / 256)), dim3(256), 0, b->stream, P.dense, b->nRows,
+					P.nColG, P.cols, b->dStageIn, q, dense);
+			g.d.tblOff = tblOff;
+			g.d.colOff = colOff;
+			colOff += q;
+			c->hasUnc = true;
+			continue;
+		}
 		// groups without row data (const, empty, SDC without entries) live on in the constants only;
 		// the group list stays one to one with the source block otherwise, so the arena can be shared
 		if(P.type != G_DDC && P.type != G_SDCZ && P.type != G_RLE) {
@@ -1257,6 +1297,8 @@ cla_handle cla_rmm_overlapping(cla_handle b, const double* B, int32_t nColB) {
 	c->maxVals = maxVals;
 	c->parent = b;
 	b->refs.fetch_add(1);
+	// (products of uncompressed groups were queued on the source block's stream; the new block has its own)
+	if(c->hasUnc && hipStreamSynchronize(b->stream) != hipSuccess) { set_error("overlapping right multiply: device failure"); cla_block_free(c); return nullptr; }
 	if(finish_finalize(c, b)) { cla_block_free(c); return nullptr; }
 	return c;
 	CLA_CATCH_NULL

@@ -433,6 +433,96 @@ __global__ __launch_bounds__(256) void k_tsmm_finish(double* __restrict__ out, i
 
 __global__ void k_count_nnz2(const double* __restrict__ x, int64_t n, unsigned long long* __restrict__ nnz);
 
+// ---------------------------------------------------------------------------
+// t(D) %*% D of a dense row-major matrix on the matrix cores: the last resort for blocks no compressed form
+// takes (overlapping groups, uncompressed groups wider than a column chunk among many columns, pair
+// accumulators beyond LDS), after decompressing the block, which is what the reference does in these cases
+// (CLALibTSMM.java:73-77). Block = (range of rows, column block ib, group of GD_NBJ column blocks jb >= ib);
+// wave w takes rows 4 w .. 4 w + 3 of every 16; lane (k4, i16) holds D[row k4, 16 cb + i16] as both operands
+// of v_mfma_f64_16x16x4_f64. Accumulator register v of lane l is cell (4 v + l / 16, l % 16) of its tile.
+// Only tiles on or above the diagonal are computed; the caller mirrors.
+// ---------------------------------------------------------------------------
+constexpr int GD_NBJ = 8;
+typedef double gd_f64x4 __attribute__((ext_vector_type(4)));
+
+__global__ __launch_bounds__(256) void k_gram_dense(const double* __restrict__ D, int64_t nRows, int nCols, int64_t rowsPerBlock,
+	double* __restrict__ out) {
+	__shared__ double red[GD_NBJ * 256];
+	const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+	const int i16 = lane & 15, k4 = lane >> 4;
+	const int nb = (nCols + 15) / 16;
+	const int ib = blockIdx.y, jb0 = ib + blockIdx.z * GD_NBJ;
+	if(jb0 >= nb) return;
+	const int nj = min(GD_NBJ, nb - jb0);
+	const int64_t r0 = (int64_t) blockIdx.x * rowsPerBlock, r1 = min(nRows, r0 + rowsPerBlock);
+	gd_f64x4 acc[GD_NBJ];
+#pragma unroll
+	for(int j = 0; j < GD_NBJ; j++) acc[j] = gd_f64x4{0.0, 0.0, 0.0, 0.0};
+	const int ca = ib * 16 + i16;
+	for(int64_t r = r0 + wave * 4; r < r1; r += 16) {
+		const int64_t row = r + k4;
+		const bool in = row < r1;
+		const double* drow = D + (size_t) (in ? row : r0) * nCols;
+		const double a = in && ca < nCols ? drow[ca] : 0.0;
+#pragma unroll
+		for(int j = 0; j < GD_NBJ; j++) {
+			if(j >= nj) break;
+			const int cbj = (jb0 + j) * 16 + i16;
+			const double bv = in && cbj < nCols ? drow[cbj] : 0.0;
+			acc[j] = __builtin_amdgcn_mfma_f64_16x16x4f64(a, bv, acc[j], 0, 0, 0);
+		}
+	}
+	for(int i = tid; i < GD_NBJ * 256; i += 256) red[i] = 0.0;
+	__syncthreads();
+#pragma unroll
+	for(int j = 0; j < GD_NBJ; j++)
+#pragma unroll
+		for(int v = 0; v < 4; v++)
+			if(j < nj) unsafeAtomicAdd(&red[j * 256 + (4 * v + k4) * 16 + i16], acc[j][v]);
+	__syncthreads();
+	for(int i = tid; i < nj * 256; i += 256) {
+		const int j = i >> 8, rr = (i >> 4) & 15, cc = i & 15;
+		const int gr = ib * 16 + rr, gc = (jb0 + j) * 16 + cc;
+		if(gr <= gc && gc < nCols && red[i] != 0.0) unsafeAtomicAdd(&out[(size_t) gr * nCols + gc], red[i]);
+	}
+}
+
+// dOut (zeroed) = t(X) %*% X through the decompressed block. -CLA_ERR_UNSUPPORTED when the dense copy does
+// not fit the free device memory.
+static int launch_tsmm_decompressed(cla_block* b, double* dOut, unsigned long long* dNnz, const char* why) {
+	const int nCols = b->nCols;
+	const int64_t nRows = b->nRows;
+	hipStream_t st = b->stream;
+	const size_t bytes = sizeof(double) * (size_t) std::max<int64_t>(nRows, 1) * nCols;
+	size_t freeB = 0, totalB = 0;
+	CLA_HIP(hipMemGetInfo(&freeB, &totalB));
+	if(bytes > freeB / 2) {
+		set_error("tsmm: %s, and the decompressed block (%zu bytes) does not fit the free device memory (%zu)", why, bytes, freeB);
+		return -CLA_ERR_UNSUPPORTED;
+	}
+	double* dense = nullptr;
+	CLA_HIP(hipMalloc((void**) &dense, bytes));
+	int rc = launch_decompress(b, dense, dNnz); // (also counts the dense copy's non-zeros into dNnz: cleared again below)
+	if(rc == 0 && hipMemsetAsync(dNnz, 0, sizeof(unsigned long long), st) != hipSuccess) rc = -CLA_ERR_DEVICE;
+	if(rc == 0 && nRows > 0) {
+		const int nb = (nCols + 15) / 16;
+		int64_t rowsPerBlock = 16384;
+		while(rowsPerBlock > 1024 && (nRows + rowsPerBlock - 1) / rowsPerBlock * nb < (int64_t) g_numCU * 4) rowsPerBlock /= 2;
+		const dim3 grid((unsigned) ((nRows + rowsPerBlock - 1) / rowsPerBlock), (unsigned) nb, (unsigned) ((nb + GD_NBJ - 1) / GD_NBJ));
+		Prof pf(b, "k_gram_dense", (long) grid.x * grid.y * grid.z, 256, 0, (double) bytes);
+		hipLaunchKernelGGL(k_gram_dense, grid, dim3(256), 0, st, dense, nRows, nCols, rowsPerBlock, dOut);
+	}
+	if(rc == 0) {
+		Prof pf(b, "k_tsmm_finish", 1, 256, 0, 0);
+		hipLaunchKernelGGL(k_tsmm_finish, dim3(1), dim3(256), 0, st, dOut, nCols, b->dConstV, b->dConstV, (double) nRows, 0, dNnz);
+		if(hipGetLastError() != hipSuccess) rc = -CLA_ERR_DEVICE;
+	}
+	(void) hipStreamSynchronize(st); // the dense copy is freed below
+	(void) hipFree(dense);
+	if(rc == -CLA_ERR_DEVICE) set_error("tsmm: decompressing fallback failed on the device");
+	return rc;
+}
+
 int launch_tsmm(cla_block* b, double* dOut, unsigned long long* dNnz) {
 	const int nG = (int) b->groups.size();
 	const int nCols = b->nCols;
@@ -441,13 +531,14 @@ int launch_tsmm(cla_block* b, double* dOut, unsigned long long* dNnz) {
 	clear_stats(b);
 	CLA_HIP(hipMemsetAsync(dOut, 0, sizeof(double) * (size_t) nCols * nCols, st));
 	CLA_HIP(hipMemsetAsync(dNnz, 0, sizeof(unsigned long long), st));
-	// overlapping column groups need the diagonal doubling of addToUpperTriangle in
-	// every kernel; reject instead (the caller falls back)
+	// Overlapping column groups (the result of an overlapping right multiply): every compressed form here
+	// assumes one group per column, and such blocks typically hold more groups than columns, where the
+	// reference decompresses as well (CLALibTSMM.java:73-77).
 	{
 		std::vector<char> seen((size_t) nCols, 0);
 		for(auto& g : b->groups)
 			for(int c : g.cols) {
-				if(seen[c]) { set_error("tsmm: overlapping column groups are not supported"); return -CLA_ERR_UNSUPPORTED; }
+				if(seen[c]) return launch_tsmm_decompressed(b, dOut, dNnz, "overlapping column groups");
 				seen[c] = 1;
 			}
 	}
@@ -501,10 +592,8 @@ int launch_tsmm(cla_block* b, double* dOut, unsigned long long* dNnz) {
 			return 0;
 		}
 	}
-	if(dense && split > 0 && nCols > 64) {
-		set_error("compressed left multiply: an uncompressed group among more than 64 columns over both blocks (have %d) needs every group to span at most 32 columns", nCols);
-		return -CLA_ERR_UNSUPPORTED;
-	}
+	if(dense && split > 0 && nCols > 64)
+		return launch_tsmm_decompressed(b, dOut, dNnz, "a group of more than 32 columns without a per-pair form among more than 64 joint columns");
 	if(dense) {
 		// t(D) %*% D of the decoded rows, constants included (no correction layer needed)
 		const bool noMfma = !b->opt.tsmmMfma;
@@ -518,10 +607,8 @@ int launch_tsmm(cla_block* b, double* dOut, unsigned long long* dNnz) {
 		}
 		int DT = 256;
 		while(DT > 8 && (size_t) DT * nCols * 8 > (size_t) 96 * 1024) DT /= 2;
-		if((size_t) DT * nCols * 8 > (size_t) 96 * 1024 || (int64_t) nCols * (nCols + 1) / 2 > 24 * 256) {
-			set_error("tsmm: dense fallback supports at most 110 columns (block has %d)", nCols);
-			return -CLA_ERR_UNSUPPORTED;
-		}
+		if((size_t) DT * nCols * 8 > (size_t) 96 * 1024 || (int64_t) nCols * (nCols + 1) / 2 > 24 * 256)
+			return launch_tsmm_decompressed(b, dOut, dNnz, "more than 110 columns with a group of more than 32 columns that has no per-pair form");
 		if(DT > SDC_TILE) DT = SDC_TILE;
 		const int64_t nTiles = (nRows + DT - 1) / DT;
 		int tpb = 1;
@@ -583,8 +670,9 @@ int launch_tsmm(cla_block* b, double* dOut, unsigned long long* dNnz) {
 			const size_t dBytes = (size_t) S.nVals * S.nColG * 8;
 			const size_t cBytes = (size_t) 2 * TT * 4;
 			if(pBytes + cBytes > (size_t) 150 * 1024) {
-				set_error("tsmm: pre-aggregate of groups %d,%d needs %zu bytes of LDS", gt, gs, pBytes);
-				return -CLA_ERR_UNSUPPORTED;
+				// (what the kernels above have added to dOut is dropped)
+				CLA_HIP(hipMemsetAsync(dOut, 0, sizeof(double) * (size_t) nCols * nCols, st));
+				return launch_tsmm_decompressed(b, dOut, dNnz, "a pair of groups whose pre-aggregate exceeds LDS");
 			}
 			const int dictInLds = pBytes + dBytes + cBytes <= (size_t) 150 * 1024;
 			ldsMax = std::max(ldsMax, pBytes + (dictInLds ? dBytes : 0) + cBytes);

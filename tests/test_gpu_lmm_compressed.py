@@ -115,22 +115,22 @@ def test_uncompressed_groups_on_wide_blocks(cla, ora):
     check(cla, ora, a["groups"], a["n_cols"], specsU, nU, a["n_rows"], "t(wide) %*% unc")
 
 
-def test_overlapping_operand_is_refused(cla, ora):
-    """An overlapping block (the result of cla_rmm_overlapping) is not linear per cell pair: refused like in TSMM."""
+def test_overlapping_operand(cla, ora):
+    """An overlapping block (the result of cla_rmm_overlapping) on either side: no per-cell-pair form exists, the
+    joint rows are decompressed and multiplied on the matrix cores."""
     n_rows = 5000
     specs, n = mixed_block(11, n_rows, with_unc=False)
-    blk = cla.build_block(n_rows, n, specs)
-    child = blk.rmm_overlapping(np.random.default_rng(1).standard_normal((n, 3)))
-    with pytest.raises(cla.ClaError) as e:
-        blk.lmm_compressed(child)
-    assert e.value.code == cla.ERR_UNSUPPORTED
-    with pytest.raises(cla.ClaError) as e:
-        child.lmm_compressed(blk)
-    assert e.value.code == cla.ERR_UNSUPPORTED
-    # the refusal leaves both blocks usable
-    out, _ = blk.lmm_compressed(blk)
     D = ora.np_decompress(specs, n_rows, n)
-    assert_matches_truth(out, D.T, D, what="after refusal")
+    B = np.random.default_rng(1).standard_normal((n, 3))
+    P = ora.longdouble_matmul(D, B)
+    blk = cla.build_block(n_rows, n, specs)
+    child = blk.rmm_overlapping(B)
+    out, _ = blk.lmm_compressed(child)      # t(XB) %*% X
+    assert_fp64_close(out, ora.longdouble_matmul(P.T, D), np.abs(P).T @ np.abs(D), what="t(XB) %*% X", n_terms=n_rows)
+    out, _ = child.lmm_compressed(blk)      # t(X) %*% XB
+    assert_fp64_close(out, ora.longdouble_matmul(D.T, P), np.abs(D).T @ np.abs(P), what="t(X) %*% XB", n_terms=n_rows)
+    out, _ = blk.lmm_compressed(blk)
+    assert_matches_truth(out, D.T, D, what="t(X) %*% X afterwards")
     child.close()
     blk.close()
 

@@ -40,9 +40,11 @@ def test_mixed_groups(cla, ora, seed, n_rows, q):
     blk.close()   # the child keeps the borrowed device copies alive
     P = ora.longdouble_matmul(D, B)
     check_child(ora, child, P, np.abs(D) @ np.abs(B), rng, "mixed")
-    with pytest.raises(cla.ClaError) as e:   # not linear in the groups
-        child.tsmm()
-    assert e.value.code == cla.ERR_UNSUPPORTED
+    # t(XB) %*% (XB) is not linear in the groups: the block is decompressed and multiplied on the matrix cores
+    # (CLALibTSMM.java:73-77; CompressedTestBase.java:507-522 testTransposeSelfLeftMultOverload)
+    out, nnz = child.tsmm()
+    assert np.array_equal(out, out.T) and nnz == np.count_nonzero(out)
+    assert_fp64_close(out, ora.longdouble_matmul(P.T, P), np.abs(P).T @ np.abs(P), what="t(XB) %*% (XB)", n_terms=n_rows)
     with pytest.raises(cla.ClaError) as e:
         child.aggregate("max", "col")
     assert e.value.code == cla.ERR_UNSUPPORTED
@@ -71,9 +73,23 @@ def test_arena_block_shares_the_arena(cla, ora):
     blk.close()
 
 
-def test_uncompressed_groups_are_refused(cla, ora):
-    specs, n_cols = mixed_block(4, 500, with_unc=True)
-    blk = cla.build_block(500, n_cols, specs)
-    with pytest.raises(cla.ClaError):
-        blk.rmm_overlapping(np.ones((n_cols, 2)))
+@pytest.mark.parametrize("seed,n_rows,q", [(4, 500, 2), (5, 40011, 6)])
+def test_uncompressed_groups(cla, ora, seed, n_rows, q):
+    """An uncompressed group returns an uncompressed group over all output columns that holds its rows times
+    B[cols, :] (ColGroupUncompressed.rightMultByMatrix, CG/ColGroupUncompressed.java:888-927)."""
+    specs, n_cols = mixed_block(seed, n_rows, with_unc=True)
+    D = ora.np_decompress(specs, n_rows, n_cols)
+    rng = np.random.default_rng(seed)
+    B = rng.standard_normal((n_cols, q))
+    blk = cla.build_block(n_rows, n_cols, specs)
+    child = blk.rmm_overlapping(B)
     blk.close()
+    P = ora.longdouble_matmul(D, B)
+    check_child(ora, child, P, np.abs(D) @ np.abs(B), rng, "with an uncompressed group")
+    out, _ = child.tsmm()
+    assert_fp64_close(out, ora.longdouble_matmul(P.T, P), np.abs(P).T @ np.abs(P), what="t(XB) %*% (XB)", n_terms=n_rows)
+    grand = child.rmm_overlapping(rng.standard_normal((q, 3)))
+    child.close()
+    out, _ = grand.decompress()
+    assert out.shape == (n_rows, 3)
+    grand.close()

@@ -96,3 +96,47 @@ def test_random_blocks_against_the_decompressed_product(cla, ora, seed, max_grou
                 left.close()
         finally:
             blk.close()
+
+
+@pytest.mark.parametrize("seed,n_rows,n_dense,n_ddc", [(3, 4097, 40, 80), (4, 30000, 70, 50), (5, 1025, 33, 140)])
+def test_wide_blocks_with_wide_uncompressed_groups(cla, ora, seed, n_rows, n_dense, n_ddc):
+    """More than 110 columns holding an uncompressed group of more than 32 columns (no column chunk takes it), for
+    t(X) %*% X and as either side of the compressed x compressed product: the block is decompressed and multiplied
+    on the matrix cores, as the reference does whenever a block holds an uncompressed group (CLALibTSMM.java:73-77);
+    then the overlapping result of a right multiply through t(X B) %*% (X B)
+    (CompressedTestBase.java:507-522 testTransposeSelfLeftMultOverload)."""
+    from systemds_amd import synth
+    rng = np.random.default_rng(seed)
+    specs = [synth.GroupSpec("unc", np.arange(0, n_dense, dtype=np.int32), dense=rng.standard_normal((n_rows, n_dense)))]
+    c = n_dense
+    for _ in range(n_ddc // 2):
+        nv = int(rng.choice([3, 40, 300]))
+        codes = rng.integers(0, nv, n_rows).astype(np.uint8 if nv <= 256 else np.uint16)
+        specs.append(synth.GroupSpec("ddc", np.arange(c, c + 2, dtype=np.int32), rng.standard_normal((nv, 2)), codes))
+        c += 2
+    specs.append(synth.sdc_group(rng, n_rows, np.arange(c, c + 1, dtype=np.int32), 5, 0.05, 0.5))
+    c += 1
+    assert c > 110
+    D = ora.np_decompress(specs, n_rows, c)
+    blk = cla.build_block(n_rows, c, specs)
+    specs2, n2 = rand_block(rng, n_rows, 6)
+    D2 = ora.np_decompress(specs2, n_rows, n2)
+    other = cla.build_block(n_rows, n2, specs2)
+    try:
+        out, nnz = blk.tsmm()
+        assert np.array_equal(out, out.T) and nnz == np.count_nonzero(out)
+        assert_matches_truth(out, D.T, D, what="tsmm, wide dense group")
+        out, _ = blk.lmm_compressed(other)
+        assert_matches_truth(out, D2.T, D, what="t(L) %*% wide")
+        out, _ = other.lmm_compressed(blk)
+        assert_matches_truth(out, D.T, D2, what="t(wide) %*% R")
+        B = rng.standard_normal((c, 9))
+        child = blk.rmm_overlapping(B)
+        P = (D.astype(np.longdouble) @ B.astype(np.longdouble)).astype(np.float64)
+        out, _ = child.tsmm()
+        child.close()
+        scale = np.abs(D) @ np.abs(B)
+        assert np.all(np.abs(out - (P.T.astype(np.longdouble) @ P.astype(np.longdouble)).astype(np.float64)) <= 2e-12 * (scale.T @ scale))
+    finally:
+        blk.close()
+        other.close()
