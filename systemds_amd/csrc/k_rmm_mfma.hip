@@ -14,7 +14,8 @@
 //   D_b[i][j]: i = l / 16, j = l % 4       (one double per lane)
 // (probed on the device with one-hot operands; checked against a CPU product by the parity tests)
 // Here the four blocks are four groups of four rows (A lane l holds row l % 16 of a 16-row tile,
-// decoded column k) and B_b is the same for all blocks: B[column k][4 jg + j] of output group jg.
+// decoded column k) and B_b is the same for all blocks: B[column k][16 j + jg] for the jg-th of a lane's
+// 16 accumulators, so that a lane ends up with 16 consecutive output columns of one row.
 #include "../../include/cla_hip.h"
 #include "cla_device.hpp"
 #include <algorithm>
@@ -29,7 +30,11 @@ constexpr int MF_NJ = 16;                    // groups of 4 output columns per p
 // bank quads (row stride 16 banks, j stride 36 banks)
 constexpr int MF_BJ = 18;
 constexpr int MF_BK = 4 * MF_BJ;
-constexpr int MF_SS = 68;                    // row stride (doubles) of the output staging: 8 rows on distinct banks
+// Output staging of a wave: 16 rows; a row is four segments of 16 columns, MF_SEG doubles apart, rows MF_SS
+// doubles apart: the sixteen 16-byte writes of lanes 0-15 (rows 0, 4, 8, 12 x four segments) fall on sixteen
+// distinct groups of four banks (row stride 148 dwords = 20 mod 64, segment stride 36 dwords)
+constexpr int MF_SEG = 18;
+constexpr int MF_SS = 74;
 
 // code stream of a decoded column (device array: at row 0; LDS copy: at the block's first row)
 struct MfSrc {
@@ -43,17 +48,17 @@ struct MfSlab {
 	int32_t dictDoubles;   // two zero doubles + the dictionaries of the slab's groups
 	int32_t width;         // bytes per element of the slab's code tiles (1 or 2)
 	int32_t kOff;          // first row of the slab in the re-laid B
-	int32_t pad;
+	int32_t pad;           // 1: a code stream of the slab is narrower than the tiles' width
 	const double* dictSrc; // the slab's dictionaries, back to back
 };
 
 // B in the slab layout: row r of the list (decoded column rowCol[r], -1 = padding) at r * MF_BK,
-// output column n0 + 4 jg + j at j * MF_BJ + jg
+// output column n0 + 16 j + jg at j * MF_BJ + jg
 __global__ __launch_bounds__(128) void k_mfma_blayout(const double* __restrict__ B, int q, int n0, const int32_t* __restrict__ rowCol,
 	double* __restrict__ Bl) {
 	const int r = blockIdx.x, t = threadIdx.x;
 	if(t >= MF_BK) return;
-	const int j = t / MF_BJ, jg = t - j * MF_BJ, col = n0 + 4 * jg + j, gc = rowCol[r];
+	const int j = t / MF_BJ, jg = t - j * MF_BJ, col = n0 + 16 * j + jg, gc = rowCol[r];
 	Bl[(size_t) r * MF_BK + t] = (jg < 16 && gc >= 0 && col < q) ? B[(size_t) gc * q + col] : 0.0;
 }
 
@@ -72,6 +77,26 @@ __global__ __launch_bounds__(128) void k_mfma_blayout(const double* __restrict__
 // LDS reads: code, value; one multiply-add).
 #define MF_GPTR(p) ((const __attribute__((address_space(1))) void*) (p))
 #define MF_LPTR(p) ((__attribute__((address_space(3))) void*) (p))
+
+// Code tiles of a slab through registers: a ragged last tile (rows behind the end of the matrix hold code 0) or
+// code streams narrower than the tile's width (widened). Piece = 16 bytes of one column's tile per lane.
+template <int W>
+__device__ __attribute__((noinline)) void mf_fill_codes_slow(const MfSrc* __restrict__ src, int nc, int64_t row0, int rowsHere, int rows,
+	uint8_t* __restrict__ dst, int wave, int waves, int lane) {
+	const int tileBytes = rows * W, total = nc * tileBytes;
+	for(int byte = (wave * 64 + lane) * 16; byte < total; byte += waves * 1024) {
+		const int c = byte / tileBytes, off = byte - c * tileBytes;
+		const MfSrc ms = src[c];
+		const uint8_t* codes = as_global(ms.codes) + (size_t) row0 * ms.width;
+		const int r0 = off / W;
+		uint32_t e[4] = {0, 0, 0, 0};
+		for(int t = 0; t < 16 / W; t++) {
+			const uint32_t code = r0 + t < rowsHere ? (uint32_t) load_code(codes, ms.width, r0 + t) : 0u;
+			e[(t * W) >> 2] |= code << (8 * ((t * W) & 3));
+		}
+		*(u32x4*) (dst + byte) = u32x4{e[0], e[1], e[2], e[3]};
+	}
+}
 
 template <int WAVES, int W>
 __global__ __launch_bounds__(WAVES * 64) void k_rmm_mfma(const MfSlab* __restrict__ slabs, int nSlabs,
@@ -97,56 +122,49 @@ __global__ __launch_bounds__(WAVES * 64) void k_rmm_mfma(const MfSlab* __restric
 	int cnt = 0;
 	__syncthreads();
 
-	// ---- fill of (tile, slab) into buffer `buf`: pieces of 1 KB, piece pc by wave pc % WAVES
+	// ---- fill of (tile, slab) into buffer `buf`: pieces of 1 KB spread over the waves. The three contiguous
+	// regions (dictionaries, rows of B, column info) and the code tiles of a full tile whose code streams have
+	// the tile's width are straight global -> LDS copies with a handful of instructions per piece (the loops are
+	// kept rolled: unrolled with the ragged path inlined, the fill was 3000 instructions per pair and took a
+	// seventh of the kernel's time); a ragged last tile or narrower codes go through mf_fill_codes_slow.
+	// (Letting only one of the two waves of a SIMD issue a fill, so that the other keeps the matrix pipe busy
+	// meanwhile, was measured slower with either assignment of waves: 2.84 / 2.91 ms against 2.79.)
+	constexpr int FW = WAVES;
+	auto copy_region = [&](const uint8_t* src, uint8_t* dst, int bytes, int fw, int rot) {
+		const int ew = (fw + rot) & (FW - 1);
+#pragma unroll 1
+		for(int off0 = ew * 1024; off0 < bytes; off0 += FW * 1024) {
+			const int off = off0 + lane * 16;
+			if(off < bytes) __builtin_amdgcn_global_load_lds(MF_GPTR(as_global(src) + off), MF_LPTR(dst + off0), 16, 0, 0);
+		}
+	};
 	auto fill = [&](int tile, int s, int buf) {
+		const int fw = wave;
 		const MfSlab sl = slabS[s];
 		const int64_t row0 = (int64_t) tile * ROWS;
 		const int rowsHere = (int) min((int64_t) ROWS, nRows - row0);
 		const int kc = (sl.nc + 3) & ~3;
 		uint8_t* const base = lds + (size_t) buf * bufBytes;
-		const int dictBytes = (sl.dictDoubles - 2) * 8, bBytes = kc * MF_BK * 8, infoBytes = kc * 4;
-		constexpr int colsPerPiece = 1024 / (ROWS * W) > 0 ? 1024 / (ROWS * W) : 1; // (ROWS * W is 256, 512 or 1024)
-		constexpr int piecesPerCol = ROWS * W / 1024 > 0 ? ROWS * W / 1024 : 1;
-		const int pDict = (dictBytes + 1023) >> 10, pB = (bBytes + 1023) >> 10, pInfo = (infoBytes + 1023) >> 10;
-		const int pCodes = (sl.nc + colsPerPiece - 1) / colsPerPiece * piecesPerCol;
-		const int nPieces = pDict + pB + pInfo + pCodes;
-		for(int pc = wave; pc < nPieces; pc += WAVES) {
-			if(pc < pDict) { // (an odd number of doubles: the last lane reads 8 bytes more; the allocation is padded)
-				const int off = pc * 1024 + lane * 16;
-				if(off < dictBytes)
-					__builtin_amdgcn_global_load_lds(MF_GPTR((const uint8_t*) as_global(sl.dictSrc) + off), MF_LPTR(base + 16 + pc * 1024), 16, 0, 0);
-			}
-			else if(pc < pDict + pB) {
-				const int j = pc - pDict, off = j * 1024 + lane * 16;
-				if(off < bBytes)
-					__builtin_amdgcn_global_load_lds(MF_GPTR((const uint8_t*) (Bl + (size_t) sl.kOff * MF_BK) + off), MF_LPTR(base + oB + j * 1024), 16, 0, 0);
-			}
-			else if(pc < pDict + pB + pInfo) {
-				const int j = pc - pDict - pB, off = j * 1024 + lane * 16;
-				if(off < infoBytes)
-					__builtin_amdgcn_global_load_lds(MF_GPTR((const uint8_t*) (infoG + sl.kOff) + off), MF_LPTR(base + oInfo + j * 1024), 16, 0, 0);
-			}
-			else { // code tiles: lane -> (column, 16 bytes of its tile)
-				const int j = pc - pDict - pB - pInfo;
-				const int byte = j * 1024 + lane * 16; // inside the slab's code tiles
-				const int c = byte / (ROWS * W), off = byte - c * (ROWS * W);
-				if(c < sl.nc) {
-					const MfSrc ms = srcS[sl.c0 + c];
-					const uint8_t* src = as_global(ms.codes) + (size_t) row0 * ms.width;
-					const int r0 = off / W;
-					if(ms.width == W && r0 + 16 / W <= rowsHere)
-						__builtin_amdgcn_global_load_lds(MF_GPTR(src + off), MF_LPTR(base + oCodes + j * 1024), 16, 0, 0);
-					else { // widened or ragged piece: through registers
-						uint32_t e[4] = {0, 0, 0, 0};
-						for(int t = 0; t < 16 / W; t++) {
-							const uint32_t code = r0 + t < rowsHere ? (uint32_t) load_code(src, ms.width, r0 + t) : 0u;
-							e[(t * W) >> 2] |= code << (8 * ((t * W) & 3));
-						}
-						*(u32x4*) (base + oCodes + byte) = u32x4{e[0], e[1], e[2], e[3]};
-					}
+		// (an odd number of dictionary doubles: the last lane reads 8 bytes more; the allocation is padded)
+		copy_region((const uint8_t*) sl.dictSrc, base + 16, (sl.dictDoubles - 2) * 8, fw, 0);
+		copy_region((const uint8_t*) (Bl + (size_t) sl.kOff * MF_BK), base + oB, kc * MF_BK * 8, fw, 1);
+		copy_region((const uint8_t*) (infoG + sl.kOff), base + oInfo, kc * 4, fw, 3);
+		constexpr int TILE_BYTES = ROWS * W; // 512 or 1024 (W = 1, 2; 8 waves) / 256 or 512 (4 waves): a power of two up to 1 KB
+		static_assert((TILE_BYTES & (TILE_BYTES - 1)) == 0 && TILE_BYTES <= 1024, "code tiles divide a 1 KB piece");
+		const int codeBytes = sl.nc * TILE_BYTES;
+		if(rowsHere == ROWS && sl.pad == 0) { // full tile, every code stream of the slab has the tile's width
+			const int ew = (fw + 2) & (FW - 1);
+#pragma unroll 1
+			for(int off0 = ew * 1024; off0 < codeBytes; off0 += FW * 1024) {
+				const int byte = off0 + lane * 16;
+				const int c = byte / TILE_BYTES, off = byte & (TILE_BYTES - 1);
+				if(byte < codeBytes) {
+					const uint8_t* src = as_global(srcS[sl.c0 + c].codes) + (size_t) row0 * W + off;
+					__builtin_amdgcn_global_load_lds(MF_GPTR(src), MF_LPTR(base + oCodes + off0), 16, 0, 0);
 				}
 			}
 		}
+		else mf_fill_codes_slow<W>(srcS + sl.c0, sl.nc, row0, rowsHere, ROWS, base + oCodes, fw, FW, lane);
 	};
 
 	// persistent block: row tiles blockIdx.x, + gridDim.x, ...
@@ -223,46 +241,48 @@ __global__ __launch_bounds__(WAVES * 64) void k_rmm_mfma(const MfSlab* __restric
 			}
 		}
 
-		// epilogue: eight rows of a 16-row tile at a time through LDS (over the buffer of the tile's last
-		// slab; the next pair's fill goes to the other one), so that every store instruction writes whole
-		// output rows; + constV x B, count non-zeros.
-		// acc[m][n] of lane l is output row 16 m + 4 b + i (b = (l / 4) % 4, i = l / 16), column 4 n + l % 4.
+		// epilogue: a 16-row tile at a time through LDS (over the buffer of the tile's last slab; the next
+		// pair's fill goes to the other one), so that every store instruction writes whole output rows;
+		// + constV x B, count non-zeros.
+		// acc[m][n] of lane l is output row 16 m + 4 b + i (b = (l / 4) % 4, i = l / 16), column 16 (l % 4) + n:
+		// a lane writes its 16 consecutive columns as eight 16-byte pieces, then lanes 0-31 / 32-63 read two
+		// rows back as 512 contiguous bytes each (1 KB per store instruction).
 		__syncthreads();
 		double* const stageS = (double*) (lds + (size_t) (buf ^ 1) * bufBytes); // (buf has moved on to the next pair's)
-		// (two columns per lane and two rows per store instruction: 1 KB per instruction)
-		const int col = n0 + 2 * (lane & 31), rsel = lane >> 5;
+		const int l32 = lane & 31, rsel = lane >> 5;
+		const int col = n0 + 2 * l32;
 		const double cadd0 = (constRow != nullptr && col < q) ? constRow[col] : 0.0;
 		const double cadd1 = (constRow != nullptr && col + 1 < q) ? constRow[col + 1] : 0.0;
-		double* st = stageS + (size_t) wave * 8 * MF_SS;
+		double* st = stageS + (size_t) wave * 16 * MF_SS;
+		double* const wp = st + (size_t) (lb * 4 + lk) * MF_SS + lj * MF_SEG;
+		const double* const rp = st + (size_t) rsel * MF_SS + (l32 >> 3) * MF_SEG + 2 * (l32 & 7);
 #pragma unroll
 		for(int m = 0; m < MF_MT; m++) {
 #pragma unroll
-			for(int h = 0; h < 2; h++) {
-				if((lb >> 1) == h) {
-					double* p = st + (size_t) ((lb & 1) * 4 + lk) * MF_SS + lj;
+			for(int n = 0; n < MF_NJ; n += 2) {
+				f64x2 w;
+				w[0] = acc[m][n]; w[1] = acc[m][n + 1];
+				*(f64x2*) (wp + n) = w;
+			}
+			__builtin_amdgcn_wave_barrier(); // same-wave LDS accesses complete in order
+			const int64_t row0 = blockRow0 + wave * (MF_MT * 16) + m * 16 + rsel;
 #pragma unroll
-					for(int n = 0; n < MF_NJ; n++) p[4 * n] = acc[m][n];
-				}
-				__builtin_amdgcn_wave_barrier(); // same-wave LDS accesses complete in order
-				const int64_t row0 = blockRow0 + wave * (MF_MT * 16) + m * 16 + h * 8 + rsel;
-#pragma unroll
-				for(int r = 0; r < 8; r += 2) {
-					f64x2 v = *(const f64x2*) (st + (size_t) (r + rsel) * MF_SS + 2 * (lane & 31));
-					v[0] += cadd0; v[1] += cadd1;
-					if(row0 + r < nRows) {
-						double* o = &out[(size_t) (row0 + r) * q + col];
-						if(col + 1 < q) {
-							cnt += (v[0] != 0.0) + (v[1] != 0.0);
-							__builtin_nontemporal_store(v, (f64x2*) o);
-						}
-						else if(col < q) {
-							cnt += v[0] != 0.0;
-							__builtin_nontemporal_store(v[0], o);
-						}
+			for(int r = 0; r < 16; r += 2) {
+				f64x2 v = *(const f64x2*) (rp + (size_t) r * MF_SS);
+				v[0] += cadd0; v[1] += cadd1;
+				if(row0 + r < nRows) {
+					double* o = &out[(size_t) (row0 + r) * q + col];
+					if(col + 1 < q) {
+						cnt += (v[0] != 0.0) + (v[1] != 0.0);
+						__builtin_nontemporal_store(v, (f64x2*) o);
+					}
+					else if(col < q) {
+						cnt += v[0] != 0.0;
+						__builtin_nontemporal_store(v[0], o);
 					}
 				}
-				__builtin_amdgcn_wave_barrier();
 			}
+			__builtin_amdgcn_wave_barrier();
 		}
 		if(tid < 2) stageS[tid] = 0.0; // the staging (of wave 0) lay over that buffer's zero doubles
 	} // tiles
@@ -290,7 +310,7 @@ int launch_rmm_mfma(cla_block* b, const double* dB, int q, const double* dConstR
 	// 8 waves per block (512-row tiles, two waves per SIMD), one block per CU with two slab buffers
 	const int waves = 8;
 	const int rows = waves * MF_MT * 16;
-	const size_t stageBytes = (size_t) waves * 8 * MF_SS * 8;
+	const size_t stageBytes = (size_t) waves * 16 * MF_SS * 8;
 	const int ldsKb = 156;
 	const size_t fixedBytes = (size_t) nColsAll * sizeof(MfSrc) + 32 * sizeof(MfSlab);
 	const size_t ldsTotal = (size_t) std::min(g_ldsPerBlock - 1024, ldsKb * 1024);
@@ -348,6 +368,9 @@ int launch_rmm_mfma(cla_block* b, const double* dB, int q, const double* dConstR
 				g = goodG; nc = goodNc; dictD = goodDict;
 			}
 			sl.g1 = g; sl.nc = nc; sl.dictDoubles = (int32_t) dictD; sl.width = blockWidth;
+			sl.pad = 0; // 1: some code stream of the slab is narrower than the tiles (no plain copy)
+			for(int gg = sl.g0; gg < g; gg++)
+				if(b->groups[gg].d.codeWidth != blockWidth) sl.pad = 1;
 			while(rowCol.size() % 4) { rowCol.push_back(-1); info.push_back(0); }
 			maxDict = std::max(maxDict, (dictD + 1) & ~(size_t) 1);
 			maxKc = std::max(maxKc, (nc + 3) & ~3);
