@@ -98,9 +98,11 @@ static int ensure_stage(double** p, size_t* cap, size_t nDoubles) {
 
 static int upload(HostGroup& g, const void* src, size_t bytes, const void** dst) {
 	void* d = nullptr;
-	CLA_HIP(hipMalloc(&d, std::max<size_t>(bytes, 16)));
+	CLA_HIP(hipMalloc(&d, bytes + UPLOAD_SLACK));
 	g.owned.push_back(d);
+	CLA_HIP(hipMemset((char*) d + bytes, 1, UPLOAD_SLACK));
 	if(bytes) CLA_HIP(hipMemcpy(d, src, bytes, hipMemcpyHostToDevice));
+	else CLA_HIP(hipStreamSynchronize(nullptr));
 	g.bytes += (int64_t) bytes;
 	*dst = d;
 	return 0;
@@ -286,6 +288,8 @@ void cla_block_free(cla_handle b) {
 	if(b->dSdcPlan) (void) hipFree(b->dSdcPlan);
 	if(b->dSdcDesc) (void) hipFree(b->dSdcDesc);
 	if(b->dSdcPacked) (void) hipFree(b->dSdcPacked);
+	if(b->dLaneMeta) (void) hipFree(b->dLaneMeta);
+	if(b->dLaneData) (void) hipFree(b->dLaneData);
 	if(b->dDictPad) (void) hipFree(b->dDictPad);
 	if(b->dCountsAll) (void) hipFree(b->dCountsAll);
 	if(b->dOnes) (void) hipFree(b->dOnes);
@@ -658,6 +662,7 @@ int cla_block_set_option(cla_handle b, const char* key, int32_t value) {
 		{"tsmm_pair_dot", &Options::tsmmPairDot, 0, 1},     {"expand_streams", &Options::expandStreams, 0, 1},
 		{"rmm_disable", &Options::rmmDisable, 0, 15},       {"lmm_disable", &Options::lmmDisable, 0, 3},
 		{"sdc_packed", &Options::sdcPacked, 0, 1},
+		{"sdc_lanes", &Options::sdcLanes, 0, 1},
 	};
 	for(const Entry& e : table)
 		if(strcmp(e.name, key) == 0) {

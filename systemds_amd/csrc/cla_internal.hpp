@@ -18,6 +18,9 @@ enum : int32_t { G_DDC = 0, G_SDCZ = 1, G_RLE = 2, G_UNC = 3 };
 // index entry with the iterator state in front of the first entry of the tile.
 constexpr int SDC_CK = 1024;
 constexpr int SDC_TILE = 1024;
+// Bytes allocated (and filled with 0x01) behind every uploaded array: list walkers read whole registers
+// from any byte position of an offset or code list without a bounds check.
+constexpr int UPLOAD_SLACK = 128;
 
 // Iterator state of an offset list in front of delta entry `idx`:
 // `row` = rows accumulated so far (last emitted row plus pending 0-entry skips),
@@ -71,6 +74,7 @@ struct Options {
 	int rmmDisable = 0;     // bit 0 byte-code mat-vec, 1 fused tables of the byte-code mat-vec, 2 matrix-core kernel, 3 decode kernel
 	int lmmDisable = 0;     // bit 0 dot form on byte codes, 1 byte-code bin kernel
 	int sdcPacked = 1;      // packed SDCZeros lists for the mat-vecs
+	int sdcLanes = 1;       // SDCZeros mat-vecs on the lists in place, one lane per group
 };
 
 struct KernelStat {
@@ -157,6 +161,13 @@ struct cla_block {
 	// built on first use for all groups (sdcPlanGroup -1) or for one group (its index)
 	int32_t* dSdcPlan = nullptr;
 	void* dSdcDesc = nullptr;        // one compact descriptor per listed group (k_*_sdc_packed)
+	void* dLaneMeta = nullptr;       // lane-per-group kernels (k_sdc_lanes.hip): descriptors, slabs, dictionaries, table index, chunk starts
+	void* dLaneData = nullptr;       // the listed groups' lists as lane-major windows, built on first use
+	int laneState = 0;               // 0 not planned yet, 1 ready, -1 the lists do not fit these kernels
+	int laneSlabs = 0, laneDictLds = 0;
+	size_t laneOff[4] = {0, 0, 0, 0};
+	bool laneLmm = false;            // every listed group has one column (the left multiply's condition)
+	bool sdcPackFailed = false;
 	uint32_t* dSdcPacked = nullptr;  // all listed groups' entries as (code << 16 | row inside its 4096-row tile), built on first use
 	int sdcPlanGroup = -2;
 	std::vector<int32_t> sdcList, sdcBinOff;
@@ -203,6 +214,8 @@ int launch_rmm_mfma(cla_block* b, const double* dB, int q, const double* dConstR
 int launch_lmm_u8(cla_block* b, const double* dY, int p, double* dPre);
 int launch_lmm_u8_dot(cla_block* b, const double* dY, int p, double* dOut);
 int launch_lmm_sdc_tiles(cla_block* b, const double* dY, int p, double* dPre, int onlyGroup, double* dOut);
+int launch_lmm_sdc_lanes(cla_block* b, const double* dY, int p, double* dOut);
+int launch_rmm_sdc_lanes(cla_block* b, int constRow, int accumulate, double* dOut, unsigned long long* dNnz);
 int launch_rmm_sdc_tiles(cla_block* b, int q, int constRow, int accumulate, double* dOut, unsigned long long* dNnz);
 int launch_tsmm_decode(cla_block* b, double* dOut);
 int launch_rmm_decode(cla_block* b, const double* dB, int q, const double* dConstRow, double* dOut,

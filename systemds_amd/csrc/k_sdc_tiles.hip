@@ -408,7 +408,28 @@ __global__ __launch_bounds__(ST_THREADS) void k_lmm_sdc_packed(const SdcDesc* __
 
 // Host side: list of SDCZeros groups and the prefix sums of their nVals, kept on the block
 // (host and device copy) and rebuilt only when the requested group selection changes.
-static int sdc_plan(cla_block* b, int onlyGroup, int32_t** dList, int32_t** dBinOff) {
+static int sdc_upload_desc(cla_block* b, bool wholeBlock) {
+	std::vector<SdcDesc> descs;
+	int64_t packedOff = 0;
+	for(int g : b->sdcList) {
+		const DGroup& G = b->groups[g].d;
+		SdcDesc d;
+		d.deltas = G.deltas; d.codes = G.codes; d.tileIdx = G.tileIdx;
+		d.nDeltas = (int32_t) G.nDeltas; d.nOffsets = (int32_t) G.nOffsets; d.first = G.first; d.tblOff = G.tblOff; d.nTiles = G.nTiles;
+		d.widths = G.deltaWidth | (G.codeWidth << 8);
+		d.nVals = G.nVals; d.col0 = b->groups[g].cols[0]; d.dict = G.dict;
+		d.packed = wholeBlock && b->dSdcPacked ? b->dSdcPacked + packedOff : nullptr; // packed lists belong to the whole-block plan
+		packedOff += G.nOffsets;
+		descs.push_back(d);
+	}
+	if(!descs.empty()) {
+		CLA_HIP(hipMemcpyAsync(b->dSdcDesc, descs.data(), descs.size() * sizeof(SdcDesc), hipMemcpyHostToDevice, b->stream));
+		CLA_HIP(hipStreamSynchronize(b->stream)); // `descs` goes out of scope
+	}
+	return 0;
+}
+
+static int sdc_plan(cla_block* b, int onlyGroup, int32_t** dList, int32_t** dBinOff, bool wantPacked = false) {
 	const size_t nG = b->groups.size();
 	if(b->dSdcPlan == nullptr) CLA_HIP(hipMalloc((void**) &b->dSdcPlan, (2 * nG + 2) * sizeof(int32_t)));
 	if(b->dSdcDesc == nullptr) CLA_HIP(hipMalloc(&b->dSdcDesc, std::max<size_t>(nG, 1) * sizeof(SdcDesc)));
@@ -422,46 +443,41 @@ static int sdc_plan(cla_block* b, int onlyGroup, int32_t** dList, int32_t** dBin
 			b->sdcBinOff.push_back(b->sdcBinOff.back() + G.nVals);
 		}
 		b->sdcPlanGroup = -2; // invalid until both copies have been issued
-		// packed entries of all listed groups (whole-block plans only), 256 entries of slack behind the last
-		std::vector<int64_t> packedOff;
-		bool packable = onlyGroup < 0 && !b->sdcList.empty();
-		int64_t totalEntries = 0;
-		for(int g : b->sdcList) {
-			packedOff.push_back(totalEntries);
-			totalEntries += b->groups[g].d.nOffsets;
-			packable &= b->groups[g].d.nVals <= 65536;
-		}
-		if(packable && b->dSdcPacked == nullptr) {
-			CLA_HIP(hipMalloc((void**) &b->dSdcPacked, sizeof(uint32_t) * (size_t) (totalEntries + 256)));
-			b->derivedBytes += (int64_t) sizeof(uint32_t) * (totalEntries + 256);
-			CLA_HIP(hipMemsetAsync(b->dSdcPacked + totalEntries, 0, sizeof(uint32_t) * 256, b->stream));
-			const int nT1 = (int) ((b->nRows + SDC_TILE - 1) / SDC_TILE);
-			for(size_t l = 0; l < b->sdcList.size(); l++)
-				hipLaunchKernelGGL(k_sdc_pack, dim3((unsigned) ((nT1 + 3) / 4)), dim3(256), 0, b->stream, b->dGroups, b->sdcList[l], b->nRows,
-					b->dSdcPacked + packedOff[l]);
-			CLA_HIP(hipGetLastError());
-		}
-		std::vector<SdcDesc> descs;
-		size_t li = 0;
-		for(int g : b->sdcList) {
-			const DGroup& G = b->groups[g].d;
-			SdcDesc d;
-			d.deltas = G.deltas; d.codes = G.codes; d.tileIdx = G.tileIdx;
-			d.nDeltas = (int32_t) G.nDeltas; d.nOffsets = (int32_t) G.nOffsets; d.first = G.first; d.tblOff = G.tblOff; d.nTiles = G.nTiles;
-			d.widths = G.deltaWidth | (G.codeWidth << 8);
-			d.nVals = G.nVals; d.col0 = b->groups[g].cols[0]; d.dict = G.dict;
-			d.packed = packable && b->dSdcPacked ? b->dSdcPacked + packedOff[li] : nullptr;
-			li++;
-			descs.push_back(d);
-		}
+		int rc = sdc_upload_desc(b, onlyGroup < 0);
+		if(rc) return rc;
 		if(!b->sdcList.empty()) {
-			CLA_HIP(hipMemcpyAsync(b->dSdcDesc, descs.data(), descs.size() * sizeof(SdcDesc), hipMemcpyHostToDevice, b->stream));
 			CLA_HIP(hipMemcpyAsync(b->dSdcPlan, b->sdcList.data(), b->sdcList.size() * 4, hipMemcpyHostToDevice, b->stream));
 			CLA_HIP(hipMemcpyAsync(b->dSdcPlan + nG, b->sdcBinOff.data(), b->sdcBinOff.size() * 4, hipMemcpyHostToDevice, b->stream));
 			// the host vectors are rewritten by the next selection: the copies must have read them
 			CLA_HIP(hipStreamSynchronize(b->stream));
 		}
 		b->sdcPlanGroup = onlyGroup;
+	}
+	// packed entries of all listed groups (whole-block plans only, when a packed kernel asks), 256 entries of slack
+	// behind the last
+	if(wantPacked && onlyGroup < 0 && !b->sdcList.empty() && b->dSdcPacked == nullptr && !b->sdcPackFailed) {
+		int64_t totalEntries = 0;
+		bool packable = true;
+		for(int g : b->sdcList) {
+			totalEntries += b->groups[g].d.nOffsets;
+			packable &= b->groups[g].d.nVals <= 65536;
+		}
+		b->sdcPackFailed = !packable;
+		if(packable) {
+			CLA_HIP(hipMalloc((void**) &b->dSdcPacked, sizeof(uint32_t) * (size_t) (totalEntries + 256)));
+			b->derivedBytes += (int64_t) sizeof(uint32_t) * (totalEntries + 256);
+			CLA_HIP(hipMemsetAsync(b->dSdcPacked + totalEntries, 0, sizeof(uint32_t) * 256, b->stream));
+			const int nT1 = (int) ((b->nRows + SDC_TILE - 1) / SDC_TILE);
+			int64_t off = 0;
+			for(int g : b->sdcList) {
+				hipLaunchKernelGGL(k_sdc_pack, dim3((unsigned) ((nT1 + 3) / 4)), dim3(256), 0, b->stream, b->dGroups, g, b->nRows,
+					b->dSdcPacked + off);
+				off += b->groups[g].d.nOffsets;
+			}
+			CLA_HIP(hipGetLastError());
+			int rc = sdc_upload_desc(b, true);
+			if(rc) return rc;
+		}
 	}
 	*dList = b->dSdcPlan;
 	*dBinOff = b->dSdcPlan + nG;
@@ -475,11 +491,18 @@ int launch_lmm_sdc_tiles(cla_block* b, const double* dY, int p, double* dPre, in
 	if(rc) return rc;
 	struct { const std::vector<int32_t>&list, &binOff; } plan{b->sdcList, b->sdcBinOff};
 	if(plan.list.empty()) return 0;
-	// all listed groups single-column with at most 64 tuples, whole-block call: products straight
-	// into dOut, the groups' part of dPre stays zero
-	const bool noPacked = !b->opt.sdcPacked;
-	bool packed = dOut != nullptr && onlyGroup < 0 && !noPacked && b->dSdcPacked != nullptr;
+	// whole-block call on single-column groups: one lane per group on lane-major lists, products straight
+	// into dOut (the groups' part of dPre stays zero)
+	if(dOut != nullptr && onlyGroup < 0 && b->opt.sdcLanes) {
+		const int r = launch_lmm_sdc_lanes(b, dY, p, dOut);
+		if(r <= 0) return r;
+	}
+	// all listed groups single-column with at most 64 tuples, whole-block call: packed lists, products
+	// straight into dOut
+	bool packed = dOut != nullptr && onlyGroup < 0 && b->opt.sdcPacked;
 	for(int g : plan.list) packed &= b->groups[g].d.nColG == 1 && b->groups[g].d.nVals <= 64;
+	if(packed && (rc = sdc_plan(b, onlyGroup, &dList, &dBinOff, true))) return rc;
+	packed &= b->dSdcPacked != nullptr;
 	if(packed) {
 		const int nTiles = (int) ((b->nRows + ST - 1) / ST);
 		int tpb = std::max(1, (nTiles * p + 4 * g_numCU - 1) / (4 * g_numCU));
@@ -538,6 +561,11 @@ int launch_rmm_sdc_tiles(cla_block* b, int q, int constRow, int accumulate, doub
 	if(rc) return rc;
 	struct { const std::vector<int32_t>&list, &binOff; } plan{b->sdcList, b->sdcBinOff};
 	if(plan.list.empty() || b->nRows == 0) return 1;
+	if(q == 1 && b->opt.sdcLanes) { // one lane per group on lane-major lists
+		const int r = launch_rmm_sdc_lanes(b, constRow, accumulate, dOut, dNnz);
+		if(r <= 0) return r;
+	}
+	if(q == 1 && b->opt.sdcPacked && (rc = sdc_plan(b, -1, &dList, &dBinOff, true))) return rc;
 	const size_t ldsMax = (size_t) std::min(g_ldsPerBlock, 160 * 1024) - 2048;
 	// rows per tile: a multiple of the tile-index granularity whose output tile takes at most ~half of LDS
 	int tileRows = ST;
