@@ -32,7 +32,8 @@ namespace cla {
 constexpr int LN_WIN = SDC_TILE;        // rows per window
 constexpr int LN_DICT_MAX = 6144;       // dictionary entries (spares included) of a slab in LDS
 constexpr int LN_YT = LN_WIN + 64;      // window + 64 slots behind it (left: 0.0; right: one dump slot per lane)
-constexpr int LN_PF = 4;                // chunks a lane keeps requested ahead
+constexpr int LN_PF = 4;                // right multiply: chunks a lane keeps requested ahead
+constexpr int LN_NC = 12;               // left multiply: chunks of a window requested a window ahead
 
 struct LaneDesc { // a lane's group, 16 bytes
 	int32_t g;        // index of the group in the block
@@ -167,35 +168,62 @@ __global__ __launch_bounds__(WAVES * 64) void k_lmm_sdc_lanes(const LaneDesc* __
 	const u32x4* base = data + S.dataOff + ln;
 	const int n = S.n;
 	double acc[4] = {0.0, 0.0, 0.0, 0.0};
-	const int w0 = min((run * WAVES + wave) * winPerWave, nWin), w1 = min(w0 + winPerWave, nWin);
-	for(int win = w0; win < w1; win++) {
-		const int64_t r0 = (int64_t) win * LN_WIN;
-		const uint32_t c0 = __builtin_amdgcn_readfirstlane(cst[win]), c1 = __builtin_amdgcn_readfirstlane(cst[win + 1]);
-		u32x4 buf[LN_PF];
+	const int waveU = __builtin_amdgcn_readfirstlane(wave); // (uniform: the chunk starts below come by scalar loads)
+	// this wave's windows: w0, w0 + WAVES, ... below w1 (the block's waves read one stretch of the lists together)
+	const int w1 = min((run + 1) * WAVES * winPerWave, nWin), w0 = min(run * WAVES * winPerWave + waveU, w1);
+	// Requested a window ahead: the window's first LN_NC chunks, the lane's share of the Y window, the chunk range.
+	// Two sets take turns. The window's work is straight-line code on the set (no loads inside: the compiler's
+	// wait counts are exact); chunks behind the first LN_NC (dense lists) come in a plain loop at the end.
+	struct Ahead {
+		u32x4 buf[LN_NC];
+		double y[LN_WIN / 64];
+		uint32_t c0, c1;
+	};
+	auto request = [&](Ahead& A, int win) { // win < w1
+		A.c0 = cst[win];
+		A.c1 = cst[win + 1];
 #pragma unroll
-		for(int j = 0; j < LN_PF; j++) buf[j] = __builtin_nontemporal_load(base + (int64_t) min(c0 + j, c1 - 1) * n); // (every window holds a chunk)
+		for(int j = 0; j < LN_NC; j++) A.buf[j] = *(base + (int64_t) min(A.c0 + j, A.c1 - 1) * n); // (every window holds a chunk)
+		const int64_t r0 = (int64_t) win * LN_WIN;
+#pragma unroll
+		for(int k = 0; k < LN_WIN / 64; k++) A.y[k] = y[min(r0 + k * 64 + lane, nRows - 1)]; // unconditional: a load under a branch is waited for at the branch's end
+	};
+	auto work = [&](Ahead& A, Ahead& B, int win) { // A holds the requests of `win`, B takes those of the wave's next window
+		const int64_t r0 = (int64_t) win * LN_WIN;
 		bool bad = false;
 #pragma unroll
 		for(int k = 0; k < LN_WIN / 64; k++) {
-			const int64_t r = r0 + k * 64 + lane;
-			double v = y[min(r, nRows - 1)]; // unconditional: a load under a branch is waited for at the branch's end
-			v = r < nRows ? v : 0.0;
+			const double v = r0 + k * 64 + lane < nRows ? A.y[k] : 0.0;
 			bad |= !isfinite(v);
 			yt[k * 64 + lane] = v;
 		}
 		const bool careful = __builtin_amdgcn_ballot_w64(bad) != 0;
 		__builtin_amdgcn_wave_barrier(); // LDS serves a wave's accesses in order: the reads below see the window
-		int r = -1;
-		for(uint32_t c = c0; c < c1; c += LN_PF) {
+		const uint32_t c0 = A.c0, c1 = A.c1;
+		u32x4 cur[LN_NC];
 #pragma unroll
-			for(int j = 0; j < LN_PF; j++) {
-				const u32x4 v = buf[j];
-				buf[j] = __builtin_nontemporal_load(base + (int64_t) min(c + j + LN_PF, c1 - 1) * n);
-				if(c + j < c1) {
-					if(careful) ln_lmm_chunk<true>(v, r, yt, dict, spare, acc);
-					else ln_lmm_chunk<false>(v, r, yt, dict, spare, acc);
-				}
+		for(int j = 0; j < LN_NC; j++) cur[j] = A.buf[j];
+		request(B, win + WAVES < w1 ? win + WAVES : win);
+		int r = -1;
+#pragma unroll
+		for(int j = 0; j < LN_NC; j++) {
+			if(c0 + j < c1) {
+				if(careful) ln_lmm_chunk<true>(cur[j], r, yt, dict, spare, acc);
+				else ln_lmm_chunk<false>(cur[j], r, yt, dict, spare, acc);
 			}
+		}
+		for(uint32_t c = c0 + LN_NC; c < c1; c++) {
+			const u32x4 v = *(base + (int64_t) c * n);
+			if(careful) ln_lmm_chunk<true>(v, r, yt, dict, spare, acc);
+			else ln_lmm_chunk<false>(v, r, yt, dict, spare, acc);
+		}
+	};
+	if(w0 < w1) {
+		Ahead A, B;
+		request(A, w0);
+		for(int win = w0; win < w1; win += 2 * WAVES) {
+			work(A, B, win);
+			if(win + WAVES < w1) work(B, A, win + WAVES);
 		}
 	}
 	if(lane < n) unsafeAtomicAdd(&out[(size_t) blockIdx.y * nCols + L.col0], (acc[0] + acc[1]) + (acc[2] + acc[3]));
@@ -404,10 +432,13 @@ static int lanes_plan(cla_block* b) {
 	return 0;
 }
 
-static int lanes_waves(const cla_block* b, size_t* lds) {
+// Waves per block (one block per CU): as many of 16, 12, 8, 4 as `most` and the LDS windows next to the dictionaries allow.
+static int lanes_waves(const cla_block* b, int most, size_t* lds) {
 	const size_t ldsMax = (size_t) std::min(g_ldsPerBlock, 160 * 1024);
 	const size_t fixed = sizeof(double) * (size_t) b->laneDictLds, perWave = sizeof(double) * LN_YT;
-	const int waves = fixed + 16 * perWave <= ldsMax ? 16 : fixed + 12 * perWave <= ldsMax ? 12 : fixed + 8 * perWave <= ldsMax ? 8 : 4;
+	int waves = 4;
+	for(int w : {16, 12, 8})
+		if(w <= most && fixed + w * perWave <= ldsMax) { waves = w; break; }
 	*lds = fixed + waves * perWave;
 	return *lds <= ldsMax ? waves : 0;
 }
@@ -419,7 +450,7 @@ int launch_lmm_sdc_lanes(cla_block* b, const double* dY, int p, double* dOut) {
 	if(rc) return rc;
 	if(b->laneState != 1 || !b->laneLmm || p > 65535) return 1;
 	size_t lds = 0;
-	const int waves = lanes_waves(b, &lds);
+	const int waves = lanes_waves(b, 8, &lds); // (the kernel's registers allow two waves per SIMD)
 	if(waves == 0) return 1;
 	const int nWin = (int) ((b->nRows + LN_WIN - 1) / LN_WIN), nS = b->laneSlabs;
 	// about one block per CU, every wave a run of windows
@@ -437,7 +468,7 @@ int launch_lmm_sdc_lanes(cla_block* b, const double* dY, int p, double* dOut) {
 			(const uint32_t*) (meta + b->laneOff[3]), (const u32x4*) b->dLaneData, dY, b->nRows, nWin, wpw, dOut, b->nCols);
 		return 0;
 	};
-	rc = waves == 16 ? go(k_lmm_sdc_lanes<16>) : waves == 12 ? go(k_lmm_sdc_lanes<12>) : waves == 8 ? go(k_lmm_sdc_lanes<8>) : go(k_lmm_sdc_lanes<4>);
+	rc = waves == 8 ? go(k_lmm_sdc_lanes<8>) : go(k_lmm_sdc_lanes<4>);
 	if(rc) return rc;
 	CLA_HIP(hipGetLastError());
 	return 0;
@@ -449,7 +480,7 @@ int launch_rmm_sdc_lanes(cla_block* b, int constRow, int accumulate, double* dOu
 	if(rc) return rc;
 	if(b->laneState != 1) return 1;
 	size_t lds = 0;
-	const int waves = lanes_waves(b, &lds);
+	const int waves = lanes_waves(b, 16, &lds);
 	if(waves == 0) return 1;
 	const int nWin = (int) ((b->nRows + LN_WIN - 1) / LN_WIN), nS = b->laneSlabs;
 	// one block per CU and round; whole rounds of the block's waves
