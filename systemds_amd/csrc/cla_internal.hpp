@@ -164,7 +164,7 @@ struct cla_block {
 	void* dLaneMeta = nullptr;       // lane-per-group kernels (k_sdc_lanes.hip): descriptors, slabs, dictionaries, table index, chunk starts
 	void* dLaneData = nullptr;       // the listed groups' lists as lane-major windows, built on first use
 	int laneState = 0;               // 0 not planned yet, 1 ready, -1 the lists do not fit these kernels
-	int laneSlabs = 0, laneDictLds = 0;
+	int laneSlabs = 0, laneDictLds = 0, laneDictTotal = 0; // slabs, dictionary entries of the largest slab / of all
 	size_t laneOff[4] = {0, 0, 0, 0};
 	bool laneLmm = false;            // every listed group has one column (the left multiply's condition)
 	bool sdcPackFailed = false;

@@ -4,23 +4,26 @@
 //   k_lmm_sdc_lanes   out[col(g)] += sum over the listed rows of Y[row] * dict_g[code]   (t(v) %*% X)
 //   k_rmm_sdc_lanes   out[row] += T_g[code] for every listed row                          (X %*% u)
 //
-// The groups are sorted by list length and cut into slabs of up to 64; a wave owns a slab, lane l
-// owns the slab's group l. Rows are cut into windows of LN_WIN. For a (slab, window) every lane's
-// entries inside the window are stored as slots of (row delta, code), one byte each, eight slots
-// per 16-byte chunk, the chunks of the slab's lanes side by side: one 16-byte load per lane brings
-// eight entries of every group of the slab, fully coalesced, and a lane decodes its list with a
-// running row - no prefix sums across lanes, no bins, no cross-lane traffic.
+// The groups are sorted by list length and cut into slabs of up to 64; lane l of a wave owns
+// the slab's group l. Rows are cut into windows of LN_WIN. For a (slab, window) every lane's
+// entries inside the window are stored in chunks of 16 bytes that hold seven entries - the row
+// of the first (16 bits, relative to the window), six row deltas and seven codes, one byte
+// each - and the chunks of the slab's lanes lie side by side: one 16-byte load per lane brings
+// seven entries of every group of the slab, fully coalesced. A chunk row stands for itself
+// (it carries its rows), so the right multiply's waves share the chunk rows of a block's
+// windows among them; a lane decodes its entries with a running row - no prefix sums across
+// lanes, no bins, no cross-lane traffic.
 //
-// Slot encoding: delta 1..255 = rows since the previous slot (since row -1 of the window for the first), code =
-// tuple index; a gap of more than 255 rows takes slots of (255, spare) first, where the spare code nVals maps to a
-// 0.0 behind the group's dictionary (or table); lanes with fewer slots than the longest of the slab are padded
-// with (0, spare). The windows' chunk counts are the maxima over the slab's lanes (sorting by list length keeps
-// them close to the lanes' own counts).
+// Chunk of a lane: word 0 = first row | delta 1 << 16 | delta 2 << 24, word 1 = deltas 3..6, words 2 and 3 = codes
+// 0..6 and, in the last byte, the window's index modulo LN_G (its place in a round of the right multiply). A gap of more than 255 rows inside a chunk takes entries of (255, spare) first, where the spare code nVals
+// maps to a 0.0 behind the group's dictionary (or table); a chunk's unused entries are (0, spare), a lane's unused
+// chunks start at row 0xffff. The chunk rows of a window are as many as its longest lane needs (sorting the groups
+// by list length keeps that close to what the others need).
 //
-// Left multiply: the Y window sits in LDS with a 0.0 at index LN_WIN, every slot adds
-// Y[min(row, LN_WIN)] * dict[code] to the lane's sum (spare slots add Y[row] * 0.0; a window of Y with non-finite
-// values takes the variant that sends spare slots to the 0.0 instead). Right multiply: the output window sits in
-// LDS, every slot adds T[code] at its row with an LDS atomic (spare slots add their 0.0 to a dump slot per lane); the slabs take turns on the block's windows, their tables staged in LDS one after the other.
+// Left multiply: every wave holds the Y window it works on in LDS, with a 0.0 behind it at index LN_WIN; every
+// entry adds Y[min(row, LN_WIN)] * dict[code] to the lane's sum (spare entries add Y[row] * 0.0; a
+// window of Y with non-finite values takes the variant that sends spare entries to the 0.0 instead). Right
+// multiply: LN_G output windows sit in LDS, every entry with a tuple adds T[code] at its row with an LDS atomic; the slabs take turns, their tables in LDS in two buffers.
 #include "../../include/cla_hip.h"
 #include "cla_device.hpp"
 #include <algorithm>
@@ -29,11 +32,18 @@
 
 namespace cla {
 
-constexpr int LN_WIN = SDC_TILE;        // rows per window
-constexpr int LN_DICT_MAX = 6144;       // dictionary entries (spares included) of a slab in LDS
-constexpr int LN_YT = LN_WIN + 64;      // window + 64 slots behind it (left: 0.0; right: one dump slot per lane)
-constexpr int LN_PF = 4;                // right multiply: chunks a lane keeps requested ahead
-constexpr int LN_NC = 12;               // left multiply: chunks of a window requested a window ahead
+constexpr int LN_TPW = 1;                  // row tiles (SDC_TILE rows) per window
+constexpr int LN_WIN = LN_TPW * SDC_TILE;  // rows per window
+constexpr int LN_E = 7;                    // entries per chunk
+constexpr int LN_DICT_MAX = 6016;          // dictionary entries (spares included) of a slab in LDS (right: two buffers next to the output windows)
+constexpr int LN_YT = LN_WIN + 64;         // left: Y window + 64 slots of 0.0 behind it
+constexpr int LN_LW = 8;                   // left: waves per block, each on windows of its own
+constexpr int LN_LK = 12;                  // left: chunk rows of a window requested a window ahead
+constexpr int LN_RW = 16;                  // right: waves per block
+constexpr int LN_G = 4;                    // right: output windows per block and round
+constexpr int LN_RK = 6;                   // right: chunk rows per wave and (slab, round) requested a turn ahead
+constexpr int LN_TMAX = (LN_DICT_MAX + LN_RW * 64 - 1) / (LN_RW * 64); // right: table entries per thread
+static_assert(LN_WIN <= 0x7fff, "a chunk's first row is 16 bits, 0xffff marks an unused chunk");
 
 struct LaneDesc { // a lane's group, 16 bytes
 	int32_t g;        // index of the group in the block
@@ -46,12 +56,13 @@ struct LaneSlab { // 32 bytes
 	int32_t l0, n;             // lanes desc[l0 .. l0 + n)
 	int32_t dictOff, dictLen;  // their dictionaries inside the concatenation
 	int64_t dataOff;           // first chunk of the slab, in 16-byte units
-	int64_t chunkOff;          // the slab's nWin + 1 chunk starts inside chunkStart
+	int64_t chunkOff;          // the slab's nWin + 1 chunk-row starts inside chunkStart
 };
 
 // ---------------------------------------------------------------------------------------------
 // Conversion. thread = (window, lane of the slab): walks the group's list inside the window from the row-tile
-// index and counts (FILL == false: maximum over the slab's lanes into slotMax) or writes (FILL == true) its slots.
+// index and counts its entries (FILL == false: maximum over the slab's lanes into slotMax) or writes its chunks
+// (FILL == true).
 // ---------------------------------------------------------------------------------------------
 template <bool FILL>
 __global__ __launch_bounds__(256) void k_lane_convert(const DGroup* __restrict__ groups, const LaneDesc* __restrict__ desc,
@@ -65,35 +76,41 @@ __global__ __launch_bounds__(256) void k_lane_convert(const DGroup* __restrict__
 	const DGroup G = dgroup(groups + L.g);
 	const int64_t r0 = (int64_t) win * LN_WIN, rEnd = r0 + LN_WIN;
 	const uint32_t spare = (uint32_t) L.spare;
+	const uint32_t spare4 = spare * 0x01010101u;
 	uint32_t cs = 0, nChunks = 0;
 	if(FILL) {
 		cs = chunkStart[S.chunkOff + win];
 		nChunks = chunkStart[S.chunkOff + win + 1] - cs;
 	}
 	u32x4* dst = data + S.dataOff + (int64_t) cs * S.n + lane;
-	int cnt = 0, prev = -1;
+	int cnt = 0, prev = -1; // prev: row of the previous entry
 	uint64_t dby = 0, cby = 0;
-	auto slot = [&](uint32_t d, uint32_t c) {
+	auto flush = [&]() { // the chunk that holds entries cnt - (cnt % LN_E) .. (whole or partial)
+		const int p = cnt % LN_E == 0 ? LN_E : cnt % LN_E;
+		for(int t = p; t < LN_E; t++) cby |= (uint64_t) spare << (8 * t);
+		cby |= (uint64_t) (win & (LN_G - 1)) << 56;
+		u32x4 v = {(uint32_t) dby, (uint32_t) (dby >> 32), (uint32_t) cby, (uint32_t) (cby >> 32)};
+		dst[(int64_t) ((cnt - 1) / LN_E) * S.n] = v;
+		dby = 0; cby = 0;
+	};
+	auto put = [&](int row, uint32_t c) {
 		if(FILL) {
-			dby |= (uint64_t) d << (8 * (cnt & 7));
-			cby |= (uint64_t) c << (8 * (cnt & 7));
-			if((cnt & 7) == 7) {
-				u32x4 v = {(uint32_t) dby, (uint32_t) (dby >> 32), (uint32_t) cby, (uint32_t) (cby >> 32)};
-				dst[(int64_t) (cnt >> 3) * S.n] = v;
-				dby = 0; cby = 0;
-			}
+			const int p = cnt % LN_E;
+			if(p == 0) dby = (uint64_t) (uint32_t) row;
+			else dby |= (uint64_t) (uint32_t) (row - prev) << (8 * (p + 1));
+			cby |= (uint64_t) c << (8 * p);
 		}
+		prev = row;
 		cnt++;
+		if(FILL && cnt % LN_E == 0) flush();
 	};
 	auto entry = [&](int rel, int di) {
-		int gap = rel - prev;
-		while(gap > 255) { slot(255u, spare); gap -= 255; }
-		slot((uint32_t) gap, (uint32_t) load_code(G.codes, G.codeWidth, di));
-		prev = rel;
+		while(cnt % LN_E != 0 && rel - prev > 255) put(prev + 255, spare);
+		put(rel, (uint32_t) load_code(G.codes, G.codeWidth, di));
 	};
 	if(G.first >= r0 && G.first < rEnd) entry((int) (G.first - r0), 0);
-	if(win < G.nTiles) {
-		const OffState st = G.tileIdx[win];
+	if(win * LN_TPW < G.nTiles) {
+		const OffState st = G.tileIdx[win * LN_TPW];
 		int64_t i = st.idx;
 		int32_t row = st.row, emit = st.emit;
 		const int maxV = G.deltaWidth == 1 ? 255 : 65535;
@@ -109,46 +126,53 @@ __global__ __launch_bounds__(256) void k_lane_convert(const DGroup* __restrict__
 		}
 	}
 	if(FILL) {
-		while(cnt < (int) nChunks * 8) slot(0u, spare);
+		if(cnt % LN_E != 0) flush();
+		const u32x4 none = {0xffffu, 0u, spare4, (spare4 & 0x00ffffffu) | (uint32_t) (win & (LN_G - 1)) << 24};
+		for(uint32_t k = (uint32_t) (cnt + LN_E - 1) / LN_E; k < nChunks; k++) dst[(int64_t) k * S.n] = none;
 	}
 	else atomicMax(&slotMax[(int64_t) blockIdx.y * nWin + win], (uint32_t) cnt);
 }
 
+// The seven rows (relative to the window; may lie behind it for unused chunks) and codes of a chunk.
+__device__ __forceinline__ void ln_decode(const u32x4 v, uint32_t (&row)[LN_E], uint32_t (&code)[LN_E]) {
+	row[0] = v.x & 0xffffu;
+	row[1] = row[0] + ((v.x >> 16) & 0xffu);
+	row[2] = row[1] + (v.x >> 24);
+#pragma unroll
+	for(int t = 3; t < LN_E; t++) row[t] = row[t - 1] + ((v.y >> (8 * (t - 3))) & 0xffu);
+#pragma unroll
+	for(int t = 0; t < LN_E; t++) code[t] = ((t < 4 ? v.z : v.w) >> (8 * (t & 3))) & 0xffu;
+}
+
 // ---------------------------------------------------------------------------------------------
-// Left multiply.
+// Left multiply. block = (run of windows, slab, row of Y); every wave works on windows of its own.
 // ---------------------------------------------------------------------------------------------
-// Eight slots of one lane. r = row of the previous slot, relative to the window.
 template <bool CAREFUL>
-__device__ __forceinline__ void ln_lmm_chunk(const u32x4 v, int& r, const double* yt, const double* dict, uint32_t spare,
+__device__ __forceinline__ void ln_lmm_chunk(const u32x4 v, const double* yt, const double* dict, uint32_t spare,
 	double (&acc)[4]) {
-	uint32_t idx[8], code[8];
+	uint32_t row[LN_E], code[LN_E];
+	ln_decode(v, row, code);
+	double yv[LN_E], dv[LN_E];
 #pragma unroll
-	for(int t = 0; t < 8; t++) {
-		const uint32_t dw = t < 4 ? v.x : v.y, cw = t < 4 ? v.z : v.w;
-		r += (int) ((dw >> (8 * (t & 3))) & 0xffu);
-		code[t] = (cw >> (8 * (t & 3))) & 0xffu;
-		idx[t] = min((uint32_t) r, (uint32_t) LN_WIN);
-		if(CAREFUL) idx[t] = code[t] == spare ? (uint32_t) LN_WIN : idx[t];
-	}
-	double yv[8], dv[8];
-#pragma unroll
-	for(int t = 0; t < 8; t++) {
-		yv[t] = yt[idx[t]];
+	for(int t = 0; t < LN_E; t++) {
+		uint32_t idx = min(row[t], (uint32_t) LN_WIN);
+		if(CAREFUL) idx = code[t] == spare ? (uint32_t) LN_WIN : idx;
+		yv[t] = yt[idx];
 		dv[t] = dict[code[t]];
 	}
 #pragma unroll
-	for(int t = 0; t < 8; t++) acc[t & 3] = __builtin_fma(yv[t], dv[t], acc[t & 3]);
+	for(int t = 0; t < LN_E; t++) acc[t & 3] = __builtin_fma(yv[t], dv[t], acc[t & 3]);
 }
 
-template <int WAVES>
-__global__ __launch_bounds__(WAVES * 64) void k_lmm_sdc_lanes(const LaneDesc* __restrict__ desc,
+__global__ __launch_bounds__(LN_LW * 64) void k_lmm_sdc_lanes(const LaneDesc* __restrict__ desc,
 	const LaneSlab* __restrict__ slabs, int nSlabs, const double* __restrict__ dictAll, int dictLds,
 	const uint32_t* __restrict__ chunkStart, const u32x4* __restrict__ data, const double* __restrict__ Y, int64_t nRows,
 	int nWin, int winPerWave, double* __restrict__ out, int nCols) {
 	extern __shared__ double smem[];
 	double* dictL = smem; // the slab's dictionaries
-	const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-	double* yt = smem + dictLds + wave * LN_YT;
+	const int tid = threadIdx.x, lane = tid & 63;
+	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6); // (uniform: the chunk starts below come by scalar loads)
+	double* yt = smem + dictLds + wave * LN_YT; // this wave's Y window
 	// Blocks go round the 8 XCDs by their index. The slabs of a run of windows read the same part of Y: they sit 8
 	// block indices apart, on one XCD and close in time, so that its L2 fetches that part of Y once.
 	const int nRuns = gridDim.x / nSlabs;
@@ -156,7 +180,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_lmm_sdc_lanes(const LaneDesc* __
 	const int inLast = nRuns - grp * 8 < 8 ? nRuns - grp * 8 : 8; // runs of the last, partial period
 	const int slab = in / inLast, run = grp * 8 + in % inLast;
 	const LaneSlab S = slabs[slab];
-	for(int k = tid; k < S.dictLen; k += WAVES * 64) dictL[k] = dictAll[S.dictOff + k];
+	for(int k = tid; k < S.dictLen; k += LN_LW * 64) dictL[k] = dictAll[S.dictOff + k];
 	yt[LN_WIN + lane] = 0.0;
 	__syncthreads();
 	const int ln = min(lane, S.n - 1); // lanes behind the slab's last repeat it, their sums are dropped
@@ -168,14 +192,13 @@ __global__ __launch_bounds__(WAVES * 64) void k_lmm_sdc_lanes(const LaneDesc* __
 	const u32x4* base = data + S.dataOff + ln;
 	const int n = S.n;
 	double acc[4] = {0.0, 0.0, 0.0, 0.0};
-	const int waveU = __builtin_amdgcn_readfirstlane(wave); // (uniform: the chunk starts below come by scalar loads)
-	// this wave's windows: w0, w0 + WAVES, ... below w1 (the block's waves read one stretch of the lists together)
-	const int w1 = min((run + 1) * WAVES * winPerWave, nWin), w0 = min(run * WAVES * winPerWave + waveU, w1);
-	// Requested a window ahead: the window's first LN_NC chunks, the lane's share of the Y window, the chunk range.
-	// Two sets take turns. The window's work is straight-line code on the set (no loads inside: the compiler's
-	// wait counts are exact); chunks behind the first LN_NC (dense lists) come in a plain loop at the end.
+	// this wave's windows: w0, w0 + LN_LW, ... below w1 (the block's waves read one stretch of the lists together)
+	const int w1 = min((run + 1) * LN_LW * winPerWave, nWin), w0 = min(run * LN_LW * winPerWave + wave, w1);
+	// Requested a window ahead: the window's first LN_LK chunk rows, the lane's share of the Y window, the chunk
+	// range. Two sets take turns. The window's work is straight-line code on the set (no loads inside: the compiler's
+	// wait counts are exact); chunk rows behind the first LN_LK (dense lists) come in a plain loop at the end.
 	struct Ahead {
-		u32x4 buf[LN_NC];
+		u32x4 buf[LN_LK];
 		double y[LN_WIN / 64];
 		uint32_t c0, c1;
 	};
@@ -183,7 +206,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_lmm_sdc_lanes(const LaneDesc* __
 		A.c0 = cst[win];
 		A.c1 = cst[win + 1];
 #pragma unroll
-		for(int j = 0; j < LN_NC; j++) A.buf[j] = *(base + (int64_t) min(A.c0 + j, A.c1 - 1) * n); // (every window holds a chunk)
+		for(int j = 0; j < LN_LK; j++) A.buf[j] = *(base + (int64_t) min(A.c0 + j, A.c1 - 1) * n); // (every window holds a chunk row)
 		const int64_t r0 = (int64_t) win * LN_WIN;
 #pragma unroll
 		for(int k = 0; k < LN_WIN / 64; k++) A.y[k] = y[min(r0 + k * 64 + lane, nRows - 1)]; // unconditional: a load under a branch is waited for at the branch's end
@@ -200,121 +223,157 @@ __global__ __launch_bounds__(WAVES * 64) void k_lmm_sdc_lanes(const LaneDesc* __
 		const bool careful = __builtin_amdgcn_ballot_w64(bad) != 0;
 		__builtin_amdgcn_wave_barrier(); // LDS serves a wave's accesses in order: the reads below see the window
 		const uint32_t c0 = A.c0, c1 = A.c1;
-		u32x4 cur[LN_NC];
+		u32x4 cur[LN_LK];
 #pragma unroll
-		for(int j = 0; j < LN_NC; j++) cur[j] = A.buf[j];
-		request(B, win + WAVES < w1 ? win + WAVES : win);
-		int r = -1;
+		for(int j = 0; j < LN_LK; j++) cur[j] = A.buf[j];
+		request(B, win + LN_LW < w1 ? win + LN_LW : win);
 #pragma unroll
-		for(int j = 0; j < LN_NC; j++) {
+		for(int j = 0; j < LN_LK; j++) {
 			if(c0 + j < c1) {
-				if(careful) ln_lmm_chunk<true>(cur[j], r, yt, dict, spare, acc);
-				else ln_lmm_chunk<false>(cur[j], r, yt, dict, spare, acc);
+				if(careful) ln_lmm_chunk<true>(cur[j], yt, dict, spare, acc);
+				else ln_lmm_chunk<false>(cur[j], yt, dict, spare, acc);
 			}
 		}
-		for(uint32_t c = c0 + LN_NC; c < c1; c++) {
+		for(uint32_t c = c0 + LN_LK; c < c1; c++) {
 			const u32x4 v = *(base + (int64_t) c * n);
-			if(careful) ln_lmm_chunk<true>(v, r, yt, dict, spare, acc);
-			else ln_lmm_chunk<false>(v, r, yt, dict, spare, acc);
+			if(careful) ln_lmm_chunk<true>(v, yt, dict, spare, acc);
+			else ln_lmm_chunk<false>(v, yt, dict, spare, acc);
 		}
 	};
 	if(w0 < w1) {
 		Ahead A, B;
 		request(A, w0);
-		for(int win = w0; win < w1; win += 2 * WAVES) {
+		for(int win = w0; win < w1; win += 2 * LN_LW) {
 			work(A, B, win);
-			if(win + WAVES < w1) work(B, A, win + WAVES);
+			if(win + LN_LW < w1) work(B, A, win + LN_LW);
 		}
 	}
 	if(lane < n) unsafeAtomicAdd(&out[(size_t) blockIdx.y * nCols + L.col0], (acc[0] + acc[1]) + (acc[2] + acc[3]));
 }
 
 // ---------------------------------------------------------------------------------------------
-// Right multiply with one output column. block = run of windows; per round every wave takes one window, and the
-// slabs take turns: tables of slab s into LDS (T gathered through tblIndex, -1 = the 0.0 of a spare code), every
-// wave adds the slab's slots of its window. accumulate == 0: a window starts from constRow (or zero) and is the
-// whole result; accumulate != 0: it starts from what other groups already wrote.
+// Right multiply with one output column. block = run of windows, in rounds of LN_G windows whose output sits in
+// LDS. In a round the slabs take turns; the block's waves share the chunk rows of the slab's LN_G windows. The
+// tables of the next turn's slab (T gathered through tblIndex, -1 = the 0.0 of a spare code) are fetched during a
+// turn and stored into the other table buffer behind it. accumulate == 0: a window starts from constRow (or zero)
+// and is the whole result; accumulate != 0: it starts from what other groups already wrote.
 // ---------------------------------------------------------------------------------------------
-template <int WAVES>
-__global__ __launch_bounds__(WAVES * 64) void k_rmm_sdc_lanes(const LaneDesc* __restrict__ desc,
-	const LaneSlab* __restrict__ slabs, int nSlabs, const int32_t* __restrict__ tblIndex, int dictLds,
+template <bool RESIDENT>
+__global__ __launch_bounds__(LN_RW * 64) void k_rmm_sdc_lanes(const LaneDesc* __restrict__ desc,
+	const LaneSlab* __restrict__ slabs, int nSlabs, const int32_t* __restrict__ tblIndex, int dictLds, int dictTotal,
 	const uint32_t* __restrict__ chunkStart, const u32x4* __restrict__ data, const double* __restrict__ T, int constRow,
 	int accumulate, double* __restrict__ out, int64_t nRows, int nWin, int winPerBlock, unsigned long long* __restrict__ nnz) {
 	extern __shared__ double smem[];
-	double* tblL = smem;
-	const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-	double* ot = smem + dictLds + wave * LN_YT;
-	const int wBeg = blockIdx.x * winPerBlock, wEnd = min(wBeg + winPerBlock, nWin);
+	double* tblAll = smem;                 // RESIDENT: the tables of all slabs (dictTotal entries); else two buffers of dictLds entries
+	double* ot = smem + (RESIDENT ? dictTotal : 2 * dictLds); // LN_G windows of output
+	const int tid = threadIdx.x, lane = tid & 63;
+	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+	constexpr int THREADS = LN_RW * 64, OPT = LN_G * LN_WIN / THREADS;
+	const int wBeg = min((int) blockIdx.x * winPerBlock, nWin), wEnd = min(wBeg + winPerBlock, nWin);
+	if(wBeg >= wEnd) return;
 	const double init = !accumulate && constRow >= 0 ? T[constRow] : 0.0;
+	const int nRounds = (wEnd - wBeg + LN_G - 1) / LN_G, nTurns = nRounds * nSlabs;
+	double treg[LN_TMAX];
+	auto tbl_request = [&](int s) {
+		const LaneSlab S = slabs[s];
+#pragma unroll
+		for(int k = 0; k < LN_TMAX; k++) {
+			const int e = k * THREADS + tid;
+			const int32_t ti = tblIndex[S.dictOff + min(e, S.dictLen - 1)];
+			treg[k] = T[max(ti, 0)];
+			treg[k] = ti >= 0 ? treg[k] : 0.0;
+		}
+	};
+	auto tbl_store = [&](int turn) {
+		double* tb = tblAll + (nSlabs > 1 ? turn & 1 : 0) * dictLds; // (one slab: its tables stay)
+#pragma unroll
+		for(int k = 0; k < LN_TMAX; k++)
+			if(k * THREADS + tid < dictLds) tb[k * THREADS + tid] = treg[k];
+	};
+	struct Ahead {
+		u32x4 buf[LN_RK];
+		uint32_t c0, c1; // this wave's first chunk row of the turn, end of the turn's chunk rows
+	};
+	auto request = [&](Ahead& A, int turn) { // turn < nTurns
+		const int s = turn % nSlabs, wg = wBeg + (turn / nSlabs) * LN_G;
+		const LaneSlab S = slabs[s];
+		const uint32_t* cst = chunkStart + S.chunkOff;
+		A.c0 = cst[wg] + wave;
+		A.c1 = cst[min(wg + LN_G, wEnd)];
+		const u32x4* base = data + S.dataOff + min(lane, S.n - 1);
+#pragma unroll
+		for(int j = 0; j < LN_RK; j++) A.buf[j] = *(base + (int64_t) min(A.c0 + j * LN_RW, A.c1 - 1) * S.n);
+	};
+	auto add_chunk = [&](const u32x4 v, const double* tbl, uint32_t spare) {
+		const uint32_t off = (v.w >> 24) * (uint32_t) LN_WIN; // the chunk row's window inside the round (rounds start at multiples of LN_G)
+		uint32_t row[LN_E], code[LN_E];
+		ln_decode(v, row, code);
+		double tv[LN_E];
+#pragma unroll
+		for(int t = 0; t < LN_E; t++) tv[t] = tbl[code[t]];
+		// (LDS adds of doubles take about a cycle per lane: spare entries stay out of them; an entry with a tuple
+		// lies inside its window)
+#pragma unroll
+		for(int t = 0; t < LN_E; t++)
+			if(code[t] != spare) unsafeAtomicAdd(&ot[row[t] + off], tv[t]);
+	};
 	int cntNz = 0;
-	for(int wb = wBeg; wb < wEnd; wb += WAVES) { // the same trip count for every wave: barriers inside
-		const int win = wb + wave;
-		const bool on = win < wEnd;
-		const int64_t r0 = (int64_t) win * LN_WIN;
-		if(on && accumulate) {
+	auto work = [&](Ahead& A, Ahead& B, int turn) {
+		const int s = turn % nSlabs, round = turn / nSlabs, wg = wBeg + round * LN_G;
+		if(s == 0) { // a new round: the output windows start from their initial values
 #pragma unroll
-			for(int k = 0; k < LN_WIN / 64; k++) ot[k * 64 + lane] = out[min(r0 + k * 64 + lane, nRows - 1)]; // (unconditional loads)
-		}
-		else if(on) {
-#pragma unroll
-			for(int k = 0; k < LN_WIN / 64; k++) ot[k * 64 + lane] = init;
-		}
-		for(int s = 0; s < nSlabs; s++) {
-			const LaneSlab S = slabs[s];
-			__syncthreads(); // the previous slab's tables are no longer read
-			for(int k = tid; k < S.dictLen; k += WAVES * 64) {
-				const int32_t ti = tblIndex[S.dictOff + k];
-				tblL[k] = ti >= 0 ? T[ti] : 0.0;
+			for(int k = 0; k < OPT; k++) {
+				const int64_t r = (int64_t) wg * LN_WIN + k * THREADS + tid;
+				ot[k * THREADS + tid] = accumulate ? out[min(r, nRows - 1)] : init;
 			}
 			__syncthreads();
-			if(!on) continue;
-			const int ln = min(lane, S.n - 1);
-			const LaneDesc L = desc[S.l0 + ln];
-			const double* tbl = tblL + L.dictOff;
-			const uint32_t spare = (uint32_t) L.spare;
-			const uint32_t* cst = chunkStart + S.chunkOff;
-			const u32x4* base = data + S.dataOff + ln;
-			const int n = S.n;
-			const uint32_t c0 = __builtin_amdgcn_readfirstlane(cst[win]), c1 = __builtin_amdgcn_readfirstlane(cst[win + 1]);
-			u32x4 buf[LN_PF];
-#pragma unroll
-			for(int j = 0; j < LN_PF; j++) buf[j] = __builtin_nontemporal_load(base + (int64_t) min(c0 + j, c1 - 1) * n);
-			int r = -1;
-			const uint32_t dump = (uint32_t) (LN_WIN + lane);
-			for(uint32_t c = c0; c < c1; c += LN_PF) {
-#pragma unroll
-				for(int j = 0; j < LN_PF; j++) {
-					const u32x4 v = buf[j];
-					buf[j] = __builtin_nontemporal_load(base + (int64_t) min(c + j + LN_PF, c1 - 1) * n);
-					if(c + j < c1 && lane < n) {
-						double tv[8];
-						uint32_t idx[8];
-#pragma unroll
-						for(int t = 0; t < 8; t++) {
-							const uint32_t dw = t < 4 ? v.x : v.y, cw = t < 4 ? v.z : v.w;
-							r += (int) ((dw >> (8 * (t & 3))) & 0xffu);
-							const uint32_t code = (cw >> (8 * (t & 3))) & 0xffu;
-							idx[t] = code != spare ? (uint32_t) r : dump; // (a slot with a tuple lies inside the window)
-							tv[t] = tbl[code];
-						}
-#pragma unroll
-						for(int t = 0; t < 8; t++) unsafeAtomicAdd(&ot[idx[t]], tv[t]);
-					}
-				}
-			}
 		}
-		if(on) {
-			__builtin_amdgcn_wave_barrier();
+		const int next = turn + 1 < nTurns ? turn + 1 : turn;
+		if(!RESIDENT && nSlabs > 1) tbl_request(next % nSlabs);
+		request(B, next);
+		const LaneSlab S = slabs[s];
+		const LaneDesc L = desc[S.l0 + min(lane, S.n - 1)];
+		const double* tbl = tblAll + (RESIDENT ? S.dictOff : (nSlabs > 1 ? turn & 1 : 0) * dictLds) + L.dictOff;
+		const uint32_t spare = (uint32_t) L.spare;
+		const u32x4* base = data + S.dataOff + min(lane, S.n - 1);
+		const uint32_t c0 = A.c0, c1 = A.c1;
+		if(lane < S.n) {
 #pragma unroll
-			for(int k = 0; k < LN_WIN / 64; k++) {
-				const int64_t r = r0 + k * 64 + lane;
-				if(r < nRows) {
-					const double v = ot[k * 64 + lane];
+			for(int j = 0; j < LN_RK; j++)
+				if(c0 + j * LN_RW < c1) add_chunk(A.buf[j], tbl, spare);
+			for(uint32_t c = c0 + LN_RK * LN_RW; c < c1; c += LN_RW) add_chunk(*(base + (int64_t) c * S.n), tbl, spare);
+		}
+		if(!RESIDENT && nSlabs > 1) tbl_store(turn + 1); // the other buffer was last read before the previous barrier
+		if(!RESIDENT || s == nSlabs - 1) __syncthreads(); // (resident tables: the waves only meet at the ends of a round)
+		if(s == nSlabs - 1) { // the round's windows are complete
+#pragma unroll
+			for(int k = 0; k < OPT; k++) {
+				const int64_t r = (int64_t) wg * LN_WIN + k * THREADS + tid;
+				if(r < nRows && r < (int64_t) wEnd * LN_WIN) {
+					const double v = ot[k * THREADS + tid];
 					cntNz += v != 0.0;
 					out[r] = v;
 				}
 			}
+			// (the next round's initial values are written by the same threads to the same slots)
 		}
+	};
+	if(RESIDENT) {
+		for(int k = tid; k < dictTotal; k += THREADS) {
+			const int32_t ti = tblIndex[k];
+			tblAll[k] = ti >= 0 ? T[ti] : 0.0;
+		}
+	}
+	else {
+		tbl_request(0);
+		tbl_store(0);
+	}
+	Ahead A, B;
+	request(A, 0);
+	// (the first round's barrier behind the initial values also orders the first tables)
+	for(int turn = 0; turn < nTurns; turn += 2) {
+		work(A, B, turn);
+		if(turn + 1 < nTurns) work(B, A, turn + 1);
 	}
 	count_add(nnz, cntNz);
 }
@@ -404,7 +463,7 @@ static int lanes_plan(cla_block* b) {
 		uint64_t c = 0;
 		for(int w = 0; w < nWin; w++) {
 			cs[(size_t) s * (nWin + 1) + w] = (uint32_t) c;
-			c += std::max<uint32_t>(1, (slotMax[(size_t) s * nWin + w] + 7) / 8); // at least one chunk: the kernels' loads are unconditional
+			c += std::max<uint32_t>(1, (slotMax[(size_t) s * nWin + w] + LN_E - 1) / LN_E); // at least one chunk row: the kernels' loads are unconditional
 		}
 		if(c > 0xffffffffull) return 0;
 		cs[(size_t) s * (nWin + 1) + nWin] = (uint32_t) c;
@@ -425,22 +484,12 @@ static int lanes_plan(cla_block* b) {
 	CLA_HIP(hipStreamSynchronize(st)); // `slabs` and `cs` go out of scope
 	b->laneSlabs = nS;
 	b->laneDictLds = dictLds;
+	b->laneDictTotal = dictOffAll[nL];
 	b->laneOff[0] = descBytes; b->laneOff[1] = descBytes + slabBytes; b->laneOff[2] = descBytes + slabBytes + dictBytes;
 	b->laneOff[3] = descBytes + slabBytes + dictBytes + idxBytes;
 	b->laneLmm = singleCols;
 	b->laneState = 1;
 	return 0;
-}
-
-// Waves per block (one block per CU): as many of 16, 12, 8, 4 as `most` and the LDS windows next to the dictionaries allow.
-static int lanes_waves(const cla_block* b, int most, size_t* lds) {
-	const size_t ldsMax = (size_t) std::min(g_ldsPerBlock, 160 * 1024);
-	const size_t fixed = sizeof(double) * (size_t) b->laneDictLds, perWave = sizeof(double) * LN_YT;
-	int waves = 4;
-	for(int w : {16, 12, 8})
-		if(w <= most && fixed + w * perWave <= ldsMax) { waves = w; break; }
-	*lds = fixed + waves * perWave;
-	return *lds <= ldsMax ? waves : 0;
 }
 
 // t(Y) %*% X of all listed groups straight into dOut. Returns 1 when the block's lists do not fit these kernels
@@ -449,27 +498,21 @@ int launch_lmm_sdc_lanes(cla_block* b, const double* dY, int p, double* dOut) {
 	int rc = lanes_plan(b);
 	if(rc) return rc;
 	if(b->laneState != 1 || !b->laneLmm || p > 65535) return 1;
-	size_t lds = 0;
-	const int waves = lanes_waves(b, 8, &lds); // (the kernel's registers allow two waves per SIMD)
-	if(waves == 0) return 1;
+	const size_t lds = sizeof(double) * ((size_t) b->laneDictLds + LN_LW * LN_YT);
+	if(lds > (size_t) std::min(g_ldsPerBlock, 160 * 1024)) return 1;
 	const int nWin = (int) ((b->nRows + LN_WIN - 1) / LN_WIN), nS = b->laneSlabs;
-	// about one block per CU, every wave a run of windows
+	// about one block per CU (what its registers and LDS allow), every wave a share of the block's run of windows
 	const int64_t runs = std::max<int64_t>(1, (int64_t) g_numCU / ((int64_t) nS * p));
-	const int wpw = (int) std::max<int64_t>(1, (nWin + runs * waves - 1) / (runs * waves));
-	const unsigned nRuns = (unsigned) ((nWin + wpw * waves - 1) / (wpw * waves));
+	const int wpw = (int) std::max<int64_t>(1, (nWin + runs * LN_LW - 1) / (runs * LN_LW));
+	const unsigned nRuns = (unsigned) ((nWin + wpw * LN_LW - 1) / (wpw * LN_LW));
 	char* meta = (char*) b->dLaneMeta;
 	double algo = (double) b->nRows * 8 * p;
 	for(int g : b->sdcList) algo += (double) p * ((double) b->groups[g].d.nDeltas * b->groups[g].d.deltaWidth + (double) b->groups[g].d.nOffsets);
-	Prof pf(b, "k_lmm_sdc_lanes", (long) nRuns * nS * p, waves * 64, (long) lds, algo);
-	auto go = [&](auto kernel) {
-		CLA_HIP(hipFuncSetAttribute((const void*) kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
-		hipLaunchKernelGGL(kernel, dim3(nRuns * nS, p), dim3(waves * 64), lds, b->stream, (const LaneDesc*) meta,
-			(const LaneSlab*) (meta + b->laneOff[0]), nS, (const double*) (meta + b->laneOff[1]), b->laneDictLds,
-			(const uint32_t*) (meta + b->laneOff[3]), (const u32x4*) b->dLaneData, dY, b->nRows, nWin, wpw, dOut, b->nCols);
-		return 0;
-	};
-	rc = waves == 8 ? go(k_lmm_sdc_lanes<8>) : go(k_lmm_sdc_lanes<4>);
-	if(rc) return rc;
+	Prof pf(b, "k_lmm_sdc_lanes", (long) nRuns * nS * p, LN_LW * 64, (long) lds, algo);
+	CLA_HIP(hipFuncSetAttribute((const void*) k_lmm_sdc_lanes, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
+	hipLaunchKernelGGL(k_lmm_sdc_lanes, dim3(nRuns * nS, p), dim3(LN_LW * 64), lds, b->stream, (const LaneDesc*) meta,
+		(const LaneSlab*) (meta + b->laneOff[0]), nS, (const double*) (meta + b->laneOff[1]), b->laneDictLds,
+		(const uint32_t*) (meta + b->laneOff[3]), (const u32x4*) b->dLaneData, dY, b->nRows, nWin, wpw, dOut, b->nCols);
 	CLA_HIP(hipGetLastError());
 	return 0;
 }
@@ -479,28 +522,29 @@ int launch_rmm_sdc_lanes(cla_block* b, int constRow, int accumulate, double* dOu
 	int rc = lanes_plan(b);
 	if(rc) return rc;
 	if(b->laneState != 1) return 1;
-	size_t lds = 0;
-	const int waves = lanes_waves(b, 16, &lds);
-	if(waves == 0) return 1;
+	// the tables of all slabs in LDS if they fit next to the output windows, else two buffers for the slab at work and the next
+	const size_t ldsMax = (size_t) std::min(g_ldsPerBlock, 160 * 1024), otBytes = sizeof(double) * ((size_t) LN_G * LN_WIN + 64);
+	const bool resident = sizeof(double) * (size_t) b->laneDictTotal + otBytes <= ldsMax;
+	const size_t lds = otBytes + sizeof(double) * (resident ? (size_t) b->laneDictTotal : 2 * (size_t) b->laneDictLds);
+	if(lds > ldsMax) return 1;
 	const int nWin = (int) ((b->nRows + LN_WIN - 1) / LN_WIN), nS = b->laneSlabs;
-	// one block per CU and round; whole rounds of the block's waves
-	int wpb = (int) std::max<int64_t>(waves, ((int64_t) nWin + g_numCU - 1) / g_numCU);
-	wpb = (wpb + waves - 1) / waves * waves;
+	// one block per CU; whole rounds of LN_G windows
+	int wpb = (int) std::max<int64_t>(LN_G, ((int64_t) nWin + g_numCU - 1) / g_numCU);
+	wpb = (wpb + LN_G - 1) / LN_G * LN_G;
 	const unsigned grid = (unsigned) ((nWin + wpb - 1) / wpb);
 	char* meta = (char*) b->dLaneMeta;
 	double algo = (double) b->nRows * 8 * (accumulate ? 2 : 1);
 	for(int g : b->sdcList) algo += (double) b->groups[g].d.nDeltas * b->groups[g].d.deltaWidth + (double) b->groups[g].d.nOffsets;
-	Prof pf(b, "k_rmm_sdc_lanes", (long) grid, waves * 64, (long) lds, algo);
+	Prof pf(b, "k_rmm_sdc_lanes", (long) grid, LN_RW * 64, (long) lds, algo);
 	auto go = [&](auto kernel) {
 		CLA_HIP(hipFuncSetAttribute((const void*) kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
-		hipLaunchKernelGGL(kernel, dim3(grid), dim3(waves * 64), lds, b->stream, (const LaneDesc*) meta,
-			(const LaneSlab*) (meta + b->laneOff[0]), nS, (const int32_t*) (meta + b->laneOff[2]), b->laneDictLds,
+		hipLaunchKernelGGL(kernel, dim3(grid), dim3(LN_RW * 64), lds, b->stream, (const LaneDesc*) meta,
+			(const LaneSlab*) (meta + b->laneOff[0]), nS, (const int32_t*) (meta + b->laneOff[2]), b->laneDictLds, b->laneDictTotal,
 			(const uint32_t*) (meta + b->laneOff[3]), (const u32x4*) b->dLaneData, (const double*) b->dTables, constRow, accumulate,
 			dOut, b->nRows, nWin, wpb, dNnz);
 		return 0;
 	};
-	rc = waves == 16 ? go(k_rmm_sdc_lanes<16>) : waves == 12 ? go(k_rmm_sdc_lanes<12>) : waves == 8 ? go(k_rmm_sdc_lanes<8>) : go(k_rmm_sdc_lanes<4>);
-	if(rc) return rc;
+	if((rc = resident ? go(k_rmm_sdc_lanes<true>) : go(k_rmm_sdc_lanes<false>))) return rc;
 	CLA_HIP(hipGetLastError());
 	return 0;
 }
