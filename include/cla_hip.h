@@ -113,7 +113,8 @@ int cla_block_set_stream(cla_handle h, void* hipStream);
  *   rmm_disable     bit 0 byte-code mat-vec kernel, 1 its fused tables, 2 matrix-core kernel, 3 decode kernel
  *   lmm_disable     bit 0 dot form on byte codes, bit 1 byte-code bin kernel
  *   sdc_packed      1 / 0: packed SDCZeros lists for the mat-vecs
- *   sdc_lanes       1 / 0: SDCZeros mat-vecs on the lists in place, one lane per group
+ *   sdc_lanes       1 / 0: SDCZeros mat-vecs on lane-major copies of the lists, one lane per group
+ *   sdc_rows        1 / 0: SDCZeros X %*% v on row lists (the lists transposed), one lane per row
  * Blocks derived from this one (overlapping results, joint blocks) inherit the values at the time of the call
  * that uses them. Returns 0, or -CLA_ERR_INVALID for an unknown key or value. */
 int cla_block_set_option(cla_handle h, const char* key, int32_t value);

@@ -290,6 +290,8 @@ void cla_block_free(cla_handle b) {
 	if(b->dSdcPacked) (void) hipFree(b->dSdcPacked);
 	if(b->dLaneMeta) (void) hipFree(b->dLaneMeta);
 	if(b->dLaneData) (void) hipFree(b->dLaneData);
+	if(b->dRowsMeta) (void) hipFree(b->dRowsMeta);
+	if(b->dRowsData) (void) hipFree(b->dRowsData);
 	if(b->dDictPad) (void) hipFree(b->dDictPad);
 	if(b->dCountsAll) (void) hipFree(b->dCountsAll);
 	if(b->dOnes) (void) hipFree(b->dOnes);
@@ -663,6 +665,7 @@ int cla_block_set_option(cla_handle b, const char* key, int32_t value) {
 		{"rmm_disable", &Options::rmmDisable, 0, 15},       {"lmm_disable", &Options::lmmDisable, 0, 3},
 		{"sdc_packed", &Options::sdcPacked, 0, 1},
 		{"sdc_lanes", &Options::sdcLanes, 0, 1},
+		{"sdc_rows", &Options::sdcRows, 0, 1},
 	};
 	for(const Entry& e : table)
 		if(strcmp(e.name, key) == 0) {

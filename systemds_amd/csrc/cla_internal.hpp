@@ -74,7 +74,8 @@ struct Options {
 	int rmmDisable = 0;     // bit 0 byte-code mat-vec, 1 fused tables of the byte-code mat-vec, 2 matrix-core kernel, 3 decode kernel
 	int lmmDisable = 0;     // bit 0 dot form on byte codes, 1 byte-code bin kernel
 	int sdcPacked = 1;      // packed SDCZeros lists for the mat-vecs
-	int sdcLanes = 1;       // SDCZeros mat-vecs on the lists in place, one lane per group
+	int sdcLanes = 1;       // SDCZeros mat-vecs on lane-major lists, one lane per group
+	int sdcRows = 1;        // SDCZeros right mat-vec on row lists, one lane per row
 };
 
 struct KernelStat {
@@ -167,6 +168,10 @@ struct cla_block {
 	int laneSlabs = 0, laneDictLds = 0, laneDictTotal = 0; // slabs, dictionary entries of the largest slab / of all
 	size_t laneOff[4] = {0, 0, 0, 0};
 	bool laneLmm = false;            // every listed group has one column (the left multiply's condition)
+	void* dRowsMeta = nullptr;       // row-list right multiply (k_sdc_rows.hip): table index, group list, headers, row order
+	void* dRowsData = nullptr;       // the listed groups' entries as row lists, built on first use
+	int rowsState = 0, rowsTbl = 0;  // 0 not planned yet, 1 ready, -1 the lists do not fit; table entries of all listed groups
+	size_t rowsOff[2] = {0, 0};
 	bool sdcPackFailed = false;
 	uint32_t* dSdcPacked = nullptr;  // all listed groups' entries as (code << 16 | row inside its 4096-row tile), built on first use
 	int sdcPlanGroup = -2;
@@ -216,6 +221,7 @@ int launch_lmm_u8_dot(cla_block* b, const double* dY, int p, double* dOut);
 int launch_lmm_sdc_tiles(cla_block* b, const double* dY, int p, double* dPre, int onlyGroup, double* dOut);
 int launch_lmm_sdc_lanes(cla_block* b, const double* dY, int p, double* dOut);
 int launch_rmm_sdc_lanes(cla_block* b, int constRow, int accumulate, double* dOut, unsigned long long* dNnz);
+int launch_rmm_sdc_rows(cla_block* b, int constRow, int accumulate, double* dOut, unsigned long long* dNnz);
 int launch_rmm_sdc_tiles(cla_block* b, int q, int constRow, int accumulate, double* dOut, unsigned long long* dNnz);
 int launch_tsmm_decode(cla_block* b, double* dOut);
 int launch_rmm_decode(cla_block* b, const double* dB, int q, const double* dConstRow, double* dOut,

@@ -1,0 +1,348 @@
+// SDCZeros right multiply with one output column on row lists (gfx950).
+//
+//   k_rows_build      one-time transposition of the listed groups' offset and code lists into row lists
+//   k_rmm_sdc_rows    out[row] = init + sum over the row's entries of T[entry]               (X %*% u)
+//
+// An SDCZeros group lists the rows that differ from the default; X %*% u needs, for every row, the sum of the
+// table values of the groups that list it. Scattering the lists into an output tile in LDS costs one LDS add of
+// a double per entry, about a cycle per lane. Here the lists are transposed once: every row gets the list of its
+// entries, an entry being the 16-bit position of the (group, tuple) pair in the concatenation of the groups'
+// tables. With the tables of a call in LDS a lane then owns a row: it reads its entries and sums the table
+// values in a register - no atomics, no output tile, no barrier behind the table load.
+//
+// Layout: rows are cut into quarters of RW_Q = 256; inside a quarter the rows are sorted by their number of
+// entries (perm holds the quarter's rows in that order) and cut into 4 slices of 64; a slice stores its entries
+// in groups of four per row (8 bytes), the 64 rows of a group side by side (512 bytes, one coalesced load per
+// wave), as many groups as its longest row needs; shorter rows are padded with the position of a 0.0 behind the
+// tables. A row's entries are sorted by position, so that its sum does not depend on the order in which the lists
+// were walked. A wave takes a quarter: it sums its four slices, puts the sums back into row order through a
+// 2 KB buffer of its own in LDS and writes 256 consecutive rows.
+#include "../../include/cla_hip.h"
+#include "cla_device.hpp"
+#include <algorithm>
+#include <vector>
+
+namespace cla {
+
+constexpr int RW_WIN = SDC_TILE;   // rows per window (the conversion starts from the row-tile index)
+constexpr int RW_SL = RW_WIN / 64; // slices per window
+constexpr int RW_KR = 40;          // most entries of a row (the conversion's staging area in LDS)
+constexpr int RW_Q = 256;          // rows per quarter: the unit of sorting and of a wave's work
+constexpr int RW_QS = RW_Q / 64;   // slices per quarter
+constexpr int RW_WAVES = 16;       // waves per block
+constexpr int RW_THREADS = RW_WAVES * 64;
+// entry groups of a quarter's slices that a lane requests a quarter ahead (the first slice holds the longest rows)
+__device__ constexpr int RW_PFS[RW_QS] = {6, 4, 3, 3};
+constexpr int RW_PFN = 6 + 4 + 3 + 3;
+constexpr int RW_TBL_MAX = 16000;  // table entries of all listed groups in LDS (125 KB, next to 2 KB per wave)
+static_assert(RW_WIN == 1024 && RW_Q == 256, "a conversion block sorts the four quarters of a window");
+
+typedef uint16_t u16x4 __attribute__((ext_vector_type(4)));
+
+// block = window. FILL == false: the window's size in entry groups into winSize. FILL == true: headers, perm, data.
+template <bool FILL>
+__global__ __launch_bounds__(256) void k_rows_build(const DGroup* __restrict__ groups, const int32_t* __restrict__ list,
+	const int32_t* __restrict__ gBase, int nL, int64_t nRows, uint32_t zeroIdx, uint32_t* __restrict__ winSize,
+	const uint64_t* __restrict__ winOff, uint2* __restrict__ hdr, uint16_t* __restrict__ perm, u16x4* __restrict__ data,
+	int* __restrict__ overflow) {
+	extern __shared__ uint32_t smemU[];
+	uint32_t* cnt = smemU;                        // RW_WIN
+	uint32_t* hist = cnt + RW_WIN;                // per quarter 64 (RW_KR + 1 used): rows per count, then first position per count
+	uint32_t* sl = hist + 256;                     // RW_SL + 1: entry groups per slice, then their prefix sums
+	uint16_t* rowOf = (uint16_t*) (sl + 32);      // RW_WIN: row at sorted position
+	uint16_t* stage = rowOf + RW_WIN;             // RW_WIN x RW_KR
+	const int tid = threadIdx.x;
+	const int win = blockIdx.x;
+	const int64_t r0 = (int64_t) win * RW_WIN, rEnd = r0 + RW_WIN;
+	for(int k = tid; k < RW_WIN; k += 256) cnt[k] = 0;
+	hist[tid] = 0;
+	__syncthreads();
+	for(int l = tid; l < nL; l += 256) {
+		const DGroup G = dgroup(groups + list[l]);
+		const uint32_t gb = (uint32_t) gBase[l];
+		auto entry = [&](int rel, int di) {
+			const uint32_t slot = atomicAdd(&cnt[rel], 1u);
+			if(slot < (uint32_t) RW_KR) stage[rel * RW_KR + slot] = (uint16_t) (gb + (uint32_t) load_code(G.codes, G.codeWidth, di));
+		};
+		if(G.first >= r0 && G.first < rEnd) entry((int) (G.first - r0), 0);
+		if(win < G.nTiles) {
+			const OffState st = G.tileIdx[win];
+			int64_t i = st.idx;
+			int32_t row = st.row, emit = st.emit;
+			const int maxV = G.deltaWidth == 1 ? 255 : 65535;
+			for(; i < G.nDeltas; i++) {
+				const int v = G.deltaWidth == 1 ? (int) ((const uint8_t*) G.deltas)[i] : (int) ((const uint16_t*) G.deltas)[i];
+				const int64_t nr = (int64_t) row + (v == 0 ? maxV : v);
+				if(nr >= rEnd) break;
+				row = (int32_t) nr;
+				if(v != 0) {
+					if(nr >= r0) entry((int) (nr - r0), emit); // (the state in front of a window holds no row of it)
+					emit++;
+				}
+			}
+		}
+	}
+	__syncthreads();
+	// the rows of every quarter sorted by their number of entries, longest first
+	bool over = false;
+	for(int k = tid; k < RW_WIN; k += 256) {
+		over |= cnt[k] > (uint32_t) RW_KR;
+		atomicAdd(&hist[(k / RW_Q) * 64 + min(cnt[k], (uint32_t) RW_KR)], 1u);
+	}
+	if(over) *overflow = 1; // a row with more entries than the staging area holds: the caller drops the row lists
+	__syncthreads();
+	if(tid < RW_WIN / RW_Q) {
+		uint32_t pos = tid * RW_Q;
+		for(int c = RW_KR; c >= 0; c--) {
+			const uint32_t n = hist[tid * 64 + c];
+			hist[tid * 64 + c] = pos;
+			pos += n;
+		}
+	}
+	__syncthreads();
+	for(int k = tid; k < RW_WIN; k += 256) rowOf[atomicAdd(&hist[(k / RW_Q) * 64 + min(cnt[k], (uint32_t) RW_KR)], 1u)] = (uint16_t) k;
+	__syncthreads();
+	if(tid < RW_SL) sl[tid] = (min(cnt[rowOf[tid * 64]], (uint32_t) RW_KR) + 3) / 4; // the slice's first row is its longest
+	__syncthreads();
+	if(tid == 0) {
+		uint32_t pos = 0;
+		for(int j = 0; j < RW_SL; j++) {
+			const uint32_t n = sl[j];
+			sl[j] = pos;
+			pos += n;
+		}
+		sl[RW_SL] = pos;
+		if(!FILL) winSize[win] = pos;
+	}
+	if(!FILL) return;
+	__syncthreads();
+	const uint64_t base = winOff[win];
+	if(tid < RW_SL) hdr[(size_t) win * RW_SL + tid] = make_uint2((uint32_t) (base + sl[tid]), sl[tid + 1] - sl[tid]);
+	for(int p = tid; p < RW_WIN; p += 256) {
+		const int r = rowOf[p], j = p >> 6, lane = p & 63;
+		perm[(size_t) win * RW_WIN + p] = (uint16_t) (r % RW_Q); // (position p lies in the quarter of its row)
+		uint16_t* e = stage + r * RW_KR;
+		const int c = (int) min(cnt[r], (uint32_t) RW_KR);
+		for(int a = 1; a < c; a++) { // ascending positions
+			const uint16_t x = e[a];
+			int z = a - 1;
+			for(; z >= 0 && e[z] > x; z--) e[z + 1] = e[z];
+			e[z + 1] = x;
+		}
+		const int k4 = (int) (sl[j + 1] - sl[j]);
+		u16x4* dst = data + (base + sl[j]) * 64 + lane;
+		for(int q = 0; q < k4; q++) {
+			u16x4 v;
+			v.x = 4 * q + 0 < c ? e[4 * q + 0] : (uint16_t) zeroIdx;
+			v.y = 4 * q + 1 < c ? e[4 * q + 1] : (uint16_t) zeroIdx;
+			v.z = 4 * q + 2 < c ? e[4 * q + 2] : (uint16_t) zeroIdx;
+			v.w = 4 * q + 3 < c ? e[4 * q + 3] : (uint16_t) zeroIdx;
+			dst[(size_t) q * 64] = v;
+		}
+	}
+}
+
+// block = 16 waves, all tables in LDS; a wave takes quarters in turn, a lane owns a row of each of their slices.
+// ACC == false: a row starts from constRow (or zero); ACC == true: from what other groups already wrote.
+template <bool ACC>
+__global__ __launch_bounds__(RW_THREADS) void k_rmm_sdc_rows(const int32_t* __restrict__ tblIndex, int nTbl,
+	const uint2* __restrict__ hdr, const uint16_t* __restrict__ perm, const u16x4* __restrict__ data,
+	const double* __restrict__ T, int constRow, double* __restrict__ out, int64_t nRows, int nQuarters,
+	unsigned long long* __restrict__ nnz) {
+	extern __shared__ double smemD[];
+	double* tbl = smemD;                 // nTbl values and a 0.0
+	const int tid = threadIdx.x, lane = tid & 63;
+	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+	double* back = smemD + (nTbl + 2) / 2 * 2 + wave * RW_Q; // this wave's sums in row order
+	for(int k = tid; k < nTbl; k += RW_THREADS) tbl[k] = T[tblIndex[k]];
+	if(tid == 0) tbl[nTbl] = 0.0;
+	const double init = !ACC && constRow >= 0 ? T[constRow] : 0.0;
+	__syncthreads();
+	int cntNz = 0;
+	// Requested a quarter ahead (two register sets take turns): the first entry groups of its slices, the lane's
+	// rows, the start values; two quarters ahead: the slices' headers. The work on a set is straight-line code.
+	struct Ahead {
+		u16x4 v[RW_PFN];
+		uint2 h[RW_QS];
+		uint16_t p[RW_QS];
+		double start[RW_QS];
+	};
+	struct Hdr { uint2 h[RW_QS]; };
+	auto header = [&](int qt) {
+		Hdr H;
+		const uint2* hp = hdr + (size_t) min(qt, nQuarters - 1) * RW_QS;
+#pragma unroll
+		for(int j = 0; j < RW_QS; j++) H.h[j] = hp[j];
+		return H;
+	};
+	auto request = [&](Ahead& A, int qt, const Hdr& H) { // qt < nQuarters
+		int o = 0;
+#pragma unroll
+		for(int j = 0; j < RW_QS; j++) {
+			A.h[j] = H.h[j];
+			const u16x4* src = data + (size_t) H.h[j].x * 64 + lane;
+			const int k4 = (int) H.h[j].y;
+#pragma unroll
+			for(int q = 0; q < RW_PFS[j]; q++) A.v[o + q] = src[(size_t) min(q, max(k4 - 1, 0)) * 64]; // (a group of slack lies behind the last slice)
+			o += RW_PFS[j];
+			A.p[j] = perm[(size_t) qt * RW_Q + j * 64 + lane];
+			A.start[j] = init;
+			if(ACC) A.start[j] = out[min((int64_t) qt * RW_Q + j * 64 + lane, nRows - 1)]; // (a template parameter: a load under a run-time branch is waited for at the branch's end)
+		}
+	};
+	const int step = gridDim.x * RW_WAVES;
+	auto work = [&](Ahead& A, Ahead& B, int qt, Hdr& hNext) { // A holds the requests of `qt`, hNext the headers of qt + step
+		request(B, min(qt + step, nQuarters - 1), hNext);
+		hNext = header(qt + 2 * step);
+		int o = 0;
+#pragma unroll
+		for(int j = 0; j < RW_QS; j++) {
+			const int k4 = (int) A.h[j].y;
+			double acc = 0.0;
+#pragma unroll
+			for(int q = 0; q < RW_PFS[j]; q++) {
+				if(q < k4) {
+					const u16x4 e = A.v[o + q];
+					const double a = tbl[e.x], b2 = tbl[e.y], c = tbl[e.z], d = tbl[e.w];
+					acc = (((acc + a) + b2) + c) + d;
+				}
+			}
+			const u16x4* src = data + (size_t) A.h[j].x * 64 + lane;
+			for(int q = RW_PFS[j]; q < k4; q++) {
+				const u16x4 e = src[(size_t) q * 64];
+				acc = (((acc + tbl[e.x]) + tbl[e.y]) + tbl[e.z]) + tbl[e.w];
+			}
+			o += RW_PFS[j];
+			back[A.p[j]] = acc;
+		}
+		__builtin_amdgcn_wave_barrier(); // LDS serves a wave's accesses in order: the reads below see the sums
+#pragma unroll
+		for(int j = 0; j < RW_QS; j++) {
+			const int64_t r = (int64_t) qt * RW_Q + j * 64 + lane;
+			const double res = A.start[j] + back[j * 64 + lane];
+			if(r < nRows) {
+				cntNz += res != 0.0;
+				out[r] = res;
+			}
+		}
+		__builtin_amdgcn_wave_barrier();
+	};
+	const int q0 = blockIdx.x * RW_WAVES + wave;
+	if(q0 < nQuarters) {
+		Ahead A, B;
+		request(A, q0, header(q0));
+		Hdr hNext = header(q0 + step);
+		for(int qt = q0; qt < nQuarters; qt += 2 * step) {
+			work(A, B, qt, hNext);
+			if(qt + step < nQuarters) work(B, A, qt + step, hNext);
+		}
+	}
+	count_add(nnz, cntNz);
+}
+
+// The row lists of the block's listed groups (whole-block plan), built once.
+static int rows_plan(cla_block* b) {
+	if(b->rowsState != 0) return 0;
+	b->rowsState = -1;
+	const std::vector<int32_t>& list = b->sdcList;
+	const int nL = (int) list.size();
+	const int nWin = (int) ((b->nRows + RW_WIN - 1) / RW_WIN);
+	if(nL == 0 || nWin == 0 || b->nRows >= ((int64_t) 1 << 31) - RW_WIN) return 0;
+	std::vector<int32_t> gBase(nL + 1, 0);
+	double entries = 0;
+	for(int l = 0; l < nL; l++) {
+		const DGroup& G = b->groups[list[l]].d;
+		gBase[l + 1] = gBase[l] + G.nVals;
+		entries += (double) G.nOffsets;
+	}
+	const int nTbl = gBase[nL];
+	if(nTbl > RW_TBL_MAX || nTbl >= 65535) return 0; // an entry is a 16-bit position; all tables sit in LDS
+	if(entries > (double) b->nRows * (RW_KR / 2)) return 0; // dense lists: rows too long for the staging area
+	if(sizeof(double) * ((size_t) nTbl + 2 + (size_t) RW_WAVES * RW_Q) > (size_t) std::min(g_ldsPerBlock, 160 * 1024)) return 0;
+	std::vector<int32_t> tblIndex(nTbl);
+	for(int l = 0; l < nL; l++) {
+		const DGroup& G = b->groups[list[l]].d;
+		for(int k = 0; k < G.nVals; k++) tblIndex[gBase[l] + k] = G.tblOff + k;
+	}
+	hipStream_t st = b->stream;
+	const size_t idxBytes = (sizeof(int32_t) * (size_t) nTbl + 15) / 16 * 16, listBytes = (sizeof(int32_t) * 2 * (size_t) nL + 15) / 16 * 16;
+	const size_t sizeBytes = (sizeof(uint64_t) * (size_t) nWin + 15) / 16 * 16, hdrBytes = sizeof(uint2) * (size_t) nWin * RW_SL;
+	const size_t permBytes = sizeof(uint16_t) * (size_t) nWin * RW_WIN;
+	char* meta = nullptr;
+	CLA_HIP(hipMalloc((void**) &meta, idxBytes + listBytes + sizeBytes + hdrBytes + permBytes + 16));
+	b->dRowsMeta = meta;
+	int32_t* dIdx = (int32_t*) meta;
+	int32_t* dList = (int32_t*) (meta + idxBytes);
+	int32_t* dBase = dList + nL;
+	uint64_t* dOff = (uint64_t*) (meta + idxBytes + listBytes); // pass 1: 32-bit sizes; pass 2: 64-bit offsets
+	uint2* dHdr = (uint2*) (meta + idxBytes + listBytes + sizeBytes);
+	uint16_t* dPerm = (uint16_t*) (meta + idxBytes + listBytes + sizeBytes + hdrBytes);
+	int* dOver = (int*) (meta + idxBytes + listBytes + sizeBytes + hdrBytes + permBytes);
+	CLA_HIP(hipMemcpyAsync(dIdx, tblIndex.data(), sizeof(int32_t) * (size_t) nTbl, hipMemcpyHostToDevice, st));
+	CLA_HIP(hipMemcpyAsync(dList, list.data(), sizeof(int32_t) * (size_t) nL, hipMemcpyHostToDevice, st));
+	CLA_HIP(hipMemcpyAsync(dBase, gBase.data(), sizeof(int32_t) * (size_t) nL, hipMemcpyHostToDevice, st));
+	CLA_HIP(hipMemsetAsync(dOver, 0, sizeof(int), st));
+	const size_t lds = sizeof(uint32_t) * (RW_WIN + 256 + 32) + sizeof(uint16_t) * ((size_t) RW_WIN + (size_t) RW_WIN * RW_KR);
+	CLA_HIP(hipFuncSetAttribute((const void*) k_rows_build<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
+	CLA_HIP(hipFuncSetAttribute((const void*) k_rows_build<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
+	hipLaunchKernelGGL(k_rows_build<false>, dim3(nWin), dim3(256), lds, st, b->dGroups, dList, dBase, nL, b->nRows, (uint32_t) nTbl,
+		(uint32_t*) dOff, nullptr, nullptr, nullptr, nullptr, dOver);
+	CLA_HIP(hipGetLastError());
+	std::vector<uint32_t> sizes(nWin);
+	int over = 0;
+	CLA_HIP(hipMemcpyAsync(sizes.data(), dOff, sizeof(uint32_t) * (size_t) nWin, hipMemcpyDeviceToHost, st));
+	CLA_HIP(hipMemcpyAsync(&over, dOver, sizeof(int), hipMemcpyDeviceToHost, st));
+	CLA_HIP(hipStreamSynchronize(st)); // (also: the host vectors above have been read)
+	if(over) return 0;
+	std::vector<uint64_t> offs(nWin);
+	uint64_t total = 0;
+	for(int w = 0; w < nWin; w++) {
+		offs[w] = total;
+		total += sizes[w];
+	}
+	if(total > 0xfffffff0ull) return 0; // (headers hold 32-bit group offsets)
+	const size_t dataBytes = (size_t) (total + 1) * 64 * sizeof(u16x4);
+	size_t freeB = 0, totalB = 0;
+	CLA_HIP(hipMemGetInfo(&freeB, &totalB));
+	if(dataBytes + ((size_t) 1 << 30) > freeB) return 0;
+	CLA_HIP(hipMalloc((void**) &b->dRowsData, dataBytes));
+	b->derivedBytes += (int64_t) (idxBytes + listBytes + sizeBytes + hdrBytes + permBytes + dataBytes);
+	CLA_HIP(hipMemsetAsync((char*) b->dRowsData + dataBytes - 64 * sizeof(u16x4), 0, 64 * sizeof(u16x4), st));
+	CLA_HIP(hipMemcpyAsync(dOff, offs.data(), sizeof(uint64_t) * (size_t) nWin, hipMemcpyHostToDevice, st));
+	hipLaunchKernelGGL(k_rows_build<true>, dim3(nWin), dim3(256), lds, st, b->dGroups, dList, dBase, nL, b->nRows, (uint32_t) nTbl,
+		nullptr, dOff, dHdr, dPerm, (u16x4*) b->dRowsData, dOver);
+	CLA_HIP(hipGetLastError());
+	CLA_HIP(hipStreamSynchronize(st)); // `offs` goes out of scope
+	b->rowsTbl = nTbl;
+	b->rowsOff[0] = idxBytes + listBytes + sizeBytes;
+	b->rowsOff[1] = idxBytes + listBytes + sizeBytes + hdrBytes;
+	b->rowsState = 1;
+	return 0;
+}
+
+// X %*% u of all listed groups (tables in b->dTables). Returns 1 when the lists do not fit (tables beyond LDS or
+// 16-bit positions, rows with too many entries), 0 when done.
+int launch_rmm_sdc_rows(cla_block* b, int constRow, int accumulate, double* dOut, unsigned long long* dNnz) {
+	int rc = rows_plan(b);
+	if(rc) return rc;
+	if(b->rowsState != 1) return 1;
+	const int nQuarters = (int) ((b->nRows + RW_Q - 1) / RW_Q);
+	const size_t lds = sizeof(double) * ((size_t) (b->rowsTbl + 2) / 2 * 2 + (size_t) RW_WAVES * RW_Q);
+	const unsigned grid = (unsigned) std::min((nQuarters + RW_WAVES - 1) / RW_WAVES, g_numCU);
+	char* meta = (char*) b->dRowsMeta;
+	double algo = (double) b->nRows * 8 * (accumulate ? 2 : 1);
+	for(int g : b->sdcList) algo += (double) b->groups[g].d.nDeltas * b->groups[g].d.deltaWidth + (double) b->groups[g].d.nOffsets * b->groups[g].d.codeWidth;
+	Prof pf(b, "k_rmm_sdc_rows", (long) grid, RW_THREADS, (long) lds, algo);
+	auto go = [&](auto kernel) {
+		CLA_HIP(hipFuncSetAttribute((const void*) kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
+		hipLaunchKernelGGL(kernel, dim3(grid), dim3(RW_THREADS), lds, b->stream, (const int32_t*) meta, b->rowsTbl,
+			(const uint2*) (meta + b->rowsOff[0]), (const uint16_t*) (meta + b->rowsOff[1]), (const u16x4*) b->dRowsData,
+			(const double*) b->dTables, constRow, dOut, b->nRows, nQuarters, dNnz);
+		return 0;
+	};
+	if((rc = accumulate ? go(k_rmm_sdc_rows<true>) : go(k_rmm_sdc_rows<false>))) return rc;
+	CLA_HIP(hipGetLastError());
+	return 0;
+}
+
+} // namespace cla

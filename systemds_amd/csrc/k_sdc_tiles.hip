@@ -561,6 +561,10 @@ int launch_rmm_sdc_tiles(cla_block* b, int q, int constRow, int accumulate, doub
 	if(rc) return rc;
 	struct { const std::vector<int32_t>&list, &binOff; } plan{b->sdcList, b->sdcBinOff};
 	if(plan.list.empty() || b->nRows == 0) return 1;
+	if(q == 1 && b->opt.sdcRows) { // one lane per row on row lists
+		const int r = launch_rmm_sdc_rows(b, constRow, accumulate, dOut, dNnz);
+		if(r <= 0) return r;
+	}
 	if(q == 1 && b->opt.sdcLanes) { // one lane per group on lane-major lists
 		const int r = launch_rmm_sdc_lanes(b, constRow, accumulate, dOut, dNnz);
 		if(r <= 0) return r;
