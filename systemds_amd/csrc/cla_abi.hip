@@ -543,6 +543,9 @@ int finish_finalize(cla_block* b, cla_block* arenaFrom, bool buildArena) {
 	{
 		size_t total = 0;
 		for(auto& g : b->groups) total += g.dict.size();
+		b->dictNonFinite = false;
+		for(auto& g : b->groups)
+			for(double v : g.dict) b->dictNonFinite |= !std::isfinite(v);
 		// (two doubles of padding: 16-byte copies of a dictionary range with an odd number of doubles read 8 bytes more)
 		CLA_HIP(hipMalloc((void**) &b->dAllDict, sizeof(double) * (total + 2)));
 		size_t off = 0;

@@ -173,6 +173,8 @@ struct cla_block {
 	int rowsState = 0, rowsTbl = 0;  // 0 not planned yet, 1 ready, -1 the lists do not fit; table entries of all listed groups
 	size_t rowsOff[2] = {0, 0};
 	bool sdcPackFailed = false;
+	bool dictNonFinite = false;      // some dictionary holds an infinity or a NaN (set at finalize): the left multiply then sums Y per tuple first, as the reference does
+	bool preUsed = false;            // left multiply: some kernel of the call wrote pre-aggregates (k_lmm_post has work)
 	uint32_t* dSdcPacked = nullptr;  // all listed groups' entries as (code << 16 | row inside its 4096-row tile), built on first use
 	int sdcPlanGroup = -2;
 	std::vector<int32_t> sdcList, sdcBinOff;

@@ -196,6 +196,7 @@ static int run_preagg(cla_block* b, const double* dY, int p, double* dPre, int o
 	// all groups DDC with byte codes in one arena: one persistent kernel for the whole block
 	if(onlyGroup < 0) {
 		const int r = launch_lmm_u8(b, dY, p, dPre);
+		if(r == 0) b->preUsed = true;
 		if(r <= 0) return r;
 	}
 	// row-parallel groups (DDC, RLE) in LDS-sized slabs
@@ -220,6 +221,7 @@ static int run_preagg(cla_block* b, const double* dY, int p, double* dPre, int o
 			if(direct) break;
 		}
 		if(nRows > 0) {
+			b->preUsed = true;
 			const size_t lds = direct ? 0 : bytes;
 			Prof pf(b, "k_lmm_preagg_rows", (long) gridRows * p, LMM_THREADS, (long) lds, 0);
 			CLA_HIP(hipFuncSetAttribute((const void*) k_lmm_preagg_rows, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
@@ -244,6 +246,7 @@ static int run_preagg(cla_block* b, const double* dY, int p, double* dPre, int o
 		const unsigned grid = (unsigned) std::max((G.nCkpt + cpb - 1) / cpb, 1);
 		const size_t bytes = direct ? 0 : (size_t) G.nVals * 8;
 		const double algo = (double) G.nDeltas * G.deltaWidth + (double) G.nOffsets * (G.codeWidth + 8.0);
+		b->preUsed = true;
 		Prof pf(b, "k_lmm_preagg_sdc", (long) grid * p, 256, (long) bytes, algo);
 		if(G.deltaWidth == 1) {
 			CLA_HIP(hipFuncSetAttribute((const void*) k_lmm_preagg_sdc<1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) bytes));
@@ -288,6 +291,7 @@ int launch_lmm(cla_block* b, const double* dY, int p, double* dOut, unsigned lon
 	CLA_HIP(hipMemsetAsync(dOut, 0, sizeof(double) * (size_t) p * b->nCols, st));
 	CLA_HIP(hipMemsetAsync(dNnz, 0, sizeof(unsigned long long), st));
 	// single-column DDC groups on byte codes: contributions go straight into dOut
+	b->preUsed = false;
 	const int dot = nRows > 0 ? launch_lmm_u8_dot(b, dY, p, dOut) : 1;
 	if(dot < 0) return dot;
 	if(dot != 0 && (rc = run_preagg(b, dY, p, dPre, -1, dOut))) return rc;
@@ -305,7 +309,7 @@ int launch_lmm(cla_block* b, const double* dY, int p, double* dOut, unsigned lon
 		Prof pf(b, "k_lmm_rowsum", (long) gridRows * p, 256, 0, 0);
 		hipLaunchKernelGGL(k_lmm_rowsum, dim3(gridRows, p), dim3(256), 0, st, dY, nRows, rowsPerBlock, dRs);
 	}
-	if(nG > 0 && dot != 0) {
+	if(nG > 0 && dot != 0 && b->preUsed) {
 		Prof pf(b, "k_lmm_post", (long) nG * p, 256, 0, 0);
 		hipLaunchKernelGGL(k_lmm_post, dim3(nG, p), dim3(256), 0, st, b->dGroups, dPre, b->totalVals, dOut, b->nCols);
 	}

@@ -318,6 +318,9 @@ int launch_lmm_u8_dot(cla_block* b, const double* dY, int p, double* dOut) {
 	const int nG = (int) b->groups.size();
 	if(!(b->dArena && b->arenaWidth == 1 && b->maxVals <= 256 && nG > 0 && b->nRows > 0)) return 1;
 	if(b->opt.lmmDisable & 1) return 1;
+	// Y[row] * dict[code] summed over the rows differs from (sum of Y per code) * dict[code], the reference's order
+	// (ADictionary pre-aggregation), where an infinite dictionary value meets values of Y of both signs
+	if(b->dictNonFinite) return 1;
 	for(int g = 0; g < nG; g++)
 		if(b->groups[g].d.nColG != 1) return 1;
 	constexpr int PER = 20;

@@ -493,13 +493,15 @@ int launch_lmm_sdc_tiles(cla_block* b, const double* dY, int p, double* dPre, in
 	if(plan.list.empty()) return 0;
 	// whole-block call on single-column groups: one lane per group on lane-major lists, products straight
 	// into dOut (the groups' part of dPre stays zero)
-	if(dOut != nullptr && onlyGroup < 0 && b->opt.sdcLanes) {
+	// (not with a non-finite dictionary value: the kernels below sum Y[row] * dict[code] over the rows, the reference
+	// sums Y per tuple first, and the two differ where an infinity meets values of Y of both signs)
+	if(dOut != nullptr && onlyGroup < 0 && b->opt.sdcLanes && !b->dictNonFinite) {
 		const int r = launch_lmm_sdc_lanes(b, dY, p, dOut);
 		if(r <= 0) return r;
 	}
 	// all listed groups single-column with at most 64 tuples, whole-block call: packed lists, products
 	// straight into dOut
-	bool packed = dOut != nullptr && onlyGroup < 0 && b->opt.sdcPacked;
+	bool packed = dOut != nullptr && onlyGroup < 0 && b->opt.sdcPacked && !b->dictNonFinite;
 	for(int g : plan.list) packed &= b->groups[g].d.nColG == 1 && b->groups[g].d.nVals <= 64;
 	if(packed && (rc = sdc_plan(b, onlyGroup, &dList, &dBinOff, true))) return rc;
 	packed &= b->dSdcPacked != nullptr;
@@ -544,6 +546,7 @@ int launch_lmm_sdc_tiles(cla_block* b, const double* dY, int p, double* dPre, in
 			const DGroup& G = b->groups[plan.list[l]].d;
 			algo += (double) p * ((double) G.nDeltas * G.deltaWidth + (double) G.nOffsets * G.codeWidth);
 		}
+		b->preUsed = true;
 		Prof pf(b, "k_lmm_sdc_tiles", (long) grid * p, ST_THREADS, (long) lds, algo);
 		CLA_HIP(hipFuncSetAttribute((const void*) k_lmm_sdc_tiles, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
 		hipLaunchKernelGGL(k_lmm_sdc_tiles, dim3(grid, p), dim3(ST_THREADS), lds, b->stream, b->dGroups, dList, dBinOff,

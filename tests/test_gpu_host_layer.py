@@ -192,8 +192,10 @@ def test_overlapping_right_multiply_stays_compressed(H, ora, cla):
     assert_fp64_close(mm(xb, H.MatrixBlock(C), 4).toArray(), ora.longdouble_matmul(P, C), absP @ np.abs(C), what="(XB) %*% C")
     Y = rng.standard_normal((2, n_rows))
     assert_fp64_close(mm(H.MatrixBlock(Y), xb, 4).toArray(), ora.longdouble_matmul(Y, P), np.abs(Y) @ absP, what="Y %*% (XB)")
-    with pytest.raises(H.NotImplementedException):
-        xb.transposeSelfMatrixMultOperations(H.MMTSJType.LEFT, 4)
+    # t(XB) %*% (XB) is not linear in the groups: the library decompresses the block and multiplies on the matrix
+    # cores, as the reference does for overlapping blocks (CLALibTSMM.java:73-77)
+    tsmm = xb.transposeSelfMatrixMultOperations(H.MMTSJType.LEFT, 4).toArray()
+    assert_fp64_close(tsmm, ora.longdouble_matmul(P.T, P), np.abs(P).T @ np.abs(P), what="t(XB) %*% (XB)", n_terms=n_rows)
     with pytest.raises(H.NotImplementedException):
         H.writeCompressedMatrixBlock(xb)
     with pytest.raises(H.NotImplementedException):   # by-value result cannot be compressed
