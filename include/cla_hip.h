@@ -109,6 +109,7 @@ int cla_block_set_stream(cla_handle h, void* hipStream);
  *   tsmm_route      0 cost model, 1 one pass per pair of groups, 2 decoded Gram matrix
  *   tsmm_chunks     1 / 0: more than 64 columns as pairs of column chunks
  *   tsmm_wide_dense 0 / 1, tsmm_mfma 1 / 0, tsmm_pair_dot 1 / 0
+ *   tsmm_narrow     1 / 0: decoded Gram matrix with a last column block of at most 4 columns on the 4x4x4 matrix instruction
  *   expand_streams  1 / 0: one code per row for small RLE / SDCZeros groups (set before the first multiply)
  *   rmm_disable     bit 0 byte-code mat-vec kernel, 1 its fused tables, 2 matrix-core kernel, 3 decode kernel
  *   lmm_disable     bit 0 dot form on byte codes, bit 1 byte-code bin kernel

@@ -69,6 +69,7 @@ struct Options {
 	int tsmmChunks = 1;     // more than 64 columns: decoded Gram matrices of pairs of column chunks
 	int tsmmWideDense = 0;  // more than 64 columns and as many groups as columns: scalar decompressing form
 	int tsmmMfma = 1;       // decoded Gram matrix on the matrix cores (0: scalar form)
+	int tsmmNarrow = 1;     // decoded Gram matrix: a last column block of at most 4 columns on the 4 x 4 x 4 matrix instruction
 	int tsmmPairDot = 1;    // DDC x DDC pairs in dot form (0: pre-aggregate form with LDS bins)
 	int expandStreams = 1;  // one code per row for small RLE / SDCZeros groups in the decode kernels
 	int rmmDisable = 0;     // bit 0 byte-code mat-vec, 1 fused tables of the byte-code mat-vec, 2 matrix-core kernel, 3 decode kernel

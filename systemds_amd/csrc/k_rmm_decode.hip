@@ -141,7 +141,36 @@ __device__ __forceinline__ void dec_load_window(uint8_t* win, const uint8_t* src
 
 // FLAT: dictionaries that do not fit LDS stay in global memory; the lookups then go through
 // generic pointers (LDS or global per lane).
-template <int GRAM, int NB, int RPL, int FLAT, int XB = 0>
+// Lanes 4 u .. 4 u + 3 of every 16 lanes (bank u) copied into the other three banks of the 16.
+// row_shr:4 d moves a bank d banks up, row_shl:4 d moves it d banks down; the bank mask picks the receiving bank.
+__device__ __forceinline__ int dec_spread_bank(int o, int u) {
+	int a = o;
+	switch(u) {
+		case 0:
+			a = __builtin_amdgcn_update_dpp(a, o, 0x114, 0xf, 0x2, false);
+			a = __builtin_amdgcn_update_dpp(a, o, 0x118, 0xf, 0x4, false);
+			a = __builtin_amdgcn_update_dpp(a, o, 0x11c, 0xf, 0x8, false);
+			break;
+		case 1:
+			a = __builtin_amdgcn_update_dpp(a, o, 0x104, 0xf, 0x1, false);
+			a = __builtin_amdgcn_update_dpp(a, o, 0x114, 0xf, 0x4, false);
+			a = __builtin_amdgcn_update_dpp(a, o, 0x118, 0xf, 0x8, false);
+			break;
+		case 2:
+			a = __builtin_amdgcn_update_dpp(a, o, 0x108, 0xf, 0x1, false);
+			a = __builtin_amdgcn_update_dpp(a, o, 0x104, 0xf, 0x2, false);
+			a = __builtin_amdgcn_update_dpp(a, o, 0x114, 0xf, 0x8, false);
+			break;
+		default:
+			a = __builtin_amdgcn_update_dpp(a, o, 0x10c, 0xf, 0x1, false);
+			a = __builtin_amdgcn_update_dpp(a, o, 0x108, 0xf, 0x2, false);
+			a = __builtin_amdgcn_update_dpp(a, o, 0x104, 0xf, 0x4, false);
+			break;
+	}
+	return a;
+}
+
+template <int GRAM, int NB, int RPL, int FLAT, int XB = 0, int NAR = 0>
 __device__ __forceinline__ void decode_body(const DecArgs& A) {
 	extern __shared__ __align__(16) double smem[];
 	double* Bs = smem + A.valDoubles;                              // bDoubles: rows of B in decoded column order, 16 outputs each
@@ -249,11 +278,20 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 	// multiply phase state
 	// tiles of the Gram matrix held by a wave: the upper triangle, or with XB > 0 (only the product of the first
 	// XB column blocks with the others is wanted) those XB x (NB - XB) tiles
-	constexpr int NTILES = !GRAM ? 1 : XB > 0 ? XB * (NB - XB) : NB * (NB + 1) / 2;
+	// NAR (the last column block holds at most 4 columns): 16 x 16 tiles only among the NB - 1 full blocks; the
+	// rows of the last block come from v_mfma_f64_4x4x4_f64, one instruction per column block (its four 4 x 4 x 4
+	// products are the last block's 4 columns against the 4 quarters of a 16-column block), which issues at four
+	// times the rate of a 16 x 16 tile and replaces NB of them.
+	static_assert(!NAR || (GRAM && XB == 0 && NB >= 2), "narrow last block: full Gram matrices only");
+	constexpr int NF = NAR ? NB - 1 : NB; // column blocks among which 16 x 16 tiles are computed
+	constexpr int NTILES = !GRAM ? 1 : XB > 0 ? XB * (NB - XB) : NF * (NF + 1) / 2;
 	f64x4 gram[NTILES];
+	double nar[NAR ? NB : 1]; // lane l: cell (row 16 (NB - 1) + l / 16, column 16 cb + l % 16)
 	if(GRAM) {
 #pragma unroll
 		for(int t = 0; t < NTILES; t++) gram[t] = f64x4{0.0, 0.0, 0.0, 0.0};
+#pragma unroll
+		for(int cb = 0; cb < (NAR ? NB : 1); cb++) nar[cb] = 0.0;
 	}
 	const int q = A.q;
 	const double cinit = (!GRAM && A.constRow != nullptr && i16 < q) ? A.constRow[i16] : 0.0;
@@ -392,28 +430,35 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 				const double* lptr[FLAT ? NB : 1];
 #pragma unroll
 				for(int cb = 0; cb < NB; cb++) {
-					const DecLook L(colS[cb * 16 + i16]);
+					// (narrow block with packed lookups: every lane of the last block works on one of its first four columns)
+					const int ci = cb * 16 + (NAR && NB <= 2 && cb == NB - 1 ? i16 & 3 : i16);
+					const DecLook L(colS[ci]);
 					lbase[cb] = L.base; lnC[cb] = L.nC; lsent[cb] = L.sent; lcoded[cb] = L.coded; ldense[cb] = L.dense; ltwo[cb] = L.two;
 					if(FLAT) {
-						const DecCol D = colS[cb * 16 + i16];
+						const DecCol D = colS[ci];
 						const double* gdict = groupS[D.pad].dict + ((unsigned) D.meta >> 18);
 						lptr[cb] = (D.meta & 8) ? gdict : (const double*) smem + L.base;
 					}
-					cst[cb] = constS[cb * 16 + i16];
-					const u32x4* cp = (const u32x4*) (slots + (L.coded ? colS[cb * 16 + i16].slotOff + rbase * (L.two ? 2 : 1) : 0));
+					cst[cb] = constS[ci];
+					const u32x4* cp = (const u32x4*) (slots + (L.coded ? colS[ci].slotOff + rbase * (L.two ? 2 : 1) : 0));
 					cq[cb][0] = cp[0];
 					cq[cb][1] = cp[1];
 				}
 				// SB steps of lookups in flight, then their products
 				constexpr int SB = NB <= 2 ? 4 : 2;
+				// the narrow block's lookups packed four steps to one (below) pay with few column blocks; with many, the value
+				// kept over two batches costs registers that the lookups in flight need
+				constexpr bool NPACK = NAR && NB <= 2;
+				constexpr int NL = NPACK ? NF : NB; // column blocks looked up per step
+				double xn = 0.0; // NAR: lane (k4, i16) holds column i16 % 4 of the last block at step 4 (sb / 4) + i16 / 4
 #pragma unroll
 				for(int sb = 0; sb < 16; sb += SB) {
-					double x[SB][NB];
+					double x[SB][NL];
 #pragma unroll
 					for(int u = 0; u < SB; u++) {
 						const int s = sb + u;
 #pragma unroll
-						for(int cb = 0; cb < NB; cb++) {
+						for(int cb = 0; cb < NL; cb++) {
 							const int c1 = (int) ((cq[cb][0][s >> 2] >> (8 * (s & 3))) & 0xff);
 							const int c2 = (int) ((cq[cb][s >> 3][(s >> 1) & 3] >> (16 * (s & 1))) & 0xffff);
 							const int c = ltwo[cb] ? c2 : c1;
@@ -431,17 +476,55 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 							x[u][cb] = valid ? v : 0.0;
 						}
 					}
+					if(NPACK && (sb & 3) == 0) {
+						// the last block's (at most 4) columns of four steps in one lookup: lanes 4 j .. 4 j + 3 of every 16
+						// take step sb + j and column i16 % 4 (their descriptors are those of lanes 0 .. 3)
+						constexpr int cb = NAR ? NB - 1 : 0;
+						const int sHi = sb >> 2, j = i16 >> 2, s = sb + j;
+						const int c1 = (int) ((cq[cb][0][sHi] >> (8 * j)) & 0xff);
+						const uint32_t lo = cq[cb][sHi >> 1][(2 * sHi) & 3], hi = cq[cb][sHi >> 1][(2 * sHi + 1) & 3]; // codes 4 sHi .. + 3 as 16-bit pieces
+						const int c2 = (int) (((j & 2 ? hi : lo) >> (16 * (j & 1))) & 0xffff);
+						const int c = ltwo[cb] ? c2 : c1;
+						const bool in = t0 + rbase + s < nRows;
+						const bool valid = in & (ldense[cb] | (lcoded[cb] & (c != lsent[cb])));
+						double v;
+						if(FLAT) {
+							const double* vp = lptr[cb] + (lcoded[cb] ? c : rbase + s) * lnC[cb];
+							v = *(valid ? vp : (const double*) smem);
+						}
+						else {
+							const int ad = lbase[cb] + (lcoded[cb] ? c : rbase + s) * lnC[cb];
+							v = smem[valid ? ad : 0];
+						}
+						v = valid ? v : 0.0;
+						xn = in ? cst[cb] + v : 0.0;
+					}
 #pragma unroll
 					for(int u = 0; u < SB; u++) {
 						const bool in = t0 + rbase + sb + u < nRows;
 #pragma unroll
-						for(int cb = 0; cb < NB; cb++) x[u][cb] = in ? cst[cb] + x[u][cb] : 0.0;
+						for(int cb = 0; cb < NL; cb++) x[u][cb] = in ? cst[cb] + x[u][cb] : 0.0;
 						int t = 0;
 #pragma unroll
-						for(int ib = 0; ib < (XB > 0 ? XB : NB); ib++)
+						for(int ib = 0; ib < (XB > 0 ? XB : NF); ib++)
 #pragma unroll
-							for(int jb = (XB > 0 ? XB : ib); jb < NB; jb++, t++)
+							for(int jb = (XB > 0 ? XB : ib); jb < NF; jb++, t++)
 								gram[t] = __builtin_amdgcn_mfma_f64_16x16x4f64(x[u][ib], x[u][jb], gram[t], 0, 0, 0);
+						if(NAR) {
+							// operands of the 4 x 4 x 4 form for step sb + u: every lane needs column l % 4 of the last block for
+							// its row group, which lane 4 ((sb + u) % 4) + l % 4 of its 16 holds: that bank spread over the others
+							// (not packed: every lane looked its own column of the last block up; lanes 0 .. 3 of 16 hold the real ones)
+							int a[2], o[2];
+							__builtin_memcpy(o, NPACK ? &xn : &x[u][NL - 1], 8);
+							a[0] = dec_spread_bank(o[0], NPACK ? (sb + u) & 3 : 0);
+							a[1] = dec_spread_bank(o[1], NPACK ? (sb + u) & 3 : 0);
+							double an;
+							__builtin_memcpy(&an, a, 8);
+#pragma unroll
+							for(int cb = 0; cb < NF; cb++) nar[cb] = __builtin_amdgcn_mfma_f64_4x4x4f64(an, x[u][cb], nar[cb], 0, 0, 0);
+							// last block x last block: all four products are the same 4 x 4 one (the first is kept)
+							nar[NAR ? NB - 1 : 0] = __builtin_amdgcn_mfma_f64_4x4x4f64(an, an, nar[NAR ? NB - 1 : 0], 0, 0, 0);
+						}
 					}
 				}
 			}
@@ -521,12 +604,20 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 		__syncthreads();
 		int t = 0;
 #pragma unroll
-		for(int ib = 0; ib < (XB > 0 ? XB : NB); ib++)
+		for(int ib = 0; ib < (XB > 0 ? XB : NF); ib++)
 #pragma unroll
-			for(int jb = (XB > 0 ? XB : ib); jb < NB; jb++, t++)
+			for(int jb = (XB > 0 ? XB : ib); jb < NF; jb++, t++)
 #pragma unroll
 				for(int v = 0; v < 4; v++)
 					unsafeAtomicAdd(&stage[(ib * 16 + 4 * v + k4) * NP + jb * 16 + i16], gram[t][v]);
+		if(NAR) {
+			// cell (16 (NB - 1) + k4, 16 cb + i16): into the upper triangle at its mirror image for the full blocks
+#pragma unroll
+			for(int cb = 0; cb < NB; cb++) {
+				const int r = (NB - 1) * 16 + k4, c = cb * 16 + i16;
+				unsafeAtomicAdd(&stage[cb < NB - 1 ? c * NP + r : r * NP + c], nar[cb]);
+			}
+		}
 		__syncthreads();
 		for(int i = tid; i < NP * NP; i += DEC_THREADS) {
 			const int r = i / NP, c = i - r * NP;
@@ -540,8 +631,8 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 template <int RPL>
 __global__ __launch_bounds__(DEC_THREADS) void k_rmm_decode(const DecArgs A) { decode_body<0, 1, RPL, 0>(A); }
 
-template <int NB, int FLAT, int XB>
-__global__ __launch_bounds__(DEC_THREADS) void k_tsmm_decode(const DecArgs A) { decode_body<1, NB, 4, FLAT, XB>(A); }
+template <int NB, int FLAT, int XB, int NAR = 0>
+__global__ __launch_bounds__(DEC_THREADS) void k_tsmm_decode(const DecArgs A) { decode_body<1, NB, 4, FLAT, XB, NAR>(A); }
 
 // One code per row for an RLE group (0xff where no run covers the row): thread = 4 rows.
 __global__ __launch_bounds__(256) void k_expand_rle(const DGroup* __restrict__ groups, int g, int64_t nRows, uint8_t* __restrict__ codes) {
@@ -802,10 +893,19 @@ int launch_tsmm_decode(cla_block* b, double* dOut) {
 	if(rc) return rc;
 	L.A.out = dOut;
 	Prof pf(b, "k_tsmm_decode", L.grid, DEC_THREADS, (long) L.lds, (double) b->device_bytes_cached);
+	// a last column block of at most 4 columns: its rows on the 4 x 4 x 4 matrix instruction
+	const bool narrow = XB == 0 && NB >= 2 && nCols - 16 * (NB - 1) <= 4 && b->opt.tsmmNarrow;
 #define GRAM_LAUNCH(NBV, FL, XBV)                                                                               \
 	do {                                                                                                        \
-		CLA_HIP(hipFuncSetAttribute((const void*) k_tsmm_decode<NBV, FL, XBV>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) L.lds)); \
-		hipLaunchKernelGGL((k_tsmm_decode<NBV, FL, XBV>), dim3(L.grid), dim3(DEC_THREADS), L.lds, b->stream, L.A); \
+		if(XBV == 0 && NBV >= 2 && narrow) {                                                                    \
+			constexpr int NARV = XBV == 0 && NBV >= 2 ? 1 : 0;                                                  \
+			CLA_HIP(hipFuncSetAttribute((const void*) k_tsmm_decode<NBV, FL, XBV, NARV>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) L.lds)); \
+			hipLaunchKernelGGL((k_tsmm_decode<NBV, FL, XBV, NARV>), dim3(L.grid), dim3(DEC_THREADS), L.lds, b->stream, L.A); \
+		}                                                                                                       \
+		else {                                                                                                  \
+			CLA_HIP(hipFuncSetAttribute((const void*) k_tsmm_decode<NBV, FL, XBV>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) L.lds)); \
+			hipLaunchKernelGGL((k_tsmm_decode<NBV, FL, XBV>), dim3(L.grid), dim3(DEC_THREADS), L.lds, b->stream, L.A); \
+		}                                                                                                       \
 	} while(0)
 #define GRAM_SHAPES(FL)                                        \
 	do {                                                       \

@@ -146,3 +146,43 @@ def test_decompress(cla, ora, seed, n_rows):
     ref = ora.decompress(ora.Groups(specs, n_rows, n_cols))
     assert np.array_equal(out, ref)
     assert nnz == np.count_nonzero(ref)
+
+
+@pytest.mark.parametrize("narrow", [1, 0])
+@pytest.mark.parametrize("n_cols,big_dict", [(17, False), (18, True), (20, False), (35, False), (36, True), (50, False), (52, True), (21, False)])
+def test_decoded_gram_with_a_narrow_last_column_block(cla, ora, n_cols, big_dict, narrow):
+    """Column counts whose last block of 16 holds at most 4 columns: its rows of the Gram matrix come from the
+    4 x 4 x 4 matrix instruction (`tsmm_narrow`, the default) instead of 16 x 16 tiles; with at most 32 columns the
+    last block's lookups of four steps are packed into one. Mixed group types, one- and two-byte codes,
+    dictionaries in LDS and (big_dict) in global memory, a ragged last tile; 21 columns (5 in the last block) take
+    the tiles either way."""
+    from systemds_amd import synth
+    n_rows = 70001
+    rng = np.random.default_rng(n_cols)
+    specs, c = [], 0
+    while c < n_cols:
+        left = n_cols - c
+        kind = ["ddc", "ddc2", "sdc", "rle", "unc"][len(specs) % 5]
+        if kind == "ddc2" and left >= 2:
+            nv = 5000 if big_dict else 300
+            codes = rng.integers(0, nv, n_rows).astype(np.uint16)
+            specs.append(synth.GroupSpec("ddc", np.arange(c, c + 2, dtype=np.int32), rng.standard_normal((nv, 2)), codes))
+            c += 2
+        elif kind == "sdc":
+            specs.append(synth.sdc_group(rng, n_rows, np.array([c], np.int32), 7, 0.1, 0.5))
+            c += 1
+        elif kind == "rle":
+            run_codes = rng.integers(-1, 4, size=n_rows // 40 + 2)
+            codes = np.repeat(run_codes, rng.integers(1, 90, size=run_codes.size))[:n_rows]
+            codes = np.concatenate([codes, np.full(n_rows - codes.size, -1)]) if codes.size < n_rows else codes
+            ptr, data = synth.encode_rle(codes, 4)
+            specs.append(synth.GroupSpec("rle", np.array([c], np.int32), rng.standard_normal((4, 1)), ptr=ptr, rle=data))
+            c += 1
+        elif kind == "unc":
+            specs.append(synth.GroupSpec("unc", np.array([c], np.int32), dense=rng.standard_normal((n_rows, 1))))
+            c += 1
+        else:
+            codes = rng.integers(0, 16, n_rows).astype(np.uint8)
+            specs.append(synth.GroupSpec("ddc", np.array([c], np.int32), rng.standard_normal((16, 1)), codes))
+            c += 1
+    check_tsmm(cla, ora, specs, n_rows, n_cols, f"{n_cols} columns, narrow {narrow}", {"tsmm_route": 2, "tsmm_narrow": narrow})
