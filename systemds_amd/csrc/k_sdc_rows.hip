@@ -38,10 +38,11 @@ constexpr int RW_TBL_MAX = 16000;  // table entries of all listed groups in LDS 
 static_assert(RW_WIN == 1024 && RW_Q == 256, "a conversion block sorts the four quarters of a window");
 
 typedef uint16_t u16x4 __attribute__((ext_vector_type(4)));
+constexpr int RB_THREADS = 1024;   // threads of a conversion block (one window)
 
 // block = window. FILL == false: the window's size in entry groups into winSize. FILL == true: headers, perm, data.
 template <bool FILL>
-__global__ __launch_bounds__(256) void k_rows_build(const DGroup* __restrict__ groups, const int32_t* __restrict__ list,
+__global__ __launch_bounds__(RB_THREADS) void k_rows_build(const DGroup* __restrict__ groups, const int32_t* __restrict__ list,
 	const int32_t* __restrict__ gBase, int nL, int64_t nRows, uint32_t zeroIdx, uint32_t* __restrict__ winSize,
 	const uint64_t* __restrict__ winOff, uint2* __restrict__ hdr, uint16_t* __restrict__ perm, u16x4* __restrict__ data,
 	int* __restrict__ overflow) {
@@ -54,38 +55,24 @@ __global__ __launch_bounds__(256) void k_rows_build(const DGroup* __restrict__ g
 	const int tid = threadIdx.x;
 	const int win = blockIdx.x;
 	const int64_t r0 = (int64_t) win * RW_WIN, rEnd = r0 + RW_WIN;
-	for(int k = tid; k < RW_WIN; k += 256) cnt[k] = 0;
-	hist[tid] = 0;
+	for(int k = tid; k < RW_WIN; k += RB_THREADS) cnt[k] = 0;
+	if(tid < 256) hist[tid] = 0;
 	__syncthreads();
-	for(int l = tid; l < nL; l += 256) {
+	// a wave walks a group's part of the window at a time (256 offsets per step, decoded with a prefix sum over the wave)
+	for(int l = tid >> 6; l < nL; l += RB_THREADS / 64) {
 		const DGroup G = dgroup(groups + list[l]);
 		const uint32_t gb = (uint32_t) gBase[l];
-		auto entry = [&](int rel, int di) {
+		const void* codes = G.codes;
+		const int cw = G.codeWidth;
+		sdc_walk_tile(G, r0, RW_WIN, [&](int rel, int di) {
 			const uint32_t slot = atomicAdd(&cnt[rel], 1u);
-			if(slot < (uint32_t) RW_KR) stage[rel * RW_KR + slot] = (uint16_t) (gb + (uint32_t) load_code(G.codes, G.codeWidth, di));
-		};
-		if(G.first >= r0 && G.first < rEnd) entry((int) (G.first - r0), 0);
-		if(win < G.nTiles) {
-			const OffState st = G.tileIdx[win];
-			int64_t i = st.idx;
-			int32_t row = st.row, emit = st.emit;
-			const int maxV = G.deltaWidth == 1 ? 255 : 65535;
-			for(; i < G.nDeltas; i++) {
-				const int v = G.deltaWidth == 1 ? (int) ((const uint8_t*) G.deltas)[i] : (int) ((const uint16_t*) G.deltas)[i];
-				const int64_t nr = (int64_t) row + (v == 0 ? maxV : v);
-				if(nr >= rEnd) break;
-				row = (int32_t) nr;
-				if(v != 0) {
-					if(nr >= r0) entry((int) (nr - r0), emit); // (the state in front of a window holds no row of it)
-					emit++;
-				}
-			}
-		}
+			if(slot < (uint32_t) RW_KR) stage[rel * RW_KR + slot] = (uint16_t) (gb + (uint32_t) load_code(codes, cw, di));
+		});
 	}
 	__syncthreads();
 	// the rows of every quarter sorted by their number of entries, longest first
 	bool over = false;
-	for(int k = tid; k < RW_WIN; k += 256) {
+	for(int k = tid; k < RW_WIN; k += RB_THREADS) {
 		over |= cnt[k] > (uint32_t) RW_KR;
 		atomicAdd(&hist[(k / RW_Q) * 64 + min(cnt[k], (uint32_t) RW_KR)], 1u);
 	}
@@ -100,7 +87,7 @@ __global__ __launch_bounds__(256) void k_rows_build(const DGroup* __restrict__ g
 		}
 	}
 	__syncthreads();
-	for(int k = tid; k < RW_WIN; k += 256) rowOf[atomicAdd(&hist[(k / RW_Q) * 64 + min(cnt[k], (uint32_t) RW_KR)], 1u)] = (uint16_t) k;
+	for(int k = tid; k < RW_WIN; k += RB_THREADS) rowOf[atomicAdd(&hist[(k / RW_Q) * 64 + min(cnt[k], (uint32_t) RW_KR)], 1u)] = (uint16_t) k;
 	__syncthreads();
 	if(tid < RW_SL) sl[tid] = (min(cnt[rowOf[tid * 64]], (uint32_t) RW_KR) + 3) / 4; // the slice's first row is its longest
 	__syncthreads();
@@ -118,7 +105,7 @@ __global__ __launch_bounds__(256) void k_rows_build(const DGroup* __restrict__ g
 	__syncthreads();
 	const uint64_t base = winOff[win];
 	if(tid < RW_SL) hdr[(size_t) win * RW_SL + tid] = make_uint2((uint32_t) (base + sl[tid]), sl[tid + 1] - sl[tid]);
-	for(int p = tid; p < RW_WIN; p += 256) {
+	for(int p = tid; p < RW_WIN; p += RB_THREADS) {
 		const int r = rowOf[p], j = p >> 6, lane = p & 63;
 		perm[(size_t) win * RW_WIN + p] = (uint16_t) (r % RW_Q); // (position p lies in the quarter of its row)
 		uint16_t* e = stage + r * RW_KR;
@@ -285,7 +272,7 @@ static int rows_plan(cla_block* b) {
 	const size_t lds = sizeof(uint32_t) * (RW_WIN + 256 + 32) + sizeof(uint16_t) * ((size_t) RW_WIN + (size_t) RW_WIN * RW_KR);
 	CLA_HIP(hipFuncSetAttribute((const void*) k_rows_build<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
 	CLA_HIP(hipFuncSetAttribute((const void*) k_rows_build<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
-	hipLaunchKernelGGL(k_rows_build<false>, dim3(nWin), dim3(256), lds, st, b->dGroups, dList, dBase, nL, b->nRows, (uint32_t) nTbl,
+	hipLaunchKernelGGL(k_rows_build<false>, dim3(nWin), dim3(RB_THREADS), lds, st, b->dGroups, dList, dBase, nL, b->nRows, (uint32_t) nTbl,
 		(uint32_t*) dOff, nullptr, nullptr, nullptr, nullptr, dOver);
 	CLA_HIP(hipGetLastError());
 	std::vector<uint32_t> sizes(nWin);
@@ -309,7 +296,7 @@ static int rows_plan(cla_block* b) {
 	b->derivedBytes += (int64_t) (idxBytes + listBytes + sizeBytes + hdrBytes + permBytes + dataBytes);
 	CLA_HIP(hipMemsetAsync((char*) b->dRowsData + dataBytes - 64 * sizeof(u16x4), 0, 64 * sizeof(u16x4), st));
 	CLA_HIP(hipMemcpyAsync(dOff, offs.data(), sizeof(uint64_t) * (size_t) nWin, hipMemcpyHostToDevice, st));
-	hipLaunchKernelGGL(k_rows_build<true>, dim3(nWin), dim3(256), lds, st, b->dGroups, dList, dBase, nL, b->nRows, (uint32_t) nTbl,
+	hipLaunchKernelGGL(k_rows_build<true>, dim3(nWin), dim3(RB_THREADS), lds, st, b->dGroups, dList, dBase, nL, b->nRows, (uint32_t) nTbl,
 		nullptr, dOff, dHdr, dPerm, (u16x4*) b->dRowsData, dOver);
 	CLA_HIP(hipGetLastError());
 	CLA_HIP(hipStreamSynchronize(st)); // `offs` goes out of scope
