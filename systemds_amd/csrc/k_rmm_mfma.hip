@@ -129,7 +129,8 @@ __global__ __launch_bounds__(WAVES * 64) void k_rmm_mfma(const MfSlab* __restric
 	// seventh of the kernel's time); a ragged last tile or narrower codes go through mf_fill_codes_slow.
 	// (Letting only one of the two waves of a SIMD issue a fill, so that the other keeps the matrix pipe busy
 	// meanwhile, was measured slower with either assignment of waves: 2.84 / 2.91 ms against 2.79; so were two
-	// single-buffered blocks of four waves per CU, one filling while the other multiplies: 3.25 ms.)
+	// single-buffered blocks of four waves per CU, one filling while the other multiplies: 3.25 ms, and two
+	// double-buffered ones on half-size slabs (256-row tiles, twice the dictionary traffic from L2): 3.18 ms.)
 	constexpr int FW = WAVES;
 	auto copy_region = [&](const uint8_t* src, uint8_t* dst, int bytes, int fw, int rot) {
 		const int ew = (fw + rot) & (FW - 1);
