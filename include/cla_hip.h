@@ -209,9 +209,10 @@ int64_t cla_decompress_dev(cla_handle h, double* dOut);
  * per-group form is counts x dictionary (AColGroupCompressed.unaryAggregateOperations,
  * CG/AColGroupCompressed.java:137-205): op = sum, sum of squares, min, max; dir = all cells
  * (out[1]), per row (out[nRows]), per column (out[nCols]). Returns the number of non-zero
- * cells of the result. Not on the device path (CLA_ERR_UNSUPPORTED, caller falls back as for
- * any unsupported combination): row minima / maxima, row sums of squares with an
- * uncompressed group, anything but plain sums on overlapping groups. */
+ * cells of the result. What has no such form is aggregated over decompressed chunks of rows (at most
+ * 256 MiB of scratch), as CLALibCompAgg.decompressingAggregate does (C/lib/CLALibCompAgg.java:220-232,
+ * 419-452, 605-720): everything but plain sums on overlapping groups, row minima / maxima, row sums of
+ * squares next to an uncompressed group. */
 enum cla_agg_op { CLA_AGG_SUM = 0, CLA_AGG_SUMSQ = 1, CLA_AGG_MIN = 2, CLA_AGG_MAX = 3 };
 enum cla_agg_dir { CLA_AGG_ALL = 0, CLA_AGG_ROW = 1, CLA_AGG_COL = 2 };
 int64_t cla_aggregate(cla_handle h, int32_t op, int32_t dir, double* out);

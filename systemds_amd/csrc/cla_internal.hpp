@@ -230,6 +230,7 @@ int launch_tsmm_decode(cla_block* b, double* dOut);
 int launch_rmm_decode(cla_block* b, const double* dB, int q, const double* dConstRow, double* dOut,
 	unsigned long long* dNnz);
 int launch_decompress(cla_block* b, double* dOut, unsigned long long* dNnz);
+int launch_decompress_rows(cla_block* b, int64_t r0, int64_t r1, double* dOut);
 int launch_lmm(cla_block* b, const double* dY, int p, double* dOut, unsigned long long* dNnz);
 int launch_preagg(cla_block* b, int group, const double* dY, int p, double* dPre);
 int launch_tsmm(cla_block* b, double* dOut, unsigned long long* dNnz);

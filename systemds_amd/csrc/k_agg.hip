@@ -8,6 +8,14 @@
 //   k_agg_cols_dict    per dictionary group and column: counts x f(dictionary)
 //   k_agg_cols_dense   uncompressed groups: partial column aggregates per row chunk
 //   k_agg_finish       constants, untouched columns, reduction over all cells, non-zero count
+// What has no such form goes through decompressed row chunks, as the reference's decompressing
+// aggregate does (CLALibCompAgg.decompressingAggregate / UAOverlappingTask, C/lib/CLALibCompAgg.java:
+// 419-452, 605-720: rows [rl, ru) of all groups into a temporary dense block, then the dense operator):
+// everything but sums on overlapping groups (requireDecompression, :220-232), row minima and maxima,
+// row sums of squares next to an uncompressed group.
+//   k_agg_chunk_rows   one value per row of a decompressed chunk
+//   k_agg_chunk_cols   partial column aggregates per 4096 rows of a decompressed chunk
+//   k_agg_chunk_finish folds the partials, reduces to one cell for all cells, counts non-zero cells
 #include "../../include/cla_hip.h"
 #include "cla_device.hpp"
 #include <vector>
@@ -123,6 +131,108 @@ __global__ __launch_bounds__(256) void k_agg_finish(double* __restrict__ colAgg,
 	count_add(nnz, cnt);
 }
 
+// ---------------------------------------------------------------------------
+// Aggregates of a decompressed chunk of rows (dense, row-major, nCols wide)
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ double agg_term(int op, double v) { return op == CLA_AGG_SUMSQ ? v * v : v; }
+
+// a wave per row
+__global__ __launch_bounds__(256) void k_agg_chunk_rows(const double* __restrict__ dense, int64_t rows, int nCols, int op,
+	double* __restrict__ out, unsigned long long* __restrict__ nnz) {
+	const int64_t r = (int64_t) blockIdx.x * 4 + (threadIdx.x >> 6);
+	const int lane = threadIdx.x & 63;
+	int cnt = 0;
+	if(r < rows) {
+		double a = agg_identity(op);
+		for(int c = lane; c < nCols; c += 64) a = agg_combine(op, a, agg_term(op, dense[(size_t) r * nCols + c]));
+#pragma unroll
+		for(int d = 32; d > 0; d >>= 1) a = agg_combine(op, a, __shfl_down(a, d, WAVE));
+		if(lane == 0) { out[r] = a; cnt = a != 0.0; }
+	}
+	count_add(nnz, cnt);
+}
+
+constexpr int AGG_CHUNK_ROWS = 4096;
+
+// block = 4096 rows: a thread keeps one column (of a pass of at most 256 columns) and walks the rows that
+// 256 threads do not cover side by side; partial[block * nCols + c]
+__global__ __launch_bounds__(256) void k_agg_chunk_cols(const double* __restrict__ dense, int64_t rows, int nCols, int op,
+	double* __restrict__ partial) {
+	__shared__ double red[256];
+	const int tid = threadIdx.x;
+	const int64_t rBeg = (int64_t) blockIdx.x * AGG_CHUNK_ROWS, rEnd = min(rows, rBeg + AGG_CHUNK_ROWS);
+	const int perPass = min(nCols, 256), side = 256 / perPass;
+	const int rr = tid / perPass, cc = tid - rr * perPass;
+	for(int cb = 0; cb < nCols; cb += perPass) {
+		const int c = cb + cc;
+		double a = agg_identity(op);
+		if(rr < side && c < nCols)
+			for(int64_t r = rBeg + rr; r < rEnd; r += side) a = agg_combine(op, a, agg_term(op, dense[(size_t) r * nCols + c]));
+		__syncthreads();
+		red[tid] = a;
+		__syncthreads();
+		if(rr == 0 && c < nCols) {
+			for(int k = 1; k < side; k++) a = agg_combine(op, a, red[k * perPass + cc]);
+			partial[(size_t) blockIdx.x * nCols + c] = a;
+		}
+	}
+}
+
+// one block
+__global__ __launch_bounds__(256) void k_agg_chunk_finish(const double* __restrict__ partial, int nParts, int nCols, int op, int dir,
+	double* __restrict__ out, unsigned long long* __restrict__ nnz) {
+	__shared__ double red[4];
+	double all = agg_identity(op);
+	int cnt = 0;
+	for(int c = threadIdx.x; c < nCols; c += 256) {
+		double v = agg_identity(op);
+		for(int i = 0; i < nParts; i++) v = agg_combine(op, v, partial[(size_t) i * nCols + c]);
+		if(dir == CLA_AGG_COL) { out[c] = v; cnt += v != 0.0; }
+		all = agg_combine(op, all, v);
+	}
+	all = block_reduce(op, all, red);
+	if(dir == CLA_AGG_ALL && threadIdx.x == 0) { out[0] = all; cnt = all != 0.0; }
+	count_add(nnz, cnt);
+}
+
+// The aggregate of the decompressed block, chunk of rows by chunk of rows (at most 256 MiB decompressed at a time).
+static int launch_aggregate_decompressed(cla_block* b, int op, int dir, double* dOut, unsigned long long* dNnz) {
+	const int nCols = b->nCols;
+	const int64_t nRows = b->nRows;
+	hipStream_t st = b->stream;
+	clear_stats(b);
+	CLA_HIP(hipMemsetAsync(dNnz, 0, sizeof(unsigned long long), st));
+	const int64_t chunkRows = std::min<int64_t>(nRows, std::max<int64_t>(AGG_CHUNK_ROWS,
+		((int64_t) 256 << 20) / ((int64_t) sizeof(double) * nCols) / AGG_CHUNK_ROWS * AGG_CHUNK_ROWS));
+	const int64_t nParts = (nRows + AGG_CHUNK_ROWS - 1) / AGG_CHUNK_ROWS;
+	const size_t denseBytes = (sizeof(double) * (size_t) chunkRows * nCols + 255) & ~(size_t) 255;
+	const size_t partBytes = dir == CLA_AGG_ROW ? 0 : sizeof(double) * (size_t) nParts * nCols;
+	int rc = ensure_scratch(b, denseBytes + partBytes);
+	if(rc) return rc;
+	double* dDense = (double*) b->dScratch;
+	double* dPartial = (double*) ((uint8_t*) b->dScratch + denseBytes);
+	for(int64_t r0 = 0; r0 < nRows; r0 += chunkRows) {
+		const int64_t r1 = std::min(nRows, r0 + chunkRows), rows = r1 - r0;
+		if((rc = launch_decompress_rows(b, r0, r1, dDense))) return rc;
+		if(dir == CLA_AGG_ROW) {
+			Prof pf(b, "k_agg_chunk_rows", (long) ((rows + 3) / 4), 256, 0, (double) rows * nCols * 8);
+			hipLaunchKernelGGL(k_agg_chunk_rows, dim3((unsigned) ((rows + 3) / 4)), dim3(256), 0, st, dDense, rows, nCols, op, dOut + r0, dNnz);
+		}
+		else {
+			const unsigned grid = (unsigned) ((rows + AGG_CHUNK_ROWS - 1) / AGG_CHUNK_ROWS);
+			Prof pf(b, "k_agg_chunk_cols", grid, 256, 0, (double) rows * nCols * 8);
+			hipLaunchKernelGGL(k_agg_chunk_cols, dim3(grid), dim3(256), 0, st, dDense, rows, nCols, op,
+				dPartial + (size_t) (r0 / AGG_CHUNK_ROWS) * nCols);
+		}
+	}
+	if(dir != CLA_AGG_ROW) {
+		Prof pf(b, "k_agg_chunk_finish", 1, 256, 0, 0);
+		hipLaunchKernelGGL(k_agg_chunk_finish, dim3(1), dim3(256), 0, st, dPartial, (int) nParts, nCols, op, dir, dOut, dNnz);
+	}
+	CLA_HIP(hipGetLastError());
+	return 0;
+}
+
 __global__ __launch_bounds__(256) void k_fill(double* __restrict__ p, int64_t n, double v) {
 	const int64_t i = (int64_t) blockIdx.x * 256 + threadIdx.x;
 	if(i < n) p[i] = v;
@@ -163,19 +273,11 @@ int launch_aggregate(cla_block* b, int op, int dir, double* dOut, unsigned long 
 			if(rowData) touched[c] = 1;
 		}
 	}
-	if(overlap && op != CLA_AGG_SUM) {
-		set_error("aggregate: overlapping column groups support sums only");
-		return -CLA_ERR_UNSUPPORTED;
+	if(nRows > 0 && nCols > 0) {
+		const bool rowNoTable = dir == CLA_AGG_ROW && (op == CLA_AGG_MIN || op == CLA_AGG_MAX || (op == CLA_AGG_SUMSQ && b->hasUnc));
+		if((overlap && op != CLA_AGG_SUM) || rowNoTable) return launch_aggregate_decompressed(b, op, dir, dOut, dNnz);
 	}
 	if(dir == CLA_AGG_ROW) {
-		if(op == CLA_AGG_MIN || op == CLA_AGG_MAX) {
-			set_error("aggregate: row minima and maxima are not on the device path");
-			return -CLA_ERR_UNSUPPORTED;
-		}
-		if(op == CLA_AGG_SUMSQ && b->hasUnc) {
-			set_error("aggregate: row sums of squares with an uncompressed group are not on the device path");
-			return -CLA_ERR_UNSUPPORTED;
-		}
 		// rowSums(X) = X %*% 1; the squares use per-tuple tables sum_j ((d + c)^2 - c^2) instead of dict x B
 		if(b->dOnes == nullptr) {
 			CLA_HIP(hipMalloc((void**) &b->dOnes, sizeof(double) * (size_t) std::max(nCols, 1)));

@@ -809,34 +809,36 @@ __global__ __launch_bounds__(256) void k_decompress_fill(double* __restrict__ ou
 	for(int64_t i = (int64_t) blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t) gridDim.x * 256) out[i] = constV[i % nCols];
 }
 
-__global__ __launch_bounds__(256) void k_decompress_rows(const DGroup* __restrict__ groups, int g, int64_t nRows, int nCols,
+__global__ __launch_bounds__(256) void k_decompress_rows(const DGroup* __restrict__ groups, int g, int64_t r0, int64_t r1, int nCols,
 	double* __restrict__ out) {
 	const DGroup G = dgroup(groups + (g));
 	const int64_t idx = (int64_t) blockIdx.x * 256 + threadIdx.x;
-	if(idx >= nRows * G.nColG) return;
-	const int64_t r = idx / G.nColG;
-	const int j = (int) (idx - r * G.nColG);
+	if(idx >= (r1 - r0) * G.nColG) return;
+	const int64_t rr = idx / G.nColG, r = r0 + rr;
+	const int j = (int) (idx - rr * G.nColG);
 	double v;
-	if(G.type == G_UNC) v = G.dense[idx];
+	if(G.type == G_UNC) v = G.dense[(size_t) r * G.nColG + j];
 	else {
 		const int code = G.type == G_DDC ? load_code(G.codes, G.codeWidth, r) : G.runCode[rle_find(G.runStart, G.nRuns, (int32_t) r)];
 		if(code < 0) return;
 		v = G.dict[(size_t) code * G.nColG + j];
 	}
-	unsafeAtomicAdd(&out[(size_t) r * nCols + G.cols[j]], v);
+	unsafeAtomicAdd(&out[(size_t) rr * nCols + G.cols[j]], v);
 }
 
+// rows [r0, r1) of the group go to out rows 0 .. r1 - r0; a block of list entries whose rows all lie outside leaves early
 template <int W>
-__global__ __launch_bounds__(256) void k_decompress_sdc(const DGroup* __restrict__ groups, int g, int nCols,
+__global__ __launch_bounds__(256) void k_decompress_sdc(const DGroup* __restrict__ groups, int g, int64_t r0, int64_t r1, int nCols,
 	double* __restrict__ out) {
 	const DGroup G = dgroup(groups + (g));
 	const int chunk = blockIdx.x, wave = threadIdx.x >> 6;
-	if(chunk == 0 && threadIdx.x == 0 && G.nOffsets > 0) {
+	if(chunk == 0 && threadIdx.x == 0 && G.nOffsets > 0 && G.first >= r0 && G.first < r1) {
 		const int code = load_code(G.codes, G.codeWidth, 0);
-		for(int j = 0; j < G.nColG; j++) unsafeAtomicAdd(&out[(size_t) G.first * nCols + G.cols[j]], G.dict[(size_t) code * G.nColG + j]);
+		for(int j = 0; j < G.nColG; j++) unsafeAtomicAdd(&out[(size_t) (G.first - r0) * nCols + G.cols[j]], G.dict[(size_t) code * G.nColG + j]);
 	}
 	if(chunk >= G.nCkpt) return;
 	const OffState st = G.ckpt[chunk];
+	if(st.row >= r1 || G.ckpt[chunk + 1].row < r0) return; // rows only grow along the list; entry nCkpt is the final state
 	int32_t row = st.row, emit = st.emit;
 	int32_t rows[4], didx[4];
 	unsigned mask;
@@ -845,10 +847,10 @@ __global__ __launch_bounds__(256) void k_decompress_sdc(const DGroup* __restrict
 	sdc_decode256<W>(G.deltas, G.nDeltas, base + wave * 256, row, emit, rows, didx, mask);
 #pragma unroll
 	for(int k = 0; k < 4; k++)
-		if(mask & (1u << k)) {
+		if((mask & (1u << k)) && rows[k] >= r0 && rows[k] < r1) {
 			const int code = load_code(G.codes, G.codeWidth, didx[k]);
 			for(int j = 0; j < G.nColG; j++)
-				unsafeAtomicAdd(&out[(size_t) rows[k] * nCols + G.cols[j]], G.dict[(size_t) code * G.nColG + j]);
+				unsafeAtomicAdd(&out[(size_t) (rows[k] - r0) * nCols + G.cols[j]], G.dict[(size_t) code * G.nColG + j]);
 		}
 }
 
@@ -858,13 +860,12 @@ __global__ __launch_bounds__(256) void k_count_nnz2(const double* __restrict__ x
 	count_add(nnz, cnt);
 }
 
-int launch_decompress(cla_block* b, double* dOut, unsigned long long* dNnz) {
+// dOut[(r - r0) * nCols + c] = X[r, c] for r0 <= r < r1
+int launch_decompress_rows(cla_block* b, int64_t r0, int64_t r1, double* dOut) {
 	const int nG = (int) b->groups.size();
-	const int64_t nRows = b->nRows, n = nRows * b->nCols;
+	const int64_t n = (r1 - r0) * b->nCols;
 	hipStream_t st = b->stream;
-	clear_stats(b);
-	CLA_HIP(hipMemsetAsync(dNnz, 0, sizeof(unsigned long long), st));
-	if(n == 0) return 0;
+	if(n <= 0) return 0;
 	const unsigned fg = (unsigned) std::min<int64_t>((n + 255) / 256, (int64_t) g_numCU * 64);
 	{
 		Prof pf(b, "k_decompress_fill", fg, 256, 0, 0);
@@ -876,16 +877,30 @@ int launch_decompress(cla_block* b, double* dOut, unsigned long long* dNnz) {
 			if(G.nOffsets == 0) continue;
 			const unsigned sg = (unsigned) std::max(G.nCkpt, 1);
 			Prof pf(b, "k_decompress_sdc", sg, 256, 0, 0);
-			if(G.deltaWidth == 1) hipLaunchKernelGGL(k_decompress_sdc<1>, dim3(sg), dim3(256), 0, st, b->dGroups, g, b->nCols, dOut);
-			else hipLaunchKernelGGL(k_decompress_sdc<2>, dim3(sg), dim3(256), 0, st, b->dGroups, g, b->nCols, dOut);
+			if(G.deltaWidth == 1) hipLaunchKernelGGL(k_decompress_sdc<1>, dim3(sg), dim3(256), 0, st, b->dGroups, g, r0, r1, b->nCols, dOut);
+			else hipLaunchKernelGGL(k_decompress_sdc<2>, dim3(sg), dim3(256), 0, st, b->dGroups, g, r0, r1, b->nCols, dOut);
 		}
 		else {
-			const int64_t m = nRows * G.nColG;
+			const int64_t m = (r1 - r0) * G.nColG;
+			if(m == 0) continue;
 			Prof pf(b, "k_decompress_rows", (long) ((m + 255) / 256), 256, 0, 0);
-			hipLaunchKernelGGL(k_decompress_rows, dim3((unsigned) ((m + 255) / 256)), dim3(256), 0, st, b->dGroups, g, nRows,
+			hipLaunchKernelGGL(k_decompress_rows, dim3((unsigned) ((m + 255) / 256)), dim3(256), 0, st, b->dGroups, g, r0, r1,
 				b->nCols, dOut);
 		}
 	}
+	CLA_HIP(hipGetLastError());
+	return 0;
+}
+
+int launch_decompress(cla_block* b, double* dOut, unsigned long long* dNnz) {
+	const int64_t nRows = b->nRows, n = nRows * b->nCols;
+	hipStream_t st = b->stream;
+	clear_stats(b);
+	CLA_HIP(hipMemsetAsync(dNnz, 0, sizeof(unsigned long long), st));
+	if(n == 0) return 0;
+	const int rc = launch_decompress_rows(b, 0, nRows, dOut);
+	if(rc) return rc;
+	const unsigned fg = (unsigned) std::min<int64_t>((n + 255) / 256, (int64_t) g_numCU * 64);
 	{
 		Prof pf(b, "k_count_nnz", fg, 256, 0, 0);
 		hipLaunchKernelGGL(k_count_nnz2, dim3(fg), dim3(256), 0, st, dOut, n, dNnz);

@@ -645,8 +645,8 @@ struct CLALibDecompress {
 
 // CLALibCompAgg.aggregateUnary (C/lib/CLALibCompAgg.java:78-127) for sum, sumSq, min, max in the
 // three directions of the reference's index functions (ReduceAll, ReduceCol = per row,
-// ReduceRow = per column). Combinations the device path does not take raise
-// NotImplementedException, where the reference's caller would decompress and aggregate.
+// ReduceRow = per column). Where the reference decompresses and aggregates (overlapping blocks
+// for all but sums, :220-232), the library does the same on the device, chunk of rows by chunk of rows.
 enum class AggOp { SUM = CLA_AGG_SUM, SUMSQ = CLA_AGG_SUMSQ, MIN = CLA_AGG_MIN, MAX = CLA_AGG_MAX };
 enum class AggDir { ReduceAll = CLA_AGG_ALL, ReduceCol = CLA_AGG_ROW, ReduceRow = CLA_AGG_COL };
 

@@ -1,5 +1,7 @@
 """GPU parity of the unary aggregates on compressed blocks (cla_aggregate), against the
-aggregate of the decompressed matrix: sum / sumSq by long-double accumulation at the 1e-12
+aggregate of the decompressed matrix (also where the library itself aggregates decompressed row chunks: row
+minima / maxima, row sums of squares next to an uncompressed group, everything but sums on overlapping groups,
+CLALibCompAgg.java:220-232, 419-452): sum / sumSq by long-double accumulation at the 1e-12
 bar of the multiply path (scale = sum of |terms|), min / max up to the rounding of the SDC
 default morph ((dict - default) + default), which the reference's decompression has as well.
 Mirrors the aggregate cases of the reference's CompressedTestBase (T/CompressedTestBase.java
@@ -44,29 +46,38 @@ def check(cla, specs, D, n_rows, n_cols, op, direction, what):
 def test_mixed_groups(cla, ora, op, direction, seed, n_rows, with_unc):
     specs, n_cols = mixed_block(seed, n_rows, with_unc=with_unc)
     D = ora.np_decompress(specs, n_rows, n_cols)
-    if direction == "row" and (op in ("min", "max") or (op == "sumsq" and with_unc)):
-        blk = cla.build_block(n_rows, n_cols, specs)
-        with pytest.raises(cla.ClaError) as e:
-            blk.aggregate(op, direction)
-        blk.close()
-        assert e.value.code == cla.ERR_UNSUPPORTED
-        return
     check(cla, specs, D, n_rows, n_cols, op, direction, "mixed")
 
 
+@pytest.mark.parametrize("op", OPS)
 @pytest.mark.parametrize("direction", DIRS)
-def test_overlapping_groups_sum_only(cla, ora, direction):
-    """Sums are linear in the groups (CLALibCompAgg.java: overlapping blocks aggregate per group for sum-like
-    operators and decompress otherwise); everything else is refused on overlapping blocks."""
-    n_rows = 5000
-    specs, n_cols = mixed_block(5, n_rows, with_unc=False, overlap=True)
+@pytest.mark.parametrize("n_rows,with_unc", [(5000, False), (9001, True)])
+def test_overlapping_groups(cla, ora, op, direction, n_rows, with_unc):
+    """Sums are linear in the groups; everything else on an overlapping block is the aggregate of the sum of the
+    groups' cells (CLALibCompAgg.requireDecompression, CLALibCompAgg.java:220-232)."""
+    specs, n_cols = mixed_block(5, n_rows, with_unc=with_unc, overlap=True)
     D = ora.np_decompress(specs, n_rows, n_cols)
-    check(cla, specs, D, n_rows, n_cols, "sum", direction, "overlap")
-    blk = cla.build_block(n_rows, n_cols, specs)
-    with pytest.raises(cla.ClaError) as e:
-        blk.aggregate("max", "col")
-    blk.close()
-    assert e.value.code == cla.ERR_UNSUPPORTED
+    check(cla, specs, D, n_rows, n_cols, op, direction, "overlap")
+
+
+def test_decompressed_chunks_of_many_rows_and_wide_blocks(cla, ora):
+    """More rows than one decompressed chunk holds and more than 256 columns (several column passes); lists with
+    2-byte offsets, whose blocks of entries are skipped where they lie outside the chunk."""
+    from systemds_amd import synth
+    rng = np.random.default_rng(8)
+    n_rows = 140001   # 300 columns: 111848 rows per 256 MiB chunk
+    specs = []
+    for g in range(100):
+        specs.append(synth.sdc_group(np.random.default_rng((8, g)), n_rows, np.array([3 * g], np.int32), 5, [0.05, 0.0008][g % 2], [None, 0.5][g % 3 == 0]))
+        specs.append(synth.GroupSpec("ddc", np.array([3 * g + 1, 3 * g + 2], np.int32), rng.standard_normal((7, 2)), rng.integers(0, 7, n_rows).astype(np.uint8)))
+    D = ora.np_decompress(specs, n_rows, 300)
+    for op, direction in (("min", "row"), ("max", "row")):
+        check(cla, specs, D, n_rows, 300, op, direction, "wide")
+    # the same cells under a second set of groups: column and overall aggregates of the summed cells
+    more = [synth.GroupSpec("ddc", np.arange(300, dtype=np.int32)[i::3].copy(), rng.standard_normal((4, 100)), rng.integers(0, 4, n_rows).astype(np.uint8)) for i in range(3)]
+    D2 = ora.np_decompress(specs + more, n_rows, 300)
+    for op, direction in (("max", "col"), ("min", "all"), ("sumsq", "col"), ("sumsq", "row")):
+        check(cla, specs + more, D2, n_rows, 300, op, direction, "wide overlap")
 
 
 @pytest.mark.parametrize("cfg,scale", [("config2", 200), ("config3", 200), ("config4", 200), ("config5", 500)])
@@ -77,8 +88,6 @@ def test_baseline_configs_scaled(cla, ora, cfg, scale):
     D = ora.np_decompress(c["groups"], n_rows, n_cols)
     for op in OPS:
         for direction in DIRS:
-            if direction == "row" and (op in ("min", "max") or (op == "sumsq" and cfg == "config5")):
-                continue
             check(cla, c["groups"], D, n_rows, n_cols, op, direction, cfg)
 
 
@@ -101,8 +110,10 @@ def test_host_layer_driver(H, ora, cla):
     a = agg(cmb, H.AggOp.SUMSQ, H.AggDir.ReduceAll, 4)
     ref, scale = truth(D, "sumsq", "all")
     assert_fp64_close(a.toArray().reshape(-1), ref, scale, what="sumSq")
-    with pytest.raises(H.NotImplementedException):
-        agg(cmb, H.AggOp.MIN, H.AggDir.ReduceCol, 4)
+    m = agg(cmb, H.AggOp.MIN, H.AggDir.ReduceCol, 4)
+    assert (m.getNumRows(), m.getNumColumns()) == (n_rows, 1)
+    ref, scale = truth(D, "min", "row")
+    assert_fp64_close(m.toArray().reshape(-1), ref, scale, what="rowMins")
 
 
 @pytest.mark.parametrize("direction", ["all", "col"])

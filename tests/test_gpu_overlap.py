@@ -45,9 +45,11 @@ def test_mixed_groups(cla, ora, seed, n_rows, q):
     out, nnz = child.tsmm()
     assert np.array_equal(out, out.T) and nnz == np.count_nonzero(out)
     assert_fp64_close(out, ora.longdouble_matmul(P.T, P), np.abs(P).T @ np.abs(P), what="t(XB) %*% (XB)", n_terms=n_rows)
-    with pytest.raises(cla.ClaError) as e:
-        child.aggregate("max", "col")
-    assert e.value.code == cla.ERR_UNSUPPORTED
+    # neither are maxima: aggregated over decompressed row chunks (CLALibCompAgg.java:220-232)
+    out, _ = child.aggregate("max", "col")
+    assert_fp64_close(out, P.max(axis=0), np.abs(D).max(axis=0) @ np.abs(B) + 2.0, what="colMaxs of XB")
+    out, _ = child.aggregate("min", "row")
+    assert_fp64_close(out, P.min(axis=1), (np.abs(D) @ np.abs(B)).max(axis=1) + 2.0, what="rowMins of XB")
     grand = child.rmm_overlapping(rng.standard_normal((q, 2)))   # and again, from the overlapping block
     child.close()
     out, _ = grand.decompress()
