@@ -291,6 +291,7 @@ void cla_block_free(cla_handle b) {
 	if(b->dLaneMeta) (void) hipFree(b->dLaneMeta);
 	if(b->dLaneData) (void) hipFree(b->dLaneData);
 	if(b->dRowsMeta) (void) hipFree(b->dRowsMeta);
+	if(b->dMfPlan) (void) hipFree(b->dMfPlan);
 	if(b->dRowsData) (void) hipFree(b->dRowsData);
 	if(b->dDictPad) (void) hipFree(b->dDictPad);
 	if(b->dCountsAll) (void) hipFree(b->dCountsAll);

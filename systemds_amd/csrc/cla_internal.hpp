@@ -169,6 +169,10 @@ struct cla_block {
 	int laneSlabs = 0, laneDictLds = 0, laneDictTotal = 0; // slabs, dictionary entries of the largest slab / of all
 	size_t laneOff[4] = {0, 0, 0, 0};
 	bool laneLmm = false;            // every listed group has one column (the left multiply's condition)
+	void* dMfPlan = nullptr;         // matrix-core right multiply (k_rmm_mfma.hip): slab descriptors, column info, code streams, B row list
+	int mfState = 0;                 // 0 not planned yet, 1 ready, -1 not eligible
+	int mfNSlabs = 0, mfNColsAll = 0, mfWidth = 1, mfMaxKc = 0, mfNRowCol = 0, mfMaxDict = 0;
+	size_t mfBufBytes = 0, mfOff[4] = {0, 0, 0, 0};
 	void* dRowsMeta = nullptr;       // row-list right multiply (k_sdc_rows.hip): table index, group list, headers, row order
 	void* dRowsData = nullptr;       // the listed groups' entries as row lists, built on first use
 	int rowsState = 0, rowsTbl = 0;  // 0 not planned yet, 1 ready, -1 the lists do not fit; table entries of all listed groups

@@ -14,28 +14,25 @@
 //   D_b[i][j]: i = l / 16, j = l % 4       (one double per lane)
 // (probed on the device with one-hot operands; checked against a CPU product by the parity tests)
 // Here the four blocks are four groups of four rows (A lane l holds row l % 16 of a 16-row tile,
-// decoded column k) and B_b is the same for all blocks: B[column k][16 j + jg] for the jg-th of a lane's
-// 16 accumulators, so that a lane ends up with 16 consecutive output columns of one row.
+// decoded column k) and B_b is the same for all blocks: B[column k][8 (jg / 2) + 2 j + jg % 2] for the jg-th of a
+// lane's 16 accumulators, so that the four lanes of a row hold eight consecutive output columns in each pair of
+// accumulators: 64 contiguous bytes per row and store instruction.
 #include "../../include/cla_hip.h"
 #include "cla_device.hpp"
 #include <algorithm>
 #include <cstring>
+#include <type_traits>
 
 namespace cla {
 
+constexpr int MF_WAVES = 8;                  // waves per block (two per SIMD): 512-row tiles
 constexpr int MF_MT = 4;                     // 16-row tiles per wave
 constexpr int MF_NJ = 16;                    // groups of 4 output columns per pass (64 output columns)
-// B slab in LDS: row k at k * MF_BK, inside it the 16 values of output columns 4 jg + j (jg = 0..15)
-// of lane column j at j * MF_BJ: the 16 distinct 16-byte pieces of a wave's read fall on 16 distinct
+// B slab in LDS: row k at k * MF_BK, inside it the 16 values of lane column j (accumulators jg = 0..15)
+// at j * MF_BJ: the 16 distinct 16-byte pieces of a wave's read fall on 16 distinct
 // bank quads (row stride 16 banks, j stride 36 banks)
 constexpr int MF_BJ = 18;
 constexpr int MF_BK = 4 * MF_BJ;
-// Output staging of a wave: 16 rows; a row is four segments of 16 columns, MF_SEG doubles apart, rows MF_SS
-// doubles apart: the sixteen 16-byte writes of lanes 0-15 (rows 0, 4, 8, 12 x four segments) fall on sixteen
-// distinct groups of four banks (row stride 148 dwords = 20 mod 64, segment stride 36 dwords)
-constexpr int MF_SEG = 18;
-constexpr int MF_SS = 74;
-
 // code stream of a decoded column (device array: at row 0; LDS copy: at the block's first row)
 struct MfSrc {
 	const uint8_t* codes;
@@ -53,12 +50,12 @@ struct MfSlab {
 };
 
 // B in the slab layout: row r of the list (decoded column rowCol[r], -1 = padding) at r * MF_BK,
-// output column n0 + 16 j + jg at j * MF_BJ + jg
+// output column n0 + 8 (jg / 2) + 2 j + jg % 2 at j * MF_BJ + jg
 __global__ __launch_bounds__(128) void k_mfma_blayout(const double* __restrict__ B, int q, int n0, const int32_t* __restrict__ rowCol,
 	double* __restrict__ Bl) {
 	const int r = blockIdx.x, t = threadIdx.x;
 	if(t >= MF_BK) return;
-	const int j = t / MF_BJ, jg = t - j * MF_BJ, col = n0 + 16 * j + jg, gc = rowCol[r];
+	const int j = t / MF_BJ, jg = t - j * MF_BJ, col = n0 + 8 * (jg >> 1) + 2 * j + (jg & 1), gc = rowCol[r];
 	Bl[(size_t) r * MF_BK + t] = (jg < 16 && gc >= 0 && col < q) ? B[(size_t) gc * q + col] : 0.0;
 }
 
@@ -243,50 +240,43 @@ __global__ __launch_bounds__(WAVES * 64) void k_rmm_mfma(const MfSlab* __restric
 			}
 		}
 
-		// epilogue: a 16-row tile at a time through LDS (over the buffer of the tile's last slab; the next
-		// pair's fill goes to the other one), so that every store instruction writes whole output rows;
-		// + constV x B, count non-zeros.
-		// acc[m][n] of lane l is output row 16 m + 4 b + i (b = (l / 4) % 4, i = l / 16), column 16 (l % 4) + n:
-		// a lane writes its 16 consecutive columns as eight 16-byte pieces, then lanes 0-31 / 32-63 read two
-		// rows back as 512 contiguous bytes each (1 KB per store instruction).
-		__syncthreads();
-		double* const stageS = (double*) (lds + (size_t) (buf ^ 1) * bufBytes); // (buf has moved on to the next pair's)
-		const int l32 = lane & 31, rsel = lane >> 5;
-		const int col = n0 + 2 * l32;
-		const double cadd0 = (constRow != nullptr && col < q) ? constRow[col] : 0.0;
-		const double cadd1 = (constRow != nullptr && col + 1 < q) ? constRow[col + 1] : 0.0;
-		double* st = stageS + (size_t) wave * 16 * MF_SS;
-		double* const wp = st + (size_t) (lb * 4 + lk) * MF_SS + lj * MF_SEG;
-		const double* const rp = st + (size_t) rsel * MF_SS + (l32 >> 3) * MF_SEG + 2 * (l32 & 7);
+		// epilogue: straight from the accumulators (+ constV x B, count non-zeros). acc[m][n] of lane l is output
+		// row 16 m + 4 b + i (b = (l / 4) % 4, i = l / 16), column 8 (n / 2) + 2 (l % 4) + n % 2: a store
+		// instruction writes 16 bytes per lane, the four lanes of a row 64 contiguous bytes, and the two halves of
+		// a 128-byte line leave with consecutive instructions. No staging in LDS and no barrier: the waves of a
+		// block reach their stores at different times.
+		const int64_t rowBase = blockRow0 + wave * (MF_MT * 16) + lb * 4 + lk;
+		// (the two forms are separate code: a load of constRow under a branch would put a wait for all outstanding
+		// memory operations, the stores before it included, behind every store)
+		auto store_rows = [&](auto withConst) {
 #pragma unroll
-		for(int m = 0; m < MF_MT; m++) {
+			for(int m = 0; m < MF_MT; m++) {
+				const int64_t row = rowBase + 16 * m;
+				if(row < nRows) {
+					double* const o = out + (size_t) row * q + n0 + 2 * lj;
 #pragma unroll
-			for(int n = 0; n < MF_NJ; n += 2) {
-				f64x2 w;
-				w[0] = acc[m][n]; w[1] = acc[m][n + 1];
-				*(f64x2*) (wp + n) = w;
-			}
-			__builtin_amdgcn_wave_barrier(); // same-wave LDS accesses complete in order
-			const int64_t row0 = blockRow0 + wave * (MF_MT * 16) + m * 16 + rsel;
-#pragma unroll
-			for(int r = 0; r < 16; r += 2) {
-				f64x2 v = *(const f64x2*) (rp + (size_t) r * MF_SS);
-				v[0] += cadd0; v[1] += cadd1;
-				if(row0 + r < nRows) {
-					double* o = &out[(size_t) (row0 + r) * q + col];
-					if(col + 1 < q) {
-						cnt += (v[0] != 0.0) + (v[1] != 0.0);
-						__builtin_nontemporal_store(v, (f64x2*) o);
-					}
-					else if(col < q) {
-						cnt += v[0] != 0.0;
-						__builtin_nontemporal_store(v[0], o);
+					for(int n = 0; n < MF_NJ; n += 2) {
+						const int col = n0 + 4 * n + 2 * lj;
+						f64x2 v;
+						v[0] = acc[m][n]; v[1] = acc[m][n + 1];
+						if constexpr(decltype(withConst)::value) {
+							v[0] += constRow[min(col, q - 1)];
+							v[1] += constRow[min(col + 1, q - 1)];
+						}
+						if(col + 1 < q) {
+							cnt += (v[0] != 0.0) + (v[1] != 0.0);
+							__builtin_nontemporal_store(v, (f64x2*) (o + 4 * n));
+						}
+						else if(col < q) {
+							cnt += v[0] != 0.0;
+							__builtin_nontemporal_store(v[0], o + 4 * n);
+						}
 					}
 				}
 			}
-			__builtin_amdgcn_wave_barrier();
-		}
-		if(tid < 2) stageS[tid] = 0.0; // the staging (of wave 0) lay over that buffer's zero doubles
+		};
+		if(constRow == nullptr) store_rows(std::false_type());
+		else store_rows(std::true_type());
 	} // tiles
 	count_add(nnz, cnt);
 }
@@ -297,10 +287,11 @@ static size_t mf_buf_bytes(size_t dictDoubles, int kc, int width, int rows) {
 	return ((dictDoubles + 1) & ~(size_t) 1) * 8 + (size_t) kc * MF_BK * 8 + (size_t) kc * 4 + (size_t) kc * rows * width;
 }
 
-// Host-side plan + launch. Returns 1 when the block/shape is not eligible (caller
-// uses the gather path), 0 on success, negative on error.
-int launch_rmm_mfma(cla_block* b, const double* dB, int q, const double* dConstRow, double* dOut,
-	unsigned long long* dNnz) {
+// The plan of a block: slabs of groups whose dictionaries, rows of B and code tiles fit a buffer, built at the
+// first call and kept on the device. Returns 1 when the block is not eligible.
+static int mf_plan(cla_block* b) {
+	if(b->mfState != 0) return b->mfState < 0 ? 1 : 0;
+	b->mfState = -1;
 	const int nG = (int) b->groups.size();
 	if(nG == 0 || b->nRows == 0) return 1;
 	int nColsAll = 0, blockWidth = 1; // bytes per element of the code tiles: the widest code of the block
@@ -310,13 +301,11 @@ int launch_rmm_mfma(cla_block* b, const double* dB, int q, const double* dConstR
 		blockWidth = std::max(blockWidth, g.d.codeWidth);
 	}
 	// 8 waves per block (512-row tiles, two waves per SIMD), one block per CU with two slab buffers
-	const int waves = 8;
-	const int rows = waves * MF_MT * 16;
-	const size_t stageBytes = (size_t) waves * 16 * MF_SS * 8;
+	const int rows = MF_WAVES * MF_MT * 16;
 	const int ldsKb = 156;
 	const size_t fixedBytes = (size_t) nColsAll * sizeof(MfSrc) + 32 * sizeof(MfSlab);
 	const size_t ldsTotal = (size_t) std::min(g_ldsPerBlock - 1024, ldsKb * 1024);
-	if(ldsTotal < fixedBytes + 2 * stageBytes) return 1;
+	if(ldsTotal < fixedBytes + 4096) return 1;
 	size_t budget = (ldsTotal - fixedBytes) / 2 & ~(size_t) 15; // per slab buffer
 	auto up16 = [](size_t n) { return (n + 15) & ~(size_t) 15; };
 
@@ -331,85 +320,102 @@ int launch_rmm_mfma(cla_block* b, const double* dB, int q, const double* dConstR
 	// The kernel lays a buffer out for the largest dictionary range and the largest column count of any slab,
 	// which need not be the same slab: when two such buffers exceed LDS, the plan is redone on a smaller budget.
 	for(int attempt = 0;; attempt++) {
-	int colCap = 1 << 30;
-	for(int pass = 0; pass < 2; pass++) {
-		slabs.clear(); info.clear(); colSrc.clear(); rowCol.clear();
-		maxDict = 0; maxKc = 0;
-		int g = 0;
-		while(g < nG) {
-			MfSlab sl;
-			memset(&sl, 0, sizeof(sl));
-			sl.g0 = g; sl.c0 = (int) colSrc.size(); sl.kOff = (int) rowCol.size();
-			sl.dictSrc = b->groups[g].d.dict; // the block's dictionaries lie back to back in group order
-			size_t dictD = 2, goodDict = 2; // the leading zero doubles
-			int nc = 0, goodG = g, goodNc = 0;
+		int colCap = 1 << 30;
+		for(int pass = 0; pass < 2; pass++) {
+			slabs.clear(); info.clear(); colSrc.clear(); rowCol.clear();
+			maxDict = 0; maxKc = 0;
+			int g = 0;
 			while(g < nG) {
-				const DGroup& G = b->groups[g].d;
-				const size_t d2 = dictD + (size_t) G.nVals * G.nColG;
-				const int nc2 = nc + G.nColG;
-				const size_t need = mf_buf_bytes(d2, (nc2 + 3) & ~3, blockWidth, rows);
-				if(need > budget || d2 > 65535 || G.nColG > 0x7fff) break; // dictionary offsets are 16 bit
-				if(nc > 0 && nc2 > colCap) break;
-				for(int j = 0; j < G.nColG; j++) {
-					info.push_back((uint32_t) (dictD + j) | ((uint32_t) G.nColG << 16));
-					MfSrc src;
-					src.codes = (const uint8_t*) G.codes; src.width = G.codeWidth; src.pad = 0;
-					colSrc.push_back(src);
-					rowCol.push_back(b->groups[g].cols[j]);
+				MfSlab sl;
+				memset(&sl, 0, sizeof(sl));
+				sl.g0 = g; sl.c0 = (int) colSrc.size(); sl.kOff = (int) rowCol.size();
+				sl.dictSrc = b->groups[g].d.dict; // the block's dictionaries lie back to back in group order
+				size_t dictD = 2, goodDict = 2; // the leading zero doubles
+				int nc = 0, goodG = g, goodNc = 0;
+				while(g < nG) {
+					const DGroup& G = b->groups[g].d;
+					const size_t d2 = dictD + (size_t) G.nVals * G.nColG;
+					const int nc2 = nc + G.nColG;
+					const size_t need = mf_buf_bytes(d2, (nc2 + 3) & ~3, blockWidth, rows);
+					if(need > budget || d2 > 65535 || G.nColG > 0x7fff) break; // dictionary offsets are 16 bit
+					if(nc > 0 && nc2 > colCap) break;
+					for(int j = 0; j < G.nColG; j++) {
+						info.push_back((uint32_t) (dictD + j) | ((uint32_t) G.nColG << 16));
+						MfSrc src;
+						src.codes = (const uint8_t*) G.codes; src.width = G.codeWidth; src.pad = 0;
+						colSrc.push_back(src);
+						rowCol.push_back(b->groups[g].cols[j]);
+					}
+					dictD = d2; nc = nc2;
+					g++;
+					if(nc % 4 == 0) { goodG = g; goodNc = nc; goodDict = dictD; }
 				}
-				dictD = d2; nc = nc2;
-				g++;
-				if(nc % 4 == 0) { goodG = g; goodNc = nc; goodDict = dictD; }
+				if(g == sl.g0) return 1; // a single group does not fit LDS
+				// a slab that is not the last ends on a multiple of four columns if it can
+				if(g < nG && nc % 4 != 0 && goodG > sl.g0) {
+					info.resize(info.size() - (size_t) (nc - goodNc));
+					colSrc.resize(colSrc.size() - (size_t) (nc - goodNc));
+					rowCol.resize(rowCol.size() - (size_t) (nc - goodNc));
+					g = goodG; nc = goodNc; dictD = goodDict;
+				}
+				sl.g1 = g; sl.nc = nc; sl.dictDoubles = (int32_t) dictD; sl.width = blockWidth;
+				sl.pad = 0; // 1: some code stream of the slab is narrower than the tiles (no plain copy)
+				for(int gg = sl.g0; gg < g; gg++)
+					if(b->groups[gg].d.codeWidth != blockWidth) sl.pad = 1;
+				while(rowCol.size() % 4) { rowCol.push_back(-1); info.push_back(0); }
+				maxDict = std::max(maxDict, (dictD + 1) & ~(size_t) 1);
+				maxKc = std::max(maxKc, (nc + 3) & ~3);
+				slabs.push_back(sl);
 			}
-			if(g == sl.g0) return 1; // a single group does not fit LDS
-			// a slab that is not the last ends on a multiple of four columns if it can
-			if(g < nG && nc % 4 != 0 && goodG > sl.g0) {
-				info.resize(info.size() - (size_t) (nc - goodNc));
-				colSrc.resize(colSrc.size() - (size_t) (nc - goodNc));
-				rowCol.resize(rowCol.size() - (size_t) (nc - goodNc));
-				g = goodG; nc = goodNc; dictD = goodDict;
-			}
-			sl.g1 = g; sl.nc = nc; sl.dictDoubles = (int32_t) dictD; sl.width = blockWidth;
-			sl.pad = 0; // 1: some code stream of the slab is narrower than the tiles (no plain copy)
-			for(int gg = sl.g0; gg < g; gg++)
-				if(b->groups[gg].d.codeWidth != blockWidth) sl.pad = 1;
-			while(rowCol.size() % 4) { rowCol.push_back(-1); info.push_back(0); }
-			maxDict = std::max(maxDict, (dictD + 1) & ~(size_t) 1);
-			maxKc = std::max(maxKc, (nc + 3) & ~3);
-			slabs.push_back(sl);
+			if(slabs.size() > 32) return 1;
+			if(pass == 0) colCap = std::max(4, (int) ((nColsAll + slabs.size() - 1) / slabs.size() + 3) / 4 * 4);
 		}
-		if(slabs.size() > 32) return 1;
-		if(pass == 0) colCap = std::max(4, (int) ((nColsAll + slabs.size() - 1) / slabs.size() + 3) / 4 * 4);
-	}
-	if(2 * up16(std::max(mf_buf_bytes(maxDict, maxKc, blockWidth, rows), stageBytes)) + fixedBytes <= ldsTotal) break;
-	if(attempt == 8) return 1;
-	budget = (budget * 3 / 4) & ~(size_t) 15;
+		if(2 * up16(mf_buf_bytes(maxDict, maxKc, blockWidth, rows)) + fixedBytes <= ldsTotal) break;
+		if(attempt == 8) return 1;
+		budget = (budget * 3 / 4) & ~(size_t) 15;
 	}
 	// (colSrc is indexed by decoded column, info and rowCol by slab row: they differ by the padding rows)
-	hipStream_t st = b->stream;
 	const size_t oSlabs = 0, oInfo = up16(oSlabs + slabs.size() * sizeof(MfSlab)), oSrc = up16(oInfo + info.size() * 4 + 16),
-		oRowCol = up16(oSrc + colSrc.size() * sizeof(MfSrc)), oBl = up16(oRowCol + rowCol.size() * 4),
-		total = oBl + rowCol.size() * MF_BK * 8;
-	int rc = ensure_scratch(b, total + 256);
-	if(rc) return rc;
-	char* base = (char*) b->dScratch;
-	MfSlab* dSlabs = (MfSlab*) (base + oSlabs);
-	uint32_t* dInfo = (uint32_t*) (base + oInfo);
-	MfSrc* dSrc = (MfSrc*) (base + oSrc);
-	int32_t* dRowCol = (int32_t*) (base + oRowCol);
-	double* dBl = (double*) (base + oBl);
-	CLA_HIP(hipMemcpyAsync(dSlabs, slabs.data(), slabs.size() * sizeof(MfSlab), hipMemcpyHostToDevice, st));
-	CLA_HIP(hipMemcpyAsync(dInfo, info.data(), info.size() * 4, hipMemcpyHostToDevice, st));
-	CLA_HIP(hipMemcpyAsync(dSrc, colSrc.data(), colSrc.size() * sizeof(MfSrc), hipMemcpyHostToDevice, st));
-	CLA_HIP(hipMemcpyAsync(dRowCol, rowCol.data(), rowCol.size() * 4, hipMemcpyHostToDevice, st));
-	CLA_HIP(hipStreamSynchronize(st)); // the host vectors go out of scope
+		oRowCol = up16(oSrc + colSrc.size() * sizeof(MfSrc)), total = up16(oRowCol + rowCol.size() * 4);
+	char* base = nullptr;
+	CLA_HIP(hipMalloc((void**) &base, total + 256));
+	b->dMfPlan = base;
+	b->derivedBytes += (int64_t) total + 256;
+	CLA_HIP(hipMemcpy(base + oSlabs, slabs.data(), slabs.size() * sizeof(MfSlab), hipMemcpyHostToDevice));
+	CLA_HIP(hipMemcpy(base + oInfo, info.data(), info.size() * 4, hipMemcpyHostToDevice));
+	CLA_HIP(hipMemcpy(base + oSrc, colSrc.data(), colSrc.size() * sizeof(MfSrc), hipMemcpyHostToDevice));
+	CLA_HIP(hipMemcpy(base + oRowCol, rowCol.data(), rowCol.size() * 4, hipMemcpyHostToDevice));
+	b->mfOff[0] = oSlabs; b->mfOff[1] = oInfo; b->mfOff[2] = oSrc; b->mfOff[3] = oRowCol;
+	b->mfNSlabs = (int) slabs.size(); b->mfNColsAll = nColsAll; b->mfWidth = blockWidth; b->mfMaxKc = maxKc;
+	b->mfNRowCol = (int) rowCol.size(); b->mfMaxDict = (int) maxDict;
+	b->mfBufBytes = up16(mf_buf_bytes(maxDict, maxKc, blockWidth, rows));
+	b->mfState = 1;
+	return 0;
+}
 
-	const size_t bufBytes = up16(std::max(mf_buf_bytes(maxDict, maxKc, blockWidth, rows), stageBytes));
-	const size_t lds = 2 * bufBytes + (size_t) nColsAll * sizeof(MfSrc) + slabs.size() * sizeof(MfSlab);
-	CLA_HIP(hipFuncSetAttribute((const void*) k_rmm_mfma<4, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
-	CLA_HIP(hipFuncSetAttribute((const void*) k_rmm_mfma<8, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
-	CLA_HIP(hipFuncSetAttribute((const void*) k_rmm_mfma<4, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
-	CLA_HIP(hipFuncSetAttribute((const void*) k_rmm_mfma<8, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
+// Plan (once per block) + launch. Returns 1 when the block/shape is not eligible (caller
+// uses the gather path), 0 on success, negative on error.
+int launch_rmm_mfma(cla_block* b, const double* dB, int q, const double* dConstRow, double* dOut,
+	unsigned long long* dNnz) {
+	int rc = mf_plan(b);
+	if(rc) return rc;
+	hipStream_t st = b->stream;
+	const int rows = MF_WAVES * MF_MT * 16;
+	if((rc = ensure_scratch(b, (size_t) b->mfNRowCol * MF_BK * 8 + 256))) return rc;
+	double* dBl = (double*) b->dScratch;
+	char* base = (char*) b->dMfPlan;
+	const MfSlab* dSlabs = (const MfSlab*) (base + b->mfOff[0]);
+	const uint32_t* dInfo = (const uint32_t*) (base + b->mfOff[1]);
+	const MfSrc* dSrc = (const MfSrc*) (base + b->mfOff[2]);
+	const int32_t* dRowCol = (const int32_t*) (base + b->mfOff[3]);
+	const size_t lds = 2 * b->mfBufBytes + (size_t) b->mfNColsAll * sizeof(MfSrc) + (size_t) b->mfNSlabs * sizeof(MfSlab);
+	static size_t ldsSet[2] = {0, 0}; // (racing callers set the same or a larger value)
+	const int wi = b->mfWidth - 1;
+	if(ldsSet[wi] < lds) {
+		if(wi == 0) CLA_HIP(hipFuncSetAttribute((const void*) k_rmm_mfma<MF_WAVES, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
+		else CLA_HIP(hipFuncSetAttribute((const void*) k_rmm_mfma<MF_WAVES, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
+		ldsSet[wi] = lds;
+	}
 	// persistent blocks: one per CU, each walks its row tiles
 	const unsigned grid = (unsigned) std::min<int64_t>((b->nRows + rows - 1) / rows, (int64_t) g_numCU);
 	double codeBytes = 0;
@@ -417,15 +423,14 @@ int launch_rmm_mfma(cla_block* b, const double* dB, int q, const double* dConstR
 	for(int n0 = 0; n0 < q; n0 += 64) {
 		const int qq = std::min(64, q - n0);
 		{
-			Prof pf(b, "k_mfma_blayout", (long) rowCol.size(), 128, 0, 0);
-			hipLaunchKernelGGL(k_mfma_blayout, dim3((unsigned) rowCol.size()), dim3(128), 0, st, dB, q, n0, dRowCol, dBl);
+			Prof pf(b, "k_mfma_blayout", (long) b->mfNRowCol, 128, 0, 0);
+			hipLaunchKernelGGL(k_mfma_blayout, dim3((unsigned) b->mfNRowCol), dim3(128), 0, st, dB, q, n0, dRowCol, dBl);
 		}
-		Prof pf(b, "k_rmm_mfma", grid, waves * 64, (long) lds, codeBytes + (double) b->nRows * qq * 8);
-#define MF_LAUNCH(WV, CW)                                                                                            \
-	hipLaunchKernelGGL((k_rmm_mfma<WV, CW>), dim3(grid), dim3(WV * 64), lds, st, dSlabs, (int) slabs.size(), dInfo, dSrc, \
-		nColsAll, dBl, q, n0, dConstRow, dOut, b->nRows, (int) maxDict, maxKc, (int) bufBytes, dNnz)
-		if(waves == 8) { if(blockWidth == 1) MF_LAUNCH(8, 1); else MF_LAUNCH(8, 2); }
-		else { if(blockWidth == 1) MF_LAUNCH(4, 1); else MF_LAUNCH(4, 2); }
+		Prof pf(b, "k_rmm_mfma", grid, MF_WAVES * 64, (long) lds, codeBytes + (double) b->nRows * qq * 8);
+#define MF_LAUNCH(CW)                                                                                                     \
+	hipLaunchKernelGGL((k_rmm_mfma<MF_WAVES, CW>), dim3(grid), dim3(MF_WAVES * 64), lds, st, dSlabs, b->mfNSlabs, dInfo, dSrc, \
+		b->mfNColsAll, dBl, q, n0, dConstRow, dOut, b->nRows, b->mfMaxDict, b->mfMaxKc, (int) b->mfBufBytes, dNnz)
+		if(b->mfWidth == 1) MF_LAUNCH(1); else MF_LAUNCH(2);
 #undef MF_LAUNCH
 	}
 	CLA_HIP(hipGetLastError());
