@@ -42,7 +42,8 @@ __device__ __forceinline__ double block_reduce(int op, double v, double* red) {
 
 // block = one dictionary group; c = constant part of the column (SDC default, 0 otherwise).
 // sum:    sum_k cnt[k] d[k,j]                      (+ nRows c in the finish)
-// sum sq: sum_k cnt[k] ((d[k,j] + c)^2 - c^2)      (+ nRows c^2 in the finish)
+// sum sq: sum_k cnt[k] (d[k,j] + c)^2 + (nRows - rows with an entry) c^2: terms of one sign, no cancellation
+//         where the cells are small next to c
 // min/max over entries that occur, and 0 when some row of the group has no entry (+ c in the finish)
 __global__ __launch_bounds__(256) void k_agg_cols_dict(const DGroup* __restrict__ groups, const int32_t* __restrict__ countsAll,
 	const double* __restrict__ constV, int64_t nRows, int op, double* __restrict__ out) {
@@ -60,7 +61,7 @@ __global__ __launch_bounds__(256) void k_agg_cols_dict(const DGroup* __restrict_
 		for(int k = tid; k < G.nVals; k += 256) {
 			const double cnt = (double) counts[k], d = G.dict[(size_t) k * nC + j];
 			if(op == CLA_AGG_SUM) a += cnt * d;
-			else if(op == CLA_AGG_SUMSQ) a += cnt * ((d + c) * (d + c) - c * c);
+			else if(op == CLA_AGG_SUMSQ) a += cnt * ((d + c) * (d + c));
 			else if(counts[k] > 0) a = agg_combine(op, a, d);
 		}
 		a = block_reduce(op, a, red);
@@ -68,6 +69,7 @@ __global__ __launch_bounds__(256) void k_agg_cols_dict(const DGroup* __restrict_
 			if(op == CLA_AGG_SUM) unsafeAtomicAdd(&out[G.cols[j]], a); // linear: overlapping groups add up
 			else {
 				if((op == CLA_AGG_MIN || op == CLA_AGG_MAX) && covered < (double) nRows) a = agg_combine(op, a, 0.0);
+				if(op == CLA_AGG_SUMSQ) a += ((double) nRows - covered) * (c * c);
 				out[G.cols[j]] = a;
 			}
 		}
@@ -75,7 +77,7 @@ __global__ __launch_bounds__(256) void k_agg_cols_dict(const DGroup* __restrict_
 }
 
 // grid (row chunks, columns of the group): partial[chunk * nC + j]
-// (sum of squares: the column's filtered constant c enters as (v + c)^2 - c^2, like the dictionary form; n c^2 is added at the end)
+// (sum of squares: with the column's filtered constant c, (v + c)^2)
 __global__ __launch_bounds__(256) void k_agg_cols_dense(const double* __restrict__ dense, int64_t nRows, int nC, int64_t rowsPerBlock,
 	int op, const int32_t* __restrict__ cols, const double* __restrict__ constV, double* __restrict__ partial) {
 	__shared__ double red[4];
@@ -85,7 +87,7 @@ __global__ __launch_bounds__(256) void k_agg_cols_dense(const double* __restrict
 	double a = agg_identity(op);
 	for(int64_t r = r0 + threadIdx.x; r < r1; r += 256) {
 		const double v = dense[(size_t) r * nC + j];
-		a = op == CLA_AGG_SUMSQ ? a + ((v + c) * (v + c) - c * c) : agg_combine(op, a, v);
+		a = op == CLA_AGG_SUMSQ ? a + (v + c) * (v + c) : agg_combine(op, a, v);
 	}
 	a = block_reduce(op, a, red);
 	if(threadIdx.x == 0) partial[(size_t) blockIdx.x * nC + j] = a;
@@ -120,7 +122,7 @@ __global__ __launch_bounds__(256) void k_agg_finish(double* __restrict__ colAgg,
 		const double k = constV[c];
 		double v = colAgg[c];
 		if(op == CLA_AGG_SUM) v += n * k;
-		else if(op == CLA_AGG_SUMSQ) v += n * k * k;
+		else if(op == CLA_AGG_SUMSQ) v = touched[c] ? v : n * k * k;
 		else v = touched[c] ? v + k : k;
 		if(nRows == 0) v = op == CLA_AGG_MIN || op == CLA_AGG_MAX ? agg_identity(op) : 0.0;
 		if(dir == CLA_AGG_COL) { out[c] = v; cnt += v != 0.0; }
