@@ -95,6 +95,20 @@ __device__ __attribute__((noinline)) void mf_fill_codes_slow(const MfSrc* __rest
 	}
 }
 
+// keep: lanes outside the banks of BANK (bit k = lanes 4 k .. 4 k + 3 of every row of 16 lanes) keep their own
+// `keep`, the others take `from` of the lane that CTRL names
+template <int CTRL, int BANK>
+__device__ __forceinline__ double mf_dpp_merge(double keep, double from) {
+	int k[2], f[2];
+	__builtin_memcpy(k, &keep, 8);
+	__builtin_memcpy(f, &from, 8);
+	k[0] = __builtin_amdgcn_update_dpp(k[0], f[0], CTRL, 0xf, BANK, false);
+	k[1] = __builtin_amdgcn_update_dpp(k[1], f[1], CTRL, 0xf, BANK, false);
+	double r;
+	__builtin_memcpy(&r, k, 8);
+	return r;
+}
+
 template <int WAVES, int W>
 __global__ __launch_bounds__(WAVES * 64) void k_rmm_mfma(const MfSlab* __restrict__ slabs, int nSlabs,
 	const uint32_t* __restrict__ infoG, const MfSrc* __restrict__ colSrc, int nColsAll, const double* __restrict__ Bl, int q, int n0,
@@ -240,38 +254,50 @@ __global__ __launch_bounds__(WAVES * 64) void k_rmm_mfma(const MfSlab* __restric
 			}
 		}
 
-		// epilogue: straight from the accumulators (+ constV x B, count non-zeros). acc[m][n] of lane l is output
-		// row 16 m + 4 b + i (b = (l / 4) % 4, i = l / 16), column 8 (n / 2) + 2 (l % 4) + n % 2: a store
-		// instruction writes 16 bytes per lane, the four lanes of a row 64 contiguous bytes, and the two halves of
-		// a 128-byte line leave with consecutive instructions. No staging in LDS and no barrier: the waves of a
-		// block reach their stores at different times.
-		const int64_t rowBase = blockRow0 + wave * (MF_MT * 16) + lb * 4 + lk;
+		// epilogue: straight from the accumulators (+ constV x B, count non-zeros), without staging in LDS and
+		// without a barrier. acc[m][n] of lane l is output row 16 m + 4 b + i (b = (l / 4) % 4, i = l / 16), column
+		// 8 (n / 2) + 2 (l % 4) + n % 2: the four lanes of a quad hold 64 contiguous bytes of a row in each pair of
+		// accumulators. Two neighbouring quads (rows r and r + 4) swap pieces through the cross-lane data path so
+		// that eight lanes hold a whole 128-byte line of one row: a store instruction then writes eight full
+		// lines (stores of half lines reach memory at half the rate on this device).
+		//   first store:  row r,     even quad keeps its first half line, odd quad takes the even quad's second half
+		//   second store: row r + 4, even quad takes the odd quad's first half, odd quad keeps its second half
+		const int odd = lb & 1;
+		const int64_t rowBase = blockRow0 + wave * (MF_MT * 16) + (lb & 2) * 4 + lk;
 		// (the two forms are separate code: a load of constRow under a branch would put a wait for all outstanding
 		// memory operations, the stores before it included, behind every store)
 		auto store_rows = [&](auto withConst) {
+			auto put = [&](int64_t row, int col, f64x2 v) {
+				if(row >= nRows) return;
+				double* const o = out + (size_t) row * q + col;
+				if constexpr(decltype(withConst)::value) {
+					v[0] += constRow[min(col, q - 1)];
+					v[1] += constRow[min(col + 1, q - 1)];
+				}
+				if(col + 1 < q) {
+					cnt += (v[0] != 0.0) + (v[1] != 0.0);
+					__builtin_nontemporal_store(v, (f64x2*) o);
+				}
+				else if(col < q) {
+					cnt += v[0] != 0.0;
+					__builtin_nontemporal_store(v[0], o);
+				}
+			};
 #pragma unroll
 			for(int m = 0; m < MF_MT; m++) {
 				const int64_t row = rowBase + 16 * m;
-				if(row < nRows) {
-					double* const o = out + (size_t) row * q + n0 + 2 * lj;
 #pragma unroll
-					for(int n = 0; n < MF_NJ; n += 2) {
-						const int col = n0 + 4 * n + 2 * lj;
-						f64x2 v;
-						v[0] = acc[m][n]; v[1] = acc[m][n + 1];
-						if constexpr(decltype(withConst)::value) {
-							v[0] += constRow[min(col, q - 1)];
-							v[1] += constRow[min(col + 1, q - 1)];
-						}
-						if(col + 1 < q) {
-							cnt += (v[0] != 0.0) + (v[1] != 0.0);
-							__builtin_nontemporal_store(v, (f64x2*) (o + 4 * n));
-						}
-						else if(col < q) {
-							cnt += v[0] != 0.0;
-							__builtin_nontemporal_store(v[0], o + 4 * n);
-						}
-					}
+				for(int L = 0; L < MF_NJ / 4; L++) {
+					const int col = n0 + 16 * L + 8 * odd + 2 * lj;
+					f64x2 first, second;
+					// odd quads: the second half line of the even quad four lanes below (row_shr:4 = 0x114, banks 1 and 3)
+					first[0] = mf_dpp_merge<0x114, 0xa>(acc[m][4 * L], acc[m][4 * L + 2]);
+					first[1] = mf_dpp_merge<0x114, 0xa>(acc[m][4 * L + 1], acc[m][4 * L + 3]);
+					// even quads: the first half line of the odd quad four lanes above (row_shl:4 = 0x104, banks 0 and 2)
+					second[0] = mf_dpp_merge<0x104, 0x5>(acc[m][4 * L + 2], acc[m][4 * L]);
+					second[1] = mf_dpp_merge<0x104, 0x5>(acc[m][4 * L + 3], acc[m][4 * L + 1]);
+					put(row, col, first);
+					put(row + 4, col, second);
 				}
 			}
 		};
