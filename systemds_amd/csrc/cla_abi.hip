@@ -292,6 +292,7 @@ void cla_block_free(cla_handle b) {
 	if(b->dLaneData) (void) hipFree(b->dLaneData);
 	if(b->dRowsMeta) (void) hipFree(b->dRowsMeta);
 	if(b->dMfPlan) (void) hipFree(b->dMfPlan);
+	dec_plans_drop(b);
 	if(b->dRowsData) (void) hipFree(b->dRowsData);
 	if(b->dDictPad) (void) hipFree(b->dDictPad);
 	if(b->dCountsAll) (void) hipFree(b->dCountsAll);
@@ -676,6 +677,7 @@ int cla_block_set_option(cla_handle b, const char* key, int32_t value) {
 		if(strcmp(e.name, key) == 0) {
 			if(value < e.lo || value > e.hi) { set_error("set_option: %s takes %d..%d (got %d)", key, e.lo, e.hi, value); return -CLA_ERR_INVALID; }
 			b->opt.*(e.field) = value;
+			dec_plans_drop(b); // plans kept with the block were made under the old options
 			return 0;
 		}
 	set_error("set_option: unknown option '%s'", key);

@@ -87,6 +87,8 @@ struct KernelStat {
 	float ms = -1.f;
 };
 
+struct DecPlanCache;
+
 } // namespace cla
 
 struct cla_block {
@@ -169,6 +171,7 @@ struct cla_block {
 	int laneSlabs = 0, laneDictLds = 0, laneDictTotal = 0; // slabs, dictionary entries of the largest slab / of all
 	size_t laneOff[4] = {0, 0, 0, 0};
 	bool laneLmm = false;            // every listed group has one column (the left multiply's condition)
+	cla::DecPlanCache* decPlans = nullptr; // decode kernels (k_rmm_decode.hip): plans per product shape, dropped by dec_plans_drop
 	void* dMfPlan = nullptr;         // matrix-core right multiply (k_rmm_mfma.hip): slab descriptors, column info, code streams, B row list
 	int mfState = 0;                 // 0 not planned yet, 1 ready, -1 not eligible
 	int mfNSlabs = 0, mfNColsAll = 0, mfWidth = 1, mfMaxKc = 0, mfNRowCol = 0, mfMaxDict = 0;
@@ -235,6 +238,7 @@ int launch_rmm_decode(cla_block* b, const double* dB, int q, const double* dCons
 	unsigned long long* dNnz);
 int launch_decompress(cla_block* b, double* dOut, unsigned long long* dNnz);
 int launch_decompress_rows(cla_block* b, int64_t r0, int64_t r1, double* dOut);
+void dec_plans_drop(cla_block* b);
 int launch_lmm(cla_block* b, const double* dY, int p, double* dOut, unsigned long long* dNnz);
 int launch_preagg(cla_block* b, int group, const double* dY, int p, double* dPre);
 int launch_tsmm(cla_block* b, double* dOut, unsigned long long* dNnz);

@@ -697,7 +697,8 @@ struct DecLaunch {
 };
 
 // Dictionaries of more than dictLimit doubles stay in global memory (t(X) %*% X only).
-static int dec_prepare(cla_block* b, bool gram, int q, int rpl, DecLaunch& L, size_t dictLimit = (size_t) 1 << 30) {
+// The plan's device image goes into *dImg (an allocation of its own, kept with the plan).
+static int dec_build_plan(cla_block* b, bool gram, int q, int rpl, DecLaunch& L, size_t dictLimit, void** dImg) {
 	const int nG = (int) b->groups.size();
 	const int nCols = b->nCols;
 	{
@@ -826,11 +827,10 @@ static int dec_prepare(cla_block* b, bool gram, int q, int rpl, DecLaunch& L, si
 	std::memcpy(img.data() + copyBytes + constBytes, cols.data(), colBytes);
 	std::memcpy(img.data() + copyBytes + constBytes + colBytes, plan.data(), planBytes);
 	std::memcpy(img.data() + copyBytes + constBytes + colBytes + planBytes, tasks.data(), taskBytes);
-	int rc = ensure_scratch(b, img.size() + 64);
-	if(rc) return rc;
-	uint8_t* d = (uint8_t*) b->dScratch;
-	CLA_HIP(hipMemcpyAsync(d, img.data(), img.size(), hipMemcpyHostToDevice, b->stream));
-	CLA_HIP(hipStreamSynchronize(b->stream));
+	uint8_t* d = nullptr;
+	CLA_HIP(hipMalloc((void**) &d, img.size() + 64));
+	*dImg = d;
+	CLA_HIP(hipMemcpy(d, img.data(), img.size(), hipMemcpyHostToDevice));
 	DecArgs& A = L.A;
 	A.groups = b->dGroups;
 	A.copies = (const DecCopy*) d;
@@ -846,6 +846,52 @@ static int dec_prepare(cla_block* b, bool gram, int q, int rpl, DecLaunch& L, si
 	const int blocksPerCU = L.lds <= 76 * 1024 ? 2 : 1;
 	L.grid = (unsigned) std::min(nTiles, g_numCU * blocksPerCU);
 	return 0;
+}
+
+// Plans are kept with the block (they depend on the block, the shape of the product and the options only):
+// a call then costs no host planning, no upload and no wait for it.
+struct DecPlanEntry {
+	bool gram;
+	int q, rpl, expand;
+	size_t dictLimit;
+	int rc;
+	DecLaunch L;
+	void* dImg;
+};
+struct DecPlanCache {
+	std::vector<DecPlanEntry> entries;
+};
+
+void dec_plans_drop(cla_block* b) {
+	if(b->decPlans == nullptr) return;
+	for(auto& e : b->decPlans->entries)
+		if(e.dImg) (void) hipFree(e.dImg);
+	delete b->decPlans;
+	b->decPlans = nullptr;
+}
+
+static int dec_prepare(cla_block* b, bool gram, int q, int rpl, DecLaunch& L, size_t dictLimit = (size_t) 1 << 30) {
+	if(b->decPlans == nullptr) b->decPlans = new DecPlanCache();
+	for(auto& e : b->decPlans->entries)
+		if(e.gram == gram && e.q == q && e.rpl == rpl && e.dictLimit == dictLimit && e.expand == b->opt.expandStreams) {
+			L = e.L;
+			return e.rc;
+		}
+	DecPlanEntry e;
+	e.gram = gram; e.q = q; e.rpl = rpl; e.expand = b->opt.expandStreams; e.dictLimit = dictLimit; e.dImg = nullptr;
+	e.rc = dec_build_plan(b, gram, q, rpl, e.L, dictLimit, &e.dImg);
+	if(e.rc < 0) { // an error is not a property of the block: not kept
+		if(e.dImg) (void) hipFree(e.dImg);
+		return e.rc;
+	}
+	if(b->decPlans->entries.size() >= 64) { // (products with many different widths of B: start over)
+		for(auto& o : b->decPlans->entries)
+			if(o.dImg) (void) hipFree(o.dImg);
+		b->decPlans->entries.clear();
+	}
+	b->decPlans->entries.push_back(e);
+	L = e.L;
+	return e.rc;
 }
 
 // Returns 1 when the block/shape is not eligible (caller uses the generic path).
