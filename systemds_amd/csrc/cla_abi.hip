@@ -7,6 +7,8 @@
 #include <cstdarg>
 #include <cstring>
 #include <map>
+#include <mutex>
+#include <unordered_set>
 #include <new>
 #include <stdexcept>
 
@@ -76,6 +78,21 @@ int ensure_tables(cla_block* b, size_t nDoubles) {
 	CLA_HIP(hipMalloc((void**) &b->dTables, nDoubles * sizeof(double)));
 	b->tablesCap = nDoubles;
 	return 0;
+}
+
+hipError_t allow_full_lds(const void* kernel) {
+	static std::mutex mu;
+	static std::unordered_set<const void*> said;
+	std::lock_guard<std::mutex> lk(mu);
+	if(said.count(kernel)) return hipSuccess;
+	// (the kernel's static shared memory counts against the same limit)
+	hipFuncAttributes fa;
+	hipError_t e = hipFuncGetAttributes(&fa, kernel);
+	if(e != hipSuccess) return e;
+	const int room = g_ldsPerBlock - (int) fa.sharedSizeBytes;
+	e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, room > 0 ? room : 0);
+	if(e == hipSuccess) said.insert(kernel);
+	return e;
 }
 
 int ensure_scratch(cla_block* b, size_t bytes) {

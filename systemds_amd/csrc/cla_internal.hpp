@@ -204,6 +204,9 @@ namespace cla {
 
 void set_error(const char* fmt, ...);
 extern int g_ldsPerBlock;   // usable LDS bytes per workgroup
+// Lets a kernel take up to the device's LDS per workgroup as dynamic shared memory; said once per kernel (a value
+// per call could be lowered by a caller on another handle between a call's setting and its launch).
+hipError_t allow_full_lds(const void* kernel);
 extern int g_numCU;
 
 #define CLA_HIP(expr)                                                                              \

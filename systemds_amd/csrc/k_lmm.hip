@@ -224,7 +224,7 @@ static int run_preagg(cla_block* b, const double* dY, int p, double* dPre, int o
 			b->preUsed = true;
 			const size_t lds = direct ? 0 : bytes;
 			Prof pf(b, "k_lmm_preagg_rows", (long) gridRows * p, LMM_THREADS, (long) lds, 0);
-			CLA_HIP(hipFuncSetAttribute((const void*) k_lmm_preagg_rows, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
+			CLA_HIP(allow_full_lds((const void*) k_lmm_preagg_rows));
 			hipLaunchKernelGGL(k_lmm_preagg_rows, dim3(gridRows, p), dim3(LMM_THREADS), lds, st, b->dGroups, g, g1, dY,
 				nRows, rowsPerBlock, dPre, b->totalVals, direct);
 		}
@@ -249,12 +249,12 @@ static int run_preagg(cla_block* b, const double* dY, int p, double* dPre, int o
 		b->preUsed = true;
 		Prof pf(b, "k_lmm_preagg_sdc", (long) grid * p, 256, (long) bytes, algo);
 		if(G.deltaWidth == 1) {
-			CLA_HIP(hipFuncSetAttribute((const void*) k_lmm_preagg_sdc<1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) bytes));
+			CLA_HIP(allow_full_lds((const void*) k_lmm_preagg_sdc<1>));
 			hipLaunchKernelGGL(k_lmm_preagg_sdc<1>, dim3(grid, p), dim3(256), bytes, st, b->dGroups, g, dY, nRows, cpb, dPre,
 				b->totalVals, direct);
 		}
 		else {
-			CLA_HIP(hipFuncSetAttribute((const void*) k_lmm_preagg_sdc<2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) bytes));
+			CLA_HIP(allow_full_lds((const void*) k_lmm_preagg_sdc<2>));
 			hipLaunchKernelGGL(k_lmm_preagg_sdc<2>, dim3(grid, p), dim3(256), bytes, st, b->dGroups, g, dY, nRows, cpb, dPre,
 				b->totalVals, direct);
 		}

@@ -129,7 +129,7 @@ int launch_lmm_u8(cla_block* b, const double* dY, int p, double* dPre) {
 		const size_t lds = (size_t) PER * R * LU_BINS * 8;                                                      \
 		Prof pf(b, "k_lmm_u8", (long) grid * p, LU_THREADS, (long) lds, algo);                                  \
 		auto kern = k_lmm_u8<PER, R, NB>;                                                                       \
-		CLA_HIP(hipFuncSetAttribute((const void*) kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds)); \
+		CLA_HIP(allow_full_lds((const void*) kern)); \
 		hipLaunchKernelGGL(kern, dim3(grid, p), dim3(LU_THREADS), lds, b->stream, b->dGroups, b->dArena,        \
 			b->arenaStride, nG, dY, b->nRows, dPre, b->totalVals);                                              \
 	} while(0)
@@ -334,7 +334,7 @@ int launch_lmm_u8_dot(cla_block* b, const double* dY, int p, double* dOut) {
 	const double algo = (double) p * ((double) b->nRows * nG + (double) b->nRows * 8);
 	Prof pf(b, "k_lmm_u8_dot", (long) grid * p, LD_THREADS, (long) lds, algo);
 	auto kern = k_lmm_u8_dot<PER, 5, 4, 2>;
-	CLA_HIP(hipFuncSetAttribute((const void*) kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
+	CLA_HIP(allow_full_lds((const void*) kern));
 	hipLaunchKernelGGL(kern, dim3(grid, p), dim3(LD_THREADS), lds, b->stream, b->dArena, b->arenaStride, nG, b->dDictPad, dCol0, dY,
 		b->nRows, dOut, b->nCols);
 	CLA_HIP(hipGetLastError());

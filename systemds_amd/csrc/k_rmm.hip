@@ -626,7 +626,7 @@ int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned lon
 #define LAUNCH_Q1(CWV, RPTV, THR)                                                                               \
 	do {                                                                                                        \
 		auto kern = k_rmm_q1_ddc<CWV, RPTV, THR>;                                                               \
-		CLA_HIP(hipFuncSetAttribute((const void*) kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds)); \
+		CLA_HIP(allow_full_lds((const void*) kern)); \
 		hipLaunchKernelGGL(kern, dim3(grid), dim3(THR), lds, st, b->dArena, b->arenaStride, nG, b->dQ1Slabs,    \
 			nSlabs, b->dTblOff, tables, constRow, dOut, nRows, dNnz);                                       \
 	} while(0)

@@ -907,11 +907,11 @@ int launch_rmm_decode(cla_block* b, const double* dB, int q, const double* dCons
 	double algo = (double) b->device_bytes_cached + (double) b->nRows * q * 8;
 	Prof pf(b, "k_rmm_decode", L.grid, DEC_THREADS, (long) L.lds, algo);
 	if(rpl == 4) {
-		CLA_HIP(hipFuncSetAttribute((const void*) k_rmm_decode<4>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) L.lds));
+		CLA_HIP(allow_full_lds((const void*) k_rmm_decode<4>));
 		hipLaunchKernelGGL(k_rmm_decode<4>, dim3(L.grid), dim3(DEC_THREADS), L.lds, b->stream, L.A);
 	}
 	else {
-		CLA_HIP(hipFuncSetAttribute((const void*) k_rmm_decode<2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) L.lds));
+		CLA_HIP(allow_full_lds((const void*) k_rmm_decode<2>));
 		hipLaunchKernelGGL(k_rmm_decode<2>, dim3(L.grid), dim3(DEC_THREADS), L.lds, b->stream, L.A);
 	}
 	CLA_HIP(hipGetLastError());
@@ -945,11 +945,11 @@ int launch_tsmm_decode(cla_block* b, double* dOut) {
 	do {                                                                                                        \
 		if(XBV == 0 && NBV >= 2 && narrow) {                                                                    \
 			constexpr int NARV = XBV == 0 && NBV >= 2 ? 1 : 0;                                                  \
-			CLA_HIP(hipFuncSetAttribute((const void*) k_tsmm_decode<NBV, FL, XBV, NARV>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) L.lds)); \
+			CLA_HIP(allow_full_lds((const void*) k_tsmm_decode<NBV, FL, XBV, NARV>)); \
 			hipLaunchKernelGGL((k_tsmm_decode<NBV, FL, XBV, NARV>), dim3(L.grid), dim3(DEC_THREADS), L.lds, b->stream, L.A); \
 		}                                                                                                       \
 		else {                                                                                                  \
-			CLA_HIP(hipFuncSetAttribute((const void*) k_tsmm_decode<NBV, FL, XBV>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) L.lds)); \
+			CLA_HIP(allow_full_lds((const void*) k_tsmm_decode<NBV, FL, XBV>)); \
 			hipLaunchKernelGGL((k_tsmm_decode<NBV, FL, XBV>), dim3(L.grid), dim3(DEC_THREADS), L.lds, b->stream, L.A); \
 		}                                                                                                       \
 	} while(0)

@@ -435,13 +435,9 @@ int launch_rmm_mfma(cla_block* b, const double* dB, int q, const double* dConstR
 	const MfSrc* dSrc = (const MfSrc*) (base + b->mfOff[2]);
 	const int32_t* dRowCol = (const int32_t*) (base + b->mfOff[3]);
 	const size_t lds = 2 * b->mfBufBytes + (size_t) b->mfNColsAll * sizeof(MfSrc) + (size_t) b->mfNSlabs * sizeof(MfSlab);
-	static size_t ldsSet[2] = {0, 0}; // (racing callers set the same or a larger value)
-	const int wi = b->mfWidth - 1;
-	if(ldsSet[wi] < lds) {
-		if(wi == 0) CLA_HIP(hipFuncSetAttribute((const void*) k_rmm_mfma<MF_WAVES, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
-		else CLA_HIP(hipFuncSetAttribute((const void*) k_rmm_mfma<MF_WAVES, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
-		ldsSet[wi] = lds;
-	}
+	if(b->mfWidth == 1) CLA_HIP(allow_full_lds((const void*) k_rmm_mfma<MF_WAVES, 1>));
+	else CLA_HIP(allow_full_lds((const void*) k_rmm_mfma<MF_WAVES, 2>));
+	if(lds > (size_t) g_ldsPerBlock) return 1;
 	// persistent blocks: one per CU, each walks its row tiles
 	const unsigned grid = (unsigned) std::min<int64_t>((b->nRows + rows - 1) / rows, (int64_t) g_numCU);
 	double codeBytes = 0;

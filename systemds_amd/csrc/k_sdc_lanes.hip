@@ -509,7 +509,7 @@ int launch_lmm_sdc_lanes(cla_block* b, const double* dY, int p, double* dOut) {
 	double algo = (double) b->nRows * 8 * p;
 	for(int g : b->sdcList) algo += (double) p * ((double) b->groups[g].d.nDeltas * b->groups[g].d.deltaWidth + (double) b->groups[g].d.nOffsets);
 	Prof pf(b, "k_lmm_sdc_lanes", (long) nRuns * nS * p, LN_LW * 64, (long) lds, algo);
-	CLA_HIP(hipFuncSetAttribute((const void*) k_lmm_sdc_lanes, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
+	CLA_HIP(allow_full_lds((const void*) k_lmm_sdc_lanes));
 	hipLaunchKernelGGL(k_lmm_sdc_lanes, dim3(nRuns * nS, p), dim3(LN_LW * 64), lds, b->stream, (const LaneDesc*) meta,
 		(const LaneSlab*) (meta + b->laneOff[0]), nS, (const double*) (meta + b->laneOff[1]), b->laneDictLds,
 		(const uint32_t*) (meta + b->laneOff[3]), (const u32x4*) b->dLaneData, dY, b->nRows, nWin, wpw, dOut, b->nCols);
@@ -537,7 +537,7 @@ int launch_rmm_sdc_lanes(cla_block* b, int constRow, int accumulate, double* dOu
 	for(int g : b->sdcList) algo += (double) b->groups[g].d.nDeltas * b->groups[g].d.deltaWidth + (double) b->groups[g].d.nOffsets;
 	Prof pf(b, "k_rmm_sdc_lanes", (long) grid, LN_RW * 64, (long) lds, algo);
 	auto go = [&](auto kernel) {
-		CLA_HIP(hipFuncSetAttribute((const void*) kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
+		CLA_HIP(allow_full_lds((const void*) kernel));
 		hipLaunchKernelGGL(kernel, dim3(grid), dim3(LN_RW * 64), lds, b->stream, (const LaneDesc*) meta,
 			(const LaneSlab*) (meta + b->laneOff[0]), nS, (const int32_t*) (meta + b->laneOff[2]), b->laneDictLds, b->laneDictTotal,
 			(const uint32_t*) (meta + b->laneOff[3]), (const u32x4*) b->dLaneData, (const double*) b->dTables, constRow, accumulate,

@@ -270,8 +270,8 @@ static int rows_plan(cla_block* b) {
 	CLA_HIP(hipMemcpyAsync(dBase, gBase.data(), sizeof(int32_t) * (size_t) nL, hipMemcpyHostToDevice, st));
 	CLA_HIP(hipMemsetAsync(dOver, 0, sizeof(int), st));
 	const size_t lds = sizeof(uint32_t) * (RW_WIN + 256 + 32) + sizeof(uint16_t) * ((size_t) RW_WIN + (size_t) RW_WIN * RW_KR);
-	CLA_HIP(hipFuncSetAttribute((const void*) k_rows_build<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
-	CLA_HIP(hipFuncSetAttribute((const void*) k_rows_build<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
+	CLA_HIP(allow_full_lds((const void*) k_rows_build<false>));
+	CLA_HIP(allow_full_lds((const void*) k_rows_build<true>));
 	hipLaunchKernelGGL(k_rows_build<false>, dim3(nWin), dim3(RB_THREADS), lds, st, b->dGroups, dList, dBase, nL, b->nRows, (uint32_t) nTbl,
 		(uint32_t*) dOff, nullptr, nullptr, nullptr, nullptr, dOver);
 	CLA_HIP(hipGetLastError());
@@ -321,7 +321,7 @@ int launch_rmm_sdc_rows(cla_block* b, int constRow, int accumulate, double* dOut
 	for(int g : b->sdcList) algo += (double) b->groups[g].d.nDeltas * b->groups[g].d.deltaWidth + (double) b->groups[g].d.nOffsets * b->groups[g].d.codeWidth;
 	Prof pf(b, "k_rmm_sdc_rows", (long) grid, RW_THREADS, (long) lds, algo);
 	auto go = [&](auto kernel) {
-		CLA_HIP(hipFuncSetAttribute((const void*) kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
+		CLA_HIP(allow_full_lds((const void*) kernel));
 		hipLaunchKernelGGL(kernel, dim3(grid), dim3(RW_THREADS), lds, b->stream, (const int32_t*) meta, b->rowsTbl,
 			(const uint2*) (meta + b->rowsOff[0]), (const uint16_t*) (meta + b->rowsOff[1]), (const u16x4*) b->dRowsData,
 			(const double*) b->dTables, constRow, dOut, b->nRows, nQuarters, dNnz);

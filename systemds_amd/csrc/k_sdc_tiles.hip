@@ -514,7 +514,7 @@ int launch_lmm_sdc_tiles(cla_block* b, const double* dY, int p, double* dPre, in
 		for(int g : plan.list) algo += (double) p * ((double) b->groups[g].d.nDeltas * b->groups[g].d.deltaWidth + (double) b->groups[g].d.nOffsets * b->groups[g].d.codeWidth);
 		const size_t lds = (size_t) ST * 8;
 		Prof pf(b, "k_lmm_sdc_packed", (long) grid * p, ST_THREADS, (long) lds, algo);
-		CLA_HIP(hipFuncSetAttribute((const void*) k_lmm_sdc_packed, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
+		CLA_HIP(allow_full_lds((const void*) k_lmm_sdc_packed));
 		hipLaunchKernelGGL(k_lmm_sdc_packed, dim3(grid, p), dim3(ST_THREADS), lds, b->stream, (const SdcDesc*) b->dSdcDesc,
 			(int) plan.list.size(), dY, b->nRows, tpb, dOut, b->nCols);
 		CLA_HIP(hipGetLastError());
@@ -548,7 +548,7 @@ int launch_lmm_sdc_tiles(cla_block* b, const double* dY, int p, double* dPre, in
 		}
 		b->preUsed = true;
 		Prof pf(b, "k_lmm_sdc_tiles", (long) grid * p, ST_THREADS, (long) lds, algo);
-		CLA_HIP(hipFuncSetAttribute((const void*) k_lmm_sdc_tiles, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
+		CLA_HIP(allow_full_lds((const void*) k_lmm_sdc_tiles));
 		hipLaunchKernelGGL(k_lmm_sdc_tiles, dim3(grid, p), dim3(ST_THREADS), lds, b->stream, b->dGroups, dList, dBinOff,
 			(int) l0, (int) l1, dY, b->nRows, tpb, dPre, b->totalVals);
 		l0 = l1;
@@ -606,13 +606,13 @@ int launch_rmm_sdc_tiles(cla_block* b, int q, int constRow, int accumulate, doub
 	if(q == 1 && !ldsTables && tileRows == ST && !noPacked && b->dSdcPacked != nullptr) {
 		const size_t ldsP = (size_t) ST * 8;
 		Prof pf(b, "k_rmm_sdc_packed", nTiles, ST_THREADS, (long) ldsP, algo);
-		CLA_HIP(hipFuncSetAttribute((const void*) k_rmm_sdc_packed, hipFuncAttributeMaxDynamicSharedMemorySize, (int) ldsP));
+		CLA_HIP(allow_full_lds((const void*) k_rmm_sdc_packed));
 		hipLaunchKernelGGL(k_rmm_sdc_packed, dim3(nTiles), dim3(ST_THREADS), ldsP, b->stream, (const SdcDesc*) b->dSdcDesc,
 			(int) plan.list.size(), b->dTables, constRow, accumulate, dOut, b->nRows, dNnz);
 	}
 	else {
 		Prof pf(b, "k_rmm_sdc_tiles", nTiles, ST_THREADS, (long) lds, algo);
-		CLA_HIP(hipFuncSetAttribute((const void*) k_rmm_sdc_tiles, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
+		CLA_HIP(allow_full_lds((const void*) k_rmm_sdc_tiles));
 		hipLaunchKernelGGL(k_rmm_sdc_tiles, dim3(nTiles), dim3(ST_THREADS), lds, b->stream, b->dGroups, dList, dBinOff,
 			(int) plan.list.size(), sl, b->dTables, q, constRow, accumulate, tileRows, dOut, b->nRows, dNnz, ldsTables ? 1 : 0);
 	}

@@ -280,7 +280,7 @@ static void launch_pair_dot_cw(int nct, int ncs, dim3 grid, size_t lds, hipStrea
 #define PD_CASE(A, B)                                                                                           \
 	if(nct == A && ncs == B) {                                                                                  \
 		auto kern = k_tsmm_pair_dot<CW, A, B>;                                                                  \
-		(void) hipFuncSetAttribute((const void*) kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds);  \
+		(void) allow_full_lds((const void*) kern);  \
 		hipLaunchKernelGGL(kern, grid, dim3(PD_THREADS), lds, st, g, pairs, nPairs, nRows, chunkRows, bpcp, out, nCols); \
 	}
 	PD_CASE(1, 1) PD_CASE(1, 2) PD_CASE(2, 1) PD_CASE(2, 2)
@@ -617,7 +617,7 @@ int launch_tsmm(cla_block* b, double* dOut, unsigned long long* dNnz) {
 		const size_t lds = (size_t) DT * nCols * 8;
 		if(nRows > 0) {
 			Prof pf(b, "k_tsmm_dense", grid, 256, (long) lds, 0);
-			CLA_HIP(hipFuncSetAttribute((const void*) k_tsmm_dense, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
+			CLA_HIP(allow_full_lds((const void*) k_tsmm_dense));
 			hipLaunchKernelGGL(k_tsmm_dense, dim3(grid), dim3(256), lds, st, b->dGroups, nG, b->dConstV, nRows, nCols, DT,
 				tpb, dOut);
 		}
@@ -731,7 +731,7 @@ int launch_tsmm(cla_block* b, double* dOut, unsigned long long* dNnz) {
 		}
 		{
 			Prof pf(b, "k_tsmm_pair", (long) bpp * (long) pairs.size(), PAIR_THREADS, (long) ldsMax, codeBytes);
-			CLA_HIP(hipFuncSetAttribute((const void*) k_tsmm_pair, hipFuncAttributeMaxDynamicSharedMemorySize, (int) ldsMax));
+			CLA_HIP(allow_full_lds((const void*) k_tsmm_pair));
 			hipLaunchKernelGGL(k_tsmm_pair, dim3(bpp, (unsigned) pairs.size()), dim3(PAIR_THREADS), ldsMax, st, b->dGroups,
 				dPairs, nRows, tpb, dOut, nCols);
 		}

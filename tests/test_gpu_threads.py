@@ -54,3 +54,30 @@ def test_parallel_calls_on_different_and_on_the_same_handle(cla, ora):
     finally:
         for j in jobs:
             j[0].close()
+
+
+def test_parallel_calls_whose_kernels_need_different_amounts_of_lds(cla, ora):
+    """Two handles whose products run the same kernels with different dynamic LDS sizes (dictionaries of 16 and of
+    3000 tuples; 20 and 90 list groups): the per-kernel LDS allowance is a property of the kernel, not of the call
+    that happened to set it last."""
+    from systemds_amd import synth
+    rng = np.random.default_rng(5)
+    n_rows = 40009
+    jobs = []
+    for n_ddc, n_vals, n_sdc in ((4, 16, 20), (12, 3000, 90)):
+        specs, c = [], 0
+        for g in range(n_ddc):
+            specs.append(synth.GroupSpec("ddc", np.array([c, c + 1], np.int32), rng.standard_normal((n_vals, 2)),
+                                         rng.integers(0, n_vals, n_rows).astype(np.uint16 if n_vals > 256 else np.uint8)))
+            c += 2
+        for g in range(n_sdc):
+            specs.append(synth.sdc_group(np.random.default_rng((5, g)), n_rows, np.array([c], np.int32), 30, 0.04, None))
+            c += 1
+        blk = cla.build_block(n_rows, c, specs)
+        B, Y, v = rng.standard_normal((c, 8)), rng.standard_normal((2, n_rows)), rng.standard_normal((c, 1))
+        jobs.append((blk, B, Y, v, blk.rmm(B)[0], blk.lmm(Y)[0], blk.tsmm()[0], blk.mmchain(v, None, 0)[0]))
+    try:
+        assert run_threads(jobs, lambda i: i % 2, cross=False) == []
+    finally:
+        for j in jobs:
+            j[0].close()
