@@ -54,7 +54,7 @@ __global__ __launch_bounds__(RB_THREADS) void k_rows_build(const DGroup* __restr
 	uint16_t* stage = rowOf + RW_WIN;             // RW_WIN x RW_KR
 	const int tid = threadIdx.x;
 	const int win = blockIdx.x;
-	const int64_t r0 = (int64_t) win * RW_WIN, rEnd = r0 + RW_WIN;
+	const int64_t r0 = (int64_t) win * RW_WIN;
 	for(int k = tid; k < RW_WIN; k += RB_THREADS) cnt[k] = 0;
 	if(tid < 256) hist[tid] = 0;
 	__syncthreads();
