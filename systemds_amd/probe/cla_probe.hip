@@ -6,6 +6,7 @@
 //   3. streaming reads from HBM: one flat buffer, and 100 strided code streams as the byte-code mat-vec reads them
 //   4. L2 -> CU: global_load_lds_dwordx4 against loads through registers, all CUs on one 256 KB region
 //   5. stores of 16 bytes per lane: 1 KB contiguous per instruction, 8 rows x 128 bytes, 16 rows x 64 bytes
+//   6. LDS table lookups as the mat-vec gather does them (byte -> ds_read_b64 -> add), random and conflict-free
 // Usage: cla_probe            (a few seconds; every kernel is a bounded loop)
 #include <hip/hip_runtime.h>
 #include <cstdint>
@@ -248,6 +249,48 @@ static void probe_l2_and_stores(unsigned* sink) {
 	CK(hipFree(d));
 }
 
+// ---- 6. LDS table lookups ----------------------------------------------------------------------------
+// 20 tables of 256 doubles; per table a thread looks 16 pseudo-random bytes up and adds the values to 16 sums
+// (MASK = 255: any entry; MASK = 3: four entries, which cannot conflict)
+template <int MASK>
+__global__ __launch_bounds__(512, 4) void k_lds_lookup(double* out, int rounds) {
+	__shared__ double tbl[20 * 256];
+	for(int i = threadIdx.x; i < 20 * 256; i += 512) tbl[i] = 0.5 * i;
+	__syncthreads();
+	const char* tb = (const char*) tbl;
+	unsigned x = threadIdx.x * 2654435761u + blockIdx.x * 40503u + 12345u;
+	double acc[16];
+#pragma unroll
+	for(int i = 0; i < 16; i++) acc[i] = 0.0;
+	for(int r = 0; r < rounds; r++) {
+#pragma unroll
+		for(int g = 0; g < 20; g++) {
+#pragma unroll
+			for(int w = 0; w < 4; w++) {
+				x = x * 1664525u + 1013904223u;
+#pragma unroll
+				for(int k = 0; k < 4; k++) acc[4 * w + k] += *(const double*) (tb + g * 2048 + (((x >> (8 * k)) & MASK) << 3));
+			}
+		}
+	}
+	double s = 0.0;
+#pragma unroll
+	for(int i = 0; i < 16; i++) s += acc[i];
+	out[(size_t) blockIdx.x * 512 + threadIdx.x] = s;
+}
+
+static void probe_lds() {
+	const int bpc = 2, blocks = g_cus * bpc, rounds = 200; // 16 waves per CU, as the mat-vec gather runs
+	double* out;
+	CK(hipMalloc(&out, sizeof(double) * (size_t) blocks * 512));
+	const double perCU = (double) bpc * 8 * rounds * 320; // wave-level lookups per CU
+	const float msAny = time_ms([&] { hipLaunchKernelGGL(k_lds_lookup<255>, dim3(blocks), dim3(512), 0, 0, out, rounds); }, 3);
+	const float msFour = time_ms([&] { hipLaunchKernelGGL(k_lds_lookup<3>, dim3(blocks), dim3(512), 0, 0, out, rounds); }, 3);
+	printf("LDS table lookup (byte -> ds_read_b64 -> v_add_f64), any of 256 entries: %.2f cycles per wave-level lookup and CU\n", msAny * 1e-3 * g_hz / perCU);
+	printf("LDS table lookup (byte -> ds_read_b64 -> v_add_f64), one of 4 entries:   %.2f cycles per wave-level lookup and CU\n", msFour * 1e-3 * g_hz / perCU);
+	CK(hipFree(out));
+}
+
 int main() {
 	hipDeviceProp_t prop;
 	CK(hipGetDeviceProperties(&prop, 0));
@@ -262,6 +305,7 @@ int main() {
 	probe_mfma();
 	probe_stream(sink);
 	probe_l2_and_stores(sink);
+	probe_lds();
 	CK(hipFree(sink));
 	return bad ? 1 : 0;
 }
