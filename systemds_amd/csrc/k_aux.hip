@@ -2,23 +2,38 @@
 // counts, offset-list checkpoints and row-tile index.
 #include "../../include/cla_hip.h"
 #include "cla_device.hpp"
+#include <algorithm>
 
 namespace cla {
 
 // ---------------------------------------------------------------------------
 // max code of a stream (validation: every code must be < nVals)
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void k_max_code(const void* __restrict__ codes, int width, int64_t n,
-	int* __restrict__ maxOut) {
-	int m = -1;
-	for(int64_t i = (int64_t) blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t) gridDim.x * blockDim.x) {
-		const int c = load_code(codes, width, i);
-		// a negative MapToInt entry is invalid as well: report it as a huge code
-		m = max(m, c < 0 ? 0x7fffffff : c);
-	}
+// 16 bytes per thread and step; the elements behind the last full 16 bytes one by one
+template <int W>
+__global__ __launch_bounds__(256) void k_max_code(const void* __restrict__ codes, int64_t n, int* __restrict__ maxOut) {
+	constexpr int PER = 16 / W;
+	const int64_t nVec = n / PER;
+	const u32x4* vec = (const u32x4*) codes;
+	unsigned m = 0; // (a negative MapToInt entry is invalid as well: as unsigned it is a huge code)
+	for(int64_t i = (int64_t) blockIdx.x * blockDim.x + threadIdx.x; i < nVec; i += (int64_t) gridDim.x * blockDim.x) {
+		const u32x4 v = __builtin_nontemporal_load(vec + i);
 #pragma unroll
-	for(int d = 32; d > 0; d >>= 1) m = max(m, __shfl_down(m, d, WAVE));
-	if((threadIdx.x & 63) == 0) atomicMax(maxOut, m);
+		for(int k = 0; k < 4; k++) {
+			const unsigned x = v[k];
+			if(W == 1) m = max(max(m, x & 0xffu), max(max((x >> 8) & 0xffu, (x >> 16) & 0xffu), x >> 24));
+			else if(W == 2) m = max(m, max(x & 0xffffu, x >> 16));
+			else m = max(m, x);
+		}
+	}
+	if(blockIdx.x == 0 && threadIdx.x < (int) (n - nVec * PER)) {
+		const int c = load_code(codes, W, nVec * PER + threadIdx.x);
+		m = max(m, (unsigned) c);
+	}
+	m = min(m, 0x7fffffffu);
+#pragma unroll
+	for(int d = 32; d > 0; d >>= 1) m = max(m, (unsigned) __shfl_down((int) m, d, WAVE));
+	if((threadIdx.x & 63) == 0) atomicMax(maxOut, (int) m);
 }
 
 int launch_validate_codes(cla_block* b, const void* codes, int width, int64_t n, int nVals, int* ok) {
@@ -29,9 +44,15 @@ int launch_validate_codes(cla_block* b, const void* codes, int width, int64_t n,
 	int* dMax = (int*) b->dScratch;
 	int init = -1;
 	CLA_HIP(hipMemcpyAsync(dMax, &init, sizeof(int), hipMemcpyHostToDevice, b->stream));
-	const int64_t blocks = (n + 256 * 16 - 1) / (256 * 16);
-	hipLaunchKernelGGL(k_max_code, dim3((unsigned) (blocks > 4096 ? 4096 : blocks)), dim3(256), 0, b->stream, codes,
-		width, n, dMax);
+	if(((uintptr_t) codes & 15) != 0 || (width != 1 && width != 2 && width != 4)) {
+		set_error("code stream: unaligned device buffer or width %d", width);
+		return -CLA_ERR_INVALID;
+	}
+	const int64_t blocks = std::max<int64_t>(1, (n * width / 16 + 256 * 4 - 1) / (256 * 4));
+	const unsigned grid = (unsigned) (blocks > 4096 ? 4096 : blocks);
+	if(width == 1) hipLaunchKernelGGL(k_max_code<1>, dim3(grid), dim3(256), 0, b->stream, codes, n, dMax);
+	else if(width == 2) hipLaunchKernelGGL(k_max_code<2>, dim3(grid), dim3(256), 0, b->stream, codes, n, dMax);
+	else hipLaunchKernelGGL(k_max_code<4>, dim3(grid), dim3(256), 0, b->stream, codes, n, dMax);
 	int mx = -1;
 	CLA_HIP(hipMemcpyAsync(&mx, dMax, sizeof(int), hipMemcpyDeviceToHost, b->stream));
 	CLA_HIP(hipStreamSynchronize(b->stream));
@@ -144,37 +165,67 @@ __global__ void k_sdc_scan(const int2* __restrict__ sums, int nCkpt, int first, 
 	ckpt[nCkpt] = s;
 }
 
-// tile t: iterator state in front of the first delta entry whose accumulated row
-// reaches t * SDC_TILE.
-template <int W>
-__global__ __launch_bounds__(256) void k_sdc_tile_index(const void* __restrict__ deltas, int64_t nDeltas,
-	const OffState* __restrict__ ckpt, int nCkpt, int first, int nTiles, OffState* __restrict__ tileIdx) {
+// tile t: iterator state in front of the first delta entry whose accumulated row reaches t * SDC_TILE.
+// k_sdc_tile_ends writes the tiles that no entry reaches (at or in front of the first row: the initial state;
+// behind the last row: the final one), k_sdc_tile_index the others: block = chunk of SDC_CK entries, a block-wide
+// prefix sum gives every entry its state in front of it, and an entry writes the tiles whose first row lies
+// in (row in front of it, row behind it].
+__global__ __launch_bounds__(256) void k_sdc_tile_ends(const OffState* __restrict__ ckpt, int nCkpt, int64_t nDeltas, int first,
+	int nTiles, OffState* __restrict__ tileIdx) {
 	const int t = blockIdx.x * blockDim.x + threadIdx.x;
 	if(t >= nTiles) return;
-	const int maxV = W == 1 ? 255 : 65535;
-	const int64_t tb = (int64_t) t * SDC_TILE;
 	OffState s;
 	s.idx = 0; s.emit = 1; s.row = first; s.pad = 0;
-	if(nCkpt > 0 && first < tb) {
-		// last chunk whose state row is < tb
-		int lo = 0, hi = nCkpt - 1;
-		while(lo < hi) {
-			const int mid = (lo + hi + 1) >> 1;
-			if(ckpt[mid].row < tb) lo = mid; else hi = mid - 1;
-		}
-		s = ckpt[lo];
-		int64_t i = s.idx;
-		const int64_t end = (i + SDC_CK < nDeltas) ? i + SDC_CK : nDeltas;
-		for(; i < end; i++) {
-			const int v = W == 1 ? (int) ((const uint8_t*) deltas)[i] : (int) ((const uint16_t*) deltas)[i];
-			const int nr = s.row + (v == 0 ? maxV : v);
-			if(nr >= tb) break;
-			s.row = nr;
-			s.emit += v != 0;
-		}
-		s.idx = (int32_t) i;
+	if(nCkpt > 0 && (int64_t) first < (int64_t) t * SDC_TILE) {
+		s = ckpt[nCkpt];
+		s.idx = (int32_t) nDeltas;
 	}
 	tileIdx[t] = s;
+}
+
+template <int W>
+__global__ __launch_bounds__(256) void k_sdc_tile_index(const void* __restrict__ deltas, int64_t nDeltas,
+	const OffState* __restrict__ ckpt, int nTiles, OffState* __restrict__ tileIdx) {
+	__shared__ int sInc[4], sNz[4];
+	const int maxV = W == 1 ? 255 : 65535;
+	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+	const OffState st = ckpt[blockIdx.x];
+	const int64_t i0 = (int64_t) blockIdx.x * SDC_CK + tid * 4;
+	int inc[4], nz[4], incSum = 0, nzSum = 0;
+#pragma unroll
+	for(int k = 0; k < 4; k++) {
+		inc[k] = 0; nz[k] = 0;
+		if(i0 + k < nDeltas) {
+			const int v = W == 1 ? (int) ((const uint8_t*) deltas)[i0 + k] : (int) ((const uint16_t*) deltas)[i0 + k];
+			inc[k] = v == 0 ? maxV : v;
+			nz[k] = v != 0;
+		}
+		incSum += inc[k]; nzSum += nz[k];
+	}
+	// exclusive prefix over the block: inside the wave by shuffles, across the four waves through LDS
+	int incPre = incSum, nzPre = nzSum;
+#pragma unroll
+	for(int d = 1; d < 64; d <<= 1) {
+		const int a = __shfl_up(incPre, d, 64), c = __shfl_up(nzPre, d, 64);
+		if(lane >= d) { incPre += a; nzPre += c; }
+	}
+	if(lane == 63) { sInc[wave] = incPre; sNz[wave] = nzPre; }
+	__syncthreads();
+	int64_t row = (int64_t) st.row + (incPre - incSum);
+	int emit = st.emit + (nzPre - nzSum);
+	for(int w = 0; w < wave; w++) { row += sInc[w]; emit += sNz[w]; }
+#pragma unroll
+	for(int k = 0; k < 4; k++) {
+		if(i0 + k >= nDeltas) break;
+		const int64_t after = row + inc[k];
+		for(int64_t t = row / SDC_TILE + 1; t <= after / SDC_TILE && t < nTiles; t++) {
+			OffState s;
+			s.idx = (int32_t) (i0 + k); s.emit = emit; s.row = (int32_t) row; s.pad = 0;
+			tileIdx[t] = s;
+		}
+		row = after;
+		emit += nz[k];
+	}
 }
 
 int launch_sdc_build(cla_block* b, HostGroup& g) {
@@ -208,12 +259,13 @@ int launch_sdc_build(cla_block* b, HostGroup& g) {
 	}
 	hipLaunchKernelGGL(k_sdc_scan, dim3(1), dim3(1), 0, st, sums, nCkpt, G.first, ckpt);
 	if(nTiles > 0) {
-		if(G.deltaWidth == 1)
-			hipLaunchKernelGGL(k_sdc_tile_index<1>, dim3((nTiles + 255) / 256), dim3(256), 0, st, G.deltas, G.nDeltas, ckpt,
-				nCkpt, G.first, nTiles, tiles);
-		else
-			hipLaunchKernelGGL(k_sdc_tile_index<2>, dim3((nTiles + 255) / 256), dim3(256), 0, st, G.deltas, G.nDeltas, ckpt,
-				nCkpt, G.first, nTiles, tiles);
+		hipLaunchKernelGGL(k_sdc_tile_ends, dim3((nTiles + 255) / 256), dim3(256), 0, st, ckpt, nCkpt, G.nDeltas, G.first, nTiles, tiles);
+		if(nCkpt > 0) {
+			if(G.deltaWidth == 1)
+				hipLaunchKernelGGL(k_sdc_tile_index<1>, dim3(nCkpt), dim3(256), 0, st, G.deltas, G.nDeltas, ckpt, nTiles, tiles);
+			else
+				hipLaunchKernelGGL(k_sdc_tile_index<2>, dim3(nCkpt), dim3(256), 0, st, G.deltas, G.nDeltas, ckpt, nTiles, tiles);
+		}
 	}
 	OffState fin;
 	CLA_HIP(hipMemcpyAsync(&fin, ckpt + nCkpt, sizeof(OffState), hipMemcpyDeviceToHost, st));
