@@ -147,3 +147,34 @@ def test_mmchain_minus_y(cla, ora):
             blk.mmchain(v, y, 3)
     finally:
         blk.close()
+
+
+def test_byte_code_block_with_non_finite_dictionary_values(cla, ora):
+    """All groups DDC with byte codes and one column (the dot-form kernel's case): the reference sums Y per tuple
+    first and multiplies once (APreAgg.leftMultByMatrix, ADictionary pre-aggregation), so an infinite dictionary
+    value under rows of Y of both signs gives one infinity, where Y[r] * dict[code] summed over the rows would give
+    NaN. Blocks with such a dictionary take the bin kernels; the cells are the oracle's."""
+    from systemds_amd import synth
+    c = synth.config2(scale=200, n_cols=24)
+    n_rows, n_cols = c["n_rows"], c["n_cols"]
+    c["groups"][3].dict[5, 0] = np.inf
+    c["groups"][8].dict[0, 0] = -np.inf
+    c["groups"][11].dict[2, 0] = np.nan
+    Y = np.random.default_rng(6).standard_normal((2, n_rows))
+    blk = cla.build_block(n_rows, n_cols, c["groups"])
+    try:
+        out, nnz = blk.lmm(Y)
+        blk.profile(True)
+        blk.lmm(Y)
+        names = [k["name"] for k in blk.stats()["kernels"]]
+        blk.profile(False)
+    finally:
+        blk.close()
+    assert "k_lmm_u8_dot" not in names, names
+    ref, rnnz = ora.lmm(ora.Groups(c["groups"], n_rows, n_cols), Y, 4)
+    fin = np.isfinite(ref)
+    assert not fin.all() and np.array_equal(np.isfinite(out), fin)
+    assert np.array_equal(out[~fin], ref[~fin], equal_nan=True)
+    D = np.nan_to_num(ora.np_decompress(c["groups"], n_rows, n_cols), nan=0.0, posinf=0.0, neginf=0.0)
+    assert_fp64_close(out[fin], ref[fin], ora.abs_matmul(Y, D)[fin], what="t(Y)%*%X, non-finite dictionary", n_terms=n_rows)
+    assert nnz == rnnz
