@@ -698,7 +698,7 @@ struct DecLaunch {
 
 // Dictionaries of more than dictLimit doubles stay in global memory (t(X) %*% X only).
 // The plan's device image goes into *dImg (an allocation of its own, kept with the plan).
-static int dec_build_plan(cla_block* b, bool gram, int q, int rpl, DecLaunch& L, size_t dictLimit, void** dImg) {
+static int dec_build_plan(cla_block* b, bool gram, int q, int rpl, DecLaunch& L, size_t dictLimit, void** dImg, int64_t* imgBytes) {
 	const int nG = (int) b->groups.size();
 	const int nCols = b->nCols;
 	{
@@ -830,6 +830,7 @@ static int dec_build_plan(cla_block* b, bool gram, int q, int rpl, DecLaunch& L,
 	uint8_t* d = nullptr;
 	CLA_HIP(hipMalloc((void**) &d, img.size() + 64));
 	*dImg = d;
+	*imgBytes = (int64_t) img.size() + 64;
 	CLA_HIP(hipMemcpy(d, img.data(), img.size(), hipMemcpyHostToDevice));
 	DecArgs& A = L.A;
 	A.groups = b->dGroups;
@@ -857,6 +858,7 @@ struct DecPlanEntry {
 	int rc;
 	DecLaunch L;
 	void* dImg;
+	int64_t bytes;
 };
 struct DecPlanCache {
 	std::vector<DecPlanEntry> entries;
@@ -865,7 +867,7 @@ struct DecPlanCache {
 void dec_plans_drop(cla_block* b) {
 	if(b->decPlans == nullptr) return;
 	for(auto& e : b->decPlans->entries)
-		if(e.dImg) (void) hipFree(e.dImg);
+		if(e.dImg) { (void) hipFree(e.dImg); b->derivedBytes -= e.bytes; }
 	delete b->decPlans;
 	b->decPlans = nullptr;
 }
@@ -878,17 +880,18 @@ static int dec_prepare(cla_block* b, bool gram, int q, int rpl, DecLaunch& L, si
 			return e.rc;
 		}
 	DecPlanEntry e;
-	e.gram = gram; e.q = q; e.rpl = rpl; e.expand = b->opt.expandStreams; e.dictLimit = dictLimit; e.dImg = nullptr;
-	e.rc = dec_build_plan(b, gram, q, rpl, e.L, dictLimit, &e.dImg);
+	e.gram = gram; e.q = q; e.rpl = rpl; e.expand = b->opt.expandStreams; e.dictLimit = dictLimit; e.dImg = nullptr; e.bytes = 0;
+	e.rc = dec_build_plan(b, gram, q, rpl, e.L, dictLimit, &e.dImg, &e.bytes);
 	if(e.rc < 0) { // an error is not a property of the block: not kept
 		if(e.dImg) (void) hipFree(e.dImg);
 		return e.rc;
 	}
 	if(b->decPlans->entries.size() >= 64) { // (products with many different widths of B: start over)
 		for(auto& o : b->decPlans->entries)
-			if(o.dImg) (void) hipFree(o.dImg);
+			if(o.dImg) { (void) hipFree(o.dImg); b->derivedBytes -= o.bytes; }
 		b->decPlans->entries.clear();
 	}
+	if(e.dImg) b->derivedBytes += e.bytes;
 	b->decPlans->entries.push_back(e);
 	L = e.L;
 	return e.rc;
