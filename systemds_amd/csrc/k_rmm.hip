@@ -651,9 +651,26 @@ int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned lon
 		if(r <= 0) return r;
 	}
 
-	// narrow B on any group mix: decode rows from LDS dictionaries, B rows as scalars
-	if(q >= 2 && q <= 16 && !noAlloc && !(b->opt.rmmDisable & 8)) {
+	// narrow B on any group mix: decode rows from LDS dictionaries, B rows as scalars. A single column as well
+	// where groups other than offset lists carry most of the block (the lists alone have kernels of their own
+	// below): C5's X %*% v takes 1.5 ms here against 4.6 ms per row and group.
+	bool vecDecode = false;
+	if(q == 1) {
+		int nLists = 0, nOther = 0;
+		for(auto& g : b->groups) {
+			if(g.d.type == G_SDCZ) nLists += g.d.nOffsets > 0;
+			else nOther += g.d.type == G_UNC || g.d.nVals > 0;
+		}
+		vecDecode = nOther > 0 && nLists <= nOther;
+	}
+	if(((q >= 2 && q <= 16) || vecDecode) && !noAlloc && !(b->opt.rmmDisable & 8)) {
 		const int r = launch_rmm_decode(b, dB, q, constRow >= 0 ? tables + (size_t) constRow * q : nullptr, dOut, dNnz);
+		if(r <= 0) return r;
+	}
+	// 2 to 7 columns of B on an all-DDC block whose dictionaries the decode kernel cannot hold in LDS: the matrix-core
+	// kernel on a zero-padded B (2.5 ms on C2 whatever the width, against 2.8 - 5 ms of the gather per row and group)
+	if(q >= 2 && q < 8 && !noAlloc && !(b->opt.rmmDisable & 4)) {
+		const int r = launch_rmm_mfma(b, dB, q, constRow >= 0 ? tables + (size_t) constRow * q : nullptr, dOut, dNnz);
 		if(r <= 0) return r;
 	}
 

@@ -900,7 +900,7 @@ static int dec_prepare(cla_block* b, bool gram, int q, int rpl, DecLaunch& L, si
 // Returns 1 when the block/shape is not eligible (caller uses the generic path).
 int launch_rmm_decode(cla_block* b, const double* dB, int q, const double* dConstRow, double* dOut,
 	unsigned long long* dNnz) {
-	if(b->groups.empty() || b->nRows == 0 || q < 2 || q > DEC_QMAX) return 1;
+	if(b->groups.empty() || b->nRows == 0 || q < 1 || q > DEC_QMAX) return 1;
 	DecLaunch L;
 	int rpl = 4; // rows per lane and pass: the smaller output staging area when LDS is short
 	int rc = dec_prepare(b, false, q, rpl, L);

@@ -65,24 +65,25 @@ __global__ __launch_bounds__(ST_THREADS) void k_lmm_sdc_tiles(const DGroup* __re
 
 // ---------------------------------------------------------------------------
 // Right multiply with q output columns, SDCZeros groups sdcList[0 .. nL): block =
-// one tile. LDS: the output tile [ST x q] and the tables of a slab of groups.
-// accumulate == 0: the tile starts from constRow (or zero) and is the whole
+// one tile of the output columns [q0, q0 + qc). LDS: the output tile [ST x qc] and the tables of a
+// slab of groups. accumulate == 0: the tile starts from constRow (or zero) and is the whole
 // result; accumulate != 0: the tile starts from what other groups already wrote.
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(ST_THREADS) void k_rmm_sdc_tiles(const DGroup* __restrict__ groups,
 	const int32_t* __restrict__ sdcList, const int32_t* __restrict__ binOff, int nL, int slabLen, const double* __restrict__ T,
-	int q, int constRow, int accumulate, int tileRows, double* __restrict__ out, int64_t nRows,
+	int q, int q0, int qc, int constRow, int accumulate, int tileRows, double* __restrict__ out, int64_t nRows,
 	unsigned long long* __restrict__ nnz, int ldsTables) {
 	extern __shared__ double smem[];
-	double* otile = smem;                       // tileRows * q
-	double* tbl = smem + (size_t) tileRows * q; // tables of the current slab, q doubles per tuple
+	double* otile = smem;                        // tileRows * qc
+	double* tbl = smem + (size_t) tileRows * qc; // tables of the current slab, qc doubles per tuple
 	const int tid = threadIdx.x, wave = tid >> 6;
 	const int tile = blockIdx.x;
 	const int64_t r0 = (int64_t) tile * tileRows;
 	const int nr = (int) min((int64_t) tileRows, nRows - r0);
-	for(int t = tid; t < tileRows * q; t += ST_THREADS) {
+	for(int t = tid; t < tileRows * qc; t += ST_THREADS) {
 		double v = 0.0;
-		if(t < nr * q) v = accumulate ? out[(size_t) r0 * q + t] : (constRow >= 0 ? T[(size_t) constRow * q + (t % q)] : 0.0);
+		const int rr = t / qc, c = t - rr * qc;
+		if(rr < nr) v = accumulate ? out[(size_t) (r0 + rr) * q + q0 + c] : (constRow >= 0 ? T[(size_t) constRow * q + q0 + c] : 0.0);
 		otile[t] = v;
 	}
 	for(int l0 = 0; l0 < nL; l0 += slabLen) {
@@ -92,29 +93,31 @@ __global__ __launch_bounds__(ST_THREADS) void k_rmm_sdc_tiles(const DGroup* __re
 		if(ldsTables) {
 			for(int l = l0; l < l1; l++) {
 				const DGroup G = dgroup(groups + (sdcList[l]));
-				double* tg = tbl + (size_t) (binOff[l] - b0) * q;
-				const double* src = T + (size_t) G.tblOff * q;
-				for(int k = tid; k < G.nVals * q; k += ST_THREADS) tg[k] = src[k];
+				double* tg = tbl + (size_t) (binOff[l] - b0) * qc;
+				const double* src = T + (size_t) G.tblOff * q + q0;
+				for(int k = tid; k < G.nVals * qc; k += ST_THREADS) tg[k] = src[(size_t) (k / qc) * q + k % qc];
 			}
 			__syncthreads();
 		}
 		for(int l = l0 + wave; l < l1; l += ST_THREADS / 64) {
 			const DGroup G = dgroup(groups + (sdcList[l]));
-			const double* tg = ldsTables ? tbl + (size_t) (binOff[l] - b0) * q : T + (size_t) G.tblOff * q;
+			const double* tg = ldsTables ? tbl + (size_t) (binOff[l] - b0) * qc : T + (size_t) G.tblOff * q + q0;
+			const int ts = ldsTables ? qc : q; // doubles between two tuples of the table
 			const void* codes = G.codes;
 			const int cw = G.codeWidth;
 			sdc_walk_tile(G, r0, tileRows, [&](int rr, int di) {
 				const int code = load_code(codes, cw, di);
-				for(int c = 0; c < q; c++) unsafeAtomicAdd(&otile[(size_t) rr * q + c], tg[(size_t) code * q + c]);
+				for(int c = 0; c < qc; c++) unsafeAtomicAdd(&otile[(size_t) rr * qc + c], tg[(size_t) code * ts + c]);
 			});
 		}
 	}
 	__syncthreads();
 	int cnt = 0;
-	for(int t = tid; t < nr * q; t += ST_THREADS) {
+	for(int t = tid; t < nr * qc; t += ST_THREADS) {
 		const double v = otile[t];
+		const int rr = t / qc, c = t - rr * qc;
 		cnt += v != 0.0;
-		out[(size_t) r0 * q + t] = v;
+		out[(size_t) (r0 + rr) * q + q0 + c] = v;
 	}
 	count_add(nnz, cnt);
 }
@@ -574,10 +577,14 @@ int launch_rmm_sdc_tiles(cla_block* b, int q, int constRow, int accumulate, doub
 	}
 	if(q == 1 && b->opt.sdcPacked && (rc = sdc_plan(b, -1, &dList, &dBinOff, true))) return rc;
 	const size_t ldsMax = (size_t) std::min(g_ldsPerBlock, 160 * 1024) - 2048;
+	// columns per pass: all of them when a tile of SDC_TILE rows fits LDS, else chunks of that many columns
+	// (each pass walks the lists again)
+	int qc = q;
+	while((size_t) SDC_TILE * qc * 8 + 4096 > ldsMax && qc > 1) qc = (qc + 1) / 2;
 	// rows per tile: a multiple of the tile-index granularity whose output tile takes at most ~half of LDS
 	int tileRows = ST;
-	while(tileRows > SDC_TILE && (size_t) tileRows * q * 8 > ldsMax / 2) tileRows /= 2;
-	if((size_t) tileRows * q * 8 + 4096 > ldsMax) return 1;
+	while(tileRows > SDC_TILE && (size_t) tileRows * qc * 8 > ldsMax / 2) tileRows /= 2;
+	if((size_t) tileRows * qc * 8 + 4096 > ldsMax) return 1;
 	size_t maxVals = 1;
 	for(size_t l = 0; l < plan.list.size(); l++) maxVals = std::max(maxVals, (size_t) (plan.binOff[l + 1] - plan.binOff[l]));
 	// Tables are read from global memory (they stay in L2): without table slabs in LDS the
@@ -586,17 +593,17 @@ int launch_rmm_sdc_tiles(cla_block* b, int q, int constRow, int accumulate, doub
 	// 0.58 ms with none).
 	size_t tblBudget = 8 * 1024;
 	const bool ldsTables = false;
-	tblBudget = std::max(tblBudget, maxVals * q * 8);
-	tblBudget = std::min(tblBudget, ldsMax - (size_t) tileRows * q * 8);
+	tblBudget = std::max(tblBudget, maxVals * qc * 8);
+	tblBudget = std::min(tblBudget, ldsMax - (size_t) tileRows * qc * 8);
 	// groups per slab: uniform count so that every slab's tables fit
-	const size_t slabLen = tblBudget / (maxVals * q * 8);
+	const size_t slabLen = tblBudget / (maxVals * qc * 8);
 	if(slabLen < 1) return 1;
 	const int nTiles = (int) ((b->nRows + tileRows - 1) / tileRows);
 	const int sl = ldsTables ? (int) std::min(slabLen, plan.list.size()) : (int) plan.list.size();
 	size_t tblDoubles = 0;
 	for(size_t l0 = 0; ldsTables && l0 < plan.list.size(); l0 += sl)
-		tblDoubles = std::max(tblDoubles, (size_t) (plan.binOff[std::min(l0 + sl, plan.list.size())] - plan.binOff[l0]) * q);
-	const size_t lds = (size_t) tileRows * q * 8 + tblDoubles * 8;
+		tblDoubles = std::max(tblDoubles, (size_t) (plan.binOff[std::min(l0 + sl, plan.list.size())] - plan.binOff[l0]) * qc);
+	const size_t lds = (size_t) tileRows * qc * 8 + tblDoubles * 8;
 	double algo = (double) b->nRows * q * 8 * (accumulate ? 2 : 1);
 	for(int g : plan.list) {
 		const DGroup& G = b->groups[g].d;
@@ -611,10 +618,13 @@ int launch_rmm_sdc_tiles(cla_block* b, int q, int constRow, int accumulate, doub
 			(int) plan.list.size(), b->dTables, constRow, accumulate, dOut, b->nRows, dNnz);
 	}
 	else {
-		Prof pf(b, "k_rmm_sdc_tiles", nTiles, ST_THREADS, (long) lds, algo);
 		CLA_HIP(allow_full_lds((const void*) k_rmm_sdc_tiles));
-		hipLaunchKernelGGL(k_rmm_sdc_tiles, dim3(nTiles), dim3(ST_THREADS), lds, b->stream, b->dGroups, dList, dBinOff,
-			(int) plan.list.size(), sl, b->dTables, q, constRow, accumulate, tileRows, dOut, b->nRows, dNnz, ldsTables ? 1 : 0);
+		for(int q0 = 0; q0 < q; q0 += qc) {
+			Prof pf(b, "k_rmm_sdc_tiles", nTiles, ST_THREADS, (long) lds, algo * std::min(qc, q - q0) / q);
+			hipLaunchKernelGGL(k_rmm_sdc_tiles, dim3(nTiles), dim3(ST_THREADS), lds, b->stream, b->dGroups, dList, dBinOff,
+				(int) plan.list.size(), sl, b->dTables, q, q0, std::min(qc, q - q0), constRow, accumulate, tileRows, dOut, b->nRows, dNnz,
+				ldsTables ? 1 : 0);
+		}
 	}
 	CLA_HIP(hipGetLastError());
 	return 0;

@@ -290,3 +290,81 @@ def test_options_and_failed_finalize(cla):
     with pytest.raises(cla.ClaError, match="earlier cla_block_finalize"):
         blk.add_const([1], np.ones((1, 1)))
     blk.close()
+
+
+def kernels_of(blk, fn):
+    blk.profile(True)
+    fn()
+    names = [k["name"] for k in blk.stats()["kernels"]]
+    blk.profile(False)
+    return names
+
+
+@pytest.mark.parametrize("q", [21, 24, 40])
+@pytest.mark.parametrize("with_other_groups", [False, True])
+def test_wide_right_multiply_on_offset_lists(cla, ora, q, with_other_groups):
+    """B wider than what a 1024-row output tile of all columns takes in LDS: the tile kernel of the offset lists runs
+    per chunk of columns (21 = 11 + 10, 40 = 4 x 10) instead of one atomic add per entry and column in global memory."""
+    from systemds_amd import synth
+    rng = np.random.default_rng(q)
+    n_rows = 30011
+    specs, c = [], 0
+    for g in range(12):
+        specs.append(synth.sdc_group(np.random.default_rng((q, g)), n_rows, np.array([c], np.int32), 20, [0.1, 0.004][g % 2], [None, 0.25][g % 3 == 0]))
+        c += 1
+    if with_other_groups:
+        specs.append(synth.GroupSpec("ddc", np.array([c, c + 1], np.int32), rng.standard_normal((9, 2)), rng.integers(0, 9, n_rows).astype(np.uint8)))
+        specs.append(synth.GroupSpec("unc", np.array([c + 2], np.int32), dense=rng.standard_normal((n_rows, 1))))
+        c += 3
+    B = rng.standard_normal((c, q))
+    D = ora.np_decompress(specs, n_rows, c)
+    blk = cla.build_block(n_rows, c, specs)
+    try:
+        out, nnz = blk.rmm(B)
+        names = kernels_of(blk, lambda: blk.rmm(B))
+    finally:
+        blk.close()
+    assert_matches_truth(out, D, B, what=f"X %*% B, {q} columns")
+    assert nnz == np.count_nonzero(out)
+    assert "k_rmm_sdc_scatter" not in names and names.count("k_rmm_sdc_tiles") >= 2, names
+
+
+@pytest.mark.parametrize("q", [2, 3, 5, 7])
+def test_narrow_right_multiply_on_a_wide_ddc_block(cla, ora, q):
+    """60 single-column groups of 256 tuples: more dictionary than the decode kernel holds in LDS; B of 2 to 7
+    columns then goes to the matrix-core kernel, zero padded."""
+    from systemds_amd import synth
+    c = synth.config2(scale=250, n_cols=60)
+    n_rows, n_cols = c["n_rows"], c["n_cols"]
+    B = np.random.default_rng(q).standard_normal((n_cols, q))
+    D = ora.np_decompress(c["groups"], n_rows, n_cols)
+    blk = cla.build_block(n_rows, n_cols, c["groups"])
+    try:
+        out, nnz = blk.rmm(B)
+        names = kernels_of(blk, lambda: blk.rmm(B))
+    finally:
+        blk.close()
+    assert_matches_truth(out, D, B, what=f"X %*% B, {q} columns")
+    assert nnz == np.count_nonzero(out)
+    assert "k_rmm_mfma" in names or "k_rmm_decode" in names, names
+
+
+def test_single_column_on_a_mixed_block_takes_the_decode_kernel(cla, ora):
+    """X %*% v on a block of RLE, DDC, dense and a few offset-list groups (C5's shape)."""
+    from systemds_amd import synth
+    c = synth.config5(scale=500)
+    n_rows, n_cols = c["n_rows"], c["n_cols"]
+    v = np.random.default_rng(4).standard_normal((n_cols, 1))
+    D = ora.np_decompress(c["groups"], n_rows, n_cols)
+    blk = cla.build_block(n_rows, n_cols, c["groups"])
+    try:
+        out, nnz = blk.rmm(v)
+        names = kernels_of(blk, lambda: blk.rmm(v))
+        w = np.random.default_rng(5).standard_normal((n_rows, 1))
+        chain, _ = blk.mmchain(v, w, 1)
+    finally:
+        blk.close()
+    assert_matches_truth(out, D, v, what="C5 X %*% v")
+    assert nnz == np.count_nonzero(out)
+    assert "k_rmm_decode" in names, names
+    assert_matches_truth(chain.reshape(-1, 1), D.T, (D @ v) * w, what="C5 chain")
