@@ -1,5 +1,5 @@
 // Decode-and-multiply on blocks of any group mix, on the matrix cores:
-//   k_rmm_decode      X %*% B for narrow B (2 <= q <= 16)
+//   k_rmm_decode      X %*% B for narrow B (q <= 16; a single column where the block is not mostly offset lists)
 //   k_tsmm_decode<NB> upper triangle of t(X) %*% X for blocks of at most 16 * NB <= 64 columns (or, for a pair of
 //               column chunks, only the tiles of the first chunk's column blocks with the second's)
 // A block owns a contiguous range of 1024-row tiles. Per tile every dictionary coded
