@@ -283,6 +283,11 @@ int launch_lmm(cla_block* b, const double* dY, int p, double* dOut, unsigned lon
 	const int64_t nRows = b->nRows;
 	hipStream_t st = b->stream;
 	clear_stats(b);
+	// mixed blocks of few columns: one pass on the decoded Gram kernel
+	{
+		const int j = launch_lmm_joint(b, dY, p, dOut, dNnz);
+		if(j <= 0) return j;
+	}
 	int rc = ensure_tables(b, (size_t) p * b->totalVals + (size_t) p + 8);
 	if(rc) return rc;
 	double* dPre = b->dTables;

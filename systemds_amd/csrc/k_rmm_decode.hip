@@ -897,6 +897,26 @@ static int dec_prepare(cla_block* b, bool gram, int q, int rpl, DecLaunch& L, si
 	return e.rc;
 }
 
+// The plan of the decoded Gram matrix: all dictionaries in LDS, else the large ones in global memory (flat).
+static int gram_prepare(cla_block* b, DecLaunch& L, bool& flat) {
+	flat = false;
+	int rc = dec_prepare(b, true, 0, 4, L);
+	if(rc == 1) { // large dictionaries stay in global memory
+		flat = true;
+		rc = dec_prepare(b, true, 0, 4, L, 512);
+	}
+	if(rc == 1) rc = dec_prepare(b, true, 0, 4, L, 64); // many mid-sized dictionaries: only the small ones in LDS
+	return rc;
+}
+
+// 0 when launch_tsmm_decode would take the block, 1 when not (LDS), negative on error.
+int tsmm_decode_fits(cla_block* b) {
+	if(b->groups.empty() || b->nRows == 0 || b->nCols > 64) return 1;
+	DecLaunch L;
+	bool flat;
+	return gram_prepare(b, L, flat);
+}
+
 // Returns 1 when the block/shape is not eligible (caller uses the generic path).
 int launch_rmm_decode(cla_block* b, const double* dB, int q, const double* dConstRow, double* dOut,
 	unsigned long long* dNnz) {
@@ -933,12 +953,7 @@ int launch_tsmm_decode(cla_block* b, double* dOut) {
 	if(XB < 1 || XB > 2 || NB - XB < 1 || NB - XB > 2) XB = 0;
 	DecLaunch L;
 	bool flat = false;
-	int rc = dec_prepare(b, true, 0, 4, L);
-	if(rc == 1) { // large dictionaries stay in global memory
-		flat = true;
-		rc = dec_prepare(b, true, 0, 4, L, 512);
-	}
-	if(rc == 1) rc = dec_prepare(b, true, 0, 4, L, 64); // many mid-sized dictionaries: only the small ones in LDS
+	int rc = gram_prepare(b, L, flat);
 	if(rc) return rc;
 	L.A.out = dOut;
 	Prof pf(b, "k_tsmm_decode", L.grid, DEC_THREADS, (long) L.lds, (double) b->device_bytes_cached);

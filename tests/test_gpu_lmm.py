@@ -178,3 +178,57 @@ def test_byte_code_block_with_non_finite_dictionary_values(cla, ora):
     D = np.nan_to_num(ora.np_decompress(c["groups"], n_rows, n_cols), nan=0.0, posinf=0.0, neginf=0.0)
     assert_fp64_close(out[fin], ref[fin], ora.abs_matmul(Y, D)[fin], what="t(Y)%*%X, non-finite dictionary", n_terms=n_rows)
     assert nnz == rnnz
+
+
+@pytest.mark.parametrize("p", [1, 2, 5, 8, 16])
+def test_mixed_block_takes_one_decoded_pass(cla, ora, p):
+    """C5's shape (RLE, two-byte DDC, offset lists with a default, dense columns): Y %*% X as the cross part of the
+    decoded Gram matrix of cbind(t(Y), X) for 2 or more rows of Y; with the option off the bin
+    kernels give the same cells."""
+    from systemds_amd import synth
+    c = synth.config5(scale=400)
+    n_rows, n_cols = c["n_rows"], c["n_cols"]
+    Y = np.random.default_rng(p).standard_normal((p, n_rows))
+    D = ora.np_decompress(c["groups"], n_rows, n_cols)
+    blk = cla.build_block(n_rows, n_cols, c["groups"])
+    try:
+        out, nnz = blk.lmm(Y)
+        blk.profile(True)
+        out2, _ = blk.lmm(Y)
+        names = [k["name"] for k in blk.stats()["kernels"]]
+        blk.profile(False)
+        blk.set_option("lmm_joint", 0)
+        bins, nnz_b = blk.lmm(Y)
+    finally:
+        blk.close()
+    if 2 <= p <= 8:
+        assert "k_tsmm_decode" in names and "k_lmm_preagg_rows" not in names, names
+    else:  # one row of Y, or t(Y)'s tile (8 KB of LDS per row of Y) does not fit next to the block's dictionaries: the bin kernels
+        assert "k_tsmm_dense" not in names, names
+    assert_matches_truth(out, Y, D, what=f"Y %*% X, {p} rows")
+    assert_matches_truth(bins, Y, D, what=f"Y %*% X, {p} rows, bin kernels")
+    assert np.array_equal(out, out2) or np.allclose(out, out2, rtol=1e-12, atol=0)
+    assert nnz == np.count_nonzero(out) and nnz_b == np.count_nonzero(bins)
+
+
+def test_mixed_block_with_non_finite_values_in_y(cla, ora):
+    """An infinite Y at a row that an RLE group's runs or an offset list do not cover stays out of that group's sums
+    (the reference aggregates listed rows only): such a Y takes the bin kernels; the cells are the oracle's."""
+    n_rows = 40001
+    specs, n_cols = mixed_block(13, n_rows, with_unc=True)
+    Y = np.random.default_rng(8).standard_normal((2, n_rows))
+    Y[0, 7] = np.inf
+    Y[1, n_rows - 3] = -np.inf
+    Y[1, 12345] = np.nan
+    blk = cla.build_block(n_rows, n_cols, specs)
+    try:
+        out, nnz = blk.lmm(Y)
+    finally:
+        blk.close()
+    ref, rnnz = ora.lmm(ora.Groups(specs, n_rows, n_cols), Y, 4)
+    fin = np.isfinite(ref)
+    assert np.array_equal(np.isfinite(out), fin)
+    assert np.array_equal(out[~fin], ref[~fin], equal_nan=True)
+    D = ora.np_decompress(specs, n_rows, n_cols)
+    Yc = np.nan_to_num(Y, nan=0.0, posinf=0.0, neginf=0.0)
+    assert_fp64_close(out[fin], ref[fin], ora.abs_matmul(Yc, D)[fin], what="Y %*% X, non-finite Y", n_terms=n_rows)
