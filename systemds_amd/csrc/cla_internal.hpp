@@ -72,6 +72,7 @@ struct Options {
 	int tsmmNarrow = 1;     // decoded Gram matrix: a last column block of at most 4 columns on the 4 x 4 x 4 matrix instruction
 	int tsmmPairDot = 1;    // DDC x DDC pairs in dot form (0: pre-aggregate form with LDS bins)
 	int expandStreams = 1;  // one code per row for small RLE / SDCZeros groups in the decode kernels
+	int rmmDirect = 1;      // X %*% B for narrow B on blocks of plain streams: codes straight from global memory, sums on the vector unit (0: the tile kernel on the matrix cores)
 	int rmmDisable = 0;     // bit 0 byte-code mat-vec, 1 fused tables of the byte-code mat-vec, 2 matrix-core kernel, 3 decode kernel
 	int lmmDisable = 0;     // bit 0 dot form on byte codes, 1 byte-code bin kernel
 	int lmmJoint = 1;       // left multiply of blocks that are not mostly offset lists or byte-code DDC groups as cbind(t(Y), X) on the decoded Gram kernel
@@ -89,6 +90,7 @@ struct KernelStat {
 };
 
 struct DecPlanCache;
+struct DirPlan;
 
 } // namespace cla
 
@@ -178,6 +180,7 @@ struct cla_block {
 	size_t laneOff[4] = {0, 0, 0, 0};
 	bool laneLmm = false;            // every listed group has one column (the left multiply's condition)
 	cla::DecPlanCache* decPlans = nullptr; // decode kernels (k_rmm_decode.hip): plans per product shape, dropped by dec_plans_drop
+	cla::DirPlan* dirPlan = nullptr;     // plan of k_rmm_direct (dropped with the decode plans)
 	void* dMfPlan = nullptr;         // matrix-core right multiply (k_rmm_mfma.hip): slab descriptors, column info, code streams, B row list
 	int mfState = 0;                 // 0 not planned yet, 1 ready, -1 not eligible
 	int mfNSlabs = 0, mfNColsAll = 0, mfWidth = 1, mfMaxKc = 0, mfNRowCol = 0, mfMaxDict = 0;

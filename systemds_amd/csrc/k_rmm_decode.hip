@@ -19,6 +19,7 @@
 #include "cla_device.hpp"
 #include <algorithm>
 #include <cstring>
+#include <type_traits>
 
 namespace cla {
 
@@ -174,8 +175,8 @@ template <int GRAM, int NB, int RPL, int FLAT, int XB = 0, int NAR = 0>
 __device__ __forceinline__ void decode_body(const DecArgs& A) {
 	extern __shared__ __align__(16) double smem[];
 	double* Bs = smem + A.valDoubles;                              // bDoubles: rows of B in decoded column order, 16 outputs each
-	double* stage = Bs + A.bDoubles;                               // stageDoubles: output staging per wave / Gram tile
-	uint8_t* slots = (uint8_t*) (stage + A.stageDoubles);          // slotBytes (multiple of 16)
+	double* stage = GRAM ? smem : Bs + A.bDoubles;                 // stageDoubles: output staging per wave; the Gram tile takes the place of the values when the rows are done
+	uint8_t* slots = (uint8_t*) (Bs + A.bDoubles + A.stageDoubles); // slotBytes (multiple of 16)
 	DecCol* colS = (DecCol*) (slots + A.slotBytes);                // nColD
 	double* constS = (double*) (colS + A.nColD);                   // nColD (Gram mode)
 	DecGroup* planS = (DecGroup*) (constS + (GRAM ? A.nColD : 0)); // nGroups
@@ -737,7 +738,9 @@ static int dec_build_plan(cla_block* b, bool gram, int q, int rpl, DecLaunch& L,
 	slotB = (slotB + 16 + 15) & ~(size_t) 15; // the multiply phase may read 16 bytes past the last tile
 	const int nColD = gram ? ((nCols + 15) / 16) * 16 : ((K + 3) / 4) * 4;
 	const size_t bD = gram ? 0 : (size_t) nColD * 16;
-	const size_t stageD = gram ? (size_t) nColD * nColD : (size_t) DEC_WAVES * 16 * rpl * q;
+	// (the Gram tile of a block is summed where its dictionaries and dense tiles were, once its rows are done)
+	if(gram) valD = std::max(valD, (size_t) nColD * nColD);
+	const size_t stageD = gram ? 0 : (size_t) DEC_WAVES * 16 * rpl * q;
 	const size_t slotBase = (valD + bD + stageD) * 8;
 	// copy list
 	std::vector<DecCopy> copies;
@@ -864,7 +867,10 @@ struct DecPlanCache {
 	std::vector<DecPlanEntry> entries;
 };
 
+void dir_plan_drop(cla_block* b);
+
 void dec_plans_drop(cla_block* b) {
+	dir_plan_drop(b);
 	if(b->decPlans == nullptr) return;
 	for(auto& e : b->decPlans->entries)
 		if(e.dImg) { (void) hipFree(e.dImg); b->derivedBytes -= e.bytes; }
@@ -917,10 +923,322 @@ int tsmm_decode_fits(cla_block* b) {
 	return gram_prepare(b, L, flat);
 }
 
+// Column classes of k_rmm_direct: its column list is sorted by class, so that each class runs a loop of its own
+// without a test per column.
+enum { DSEG_DDC1 = 0, DSEG_DDC2, DSEG_GAP1, DSEG_GAP2, DSEG_DENSE, DSEG_N };
+typedef const __attribute__((address_space(4))) double* dec_cdp; // read-only for the kernel's duration: uniform addresses become scalar loads
+
+// ---- X %*% B for narrow B without code tiles: k_rmm_direct
+// For blocks whose groups are all plain streams (DDC codes of one or two bytes, the one-code-per-row copies of RLE
+// and SDCZeros groups, rows of uncompressed groups) and whose dictionaries fit LDS together. A wave owns slices of
+// 128 consecutive rows, lane l rows 2 l and 2 l + 1 of the slice: it loads its two codes of a column straight from
+// global memory (64 lanes = one or two full lines), looks the values up in the block's LDS copy of the dictionaries
+// and adds value x B[column, j] to its QV sums per row, B's row coming through scalar loads. No barrier after the
+// dictionaries are in place: the 16 waves of a block drift apart, so that the loads, the multiply-adds and the stores
+// of different waves overlap (the tile kernel's waves walk through fill, multiply and store in step).
+constexpr int DIR_THREADS = 1024;
+constexpr int DIR_WAVES = DIR_THREADS / 64;
+constexpr int DIR_SLICE = 128;   // rows per wave and step
+constexpr int DIR_SROWS = 32;    // rows of a slice that go through the wave's staging area at a time
+
+struct DirCol {          // 32 bytes, read through scalar loads
+	const uint8_t* src;  // code stream, or the column's first value of an uncompressed group
+	int32_t base8;       // bytes from the LDS base: the column's value of tuple 0
+	int32_t nC8;         // bytes per tuple; uncompressed: bytes per row
+	int32_t orig;        // column of the matrix (row of B); below zero: a filler column
+	int32_t r0, r1, r2;
+};
+struct DirDict {
+	const double* src;
+	int32_t n, off;      // doubles, doubles from the LDS base
+};
+struct DirArgs {
+	const DirCol* cols;
+	const DirDict* dicts;
+	const double* zeroRow;
+	int nDicts, dictDoubles;
+	int segEnd[DSEG_N];
+	const double* B;
+	const double* constRow;
+	double* out;
+	int64_t nRows;
+	unsigned long long* nnz;
+};
+typedef const __attribute__((address_space(4))) DirCol* dir_ccp;
+typedef unsigned long long dir_u64x4 __attribute__((ext_vector_type(4)));
+
+template <int QV>
+__global__ __launch_bounds__(DIR_THREADS) void k_rmm_direct(const DirArgs A) {
+	extern __shared__ __align__(16) double smem[];
+	const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+	for(int g = 0; g < A.nDicts; g++) {
+		const DirDict D = A.dicts[g];
+		const double* __restrict__ src = as_global(D.src);
+		for(int i = tid; i < D.n; i += DIR_THREADS) smem[D.off + i] = src[i];
+	}
+	if(tid < 2) smem[A.dictDoubles - 2 + tid] = 0.0; // what a filler column looks up
+	__syncthreads();
+	const uint8_t* const ldsBytes = (const uint8_t*) smem;
+	double* const wstage = smem + A.dictDoubles + (size_t) wave * DIR_SROWS * QV;
+	const dec_cdp Bc = (dec_cdp) A.B;
+	const int64_t nRows = A.nRows;
+	const int64_t nSlices = (nRows + DIR_SLICE - 1) / DIR_SLICE;
+	int cnt = 0;
+	for(int64_t slice = (int64_t) blockIdx.x * DIR_WAVES + wave; slice < nSlices; slice += (int64_t) gridDim.x * DIR_WAVES) {
+		const int64_t s0 = slice * DIR_SLICE, row0 = s0 + 2 * lane;
+		const bool full = s0 + DIR_SLICE <= nRows; // (uniform)
+		const bool in0 = row0 < nRows, in1 = row0 + 1 < nRows;
+		double acc[2][QV];
+#pragma unroll
+		for(int j = 0; j < QV; j++) {
+			const double c0 = A.constRow != nullptr ? ((dec_cdp) A.constRow)[j] : 0.0;
+			acc[0][j] = c0; acc[1][j] = c0;
+		}
+		// NBAT columns of one class at a time; GUARD: the last slice, whose rows may lie behind the end of the matrix
+		auto batch = [&](auto kindTag, auto twoTag, auto nTag, auto guardTag, int k) {
+			constexpr int KIND = decltype(kindTag)::value;
+			constexpr bool TWO = decltype(twoTag)::value;
+			constexpr int NBAT = decltype(nTag)::value;
+			constexpr bool GUARD = decltype(guardTag)::value;
+			double x[NBAT][2];
+			dec_cdp brow[NBAT];
+			const uint8_t* src[NBAT];
+			int base8[NBAT], nC8[NBAT];
+			uint32_t cc[NBAT];
+			dir_u64x4 D[NBAT];
+#pragma unroll
+			for(int u = 0; u < NBAT; u++) D[u] = *(const __attribute__((address_space(4))) dir_u64x4*) (A.cols + k + u);
+			__builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+			for(int u = 0; u < NBAT; u++) {
+				src[u] = (const uint8_t*) D[u][0];
+				base8[u] = (int) (uint32_t) D[u][1]; nC8[u] = (int) (D[u][1] >> 32);
+				const int orig = (int) (uint32_t) D[u][2];
+				brow[u] = orig < 0 ? (dec_cdp) A.zeroRow : Bc + (size_t) orig * QV;
+			}
+#pragma unroll
+			for(int u = 0; u < NBAT; u++) {
+				// (the slice's start goes into the uniform part of the address, the lane's part stays small)
+				typedef const __attribute__((address_space(1))) uint8_t* gp8;
+				if(KIND == 2) {
+					const gp8 p = (gp8) src[u] + (size_t) s0 * nC8[u];
+					const int lo = __umul24(2 * lane, nC8[u]);
+					x[u][0] = !GUARD || in0 ? *(const __attribute__((address_space(1))) double*) (p + lo) : 0.0;
+					x[u][1] = !GUARD || in1 ? *(const __attribute__((address_space(1))) double*) (p + lo + nC8[u]) : 0.0;
+				}
+				else if(TWO) {
+					const gp8 p = (gp8) src[u] + (size_t) s0 * 2;
+					if(!GUARD || in1) cc[u] = *(const __attribute__((address_space(1))) uint32_t*) (p + 4 * lane);
+					else cc[u] = in0 ? *(const __attribute__((address_space(1))) uint16_t*) (p + 4 * lane) : 0u;
+				}
+				else {
+					const gp8 p = (gp8) src[u] + (size_t) s0;
+					if(!GUARD || in1) cc[u] = *(const __attribute__((address_space(1))) uint16_t*) (p + 2 * lane);
+					else cc[u] = in0 ? *(p + 2 * lane) : 0u;
+				}
+			}
+			__builtin_amdgcn_sched_barrier(0);
+			if(KIND != 2) {
+				bool valid[NBAT][2];
+#pragma unroll
+				for(int u = 0; u < NBAT; u++)
+#pragma unroll
+					for(int r = 0; r < 2; r++) {
+						const int c = TWO ? (int) ((cc[u] >> (16 * r)) & 0xffff) : (int) ((cc[u] >> (8 * r)) & 0xff);
+						valid[u][r] = (!GUARD || (r == 0 ? in0 : in1)) & (KIND == 3 || c != 0xff);
+						x[u][r] = *(const double*) (ldsBytes + (base8[u] + __umul24(KIND == 3 && !GUARD ? c : valid[u][r] ? c : 0, nC8[u])));
+					}
+				__builtin_amdgcn_sched_barrier(0);
+				if(KIND == 1) {
+#pragma unroll
+					for(int u = 0; u < NBAT; u++)
+#pragma unroll
+						for(int r = 0; r < 2; r++) x[u][r] = valid[u][r] ? x[u][r] : 0.0;
+				}
+			}
+#pragma unroll
+			for(int u = 0; u < NBAT; u++)
+#pragma unroll
+				for(int j = 0; j < QV; j++) {
+					const double bv = brow[u][j];
+					acc[0][j] = __builtin_fma(x[u][0], bv, acc[0][j]);
+					acc[1][j] = __builtin_fma(x[u][1], bv, acc[1][j]);
+				}
+		};
+		auto seg = [&](auto kindTag, auto twoTag, int k0, int k1) {
+			int k = k0; // (every class holds an even number of columns)
+			if(full) {
+#pragma unroll 1
+				for(; k + 8 <= k1; k += 8) batch(kindTag, twoTag, std::integral_constant<int, 8>(), std::false_type(), k);
+				if(k + 4 <= k1) { batch(kindTag, twoTag, std::integral_constant<int, 4>(), std::false_type(), k); k += 4; }
+				if(k + 2 <= k1) batch(kindTag, twoTag, std::integral_constant<int, 2>(), std::false_type(), k);
+			}
+			else {
+#pragma unroll 1
+				for(; k + 2 <= k1; k += 2) batch(kindTag, twoTag, std::integral_constant<int, 2>(), std::true_type(), k);
+			}
+		};
+		seg(std::integral_constant<int, 3>(), std::false_type(), 0, A.segEnd[DSEG_DDC1]);
+		seg(std::integral_constant<int, 3>(), std::true_type(), A.segEnd[DSEG_DDC1], A.segEnd[DSEG_DDC2]);
+		seg(std::integral_constant<int, 1>(), std::false_type(), A.segEnd[DSEG_DDC2], A.segEnd[DSEG_GAP1]);
+		seg(std::integral_constant<int, 2>(), std::false_type(), A.segEnd[DSEG_GAP2], A.segEnd[DSEG_DENSE]);
+		// through the wave's staging area, 32 rows (16 lanes) at a time: full-line stores of consecutive output rows
+#pragma unroll 1
+		for(int part = 0; part < DIR_SLICE / DIR_SROWS; part++) {
+			dec_wave_sync(); // the readers of the staging area are done
+			if((lane >> 4) == part) {
+				double* w = wstage + (size_t) (lane & 15) * 2 * QV;
+#pragma unroll
+				for(int j = 0; j < QV; j++) { w[j] = acc[0][j]; w[QV + j] = acc[1][j]; }
+			}
+			dec_wave_sync();
+			const int64_t rowBase = s0 + part * DIR_SROWS;
+			const int nr = (int) max((int64_t) 0, min((int64_t) DIR_SROWS, nRows - rowBase));
+			const int n = nr * QV;
+			double* o = A.out + (size_t) rowBase * QV; // (a multiple of 16 bytes: rowBase is even)
+#pragma unroll
+			for(int i = 2 * lane; i < DIR_SROWS * QV; i += 128) {
+				if(i + 1 < n) {
+					const f64x2 v = *(const f64x2*) (wstage + i);
+					cnt += (v[0] != 0.0) + (v[1] != 0.0);
+					__builtin_nontemporal_store(v, (f64x2*) (o + i));
+				}
+				else if(i < n) {
+					const double v = wstage[i];
+					cnt += v != 0.0;
+					__builtin_nontemporal_store(v, o + i);
+				}
+			}
+		}
+	}
+	count_add(A.nnz, cnt);
+}
+
+struct DirPlan {
+	int rc = 1;            // 0 usable, 1 the block does not qualify
+	void* dImg = nullptr;
+	int64_t bytes = 0;
+	DirArgs A;
+};
+
+static int dir_build_plan(cla_block* b, DirPlan& P) {
+	P.rc = 1;
+	const int nG = (int) b->groups.size();
+	{
+		const int rc = ensure_expanded(b);
+		if(rc) return rc;
+	}
+	std::vector<DirDict> dicts;
+	std::vector<DirCol> cols[DSEG_N];
+	size_t valD = 0;
+	for(int g = 0; g < nG; g++) {
+		const DGroup& G = b->groups[g].d;
+		const auto& hc = b->groups[g].cols;
+		if(G.nColG >= (1 << 14)) return 0;
+		if(G.type == G_UNC) {
+			if(((uintptr_t) G.dense & 7) != 0) return 0;
+			for(int h = 0; h < G.nColG; h++) cols[DSEG_DENSE].push_back(DirCol{(const uint8_t*) (G.dense + h), 0, G.nColG * 8, hc[h], 0, 0, 0});
+			continue;
+		}
+		if(G.type != G_DDC && G.type != G_RLE && !(G.type == G_SDCZ && G.nOffsets > 0)) continue; // no row data
+		const uint8_t* src;
+		int cls;
+		if(G.type == G_DDC) {
+			if(G.codeWidth > 2 || ((uintptr_t) G.codes & 3) != 0) return 0;
+			src = (const uint8_t*) G.codes;
+			cls = G.codeWidth == 2 ? DSEG_DDC2 : DSEG_DDC1;
+		}
+		else {
+			if(b->expCodes[g] == nullptr) return 0;
+			src = b->expCodes[g];
+			cls = DSEG_GAP1;
+		}
+		dicts.push_back(DirDict{G.dict, G.nVals * G.nColG, (int32_t) valD});
+		for(int h = 0; h < G.nColG; h++) cols[cls].push_back(DirCol{src, (int32_t) (8 * (valD + h)), G.nColG * 8, hc[h], 0, 0, 0});
+		valD += (size_t) G.nVals * G.nColG;
+		if(valD * 8 > (size_t) 150 * 1024) return 0;
+	}
+	valD = (valD + 1) & ~(size_t) 1;
+	const size_t zeroAt = valD; // two zeros behind the dictionaries
+	valD += 2;
+	std::vector<DirCol> all;
+	for(int sgm = 0; sgm < DSEG_N; sgm++) {
+		for(const DirCol& C : cols[sgm]) all.push_back(C);
+		if((cols[sgm].size() & 1) != 0) { // classes of even size: a filler column (a real stream, the zero behind the dictionaries, a row of zeros for B)
+			DirCol F = cols[sgm].back();
+			if(sgm == DSEG_DENSE) return 0; // (a dense filler would need a stream of its own: odd numbers of dense columns take the tile kernel)
+			F.base8 = (int32_t) (8 * zeroAt); F.nC8 = 0; F.orig = -1;
+			all.push_back(F);
+		}
+		P.A.segEnd[sgm] = (int) all.size();
+	}
+	if(all.empty()) return 0;
+	const size_t colBytes = all.size() * sizeof(DirCol), dictBytes = dicts.size() * sizeof(DirDict);
+	std::vector<uint8_t> img(colBytes + dictBytes + 16 * 8, 0);
+	std::memcpy(img.data(), all.data(), colBytes);
+	if(dictBytes) std::memcpy(img.data() + colBytes, dicts.data(), dictBytes);
+	uint8_t* d = nullptr;
+	CLA_HIP(hipMalloc((void**) &d, img.size() + 64));
+	P.dImg = d;
+	P.bytes = (int64_t) img.size() + 64;
+	CLA_HIP(hipMemcpy(d, img.data(), img.size(), hipMemcpyHostToDevice));
+	P.A.cols = (const DirCol*) d;
+	P.A.dicts = (const DirDict*) (d + colBytes);
+	P.A.zeroRow = (const double*) (d + colBytes + dictBytes);
+	P.A.nDicts = (int) dicts.size();
+	P.A.dictDoubles = (int) valD;
+	P.A.nRows = b->nRows;
+	P.rc = 0;
+	return 0;
+}
+
+void dir_plan_drop(cla_block* b) {
+	if(b->dirPlan == nullptr) return;
+	if(b->dirPlan->dImg) { (void) hipFree(b->dirPlan->dImg); b->derivedBytes -= b->dirPlan->bytes; }
+	delete b->dirPlan;
+	b->dirPlan = nullptr;
+}
+
+// Returns 1 when the block does not qualify (the caller takes the tile kernel).
+static int launch_rmm_direct(cla_block* b, const double* dB, int q, const double* dConstRow, double* dOut, unsigned long long* dNnz) {
+	if(b->dirPlan == nullptr) {
+		b->dirPlan = new DirPlan();
+		const int rc = dir_build_plan(b, *b->dirPlan);
+		if(rc < 0) { dir_plan_drop(b); return rc; }
+		if(b->dirPlan->dImg) b->derivedBytes += b->dirPlan->bytes;
+	}
+	if(b->dirPlan->rc) return 1;
+	DirArgs A = b->dirPlan->A;
+	const size_t lds = ((size_t) A.dictDoubles + (size_t) DIR_WAVES * DIR_SROWS * q) * 8;
+	if(lds > (size_t) std::min(g_ldsPerBlock, 160 * 1024) - 1024) return 1;
+	A.B = dB; A.constRow = dConstRow; A.out = dOut; A.nnz = dNnz;
+	const int64_t nSlices = (b->nRows + DIR_SLICE - 1) / DIR_SLICE;
+	const unsigned grid = (unsigned) std::min<int64_t>((nSlices + DIR_WAVES - 1) / DIR_WAVES, g_numCU);
+	const double algo = (double) b->device_bytes_cached + (double) b->nRows * q * 8;
+	Prof pf(b, "k_rmm_direct", grid, DIR_THREADS, (long) lds, algo);
+	switch(q) {
+#define DIR_CASE(QV)                                                                              \
+	case QV:                                                                                      \
+		CLA_HIP(allow_full_lds((const void*) k_rmm_direct<QV>));                                  \
+		hipLaunchKernelGGL(k_rmm_direct<QV>, dim3(grid), dim3(DIR_THREADS), lds, b->stream, A); \
+		break;
+		DIR_CASE(1) DIR_CASE(2) DIR_CASE(3) DIR_CASE(4) DIR_CASE(5) DIR_CASE(6) DIR_CASE(7) DIR_CASE(8)
+		DIR_CASE(9) DIR_CASE(10) DIR_CASE(11) DIR_CASE(12) DIR_CASE(13) DIR_CASE(14) DIR_CASE(15) DIR_CASE(16)
+#undef DIR_CASE
+		default: return 1;
+	}
+	CLA_HIP(hipGetLastError());
+	return 0;
+}
+
 // Returns 1 when the block/shape is not eligible (caller uses the generic path).
 int launch_rmm_decode(cla_block* b, const double* dB, int q, const double* dConstRow, double* dOut,
 	unsigned long long* dNnz) {
 	if(b->groups.empty() || b->nRows == 0 || q < 1 || q > DEC_QMAX) return 1;
+	if(b->opt.rmmDirect) {
+		const int rc = launch_rmm_direct(b, dB, q, dConstRow, dOut, dNnz);
+		if(rc != 1) return rc;
+	}
 	DecLaunch L;
 	int rpl = 4; // rows per lane and pass: the smaller output staging area when LDS is short
 	int rc = dec_prepare(b, false, q, rpl, L);

@@ -331,10 +331,10 @@ def test_wide_right_multiply_on_offset_lists(cla, ora, q, with_other_groups):
 
 @pytest.mark.parametrize("q", [2, 3, 5, 7])
 def test_narrow_right_multiply_on_a_wide_ddc_block(cla, ora, q):
-    """60 single-column groups of 256 tuples: more dictionary than the decode kernel holds in LDS; B of 2 to 7
+    """80 single-column groups of 256 tuples: more dictionary than the narrow-B kernels hold in LDS; B of 2 to 7
     columns then goes to the matrix-core kernel, zero padded."""
     from systemds_amd import synth
-    c = synth.config2(scale=250, n_cols=60)
+    c = synth.config2(scale=250, n_cols=80)
     n_rows, n_cols = c["n_rows"], c["n_cols"]
     B = np.random.default_rng(q).standard_normal((n_cols, q))
     D = ora.np_decompress(c["groups"], n_rows, n_cols)
@@ -346,7 +346,7 @@ def test_narrow_right_multiply_on_a_wide_ddc_block(cla, ora, q):
         blk.close()
     assert_matches_truth(out, D, B, what=f"X %*% B, {q} columns")
     assert nnz == np.count_nonzero(out)
-    assert "k_rmm_mfma" in names or "k_rmm_decode" in names, names
+    assert "k_rmm_mfma" in names, names
 
 
 def test_single_column_on_a_mixed_block_takes_the_decode_kernel(cla, ora):
@@ -366,5 +366,106 @@ def test_single_column_on_a_mixed_block_takes_the_decode_kernel(cla, ora):
         blk.close()
     assert_matches_truth(out, D, v, what="C5 X %*% v")
     assert nnz == np.count_nonzero(out)
-    assert "k_rmm_decode" in names, names
+    assert "k_rmm_direct" in names, names
     assert_matches_truth(chain.reshape(-1, 1), D.T, (D @ v) * w, what="C5 chain")
+
+
+def _plain_stream_block(seed, n_rows, odd_dense=False, overlap=False):
+    """Groups that are plain streams on the device: DDC with one- and two-byte codes (single and co-coded columns),
+    small RLE and SDC groups (which get one code per row), dense columns, a constant and an empty group. Odd numbers
+    of columns per class, so that the filler columns of the kernel take part."""
+    from systemds_amd import synth
+    rng = np.random.default_rng(seed)
+    specs, c = [], 0
+
+    def cols(n):
+        nonlocal c
+        r = np.arange(c, c + n, dtype=np.int32)
+        c += n
+        return r
+    specs.append(synth.GroupSpec("ddc", cols(1), rng.standard_normal((7, 1)), rng.integers(0, 7, n_rows).astype(np.uint8)))
+    specs.append(synth.GroupSpec("ddc", cols(2), rng.standard_normal((200, 2)), rng.integers(0, 200, n_rows).astype(np.uint8)))
+    specs.append(synth.GroupSpec("ddc", cols(2), rng.standard_normal((300, 2)), rng.integers(0, 300, n_rows).astype(np.uint16)))
+    specs.append(synth.GroupSpec("ddc", cols(1), rng.standard_normal((1500, 1)), rng.integers(0, 1500, n_rows).astype(np.uint16)))
+    specs.append(synth.sdc_group(rng, n_rows, cols(1), 5, 0.1, None))
+    specs.append(synth.sdc_group(rng, n_rows, cols(2), 6, 0.3, 1.5))
+    run_codes = rng.integers(-1, 4, size=n_rows // 20 + 2)
+    codes = np.repeat(run_codes, rng.integers(1, 60, size=run_codes.size))[:n_rows]
+    if codes.size < n_rows:
+        codes = np.concatenate([codes, np.full(n_rows - codes.size, -1)])
+    ptr, data = synth.encode_rle(codes, 4)
+    specs.append(synth.GroupSpec("rle", cols(1), rng.standard_normal((4, 1)), ptr=ptr, rle=data))
+    specs.append(synth.GroupSpec("unc", cols(1 if odd_dense else 2), dense=rng.standard_normal((n_rows, 1 if odd_dense else 2))))
+    specs.append(synth.GroupSpec("const", cols(1), np.array([[2.5]])))
+    specs.append(synth.GroupSpec("empty", cols(1)))
+    if overlap:
+        specs.append(synth.GroupSpec("ddc", np.array([0, 3], np.int32), rng.standard_normal((9, 2)), rng.integers(0, 9, n_rows).astype(np.uint8)))
+    return specs, c
+
+
+@pytest.mark.parametrize("n_rows", [1, 2, 127, 128, 129, 255, 4097, 70001])
+@pytest.mark.parametrize("q", [1, 2, 3, 7, 10, 16])
+def test_narrow_right_multiply_straight_from_the_streams(cla, ora, n_rows, q):
+    """X %*% B for at most 16 columns of B on a block of plain streams: codes read straight from global memory
+    (`k_rmm_direct`), against the oracle, the long-double truth and the tile kernel (`rmm_direct` 0)."""
+    specs, n_cols = _plain_stream_block(n_rows + q, n_rows, overlap=q == 3)
+    B = np.random.default_rng(q).standard_normal((n_cols, q))
+    D = ora.np_decompress(specs, n_rows, n_cols)
+    ref, rnnz = ora.rmm(ora.Groups(specs, n_rows, n_cols), B, 4)
+    blk = cla.build_block(n_rows, n_cols, specs)
+    try:
+        out, nnz = blk.rmm(B)
+        names = kernels_of(blk, lambda: blk.rmm(B))
+        blk.set_option("rmm_direct", 0)
+        out0, nnz0 = blk.rmm(B)
+        names0 = kernels_of(blk, lambda: blk.rmm(B))
+    finally:
+        blk.close()
+    assert "k_rmm_direct" in names and "k_rmm_direct" not in names0, (names, names0)
+    assert_fp64_close(out, ref, ora.abs_matmul(D, B), what=f"direct q={q}", n_terms=n_cols)
+    assert_matches_truth(out[:5000], D[:5000], B, what=f"direct q={q}")
+    assert_matches_truth(out[-300:], D[-300:], B, what=f"direct q={q}, last rows")
+    assert_matches_truth(out0[:5000], D[:5000], B, what=f"tiles q={q}")
+    assert nnz == rnnz == np.count_nonzero(out) and nnz0 == rnnz
+
+
+@pytest.mark.parametrize("q", [4, 5, 6, 8, 9, 11, 12, 13, 14, 15])
+def test_narrow_right_multiply_straight_from_the_streams_other_widths(cla, ora, q):
+    n_rows = 3000 + q
+    specs, n_cols = _plain_stream_block(q, n_rows)
+    B = np.random.default_rng(q).standard_normal((n_cols, q))
+    D = ora.np_decompress(specs, n_rows, n_cols)
+    blk = cla.build_block(n_rows, n_cols, specs)
+    try:
+        out, nnz = blk.rmm(B)
+        names = kernels_of(blk, lambda: blk.rmm(B))
+    finally:
+        blk.close()
+    assert "k_rmm_direct" in names, names
+    assert_matches_truth(out, D, B, what=f"direct q={q}")
+    assert nnz == np.count_nonzero(out)
+
+
+def test_blocks_the_stream_kernel_does_not_take(cla, ora):
+    """An odd number of dense columns, four-byte codes: the tile kernel as before."""
+    from systemds_amd import synth
+    n_rows = 5000
+    B = None
+    for variant in ("odd_dense", "int_codes"):
+        specs, n_cols = _plain_stream_block(11, n_rows, odd_dense=variant == "odd_dense")
+        if variant == "int_codes":
+            rng = np.random.default_rng(3)
+            specs.append(synth.GroupSpec("ddc", np.array([n_cols], np.int32), rng.standard_normal((70000, 1)),
+                                         rng.integers(0, 70000, n_rows).astype(np.int32)))
+            n_cols += 1
+        B = np.random.default_rng(1).standard_normal((n_cols, 5))
+        D = ora.np_decompress(specs, n_rows, n_cols)
+        blk = cla.build_block(n_rows, n_cols, specs)
+        try:
+            out, nnz = blk.rmm(B)
+            names = kernels_of(blk, lambda: blk.rmm(B))
+        finally:
+            blk.close()
+        assert "k_rmm_direct" not in names, (variant, names)
+        assert_matches_truth(out, D, B, what=f"{variant}")
+        assert nnz == np.count_nonzero(out)
