@@ -1199,15 +1199,22 @@ void dir_plan_drop(cla_block* b) {
 	b->dirPlan = nullptr;
 }
 
-// Returns 1 when the block does not qualify (the caller takes the tile kernel).
-static int launch_rmm_direct(cla_block* b, const double* dB, int q, const double* dConstRow, double* dOut, unsigned long long* dNnz) {
+static int dir_plan_get(cla_block* b) {
 	if(b->dirPlan == nullptr) {
 		b->dirPlan = new DirPlan();
 		const int rc = dir_build_plan(b, *b->dirPlan);
 		if(rc < 0) { dir_plan_drop(b); return rc; }
 		if(b->dirPlan->dImg) b->derivedBytes += b->dirPlan->bytes;
 	}
-	if(b->dirPlan->rc) return 1;
+	return b->dirPlan->rc;
+}
+
+// Returns 1 when the block does not qualify (the caller takes the tile kernel).
+static int launch_rmm_direct(cla_block* b, const double* dB, int q, const double* dConstRow, double* dOut, unsigned long long* dNnz) {
+	{
+		const int rc = dir_plan_get(b);
+		if(rc) return rc;
+	}
 	DirArgs A = b->dirPlan->A;
 	const size_t lds = ((size_t) A.dictDoubles + (size_t) DIR_WAVES * DIR_SROWS * q) * 8;
 	if(lds > (size_t) std::min(g_ldsPerBlock, 160 * 1024) - 1024) return 1;

@@ -9,6 +9,7 @@
 //   6. LDS table lookups as the mat-vec gather does them (byte -> ds_read_b64 -> add), random and conflict-free
 // Usage: cla_probe            (a few seconds; every kernel is a bounded loop)
 #include <hip/hip_runtime.h>
+#include <algorithm>
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
@@ -106,6 +107,91 @@ __global__ __launch_bounds__(256) void k_mfma16(double* out, int iters) {
 	out[8 + blockIdx.x * 256 + threadIdx.x] = s;
 }
 
+// Two waves per SIMD (one block of 8 waves per CU): the first four waves issue matrix instructions, the last four
+// vector instructions (fp64 multiply-adds or integer adds), alone and together. If the two kinds ran on units of their
+// own, "together" would take as long as the longer of the two; if they share the fp64 datapath, as long as their sum.
+template <int MODE_A, int MODE_B>
+__global__ __launch_bounds__(512) void k_mix(double* out, int iters) {
+	const int wave = threadIdx.x >> 6;
+	const int mode = wave < 4 ? MODE_A : MODE_B; // 0 idle, 1 v_mfma_f64_4x4x4, 2 v_mfma_f64_16x16x4, 3 v_fma_f64, 4 v_add_u32
+	const double a = out[threadIdx.x & 7], b = out[(threadIdx.x + 1) & 7];
+	double s = 0;
+	if(mode == 1) {
+		double acc[8];
+#pragma unroll
+		for(int i = 0; i < 8; i++) acc[i] = 0;
+		for(int it = 0; it < iters; it++)
+#pragma unroll
+			for(int i = 0; i < 8; i++) acc[i] = __builtin_amdgcn_mfma_f64_4x4x4f64(a, b, acc[i], 0, 0, 0);
+#pragma unroll
+		for(int i = 0; i < 8; i++) s += acc[i];
+	}
+	else if(mode == 2) {
+		f64x4 acc[8];
+#pragma unroll
+		for(int i = 0; i < 8; i++) acc[i] = f64x4{0, 0, 0, 0};
+		for(int it = 0; it < iters / 4; it++)
+#pragma unroll
+			for(int i = 0; i < 8; i++) acc[i] = __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, acc[i], 0, 0, 0);
+#pragma unroll
+		for(int i = 0; i < 8; i++) s += acc[i][0] + acc[i][3];
+	}
+	else if(mode == 3) {
+		double acc[8];
+#pragma unroll
+		for(int i = 0; i < 8; i++) acc[i] = i;
+		for(int it = 0; it < iters * 4; it++)
+#pragma unroll
+			for(int i = 0; i < 8; i++) acc[i] = __builtin_fma(acc[i], a, b);
+#pragma unroll
+		for(int i = 0; i < 8; i++) s += acc[i];
+	}
+	else if(mode == 4) {
+		unsigned acc[8];
+#pragma unroll
+		for(int i = 0; i < 8; i++) acc[i] = threadIdx.x + i;
+		const unsigned k = (unsigned) (a * 1e6);
+		for(int it = 0; it < iters * 4; it++)
+#pragma unroll
+			for(int i = 0; i < 8; i++) acc[i] = (acc[i] + k) ^ (unsigned) it;
+#pragma unroll
+		for(int i = 0; i < 8; i++) s += acc[i];
+	}
+	out[8 + blockIdx.x * 512 + threadIdx.x] = s;
+}
+
+template <int MA, int MB>
+static float mix_ms(double* out, int iters) {
+	return time_ms([&] { hipLaunchKernelGGL((k_mix<MA, MB>), dim3(g_cus), dim3(512), 0, 0, out, iters); }, 2);
+}
+
+static void probe_mix() {
+	double* out;
+	CK(hipMalloc(&out, sizeof(double) * (8 + (size_t) g_cus * 512)));
+	double h[8];
+	for(int i = 0; i < 8; i++) h[i] = (double) rand() / RAND_MAX - 0.5 + 1e-7 * i;
+	CK(hipMemcpy(out, h, 64, hipMemcpyHostToDevice));
+	const int iters = 4000;
+	const double kc = 1e-3 * g_hz / 1e3; // ms -> thousands of cycles
+	const float m4 = mix_ms<1, 0>(out, iters), m16 = mix_ms<2, 0>(out, iters), f = mix_ms<0, 3>(out, iters), u = mix_ms<0, 4>(out, iters);
+	printf("one wave per SIMD alone (k cycles): 4x4x4 %.0f, 16x16x4 %.0f, v_fma_f64 %.0f, integer %.0f\n", m4 * kc, m16 * kc, f * kc, u * kc);
+	printf("4x4x4 with v_fma_f64 on the SIMD's other wave: %.0f (sum %.0f, longer %.0f); with integer: %.0f (sum %.0f, longer %.0f)\n",
+		mix_ms<1, 3>(out, iters) * kc, (m4 + f) * kc, std::max(m4, f) * kc, mix_ms<1, 4>(out, iters) * kc, (m4 + u) * kc, std::max(m4, u) * kc);
+	printf("16x16x4 with v_fma_f64 on the SIMD's other wave: %.0f (sum %.0f, longer %.0f); with integer: %.0f (sum %.0f, longer %.0f)\n",
+		mix_ms<2, 3>(out, iters) * kc, (m16 + f) * kc, std::max(m16, f) * kc, mix_ms<2, 4>(out, iters) * kc, (m16 + u) * kc, std::max(m16, u) * kc);
+	{
+		const float both4 = mix_ms<1, 1>(out, iters), both16 = mix_ms<2, 2>(out, iters);
+		// per SIMD: two waves x 8 x iters instructions of the 4 x 4 x 4 form, two waves x 8 x iters / 4 of the 16 x 16 x 4 form
+		printf("sums in vector registers, two waves per SIMD: 4x4x4 %.1f TFLOP/s, %.1f cycles per instruction; 16x16x4 %.1f TFLOP/s, %.1f cycles per instruction\n",
+			16.0 * iters * g_cus * 4 * 512 / both4 / 1e9, both4 * 1e-3 * g_hz / (16.0 * iters), 4.0 * iters * g_cus * 4 * 2048 / both16 / 1e9,
+			both16 * 1e-3 * g_hz / (4.0 * iters));
+	}
+	printf("matrix instructions on both waves of a SIMD: 4x4x4 %.0f (twice alone %.0f), 16x16x4 %.0f (twice alone %.0f)\n", mix_ms<1, 1>(out, iters) * kc, 2 * m4 * kc,
+		mix_ms<2, 2>(out, iters) * kc, 2 * m16 * kc);
+	printf("v_fma_f64 with integer on the SIMD's other wave: %.0f (sum %.0f, longer %.0f)\n", mix_ms<3, 4>(out, iters) * kc, (f + u) * kc, std::max(f, u) * kc);
+	CK(hipFree(out));
+}
+
 static void probe_mfma() {
 	const int bpc = 2, blocks = g_cus * bpc; // 2 blocks of 4 waves per CU = 2 waves per SIMD
 	double* out;
@@ -122,9 +208,16 @@ static void probe_mfma() {
 	}
 	{
 		const int iters = 1000;
+		const float ms = time_ms([&] { hipLaunchKernelGGL(k_mfma16<8>, dim3(blocks), dim3(256), 0, 0, out, iters); }, 2);
+		const double n = 8.0 * iters * blocks * 4;
+		printf("v_mfma_f64_16x16x4_f64 (2048 flop),  8 sums in accumulation registers (a[..] as C and D: the compiler's choice for this loop): %6.1f TFLOP/s, %5.1f cycles per instruction and SIMD\n", n * 2048 / ms / 1e9,
+			ms * 1e-3 * g_hz / (8.0 * iters * bpc));
+	}
+	{
+		const int iters = 1000;
 		const float ms = time_ms([&] { hipLaunchKernelGGL(k_mfma16<16>, dim3(blocks), dim3(256), 0, 0, out, iters); }, 2);
 		const double n = 16.0 * iters * blocks * 4;
-		printf("v_mfma_f64_16x16x4_f64 (2048 flop): %6.1f TFLOP/s, %5.1f cycles per instruction and SIMD\n", n * 2048 / ms / 1e9,
+		printf("v_mfma_f64_16x16x4_f64 (2048 flop), 16 sums in accumulation registers: %6.1f TFLOP/s, %5.1f cycles per instruction and SIMD\n", n * 2048 / ms / 1e9,
 			ms * 1e-3 * g_hz / (16.0 * iters * bpc));
 	}
 	CK(hipFree(out));
@@ -303,6 +396,7 @@ int main() {
 	CK(hipMalloc(&sink, 64));
 	const int bad = probe_layout();
 	probe_mfma();
+	probe_mix();
 	probe_stream(sink);
 	probe_l2_and_stores(sink);
 	probe_lds();

@@ -21,3 +21,4 @@ def test_probe_runs_and_the_matrix_instruction_layout_is_the_assumed_one():
     assert "layout of v_mfma_f64_4x4x4_f64: as assumed" in r.stdout
     rates = [float(x) for x in re.findall(r"([0-9.]+) TB/s", r.stdout)]
     assert len(rates) >= 10 and all(x > 0.1 for x in rates)
+    assert "sums in vector registers, two waves per SIMD" in r.stdout and "on the SIMD's other wave" in r.stdout
