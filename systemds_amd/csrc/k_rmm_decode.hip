@@ -421,20 +421,21 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 
 		if(GRAM) {
 			// wave: 128 rows of the tile; lane (k4, i16): rows k4 * 32 .. + 31, column 16 cb + i16
+			const int rowsLeft = (int) min((int64_t) DEC_TILE, nRows - t0); // rows of the tile inside the matrix
 #pragma unroll 1
 			for(int half = 0; half < 2; half++) {
 				const int rbase = wave * DEC_WROWS + k4 * 32 + half * 16;
 				double cst[NB];
 				u32x4 cq[NB][2];
 				int lbase[NB], lnC[NB], lsent[NB];
-				bool lcoded[NB], ldense[NB], ltwo[NB];
+				bool lcoded[NB], ltwo[NB];
 				const double* lptr[FLAT ? NB : 1];
 #pragma unroll
 				for(int cb = 0; cb < NB; cb++) {
 					// (narrow block with packed lookups: every lane of the last block works on one of its first four columns)
 					const int ci = cb * 16 + (NAR && NB <= 2 && cb == NB - 1 ? i16 & 3 : i16);
 					const DecLook L(colS[ci]);
-					lbase[cb] = L.base; lnC[cb] = L.nC; lsent[cb] = L.sent; lcoded[cb] = L.coded; ldense[cb] = L.dense; ltwo[cb] = L.two;
+					lbase[cb] = L.base; lnC[cb] = L.nC; lsent[cb] = L.sent; lcoded[cb] = L.coded; ltwo[cb] = L.two;
 					if(FLAT) {
 						const DecCol D = colS[ci];
 						const double* gdict = groupS[D.pad].dict + ((unsigned) D.meta >> 18);
@@ -464,14 +465,15 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 							const int c2 = (int) ((cq[cb][s >> 3][(s >> 1) & 3] >> (16 * (s & 1))) & 0xffff);
 							const int c = ltwo[cb] ? c2 : c1;
 							// rows behind the end of the matrix hold stale codes: never used as an index
-							const bool valid = (t0 + rbase + s < nRows) & (ldense[cb] | (lcoded[cb] & (c != lsent[cb])));
+							// (a column without row data reads a zero that stays zero: no test for it)
+							const bool valid = (rbase + s < rowsLeft) & (c != lsent[cb]);
 							double v;
 							if(FLAT) {
-								const double* vp = lptr[cb] + (lcoded[cb] ? c : rbase + s) * lnC[cb];
+								const double* vp = lptr[cb] + __umul24(lcoded[cb] ? c : rbase + s, lnC[cb]);
 								v = *(valid ? vp : (const double*) smem);
 							}
 							else {
-								const int ad = lbase[cb] + (lcoded[cb] ? c : rbase + s) * lnC[cb];
+								const int ad = lbase[cb] + __umul24(lcoded[cb] ? c : rbase + s, lnC[cb]);
 								v = smem[valid ? ad : 0];
 							}
 							x[u][cb] = valid ? v : 0.0;
@@ -486,15 +488,15 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 						const uint32_t lo = cq[cb][sHi >> 1][(2 * sHi) & 3], hi = cq[cb][sHi >> 1][(2 * sHi + 1) & 3]; // codes 4 sHi .. + 3 as 16-bit pieces
 						const int c2 = (int) (((j & 2 ? hi : lo) >> (16 * (j & 1))) & 0xffff);
 						const int c = ltwo[cb] ? c2 : c1;
-						const bool in = t0 + rbase + s < nRows;
-						const bool valid = in & (ldense[cb] | (lcoded[cb] & (c != lsent[cb])));
+						const bool in = rbase + s < rowsLeft;
+						const bool valid = in & (c != lsent[cb]);
 						double v;
 						if(FLAT) {
-							const double* vp = lptr[cb] + (lcoded[cb] ? c : rbase + s) * lnC[cb];
+							const double* vp = lptr[cb] + __umul24(lcoded[cb] ? c : rbase + s, lnC[cb]);
 							v = *(valid ? vp : (const double*) smem);
 						}
 						else {
-							const int ad = lbase[cb] + (lcoded[cb] ? c : rbase + s) * lnC[cb];
+							const int ad = lbase[cb] + __umul24(lcoded[cb] ? c : rbase + s, lnC[cb]);
 							v = smem[valid ? ad : 0];
 						}
 						v = valid ? v : 0.0;
@@ -502,7 +504,7 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 					}
 #pragma unroll
 					for(int u = 0; u < SB; u++) {
-						const bool in = t0 + rbase + sb + u < nRows;
+						const bool in = rbase + sb + u < rowsLeft;
 #pragma unroll
 						for(int cb = 0; cb < NL; cb++) x[u][cb] = in ? cst[cb] + x[u][cb] : 0.0;
 						int t = 0;
@@ -733,8 +735,9 @@ static int dec_build_plan(cla_block* b, bool gram, int q, int rpl, DecLaunch& L,
 		P.slotOff = (int32_t) slotB;
 		slotB += (size_t) DEC_TILE * P.slotW + DEC_SLOT_PAD;
 	}
-	if(valD == 0) valD = 2;
 	valD = (valD + 1) & ~(size_t) 1;
+	const size_t zeroAt = valD; // a value that stays zero: what a column without row data looks up
+	valD += 2;
 	slotB = (slotB + 16 + 15) & ~(size_t) 15; // the multiply phase may read 16 bytes past the last tile
 	const int nColD = gram ? ((nCols + 15) / 16) * 16 : ((K + 3) / 4) * 4;
 	const size_t bD = gram ? 0 : (size_t) nColD * 16;
@@ -802,7 +805,7 @@ static int dec_build_plan(cla_block* b, bool gram, int q, int rpl, DecLaunch& L,
 	L.lds = ldsEnd + 64;
 	if(L.lds > (size_t) std::min(g_ldsPerBlock, 160 * 1024) - 1024) return 1;
 	// column descriptors: decoded column order (X %*% B) or matrix column order (t(X) %*% X)
-	std::vector<DecCol> cols((size_t) nColD, DecCol{0, 0, 0, 0});
+	std::vector<DecCol> cols((size_t) nColD, DecCol{0, (int32_t) zeroAt, 0, 0});
 	std::vector<double> colConst((size_t) (gram ? nColD : 0), 0.0);
 	if(gram)
 		for(int c = 0; c < nCols; c++) colConst[c] = b->constV[c];
@@ -816,7 +819,7 @@ static int dec_build_plan(cla_block* b, bool gram, int q, int rpl, DecLaunch& L,
 			DecCol& C = cols[gram ? hc[h] : P.kOff + h];
 			const int kind = P.type == G_UNC ? 2 : P.slotOff >= 0 ? (P.type == G_DDC ? 3 : 1) : 0;
 			C.slotOff = kind == 1 || kind == 3 ? P.slotOff : 0;
-			C.valOff = kind && P.dictOff >= 0 ? P.dictOff : 0;
+			C.valOff = kind && P.dictOff >= 0 ? P.dictOff : kind ? 0 : (int32_t) zeroAt;
 			C.pad = g;
 			C.meta = (int32_t) ((uint32_t) kind | (P.slotW == 2 ? 4u : 0u) | ((kind == 1 || kind == 3) && P.dictOff < 0 ? 8u : 0u) | ((uint32_t) P.nC << 4) | ((uint32_t) h << 18));
 		}
