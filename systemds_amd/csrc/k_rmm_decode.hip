@@ -821,7 +821,8 @@ static int dec_build_plan(cla_block* b, bool gram, int q, int rpl, DecLaunch& L,
 			C.slotOff = kind == 1 || kind == 3 ? P.slotOff : 0;
 			C.valOff = kind && P.dictOff >= 0 ? P.dictOff : kind ? 0 : (int32_t) zeroAt;
 			C.pad = g;
-			C.meta = (int32_t) ((uint32_t) kind | (P.slotW == 2 ? 4u : 0u) | ((kind == 1 || kind == 3) && P.dictOff < 0 ? 8u : 0u) | ((uint32_t) P.nC << 4) | ((uint32_t) h << 18));
+			// (a column without row data looks the zero up whatever the row: no stride, no place in a tuple)
+			C.meta = kind == 0 ? 0 : (int32_t) ((uint32_t) kind | (P.slotW == 2 ? 4u : 0u) | ((kind == 1 || kind == 3) && P.dictOff < 0 ? 8u : 0u) | ((uint32_t) P.nC << 4) | ((uint32_t) h << 18));
 		}
 	}
 	const size_t planBytes = plan.size() * sizeof(DecGroup), copyBytes = copies.size() * sizeof(DecCopy);
