@@ -217,7 +217,8 @@ int64_t cla_decompress_dev(cla_handle h, double* dOut);
  * cells of the result. What has no such form is aggregated over decompressed chunks of rows (at most
  * 256 MiB of scratch), as CLALibCompAgg.decompressingAggregate does (C/lib/CLALibCompAgg.java:220-232,
  * 419-452, 605-720): everything but plain sums on overlapping groups, row minima / maxima, row sums of
- * squares next to an uncompressed group. */
+ * squares next to an uncompressed group or over an SDC group with a non-zero default (its tuples are held
+ * relative to the default, so their squares would come from a cancelling difference). */
 enum cla_agg_op { CLA_AGG_SUM = 0, CLA_AGG_SUMSQ = 1, CLA_AGG_MIN = 2, CLA_AGG_MAX = 3 };
 enum cla_agg_dir { CLA_AGG_ALL = 0, CLA_AGG_ROW = 1, CLA_AGG_COL = 2 };
 int64_t cla_aggregate(cla_handle h, int32_t op, int32_t dir, double* out);

@@ -276,7 +276,14 @@ int launch_aggregate(cla_block* b, int op, int dir, double* dOut, unsigned long 
 		}
 	}
 	if(nRows > 0 && nCols > 0) {
-		const bool rowNoTable = dir == CLA_AGG_ROW && (op == CLA_AGG_MIN || op == CLA_AGG_MAX || (op == CLA_AGG_SUMSQ && b->hasUnc));
+		// (row sums of squares from tables: a tuple's table entry is (d + c)^2 - c^2 under the constant row's c^2, which
+		// cancels where an offset list's default c is large against the values; such blocks are decompressed instead)
+		bool listOverDefault = false;
+		if(op == CLA_AGG_SUMSQ && dir == CLA_AGG_ROW)
+			for(auto& g : b->groups)
+				if(g.d.type == G_SDCZ && g.d.nOffsets > 0)
+					for(int c : g.cols) listOverDefault |= b->constV[c] != 0.0;
+		const bool rowNoTable = dir == CLA_AGG_ROW && (op == CLA_AGG_MIN || op == CLA_AGG_MAX || (op == CLA_AGG_SUMSQ && (b->hasUnc || listOverDefault)));
 		if((overlap && op != CLA_AGG_SUM) || rowNoTable) return launch_aggregate_decompressed(b, op, dir, dOut, dNnz);
 	}
 	if(dir == CLA_AGG_ROW) {

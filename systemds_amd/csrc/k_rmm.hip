@@ -663,7 +663,8 @@ int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned lon
 		}
 		vecDecode = nOther > 0 && nLists <= nOther;
 	}
-	if(((q >= 2 && q <= 16) || vecDecode) && !noAlloc && !(b->opt.rmmDisable & 8)) {
+	// (not for the row sums of squares: the decode kernels multiply decoded values, the squares live in the tables)
+	if(((q >= 2 && q <= 16) || vecDecode) && !squares && !noAlloc && !(b->opt.rmmDisable & 8)) {
 		const int r = launch_rmm_decode(b, dB, q, constRow >= 0 ? tables + (size_t) constRow * q : nullptr, dOut, dNnz);
 		if(r <= 0) return r;
 	}

@@ -129,3 +129,25 @@ def test_sum_of_squares_of_a_dense_column_under_a_constant(cla, ora, direction):
     D = ora.np_decompress(specs, n_rows, 4)
     check(cla, specs, D, n_rows, 4, "sumsq", direction, "dense + const")
     check(cla, specs, D, n_rows, 4, "sum", direction, "dense + const")
+
+
+@pytest.mark.parametrize("n_rows", [1023, 2049, 70001])
+def test_row_sums_of_squares_on_a_block_with_few_offset_lists(cla, ora, n_rows):
+    """One SDC group next to DDC, RLE and constant groups, no uncompressed group: the single-column right multiply of
+    such a block decodes rows (value x 1), which the row sums of squares must not take (their squares sit in the
+    per-tuple tables)."""
+    from systemds_amd import synth
+    rng = np.random.default_rng(n_rows)
+    specs = [synth.sdc_group(rng, n_rows, np.array([0], np.int32), 17, 0.3, None),
+             synth.GroupSpec("ddc", np.array([1, 2], np.int32), rng.standard_normal((300, 2)), rng.integers(0, 300, n_rows).astype(np.uint16)),
+             synth.GroupSpec("const", np.array([3], np.int32), np.array([[-0.75]]))]
+    run_codes = rng.integers(-1, 4, size=n_rows // 20 + 2)
+    codes = np.repeat(run_codes, rng.integers(1, 60, size=run_codes.size))[:n_rows]
+    if codes.size < n_rows:
+        codes = np.concatenate([codes, np.full(n_rows - codes.size, -1)])
+    ptr, data = synth.encode_rle(codes, 4)
+    specs.append(synth.GroupSpec("rle", np.array([4], np.int32), rng.standard_normal((4, 1)), ptr=ptr, rle=data))
+    D = ora.np_decompress(specs, n_rows, 5)
+    for op in OPS:
+        for direction in DIRS:
+            check(cla, specs, D, n_rows, 5, op, direction, "few lists")
