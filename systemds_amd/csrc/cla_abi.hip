@@ -286,8 +286,6 @@ void cla_block_free(cla_handle b) {
 	if(b->refs.fetch_sub(1) > 1) return; // blocks made from this one still use its streams
 	cla_block* parent = b->parent;
 	if(b->joint) { cla_block_free(b->joint); b->joint = nullptr; }
-	if(b->yJoint) { cla_block_free(b->yJoint); b->yJoint = nullptr; }
-	if(b->yBlock) { cla_block_free(b->yBlock); b->yBlock = nullptr; }
 	free_subs(b);
 	if(g_device >= 0) (void) hipSetDevice(g_device);
 	if(b->stream) (void) hipStreamSynchronize(b->stream);
@@ -731,8 +729,6 @@ int64_t cla_block_derived_bytes(cla_handle b) {
 	std::lock_guard<std::recursive_mutex> lk(b->mu);
 	int64_t s = b->derivedBytes;
 	if(b->joint) s += b->joint->derivedBytes;
-	if(b->yJoint) s += b->yJoint->derivedBytes;
-	if(b->yBlock) s += b->yBlock->derivedBytes + (int64_t) sizeof(double) * b->yBlock->nRows * b->yBlock->nCols;
 	for(void* p : b->subs) s += ((SubBlock*) p)->blk ? ((SubBlock*) p)->blk->derivedBytes : 0;
 	return s;
 }
@@ -1177,33 +1173,13 @@ int launch_tsmm_chunked(cla_block* b, double* dOut) {
 	return 0;
 }
 
-// dst[r * p + i] = Y[i * nRows + r] for 256 rows per block through LDS (coalesced reads of every row of Y, one
-// contiguous write of 256 x p values); *bad != 0 afterwards when Y holds a non-finite value
-__global__ __launch_bounds__(256) void k_transpose_y(const double* __restrict__ Y, int64_t nRows, int p, double* __restrict__ dst,
-	unsigned long long* __restrict__ bad) {
-	__shared__ double tile[256 * 17]; // row stride p + 1 when p is even: the column reads of the write phase spread over the banks
-	const int64_t r0 = (int64_t) blockIdx.x * 256;
-	const int nr = (int) min((int64_t) 256, nRows - r0), ps = p | 1;
-	int nf = 0;
-	if((int) threadIdx.x < nr)
-		for(int i = 0; i < p; i++) {
-			const double v = Y[(size_t) i * nRows + r0 + threadIdx.x];
-			nf |= !isfinite(v);
-			tile[threadIdx.x * ps + i] = v;
-		}
-	if(__builtin_amdgcn_ballot_w64(nf != 0) != 0 && (threadIdx.x & 63) == 0) atomicOr(bad, 1ull);
-	__syncthreads();
-	for(int k = threadIdx.x; k < nr * p; k += 256) dst[(size_t) r0 * p + k] = tile[(k / p) * ps + k % p];
-}
-
 // Y %*% X as the (left, right) part of the decoded Gram matrix of cbind(t(Y), X): one pass over X's row data on the
 // matrix cores whatever its group mix and however many rows Y has (2 to 16), where the bin kernels take a pass per
 // row of Y and group type (C5, 50 M x 20: 2.9 / 3.7 / 4.7 ms against 5.1 / 8.9 / 18 ms for 2 / 4 / 8 rows of Y). Taken for
 // blocks of at most 48 columns that neither the byte-code dot form nor the offset-list kernels serve. Returns 1 when
 // the block is not eligible, 0 when dOut (p x nCols) holds the result and *dNnz its non-zero count.
 int launch_lmm_joint(cla_block* b, const double* dY, int p, double* dOut, unsigned long long* dNnz) {
-	// (one row of Y: the bin kernels take as long and need neither the copy of Y nor a look at it)
-	if(!b->opt.lmmJoint || !b->opt.tsmmMfma || p < 2 || p > 16 || b->nCols > 48 || b->nRows == 0 || b->crossSplit > 0) return 1;
+	if(!b->opt.lmmJoint || !b->opt.tsmmMfma || p < 1 || p > 16 || b->nCols > 64 || b->nRows == 0 || b->crossSplit > 0) return 1;
 	if(b->dictNonFinite) return 1; // (the reference sums Y per tuple first: an infinite dictionary value times Y of both signs is no NaN)
 	int nLists = 0, nOther = 0;
 	bool dotForm = b->dArena != nullptr && b->arenaWidth == 1 && b->maxVals <= 256;
@@ -1214,80 +1190,34 @@ int launch_lmm_joint(cla_block* b, const double* dY, int p, double* dOut, unsign
 		if(g.d.nColG != 1) dotForm = false;
 		if(g.d.type == G_UNC || g.d.nVals > 0)
 			for(int c : g.cols) {
-				if(seen[c]) return 1; // overlapping groups: the decoded Gram kernel wants one group per column
+				if(seen[c]) return 1; // overlapping groups: the decode kernel wants one group per column
 				seen[c] = 1;
 			}
 	}
 	if(nOther == 0 || nLists > nOther || dotForm) return 1;
 	hipStream_t st = b->stream;
-	if(b->yBlock == nullptr || b->yRows != p) {
-		if(b->yJoint) { cla_block_free(b->yJoint); b->yJoint = nullptr; }
-		if(b->yBlock) { cla_block_free(b->yBlock); b->yBlock = nullptr; }
-		cla_block* y = cla_block_create(b->nRows, p);
-		if(!y) return -CLA_ERR_DEVICE;
-		std::vector<int32_t> cols((size_t) p);
-		for(int i = 0; i < p; i++) cols[i] = i;
-		HostGroup g;
-		int rc = init_group(y, g, G_UNC, cols.data(), p, nullptr, 0);
-		void* d = nullptr;
-		const size_t bytes = sizeof(double) * (size_t) b->nRows * p;
-		if(!rc && hipMalloc(&d, bytes + UPLOAD_SLACK) != hipSuccess) { set_error("left multiply: %zu bytes for t(Y) could not be allocated", bytes); rc = -CLA_ERR_DEVICE; }
-		if(rc) { free_group(g); cla_block_free(y); return rc; }
-		g.owned.push_back(d);
-		(void) hipMemset(d, 0, bytes + UPLOAD_SLACK);
-		g.d.dense = (const double*) d;
-		y->groups.push_back(std::move(g));
-		if((rc = cla_block_finalize(y))) { cla_block_free(y); return rc; }
-		b->yBlock = y;
-		b->yRows = p;
-	}
-	if(b->yJoint == nullptr) {
-		b->yJoint = make_joint(b->yBlock, b);
-		if(!b->yJoint) return -CLA_ERR_DEVICE;
-	}
-	cla_block* c = b->yJoint;
-	if(c->crossBlocks == 0) return 1; // (not padded: more than 64 joint columns)
-	c->opt = b->opt;
-	{
-		const int fits = tsmm_decode_fits(c); // (t(Y)'s tile takes 8 KB of LDS per row of Y)
-		if(fits) return fits;
-	}
-	c->profile = b->profile;
-	c->opt = b->opt;
-	if(c->stream != st) {
-		if(c->ownStream && c->stream) { (void) hipStreamSynchronize(c->stream); (void) hipStreamDestroy(c->stream); }
-		c->stream = st;
-		c->ownStream = false;
-	}
+	const size_t n = (size_t) p * b->nCols;
+	int rc = ensure_stage(&b->dStageOut, &b->stageOutCap, n);
+	if(rc) return rc;
+	CLA_HIP(hipMemsetAsync(b->dStageOut, 0, n * sizeof(double), st));
+	CLA_HIP(hipMemsetAsync(dNnz, 0, sizeof(unsigned long long), st));
+	if((rc = launch_lmm_decode(b, dY, p, b->dStageOut, dNnz))) return rc;
 	{
 		// A row that a group does not cover (outside its runs or its offset list) does not enter that group's sums in
-		// the reference, whatever Y holds there; as a decoded 0.0 it would turn an infinite Y into NaN. Y with a
-		// non-finite value therefore takes the bin kernels (the host has to look: one wait for the stream).
-		CLA_HIP(hipMemsetAsync(dNnz, 0, sizeof(unsigned long long), st));
-		{
-			Prof pf(b, "k_transpose_y", (long) ((b->nRows + 255) / 256), 256, 0, (double) b->nRows * p * 16);
-			hipLaunchKernelGGL(k_transpose_y, dim3((unsigned) ((b->nRows + 255) / 256)), dim3(256), 0, st, dY, b->nRows, p,
-				const_cast<double*>(b->yBlock->groups[0].d.dense), dNnz);
-		}
+		// the reference, whatever Y holds there; as a decoded 0.0 it turns an infinite Y into NaN. The kernel reports a
+		// non-finite value of Y, and such a Y takes the bin kernels (the host has to look: one wait for the stream).
 		unsigned long long bad = 0;
 		CLA_HIP(hipMemcpyAsync(&bad, dNnz, sizeof(bad), hipMemcpyDeviceToHost, st));
 		CLA_HIP(hipStreamSynchronize(st));
-		if(bad) return 1;
+		if(bad) { clear_stats(b); return 1; }
 	}
-	const size_t n = (size_t) c->nCols;
-	int rc = ensure_stage(&c->dStageOut, &c->stageOutCap, n * n);
-	if(rc) return rc;
-	if((rc = launch_tsmm(c, c->dStageOut, c->dCounters))) return rc;
 	CLA_HIP(hipMemsetAsync(dNnz, 0, sizeof(unsigned long long), st));
-	const int nOut = p * b->nCols;
 	{
-		Prof pf(c, "k_take_block", (nOut + 255) / 256, 256, 0, 0);
-		hipLaunchKernelGGL(k_take_block, dim3((unsigned) std::min((nOut + 255) / 256, 1024)), dim3(256), 0, st, c->dStageOut, (int) n, 0,
-			c->nCols - b->nCols, p, b->nCols, dOut, dNnz);
+		Prof pf(b, "k_take_block", ((int) n + 255) / 256, 256, 0, 0);
+		hipLaunchKernelGGL(k_take_block, dim3((unsigned) std::min(((int) n + 255) / 256, 1024)), dim3(256), 0, st, b->dStageOut, b->nCols, 0, 0, p,
+			b->nCols, dOut, dNnz);
 	}
 	CLA_HIP(hipGetLastError());
-	b->lastStats.insert(b->lastStats.end(), c->lastStats.begin(), c->lastStats.end());
-	c->lastStats.clear(); // (the events moved along)
 	return 0;
 }
 

@@ -75,7 +75,7 @@ struct Options {
 	int rmmDirect = 1;      // X %*% B for narrow B on blocks of plain streams: codes straight from global memory, sums on the vector unit (0: the tile kernel on the matrix cores)
 	int rmmDisable = 0;     // bit 0 byte-code mat-vec, 1 fused tables of the byte-code mat-vec, 2 matrix-core kernel, 3 decode kernel
 	int lmmDisable = 0;     // bit 0 dot form on byte codes, 1 byte-code bin kernel
-	int lmmJoint = 1;       // left multiply of blocks that are not mostly offset lists or byte-code DDC groups as cbind(t(Y), X) on the decoded Gram kernel
+	int lmmJoint = 1;       // left multiply of blocks that are not mostly offset lists or byte-code DDC groups in one pass over the decoded rows on the matrix cores (k_lmm_decode)
 	int sdcPacked = 1;      // packed SDCZeros lists for the mat-vecs
 	int sdcLanes = 1;       // SDCZeros mat-vecs on lane-major lists, one lane per group
 	int sdcRows = 1;        // SDCZeros right mat-vec on row lists, one lane per row
@@ -110,11 +110,6 @@ struct cla_block {
 	uint64_t serial = 0;
 	cla_block* joint = nullptr;
 	uint64_t jointSerial = 0;
-	// left multiply through the decoded Gram kernel: Y transposed into a one-group dense block of yRows columns and
-	// cbind(that, this), both kept until another number of rows of Y comes or the block is freed
-	cla_block* yBlock = nullptr;
-	cla_block* yJoint = nullptr;
-	int yRows = 0;
 	int32_t crossSplit = 0;          // > 0: joint block, groups [0, crossSplit) are the left side's
 	int32_t crossBlocks = 0;         // > 0: the left side's columns fill the first crossBlocks blocks of 16 columns (padded) and only left x right is read
 	int32_t crossCol = 0;            // joint block: first column of the right side
@@ -252,6 +247,7 @@ int launch_decompress(cla_block* b, double* dOut, unsigned long long* dNnz);
 int launch_decompress_rows(cla_block* b, int64_t r0, int64_t r1, double* dOut);
 void dec_plans_drop(cla_block* b);
 int tsmm_decode_fits(cla_block* b);
+int launch_lmm_decode(cla_block* b, const double* dY, int p, double* dOut, unsigned long long* dBad);
 int launch_lmm_joint(cla_block* b, const double* dY, int p, double* dOut, unsigned long long* dNnz);
 int launch_lmm(cla_block* b, const double* dY, int p, double* dOut, unsigned long long* dNnz);
 int launch_preagg(cla_block* b, int group, const double* dY, int p, double* dPre);

@@ -76,6 +76,9 @@ struct DecArgs {
 	const double* B;
 	int q;
 	const double* constRow;
+	const double* Y;                   // left multiply: Y (P x nRows, row-major); out is P x nCols
+	int P;
+	unsigned long long* badY;          // left multiply: set when Y holds a value that is not finite
 	double* out;
 	int64_t nRows;
 	unsigned long long* nnz;
@@ -171,7 +174,10 @@ __device__ __forceinline__ int dec_spread_bank(int o, int u) {
 	return a;
 }
 
-template <int GRAM, int NB, int RPL, int FLAT, int XB = 0, int NAR = 0>
+// LM (with GRAM): Y %*% X instead of t(X) %*% X. The decoded rows are the B operand as before, the A operand is Y
+// (lane l: row l % 16 of Y at matrix row ... + l / 16), read straight from global memory, 16 consecutive values per lane
+// and half; one 16 x 16 tile per column block.
+template <int GRAM, int NB, int RPL, int FLAT, int XB = 0, int NAR = 0, int LM = 0>
 __device__ __forceinline__ void decode_body(const DecArgs& A) {
 	extern __shared__ __align__(16) double smem[];
 	double* Bs = smem + A.valDoubles;                              // bDoubles: rows of B in decoded column order, 16 outputs each
@@ -284,8 +290,10 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 	// products are the last block's 4 columns against the 4 quarters of a 16-column block), which issues at four
 	// times the rate of a 16 x 16 tile and replaces NB of them.
 	static_assert(!NAR || (GRAM && XB == 0 && NB >= 2), "narrow last block: full Gram matrices only");
+	static_assert(!LM || (GRAM && XB == 0 && NAR == 0), "left multiply: one tile per column block");
 	constexpr int NF = NAR ? NB - 1 : NB; // column blocks among which 16 x 16 tiles are computed
-	constexpr int NTILES = !GRAM ? 1 : XB > 0 ? XB * (NB - XB) : NF * (NF + 1) / 2;
+	constexpr int NTILES = !GRAM ? 1 : LM ? NB : XB > 0 ? XB * (NB - XB) : NF * (NF + 1) / 2;
+	bool badY = false;
 	f64x4 gram[NTILES];
 	double nar[NAR ? NB : 1]; // lane l: cell (row 16 (NB - 1) + l / 16, column 16 cb + l % 16)
 	if(GRAM) {
@@ -446,6 +454,38 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 					cq[cb][0] = cp[0];
 					cq[cb][1] = cp[1];
 				}
+				double yv[LM ? 16 : 1];
+				if(LM) {
+					// row i16 of Y at the lane's 16 matrix rows of this half (rows of Y beyond P and rows behind the end: zeros)
+					const double* __restrict__ yp = as_global(A.Y) + (size_t) i16 * nRows + t0 + rbase;
+#pragma unroll
+					for(int s = 0; s < 16; s++) yv[s] = 0.0;
+					if(rowsLeft == DEC_TILE) { // (uniform) all 16 rows exist: 16 bytes per load, around an odd first value where the row of Y starts on one
+						if(i16 < A.P) {
+							if(((uintptr_t) yp & 15) == 0) {
+#pragma unroll
+								for(int j = 0; j < 8; j++) {
+									const f64x2 v = *(const f64x2*) (yp + 2 * j);
+									yv[2 * j] = v[0]; yv[2 * j + 1] = v[1];
+								}
+							}
+							else {
+								yv[0] = yp[0];
+#pragma unroll
+								for(int j = 0; j < 7; j++) {
+									const f64x2 v = *(const f64x2*) (yp + 1 + 2 * j);
+									yv[1 + 2 * j] = v[0]; yv[2 + 2 * j] = v[1];
+								}
+								yv[15] = yp[15];
+							}
+						}
+					}
+					else {
+#pragma unroll
+						for(int s = 0; s < 16; s++)
+							if(i16 < A.P && rbase + s < rowsLeft) yv[s] = yp[s];
+					}
+				}
 				// SB steps of lookups in flight, then their products
 				constexpr int SB = NB <= 2 ? 4 : 2;
 				// the narrow block's lookups packed four steps to one (below) pay with few column blocks; with many, the value
@@ -508,6 +548,13 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 #pragma unroll
 						for(int cb = 0; cb < NL; cb++) x[u][cb] = in ? cst[cb] + x[u][cb] : 0.0;
 						int t = 0;
+						if(LM) {
+							const double y = yv[sb + u];
+							badY |= !(__builtin_fabs(y) <= 1.7976931348623157e308);
+#pragma unroll
+							for(int cb = 0; cb < NB; cb++) gram[cb] = __builtin_amdgcn_mfma_f64_16x16x4f64(y, x[u][cb], gram[cb], 0, 0, 0);
+						}
+						else
 #pragma unroll
 						for(int ib = 0; ib < (XB > 0 ? XB : NF); ib++)
 #pragma unroll
@@ -598,6 +645,25 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 			}
 		}
 	}
+	if(GRAM && LM) {
+		// tiles of the block's waves summed in LDS (16 rows of Y x NB * 16 columns), then one global add per cell:
+		// accumulator register v of lane l is cell (row 4 v + l / 16 of Y, column 16 cb + l % 16)
+		constexpr int NP = NB * 16;
+		__syncthreads();
+		for(int i = tid; i < 16 * NP; i += DEC_THREADS) stage[i] = 0.0;
+		__syncthreads();
+#pragma unroll
+		for(int cb = 0; cb < NB; cb++)
+#pragma unroll
+			for(int v = 0; v < 4; v++) unsafeAtomicAdd(&stage[(4 * v + k4) * NP + cb * 16 + i16], gram[cb][v]);
+		__syncthreads();
+		for(int i = tid; i < 16 * NP; i += DEC_THREADS) {
+			const int r = i / NP, c = i - r * NP;
+			if(r < A.P && c < A.nCols && stage[i] != 0.0) unsafeAtomicAdd(&A.out[(size_t) r * A.nCols + c], stage[i]);
+		}
+		if(__ballot(badY) != 0 && lane == 0) atomicOr(A.badY, 1ull);
+		return;
+	}
 	if(GRAM) {
 		// Gram tiles of the block's waves summed in LDS, then one global add per cell of the
 		// upper triangle. Accumulator register v of lane l is cell (4 v + l / 16, l % 16) of its tile.
@@ -636,6 +702,9 @@ __global__ __launch_bounds__(DEC_THREADS) void k_rmm_decode(const DecArgs A) { d
 
 template <int NB, int FLAT, int XB, int NAR = 0>
 __global__ __launch_bounds__(DEC_THREADS) void k_tsmm_decode(const DecArgs A) { decode_body<1, NB, 4, FLAT, XB, NAR>(A); }
+
+template <int NB, int FLAT>
+__global__ __launch_bounds__(DEC_THREADS) void k_lmm_decode(const DecArgs A) { decode_body<1, NB, 4, FLAT, 0, 0, 1>(A); }
 
 // One code per row for an RLE group (0xff where no run covers the row): thread = 4 rows.
 __global__ __launch_bounds__(256) void k_expand_rle(const DGroup* __restrict__ groups, int g, int64_t nRows, uint8_t* __restrict__ codes) {
@@ -849,7 +918,7 @@ static int dec_build_plan(cla_block* b, bool gram, int q, int rpl, DecLaunch& L,
 	A.nTasks = (int) taskCost.size();
 	A.nGroups = nG; A.nCopies = (int) copies.size(); A.nChunks = nChunks; A.nColD = nColD;
 	A.valDoubles = (int) valD; A.bDoubles = (int) bD; A.stageDoubles = (int) stageD; A.slotBytes = (int) slotB;
-	A.B = nullptr; A.q = q; A.constRow = nullptr; A.out = nullptr; A.nRows = b->nRows; A.nnz = nullptr; A.nCols = nCols;
+	A.B = nullptr; A.q = q; A.constRow = nullptr; A.Y = nullptr; A.P = 0; A.badY = nullptr; A.out = nullptr; A.nRows = b->nRows; A.nnz = nullptr; A.nCols = nCols;
 	const int nTiles = (int) ((b->nRows + DEC_TILE - 1) / DEC_TILE);
 	const int blocksPerCU = L.lds <= 76 * 1024 ? 2 : 1;
 	L.grid = (unsigned) std::min(nTiles, g_numCU * blocksPerCU);
@@ -1266,6 +1335,31 @@ int launch_rmm_decode(cla_block* b, const double* dB, int q, const double* dCons
 		CLA_HIP(allow_full_lds((const void*) k_rmm_decode<2>));
 		hipLaunchKernelGGL(k_rmm_decode<2>, dim3(L.grid), dim3(DEC_THREADS), L.lds, b->stream, L.A);
 	}
+	CLA_HIP(hipGetLastError());
+	return 0;
+}
+
+// dOut (p x nCols, zeroed) += Y %*% D of the decoded rows, constants included; *dBad is set when Y holds a value that is
+// not finite (the result is then not the reference's: a row that a group does not cover stays out of that group's sums
+// there, here it is a decoded zero). Returns 1 when the block is not eligible (more than 64 columns, LDS plan too large).
+int launch_lmm_decode(cla_block* b, const double* dY, int p, double* dOut, unsigned long long* dBad) {
+	const int nCols = b->nCols;
+	if(b->groups.empty() || b->nRows == 0 || nCols > 64 || p < 1 || p > 16) return 1;
+	const int NB = (nCols + 15) / 16;
+	DecLaunch L;
+	bool flat = false;
+	int rc = gram_prepare(b, L, flat);
+	if(rc) return rc;
+	L.A.out = dOut; L.A.Y = dY; L.A.P = p; L.A.badY = dBad;
+	Prof pf(b, "k_lmm_decode", L.grid, DEC_THREADS, (long) L.lds, (double) b->device_bytes_cached + (double) b->nRows * p * 8);
+#define LM_LAUNCH(NBV, FL)                                                                                      \
+	do {                                                                                                        \
+		CLA_HIP(allow_full_lds((const void*) k_lmm_decode<NBV, FL>));                                           \
+		hipLaunchKernelGGL((k_lmm_decode<NBV, FL>), dim3(L.grid), dim3(DEC_THREADS), L.lds, b->stream, L.A); \
+	} while(0)
+	if(!flat) { if(NB == 1) LM_LAUNCH(1, 0); else if(NB == 2) LM_LAUNCH(2, 0); else if(NB == 3) LM_LAUNCH(3, 0); else LM_LAUNCH(4, 0); }
+	else { if(NB == 1) LM_LAUNCH(1, 1); else if(NB == 2) LM_LAUNCH(2, 1); else if(NB == 3) LM_LAUNCH(3, 1); else LM_LAUNCH(4, 1); }
+#undef LM_LAUNCH
 	CLA_HIP(hipGetLastError());
 	return 0;
 }

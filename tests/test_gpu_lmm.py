@@ -182,9 +182,9 @@ def test_byte_code_block_with_non_finite_dictionary_values(cla, ora):
 
 @pytest.mark.parametrize("p", [1, 2, 5, 8, 16])
 def test_mixed_block_takes_one_decoded_pass(cla, ora, p):
-    """C5's shape (RLE, two-byte DDC, offset lists with a default, dense columns): Y %*% X as the cross part of the
-    decoded Gram matrix of cbind(t(Y), X) for 2 or more rows of Y; with the option off the bin
-    kernels give the same cells."""
+    """C5's shape (RLE, two-byte DDC, offset lists with a default, dense columns): Y %*% X in one pass over the decoded
+    rows on the matrix cores, Y as the other operand (`k_lmm_decode`); with the option off the bin kernels give the
+    same cells."""
     from systemds_amd import synth
     c = synth.config5(scale=400)
     n_rows, n_cols = c["n_rows"], c["n_cols"]
@@ -201,10 +201,7 @@ def test_mixed_block_takes_one_decoded_pass(cla, ora, p):
         bins, nnz_b = blk.lmm(Y)
     finally:
         blk.close()
-    if 2 <= p <= 8:
-        assert "k_tsmm_decode" in names and "k_lmm_preagg_rows" not in names, names
-    else:  # one row of Y, or t(Y)'s tile (8 KB of LDS per row of Y) does not fit next to the block's dictionaries: the bin kernels
-        assert "k_tsmm_dense" not in names, names
+    assert "k_lmm_decode" in names and "k_lmm_preagg_rows" not in names, names
     assert_matches_truth(out, Y, D, what=f"Y %*% X, {p} rows")
     assert_matches_truth(bins, Y, D, what=f"Y %*% X, {p} rows, bin kernels")
     assert np.array_equal(out, out2) or np.allclose(out, out2, rtol=1e-12, atol=0)
