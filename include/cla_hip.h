@@ -118,7 +118,7 @@ int cla_block_set_stream(cla_handle h, void* hipStream);
  *   sdc_packed      1 / 0: packed SDCZeros lists for the mat-vecs
  *   sdc_lanes       1 / 0: SDCZeros mat-vecs on lane-major copies of the lists, one lane per group
  *   sdc_rows        1 / 0: SDCZeros X %*% v on row lists (the lists transposed), one lane per row
- *   lmm_joint       1 / 0: Y %*% X for at most 16 rows of Y on a block of at most 64 columns that is neither mostly offset lists nor
+ *   lmm_joint       1 / 0: Y %*% X (16 rows of Y per pass) on a block of at most 64 columns that is neither mostly offset lists nor
  *                   byte-code DDC groups in one pass over the decoded rows on the matrix cores (the kernel reports non-finite
  *                   values of Y and the host looks, i.e. waits for the stream once per call; such a Y takes the bin kernels)
  * Blocks derived from this one (overlapping results, joint blocks) inherit the values at the time of the call

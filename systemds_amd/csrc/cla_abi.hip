@@ -1179,7 +1179,7 @@ int launch_tsmm_chunked(cla_block* b, double* dOut) {
 // blocks of at most 48 columns that neither the byte-code dot form nor the offset-list kernels serve. Returns 1 when
 // the block is not eligible, 0 when dOut (p x nCols) holds the result and *dNnz its non-zero count.
 int launch_lmm_joint(cla_block* b, const double* dY, int p, double* dOut, unsigned long long* dNnz) {
-	if(!b->opt.lmmJoint || !b->opt.tsmmMfma || p < 1 || p > 16 || b->nCols > 64 || b->nRows == 0 || b->crossSplit > 0) return 1;
+	if(!b->opt.lmmJoint || !b->opt.tsmmMfma || p < 1 || b->nCols > 64 || b->nRows == 0 || b->crossSplit > 0) return 1;
 	if(b->dictNonFinite) return 1; // (the reference sums Y per tuple first: an infinite dictionary value times Y of both signs is no NaN)
 	int nLists = 0, nOther = 0;
 	bool dotForm = b->dArena != nullptr && b->arenaWidth == 1 && b->maxVals <= 256;
@@ -1201,7 +1201,11 @@ int launch_lmm_joint(cla_block* b, const double* dY, int p, double* dOut, unsign
 	if(rc) return rc;
 	CLA_HIP(hipMemsetAsync(b->dStageOut, 0, n * sizeof(double), st));
 	CLA_HIP(hipMemsetAsync(dNnz, 0, sizeof(unsigned long long), st));
-	if((rc = launch_lmm_decode(b, dY, p, b->dStageOut, dNnz))) return rc;
+	for(int p0 = 0; p0 < p; p0 += 16) // 16 rows of Y per pass over the block
+		if((rc = launch_lmm_decode(b, dY + (size_t) p0 * b->nRows, std::min(16, p - p0), b->dStageOut + (size_t) p0 * b->nCols, dNnz))) {
+			if(p0 > 0) clear_stats(b);
+			return rc;
+		}
 	{
 		// A row that a group does not cover (outside its runs or its offset list) does not enter that group's sums in
 		// the reference, whatever Y holds there; as a decoded 0.0 it turns an infinite Y into NaN. The kernel reports a
