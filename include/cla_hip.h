@@ -112,8 +112,8 @@ int cla_block_set_stream(cla_handle h, void* hipStream);
  *   tsmm_narrow     1 / 0: decoded Gram matrix with a last column block of at most 4 columns on the 4x4x4 matrix instruction
  *   expand_streams  1 / 0: one code per row for small RLE / SDCZeros groups (set before the first multiply)
  *   rmm_disable     bit 0 byte-code mat-vec kernel, 1 its fused tables, 2 matrix-core kernel, 3 decode kernel
- *   rmm_direct      1 / 0: X %*% B for at most 16 columns of B on blocks of plain streams with codes read straight from global memory
- *                   (0: the tile kernel on the matrix cores)
+ *   rmm_direct      1 / 0: X %*% B on blocks of plain streams with codes read straight from global memory, 16 columns of B per pass
+ *                   (0: at most 16 columns of B on the tile kernel on the matrix cores, wider B per row and group)
  *   lmm_disable     bit 0 dot form on byte codes, bit 1 byte-code bin kernel
  *   sdc_packed      1 / 0: packed SDCZeros lists for the mat-vecs
  *   sdc_lanes       1 / 0: SDCZeros mat-vecs on lane-major copies of the lists, one lane per group

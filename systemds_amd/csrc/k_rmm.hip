@@ -664,7 +664,8 @@ int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned lon
 		vecDecode = nOther > 0 && nLists <= nOther;
 	}
 	// (not for the row sums of squares: the decode kernels multiply decoded values, the squares live in the tables)
-	if(((q >= 2 && q <= 16) || vecDecode) && !squares && !noAlloc && !(b->opt.rmmDisable & 8)) {
+	// (B wider than 16 columns: only blocks of plain streams, 16 columns of B per pass)
+	if((q >= 2 || vecDecode) && !squares && !noAlloc && !(b->opt.rmmDisable & 8)) {
 		const int r = launch_rmm_decode(b, dB, q, constRow >= 0 ? tables + (size_t) constRow * q : nullptr, dOut, dNnz);
 		if(r <= 0) return r;
 	}

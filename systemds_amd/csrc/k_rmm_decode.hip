@@ -1031,9 +1031,10 @@ struct DirArgs {
 	const double* zeroRow;
 	int nDicts, dictDoubles;
 	int segEnd[DSEG_N];
-	const double* B;
+	const double* B;        // first of the QV columns of this launch
 	const double* constRow;
-	double* out;
+	double* out;            // likewise
+	int ld;                 // columns of B and of the output (>= QV: wide B goes in chunks of 16 columns)
 	int64_t nRows;
 	unsigned long long* nnz;
 };
@@ -1087,7 +1088,7 @@ __global__ __launch_bounds__(DIR_THREADS) void k_rmm_direct(const DirArgs A) {
 				src[u] = (const uint8_t*) D[u][0];
 				base8[u] = (int) (uint32_t) D[u][1]; nC8[u] = (int) (D[u][1] >> 32);
 				const int orig = (int) (uint32_t) D[u][2];
-				brow[u] = orig < 0 ? (dec_cdp) A.zeroRow : Bc + (size_t) orig * QV;
+				brow[u] = orig < 0 ? (dec_cdp) A.zeroRow : Bc + (size_t) orig * A.ld;
 			}
 #pragma unroll
 			for(int u = 0; u < NBAT; u++) {
@@ -1141,10 +1142,15 @@ __global__ __launch_bounds__(DIR_THREADS) void k_rmm_direct(const DirArgs A) {
 		auto seg = [&](auto kindTag, auto twoTag, int k0, int k1) {
 			int k = k0; // (every class holds an even number of columns)
 			if(full) {
+				// (columns in flight: eight next to at most 2 x 12 sums, two next to more: C5 with 13 / 15 columns of B 1.86 / 2.02
+				// instead of 2.14 / 2.67 ms)
+				if constexpr(QV <= 12) {
 #pragma unroll 1
-				for(; k + 8 <= k1; k += 8) batch(kindTag, twoTag, std::integral_constant<int, 8>(), std::false_type(), k);
-				if(k + 4 <= k1) { batch(kindTag, twoTag, std::integral_constant<int, 4>(), std::false_type(), k); k += 4; }
-				if(k + 2 <= k1) batch(kindTag, twoTag, std::integral_constant<int, 2>(), std::false_type(), k);
+					for(; k + 8 <= k1; k += 8) batch(kindTag, twoTag, std::integral_constant<int, 8>(), std::false_type(), k);
+					if(k + 4 <= k1) { batch(kindTag, twoTag, std::integral_constant<int, 4>(), std::false_type(), k); k += 4; }
+				}
+#pragma unroll 1
+				for(; k + 2 <= k1; k += 2) batch(kindTag, twoTag, std::integral_constant<int, 2>(), std::false_type(), k);
 			}
 			else {
 #pragma unroll 1
@@ -1168,18 +1174,45 @@ __global__ __launch_bounds__(DIR_THREADS) void k_rmm_direct(const DirArgs A) {
 			const int64_t rowBase = s0 + part * DIR_SROWS;
 			const int nr = (int) max((int64_t) 0, min((int64_t) DIR_SROWS, nRows - rowBase));
 			const int n = nr * QV;
-			double* o = A.out + (size_t) rowBase * QV; // (a multiple of 16 bytes: rowBase is even)
+			if(A.ld == QV) { // (uniform) the rows are one contiguous range of the output
+				double* o = A.out + (size_t) rowBase * QV; // (a multiple of 16 bytes: rowBase is even)
 #pragma unroll
-			for(int i = 2 * lane; i < DIR_SROWS * QV; i += 128) {
-				if(i + 1 < n) {
-					const f64x2 v = *(const f64x2*) (wstage + i);
-					cnt += (v[0] != 0.0) + (v[1] != 0.0);
-					__builtin_nontemporal_store(v, (f64x2*) (o + i));
+				for(int i = 2 * lane; i < DIR_SROWS * QV; i += 128) {
+					if(i + 1 < n) {
+						const f64x2 v = *(const f64x2*) (wstage + i);
+						cnt += (v[0] != 0.0) + (v[1] != 0.0);
+						__builtin_nontemporal_store(v, (f64x2*) (o + i));
+					}
+					else if(i < n) {
+						const double v = wstage[i];
+						cnt += v != 0.0;
+						__builtin_nontemporal_store(v, o + i);
+					}
 				}
-				else if(i < n) {
-					const double v = wstage[i];
-					cnt += v != 0.0;
-					__builtin_nontemporal_store(v, o + i);
+			}
+			else { // QV of the output's ld columns: pieces of QV values per row (pairs where QV is even and the output allows 16-byte stores)
+				double* o = A.out + (size_t) rowBase * A.ld;
+				const bool pairs = (QV & 1) == 0 && (A.ld & 1) == 0 && ((uintptr_t) A.out & 15) == 0;
+#pragma unroll
+				for(int i = 2 * lane; i < DIR_SROWS * QV; i += 128) {
+					const int r0 = i / QV, c0 = i - r0 * QV;
+					if(pairs) {
+						if(i + 1 < n) {
+							const f64x2 v = *(const f64x2*) (wstage + i);
+							cnt += (v[0] != 0.0) + (v[1] != 0.0);
+							__builtin_nontemporal_store(v, (f64x2*) (o + (size_t) r0 * A.ld + c0));
+						}
+					}
+					else {
+#pragma unroll
+						for(int e = 0; e < 2; e++)
+							if(i + e < n) {
+								const int r = (i + e) / QV, c = (i + e) - r * QV;
+								const double v = wstage[i + e];
+								cnt += v != 0.0;
+								__builtin_nontemporal_store(v, o + (size_t) r * A.ld + c);
+							}
+					}
 				}
 			}
 		}
@@ -1289,23 +1322,31 @@ static int launch_rmm_direct(cla_block* b, const double* dB, int q, const double
 		if(rc) return rc;
 	}
 	DirArgs A = b->dirPlan->A;
-	const size_t lds = ((size_t) A.dictDoubles + (size_t) DIR_WAVES * DIR_SROWS * q) * 8;
-	if(lds > (size_t) std::min(g_ldsPerBlock, 160 * 1024) - 1024) return 1;
-	A.B = dB; A.constRow = dConstRow; A.out = dOut; A.nnz = dNnz;
+	const size_t ldsMax = ((size_t) A.dictDoubles + (size_t) DIR_WAVES * DIR_SROWS * std::min(q, 16)) * 8;
+	if(ldsMax > (size_t) std::min(g_ldsPerBlock, 160 * 1024) - 1024) return 1;
+	A.nnz = dNnz; A.ld = q;
 	const int64_t nSlices = (b->nRows + DIR_SLICE - 1) / DIR_SLICE;
 	const unsigned grid = (unsigned) std::min<int64_t>((nSlices + DIR_WAVES - 1) / DIR_WAVES, g_numCU);
-	const double algo = (double) b->device_bytes_cached + (double) b->nRows * q * 8;
-	Prof pf(b, "k_rmm_direct", grid, DIR_THREADS, (long) lds, algo);
-	switch(q) {
+	// B wider than 16 columns: 16 columns per pass over the block (whole 128-byte lines of the output rows; 12 columns
+	// per pass take less time per column to compute and twice as long to store: C5, 64 columns: 23 against 10 ms)
+	const int chunk = 16;
+	for(int c0 = 0; c0 < q; c0 += chunk) {
+		const int qv = std::min(chunk, q - c0);
+		const size_t lds = ((size_t) A.dictDoubles + (size_t) DIR_WAVES * DIR_SROWS * qv) * 8;
+		A.B = dB + c0; A.constRow = dConstRow ? dConstRow + c0 : nullptr; A.out = dOut + c0;
+		const double algo = (double) b->device_bytes_cached + (double) b->nRows * qv * 8;
+		Prof pf(b, "k_rmm_direct", grid, DIR_THREADS, (long) lds, algo);
+		switch(qv) {
 #define DIR_CASE(QV)                                                                              \
 	case QV:                                                                                      \
 		CLA_HIP(allow_full_lds((const void*) k_rmm_direct<QV>));                                  \
 		hipLaunchKernelGGL(k_rmm_direct<QV>, dim3(grid), dim3(DIR_THREADS), lds, b->stream, A); \
 		break;
-		DIR_CASE(1) DIR_CASE(2) DIR_CASE(3) DIR_CASE(4) DIR_CASE(5) DIR_CASE(6) DIR_CASE(7) DIR_CASE(8)
-		DIR_CASE(9) DIR_CASE(10) DIR_CASE(11) DIR_CASE(12) DIR_CASE(13) DIR_CASE(14) DIR_CASE(15) DIR_CASE(16)
+			DIR_CASE(1) DIR_CASE(2) DIR_CASE(3) DIR_CASE(4) DIR_CASE(5) DIR_CASE(6) DIR_CASE(7) DIR_CASE(8)
+			DIR_CASE(9) DIR_CASE(10) DIR_CASE(11) DIR_CASE(12) DIR_CASE(13) DIR_CASE(14) DIR_CASE(15) DIR_CASE(16)
 #undef DIR_CASE
-		default: return 1;
+			default: return -CLA_ERR_INVALID;
+		}
 	}
 	CLA_HIP(hipGetLastError());
 	return 0;
@@ -1314,15 +1355,19 @@ static int launch_rmm_direct(cla_block* b, const double* dB, int q, const double
 // Returns 1 when the block/shape is not eligible (caller uses the generic path).
 int launch_rmm_decode(cla_block* b, const double* dB, int q, const double* dConstRow, double* dOut,
 	unsigned long long* dNnz) {
-	if(b->groups.empty() || b->nRows == 0 || q < 1 || q > DEC_QMAX) return 1;
-	if(b->opt.rmmDirect) {
+	if(b->groups.empty() || b->nRows == 0 || q < 1) return 1;
+	// (16 columns: no padding of B left for the tile kernel to lose, and the stream kernel short of registers: C5 2.1 against 2.5 ms)
+	const bool tilesFirst = q == DEC_QMAX;
+	if(b->opt.rmmDirect && !tilesFirst) {
 		const int rc = launch_rmm_direct(b, dB, q, dConstRow, dOut, dNnz);
 		if(rc != 1) return rc;
 	}
+	if(q > DEC_QMAX) return 1;
 	DecLaunch L;
 	int rpl = 4; // rows per lane and pass: the smaller output staging area when LDS is short
 	int rc = dec_prepare(b, false, q, rpl, L);
 	if(rc == 1) rc = dec_prepare(b, false, q, rpl = 2, L);
+	if(rc == 1 && tilesFirst && b->opt.rmmDirect) return launch_rmm_direct(b, dB, q, dConstRow, dOut, dNnz);
 	if(rc) return rc;
 	L.A.B = dB; L.A.constRow = dConstRow; L.A.out = dOut; L.A.nnz = dNnz;
 	double algo = (double) b->device_bytes_cached + (double) b->nRows * q * 8;
