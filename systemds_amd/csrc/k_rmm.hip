@@ -670,7 +670,7 @@ int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned lon
 		if(r <= 0) return r;
 	}
 	// 2 to 7 columns of B on an all-DDC block whose dictionaries the decode kernel cannot hold in LDS: the matrix-core
-	// kernel on a zero-padded B (2.5 ms on C2 whatever the width, against 2.8 - 5 ms of the gather per row and group)
+	// kernel on a zero-padded B (1.2 ms on C2, against 2.8 - 5 ms of the gather per row and group)
 	if(q >= 2 && q < 8 && !noAlloc && !(b->opt.rmmDisable & 4)) {
 		const int r = launch_rmm_mfma(b, dB, q, constRow >= 0 ? tables + (size_t) constRow * q : nullptr, dOut, dNnz);
 		if(r <= 0) return r;

@@ -109,7 +109,9 @@ __device__ __forceinline__ double mf_dpp_merge(double keep, double from) {
 	return r;
 }
 
-template <int WAVES, int W>
+// NQ: quarters of the 64 output columns of a pass that B has (16 columns each): the others are neither multiplied nor
+// stored (a pass costs 0.7 ms of fill, decode and output + 0.5 ms per quarter on C2)
+template <int WAVES, int W, int NQ = 4>
 __global__ __launch_bounds__(WAVES * 64) void k_rmm_mfma(const MfSlab* __restrict__ slabs, int nSlabs,
 	const uint32_t* __restrict__ infoG, const MfSrc* __restrict__ colSrc, int nColsAll, const double* __restrict__ Bl, int q, int n0,
 	const double* __restrict__ constRow, double* __restrict__ out, int64_t nRows, int ldsDictDoubles, int ldsKc, int bufBytes,
@@ -185,11 +187,11 @@ __global__ __launch_bounds__(WAVES * 64) void k_rmm_mfma(const MfSlab* __restric
 	if((int) blockIdx.x < nTiles) fill(blockIdx.x, 0, 0);
 	for(int tile = blockIdx.x; tile < nTiles; tile += gridDim.x) {
 		const int64_t blockRow0 = (int64_t) tile * ROWS;
-		double acc[MF_MT][MF_NJ];
+		double acc[MF_MT][4 * NQ];
 #pragma unroll
 		for(int m = 0; m < MF_MT; m++)
 #pragma unroll
-			for(int n = 0; n < MF_NJ; n++) acc[m][n] = 0.0;
+			for(int n = 0; n < 4 * NQ; n++) acc[m][n] = 0.0;
 
 		for(int s = 0; s < nSlabs; s++, buf ^= 1) {
 			const int kc = (slabS[s].nc + 3) & ~3;
@@ -241,15 +243,33 @@ __global__ __launch_bounds__(WAVES * 64) void k_rmm_mfma(const MfSlab* __restric
 				const int k2 = min(kt + 8, kc - 4), k1 = min(kt + 4, kc - 4);
 				codes_at(k2, c2, i2);
 				values_at(c1, i1, a1);
-#define MF_QUARTER(QI, CUR, NXT, NKT, NQ)                                                                          \
-				b_quarter(NKT, NQ, NXT);                                                                             \
+#define MF_QUARTER(QI, CUR, NXT, NKT, NQI)                                                                         \
+				b_quarter(NKT, NQI, NXT);                                                                            \
 				_Pragma("unroll") for(int m = 0; m < MF_MT; m++)                                                      \
 					_Pragma("unroll") for(int n = 0; n < 4; n++)                                                      \
 						acc[m][4 * QI + n] = __builtin_amdgcn_mfma_f64_4x4x4f64(a0[m], CUR[n], acc[m][4 * QI + n], 0, 0, 0);
-				MF_QUARTER(0, bA, bB, kt, 1)
-				MF_QUARTER(1, bB, bA, kt, 2)
-				MF_QUARTER(2, bA, bB, kt, 3)
-				MF_QUARTER(3, bB, bA, k1, 0)
+				if constexpr(NQ == 4) {
+					MF_QUARTER(0, bA, bB, kt, 1)
+					MF_QUARTER(1, bB, bA, kt, 2)
+					MF_QUARTER(2, bA, bB, kt, 3)
+					MF_QUARTER(3, bB, bA, k1, 0)
+				}
+				else if constexpr(NQ == 3) {
+					MF_QUARTER(0, bA, bB, kt, 1)
+					MF_QUARTER(1, bB, bA, kt, 2)
+					MF_QUARTER(2, bA, bB, k1, 0)
+#pragma unroll
+					for(int n = 0; n < 4; n++) bA[n] = bB[n];
+				}
+				else if constexpr(NQ == 2) {
+					MF_QUARTER(0, bA, bB, kt, 1)
+					MF_QUARTER(1, bB, bA, k1, 0)
+				}
+				else {
+					MF_QUARTER(0, bA, bB, k1, 0)
+#pragma unroll
+					for(int n = 0; n < 4; n++) bA[n] = bB[n];
+				}
 #undef MF_QUARTER
 			}
 		}
@@ -287,7 +307,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_rmm_mfma(const MfSlab* __restric
 			for(int m = 0; m < MF_MT; m++) {
 				const int64_t row = rowBase + 16 * m;
 #pragma unroll
-				for(int L = 0; L < MF_NJ / 4; L++) {
+				for(int L = 0; L < NQ; L++) {
 					const int col = n0 + 16 * L + 8 * odd + 2 * lj;
 					f64x2 first, second;
 					// odd quads: the second half line of the even quad four lanes below (row_shr:4 = 0x114, banks 1 and 3)
@@ -435,8 +455,6 @@ int launch_rmm_mfma(cla_block* b, const double* dB, int q, const double* dConstR
 	const MfSrc* dSrc = (const MfSrc*) (base + b->mfOff[2]);
 	const int32_t* dRowCol = (const int32_t*) (base + b->mfOff[3]);
 	const size_t lds = 2 * b->mfBufBytes + (size_t) b->mfNColsAll * sizeof(MfSrc) + (size_t) b->mfNSlabs * sizeof(MfSlab);
-	if(b->mfWidth == 1) CLA_HIP(allow_full_lds((const void*) k_rmm_mfma<MF_WAVES, 1>));
-	else CLA_HIP(allow_full_lds((const void*) k_rmm_mfma<MF_WAVES, 2>));
 	if(lds > (size_t) g_ldsPerBlock) return 1;
 	// persistent blocks: one per CU, each walks its row tiles
 	const unsigned grid = (unsigned) std::min<int64_t>((b->nRows + rows - 1) / rows, (int64_t) g_numCU);
@@ -449,10 +467,19 @@ int launch_rmm_mfma(cla_block* b, const double* dB, int q, const double* dConstR
 			hipLaunchKernelGGL(k_mfma_blayout, dim3((unsigned) b->mfNRowCol), dim3(128), 0, st, dB, q, n0, dRowCol, dBl);
 		}
 		Prof pf(b, "k_rmm_mfma", grid, MF_WAVES * 64, (long) lds, codeBytes + (double) b->nRows * qq * 8);
-#define MF_LAUNCH(CW)                                                                                                     \
-	hipLaunchKernelGGL((k_rmm_mfma<MF_WAVES, CW>), dim3(grid), dim3(MF_WAVES * 64), lds, st, dSlabs, b->mfNSlabs, dInfo, dSrc, \
-		b->mfNColsAll, dBl, q, n0, dConstRow, dOut, b->nRows, b->mfMaxDict, b->mfMaxKc, (int) b->mfBufBytes, dNnz)
-		if(b->mfWidth == 1) MF_LAUNCH(1); else MF_LAUNCH(2);
+		const int nq = (qq + 15) / 16; // quarters of the pass's 64 columns that B has
+#define MF_LAUNCH(CW, NQV)                                                                                                     \
+	do {                                                                                                                       \
+		CLA_HIP(allow_full_lds((const void*) k_rmm_mfma<MF_WAVES, CW, NQV>));                                                  \
+		hipLaunchKernelGGL((k_rmm_mfma<MF_WAVES, CW, NQV>), dim3(grid), dim3(MF_WAVES * 64), lds, st, dSlabs, b->mfNSlabs, dInfo, dSrc, \
+			b->mfNColsAll, dBl, q, n0, dConstRow, dOut, b->nRows, b->mfMaxDict, b->mfMaxKc, (int) b->mfBufBytes, dNnz);               \
+	} while(0)
+#define MF_WIDTH(NQV)                                                   \
+	do {                                                                \
+		if(b->mfWidth == 1) MF_LAUNCH(1, NQV); else MF_LAUNCH(2, NQV); \
+	} while(0)
+		if(nq == 1) MF_WIDTH(1); else if(nq == 2) MF_WIDTH(2); else if(nq == 3) MF_WIDTH(3); else MF_WIDTH(4);
+#undef MF_WIDTH
 #undef MF_LAUNCH
 	}
 	CLA_HIP(hipGetLastError());
