@@ -75,6 +75,7 @@ struct DecArgs {
 	int valDoubles, bDoubles, stageDoubles, slotBytes; // LDS sizes
 	const double* B;
 	int q;
+	int ld;                            // columns of B and of the output (>= q: wide B goes in passes of 16 columns)
 	const double* constRow;
 	const double* Y;                   // left multiply: Y (P x nRows, row-major); out is P x nCols
 	int P;
@@ -227,7 +228,7 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 		if(!GRAM)
 			for(int i = tid; i < P.nC * A.q; i += DEC_THREADS) {
 				const int h = i / A.q, c = i - h * A.q;
-				Bs[(size_t) (P.kOff + h) * 16 + c] = A.B[(size_t) G.cols[h] * A.q + c];
+				Bs[(size_t) (P.kOff + h) * 16 + c] = A.B[(size_t) G.cols[h] * A.ld + c];
 			}
 	}
 
@@ -629,7 +630,7 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 			const int nr = (int) max((int64_t) 0, min((int64_t) PROWS, nRows - rowBase));
 			// the pass's rows are one contiguous range of the output: 16 bytes per lane (the range starts on a
 			// multiple of 16 bytes: rowBase is a multiple of 16 rows), a single double at an odd end
-			{
+			if(A.ld == q) {
 				const int n = nr * q;
 				double* o = A.out + (size_t) rowBase * q;
 				for(int i = 2 * lane; i + 1 < n; i += 128) {
@@ -641,6 +642,27 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 					const double v = wstage[n - 1];
 					cnt += v != 0.0;
 					__builtin_nontemporal_store(v, o + n - 1);
+				}
+			}
+			else {
+				// q of the output's ld columns (a pass over wide B): pieces of q values per row
+				const int n = nr * q;
+				double* o = A.out + (size_t) rowBase * A.ld;
+				const bool pairs = (q & 1) == 0 && (A.ld & 1) == 0 && ((uintptr_t) A.out & 15) == 0;
+				for(int i = 2 * lane; i < n; i += 128) {
+					const int r0 = i / q, c0 = i - r0 * q;
+					if(pairs) {
+						const f64x2 v = *(const f64x2*) (wstage + i);
+						cnt += (v[0] != 0.0) + (v[1] != 0.0);
+						__builtin_nontemporal_store(v, (f64x2*) (o + (size_t) r0 * A.ld + c0));
+					}
+					else
+						for(int e = 0; e < 2 && i + e < n; e++) {
+							const int r = (i + e) / q, c = (i + e) - r * q;
+							const double v = wstage[i + e];
+							cnt += v != 0.0;
+							__builtin_nontemporal_store(v, o + (size_t) r * A.ld + c);
+						}
 				}
 			}
 		}
@@ -918,7 +940,7 @@ static int dec_build_plan(cla_block* b, bool gram, int q, int rpl, DecLaunch& L,
 	A.nTasks = (int) taskCost.size();
 	A.nGroups = nG; A.nCopies = (int) copies.size(); A.nChunks = nChunks; A.nColD = nColD;
 	A.valDoubles = (int) valD; A.bDoubles = (int) bD; A.stageDoubles = (int) stageD; A.slotBytes = (int) slotB;
-	A.B = nullptr; A.q = q; A.constRow = nullptr; A.Y = nullptr; A.P = 0; A.badY = nullptr; A.out = nullptr; A.nRows = b->nRows; A.nnz = nullptr; A.nCols = nCols;
+	A.B = nullptr; A.q = q; A.ld = q; A.constRow = nullptr; A.Y = nullptr; A.P = 0; A.badY = nullptr; A.out = nullptr; A.nRows = b->nRows; A.nnz = nullptr; A.nCols = nCols;
 	const int nTiles = (int) ((b->nRows + DEC_TILE - 1) / DEC_TILE);
 	const int blocksPerCU = L.lds <= 76 * 1024 ? 2 : 1;
 	L.grid = (unsigned) std::min(nTiles, g_numCU * blocksPerCU);
@@ -1362,23 +1384,35 @@ int launch_rmm_decode(cla_block* b, const double* dB, int q, const double* dCons
 		const int rc = launch_rmm_direct(b, dB, q, dConstRow, dOut, dNnz);
 		if(rc != 1) return rc;
 	}
-	if(q > DEC_QMAX) return 1;
-	DecLaunch L;
-	int rpl = 4; // rows per lane and pass: the smaller output staging area when LDS is short
-	int rc = dec_prepare(b, false, q, rpl, L);
-	if(rc == 1) rc = dec_prepare(b, false, q, rpl = 2, L);
-	if(rc == 1 && tilesFirst && b->opt.rmmDirect) return launch_rmm_direct(b, dB, q, dConstRow, dOut, dNnz);
-	if(rc) return rc;
-	L.A.B = dB; L.A.constRow = dConstRow; L.A.out = dOut; L.A.nnz = dNnz;
-	double algo = (double) b->device_bytes_cached + (double) b->nRows * q * 8;
-	Prof pf(b, "k_rmm_decode", L.grid, DEC_THREADS, (long) L.lds, algo);
-	if(rpl == 4) {
-		CLA_HIP(allow_full_lds((const void*) k_rmm_decode<4>));
-		hipLaunchKernelGGL(k_rmm_decode<4>, dim3(L.grid), dim3(DEC_THREADS), L.lds, b->stream, L.A);
+	// (B wider than 16 columns: 16 columns per pass over the block, as in the stream kernel; not where offset lists
+	// carry most of the block: their own tile kernel works per entry, this one per row)
+	if(q > DEC_QMAX) {
+		int nLists = 0, nOther = 0;
+		for(auto& g : b->groups) {
+			if(g.d.type == G_SDCZ) nLists += g.d.nOffsets > 0;
+			else nOther += g.d.type == G_UNC || g.d.nVals > 0;
+		}
+		if(nOther == 0 || nLists > nOther) return 1;
 	}
-	else {
-		CLA_HIP(allow_full_lds((const void*) k_rmm_decode<2>));
-		hipLaunchKernelGGL(k_rmm_decode<2>, dim3(L.grid), dim3(DEC_THREADS), L.lds, b->stream, L.A);
+	for(int c0 = 0; c0 < q; c0 += DEC_QMAX) {
+		const int qv = std::min(DEC_QMAX, q - c0);
+		DecLaunch L;
+		int rpl = 4; // rows per lane and pass: the smaller output staging area when LDS is short
+		int rc = dec_prepare(b, false, qv, rpl, L);
+		if(rc == 1) rc = dec_prepare(b, false, qv, rpl = 2, L);
+		if(rc == 1 && c0 == 0 && tilesFirst && b->opt.rmmDirect) return launch_rmm_direct(b, dB, q, dConstRow, dOut, dNnz);
+		if(rc) return rc;
+		L.A.B = dB + c0; L.A.ld = q; L.A.constRow = dConstRow ? dConstRow + c0 : nullptr; L.A.out = dOut + c0; L.A.nnz = dNnz;
+		double algo = (double) b->device_bytes_cached + (double) b->nRows * qv * 8;
+		Prof pf(b, "k_rmm_decode", L.grid, DEC_THREADS, (long) L.lds, algo);
+		if(rpl == 4) {
+			CLA_HIP(allow_full_lds((const void*) k_rmm_decode<4>));
+			hipLaunchKernelGGL(k_rmm_decode<4>, dim3(L.grid), dim3(DEC_THREADS), L.lds, b->stream, L.A);
+		}
+		else {
+			CLA_HIP(allow_full_lds((const void*) k_rmm_decode<2>));
+			hipLaunchKernelGGL(k_rmm_decode<2>, dim3(L.grid), dim3(DEC_THREADS), L.lds, b->stream, L.A);
+		}
 	}
 	CLA_HIP(hipGetLastError());
 	return 0;

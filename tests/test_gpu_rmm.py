@@ -470,3 +470,36 @@ def test_blocks_the_stream_kernel_does_not_take(cla, ora):
         assert "k_rmm_direct" not in names, (variant, names)
         assert_matches_truth(out, D, B, what=f"{variant}")
         assert nnz == np.count_nonzero(out)
+
+
+@pytest.mark.parametrize("q", [17, 40, 64])
+def test_wide_right_multiply_in_passes_of_the_tile_kernel(cla, ora, q):
+    """Long runs (no one-code-per-row copy: it would dwarf the group), two-byte DDC codes and three dense columns: the
+    tile kernel takes B 16 columns per pass."""
+    from systemds_amd import synth
+    n_rows = 150001
+    rng = np.random.default_rng(q)
+    specs, c = [], 0
+    for _ in range(3):
+        lens = rng.geometric(1.0 / 3000.0, size=n_rows // 2000 + 16)
+        codes = np.repeat(rng.integers(-1, 8, size=lens.size), lens)[:n_rows]
+        if codes.size < n_rows:
+            codes = np.concatenate([codes, np.full(n_rows - codes.size, -1)])
+        ptr, data = synth.encode_rle(codes, 8)
+        specs.append(synth.GroupSpec("rle", np.array([c], np.int32), rng.standard_normal((8, 1)), ptr=ptr, rle=data))
+        c += 1
+    specs.append(synth.GroupSpec("ddc", np.array([c, c + 1], np.int32), rng.standard_normal((700, 2)), rng.integers(0, 700, n_rows).astype(np.uint16)))
+    c += 2
+    specs.append(synth.GroupSpec("unc", np.arange(c, c + 3, dtype=np.int32), dense=rng.standard_normal((n_rows, 3))))
+    c += 3
+    B = rng.standard_normal((c, q))
+    D = ora.np_decompress(specs, n_rows, c)
+    blk = cla.build_block(n_rows, c, specs)
+    try:
+        out, nnz = blk.rmm(B)
+        names = kernels_of(blk, lambda: blk.rmm(B))
+    finally:
+        blk.close()
+    assert names.count("k_rmm_decode") == (q + 15) // 16, names
+    assert_matches_truth(out, D, B, what=f"tile passes q={q}")
+    assert nnz == np.count_nonzero(out)
