@@ -1,7 +1,11 @@
 // Decode-and-multiply on blocks of any group mix, on the matrix cores:
-//   k_rmm_decode      X %*% B for narrow B (q <= 16; a single column where the block is not mostly offset lists)
+//   k_rmm_decode      X %*% B for narrow B (q <= 16; a single column where the block is not mostly offset lists;
+//               wider B 16 columns per pass)
 //   k_tsmm_decode<NB> upper triangle of t(X) %*% X for blocks of at most 16 * NB <= 64 columns (or, for a pair of
 //               column chunks, only the tiles of the first chunk's column blocks with the second's)
+//   k_lmm_decode<NB>  Y %*% X for such blocks, 16 rows of Y per pass: the Gram kernel with Y as the other operand
+// and, further down, for blocks whose groups are all plain streams, on the vector unit and without code tiles:
+//   k_rmm_direct<q>   X %*% B, codes read straight from global memory (wider B 16 columns per pass)
 // A block owns a contiguous range of 1024-row tiles. Per tile every dictionary coded
 // group gets its codes expanded into an LDS code tile (DDC: straight copy, prefetched one
 // tile ahead in registers together with the rows of uncompressed groups; SDCZeros:
