@@ -27,7 +27,6 @@ namespace cla {
 
 constexpr int MF_WAVES = 8;                  // waves per block (two per SIMD): 512-row tiles
 constexpr int MF_MT = 4;                     // 16-row tiles per wave
-constexpr int MF_NJ = 16;                    // groups of 4 output columns per pass (64 output columns)
 // B slab in LDS: row k at k * MF_BK, inside it the 16 values of lane column j (accumulators jg = 0..15)
 // at j * MF_BJ: the 16 distinct 16-byte pieces of a wave's read fall on 16 distinct
 // bank quads (row stride 16 banks, j stride 36 banks)

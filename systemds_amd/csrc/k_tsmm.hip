@@ -490,37 +490,34 @@ __global__ __launch_bounds__(256) void k_gram_dense(const double* __restrict__ D
 // dOut (zeroed) = t(X) %*% X through the decompressed block. -CLA_ERR_UNSUPPORTED when the dense copy does
 // not fit the free device memory.
 static int launch_tsmm_decompressed(cla_block* b, double* dOut, unsigned long long* dNnz, const char* why) {
+	// chunks of rows decompressed into the block's scratch buffer (at most 512 MiB), their Gram matrices added up
+	(void) why;
 	const int nCols = b->nCols;
 	const int64_t nRows = b->nRows;
 	hipStream_t st = b->stream;
-	const size_t bytes = sizeof(double) * (size_t) std::max<int64_t>(nRows, 1) * nCols;
-	size_t freeB = 0, totalB = 0;
-	CLA_HIP(hipMemGetInfo(&freeB, &totalB));
-	if(bytes > freeB / 2) {
-		set_error("tsmm: %s, and the decompressed block (%zu bytes) does not fit the free device memory (%zu)", why, bytes, freeB);
-		return -CLA_ERR_UNSUPPORTED;
-	}
-	double* dense = nullptr;
-	CLA_HIP(hipMalloc((void**) &dense, bytes));
-	int rc = launch_decompress(b, dense, dNnz); // (also counts the dense copy's non-zeros into dNnz: cleared again below)
-	if(rc == 0 && hipMemsetAsync(dNnz, 0, sizeof(unsigned long long), st) != hipSuccess) rc = -CLA_ERR_DEVICE;
-	if(rc == 0 && nRows > 0) {
+	int rc = 0;
+	if(nRows > 0 && nCols > 0) {
+		int64_t rowsPerChunk = std::max<int64_t>((int64_t) 512 * 1024 * 1024 / ((int64_t) nCols * 8) / 1024 * 1024, 1024);
+		rowsPerChunk = std::min(rowsPerChunk, (nRows + 1023) / 1024 * 1024);
+		if((rc = ensure_scratch(b, sizeof(double) * (size_t) rowsPerChunk * nCols))) return rc;
+		double* dense = (double*) b->dScratch;
 		const int nb = (nCols + 15) / 16;
-		int64_t rowsPerBlock = 16384;
-		while(rowsPerBlock > 1024 && (nRows + rowsPerBlock - 1) / rowsPerBlock * nb < (int64_t) g_numCU * 4) rowsPerBlock /= 2;
-		const dim3 grid((unsigned) ((nRows + rowsPerBlock - 1) / rowsPerBlock), (unsigned) nb, (unsigned) ((nb + GD_NBJ - 1) / GD_NBJ));
-		Prof pf(b, "k_gram_dense", (long) grid.x * grid.y * grid.z, 256, 0, (double) bytes);
-		hipLaunchKernelGGL(k_gram_dense, grid, dim3(256), 0, st, dense, nRows, nCols, rowsPerBlock, dOut);
+		for(int64_t r0 = 0; r0 < nRows; r0 += rowsPerChunk) {
+			const int64_t rows = std::min(rowsPerChunk, nRows - r0);
+			if((rc = launch_decompress_rows(b, r0, r0 + rows, dense))) return rc;
+			int64_t rowsPerBlock = 16384;
+			while(rowsPerBlock > 1024 && (rows + rowsPerBlock - 1) / rowsPerBlock * nb < (int64_t) g_numCU * 4) rowsPerBlock /= 2;
+			const dim3 grid((unsigned) ((rows + rowsPerBlock - 1) / rowsPerBlock), (unsigned) nb, (unsigned) ((nb + GD_NBJ - 1) / GD_NBJ));
+			Prof pf(b, "k_gram_dense", (long) grid.x * grid.y * grid.z, 256, 0, (double) rows * nCols * 8);
+			hipLaunchKernelGGL(k_gram_dense, grid, dim3(256), 0, st, dense, rows, nCols, rowsPerBlock, dOut);
+		}
 	}
-	if(rc == 0) {
+	{
 		Prof pf(b, "k_tsmm_finish", 1, 256, 0, 0);
 		hipLaunchKernelGGL(k_tsmm_finish, dim3(1), dim3(256), 0, st, dOut, nCols, b->dConstV, b->dConstV, (double) nRows, 0, dNnz);
-		if(hipGetLastError() != hipSuccess) rc = -CLA_ERR_DEVICE;
 	}
-	(void) hipStreamSynchronize(st); // the dense copy is freed below
-	(void) hipFree(dense);
-	if(rc == -CLA_ERR_DEVICE) set_error("tsmm: decompressing fallback failed on the device");
-	return rc;
+	CLA_HIP(hipGetLastError());
+	return 0;
 }
 
 int launch_tsmm(cla_block* b, double* dOut, unsigned long long* dNnz) {
@@ -605,6 +602,9 @@ int launch_tsmm(cla_block* b, double* dOut, unsigned long long* dNnz) {
 			CLA_HIP(hipGetLastError());
 			return 0;
 		}
+		// (the decode kernel does not take the block: its code tiles, list windows or dictionaries exceed LDS. The scalar
+		// form below beats decompressed chunks of rows on the matrix cores where the block has many groups, one strided
+		// decompression pass each: 4 M rows x 60 columns of two-byte codes 6.7 against 13 ms)
 		int DT = 256;
 		while(DT > 8 && (size_t) DT * nCols * 8 > (size_t) 96 * 1024) DT /= 2;
 		if((size_t) DT * nCols * 8 > (size_t) 96 * 1024 || (int64_t) nCols * (nCols + 1) / 2 > 24 * 256)
