@@ -164,9 +164,10 @@ int cla_lmm_dev_async(cla_handle h, const double* dY, int32_t nRowY, double* dOu
 
 /* CLALibTSMM.leftMultByTransposeSelf (C/lib/CLALibTSMM.java:59-94):
  * out[nCols x nCols] = t(X) %*% X, full symmetric. Blocks no compressed form takes (overlapping
- * groups, more than 110 columns holding an uncompressed group of more than 32, a pair of groups whose
- * pre-aggregate exceeds LDS) are decompressed in chunks of rows (at most 512 MiB of scratch kept with the
- * block) and multiplied on the matrix cores, as the reference's own fallback does (:73-77). */
+ * groups, an uncompressed group of more than 32 columns among more than 64, a pair of groups whose
+ * pre-aggregate exceeds LDS, code tiles, list windows or dictionaries that exceed LDS in the decode
+ * kernel) are decompressed in chunks of rows (at most 512 MiB of scratch kept with the block) and
+ * multiplied on the matrix cores, as the reference's own fallback does (:73-77). */
 int64_t cla_tsmm(cla_handle h, double* out);
 int64_t cla_tsmm_dev(cla_handle h, double* dOut);
 int cla_tsmm_dev_async(cla_handle h, double* dOut);

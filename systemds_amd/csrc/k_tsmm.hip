@@ -7,7 +7,7 @@
 //   k_tsmm_pair         P[code_t(r), :] += dict_s[code_s(r), :] in LDS (the reference's
 //                       preAggregateThatIndexStructure), contracted with dict_t per block
 //   k_tsmm_self         counts x dict (x) dict, and column sums for the correction layer
-//   k_tsmm_dense        fallback: decode row tiles and accumulate the Gram matrix
+//   k_tsmm_dense        scalar form (option tsmm_mfma = 0): decode row tiles and accumulate the Gram matrix
 //   k_tsmm_finish       correction layer, mirror upper -> lower, non-zero count
 //   k_cooc_*            exact integer co-occurrence counts
 //   k_decompress_*      additive decompression into a dense block
@@ -602,9 +602,11 @@ int launch_tsmm(cla_block* b, double* dOut, unsigned long long* dNnz) {
 			CLA_HIP(hipGetLastError());
 			return 0;
 		}
-		// (the decode kernel does not take the block: its code tiles, list windows or dictionaries exceed LDS. The scalar
-		// form below beats decompressed chunks of rows on the matrix cores where the block has many groups, one strided
-		// decompression pass each: 4 M rows x 60 columns of two-byte codes 6.7 against 13 ms)
+		// (the decode kernel does not take the block: its code tiles, list windows or dictionaries exceed LDS. Chunks of
+		// rows decompressed through LDS tiles, their Gram matrices on the matrix cores: 4 M rows x 60 columns of two-byte
+		// codes in 3 ms; the scalar form below, 6.7 ms, stays for the option tsmm_mfma = 0)
+		if(!noMfma && nRows > 0)
+			return launch_tsmm_decompressed(b, dOut, dNnz, "the decode plan exceeds LDS");
 		int DT = 256;
 		while(DT > 8 && (size_t) DT * nCols * 8 > (size_t) 96 * 1024) DT /= 2;
 		if((size_t) DT * nCols * 8 > (size_t) 96 * 1024 || (int64_t) nCols * (nCols + 1) / 2 > 24 * 256)
@@ -826,6 +828,50 @@ __global__ __launch_bounds__(256) void k_decompress_rows(const DGroup* __restric
 	unsafeAtomicAdd(&out[(size_t) rr * nCols + G.cols[j]], v);
 }
 
+// The constants and all groups but the offset lists, a tile of rows at a time through LDS: a block sets its tile to the
+// constants, its waves add the values of (group, 64 rows) items (a lane reads its row's code once and walks the tuple;
+// a dense group is read in the order it is stored), then the block writes whole rows. The adds are LDS atomics, since
+// groups may share columns. The per-group form above writes one value per row with the row stride of the matrix
+// between threads, through an atomic add in HBM: 0.18 ms per column of 4 M rows.
+constexpr int DCT_THREADS = 512;
+__global__ __launch_bounds__(DCT_THREADS) void k_decompress_tiles(const DGroup* __restrict__ groups, int nGroups, int64_t r0, int64_t r1, int nCols,
+	const double* __restrict__ constV, int tileRows, double* __restrict__ out) {
+	extern __shared__ __align__(16) double dtile[];
+	const int tid = threadIdx.x, lane = tid & 63;
+	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+	for(int64_t t0 = r0 + (int64_t) blockIdx.x * tileRows; t0 < r1; t0 += (int64_t) gridDim.x * tileRows) {
+		const int rows = (int) min((int64_t) tileRows, r1 - t0);
+		const int cells = rows * nCols, nChunks = (rows + 63) >> 6;
+		for(int i = tid; i < cells; i += DCT_THREADS) dtile[i] = constV[i % nCols];
+		__syncthreads();
+		for(int item = wave; item < nGroups * nChunks; item += DCT_THREADS / 64) {
+			const int g = item / nChunks, c0 = (item - g * nChunks) << 6;
+			const DGroup G = dgroup(groups + g);
+			if(G.type == G_SDCZ) continue;
+			if(G.type == G_UNC) {
+				const int n = min(64, rows - c0) * G.nColG;
+				const double* src = G.dense + (size_t) (t0 + c0) * G.nColG;
+				for(int idx = lane; idx < n; idx += 64) {
+					const int rr = idx / G.nColG, j = idx - rr * G.nColG;
+					unsafeAtomicAdd(&dtile[(c0 + rr) * nCols + G.cols[j]], src[idx]);
+				}
+				continue;
+			}
+			const int rr = c0 + lane;
+			if(G.nVals <= 0 || rr >= rows) continue;
+			const int64_t r = t0 + rr;
+			const int code = G.type == G_DDC ? load_code(G.codes, G.codeWidth, r) : G.runCode[rle_find(G.runStart, G.nRuns, (int32_t) r)];
+			if(code < 0) continue;
+			const double* tup = G.dict + (size_t) code * G.nColG;
+			for(int j = 0; j < G.nColG; j++) unsafeAtomicAdd(&dtile[rr * nCols + G.cols[j]], tup[j]);
+		}
+		__syncthreads();
+		double* o = out + (size_t) (t0 - r0) * nCols;
+		for(int i = tid; i < cells; i += DCT_THREADS) o[i] = dtile[i];
+		__syncthreads();
+	}
+}
+
 // rows [r0, r1) of the group go to out rows 0 .. r1 - r0; a block of list entries whose rows all lie outside leaves early
 template <int W>
 __global__ __launch_bounds__(256) void k_decompress_sdc(const DGroup* __restrict__ groups, int g, int64_t r0, int64_t r1, int nCols,
@@ -866,13 +912,27 @@ int launch_decompress_rows(cla_block* b, int64_t r0, int64_t r1, double* dOut) {
 	const int64_t n = (r1 - r0) * b->nCols;
 	hipStream_t st = b->stream;
 	if(n <= 0) return 0;
-	const unsigned fg = (unsigned) std::min<int64_t>((n + 255) / 256, (int64_t) g_numCU * 64);
-	{
+	// tiles of rows through LDS (at most 64 KB: two blocks per CU; whole chunks of 64 rows where 64 rows fit, at least 8
+	// rows); blocks too wide for that: group by group
+	int tileRows = (int) std::min<int64_t>(512, 8192 / std::max(b->nCols, 1));
+	if(tileRows >= 64) tileRows &= ~63;
+	const bool tiled = tileRows >= 8;
+	if(tiled) {
+		const int64_t nTiles = (r1 - r0 + tileRows - 1) / tileRows;
+		const unsigned tg = (unsigned) std::min<int64_t>(nTiles, (int64_t) g_numCU * 8);
+		const size_t lds = (size_t) tileRows * b->nCols * 8;
+		Prof pf(b, "k_decompress_tiles", tg, DCT_THREADS, (long) lds, (double) n * 8);
+		CLA_HIP(allow_full_lds((const void*) k_decompress_tiles));
+		hipLaunchKernelGGL(k_decompress_tiles, dim3(tg), dim3(DCT_THREADS), lds, st, b->dGroups, nG, r0, r1, b->nCols, b->dConstV, tileRows, dOut);
+	}
+	else {
+		const unsigned fg = (unsigned) std::min<int64_t>((n + 255) / 256, (int64_t) g_numCU * 64);
 		Prof pf(b, "k_decompress_fill", fg, 256, 0, 0);
 		hipLaunchKernelGGL(k_decompress_fill, dim3(fg), dim3(256), 0, st, dOut, n, b->nCols, b->dConstV);
 	}
 	for(int g = 0; g < nG; g++) {
 		const DGroup& G = b->groups[g].d;
+		if(G.type != G_SDCZ && tiled) continue;
 		if(G.type == G_SDCZ) {
 			if(G.nOffsets == 0) continue;
 			const unsigned sg = (unsigned) std::max(G.nCkpt, 1);
