@@ -229,3 +229,32 @@ def test_mixed_block_with_non_finite_values_in_y(cla, ora):
     D = ora.np_decompress(specs, n_rows, n_cols)
     Yc = np.nan_to_num(Y, nan=0.0, posinf=0.0, neginf=0.0)
     assert_fp64_close(out[fin], ref[fin], ora.abs_matmul(Yc, D)[fin], what="Y %*% X, non-finite Y", n_terms=n_rows)
+
+
+@pytest.mark.parametrize("p", [1, 16, 17, 33])
+def test_wide_dense_groups_on_the_matrix_cores(cla, ora, p):
+    """Uncompressed groups of 70 and 5 columns (more than one set of four 16-column blocks, a ragged last block) beside
+    a DDC group, 20,011 rows (a ragged last row tile per wave): `k_lmm_unc` takes 16 rows of Y per pass."""
+    from systemds_amd import synth
+    rng = np.random.default_rng(40 + p)
+    n_rows, n_cols = 20011, 77
+    perm = rng.permutation(n_cols).astype(np.int32)
+    dense_a = rng.standard_normal((n_rows, 70))
+    dense_a[rng.random((n_rows, 70)) < 0.3] = 0.0
+    specs = [synth.GroupSpec("unc", np.sort(perm[:70]), dense=dense_a),
+             synth.GroupSpec("unc", np.sort(perm[70:75]), dense=rng.standard_normal((n_rows, 5))),
+             synth.GroupSpec("ddc", np.sort(perm[75:]), rng.standard_normal((9, 2)), rng.integers(0, 9, n_rows).astype(np.uint8))]
+    Y = rng.standard_normal((p, n_rows))
+    D = ora.np_decompress(specs, n_rows, n_cols)
+    blk = cla.build_block(n_rows, n_cols, specs)
+    try:
+        blk.profile(True)
+        out, nnz = blk.lmm(Y)
+        names = [k["name"] for k in blk.stats()["kernels"]]
+    finally:
+        blk.close()
+    assert "k_lmm_unc" in names, names
+    ref, rnnz = ora.lmm(ora.Groups(specs, n_rows, n_cols), Y, 4)
+    assert_matches_truth(out, Y, D, what=f"Y %*% X, dense groups, {p} rows")
+    assert_fp64_close(out, ref, ora.abs_matmul(Y, D), what=f"Y %*% X, dense groups, {p} rows", n_terms=n_rows)
+    assert nnz == rnnz
