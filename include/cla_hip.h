@@ -118,9 +118,11 @@ int cla_block_set_stream(cla_handle h, void* hipStream);
  *   sdc_packed      1 / 0: packed SDCZeros lists for the mat-vecs
  *   sdc_lanes       1 / 0: SDCZeros mat-vecs on lane-major copies of the lists, one lane per group
  *   sdc_rows        1 / 0: SDCZeros X %*% v on row lists (the lists transposed), one lane per row
- *   lmm_joint       1 / 0: Y %*% X (16 rows of Y per pass) on a block of at most 64 columns that is neither mostly offset lists nor
- *                   byte-code DDC groups in one pass over the decoded rows on the matrix cores (the kernel reports non-finite
- *                   values of Y and the host looks, i.e. waits for the stream once per call; such a Y takes the bin kernels)
+ *   lmm_joint       1 / 0: Y %*% X (16 rows of Y per pass) on a block that is not mostly offset lists in passes over the decoded
+ *                   rows on the matrix cores; blocks of more than 64 columns, or whose code tiles exceed LDS together, go chunk of
+ *                   columns by chunk (sub-blocks kept with the block); single-column byte-code blocks only from 13 rows of Y
+ *                   on (the kernel reports non-finite values of Y and the host looks, i.e. waits for the stream once per call;
+ *                   such a Y takes the bin kernels)
  * Blocks derived from this one (overlapping results, joint blocks) inherit the values at the time of the call
  * that uses them. Returns 0, or -CLA_ERR_INVALID for an unknown key or value. */
 int cla_block_set_option(cla_handle h, const char* key, int32_t value);

@@ -2,7 +2,7 @@
 // host/device entry points of the multiply drivers. Host-side logic only; the
 // kernels live in k_*.hip.
 #include "../../include/cla_hip.h"
-#include "cla_internal.hpp"
+#include "cla_device.hpp"
 #include <algorithm>
 #include <cstdarg>
 #include <cstring>
@@ -193,6 +193,7 @@ struct SubBlock {
 
 int finish_finalize(cla_block* b, cla_block* arenaFrom, bool buildArena = true);
 static void free_subs(cla_block* b);
+static void free_lmm_subs(cla_block* b);
 
 } // namespace cla
 
@@ -287,6 +288,7 @@ void cla_block_free(cla_handle b) {
 	cla_block* parent = b->parent;
 	if(b->joint) { cla_block_free(b->joint); b->joint = nullptr; }
 	free_subs(b);
+	free_lmm_subs(b);
 	if(g_device >= 0) (void) hipSetDevice(g_device);
 	if(b->stream) (void) hipStreamSynchronize(b->stream);
 	clear_stats(b);
@@ -1173,13 +1175,197 @@ int launch_tsmm_chunked(cla_block* b, double* dOut) {
 	return 0;
 }
 
-// Y %*% X as the (left, right) part of the decoded Gram matrix of cbind(t(Y), X): one pass over X's row data on the
-// matrix cores whatever its group mix and however many rows Y has (2 to 16), where the bin kernels take a pass per
-// row of Y and group type (C5, 50 M x 20: 2.9 / 3.7 / 4.7 ms against 5.1 / 8.9 / 18 ms for 2 / 4 / 8 rows of Y). Taken for
-// blocks of at most 48 columns that neither the byte-code dot form nor the offset-list kernels serve. Returns 1 when
-// the block is not eligible, 0 when dOut (p x nCols) holds the result and *dNnz its non-zero count.
+// ---- Y %*% X on the decode kernel
+struct LmmSub {
+	cla_block* blk;   // null: the columns that no group covers (row sums of Y times their constants)
+	int32_t* dColMap; // column of the block per column of blk
+	int k;
+};
+
+static void free_lmm_subs(cla_block* b) {
+	for(void* p : b->lmmSubs) {
+		LmmSub* sb = (LmmSub*) p;
+		if(sb->dColMap) (void) hipFree(sb->dColMap);
+		if(sb->blk) cla_block_free(sb->blk);
+		delete sb;
+	}
+	b->lmmSubs.clear();
+}
+
+// out[i, colMap[j]] = S[i, j] for the k columns of a chunk; counts the non-zero cells it writes
+__global__ __launch_bounds__(256) void k_scatter_cols(const double* __restrict__ S, int k, const int32_t* __restrict__ colMap, int p,
+	double* __restrict__ out, int n, unsigned long long* __restrict__ nnz) {
+	int cnt = 0;
+	for(int idx = threadIdx.x + blockIdx.x * 256; idx < p * k; idx += 256 * gridDim.x) {
+		const int i = idx / k, j = idx - i * k;
+		const double v = S[idx];
+		out[(size_t) i * n + colMap[j]] = v;
+		cnt += v != 0.0;
+	}
+	if(cnt) atomicAdd(nnz, (unsigned long long) cnt);
+}
+
+// rs[i] += sum of Y[i, rows of the block]
+__global__ __launch_bounds__(256) void k_y_rowsum(const double* __restrict__ Y, int64_t nRows, int64_t rowsPerBlock, double* __restrict__ rs) {
+	__shared__ double red[4];
+	const double* y = Y + (size_t) blockIdx.y * nRows;
+	const int64_t rb = (int64_t) blockIdx.x * rowsPerBlock, re = min(rb + rowsPerBlock, nRows);
+	double s = 0.0;
+	for(int64_t r = rb + threadIdx.x; r < re; r += 256) s += y[r];
+	s = wave_sum_f64(s);
+	if((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
+	__syncthreads();
+	if(threadIdx.x == 0) unsafeAtomicAdd(&rs[blockIdx.y], red[0] + red[1] + red[2] + red[3]);
+}
+
+// out[i, cols[j]] = rs[i] * constV[cols[j]] for the k columns that no group covers
+__global__ __launch_bounds__(256) void k_const_cols(const double* __restrict__ rs, const double* __restrict__ constV, const int32_t* __restrict__ cols,
+	int k, int p, double* __restrict__ out, int n, unsigned long long* __restrict__ nnz) {
+	int cnt = 0;
+	for(int idx = threadIdx.x + blockIdx.x * 256; idx < p * k; idx += 256 * gridDim.x) {
+		const int i = idx / k, c = cols[idx - i * k];
+		const double v = rs[i] * constV[c];
+		out[(size_t) i * n + c] = v;
+		cnt += v != 0.0;
+	}
+	if(cnt) atomicAdd(nnz, (unsigned long long) cnt);
+}
+
+// Cuts the block into chunks of whole groups of at most `width` columns, a block of its own each; the columns that
+// no group covers make a list of their own. 1 when a group is wider than that.
+static int build_lmm_subs(cla_block* b, int width) {
+	const int n = b->nCols, nG = (int) b->groups.size();
+	std::vector<char> covered((size_t) n, 0);
+	for(auto& g : b->groups)
+		for(int c : g.cols) covered[c] = 1;
+	std::vector<Chunk> chunks;
+	auto add_item = [&](int group, int w) -> bool {
+		if(w > width) return false;
+		if(chunks.empty() || chunks.back().nCols + w > width) chunks.emplace_back();
+		chunks.back().groups.push_back(group);
+		chunks.back().nCols += w;
+		return true;
+	};
+	for(int g = 0; g < nG; g++)
+		if(!add_item(g, b->groups[g].d.nColG)) return 1;
+	std::vector<int32_t> constOnly;
+	for(int c = 0; c < n; c++)
+		if(!covered[c]) constOnly.push_back(c);
+	const Chunk none;
+	for(size_t ci = 0; ci < chunks.size() + (constOnly.empty() ? 0 : 1); ci++) {
+		LmmSub* sb = new LmmSub();
+		sb->blk = nullptr; sb->dColMap = nullptr; sb->k = 0;
+		b->lmmSubs.push_back(sb);
+		std::vector<int32_t> colMap;
+		if(ci < chunks.size()) {
+			sb->blk = make_sub(b, chunks[ci], none, false, colMap);
+			if(!sb->blk) { free_lmm_subs(b); return -CLA_ERR_DEVICE; }
+		}
+		else colMap = constOnly;
+		sb->k = (int) colMap.size();
+		if(hipMalloc((void**) &sb->dColMap, sizeof(int32_t) * colMap.size()) != hipSuccess ||
+			hipMemcpy(sb->dColMap, colMap.data(), sizeof(int32_t) * colMap.size(), hipMemcpyHostToDevice) != hipSuccess) {
+			set_error("left multiply: column map of a column chunk could not be uploaded");
+			free_lmm_subs(b);
+			return -CLA_ERR_DEVICE;
+		}
+	}
+	return 0;
+}
+
+// Y %*% X chunk of columns by chunk on the decode kernel: blocks of more than 64 columns, or whose code tiles exceed
+// LDS together. The widest chunks that the kernel takes (64, 32, 16 columns) are kept with the block. Returns 1 when
+// no width fits or Y holds a value that is not finite, 0 when dOut holds the result and *dNnz its non-zero count.
+static int launch_lmm_chunked(cla_block* b, const double* dY, int p, double* dOut, unsigned long long* dNnz) {
+	if(b->lmmSubWidth < 0) return 1;
+	hipStream_t st = b->stream;
+	CLA_HIP(hipMemsetAsync(dNnz, 0, sizeof(unsigned long long), st));
+	int width = b->lmmSubWidth ? b->lmmSubWidth : 64;
+	for(;;) {
+		if(b->lmmSubs.empty()) {
+			const int rc = build_lmm_subs(b, width);
+			if(rc < 0) return rc;
+			if(rc == 1) { free_lmm_subs(b); b->lmmSubWidth = -1; return 1; }
+		}
+		bool fits = true;
+		for(void* q : b->lmmSubs) {
+			LmmSub* sb = (LmmSub*) q;
+			cla_block* c = sb->blk;
+			if(!c) { // row sums of Y for the columns that no group covers
+				int rc = ensure_tables(b, (size_t) p); // (the caller's dOut may be the block's output staging buffer)
+				if(rc) return rc;
+				CLA_HIP(hipMemsetAsync(b->dTables, 0, (size_t) p * sizeof(double), st));
+				int64_t rpb = 256 * 1024;
+				while(rpb > 8192 && (b->nRows + rpb - 1) / rpb * p < (int64_t) g_numCU * 2) rpb /= 2;
+				const dim3 grid((unsigned) ((b->nRows + rpb - 1) / rpb), (unsigned) p);
+				Prof pf(b, "k_y_rowsum", (long) grid.x * p, 256, 0, (double) b->nRows * p * 8);
+				hipLaunchKernelGGL(k_y_rowsum, grid, dim3(256), 0, st, dY, b->nRows, rpb, b->dTables);
+				continue;
+			}
+			c->profile = b->profile;
+			c->opt = b->opt;
+			if(c->stream != b->stream) {
+				if(c->ownStream && c->stream) { (void) hipStreamSynchronize(c->stream); (void) hipStreamDestroy(c->stream); }
+				c->stream = b->stream;
+				c->ownStream = false;
+			}
+			const int k = c->nCols;
+			const size_t n = (size_t) p * k;
+			int rc = ensure_stage(&c->dStageOut, &c->stageOutCap, n);
+			if(rc) return rc;
+			CLA_HIP(hipMemsetAsync(c->dStageOut, 0, n * sizeof(double), st));
+			for(int p0 = 0; p0 < p && fits; p0 += 16) { // 16 rows of Y per pass over the chunk
+				rc = launch_lmm_decode(c, dY + (size_t) p0 * b->nRows, std::min(16, p - p0), c->dStageOut + (size_t) p0 * k, dNnz);
+				if(rc < 0) return rc;
+				if(rc == 1) fits = false; // (the plan is the same for every pass: only the first can say so)
+			}
+			b->lastStats.insert(b->lastStats.end(), c->lastStats.begin(), c->lastStats.end());
+			c->lastStats.clear(); // (the events moved along)
+			if(!fits) break;
+		}
+		if(fits) break;
+		// (what the chunks in front of the one that does not fit have queued finishes on the stream before their blocks go)
+		CLA_HIP(hipStreamSynchronize(st));
+		clear_stats(b);
+		free_lmm_subs(b);
+		CLA_HIP(hipMemsetAsync(dNnz, 0, sizeof(unsigned long long), st));
+		if(width == 16) { b->lmmSubWidth = -1; return 1; }
+		width /= 2;
+	}
+	b->lmmSubWidth = width;
+	{
+		unsigned long long bad = 0; // (see launch_lmm_joint)
+		CLA_HIP(hipMemcpyAsync(&bad, dNnz, sizeof(bad), hipMemcpyDeviceToHost, st));
+		CLA_HIP(hipStreamSynchronize(st));
+		if(bad) { clear_stats(b); return 1; }
+	}
+	CLA_HIP(hipMemsetAsync(dNnz, 0, sizeof(unsigned long long), st));
+	for(void* q : b->lmmSubs) {
+		LmmSub* sb = (LmmSub*) q;
+		const int k = sb->k;
+		const int n = p * k;
+		if(!sb->blk) {
+			Prof pf(b, "k_const_cols", (n + 255) / 256, 256, 0, 0);
+			hipLaunchKernelGGL(k_const_cols, dim3((unsigned) std::min((n + 255) / 256, 1024)), dim3(256), 0, st, b->dTables, b->dConstV, sb->dColMap,
+				k, p, dOut, b->nCols, dNnz);
+			continue;
+		}
+		Prof pf(b, "k_scatter_cols", (n + 255) / 256, 256, 0, 0);
+		hipLaunchKernelGGL(k_scatter_cols, dim3((unsigned) std::min((n + 255) / 256, 1024)), dim3(256), 0, st, sb->blk->dStageOut, k, sb->dColMap, p,
+			dOut, b->nCols, dNnz);
+	}
+	CLA_HIP(hipGetLastError());
+	return 0;
+}
+
+// Y %*% X in passes over the decoded rows on the matrix cores, 16 rows of Y as the other operand of a pass
+// (k_lmm_decode), whatever the block's group mix, where the bin kernels take a pass per row of Y and group type
+// (C5, 50 M x 20: 2.0 - 2.35 ms for 1 to 16 rows of Y against 2.9 - 88 ms). Taken for blocks that the offset-list
+// kernels do not serve better and, for few rows of Y, the byte-code dot form neither; blocks of more than 64 columns
+// or with too many code tiles for LDS go chunk of columns by chunk. Returns 1 when the block is not eligible, 0 when
+// dOut (p x nCols) holds the result and *dNnz its non-zero count.
 int launch_lmm_joint(cla_block* b, const double* dY, int p, double* dOut, unsigned long long* dNnz) {
-	if(!b->opt.lmmJoint || !b->opt.tsmmMfma || p < 1 || b->nCols > 64 || b->nRows == 0 || b->crossSplit > 0) return 1;
+	if(!b->opt.lmmJoint || !b->opt.tsmmMfma || p < 1 || b->nRows == 0 || b->crossSplit > 0) return 1;
 	if(b->dictNonFinite) return 1; // (the reference sums Y per tuple first: an infinite dictionary value times Y of both signs is no NaN)
 	int nLists = 0, nOther = 0;
 	bool dotForm = b->dArena != nullptr && b->arenaWidth == 1 && b->maxVals <= 256;
@@ -1194,7 +1380,11 @@ int launch_lmm_joint(cla_block* b, const double* dY, int p, double* dOut, unsign
 				seen[c] = 1;
 			}
 	}
-	if(nOther == 0 || nLists > nOther || dotForm) return 1;
+	if(nOther == 0 || nLists > nOther) return 1;
+	// single-column byte codes: the dot kernel takes a pass per row of Y, a twelfth of what a pass of the decode kernel
+	// over 16 rows of Y costs (C2: 0.21 against 2.5 ms)
+	if(dotForm && (p + 15) / 16 * 12 >= p) return 1;
+	if(b->nCols > 64) return launch_lmm_chunked(b, dY, p, dOut, dNnz);
 	hipStream_t st = b->stream;
 	const size_t n = (size_t) p * b->nCols;
 	int rc = ensure_stage(&b->dStageOut, &b->stageOutCap, n);
@@ -1203,6 +1393,7 @@ int launch_lmm_joint(cla_block* b, const double* dY, int p, double* dOut, unsign
 	CLA_HIP(hipMemsetAsync(dNnz, 0, sizeof(unsigned long long), st));
 	for(int p0 = 0; p0 < p; p0 += 16) // 16 rows of Y per pass over the block
 		if((rc = launch_lmm_decode(b, dY + (size_t) p0 * b->nRows, std::min(16, p - p0), b->dStageOut + (size_t) p0 * b->nCols, dNnz))) {
+			if(rc == 1 && p0 == 0) return launch_lmm_chunked(b, dY, p, dOut, dNnz); // (nothing queued yet)
 			if(p0 > 0) clear_stats(b);
 			return rc;
 		}

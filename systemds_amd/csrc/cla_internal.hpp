@@ -116,6 +116,10 @@ struct cla_block {
 	// blocks of pairs of column chunks for t(X) %*% X on more than 64 columns (launch_tsmm_chunked): built on
 	// first use, they borrow this block's row data and are freed with it
 	std::vector<void*> subs;
+	// blocks of column chunks for Y %*% X on the decode kernel (launch_lmm_chunked), likewise; lmmSubWidth: columns
+	// per chunk they were cut for, 0 not tried yet, -1 no width fits
+	std::vector<void*> lmmSubs;
+	int lmmSubWidth = 0;
 	std::vector<cla::HostGroup> groups;
 	std::vector<double> constV;      // filtered constants (SDC defaults, const groups), nCols
 	bool hasConst = false;

@@ -258,3 +258,49 @@ def test_wide_dense_groups_on_the_matrix_cores(cla, ora, p):
     assert_matches_truth(out, Y, D, what=f"Y %*% X, dense groups, {p} rows")
     assert_fp64_close(out, ref, ora.abs_matmul(Y, D), what=f"Y %*% X, dense groups, {p} rows", n_terms=n_rows)
     assert nnz == rnnz
+
+
+@pytest.mark.parametrize("shape", ["bytes100", "words60", "mixed"])
+@pytest.mark.parametrize("p", [14, 40])
+def test_many_rows_of_y_in_chunks_of_columns(cla, ora, shape, p):
+    """Blocks that the decode kernel does not take whole go chunk of columns by chunk: 100 single-column byte-code
+    groups (the dot kernel serves few rows of Y), 60 columns of two-byte codes (their code tiles exceed LDS
+    together), about 100 columns of mixed groups with constant-only columns between them."""
+    from systemds_amd import synth
+    rng = np.random.default_rng(len(shape) + p)
+    n_rows = 30011
+    if shape == "bytes100":
+        n_cols = 100
+        specs = [synth.GroupSpec("ddc", np.array([c], np.int32), rng.standard_normal((50, 1)), rng.integers(0, 50, n_rows).astype(np.uint8))
+                 for c in range(n_cols)]
+    elif shape == "words60":
+        n_cols = 60
+        specs = [synth.GroupSpec("ddc", np.array([c], np.int32), rng.standard_normal((700, 1)), rng.integers(0, 700, n_rows).astype(np.uint16))
+                 for c in range(n_cols)]
+    else:
+        specs, n_cols = [], 0
+        for k in range(7):
+            part, m = mixed_block(50 + k, n_rows, with_unc=True, big_dict=False)
+            for g in part:
+                g.cols = (np.asarray(g.cols) + n_cols).astype(np.int32)
+            specs += part
+            n_cols += m + 2  # two columns that no group covers
+        specs.append(synth.GroupSpec("const", np.array([n_cols - 1], np.int32), np.array([[0.75]])))
+    Y = rng.standard_normal((p, n_rows))
+    D = ora.np_decompress(specs, n_rows, n_cols)
+    blk = cla.build_block(n_rows, n_cols, specs)
+    try:
+        out, nnz = blk.lmm(Y)
+        blk.profile(True)
+        out2, nnz2 = blk.lmm(Y)
+        names = [k["name"] for k in blk.stats()["kernels"]]
+        blk.profile(False)
+        blk.set_option("lmm_joint", 0)
+        bins, nnz_b = blk.lmm(Y)
+    finally:
+        blk.close()
+    assert "k_lmm_decode" in names and "k_scatter_cols" in names, (n_cols, names)
+    assert_matches_truth(out, Y, D, what=f"Y %*% X in column chunks, {shape}, {p} rows")
+    assert_matches_truth(out2, Y, D, what=f"Y %*% X in column chunks, {shape}, {p} rows, second call")
+    assert_matches_truth(bins, Y, D, what=f"Y %*% X, {shape}, {p} rows, bin kernels")
+    assert nnz == np.count_nonzero(out) and nnz2 == np.count_nonzero(out2) and nnz_b == np.count_nonzero(bins)
