@@ -487,6 +487,58 @@ __global__ __launch_bounds__(256) void k_gram_dense(const double* __restrict__ D
 	}
 }
 
+// The same for at most 16 NB columns with all tiles on or above the diagonal in one block: a row's values are loaded
+// once (NB loads for NB (NB + 1) / 2 matrix instructions) where the kernel above loads them once per column block of
+// the grid (4M x 60: 1.75 ms there).
+template <int NB>
+__global__ __launch_bounds__(256) void k_gram_dense_all(const double* __restrict__ D, int64_t nRows, int nCols, int64_t rowsPerBlock,
+	double* __restrict__ out) {
+	constexpr int NT = NB * (NB + 1) / 2;
+	__shared__ double red[NT * 256];
+	const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+	const int i16 = lane & 15, k4 = lane >> 4;
+	const int64_t r0 = (int64_t) blockIdx.x * rowsPerBlock, r1 = min(nRows, r0 + rowsPerBlock);
+	gd_f64x4 acc[NT];
+#pragma unroll
+	for(int t = 0; t < NT; t++) acc[t] = gd_f64x4{0.0, 0.0, 0.0, 0.0};
+#pragma unroll 2
+	for(int64_t r = r0 + wave * 4; r < r1; r += 16) {
+		const int64_t row = r + k4;
+		const bool in = row < r1;
+		const double* drow = D + (size_t) (in ? row : r0) * nCols;
+		double v[NB];
+#pragma unroll
+		for(int c = 0; c < NB; c++) {
+			const int col = c * 16 + i16;
+			v[c] = in && col < nCols ? drow[col] : 0.0;
+		}
+		int t = 0;
+#pragma unroll
+		for(int i = 0; i < NB; i++)
+#pragma unroll
+			for(int j = i; j < NB; j++) {
+				acc[t] = __builtin_amdgcn_mfma_f64_16x16x4f64(v[i], v[j], acc[t], 0, 0, 0);
+				t++;
+			}
+	}
+	for(int i = tid; i < NT * 256; i += 256) red[i] = 0.0;
+	__syncthreads();
+#pragma unroll
+	for(int t = 0; t < NT; t++)
+#pragma unroll
+		for(int v = 0; v < 4; v++) unsafeAtomicAdd(&red[t * 256 + (4 * v + k4) * 16 + i16], acc[t][v]);
+	__syncthreads();
+	int t = 0;
+	for(int i = 0; i < NB; i++)
+		for(int j = i; j < NB; j++) {
+			const int rr = tid >> 4, cc = tid & 15;
+			const int gr = i * 16 + rr, gc = j * 16 + cc;
+			const double s = red[t * 256 + tid];
+			if(gr <= gc && gc < nCols && s != 0.0) unsafeAtomicAdd(&out[(size_t) gr * nCols + gc], s);
+			t++;
+		}
+}
+
 // dOut (zeroed) = t(X) %*% X through the decompressed block. -CLA_ERR_UNSUPPORTED when the dense copy does
 // not fit the free device memory.
 static int launch_tsmm_decompressed(cla_block* b, double* dOut, unsigned long long* dNnz, const char* why) {
@@ -506,6 +558,16 @@ static int launch_tsmm_decompressed(cla_block* b, double* dOut, unsigned long lo
 			const int64_t rows = std::min(rowsPerChunk, nRows - r0);
 			if((rc = launch_decompress_rows(b, r0, r0 + rows, dense))) return rc;
 			int64_t rowsPerBlock = 16384;
+			if(nb <= 4) { // all tiles of a range of rows in one block
+				while(rowsPerBlock > 1024 && (rows + rowsPerBlock - 1) / rowsPerBlock < (int64_t) g_numCU * 4) rowsPerBlock /= 2;
+				const unsigned grid = (unsigned) ((rows + rowsPerBlock - 1) / rowsPerBlock);
+				Prof pf(b, "k_gram_dense", grid, 256, 0, (double) rows * nCols * 8);
+				if(nb == 1) hipLaunchKernelGGL(k_gram_dense_all<1>, dim3(grid), dim3(256), 0, st, dense, rows, nCols, rowsPerBlock, dOut);
+				else if(nb == 2) hipLaunchKernelGGL(k_gram_dense_all<2>, dim3(grid), dim3(256), 0, st, dense, rows, nCols, rowsPerBlock, dOut);
+				else if(nb == 3) hipLaunchKernelGGL(k_gram_dense_all<3>, dim3(grid), dim3(256), 0, st, dense, rows, nCols, rowsPerBlock, dOut);
+				else hipLaunchKernelGGL(k_gram_dense_all<4>, dim3(grid), dim3(256), 0, st, dense, rows, nCols, rowsPerBlock, dOut);
+				continue;
+			}
 			while(rowsPerBlock > 1024 && (rows + rowsPerBlock - 1) / rowsPerBlock * nb < (int64_t) g_numCU * 4) rowsPerBlock /= 2;
 			const dim3 grid((unsigned) ((rows + rowsPerBlock - 1) / rowsPerBlock), (unsigned) nb, (unsigned) ((nb + GD_NBJ - 1) / GD_NBJ));
 			Prof pf(b, "k_gram_dense", (long) grid.x * grid.y * grid.z, 256, 0, (double) rows * nCols * 8);
