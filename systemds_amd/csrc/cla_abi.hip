@@ -639,6 +639,16 @@ int finish_finalize(cla_block* b, cla_block* arenaFrom, bool buildArena) {
 		// a thread stages at most 16 table values (Q1_TPT) for the next slab; the smallest block has 256 threads
 		per = std::min(per, 16 * 256 / mx);
 		per = per / 8 * 8;
+		b->q1Threads = 256;
+		if(per < 8) { // large dictionaries: two blocks of 512 threads per CU with half of its LDS each, else one of 1024 threads
+			const int all = std::min(g_ldsPerBlock, 160 * 1024) - 8 * 1024;
+			per = std::min(all / 2 / (mx * 8) - 1, 16 * 512 / mx) / 8 * 8;
+			if(per >= 8) b->q1Threads = 512;
+			else {
+				per = std::min(all / (mx * 8) - 1, 16 * 1024 / mx) / 8 * 8;
+				if(per >= 8) b->q1Threads = 1024;
+			}
+		}
 		if(nG > 0 && per >= 8) {
 			for(size_t i = 0; i < nG; i += per) {
 				const size_t j = std::min(nG, i + (size_t) per);

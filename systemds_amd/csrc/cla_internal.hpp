@@ -149,6 +149,7 @@ struct cla_block {
 	std::vector<int4> q1Slabs;
 	int4* dQ1Slabs = nullptr;
 	int32_t q1LdsBytes = 0;
+	int32_t q1Threads = 256;         // threads per block of k_rmm_q1_ddc: 512 or 1024 where only then 8 tables fit a slab
 
 	// reusable workspaces
 	double* dTables = nullptr;  size_t tablesCap = 0;

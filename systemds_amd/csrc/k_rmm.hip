@@ -616,7 +616,7 @@ int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned lon
 	}
 	if(q == 1 && b->dArena && b->q1LdsBytes > 0) {
 		const int cw = b->arenaWidth;
-		const int threads = 256, rpt = cw == 4 ? 8 : 16;
+		const int threads = b->q1Threads, rpt = cw == 4 ? 8 : 16;
 		const int64_t rowsPerBlock = (int64_t) threads * rpt;
 		const unsigned grid = (unsigned) ((nRows + rowsPerBlock - 1) / rowsPerBlock);
 		const int nSlabs = (int) b->q1Slabs.size();

@@ -503,3 +503,26 @@ def test_wide_right_multiply_in_passes_of_the_tile_kernel(cla, ora, q):
     assert names.count("k_rmm_decode") == (q + 15) // 16, names
     assert_matches_truth(out, D, B, what=f"tile passes q={q}")
     assert nnz == np.count_nonzero(out)
+
+
+@pytest.mark.parametrize("n_vals,n_groups", [(1000, 20), (1900, 11)])
+def test_mat_vec_on_two_byte_codes_with_large_dictionaries(cla, ora, n_vals, n_groups):
+    """Single-column DDC groups with two-byte codes whose tables fit a slab of 8 only in blocks of 512 threads (1000
+    values) or 1024 threads (1900 values): X %*% v stays on the slab kernel with its tables in LDS."""
+    from systemds_amd import synth
+    rng = np.random.default_rng(n_vals)
+    n_rows = 70003
+    specs = [synth.GroupSpec("ddc", np.array([c], np.int32), rng.standard_normal((n_vals, 1)), rng.integers(0, n_vals, n_rows).astype(np.uint16))
+             for c in range(n_groups)]
+    v = rng.standard_normal((n_groups, 1))
+    D = ora.np_decompress(specs, n_rows, n_groups)
+    blk = cla.build_block(n_rows, n_groups, specs)
+    try:
+        blk.profile(True)
+        out, nnz = blk.rmm(v)
+        names = [k["name"] for k in blk.stats()["kernels"]]
+    finally:
+        blk.close()
+    assert "k_rmm_q1_ddc" in names, names
+    assert_matches_truth(out, D, v, what=f"X %*% v, {n_vals} values per column")
+    assert nnz == np.count_nonzero(out)
