@@ -111,7 +111,8 @@ int cla_block_set_stream(cla_handle h, void* hipStream);
  *   tsmm_wide_dense 0 / 1, tsmm_mfma 1 / 0, tsmm_pair_dot 1 / 0
  *   tsmm_narrow     1 / 0: decoded Gram matrix with a last column block of at most 4 columns on the 4x4x4 matrix instruction
  *   expand_streams  1 / 0: one code per row for small RLE / SDCZeros groups (set before the first multiply)
- *   rmm_disable     bit 0 byte-code mat-vec kernel, 1 its fused tables, 2 matrix-core kernel, 3 decode kernel
+ *   rmm_disable     bit 0 byte-code mat-vec kernel, 1 its fused tables, 2 matrix-core kernel, 3 decode kernels (tile, stream and
+ *                   the decompressed rows times a wide B)
  *   rmm_direct      1 / 0: X %*% B on blocks of plain streams with codes read straight from global memory, 16 columns of B per pass
  *                   (0: at most 16 columns of B on the tile kernel on the matrix cores, wider B per row and group)
  *   lmm_disable     bit 0 dot form on byte codes, bit 1 byte-code bin kernel

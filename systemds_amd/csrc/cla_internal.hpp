@@ -250,6 +250,7 @@ int launch_rmm_decode(cla_block* b, const double* dB, int q, const double* dCons
 	unsigned long long* dNnz);
 int launch_decompress(cla_block* b, double* dOut, unsigned long long* dNnz);
 int launch_decompress_rows(cla_block* b, int64_t r0, int64_t r1, double* dOut);
+int launch_rmm_decompressed(cla_block* b, const double* dB, int q, double* dOut, unsigned long long* dNnz);
 void dec_plans_drop(cla_block* b);
 int tsmm_decode_fits(cla_block* b);
 int launch_lmm_decode(cla_block* b, const double* dY, int p, double* dOut, unsigned long long* dBad);

@@ -676,6 +676,13 @@ int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned lon
 		if(r <= 0) return r;
 	}
 
+	// wide B on a block that none of the kernels above takes: decompressed chunks of rows times B on the matrix cores
+	// where that moves fewer bytes than the gather below (as a decoding kernel it multiplies every decoded value)
+	if(q >= 16 && !squares && !noAlloc && !(b->opt.rmmDisable & 8)) {
+		const int r = launch_rmm_decompressed(b, dB, q, dOut, dNnz);
+		if(r <= 0) return r;
+	}
+
 	// generic path: row-parallel gather for DDC / RLE / uncompressed groups, then the
 	// SDCZeros groups tile by tile (or per-entry scatter when their tables do not fit LDS)
 	{

@@ -936,9 +936,11 @@ __global__ __launch_bounds__(DCT_THREADS) void k_decompress_tiles(const DGroup* 
 
 // rows [r0, r1) of the group go to out rows 0 .. r1 - r0; a block of list entries whose rows all lie outside leaves early
 template <int W>
-__global__ __launch_bounds__(256) void k_decompress_sdc(const DGroup* __restrict__ groups, int g, int64_t r0, int64_t r1, int nCols,
+__global__ __launch_bounds__(256) void k_decompress_sdc(const DGroup* __restrict__ groups, int64_t r0, int64_t r1, int nCols,
 	double* __restrict__ out) {
-	const DGroup G = dgroup(groups + (g));
+	// one launch for all offset lists with entries of W bytes (a launch per list: 5 us of work behind 6 us of launch)
+	const DGroup G = dgroup(groups + blockIdx.y);
+	if(G.type != G_SDCZ || G.deltaWidth != W || G.nOffsets == 0) return;
 	const int chunk = blockIdx.x, wave = threadIdx.x >> 6;
 	if(chunk == 0 && threadIdx.x == 0 && G.nOffsets > 0 && G.first >= r0 && G.first < r1) {
 		const int code = load_code(G.codes, G.codeWidth, 0);
@@ -1014,15 +1016,12 @@ int launch_decompress_rows(cla_block* b, int64_t r0, int64_t r1, double* dOut) {
 		Prof pf(b, "k_decompress_fill", fg, 256, 0, 0);
 		hipLaunchKernelGGL(k_decompress_fill, dim3(fg), dim3(256), 0, st, dOut, n, b->nCols, b->dConstV);
 	}
+	int maxCkpt[3] = {0, 0, 0}; // offset lists by entry width
 	for(int g = 0; g < nG; g++) {
 		const DGroup& G = b->groups[g].d;
 		if(G.type != G_SDCZ && tiled) continue;
 		if(G.type == G_SDCZ) {
-			if(G.nOffsets == 0) continue;
-			const unsigned sg = (unsigned) std::max(G.nCkpt, 1);
-			Prof pf(b, "k_decompress_sdc", sg, 256, 0, 0);
-			if(G.deltaWidth == 1) hipLaunchKernelGGL(k_decompress_sdc<1>, dim3(sg), dim3(256), 0, st, b->dGroups, g, r0, r1, b->nCols, dOut);
-			else hipLaunchKernelGGL(k_decompress_sdc<2>, dim3(sg), dim3(256), 0, st, b->dGroups, g, r0, r1, b->nCols, dOut);
+			if(G.nOffsets > 0) maxCkpt[G.deltaWidth == 1 ? 1 : 2] = std::max(maxCkpt[G.deltaWidth == 1 ? 1 : 2], std::max(G.nCkpt, 1));
 		}
 		else {
 			const int64_t m = (r1 - r0) * G.nColG;
@@ -1030,6 +1029,133 @@ int launch_decompress_rows(cla_block* b, int64_t r0, int64_t r1, double* dOut) {
 			Prof pf(b, "k_decompress_rows", (long) ((m + 255) / 256), 256, 0, 0);
 			hipLaunchKernelGGL(k_decompress_rows, dim3((unsigned) ((m + 255) / 256)), dim3(256), 0, st, b->dGroups, g, r0, r1,
 				b->nCols, dOut);
+		}
+	}
+	if(maxCkpt[1] > 0) {
+		Prof pf(b, "k_decompress_sdc", (long) maxCkpt[1] * nG, 256, 0, 0);
+		hipLaunchKernelGGL(k_decompress_sdc<1>, dim3((unsigned) maxCkpt[1], (unsigned) nG), dim3(256), 0, st, b->dGroups, r0, r1, b->nCols, dOut);
+	}
+	if(maxCkpt[2] > 0) {
+		Prof pf(b, "k_decompress_sdc", (long) maxCkpt[2] * nG, 256, 0, 0);
+		hipLaunchKernelGGL(k_decompress_sdc<2>, dim3((unsigned) maxCkpt[2], (unsigned) nG), dim3(256), 0, st, b->dGroups, r0, r1, b->nCols, dOut);
+	}
+	CLA_HIP(hipGetLastError());
+	return 0;
+}
+
+// ---------------------------------------------------------------------------
+// out[rows x qv] = D[rows x m] %*% B[m x qv] for a dense row-major D (decompressed rows) on v_mfma_f64_16x16x4_f64.
+// A wave takes tiles of 16 rows: lane (k4, i16) reads the four values D[row i16, 16 kk + 4 k4 ..+3] in one piece
+// (16 lanes = one or two whole lines of the row) and feeds them to four instructions, whose other operand is
+// B[16 kk + 4 k4 + s, 16 jt + i16] from the block's LDS copy of B (row stride 16 NQ + 4 doubles: the four rows that a
+// wave reads together fall into different halves of the banks). Register v of the result is cell (4 v + k4, i16).
+// ---------------------------------------------------------------------------
+typedef double dg_f64x4u __attribute__((ext_vector_type(4), aligned(8)));
+template <int NQ>
+__global__ __launch_bounds__(256) void k_dense_rmm(const double* __restrict__ D, int64_t nRows, int m, const double* __restrict__ B, int ldb,
+	int qv, double* __restrict__ out, int ldo, unsigned long long* __restrict__ nnz) {
+	extern __shared__ __align__(16) double dgB[];
+	constexpr int LD = 16 * NQ + 4;
+	const int mPad = (m + 15) & ~15;
+	const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+	const int i16 = lane & 15, k4 = lane >> 4;
+	for(int i = tid; i < mPad * 16 * NQ; i += 256) {
+		const int k = i / (16 * NQ), j = i - k * (16 * NQ);
+		dgB[k * LD + j] = k < m && j < qv ? B[(size_t) k * ldb + j] : 0.0;
+	}
+	__syncthreads();
+	int cnt = 0;
+	const int64_t nTiles = (nRows + 15) / 16;
+	for(int64_t t = (int64_t) blockIdx.x * 4 + wave; t < nTiles; t += (int64_t) gridDim.x * 4) {
+		const int64_t r0 = t * 16;
+		const double* drow = D + (size_t) min(r0 + i16, nRows - 1) * m; // (rows past the end: computed, not stored)
+		gd_f64x4 acc[NQ];
+#pragma unroll
+		for(int jt = 0; jt < NQ; jt++) acc[jt] = gd_f64x4{0.0, 0.0, 0.0, 0.0};
+#pragma unroll 2
+		for(int kk = 0; kk < mPad; kk += 16) {
+			const int kb = kk + 4 * k4;
+			double a[4];
+			if(kb + 3 < m) {
+				const dg_f64x4u v = *(const dg_f64x4u*) (drow + kb);
+				a[0] = v.x; a[1] = v.y; a[2] = v.z; a[3] = v.w;
+			}
+			else {
+#pragma unroll
+				for(int s = 0; s < 4; s++) a[s] = kb + s < m ? drow[kb + s] : 0.0;
+			}
+#pragma unroll
+			for(int s = 0; s < 4; s++)
+#pragma unroll
+				for(int jt = 0; jt < NQ; jt++)
+					acc[jt] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[s], dgB[(kb + s) * LD + jt * 16 + i16], acc[jt], 0, 0, 0);
+		}
+#pragma unroll
+		for(int jt = 0; jt < NQ; jt++)
+#pragma unroll
+			for(int v = 0; v < 4; v++) {
+				const int64_t r = r0 + 4 * v + k4;
+				const int c = jt * 16 + i16;
+				if(r < nRows && c < qv) {
+					out[(size_t) r * ldo + c] = acc[jt][v];
+					cnt += acc[jt][v] != 0.0;
+				}
+			}
+	}
+	__shared__ int part[4];
+	cnt = wave_sum_i32(cnt);
+	if(lane == 0) part[wave] = cnt;
+	__syncthreads();
+	if(tid == 0) {
+		const int s = part[0] + part[1] + part[2] + part[3];
+		if(s) atomicAdd(nnz, (unsigned long long) s);
+	}
+}
+
+// X %*% B through decompressed chunks of rows (at most 512 MiB in the block's scratch buffer) for blocks that only the
+// gather kernels per row and group would take, where B is wide: those move a table row of q values per group and row
+// (or list entry) through L2, this a dense row per row. dOut (nRows x q) and *dNnz (cleared by the caller) are
+// written. Returns 1 when the gather kernels are expected to be faster or the block is too wide for B in LDS.
+int launch_rmm_decompressed(cla_block* b, const double* dB, int q, double* dOut, unsigned long long* dNnz) {
+	const int m = b->nCols;
+	const int64_t nRows = b->nRows;
+	if(m > 256 || q < 16 || nRows == 0) return 1;
+	int64_t rowsPerChunk = std::max<int64_t>((int64_t) 512 * 1024 * 1024 / ((int64_t) m * 8) / 1024 * 1024, 1024);
+	rowsPerChunk = std::min(rowsPerChunk, (nRows + 1023) / 1024 * 1024);
+	const int64_t nChunks = (nRows + rowsPerChunk - 1) / rowsPerChunk;
+	{
+		// gather kernels: (list entries + rows x other groups) table rows of q values at about 1.5 TB/s (measured 1.45 -
+		// 2.2); here the dense rows written, read for the lists and read again at about 1 TB/s together (0.9 - 1.3)
+		double entries = 0.0, lists = 0.0;
+		for(auto& g : b->groups) {
+			if(g.d.type == G_SDCZ) { entries += (double) g.d.nOffsets; lists += g.d.nOffsets > 0; }
+			else entries += (double) nRows;
+		}
+		const double gather = entries * q * 8 / 1.5e12;
+		const double dense = (double) nRows * m * 8 / 1.0e12 + (double) nRows * q * 8 / 4e12 + (20e-6 + lists * 1e-6) * (double) nChunks;
+		if(gather <= dense) return 1;
+	}
+	int rc = ensure_scratch(b, sizeof(double) * (size_t) rowsPerChunk * m);
+	if(rc) return rc;
+	double* dense = (double*) b->dScratch;
+	hipStream_t st = b->stream;
+	const int mPad = (m + 15) & ~15;
+	for(int64_t r0 = 0; r0 < nRows; r0 += rowsPerChunk) {
+		const int64_t rows = std::min(rowsPerChunk, nRows - r0);
+		if((rc = launch_decompress_rows(b, r0, r0 + rows, dense))) return rc;
+		const unsigned grid = (unsigned) std::min<int64_t>(((rows + 15) / 16 + 3) / 4, (int64_t) g_numCU * 8);
+		for(int c0 = 0; c0 < q; c0 += 64) {
+			const int qv = std::min(64, q - c0), nq = (qv + 15) / 16;
+			const size_t lds = (size_t) mPad * (16 * nq + 4) * 8;
+			Prof pf(b, "k_dense_rmm", grid, 256, (long) lds, (double) rows * (m + qv) * 8);
+#define DG_LAUNCH(NQV)                                                                                          \
+	do {                                                                                                        \
+		CLA_HIP(allow_full_lds((const void*) k_dense_rmm<NQV>));                                                \
+		hipLaunchKernelGGL(k_dense_rmm<NQV>, dim3(grid), dim3(256), lds, st, dense, rows, m, dB + c0, q, qv,    \
+			dOut + (size_t) r0 * q + c0, q, dNnz);                                                              \
+	} while(0)
+			if(nq == 1) DG_LAUNCH(1); else if(nq == 2) DG_LAUNCH(2); else if(nq == 3) DG_LAUNCH(3); else DG_LAUNCH(4);
+#undef DG_LAUNCH
 		}
 	}
 	CLA_HIP(hipGetLastError());

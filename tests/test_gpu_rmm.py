@@ -526,3 +526,33 @@ def test_mat_vec_on_two_byte_codes_with_large_dictionaries(cla, ora, n_vals, n_g
     assert "k_rmm_q1_ddc" in names, names
     assert_matches_truth(out, D, v, what=f"X %*% v, {n_vals} values per column")
     assert nnz == np.count_nonzero(out)
+
+
+@pytest.mark.parametrize("q", [56, 64, 70])
+def test_wide_right_multiply_through_decompressed_rows(cla, ora, q):
+    """A block that is mostly offset lists (12 lists beside 4 DDC columns; the tile kernel does not take it) with a
+    wide B: decompressed chunks of rows times B on the matrix cores (`k_dense_rmm`; 200,003 rows: a ragged last tile of
+    16 rows, 70 columns of B: a second pass of 6 columns); with the decoding kernels off the gather kernels give the
+    same cells."""
+    from systemds_amd import synth
+    rng = np.random.default_rng(q)
+    n_rows, n_cols = 200003, 16
+    specs = [synth.sdc_group(rng, n_rows, np.array([c], np.int32), 9, 0.1, 0.5 if c % 2 else None) for c in range(12)]
+    specs += [synth.GroupSpec("ddc", np.array([12 + c], np.int32), rng.standard_normal((40, 1)), rng.integers(0, 40, n_rows).astype(np.uint8))
+              for c in range(4)]
+    B = rng.standard_normal((n_cols, q))
+    D = ora.np_decompress(specs, n_rows, n_cols)
+    blk = cla.build_block(n_rows, n_cols, specs)
+    try:
+        blk.profile(True)
+        out, nnz = blk.rmm(B)
+        names = [k["name"] for k in blk.stats()["kernels"]]
+        blk.profile(False)
+        blk.set_option("rmm_disable", 12)
+        gather, nnz_g = blk.rmm(B)
+    finally:
+        blk.close()
+    assert "k_dense_rmm" in names and "k_rmm_rows" not in names, names
+    assert_matches_truth(out, D, B, what=f"X %*% B through decompressed rows, {q} columns")
+    assert_matches_truth(gather, D, B, what=f"X %*% B, gather kernels, {q} columns")
+    assert nnz == np.count_nonzero(out) and nnz_g == np.count_nonzero(gather)
