@@ -191,6 +191,13 @@ struct SubBlock {
 	bool writeA, writeB, crossOnly;
 };
 
+// One chunk of columns of Y %*% X on the decode kernel (launch_lmm_chunked), likewise.
+struct LmmSub {
+	cla_block* blk;   // null: the columns that no group covers (row sums of Y times their constants)
+	int32_t* dColMap; // column of the block per column of blk
+	int k;
+};
+
 int finish_finalize(cla_block* b, cla_block* arenaFrom, bool buildArena = true);
 static void free_subs(cla_block* b);
 static void free_lmm_subs(cla_block* b);
@@ -742,6 +749,7 @@ int64_t cla_block_derived_bytes(cla_handle b) {
 	int64_t s = b->derivedBytes;
 	if(b->joint) s += b->joint->derivedBytes;
 	for(void* p : b->subs) s += ((SubBlock*) p)->blk ? ((SubBlock*) p)->blk->derivedBytes : 0;
+	for(void* p : b->lmmSubs) s += ((LmmSub*) p)->blk ? ((LmmSub*) p)->blk->derivedBytes : 0;
 	return s;
 }
 
@@ -1186,11 +1194,6 @@ int launch_tsmm_chunked(cla_block* b, double* dOut) {
 }
 
 // ---- Y %*% X on the decode kernel
-struct LmmSub {
-	cla_block* blk;   // null: the columns that no group covers (row sums of Y times their constants)
-	int32_t* dColMap; // column of the block per column of blk
-	int k;
-};
 
 static void free_lmm_subs(cla_block* b) {
 	for(void* p : b->lmmSubs) {
