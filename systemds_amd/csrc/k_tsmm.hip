@@ -929,7 +929,13 @@ __global__ __launch_bounds__(DCT_THREADS) void k_decompress_tiles(const DGroup* 
 		}
 		__syncthreads();
 		double* o = out + (size_t) (t0 - r0) * nCols;
-		for(int i = tid; i < cells; i += DCT_THREADS) o[i] = dtile[i];
+		if(((uintptr_t) o & 15) == 0) { // 16 bytes per lane
+			typedef double dct_f64x2 __attribute__((ext_vector_type(2)));
+			for(int i = tid; i < (cells >> 1); i += DCT_THREADS) ((dct_f64x2*) o)[i] = ((const dct_f64x2*) dtile)[i];
+			if((cells & 1) && tid == 0) o[cells - 1] = dtile[cells - 1];
+		}
+		else
+			for(int i = tid; i < cells; i += DCT_THREADS) o[i] = dtile[i];
 		__syncthreads();
 	}
 }
