@@ -93,20 +93,6 @@ def build_c_driver(verbose=True):
     return C_DRIVER
 
 
-PROBE = os.path.join(HERE, "cla_probe")
-
-
-def build_probe(verbose=True):
-    """The device probe (probe/cla_probe.hip): a stand-alone executable, not part of the library."""
-    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc, "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-           os.path.join(HERE, "probe", "cla_probe.hip"), "-o", PROBE]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    subprocess.run(cmd, check=True)
-    return PROBE
-
-
 def build_jni(verbose=True):
     """The JNI shim (jni/cla_jni.c) when a JDK is present ($JAVA_HOME/include/jni.h); returns None otherwise."""
     jh = os.environ.get("JAVA_HOME")
@@ -127,6 +113,5 @@ if __name__ == "__main__":
     if "--no-host" not in sys.argv:
         build_host()
         build_c_driver()
-        build_probe()
         build_jni()
     sys.exit(0)
