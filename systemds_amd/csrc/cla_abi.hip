@@ -703,6 +703,7 @@ int cla_block_set_option(cla_handle b, const char* key, int32_t value) {
 		{"tsmm_route", &Options::tsmmRoute, 0, 2},         {"tsmm_chunks", &Options::tsmmChunks, 0, 1},
 		{"tsmm_wide_dense", &Options::tsmmWideDense, 0, 1}, {"tsmm_mfma", &Options::tsmmMfma, 0, 1},
 		{"tsmm_pair_dot", &Options::tsmmPairDot, 0, 1},     {"rmm_direct", &Options::rmmDirect, 0, 1},
+		{"tsmm_direct", &Options::tsmmDirect, 0, 1},
 		{"tsmm_narrow", &Options::tsmmNarrow, 0, 1},     {"expand_streams", &Options::expandStreams, 0, 1},
 		{"rmm_disable", &Options::rmmDisable, 0, 15},       {"lmm_disable", &Options::lmmDisable, 0, 3},
 		{"sdc_packed", &Options::sdcPacked, 0, 1},

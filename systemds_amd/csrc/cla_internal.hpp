@@ -72,6 +72,7 @@ struct Options {
 	int tsmmNarrow = 1;     // decoded Gram matrix: a last column block of at most 4 columns on the 4 x 4 x 4 matrix instruction
 	int tsmmPairDot = 1;    // DDC x DDC pairs in dot form (0: pre-aggregate form with LDS bins)
 	int expandStreams = 1;  // one code per row for small RLE / SDCZeros groups in the decode kernels
+	int tsmmDirect = 1;     // decoded Gram matrix of blocks with few columns besides run-length columns on the vector unit, run-length columns by run (0: the tile kernel on the matrix cores)
 	int rmmDirect = 1;      // X %*% B for narrow B on blocks of plain streams: codes straight from global memory, sums on the vector unit (0: the tile kernel on the matrix cores)
 	int rmmDisable = 0;     // bit 0 byte-code mat-vec, 1 fused tables of the byte-code mat-vec, 2 matrix-core kernel, 3 decode kernel
 	int lmmDisable = 0;     // bit 0 dot form on byte codes, 1 byte-code bin kernel
@@ -91,6 +92,7 @@ struct KernelStat {
 
 struct DecPlanCache;
 struct DirPlan;
+struct GdrPlan;
 
 } // namespace cla
 
@@ -181,6 +183,7 @@ struct cla_block {
 	bool laneLmm = false;            // every listed group has one column (the left multiply's condition)
 	cla::DecPlanCache* decPlans = nullptr; // decode kernels (k_rmm_decode.hip): plans per product shape, dropped by dec_plans_drop
 	cla::DirPlan* dirPlan = nullptr;     // plan of k_rmm_direct (dropped with the decode plans)
+	cla::GdrPlan* gdrPlan = nullptr;     // plan of k_tsmm_direct (likewise)
 	void* dMfPlan = nullptr;         // matrix-core right multiply (k_rmm_mfma.hip): slab descriptors, column info, code streams, B row list
 	int mfState = 0;                 // 0 not planned yet, 1 ready, -1 not eligible
 	int mfNSlabs = 0, mfNColsAll = 0, mfWidth = 1, mfMaxKc = 0, mfNRowCol = 0, mfMaxDict = 0;
@@ -246,6 +249,8 @@ int launch_rmm_sdc_lanes(cla_block* b, int constRow, int accumulate, double* dOu
 int launch_rmm_sdc_rows(cla_block* b, int constRow, int accumulate, double* dOut, unsigned long long* dNnz);
 int launch_rmm_sdc_tiles(cla_block* b, int q, int constRow, int accumulate, double* dOut, unsigned long long* dNnz);
 int launch_tsmm_decode(cla_block* b, double* dOut);
+int launch_tsmm_direct(cla_block* b, double* dOut);
+int ensure_expanded(cla_block* b);
 int launch_rmm_decode(cla_block* b, const double* dB, int q, const double* dConstRow, double* dOut,
 	unsigned long long* dNnz);
 int launch_decompress(cla_block* b, double* dOut, unsigned long long* dNnz);

@@ -1,0 +1,118 @@
+// Run cursors: how a wave that walks consecutive rows follows the run-length columns of a block without
+// looking any row up. A run-length column (one column of a ColGroupRLE, CG/ColGroupRLE.java:104-141) is
+// constant over a run, and a run is long against the 64 rows a wave handles per step, so the wave keeps per
+// column the current value and the row where its run ends and only acts where a run ends inside its step.
+// Lane RC_LANE0 + a of the wave is the cursor of run-length column a; a window of the next RC_WIN runs of
+// every column sits in LDS and is refilled (run ends, codes, dictionary values: three dependent loads) only
+// when a cursor leaves it.
+#pragma once
+#include "cla_device.hpp"
+
+namespace cla {
+
+constexpr int RC_MAX = 8;     // run-length columns a wave follows
+constexpr int RC_WIN = 8;     // runs per column in the wave's window (RC_MAX * RC_WIN = 64 lanes refill it)
+constexpr int RC_LANE0 = 16;  // first cursor lane
+constexpr int32_t RC_NEVER = 0x7fffffff;
+
+struct RunCol {
+	const int32_t* runStart;  // nRuns + 1 run starts of the merged run table (last = nRows)
+	const int32_t* runCode;   // tuple per run, -1 = rows that no run covers
+	const double* dict;       // nVals x nC
+	double add;               // added to every value of the column (its constant where the caller wants decoded cells)
+	int32_t nRuns, nC, h;     // h: the column's place in a tuple
+	int32_t col;              // column of the matrix
+};
+
+// Same-wave LDS traffic is ordered by the hardware; this keeps the compiler from moving accesses across.
+__device__ __forceinline__ void wave_lds_sync() {
+	__builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+	__builtin_amdgcn_wave_barrier();
+	__builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+struct RunCursors {
+	int32_t j;     // cursor lanes: run the column is in
+	int32_t jw;    // cursor lanes: run in slot 0 of the column's window
+	int32_t end;   // cursor lanes: first row behind the run; RC_NEVER on all other lanes and behind the last run
+	double val;    // cursor lanes: the column's value on the run
+	const RunCol* cols;
+	int nR;
+	int32_t* winEnd;   // RC_MAX * RC_WIN, wave-private LDS
+	double* winVal;
+
+	// Window slot (a, k) = run jw_a + k of column a, loaded by lane 8 a + k.
+	__device__ __forceinline__ void refill(int lane) {
+		const int a = lane >> 3, k = lane & 7;
+		const int jb = __shfl(j, RC_LANE0 + a, WAVE);
+		int32_t e = RC_NEVER;
+		double v = 0.0;
+		if(a < nR) {
+			const RunCol* C = as_global(cols + a);
+			const int jj = jb + k;
+			if(jj < C->nRuns) {
+				e = as_global(C->runStart)[jj + 1];
+				const int code = as_global(C->runCode)[jj];
+				v = C->add + (code < 0 ? 0.0 : as_global(C->dict)[(size_t) code * C->nC + C->h]);
+			}
+		}
+		wave_lds_sync();
+		winEnd[lane] = e;
+		winVal[lane] = v;
+		wave_lds_sync();
+		jw = j;
+	}
+
+	__device__ __forceinline__ void read_window(int lane) {
+		const int a = lane - RC_LANE0;
+		if(a >= 0 && a < nR) {
+			end = winEnd[a * RC_WIN + (j - jw)];
+			val = winVal[a * RC_WIN + (j - jw)];
+		}
+	}
+
+	// Cursors at row r0 (every column's run that holds r0).
+	__device__ __forceinline__ void start(const RunCol* c, int n, int32_t* we, double* wv, int32_t r0, int lane) {
+		cols = c; nR = n; winEnd = we; winVal = wv;
+		j = 0; jw = 0; end = RC_NEVER; val = 0.0;
+		const int a = lane - RC_LANE0;
+		if(a >= 0 && a < nR) {
+			const RunCol* C = as_global(cols + a);
+			j = rle_find(as_global(C->runStart), C->nRuns, r0);
+		}
+		if(nR > 0) {
+			refill(lane);
+			read_window(lane);
+		}
+	}
+
+	// First row at which some column's run ends (RC_NEVER: none does any more).
+	__device__ __forceinline__ int32_t next_end() const {
+		int32_t v = end;
+		v = min(v, __builtin_amdgcn_update_dpp(v, v, 0x111, 0xf, 0xf, false)); // row_shr:1
+		v = min(v, __builtin_amdgcn_update_dpp(v, v, 0x112, 0xf, 0xf, false)); // row_shr:2
+		v = min(v, __builtin_amdgcn_update_dpp(v, v, 0x114, 0xf, 0xf, false)); // row_shr:4
+		return __builtin_amdgcn_readlane(v, RC_LANE0 + RC_MAX - 1);
+	}
+
+	// Every column whose run ends at row e moves to its next run.
+	__device__ __forceinline__ void advance(int32_t e, int lane) {
+		const bool mine = end == e; // (never true outside the cursor lanes: e < RC_NEVER)
+		if(mine) j++;
+		if(__ballot(mine && j - jw >= RC_WIN) != 0) refill(lane);
+		if(mine) read_window(lane);
+	}
+
+	// Value of column a (uniform).
+	__device__ __forceinline__ double value(int a) const {
+		int p[2];
+		__builtin_memcpy(p, &val, 8);
+		p[0] = __builtin_amdgcn_readlane(p[0], RC_LANE0 + a);
+		p[1] = __builtin_amdgcn_readlane(p[1], RC_LANE0 + a);
+		double r;
+		__builtin_memcpy(&r, p, 8);
+		return r;
+	}
+};
+
+} // namespace cla

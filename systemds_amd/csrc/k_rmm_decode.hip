@@ -754,9 +754,11 @@ __global__ __launch_bounds__(256) void k_expand_sdc(const DGroup* __restrict__ g
 	sdc_walk_tile(G, r0, SDC_TILE, [&](int rr, int di) { codes[r0 + rr] = (uint8_t) load_code(src, cw, di); });
 }
 
+constexpr int RLE_LONG_RUN = 64; // mean rows per run from which a run-length group counts as long
+
 // Expanded code streams make every dictionary-coded group of a block a plain copy in the tile
 // fill. Built once, when they cost at most half of what the block itself takes in HBM.
-static int ensure_expanded(cla_block* b) {
+int ensure_expanded(cla_block* b) {
 	if(b->expTried) return 0;
 	b->expTried = true;
 	const int nG = (int) b->groups.size();
@@ -765,7 +767,9 @@ static int ensure_expanded(cla_block* b) {
 	std::vector<int> cand;
 	for(int g = 0; g < nG; g++) {
 		const DGroup& G = b->groups[g].d;
-		if((G.type == G_RLE || (G.type == G_SDCZ && G.nOffsets > 0)) && G.nVals <= 255) cand.push_back(g);
+		// (run-length groups with long runs get no copy: the stream kernels follow their runs, cla_runs.hpp)
+		const bool shortRuns = G.type == G_RLE && (int64_t) G.nRuns * RLE_LONG_RUN > b->nRows;
+		if((shortRuns || (G.type == G_SDCZ && G.nOffsets > 0)) && G.nVals <= 255) cand.push_back(g);
 	}
 	if(cand.empty() || (int64_t) cand.size() * b->nRows > b->device_bytes_cached / 2) return 0;
 	for(int g : cand) {
@@ -967,9 +971,11 @@ struct DecPlanCache {
 };
 
 void dir_plan_drop(cla_block* b);
+void gdr_plan_drop(cla_block* b);
 
 void dec_plans_drop(cla_block* b) {
 	dir_plan_drop(b);
+	gdr_plan_drop(b);
 	if(b->decPlans == nullptr) return;
 	for(auto& e : b->decPlans->entries)
 		if(e.dImg) { (void) hipFree(e.dImg); b->derivedBytes -= e.bytes; }
@@ -1452,6 +1458,10 @@ int launch_lmm_decode(cla_block* b, const double* dY, int p, double* dOut, unsig
 int launch_tsmm_decode(cla_block* b, double* dOut) {
 	const int nCols = b->nCols;
 	if(b->groups.empty() || b->nRows == 0 || nCols > 64) return 1;
+	{
+		const int rc = launch_tsmm_direct(b, dOut);
+		if(rc != 1) return rc;
+	}
 	const int NB = (nCols + 15) / 16;
 	// only the product of the first crossBlocks column blocks with the others is wanted (a pair of column chunks
 	// whose own Gram matrices nobody reads): shapes 1 x 1, 1 x 2, 2 x 1, 2 x 2 blocks, anything else in full
