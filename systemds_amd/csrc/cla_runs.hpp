@@ -7,6 +7,7 @@
 // when a cursor leaves it.
 #pragma once
 #include "cla_device.hpp"
+#include <vector>
 
 namespace cla {
 
@@ -24,12 +25,29 @@ struct RunCol {
 	int32_t col;              // column of the matrix
 };
 
+// Merged run table of a block's run-length columns (k_runs.hip).
+struct Mrt {
+	void* base = nullptr;
+	int32_t* start = nullptr;     // nSeg + 1
+	int32_t* codes = nullptr;     // nSeg x nR
+	int32_t* sliceRec = nullptr;  // 8 per slice: segment of the first row, run starts inside the slice, the first six of them
+	double* sums = nullptr;       // nSeg x 16: workspace of the product at hand
+	int nSeg = 0, nR = 0, sliceRows = 0;
+	int64_t nSlices = 0, bytes = 0;
+};
+
 // Same-wave LDS traffic is ordered by the hardware; this keeps the compiler from moving accesses across.
 __device__ __forceinline__ void wave_lds_sync() {
 	__builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
 	__builtin_amdgcn_wave_barrier();
 	__builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
+
+// The cursors' state in LDS (one per wave), for kernels that are short of registers between two run ends.
+struct RunPark {
+	double val[RC_MAX];
+	int32_t j[RC_MAX], jw[RC_MAX], end[RC_MAX];
+};
 
 struct RunCursors {
 	int32_t j;     // cursor lanes: run the column is in
@@ -86,6 +104,19 @@ struct RunCursors {
 		}
 	}
 
+	__device__ __forceinline__ void park(RunPark* p, int lane) const {
+		const int a = lane - RC_LANE0;
+		wave_lds_sync();
+		if(a >= 0 && a < RC_MAX) { p->val[a] = val; p->j[a] = j; p->jw[a] = jw; p->end[a] = end; }
+		wave_lds_sync();
+	}
+	__device__ __forceinline__ void unpark(const RunPark* p, const RunCol* c, int n, int32_t* we, double* wv, int lane) {
+		cols = c; nR = n; winEnd = we; winVal = wv;
+		const int a = lane - RC_LANE0;
+		j = 0; jw = 0; end = RC_NEVER; val = 0.0;
+		if(a >= 0 && a < RC_MAX) { val = p->val[a]; j = p->j[a]; jw = p->jw[a]; end = p->end[a]; }
+	}
+
 	// First row at which some column's run ends (RC_NEVER: none does any more).
 	__device__ __forceinline__ int32_t next_end() const {
 		int32_t v = end;
@@ -114,5 +145,9 @@ struct RunCursors {
 		return r;
 	}
 };
+
+int mrt_build(cla_block* b, const std::vector<RunCol>& runs, int sliceRows, Mrt& T);
+void mrt_free(Mrt& T);
+int launch_run_sums(cla_block* b, const std::vector<RunCol>& runs, const Mrt& T, const double* dB, int ld, int q, const double* dConstRow);
 
 } // namespace cla

@@ -20,7 +20,7 @@
 //               the block has walked all its row tiles.
 // (Wide B on all-DDC blocks uses k_rmm_mfma instead.)
 #include "../../include/cla_hip.h"
-#include "cla_device.hpp"
+#include "cla_runs.hpp"
 #include <algorithm>
 #include <cstring>
 #include <type_traits>
@@ -1061,6 +1061,12 @@ struct DirArgs {
 	const DirCol* cols;
 	const DirDict* dicts;
 	const double* zeroRow;
+	// run-length columns (never looked up per row): the merged run table's segment starts, its record per slice (segment
+	// of the first row, run starts inside), and per segment the columns' part of the output row (k_run_sums, 16 doubles)
+	const int32_t* mrtStart;
+	const int32_t* sliceRec;
+	const double* runSums;
+	int nR;
 	int nDicts, dictDoubles;
 	int segEnd[DSEG_N];
 	const double* B;        // first of the QV columns of this launch
@@ -1072,15 +1078,21 @@ struct DirArgs {
 };
 typedef const __attribute__((address_space(4))) DirCol* dir_ccp;
 typedef unsigned long long dir_u64x4 __attribute__((ext_vector_type(4)));
+typedef int32_t dir_i32x8 __attribute__((ext_vector_type(8)));
 
-template <int QV>
+// HASR: the block has run-length columns. Their part of an output row (plus the constant row) is the same for all rows
+// of a segment of the merged run table and comes from k_run_sums: a lane finds its two rows' segments (the slice's
+// first one from the table's index, the few run starts inside the slice compared one by one) and adds the segments'
+// sums to its rows at the end.
+template <int QV, bool HASR>
 __global__ __launch_bounds__(DIR_THREADS) void k_rmm_direct(const DirArgs A) {
+	constexpr int THREADS = DIR_THREADS, WAVES = THREADS / 64;
 	extern __shared__ __align__(16) double smem[];
 	const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
 	for(int g = 0; g < A.nDicts; g++) {
 		const DirDict D = A.dicts[g];
 		const double* __restrict__ src = as_global(D.src);
-		for(int i = tid; i < D.n; i += DIR_THREADS) smem[D.off + i] = src[i];
+		for(int i = tid; i < D.n; i += THREADS) smem[D.off + i] = src[i];
 	}
 	if(tid < 2) smem[A.dictDoubles - 2 + tid] = 0.0; // what a filler column looks up
 	__syncthreads();
@@ -1090,15 +1102,49 @@ __global__ __launch_bounds__(DIR_THREADS) void k_rmm_direct(const DirArgs A) {
 	const int64_t nRows = A.nRows;
 	const int64_t nSlices = (nRows + DIR_SLICE - 1) / DIR_SLICE;
 	int cnt = 0;
-	for(int64_t slice = (int64_t) blockIdx.x * DIR_WAVES + wave; slice < nSlices; slice += (int64_t) gridDim.x * DIR_WAVES) {
+	dir_i32x8 rec = {0, 0, 0, 0, 0, 0, 0, 0};
+	const int64_t slice0u = (int64_t) blockIdx.x * WAVES + __builtin_amdgcn_readfirstlane(wave); // (a scalar, so that the records come through scalar loads)
+	if(HASR && slice0u < nSlices) rec = *(const __attribute__((address_space(4))) dir_i32x8*) (A.sliceRec + 8 * slice0u);
+	int64_t sliceU = slice0u;
+	for(int64_t slice = (int64_t) blockIdx.x * WAVES + wave; slice < nSlices; slice += (int64_t) gridDim.x * WAVES) {
 		const int64_t s0 = slice * DIR_SLICE, row0 = s0 + 2 * lane;
 		const bool full = s0 + DIR_SLICE <= nRows; // (uniform)
 		const bool in0 = row0 < nRows, in1 = row0 + 1 < nRows;
 		double acc[2][QV];
 #pragma unroll
 		for(int j = 0; j < QV; j++) {
-			const double c0 = A.constRow != nullptr ? ((dec_cdp) A.constRow)[j] : 0.0;
+			const double c0 = !HASR && A.constRow != nullptr ? ((dec_cdp) A.constRow)[j] : 0.0; // (HASR: the segments' sums hold the constant row)
 			acc[0][j] = c0; acc[1][j] = c0;
+		}
+		if(HASR) {
+			// segments of the lane's two rows: the slice's first one plus the run starts inside the slice that lie at or in
+			// front of the row (the slice's record: one scalar load, requested a slice ahead)
+			int sid0 = rec[0], sid1 = rec[0];
+#pragma unroll
+			for(int k = 0; k < 6; k++) {
+				sid0 += row0 >= (int64_t) rec[2 + k] ? 1 : 0;
+				sid1 += row0 + 1 >= (int64_t) rec[2 + k] ? 1 : 0;
+			}
+			for(int k = 6; k < rec[1]; k++) { // (uniform, rare) more than six run starts inside the slice
+				const int64_t st = ((const __attribute__((address_space(4))) int32_t*) A.mrtStart)[rec[0] + 1 + k];
+				sid0 += row0 >= st ? 1 : 0;
+				sid1 += row0 + 1 >= st ? 1 : 0;
+			}
+			{
+				const int64_t next = sliceU + (int64_t) gridDim.x * WAVES;
+				rec = *(const __attribute__((address_space(4))) dir_i32x8*) (A.sliceRec + 8 * (next < nSlices ? next : sliceU));
+				sliceU = next;
+			}
+			// the rows' sums start from their segments' (requested here, needed by the first column's multiply-adds: the
+			// wait falls together with the one for that column's codes)
+			const double* __restrict__ r0 = as_global(A.runSums) + (size_t) sid0 * 16, * __restrict__ r1 = as_global(A.runSums) + (size_t) sid1 * 16;
+#pragma unroll
+			for(int j = 0; j + 1 < QV; j += 2) {
+				const f64x2 v0 = *(const f64x2*) (r0 + j), v1 = *(const f64x2*) (r1 + j);
+				acc[0][j] = v0[0]; acc[0][j + 1] = v0[1];
+				acc[1][j] = v1[0]; acc[1][j + 1] = v1[1];
+			}
+			if(QV & 1) { acc[0][QV - 1] = r0[QV - 1]; acc[1][QV - 1] = r1[QV - 1]; }
 		}
 		// NBAT columns of one class at a time; GUARD: the last slice, whose rows may lie behind the end of the matrix
 		auto batch = [&](auto kindTag, auto twoTag, auto nTag, auto guardTag, int k) {
@@ -1257,6 +1303,8 @@ struct DirPlan {
 	void* dImg = nullptr;
 	int64_t bytes = 0;
 	DirArgs A;
+	std::vector<RunCol> runs; // run-length columns that are followed by run, and their merged run table
+	Mrt mrt;
 };
 
 static int dir_build_plan(cla_block* b, DirPlan& P) {
@@ -1267,6 +1315,7 @@ static int dir_build_plan(cla_block* b, DirPlan& P) {
 		if(rc) return rc;
 	}
 	std::vector<DirDict> dicts;
+	std::vector<RunCol> runs;
 	std::vector<DirCol> cols[DSEG_N];
 	size_t valD = 0;
 	for(int g = 0; g < nG; g++) {
@@ -1287,7 +1336,12 @@ static int dir_build_plan(cla_block* b, DirPlan& P) {
 			cls = G.codeWidth == 2 ? DSEG_DDC2 : DSEG_DDC1;
 		}
 		else {
-			if(b->expCodes[g] == nullptr) return 0;
+			if(b->expCodes[g] == nullptr) {
+				if(G.type != G_RLE) return 0;
+				// a run-length group of long runs: its columns are followed by run (the constant row carries the columns' constants)
+				for(int h = 0; h < G.nColG; h++) runs.push_back(RunCol{G.runStart, G.runCode, G.dict, 0.0, G.nRuns, G.nColG, h, hc[h]});
+				continue;
+			}
 			src = b->expCodes[g];
 			cls = DSEG_GAP1;
 		}
@@ -1310,7 +1364,7 @@ static int dir_build_plan(cla_block* b, DirPlan& P) {
 		}
 		P.A.segEnd[sgm] = (int) all.size();
 	}
-	if(all.empty()) return 0;
+	if(all.empty() || runs.size() > (size_t) RC_MAX || (!runs.empty() && b->nRows >= ((int64_t) 1 << 31) - 2 * DIR_SLICE)) return 0;
 	const size_t colBytes = all.size() * sizeof(DirCol), dictBytes = dicts.size() * sizeof(DirDict);
 	std::vector<uint8_t> img(colBytes + dictBytes + 16 * 8, 0);
 	std::memcpy(img.data(), all.data(), colBytes);
@@ -1323,6 +1377,15 @@ static int dir_build_plan(cla_block* b, DirPlan& P) {
 	P.A.cols = (const DirCol*) d;
 	P.A.dicts = (const DirDict*) (d + colBytes);
 	P.A.zeroRow = (const double*) (d + colBytes + dictBytes);
+	P.A.nR = (int) runs.size();
+	P.A.mrtStart = nullptr; P.A.sliceRec = nullptr; P.A.runSums = nullptr;
+	if(!runs.empty()) {
+		const int rc = mrt_build(b, runs, DIR_SLICE, P.mrt);
+		if(rc) return rc < 0 ? rc : 0;
+		P.runs = runs;
+		P.bytes += P.mrt.bytes;
+		P.A.mrtStart = P.mrt.start; P.A.sliceRec = P.mrt.sliceRec; P.A.runSums = P.mrt.sums;
+	}
 	P.A.nDicts = (int) dicts.size();
 	P.A.dictDoubles = (int) valD;
 	P.A.nRows = b->nRows;
@@ -1333,6 +1396,7 @@ static int dir_build_plan(cla_block* b, DirPlan& P) {
 void dir_plan_drop(cla_block* b) {
 	if(b->dirPlan == nullptr) return;
 	if(b->dirPlan->dImg) { (void) hipFree(b->dirPlan->dImg); b->derivedBytes -= b->dirPlan->bytes; }
+	mrt_free(b->dirPlan->mrt);
 	delete b->dirPlan;
 	b->dirPlan = nullptr;
 }
@@ -1367,12 +1431,22 @@ static int launch_rmm_direct(cla_block* b, const double* dB, int q, const double
 		const size_t lds = ((size_t) A.dictDoubles + (size_t) DIR_WAVES * DIR_SROWS * qv) * 8;
 		A.B = dB + c0; A.constRow = dConstRow ? dConstRow + c0 : nullptr; A.out = dOut + c0;
 		const double algo = (double) b->device_bytes_cached + (double) b->nRows * qv * 8;
+		if(A.nR > 0) {
+			const int rc = launch_run_sums(b, b->dirPlan->runs, b->dirPlan->mrt, A.B, q, qv, A.constRow);
+			if(rc) return rc;
+		}
 		Prof pf(b, "k_rmm_direct", grid, DIR_THREADS, (long) lds, algo);
 		switch(qv) {
-#define DIR_CASE(QV)                                                                              \
-	case QV:                                                                                      \
-		CLA_HIP(allow_full_lds((const void*) k_rmm_direct<QV>));                                  \
-		hipLaunchKernelGGL(k_rmm_direct<QV>, dim3(grid), dim3(DIR_THREADS), lds, b->stream, A); \
+#define DIR_CASE(QV)                                                                                         \
+	case QV:                                                                                                 \
+		if(A.nR > 0) {                                                                                       \
+			CLA_HIP(allow_full_lds((const void*) k_rmm_direct<QV, true>));                                   \
+			hipLaunchKernelGGL((k_rmm_direct<QV, true>), dim3(grid), dim3(DIR_THREADS), lds, b->stream, A);  \
+		}                                                                                                    \
+		else {                                                                                               \
+			CLA_HIP(allow_full_lds((const void*) k_rmm_direct<QV, false>));                                  \
+			hipLaunchKernelGGL((k_rmm_direct<QV, false>), dim3(grid), dim3(DIR_THREADS), lds, b->stream, A); \
+		}                                                                                                    \
 		break;
 			DIR_CASE(1) DIR_CASE(2) DIR_CASE(3) DIR_CASE(4) DIR_CASE(5) DIR_CASE(6) DIR_CASE(7) DIR_CASE(8)
 			DIR_CASE(9) DIR_CASE(10) DIR_CASE(11) DIR_CASE(12) DIR_CASE(13) DIR_CASE(14) DIR_CASE(15) DIR_CASE(16)
