@@ -128,6 +128,12 @@ int cla_block_set_stream(cla_handle h, void* hipStream);
  * that uses them. Returns 0, or -CLA_ERR_INVALID for an unknown key or value. */
 int cla_block_set_option(cla_handle h, const char* key, int32_t value);
 int32_t cla_block_num_groups(cla_handle h);
+/* Dimensions of the block (CompressedMatrixBlock.getNumRows / getNumColumns) and the number of tuples of a group's
+ * dictionary (AColGroupValue.getNumValues; 0 for groups without one): what a binding needs to check the lengths
+ * of the arrays a caller hands it. Negative: -CLA_ERR_INVALID. */
+int64_t cla_block_num_rows(cla_handle h);
+int32_t cla_block_num_cols(cla_handle h);
+int32_t cla_block_group_num_values(cla_handle h, int32_t group);
 /* Bytes of HBM held by the block's compressed representation. */
 int64_t cla_block_device_bytes(cla_handle h);
 /* Bytes of HBM held by the formats the library has derived from that representation so far (padded
@@ -145,22 +151,28 @@ int64_t cla_rmm_dev(cla_handle h, const double* dB, int32_t nColB, double* dOut)
 /* The same without the wait: returns 0 once the kernels are queued on the block's stream (or a negative
  * error); the non-zero count stays in a device counter until cla_block_nnz asks for it. */
 int cla_rmm_dev_async(cla_handle h, const double* dB, int32_t nColB, double* dOut);
-/* cla_rmm_dev for callers that cannot allocate device memory (code under HIP graph capture, tight serving
- * loops, harnesses that forbid hipMalloc). It has no counterpart in the reference. The pre-aggregated tables
- * dict_g x B and the non-zero counter live in a static device array of 4 MiB that the library holds per GPU
- * until the process ends; the call makes no hipMalloc / hipFree and builds no derived format, so it always
- * takes the table-reading kernels (never the matrix-core or decode kernels). -CLA_ERR_UNSUPPORTED when the
- * tables ((sum of dictionary sizes + 1) x nColB doubles, plus 256 per group for byte-code mat-vecs) exceed
- * the array, or when the block holds SDC groups with entries (their row-tile plan is an allocation). All calls
- * on one GPU share the array: calls that overlap in time on one GPU (two blocks, two threads) race. The
- * count returned by cla_block_nnz is not updated by this entry point. */
+/* cla_rmm_dev for callers that cannot allocate device memory (tight serving loops, harnesses that forbid
+ * hipMalloc). It has no counterpart in the reference. The pre-aggregated tables dict_g x B and the non-zero
+ * counter live in a static device array of 4 MiB that the library holds per GPU until the process ends; the
+ * call makes no hipMalloc / hipFree and builds no derived format, so it always takes the table-reading kernels
+ * (never the matrix-core or decode kernels). -CLA_ERR_UNSUPPORTED when the tables ((sum of dictionary sizes
+ * + 1) x nColB doubles, plus 256 per group for byte-code mat-vecs) exceed the array, or when the block holds
+ * SDC groups with entries (their row-tile plan is an allocation). All calls on one GPU share the array: the
+ * library serialises them (a lock per GPU, held until the call's kernels have finished), so calls on different
+ * blocks from different threads are safe and run one after the other. The call waits for the block's stream
+ * before it returns (it cannot run under stream capture). The count returned by cla_block_nnz is not updated
+ * by this entry point. */
 int64_t cla_rmm_dev_noalloc(cla_handle h, const double* dB, int32_t nColB, double* dOut);
 /* nnz of the result of the last driver call on this block (MatrixBlock.recomputeNonZeros of the reference
  * drivers, C/lib/CLALibRightMultBy.java:98); waits for the block's stream. */
 int64_t cla_block_nnz(cla_handle h);
 
 /* CLALibLeftMultBy.leftMultByMatrix (C/lib/CLALibLeftMultBy.java:126-145,
- * 286-346): out[nRowY x nCols] = Y %*% X, Y is nRowY x nRows. */
+ * 286-346): out[nRowY x nCols] = Y %*% X, Y is nRowY x nRows.
+ * The _dev_async form returns without waiting except where the block takes the one-pass kernel on the decoded rows
+ * (option lmm_joint, blocks that are neither byte-code DDC nor mostly offset lists): that kernel reports a value
+ * of Y that is not finite, the host reads the flag (one wait for the block's stream per call) and such a Y takes
+ * the bin kernels. The same holds for cla_mmchain_dev_async, whose second half is this product. */
 int64_t cla_lmm(cla_handle h, const double* Y, int32_t nRowY, double* out);
 int64_t cla_lmm_dev(cla_handle h, const double* dY, int32_t nRowY, double* dOut);
 int cla_lmm_dev_async(cla_handle h, const double* dY, int32_t nRowY, double* dOut);

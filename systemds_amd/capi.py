@@ -47,6 +47,9 @@ SIGNATURES = {
     "cla_block_set_stream": (C.c_int, [C.c_void_p, C.c_void_p]),
     "cla_block_set_option": (C.c_int, [C.c_void_p, C.c_char_p, C.c_int32]),
     "cla_block_num_groups": (C.c_int32, [C.c_void_p]),
+    "cla_block_num_rows": (C.c_int64, [C.c_void_p]),
+    "cla_block_num_cols": (C.c_int32, [C.c_void_p]),
+    "cla_block_group_num_values": (C.c_int32, [C.c_void_p, C.c_int32]),
     "cla_block_device_bytes": (C.c_int64, [C.c_void_p]),
     "cla_block_derived_bytes": (C.c_int64, [C.c_void_p]),
     "cla_rmm": (C.c_int64, [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),

@@ -34,6 +34,7 @@ namespace cla {
 
 constexpr int MAX_DEVICES = 64;
 static unsigned char* g_scratchPtr[MAX_DEVICES] = {}; // device address of `scratch` per device (set at cla_init)
+static std::mutex g_scratchMu[MAX_DEVICES];           // one call at a time works in a device's copy of `scratch`
 
 static thread_local char t_err[1024] = "";
 int g_ldsPerBlock = 65536;
@@ -734,6 +735,16 @@ int cla_selftest_exception(int kind) {
 }
 
 int32_t cla_block_num_groups(cla_handle b) { return b ? (int32_t) b->groups.size() : -CLA_ERR_INVALID; }
+int64_t cla_block_num_rows(cla_handle b) { return b ? b->nRows : -CLA_ERR_INVALID; }
+int32_t cla_block_num_cols(cla_handle b) { return b ? b->nCols : -CLA_ERR_INVALID; }
+int32_t cla_block_group_num_values(cla_handle b, int32_t group) {
+	CLA_TRY
+	if(!b) return -CLA_ERR_INVALID;
+	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	if(group < 0 || group >= (int32_t) b->groups.size()) return -CLA_ERR_INVALID;
+	return b->groups[group].d.type == G_UNC ? 0 : b->groups[group].d.nVals;
+	CLA_CATCH_CODE(int32_t)
+}
 
 int64_t cla_block_device_bytes(cla_handle b) {
 	CLA_TRY
@@ -795,6 +806,9 @@ int64_t cla_rmm_dev_noalloc(cla_handle b, const double* dB, int32_t nColB, doubl
 	unsigned char* ws = g_device < MAX_DEVICES ? g_scratchPtr[g_device] : nullptr;
 	if(!ws) { set_error("rmm without allocation: no static workspace on device %d", g_device); return -CLA_ERR_STATE; }
 	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	// All calls on a GPU share its copy of the workspace, whatever block and stream they come from: held from the first
+	// kernel's launch until the stream has drained (the call waits for that anyway, so the lock costs nothing).
+	std::lock_guard<std::mutex> lkScratch(g_scratchMu[g_device]);
 	// the counter and the tables live in the static workspace (the pre-aggregation kernel clears the counter
 	// and rewrites every table entry that is read); event pairs of the profiling mode would be allocations
 	unsigned long long* dNnz = (unsigned long long*) ws;

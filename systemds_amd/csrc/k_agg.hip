@@ -25,8 +25,12 @@ namespace cla {
 __device__ __forceinline__ double agg_identity(int op) {
 	return op == CLA_AGG_MIN ? __builtin_inf() : op == CLA_AGG_MAX ? -__builtin_inf() : 0.0;
 }
+// (min / max as Math.min / Math.max, which the reference's Builtin MIN / MAX use (functionobjects/Builtin.java:259-264,
+// 308-312): a NaN operand gives NaN, where fmin / fmax would drop it)
 __device__ __forceinline__ double agg_combine(int op, double a, double v) {
-	return op == CLA_AGG_MIN ? fmin(a, v) : op == CLA_AGG_MAX ? fmax(a, v) : a + v;
+	if(op == CLA_AGG_MIN) return a != a || v != v ? __builtin_nan("") : fmin(a, v);
+	if(op == CLA_AGG_MAX) return a != a || v != v ? __builtin_nan("") : fmax(a, v);
+	return a + v;
 }
 
 __device__ __forceinline__ double block_reduce(int op, double v, double* red) {

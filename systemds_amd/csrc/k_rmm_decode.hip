@@ -1463,7 +1463,9 @@ int launch_rmm_decode(cla_block* b, const double* dB, int q, const double* dCons
 	unsigned long long* dNnz) {
 	if(b->groups.empty() || b->nRows == 0 || q < 1) return 1;
 	// (16 columns: no padding of B left for the tile kernel to lose, and the stream kernel short of registers: C5 2.1 against 2.5 ms)
-	const bool tilesFirst = q == DEC_QMAX;
+	// (... unless run-length columns are followed by run: the tile kernel would expand them tile by tile, 2.4 against 2.2 ms)
+	bool tilesFirst = q == DEC_QMAX;
+	if(tilesFirst && b->opt.rmmDirect && dir_plan_get(b) == 0 && b->dirPlan->A.nR > 0) tilesFirst = false;
 	if(b->opt.rmmDirect && !tilesFirst) {
 		const int rc = launch_rmm_direct(b, dB, q, dConstRow, dOut, dNnz);
 		if(rc != 1) return rc;

@@ -4,7 +4,10 @@
  * (src/main/cpp/systemds.cpp:38-84): arrays are pinned with GetPrimitiveArrayCritical, inputs are
  * released with JNI_ABORT (no copy back), outputs with 0 (copy back when the VM handed out a copy).
  * No JNI call is made while an array is pinned; the library throws no C++ exception across its
- * boundary, so nothing can unwind through these frames.
+ * boundary, so nothing can unwind through these frames. Array references are checked for NULL and for the
+ * length the library will read or write before anything is pinned.
+ * This file has not been compiled or run where it was written (no JDK there): it is the binding as a
+ * maintainer would add it, checked by reading only.
  *
  * Build (needs a JDK; systemds_amd/build.py compiles it when $JAVA_HOME/include/jni.h exists):
  *   cc -O2 -fPIC -shared -I$JAVA_HOME/include -I$JAVA_HOME/include/linux -Iinclude \
@@ -16,6 +19,12 @@
 
 #define FN(name) Java_org_apache_sysds_utils_ClaHipNative_##name
 #define H(h) ((cla_handle) (intptr_t) (h))
+
+/* Length of a Java array, -1 for a NULL reference (GetArrayLength on NULL crashes the VM). */
+static jlong len(JNIEnv* env, jarray a) { return a ? (jlong) (*env)->GetArrayLength(env, a) : -1; }
+/* An array the library reads or writes `need` elements of: not NULL and long enough. Checked before anything is
+ * pinned: a short array would otherwise be a heap overwrite inside a critical region. */
+static int holds(JNIEnv* env, jarray a, jlong need) { return need >= 0 && len(env, a) >= need; }
 
 /* pin / unpin; a NULL Java array pins to NULL */
 static void* pin(JNIEnv* env, jarray a) { return a ? (*env)->GetPrimitiveArrayCritical(env, a, NULL) : NULL; }
@@ -36,6 +45,7 @@ JNIEXPORT void JNICALL FN(blockFree)(JNIEnv* env, jclass c, jlong h) { (void) en
 JNIEXPORT jint JNICALL FN(addDDC)(JNIEnv* env, jclass c, jlong h, jintArray cols, jdoubleArray dict, jint nVals,
 	jobject codes, jint codeWidth) {
 	(void) c;
+	if(!cols || !holds(env, dict, (jlong) nVals * len(env, cols)) || !holds(env, (jarray) codes, cla_block_num_rows(H(h)))) return -CLA_ERR_INVALID;
 	const jint nColG = (*env)->GetArrayLength(env, cols);
 	jint* pc = pin(env, cols);
 	double* pd = pin(env, dict);
@@ -51,6 +61,8 @@ JNIEXPORT jint JNICALL FN(addSDC)(JNIEnv* env, jclass c, jlong h, jintArray cols
 	jdoubleArray defaultTuple, jobject codes, jint codeWidth, jobject deltas, jint deltaWidth, jlong nDeltas, jint offsetToFirst,
 	jint offsetToLast, jlong nOffsets) {
 	(void) c;
+	if(!cols || !holds(env, dict, (jlong) nVals * len(env, cols)) || (defaultTuple && !holds(env, defaultTuple, len(env, cols))) ||
+		(nOffsets > 0 && (!holds(env, (jarray) codes, nOffsets) || !holds(env, (jarray) deltas, nDeltas)))) return -CLA_ERR_INVALID;
 	const jint nColG = (*env)->GetArrayLength(env, cols);
 	jint* pc = pin(env, cols);
 	double* pd = pin(env, dict);
@@ -70,6 +82,7 @@ JNIEXPORT jint JNICALL FN(addSDC)(JNIEnv* env, jclass c, jlong h, jintArray cols
 JNIEXPORT jint JNICALL FN(addRLE)(JNIEnv* env, jclass c, jlong h, jintArray cols, jdoubleArray dict, jint nVals, jintArray ptr,
 	jcharArray data) {
 	(void) c;
+	if(!cols || !data || !holds(env, dict, (jlong) nVals * len(env, cols)) || !holds(env, ptr, (jlong) nVals + 1)) return -CLA_ERR_INVALID;
 	const jint nColG = (*env)->GetArrayLength(env, cols);
 	const jlong nData = (*env)->GetArrayLength(env, data);
 	jint* pc = pin(env, cols);
@@ -89,6 +102,7 @@ JNIEXPORT jint JNICALL FN(addRLE)(JNIEnv* env, jclass c, jlong h, jintArray cols
 #define ADD_COLS_VALUES(name, call)                                                                         \
 	JNIEXPORT jint JNICALL FN(name)(JNIEnv* env, jclass c, jlong h, jintArray cols, jdoubleArray values) { \
 		(void) c;                                                                                           \
+		if(!cols || !values) return -CLA_ERR_INVALID;                                                       \
 		const jint nColG = (*env)->GetArrayLength(env, cols);                                               \
 		jint* pc = pin(env, cols);                                                                          \
 		double* pv = pin(env, values);                                                                      \
@@ -102,6 +116,7 @@ ADD_COLS_VALUES(addConst, cla_block_add_const)
 
 JNIEXPORT jint JNICALL FN(addEmpty)(JNIEnv* env, jclass c, jlong h, jintArray cols) {
 	(void) c;
+	if(!cols) return -CLA_ERR_INVALID;
 	const jint nColG = (*env)->GetArrayLength(env, cols);
 	jint* pc = pin(env, cols);
 	const jint rc = pc ? cla_block_add_empty(H(h), (const int32_t*) pc, nColG) : -CLA_ERR_INVALID;
@@ -123,6 +138,8 @@ JNIEXPORT jint JNICALL FN(setOption)(JNIEnv* env, jclass c, jlong h, jstring key
 /* one input array, one output array */
 JNIEXPORT jlong JNICALL FN(rmm)(JNIEnv* env, jclass c, jlong h, jdoubleArray B, jint nColB, jdoubleArray out) {
 	(void) c;
+	const jlong nR = cla_block_num_rows(H(h)), nC = cla_block_num_cols(H(h));
+	if(nColB <= 0 || !holds(env, B, nC * nColB) || !holds(env, out, nR * nColB)) return -CLA_ERR_INVALID;
 	double* b = pin(env, B);
 	double* o = pin(env, out);
 	const jlong nnz = (b && o) ? cla_rmm(H(h), b, nColB, o) : -CLA_ERR_INVALID;
@@ -133,6 +150,8 @@ JNIEXPORT jlong JNICALL FN(rmm)(JNIEnv* env, jclass c, jlong h, jdoubleArray B, 
 
 JNIEXPORT jlong JNICALL FN(lmm)(JNIEnv* env, jclass c, jlong h, jdoubleArray Y, jint nRowY, jdoubleArray out) {
 	(void) c;
+	const jlong nR = cla_block_num_rows(H(h)), nC = cla_block_num_cols(H(h));
+	if(nRowY <= 0 || !holds(env, Y, nR * nRowY) || !holds(env, out, nC * nRowY)) return -CLA_ERR_INVALID;
 	double* y = pin(env, Y);
 	double* o = pin(env, out);
 	const jlong nnz = (y && o) ? cla_lmm(H(h), y, nRowY, o) : -CLA_ERR_INVALID;
@@ -143,6 +162,8 @@ JNIEXPORT jlong JNICALL FN(lmm)(JNIEnv* env, jclass c, jlong h, jdoubleArray Y, 
 
 JNIEXPORT jlong JNICALL FN(tsmm)(JNIEnv* env, jclass c, jlong h, jdoubleArray out) {
 	(void) c;
+	const jlong nC = cla_block_num_cols(H(h));
+	if(!holds(env, out, nC * nC)) return -CLA_ERR_INVALID;
 	double* o = pin(env, out);
 	const jlong nnz = o ? cla_tsmm(H(h), o) : -CLA_ERR_INVALID;
 	unpin_out(env, out, o);
@@ -151,6 +172,8 @@ JNIEXPORT jlong JNICALL FN(tsmm)(JNIEnv* env, jclass c, jlong h, jdoubleArray ou
 
 JNIEXPORT jlong JNICALL FN(mmchain)(JNIEnv* env, jclass c, jlong h, jdoubleArray v, jdoubleArray w, jint ctype, jdoubleArray out) {
 	(void) c;
+	const jlong nR = cla_block_num_rows(H(h)), nC = cla_block_num_cols(H(h));
+	if(!holds(env, v, nC) || (w && !holds(env, w, nR)) || !holds(env, out, nC)) return -CLA_ERR_INVALID;
 	double* pv = pin(env, v);
 	double* pw = pin(env, w);
 	double* o = pin(env, out);
@@ -163,6 +186,7 @@ JNIEXPORT jlong JNICALL FN(mmchain)(JNIEnv* env, jclass c, jlong h, jdoubleArray
 
 JNIEXPORT jlong JNICALL FN(rmmOverlapping)(JNIEnv* env, jclass c, jlong h, jdoubleArray B, jint nColB) {
 	(void) c;
+	if(nColB <= 0 || !holds(env, B, (jlong) cla_block_num_cols(H(h)) * nColB)) return 0;
 	double* b = pin(env, B);
 	const jlong r = b ? (jlong) (intptr_t) cla_rmm_overlapping(H(h), b, nColB) : 0;
 	unpin_in(env, B, b);
@@ -171,6 +195,7 @@ JNIEXPORT jlong JNICALL FN(rmmOverlapping)(JNIEnv* env, jclass c, jlong h, jdoub
 
 JNIEXPORT jlong JNICALL FN(lmmCompressed)(JNIEnv* env, jclass c, jlong hRight, jlong hLeft, jdoubleArray out) {
 	(void) c;
+	if(!holds(env, out, (jlong) cla_block_num_cols(H(hLeft)) * cla_block_num_cols(H(hRight)))) return -CLA_ERR_INVALID;
 	double* o = pin(env, out);
 	const jlong nnz = o ? cla_lmm_compressed(H(hRight), H(hLeft), o) : -CLA_ERR_INVALID;
 	unpin_out(env, out, o);
@@ -179,6 +204,7 @@ JNIEXPORT jlong JNICALL FN(lmmCompressed)(JNIEnv* env, jclass c, jlong hRight, j
 
 JNIEXPORT jlong JNICALL FN(decompress)(JNIEnv* env, jclass c, jlong h, jdoubleArray out) {
 	(void) c;
+	if(!holds(env, out, cla_block_num_rows(H(h)) * cla_block_num_cols(H(h)))) return -CLA_ERR_INVALID;
 	double* o = pin(env, out);
 	const jlong nnz = o ? cla_decompress(H(h), o) : -CLA_ERR_INVALID;
 	unpin_out(env, out, o);
@@ -187,6 +213,8 @@ JNIEXPORT jlong JNICALL FN(decompress)(JNIEnv* env, jclass c, jlong h, jdoubleAr
 
 JNIEXPORT jlong JNICALL FN(aggregate)(JNIEnv* env, jclass c, jlong h, jint op, jint dir, jdoubleArray out) {
 	(void) c;
+	/* (CLA_AGG_ALL one value, CLA_AGG_ROW one per row, CLA_AGG_COL one per column) */
+	if(!holds(env, out, dir == CLA_AGG_ALL ? 1 : dir == CLA_AGG_ROW ? cla_block_num_rows(H(h)) : cla_block_num_cols(H(h)))) return -CLA_ERR_INVALID;
 	double* o = pin(env, out);
 	const jlong nnz = o ? cla_aggregate(H(h), op, dir, o) : -CLA_ERR_INVALID;
 	unpin_out(env, out, o);
@@ -195,6 +223,7 @@ JNIEXPORT jlong JNICALL FN(aggregate)(JNIEnv* env, jclass c, jlong h, jint op, j
 
 JNIEXPORT jint JNICALL FN(counts)(JNIEnv* env, jclass c, jlong h, jint group, jintArray counts) {
 	(void) c;
+	if(!holds(env, counts, cla_block_group_num_values(H(h), group))) return -CLA_ERR_INVALID;
 	jint* p = pin(env, counts);
 	const jint rc = p ? cla_counts(H(h), group, (int32_t*) p) : -CLA_ERR_INVALID;
 	unpin_out(env, counts, p);
@@ -203,6 +232,7 @@ JNIEXPORT jint JNICALL FN(counts)(JNIEnv* env, jclass c, jlong h, jint group, ji
 
 JNIEXPORT jint JNICALL FN(cooc)(JNIEnv* env, jclass c, jlong h, jint groupA, jint groupB, jlongArray out) {
 	(void) c;
+	if(!holds(env, out, (jlong) cla_block_group_num_values(H(h), groupA) * cla_block_group_num_values(H(h), groupB))) return -CLA_ERR_INVALID;
 	jlong* p = pin(env, out);
 	const jint rc = p ? cla_cooc(H(h), groupA, groupB, (int64_t*) p) : -CLA_ERR_INVALID;
 	unpin_out(env, out, p);
@@ -211,6 +241,8 @@ JNIEXPORT jint JNICALL FN(cooc)(JNIEnv* env, jclass c, jlong h, jint groupA, jin
 
 JNIEXPORT jint JNICALL FN(preagg)(JNIEnv* env, jclass c, jlong h, jint group, jdoubleArray Y, jint nRowY, jdoubleArray preAgg) {
 	(void) c;
+	if(nRowY <= 0 || !holds(env, Y, cla_block_num_rows(H(h)) * nRowY) ||
+		!holds(env, preAgg, (jlong) nRowY * cla_block_group_num_values(H(h), group))) return -CLA_ERR_INVALID;
 	double* y = pin(env, Y);
 	double* p = pin(env, preAgg);
 	const jint rc = (y && p) ? cla_preagg(H(h), group, y, nRowY, p) : -CLA_ERR_INVALID;

@@ -17,12 +17,21 @@ def hip():
         _hip.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
         _hip.hipMemset.argtypes = [C.c_void_p, C.c_int, C.c_size_t]
         _hip.hipDeviceSynchronize.argtypes = []
+        _hip.hipMemGetInfo.argtypes = [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]
     return _hip
 
 
 def _ok(rc, what):
     if rc != 0:
         raise RuntimeError(f"{what} failed with HIP error {rc}")
+
+
+def free_device_bytes():
+    """Free device memory as hipMemGetInfo reports it (after a device synchronisation)."""
+    _ok(hip().hipDeviceSynchronize(), "hipDeviceSynchronize")
+    free, total = C.c_size_t(), C.c_size_t()
+    _ok(hip().hipMemGetInfo(C.byref(free), C.byref(total)), "hipMemGetInfo")
+    return free.value
 
 
 class DevBuf:

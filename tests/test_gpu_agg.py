@@ -151,3 +151,35 @@ def test_row_sums_of_squares_on_a_block_with_few_offset_lists(cla, ora, n_rows):
     for op in OPS:
         for direction in DIRS:
             check(cla, specs, D, n_rows, 5, op, direction, "few lists")
+
+
+@pytest.mark.parametrize("direction", DIRS)
+@pytest.mark.parametrize("op", ["min", "max"])
+def test_nan_cells_propagate_like_math_min_max(cla, ora, op, direction):
+    """The reference's Builtin MIN / MAX are Math.min / Math.max (functionobjects/Builtin.java:259-264, 308-312): a NaN
+    cell makes the aggregate over it NaN. One NaN tuple in a dictionary (it occurs in some rows) and one NaN cell of an
+    uncompressed group."""
+    from systemds_amd import synth
+    n_rows = 5000
+    rng = np.random.default_rng(77)
+    d = rng.standard_normal((9, 1))
+    d[4, 0] = np.nan
+    codes = rng.integers(0, 9, n_rows).astype(np.uint8)
+    dense = rng.standard_normal((n_rows, 2))
+    dense[1234, 1] = np.nan
+    specs = [synth.GroupSpec("ddc", np.array([0], np.int32), d, codes),
+             synth.GroupSpec("ddc", np.array([1], np.int32), rng.standard_normal((5, 1)), rng.integers(0, 5, n_rows).astype(np.uint8)),
+             synth.GroupSpec("unc", np.array([2, 3], np.int32), dense=dense)]
+    D = ora.np_decompress(specs, n_rows, 4)
+    blk = cla.build_block(n_rows, 4, specs)
+    try:
+        out, nnz = blk.aggregate(op, direction)
+    finally:
+        blk.close()
+    axis = {"all": None, "row": 1, "col": 0}[direction]
+    with np.errstate(invalid="ignore"):
+        ref = np.asarray((np.min if op == "min" else np.max)(D, axis=axis)).reshape(-1)
+    assert np.array_equal(np.isnan(out), np.isnan(ref)), (op, direction)
+    fin = ~np.isnan(ref)
+    assert np.allclose(out[fin], ref[fin], rtol=1e-15, atol=0)
+    assert nnz == np.count_nonzero(out)

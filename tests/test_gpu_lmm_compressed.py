@@ -80,7 +80,9 @@ def test_same_block_is_tsmm(cla, ora):
     out, _ = blk.lmm_compressed(blk)
     ts, _ = blk.tsmm()
     D = ora.np_decompress(specs, 30000, n)
-    assert_fp64_close(out, ts, 2 * ora.abs_matmul(D.T, D), what="t(X) %*% X", n_terms=30000)
+    assert_matches_truth(out, D.T, D, what="t(X) %*% X as compressed x compressed")
+    assert_matches_truth(ts, D.T, D, what="t(X) %*% X")
+    assert_fp64_close(out, ts, 2 * ora.abs_matmul(D.T, D), what="the two against each other")
     blk.close()
 
 
@@ -126,9 +128,10 @@ def test_overlapping_operand(cla, ora):
     blk = cla.build_block(n_rows, n, specs)
     child = blk.rmm_overlapping(B)
     out, _ = blk.lmm_compressed(child)      # t(XB) %*% X
-    assert_fp64_close(out, ora.longdouble_matmul(P.T, D), np.abs(P).T @ np.abs(D), what="t(XB) %*% X", n_terms=n_rows)
+    absP = np.abs(D) @ np.abs(B)            # (bounds P's own rounding as well as its cells)
+    assert_fp64_close(out, ora.longdouble_matmul(P.T, D), absP.T @ np.abs(D), what="t(XB) %*% X")
     out, _ = child.lmm_compressed(blk)      # t(X) %*% XB
-    assert_fp64_close(out, ora.longdouble_matmul(D.T, P), np.abs(D).T @ np.abs(P), what="t(X) %*% XB", n_terms=n_rows)
+    assert_fp64_close(out, ora.longdouble_matmul(D.T, P), np.abs(D).T @ absP, what="t(X) %*% XB")
     out, _ = blk.lmm_compressed(blk)
     assert_matches_truth(out, D.T, D, what="t(X) %*% X afterwards")
     child.close()

@@ -44,7 +44,9 @@ def test_mixed_groups(cla, ora, seed, n_rows, q):
     # (CLALibTSMM.java:73-77; CompressedTestBase.java:507-522 testTransposeSelfLeftMultOverload)
     out, nnz = child.tsmm()
     assert np.array_equal(out, out.T) and nnz == np.count_nonzero(out)
-    assert_fp64_close(out, ora.longdouble_matmul(P.T, P), np.abs(P).T @ np.abs(P), what="t(XB) %*% (XB)", n_terms=n_rows)
+    # (scale: the rounding of P = X B itself enters, bounded by |D| |B| per cell of P)
+    absP = np.abs(D) @ np.abs(B)
+    assert_fp64_close(out, ora.longdouble_matmul(P.T, P), absP.T @ absP, what="t(XB) %*% (XB)")
     # neither are maxima: aggregated over decompressed row chunks (CLALibCompAgg.java:220-232)
     out, _ = child.aggregate("max", "col")
     assert_fp64_close(out, P.max(axis=0), np.abs(D).max(axis=0) @ np.abs(B) + 2.0, what="colMaxs of XB")
@@ -89,7 +91,8 @@ def test_uncompressed_groups(cla, ora, seed, n_rows, q):
     P = ora.longdouble_matmul(D, B)
     check_child(ora, child, P, np.abs(D) @ np.abs(B), rng, "with an uncompressed group")
     out, _ = child.tsmm()
-    assert_fp64_close(out, ora.longdouble_matmul(P.T, P), np.abs(P).T @ np.abs(P), what="t(XB) %*% (XB)", n_terms=n_rows)
+    absP = np.abs(D) @ np.abs(B)
+    assert_fp64_close(out, ora.longdouble_matmul(P.T, P), absP.T @ absP, what="t(XB) %*% (XB)")
     grand = child.rmm_overlapping(rng.standard_normal((q, 3)))
     child.close()
     out, _ = grand.decompress()

@@ -109,9 +109,19 @@ def test_tsmm_equals_gram_matrix(ora, seed, n_rows, k):
         D = ora.np_decompress(specs, n_rows, n_cols)
         out, nnz = ora.tsmm(G, k)
         truth = ora.longdouble_matmul(D.T, D)
-        assert_close(out, truth, ora.abs_matmul(D.T, D), tol=4e-12 if n_rows > 10000 else TOL)
+        assert_close(out, truth, ora.abs_matmul(D.T, D), tol=TOL)
         assert np.array_equal(out, out.T)
         assert nnz == np.count_nonzero(out)
+        # every pair of DDC groups against the closed form t(dictA) %*% N %*% dictB with the integer co-occurrence
+        # counts N = bincount(codeA * nB + codeB) (what preAggregateDDC_DDC + the dictionary product compute), in long double
+        ddc = [s for s in specs if s.type == "ddc"]
+        for i, a in enumerate(ddc):
+            for b in ddc[i + 1:]:
+                nA, nB = a.dict.shape[0], b.dict.shape[0]
+                N = np.bincount(a.codes.astype(np.int64) * nB + b.codes.astype(np.int64), minlength=nA * nB).reshape(nA, nB)
+                want = (a.dict.astype(np.longdouble).T @ N.astype(np.longdouble) @ b.dict.astype(np.longdouble)).astype(np.float64)
+                scale = np.abs(a.dict).T @ N.astype(np.float64) @ np.abs(b.dict)
+                assert_close(out[np.ix_(a.cols, b.cols)], want, scale, tol=TOL)
 
 
 def test_tsmm_diagonal_closed_form(ora):

@@ -71,3 +71,58 @@ def test_refusals(cla):
         blk.rmm_dev_noalloc(dB.ptr, 1, dOut.ptr)
     assert e.value.code == cla.ERR_UNSUPPORTED
     blk.close()
+
+
+def test_the_call_allocates_nothing(cla):
+    """Free device memory (hipMemGetInfo) and the block's derived bytes are the same before and after the call, also on
+    the first call on a fresh block (where cla_rmm_dev builds its padded dictionaries and tables)."""
+    from devmem import free_device_bytes
+    from systemds_amd import synth
+    c = synth.config2(scale=100)
+    n, m = c["n_rows"], c["n_cols"]
+    blk = cla.build_block(n, m, c["groups"])
+    dB = DevBuf.from_numpy(c["v"][:m])
+    dOut = DevBuf(n * 8)
+    free0, derived0 = free_device_bytes(), blk.derived_bytes()
+    for _ in range(3):
+        blk.rmm_dev_noalloc(dB.ptr, 1, dOut.ptr)
+        assert free_device_bytes() == free0
+        assert blk.derived_bytes() == derived0
+    blk.close()
+
+
+def test_two_threads_on_two_blocks(cla, ora):
+    """Calls from two threads on two blocks (own streams) share the GPU's workspace: the library runs them one after the
+    other, and each result equals cla_rmm_dev's."""
+    import threading
+    from systemds_amd import synth
+    cfgs = [synth.config2(scale=100), synth.config2(scale=150, n_cols=40)]
+    blks, want, bufs = [], [], []
+    for c in cfgs:
+        n, m = c["n_rows"], c["n_cols"]
+        blk = cla.build_block(n, m, c["groups"])
+        dB, d1, d2 = DevBuf.from_numpy(c["v"][:m]), DevBuf(n * 8), DevBuf(n * 8)
+        nnz = blk.rmm_dev(dB.ptr, 1, d1.ptr)
+        blks.append(blk)
+        want.append((d1.to_numpy((n, 1)), nnz))
+        bufs.append((dB, d2))
+    errors = []
+
+    def work(i):
+        try:
+            n = blks[i].n_rows
+            for _ in range(20):
+                nnz = blks[i].rmm_dev_noalloc(bufs[i][0].ptr, 1, bufs[i][1].ptr)
+                got = bufs[i][1].to_numpy((n, 1))
+                if nnz != want[i][1] or not np.array_equal(got, want[i][0]):
+                    errors.append((i, nnz))
+        except Exception as e:  # noqa: BLE001 - reported by the assertion below
+            errors.append((i, repr(e)))
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    for blk in blks:
+        blk.close()
+    assert not errors, errors
