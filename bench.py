@@ -4,7 +4,8 @@ A step = one pass of compressed X %*% v over BASELINE config 2 (10,000,000 x 100
 single-column DDC groups, 256 values per column, Zipf(1.1) uint8 codes), with the
 compressed block, v and the output resident in HBM. Prints ONE JSON line: the headline
 (`value`, `roofline`, `cpu_baseline`) plus, under `extra`, one row per other product of the
-BASELINE configs (kernel, kernel time, algorithmic bytes or flops, fraction of the bound).
+BASELINE configs (kernel, kernel time, algorithmic bytes or flops, fraction of the bound, and the CPU
+oracle's rate on the same input).
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--scale S] [--no-cpu] [--no-extra]
 """
@@ -50,6 +51,21 @@ def profiled_traffic():
     if m.group(2) != headline_source_hash():
         return None, f"stale: measured at source hash {m.group(2)}, sources now {headline_source_hash()}"
     return float(m.group(1)), f"rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, {os.path.relpath(TRAFFIC_FILE, ROOT)}"
+
+
+def cpu_row(fn, n_rows, what):
+    """CPU baseline of one row: the oracle's multithreaded restatement of the reference algorithm (a port, not the
+    SystemDS JVM) on the same compressed input as the GPU row (the whole workload: the longest, C5 t(X)%*%X, takes
+    under ten seconds a pass), host cores of this box, median of 3 passes."""
+    cores = min(len(os.sched_getaffinity(0)), int(os.environ.get("OMP_NUM_THREADS", "64")))
+    times = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        fn(cores)
+        times.append(time.perf_counter() - t0)
+    sec = statistics.median(times)
+    return {"value": n_rows / sec, "unit": "rows/s", "cores": cores, "kind": "port",
+            "sample": f"{what}: the full workload ({n_rows} rows), median of 3 passes, {sec:.3f} s per pass"}
 
 
 def time_async(blk, launch, reps, warm=2):
@@ -112,7 +128,7 @@ def extra_row(blk, launch, n_rows, algo_bytes, flops=0.0, reps=10):
     return row
 
 
-def other_rows(scale, c2, c2_blk, out):
+def other_rows(scale, c2, c2_blk, out, cpu=True):
     """The other products of C2 on the headline block, then C3, C4 and C5 (generated, uploaded, measured and
     freed one after the other)."""
     import numpy as np
@@ -139,8 +155,21 @@ def other_rows(scale, c2, c2_blk, out):
                                          2 * comp + 2 * n * 8.0)
     c2_blk.close()
     torch.cuda.empty_cache()
+    def cpu_rows(cs, legs):
+        """CPU legs of one configuration on the GPU rows' own input: legs = [(row name, what, fn(ora, G, cfg, k))]."""
+        if not cpu:
+            return
+        from oracle import cla_oracle as ora
+        G = ora.Groups(cs["groups"], cs["n_rows"], cs["n_cols"])
+        for name, what, fn in legs:
+            if name in out:
+                out[name]["cpu_baseline"] = cpu_row(lambda k: fn(ora, G, cs, k), cs["n_rows"], what)
+    ys = dy.cpu().numpy()
+    cpu_rows(c2, [("C2 X%*%B", "X%*%B", lambda ora, G, c, k: ora.rmm(G, c["B"], k)),
+                  ("C2 t(y)%*%X", "t(y)%*%X", lambda ora, G, c, k: ora.lmm(G, ys, k)),
+                  ("C2 t(X)%*%(X%*%v)", "t(X)%*%(X%*%v)", lambda ora, G, c, k: ora.mmchain(G, c["v"], None, 0, k))])
 
-    def with_block(cfg, fn):
+    def with_block(cfg, fn, legs=()):
         t0 = time.time()
         blk = capi.build_block(cfg["n_rows"], cfg["n_cols"], cfg["groups"])
         up = round(time.time() - t0, 2)
@@ -153,6 +182,7 @@ def other_rows(scale, c2, c2_blk, out):
         finally:
             blk.close()
             torch.cuda.empty_cache()
+        cpu_rows(cfg, legs)
 
     # ---- C3: t(X) %*% X (50 x 50); useful flops: the upper triangle once
     def c3_rows(blk, cfg):
@@ -160,7 +190,7 @@ def other_rows(scale, c2, c2_blk, out):
         do = torch.empty((m, m), dtype=torch.float64, device="cuda")
         yield "C3 t(X)%*%X", extra_row(blk, lambda: blk.tsmm_dev_async(do.data_ptr()), n, float(blk.device_bytes()),
                                        flops=2.0 * n * m * (m + 1) / 2)
-    with_block(synth.config3(scale=scale), c3_rows)
+    with_block(synth.config3(scale=scale), c3_rows, [("C3 t(X)%*%X", "t(X)%*%X", lambda ora, G, c, k: ora.tsmm(G, k))])
 
     # ---- C4: t(v) %*% X and X %*% u on SDC lists (compulsory bytes: delta and code bytes once, the vector once)
     def c4_rows(blk, cfg):
@@ -171,7 +201,9 @@ def other_rows(scale, c2, c2_blk, out):
         lists = float(sum(g.deltas.nbytes + g.codes.nbytes for g in cfg["groups"]))
         yield "C4 t(v)%*%X", extra_row(blk, lambda: blk.lmm_dev_async(dv4.data_ptr(), 1, do1.data_ptr()), n, lists + n * 8.0)
         yield "C4 X%*%u", extra_row(blk, lambda: blk.rmm_dev_async(du.data_ptr(), 1, do2.data_ptr()), n, lists + n * 8.0)
-    with_block(synth.config4(scale=scale), c4_rows)
+    with_block(synth.config4(scale=scale), c4_rows,
+               [("C4 t(v)%*%X", "t(v)%*%X", lambda ora, G, c, k: ora.lmm(G, c["v"].reshape(1, -1), k)),
+                ("C4 X%*%u", "X%*%u", lambda ora, G, c, k: ora.rmm(G, c["u"], k))])
 
     # ---- C5: X %*% B (20 x 10) and t(X) %*% X on the mixed block
     def c5_rows(blk, cfg):
@@ -184,7 +216,9 @@ def other_rows(scale, c2, c2_blk, out):
                                     flops=2.0 * n * m * 10, reps=5)
         yield "C5 t(X)%*%X", extra_row(blk, lambda: blk.tsmm_dev_async(do2.data_ptr()), n, comp,
                                        flops=2.0 * n * m * (m + 1) / 2, reps=5)
-    with_block(synth.config5(scale=scale), c5_rows)
+    with_block(synth.config5(scale=scale), c5_rows,
+               [("C5 X%*%B", "X%*%B", lambda ora, G, c, k: ora.rmm(G, c["B"], k)),
+                ("C5 t(X)%*%X", "t(X)%*%X", lambda ora, G, c, k: ora.tsmm(G, k))])
 
 
 def main():
@@ -234,6 +268,20 @@ def main():
         # queues the step's kernels on the block's stream; the non-zero count stays on the device
         blk.rmm_dev_async(dv.data_ptr(), 1, dout.data_ptr())
 
+    # Cold figure: the first steps after upload, clocks as the device left them (one untimed call builds what the
+    # first call builds; BASELINE's protocol of 3 warm-ups then 20 steps)
+    step()
+    blk.nnz()
+    torch.cuda.synchronize()
+    for _ in range(3):
+        step()
+    blk.nnz()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(20):
+        step()
+    torch.cuda.synchronize()
+    cold_ms_per_step = (time.perf_counter() - t0) / 20 * 1e3
     # Device warm-up (untimed, in front of the W warm-up steps): the first ~10 ms of load after idle run at
     # transient clocks on this device (per-kernel time 0.23 -> 0.28 -> 0.225 ms over the first 60 launches in
     # a rocprofv3 kernel trace), which a 20-step timed region would measure instead of the kernel.
@@ -248,16 +296,25 @@ def main():
         step()
     blk.nnz()
     torch.cuda.synchronize()
-    # whole-job throughput: wall clock over exactly K steps, device idle on both sides
+    # whole-job throughput: wall clock over exactly K steps, device idle on both sides; the same K steps are
+    # bracketed by one pair of HIP events on the stream the kernels are launched on (the kernel time of a step is
+    # that bracket / K: it cannot exceed the wall time, and it carries no per-launch event overhead)
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
+    with torch.cuda.stream(stream):
+        ev0.record(stream)
     for _ in range(args.steps):
         step()
+    with torch.cuda.stream(stream):
+        ev1.record(stream)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     nnz = blk.nnz()
     ms_per_step = elapsed / args.steps * 1e3
+    train_ms = ev0.elapsed_time(ev1) / args.steps
 
-    # dominant kernel: HIP events on the stream the kernel is launched on
+    # dominant kernel: name and algorithmic bytes from the library's own record of one more step; per-launch HIP
+    # events (with their bracket overhead) are reported as kernel_ms_events
     blk.profile(True)
     kms, kbytes, kname = [], 0.0, ""
     for _ in range(min(args.steps, 20)):
@@ -267,7 +324,10 @@ def main():
         kms.append(dom["ms"])
         kbytes, kname = dom["algo_bytes"], dom["name"]
     blk.profile(False)
-    k_ms = statistics.mean(kms)
+    n_kernels_per_step = len(ks)
+    # (a step of this workload is one launch of one kernel: the train's time per step is that kernel's duration plus
+    # the gap between two launches)
+    k_ms = train_ms if n_kernels_per_step == 1 else statistics.mean(kms)
     achieved = kbytes / (k_ms * 1e-3) / 1e9
     traffic, traffic_note = profiled_traffic() if args.scale == 1 else (None, "scaled-down run")
 
@@ -283,9 +343,9 @@ def main():
                    "nnz": int(nnz), "gen_s": round(t_gen, 2), "upload_s": round(t_upload, 2),
                    "block_bytes": int(blk.device_bytes()), "derived_bytes": int(blk.derived_bytes()),
                    "kernels_per_step": sorted({k["name"] for k in ks}),
-                   "device_warmup_steps": n_dev_warm},
+                   "device_warmup_steps": n_dev_warm, "cold_ms_per_step": cold_ms_per_step},
         "roofline": {"bound": "hbm", "kernel": kname, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "kernel_ms": k_ms, "kernel_ms_min": min(kms),
+                     "frac": achieved / HBM_PEAK_GBS, "kernel_ms": k_ms, "kernel_ms_events": statistics.mean(kms), "kernel_ms_min": min(kms),
                      "algo_bytes_per_launch": kbytes, "traffic": traffic, "traffic_source": traffic_note},
     }
 
@@ -319,7 +379,7 @@ def main():
     if not args.no_extra:
         extra = {}
         try:
-            other_rows(args.scale, cfg, blk, extra)
+            other_rows(args.scale, cfg, blk, extra, cpu=not args.no_cpu)
         except Exception as e:  # the headline stands on its own: report what was measured and why the rest is missing
             extra["error"] = repr(e)
         result["extra"] = extra
