@@ -95,18 +95,32 @@ def time_async(blk, launch, reps, warm=2):
     return ms, agg
 
 
-def extra_row(blk, launch, n_rows, algo_bytes, flops=0.0, reps=10):
+def extra_row(blk, launch, n_rows, algo_bytes, flops=0.0, reps=10, prepare=None):
     """One row of `extra`: first-call time (includes derived formats built on first use), steady-state wall
     time per call, the dominant kernel with its HIP-event time, and the fraction of the bound that limits the
     call (the larger of the HBM floor and the fp64 matrix floor) over the summed HIP-event times of all its
-    kernels."""
+    kernels. With `prepare` (a call of cla_block_prepare for this product) the row starts from a block without
+    derived formats, so that `derived_bytes_built` is this product's alone, and also gives the time of the prepare
+    call and of the first product call behind it."""
     import torch
+    if prepare:
+        blk.drop_derived()
     torch.cuda.synchronize()
     d0 = blk.derived_bytes()
     t0 = time.perf_counter()
     launch()
     blk.nnz()
     first_ms = (time.perf_counter() - t0) * 1e3
+    prep = {}
+    if prepare:
+        blk.drop_derived()
+        t0 = time.perf_counter()
+        prepare()
+        prep["prepare_ms"] = round((time.perf_counter() - t0) * 1e3, 3)
+        t0 = time.perf_counter()
+        launch()
+        blk.nnz()
+        prep["first_call_after_prepare_ms"] = round((time.perf_counter() - t0) * 1e3, 3)
     ms, ks = time_async(blk, launch, reps)
     kname = max(ks, key=lambda k: ks[k]["ms"])
     kms = ks[kname]["ms"]
@@ -117,7 +131,7 @@ def extra_row(blk, launch, n_rows, algo_bytes, flops=0.0, reps=10):
            "kernel": kname, "kernel_ms": round(kms, 5), "kernels": {k: round(v["ms"], 5) for k, v in ks.items()},
            "kernels_ms": round(ksum, 5), "algo_bytes": algo_bytes, "algo_GBs": algo_bytes / (ksum * 1e-3) / 1e9,
            "frac_hbm": algo_bytes / (ksum * 1e-3) / 1e9 / HBM_PEAK_GBS,
-           "derived_bytes_built": int(blk.derived_bytes() - d0)}
+           "derived_bytes_built": int(blk.derived_bytes() - d0), **prep}
     if flops:
         row["flops"] = flops
         row["frac_mfma_f64"] = flops / (ksum * 1e-3) / 1e12 / MFMA_F64_PEAK_TF
@@ -199,8 +213,10 @@ def other_rows(scale, c2, c2_blk, out, cpu=True):
         do1 = torch.empty((1, m), dtype=torch.float64, device="cuda")
         do2 = torch.empty((n, 1), dtype=torch.float64, device="cuda")
         lists = float(sum(g.deltas.nbytes + g.codes.nbytes for g in cfg["groups"]))
-        yield "C4 t(v)%*%X", extra_row(blk, lambda: blk.lmm_dev_async(dv4.data_ptr(), 1, do1.data_ptr()), n, lists + n * 8.0)
-        yield "C4 X%*%u", extra_row(blk, lambda: blk.rmm_dev_async(du.data_ptr(), 1, do2.data_ptr()), n, lists + n * 8.0)
+        yield "C4 t(v)%*%X", extra_row(blk, lambda: blk.lmm_dev_async(dv4.data_ptr(), 1, do1.data_ptr()), n, lists + n * 8.0,
+                                       prepare=lambda: blk.prepare(lmm_rows=1))
+        yield "C4 X%*%u", extra_row(blk, lambda: blk.rmm_dev_async(du.data_ptr(), 1, do2.data_ptr()), n, lists + n * 8.0,
+                                    prepare=lambda: blk.prepare(rmm_cols=1))
     with_block(synth.config4(scale=scale), c4_rows,
                [("C4 t(v)%*%X", "t(v)%*%X", lambda ora, G, c, k: ora.lmm(G, c["v"].reshape(1, -1), k)),
                 ("C4 X%*%u", "X%*%u", lambda ora, G, c, k: ora.rmm(G, c["u"], k))])
@@ -213,9 +229,9 @@ def other_rows(scale, c2, c2_blk, out, cpu=True):
         do2 = torch.empty((m, m), dtype=torch.float64, device="cuda")
         comp = float(blk.device_bytes())
         yield "C5 X%*%B", extra_row(blk, lambda: blk.rmm_dev_async(dB5.data_ptr(), 10, do1.data_ptr()), n, comp + n * 80.0,
-                                    flops=2.0 * n * m * 10, reps=5)
+                                    flops=2.0 * n * m * 10, reps=5, prepare=lambda: blk.prepare(rmm_cols=10))
         yield "C5 t(X)%*%X", extra_row(blk, lambda: blk.tsmm_dev_async(do2.data_ptr()), n, comp,
-                                       flops=2.0 * n * m * (m + 1) / 2, reps=5)
+                                       flops=2.0 * n * m * (m + 1) / 2, reps=5, prepare=lambda: blk.prepare(tsmm=True))
     with_block(synth.config5(scale=scale), c5_rows,
                [("C5 X%*%B", "X%*%B", lambda ora, G, c, k: ora.rmm(G, c["B"], k)),
                 ("C5 t(X)%*%X", "t(X)%*%X", lambda ora, G, c, k: ora.tsmm(G, k))])

@@ -141,6 +141,22 @@ int64_t cla_block_device_bytes(cla_handle h);
  * first call of the driver that uses them). */
 int64_t cla_block_derived_bytes(cla_handle h);
 
+/* Frees every format the library derived from the block since finalize (and the blocks it made from it for its own
+ * use); the next call that wants one builds it again. Waits for the block's stream. It has no counterpart in the reference,
+ * whose derived state (cached counts, pre-aggregates) is soft-referenced and goes under memory pressure
+ * (CG/AColGroupValue.java getCounts); here the caller decides. Returns 0 or a negative error. */
+int cla_block_drop_derived(cla_handle h);
+/* Builds now what the first call of the named products would build (so that a caller can pay for it at upload
+ * instead of inside the first multiply): each product runs once on operands of zeros in temporary device
+ * buffers (for CLA_PRODUCT_RMM an output of nRows x nColB doubles) that are freed before the call returns.
+ * nColB: columns of B of the right multiplies to come (which forms a right multiply uses depends on it; 1 for
+ * X %*% v), nRowY: rows of Y of the left multiplies; either is ignored when its product is not named. Waits for
+ * the stream. It has no counterpart in the reference. Returns 0 or a negative error. */
+#define CLA_PRODUCT_RMM 1u
+#define CLA_PRODUCT_LMM 2u
+#define CLA_PRODUCT_TSMM 4u
+int cla_block_prepare(cla_handle h, uint32_t products, int32_t nColB, int32_t nRowY);
+
 /* ---- multiply drivers ---- */
 
 /* CLALibRightMultBy.rightMultByMatrix with allowOverlap=false (RMM,

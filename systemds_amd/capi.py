@@ -18,6 +18,8 @@ _f64p = C.POINTER(C.c_double)
 
 # negative return codes of the C ABI (include/cla_hip.h, enum cla_error)
 ERR_INVALID, ERR_UNSUPPORTED, ERR_DEVICE, ERR_STATE = -1, -2, -3, -4
+# product bits of cla_block_prepare
+PRODUCT_RMM, PRODUCT_LMM, PRODUCT_TSMM = 1, 2, 4
 
 
 class ClaError(RuntimeError):
@@ -52,6 +54,8 @@ SIGNATURES = {
     "cla_block_group_num_values": (C.c_int32, [C.c_void_p, C.c_int32]),
     "cla_block_device_bytes": (C.c_int64, [C.c_void_p]),
     "cla_block_derived_bytes": (C.c_int64, [C.c_void_p]),
+    "cla_block_drop_derived": (C.c_int, [C.c_void_p]),
+    "cla_block_prepare": (C.c_int, [C.c_void_p, C.c_uint32, C.c_int32, C.c_int32]),
     "cla_rmm": (C.c_int64, [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
     "cla_rmm_dev": (C.c_int64, [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
     "cla_rmm_dev_async": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
@@ -245,6 +249,15 @@ class ClaBlock:
 
     def derived_bytes(self):
         return _check(self.lib.cla_block_derived_bytes(self.h))
+
+    def drop_derived(self):
+        """Free every format derived since finalize (cla_block_drop_derived)."""
+        _check(self.lib.cla_block_drop_derived(self.h))
+
+    def prepare(self, rmm_cols=0, lmm_rows=0, tsmm=False):
+        """Build now what the first call of the named products would build (cla_block_prepare)."""
+        mask = (PRODUCT_RMM if rmm_cols else 0) | (PRODUCT_LMM if lmm_rows else 0) | (PRODUCT_TSMM if tsmm else 0)
+        _check(self.lib.cla_block_prepare(self.h, mask, int(rmm_cols), int(lmm_rows)))
 
     # ---- host-pointer drivers (what a JNI caller uses) ----
     def rmm(self, B):

@@ -765,6 +765,91 @@ int64_t cla_block_derived_bytes(cla_handle b) {
 	return s;
 }
 
+// Everything the library derived from the block's own representation after finalize goes: the next call that wants a form builds it
+// again. (Workspaces of the host-pointer entry points are no derived forms and stay.)
+static int drop_derived(cla_block* b) {
+	if(g_device >= 0) (void) hipSetDevice(g_device);
+	if(b->stream) CLA_HIP(hipStreamSynchronize(b->stream));
+	if(b->joint) { cla_block_free(b->joint); b->joint = nullptr; b->jointSerial = 0; }
+	free_subs(b);
+	free_lmm_subs(b);
+	b->lmmSubWidth = 0;
+	dec_plans_drop(b);
+	auto drop = [](auto*& p) { if(p) { (void) hipFree((void*) p); p = nullptr; } };
+	drop(b->dSdcPlan); drop(b->dSdcDesc); drop(b->dSdcPacked);
+	b->sdcPlanGroup = -2; b->sdcPackFailed = false;
+	drop(b->dLaneMeta); drop(b->dLaneData);
+	b->laneState = 0; b->laneSlabs = 0; b->laneDictLds = 0; b->laneDictTotal = 0; b->laneLmm = false;
+	drop(b->dRowsMeta); drop(b->dRowsData);
+	b->rowsState = 0; b->rowsTbl = 0;
+	drop(b->dMfPlan);
+	b->mfState = 0;
+	drop(b->dCountsAll);
+	for(uint8_t*& p : b->expCodes) drop(p);
+	b->expCodes.clear();
+	b->expTried = false;
+	b->derivedBytes = b->dDictPad ? b->dictPadBytes : 0; // (the padded dictionary image is made at finalize and stays)
+	return 0;
+}
+
+int cla_block_drop_derived(cla_handle b) {
+	CLA_TRY
+	int rc = check_final(b);
+	if(rc) return rc;
+	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	return drop_derived(b);
+	CLA_CATCH_CODE(int)
+}
+
+static int64_t rmm_dev(cla_handle b, const double* dB, int32_t nColB, double* dOut, bool sync);
+static int64_t lmm_dev(cla_handle b, const double* dY, int32_t nRowY, double* dOut, bool sync);
+static int64_t tsmm_dev(cla_handle b, double* dOut, bool sync);
+
+int cla_block_prepare(cla_handle b, uint32_t products, int32_t nColB, int32_t nRowY) {
+	CLA_TRY
+	int rc = check_final(b);
+	if(rc) return rc;
+	if((products & ~(uint32_t) (CLA_PRODUCT_RMM | CLA_PRODUCT_LMM | CLA_PRODUCT_TSMM)) != 0 ||
+		((products & CLA_PRODUCT_RMM) && nColB <= 0) || ((products & CLA_PRODUCT_LMM) && nRowY <= 0)) {
+		set_error("prepare: unknown product bit or a product without its operand's width");
+		return -CLA_ERR_INVALID;
+	}
+	std::lock_guard<std::recursive_mutex> lk(b->mu);
+	// Each product runs once on operands of zeros in buffers of this call: the drivers build what they would build on
+	// their first call (which forms that is depends on the block, the operand's width and the options, nothing else).
+	struct Tmp {
+		double* p = nullptr;
+		~Tmp() { if(p) (void) hipFree(p); }
+		int zeros(size_t n, hipStream_t st) {
+			CLA_HIP(hipMalloc((void**) &p, std::max<size_t>(n, 1) * sizeof(double)));
+			CLA_HIP(hipMemsetAsync(p, 0, std::max<size_t>(n, 1) * sizeof(double), st));
+			return 0;
+		}
+	};
+	const bool profile = b->profile;
+	b->profile = false;
+	int64_t r = 0;
+	if(r >= 0 && (products & CLA_PRODUCT_RMM)) {
+		Tmp in, out;
+		if((rc = in.zeros((size_t) b->nCols * nColB, b->stream)) || (rc = out.zeros((size_t) b->nRows * nColB, b->stream))) r = rc;
+		else r = rmm_dev(b, in.p, nColB, out.p, true);
+	}
+	if(r >= 0 && (products & CLA_PRODUCT_LMM)) {
+		Tmp in, out;
+		if((rc = in.zeros((size_t) b->nRows * nRowY, b->stream)) || (rc = out.zeros((size_t) b->nCols * nRowY, b->stream))) r = rc;
+		else r = lmm_dev(b, in.p, nRowY, out.p, true);
+	}
+	if(r >= 0 && (products & CLA_PRODUCT_TSMM)) {
+		Tmp out;
+		if((rc = out.zeros((size_t) b->nCols * b->nCols, b->stream))) r = rc;
+		else r = tsmm_dev(b, out.p, true);
+	}
+	b->profile = profile;
+	clear_stats(b);
+	return r < 0 ? (int) r : 0;
+	CLA_CATCH_CODE(int)
+}
+
 // ---- drivers -------------------------------------------------------------
 
 // sync: wait for the driver's kernels and return its non-zero count; otherwise leave the count in the

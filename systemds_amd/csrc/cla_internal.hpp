@@ -171,6 +171,7 @@ struct cla_block {
 	// all groups single-column DDC with byte codes: dictionaries at a fixed stride of 256 entries
 	// (zero beyond nVals) followed by the groups' column indexes; built on first use
 	double* dDictPad = nullptr;
+	int64_t dictPadBytes = 0;
 	// list of SDCZeros groups + prefix sums of their nVals, as the row-tile kernels read it;
 	// built on first use for all groups (sdcPlanGroup -1) or for one group (its index)
 	int32_t* dSdcPlan = nullptr;

@@ -308,7 +308,8 @@ int ensure_dict_pad(cla_block* b) {
 		cols[g] = H.cols[0];
 	}
 	CLA_HIP(hipMalloc((void**) &b->dDictPad, img.size() * sizeof(double)));
-	b->derivedBytes += (int64_t) (img.size() * sizeof(double));
+	b->dictPadBytes = (int64_t) (img.size() * sizeof(double));
+	b->derivedBytes += b->dictPadBytes;
 	CLA_HIP(hipMemcpy(b->dDictPad, img.data(), img.size() * sizeof(double), hipMemcpyHostToDevice));
 	return 0;
 }
