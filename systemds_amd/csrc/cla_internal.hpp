@@ -180,7 +180,7 @@ struct cla_block {
 	void* dLaneData = nullptr;       // the listed groups' lists as lane-major windows, built on first use
 	int laneState = 0;               // 0 not planned yet, 1 ready, -1 the lists do not fit these kernels
 	int laneSlabs = 0, laneDictLds = 0, laneDictTotal = 0; // slabs, dictionary entries of the largest slab / of all
-	size_t laneOff[4] = {0, 0, 0, 0};
+	size_t laneOff[5] = {0, 0, 0, 0, 0};
 	bool laneLmm = false;            // every listed group has one column (the left multiply's condition)
 	cla::DecPlanCache* decPlans = nullptr; // decode kernels (k_rmm_decode.hip): plans per product shape, dropped by dec_plans_drop
 	cla::DirPlan* dirPlan = nullptr;     // plan of k_rmm_direct (dropped with the decode plans)

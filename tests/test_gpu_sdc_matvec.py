@@ -60,8 +60,9 @@ CASES = [
     # n_rows, groups, density, tuples
     (1, 3, 0.9, 4),
     (1023, 5, 0.3, 7),
-    (1025, 70, 0.05, 64),          # last window of one row, more than 64 groups (two slabs)
-    (70001, 130, 0.05, 64),
+    (1025, 70, 0.05, 64),          # last window of one row, more groups than lanes
+    (70001, 130, 0.05, 64),        # dictionaries beyond one slab's share of LDS: two slabs
+    (20000, 300, 0.05, 8),         # more groups than a chunk's tag numbers: two slabs
     (200000, 40, 0.0015, 5),       # gaps beyond 255 rows: skip entries, windows without entries
     (300007, 70, 0.001, 3),        # 2-byte offsets
     (50000, 9, 0.0002, 200),
