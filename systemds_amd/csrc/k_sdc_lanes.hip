@@ -117,9 +117,26 @@ __global__ __launch_bounds__(256) void k_lane_convert(const DGroup* __restrict__
 			nE++;
 			if(FILL && nE % LN_E == 0) flush();
 		};
+		// the lists come in aligned pieces of 16 bytes (a piece behind the end of a list lies in the slack of its allocation)
+		struct Piece {
+			u32x4 v;
+			int64_t at = -1;
+		} pd, pc;
+		auto word = [](const Piece& P, int k) { return k == 0 ? P.v.x : k == 1 ? P.v.y : k == 2 ? P.v.z : P.v.w; };
+		auto fetch = [](Piece& P, const void* src, int64_t piece) {
+			if(piece != P.at) {
+				P.at = piece;
+				P.v = *(const u32x4*) ((const uint8_t*) src + (piece << 4));
+			}
+		};
 		auto entry = [&](int rel, int di) {
 			while(nE % LN_E != 0 && rel - prev > 255) put(prev + 255, spare);
-			put(rel, (uint32_t) load_code(G.codes, G.codeWidth, di));
+			uint32_t c = 0;
+			if(FILL) { // (the groups of this form have codes of one byte)
+				fetch(pc, G.codes, (int64_t) di >> 4);
+				c = (word(pc, (di >> 2) & 3) >> (8 * (di & 3))) & 0xffu;
+			}
+			put(rel, c);
 		};
 		if(G.first >= r0 && G.first < rEnd) entry((int) (G.first - r0), 0);
 		if(win * LN_TPW < G.nTiles) {
@@ -128,7 +145,15 @@ __global__ __launch_bounds__(256) void k_lane_convert(const DGroup* __restrict__
 			int32_t row = st.row, emit = st.emit;
 			const int maxV = G.deltaWidth == 1 ? 255 : 65535;
 			for(; i < G.nDeltas; i++) {
-				const int v = G.deltaWidth == 1 ? (int) ((const uint8_t*) G.deltas)[i] : (int) ((const uint16_t*) G.deltas)[i];
+				int v;
+				if(G.deltaWidth == 1) {
+					fetch(pd, G.deltas, i >> 4);
+					v = (int) ((word(pd, (int) (i >> 2) & 3) >> (8 * (int) (i & 3))) & 0xffu);
+				}
+				else {
+					fetch(pd, G.deltas, i >> 3);
+					v = (int) ((word(pd, (int) (i >> 1) & 3) >> (16 * (int) (i & 1))) & 0xffffu);
+				}
 				const int64_t nr = (int64_t) row + (v == 0 ? maxV : v);
 				if(nr >= rEnd) break;
 				row = (int32_t) nr;

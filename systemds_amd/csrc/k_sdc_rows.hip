@@ -35,7 +35,7 @@ constexpr int RW_THREADS = RW_WAVES * 64;
 __device__ constexpr int RW_PFS[RW_QS] = {6, 4, 3, 3};
 constexpr int RW_PFN = 6 + 4 + 3 + 3;
 constexpr int RW_TBL_MAX = 16000;  // table entries of all listed groups in LDS (125 KB, next to 2 KB per wave)
-static_assert(RW_WIN == 1024 && RW_Q == 256, "a conversion block sorts the four quarters of a window");
+static_assert(RW_WIN == 1024 && RW_Q == 256 /* (a row's place in its quarter is a byte) */, "a conversion block sorts the four quarters of a window");
 
 typedef uint16_t u16x4 __attribute__((ext_vector_type(4)));
 constexpr int RB_THREADS = 1024;   // threads of a conversion block (one window)
@@ -44,7 +44,7 @@ constexpr int RB_THREADS = 1024;   // threads of a conversion block (one window)
 template <bool FILL>
 __global__ __launch_bounds__(RB_THREADS) void k_rows_build(const DGroup* __restrict__ groups, const int32_t* __restrict__ list,
 	const int32_t* __restrict__ gBase, int nL, int64_t nRows, uint32_t zeroIdx, uint32_t* __restrict__ winSize,
-	const uint64_t* __restrict__ winOff, uint2* __restrict__ hdr, uint16_t* __restrict__ perm, u16x4* __restrict__ data,
+	const uint64_t* __restrict__ winOff, uint2* __restrict__ hdr, uint8_t* __restrict__ perm, u16x4* __restrict__ data,
 	int* __restrict__ overflow) {
 	extern __shared__ uint32_t smemU[];
 	uint32_t* cnt = smemU;                        // RW_WIN
@@ -66,7 +66,7 @@ __global__ __launch_bounds__(RB_THREADS) void k_rows_build(const DGroup* __restr
 		const int cw = G.codeWidth;
 		sdc_walk_tile(G, r0, RW_WIN, [&](int rel, int di) {
 			const uint32_t slot = atomicAdd(&cnt[rel], 1u);
-			if(slot < (uint32_t) RW_KR) stage[rel * RW_KR + slot] = (uint16_t) (gb + (uint32_t) load_code(codes, cw, di));
+			if(FILL && slot < (uint32_t) RW_KR) stage[rel * RW_KR + slot] = (uint16_t) (gb + (uint32_t) load_code(codes, cw, di));
 		});
 	}
 	__syncthreads();
@@ -107,7 +107,7 @@ __global__ __launch_bounds__(RB_THREADS) void k_rows_build(const DGroup* __restr
 	if(tid < RW_SL) hdr[(size_t) win * RW_SL + tid] = make_uint2((uint32_t) (base + sl[tid]), sl[tid + 1] - sl[tid]);
 	for(int p = tid; p < RW_WIN; p += RB_THREADS) {
 		const int r = rowOf[p], j = p >> 6, lane = p & 63;
-		perm[(size_t) win * RW_WIN + p] = (uint16_t) (r % RW_Q); // (position p lies in the quarter of its row)
+		perm[(size_t) win * RW_WIN + p] = (uint8_t) (r % RW_Q); // (position p lies in the quarter of its row)
 		uint16_t* e = stage + r * RW_KR;
 		const int c = (int) min(cnt[r], (uint32_t) RW_KR);
 		for(int a = 1; a < c; a++) { // ascending positions
@@ -133,7 +133,7 @@ __global__ __launch_bounds__(RB_THREADS) void k_rows_build(const DGroup* __restr
 // ACC == false: a row starts from constRow (or zero); ACC == true: from what other groups already wrote.
 template <bool ACC>
 __global__ __launch_bounds__(RW_THREADS) void k_rmm_sdc_rows(const int32_t* __restrict__ tblIndex, int nTbl,
-	const uint2* __restrict__ hdr, const uint16_t* __restrict__ perm, const u16x4* __restrict__ data,
+	const uint2* __restrict__ hdr, const uint8_t* __restrict__ perm, const u16x4* __restrict__ data,
 	const double* __restrict__ T, int constRow, double* __restrict__ out, int64_t nRows, int nQuarters,
 	unsigned long long* __restrict__ nnz) {
 	extern __shared__ double smemD[];
@@ -151,7 +151,7 @@ __global__ __launch_bounds__(RW_THREADS) void k_rmm_sdc_rows(const int32_t* __re
 	struct Ahead {
 		u16x4 v[RW_PFN];
 		uint2 h[RW_QS];
-		uint16_t p[RW_QS];
+		uint8_t p[RW_QS];
 		double start[RW_QS];
 	};
 	struct Hdr { uint2 h[RW_QS]; };
@@ -254,7 +254,7 @@ static int rows_plan(cla_block* b) {
 	hipStream_t st = b->stream;
 	const size_t idxBytes = (sizeof(int32_t) * (size_t) nTbl + 15) / 16 * 16, listBytes = (sizeof(int32_t) * 2 * (size_t) nL + 15) / 16 * 16;
 	const size_t sizeBytes = (sizeof(uint64_t) * (size_t) nWin + 15) / 16 * 16, hdrBytes = sizeof(uint2) * (size_t) nWin * RW_SL;
-	const size_t permBytes = sizeof(uint16_t) * (size_t) nWin * RW_WIN;
+	const size_t permBytes = sizeof(uint8_t) * (size_t) nWin * RW_WIN;
 	char* meta = nullptr;
 	CLA_HIP(hipMalloc((void**) &meta, idxBytes + listBytes + sizeBytes + hdrBytes + permBytes + 16));
 	b->dRowsMeta = meta;
@@ -263,7 +263,7 @@ static int rows_plan(cla_block* b) {
 	int32_t* dBase = dList + nL;
 	uint64_t* dOff = (uint64_t*) (meta + idxBytes + listBytes); // pass 1: 32-bit sizes; pass 2: 64-bit offsets
 	uint2* dHdr = (uint2*) (meta + idxBytes + listBytes + sizeBytes);
-	uint16_t* dPerm = (uint16_t*) (meta + idxBytes + listBytes + sizeBytes + hdrBytes);
+	uint8_t* dPerm = (uint8_t*) (meta + idxBytes + listBytes + sizeBytes + hdrBytes);
 	int* dOver = (int*) (meta + idxBytes + listBytes + sizeBytes + hdrBytes + permBytes);
 	CLA_HIP(hipMemcpyAsync(dIdx, tblIndex.data(), sizeof(int32_t) * (size_t) nTbl, hipMemcpyHostToDevice, st));
 	CLA_HIP(hipMemcpyAsync(dList, list.data(), sizeof(int32_t) * (size_t) nL, hipMemcpyHostToDevice, st));
@@ -323,7 +323,7 @@ int launch_rmm_sdc_rows(cla_block* b, int constRow, int accumulate, double* dOut
 	auto go = [&](auto kernel) {
 		CLA_HIP(allow_full_lds((const void*) kernel));
 		hipLaunchKernelGGL(kernel, dim3(grid), dim3(RW_THREADS), lds, b->stream, (const int32_t*) meta, b->rowsTbl,
-			(const uint2*) (meta + b->rowsOff[0]), (const uint16_t*) (meta + b->rowsOff[1]), (const u16x4*) b->dRowsData,
+			(const uint2*) (meta + b->rowsOff[0]), (const uint8_t*) (meta + b->rowsOff[1]), (const u16x4*) b->dRowsData,
 			(const double*) b->dTables, constRow, dOut, b->nRows, nQuarters, dNnz);
 		return 0;
 	};
