@@ -242,7 +242,14 @@ __global__ __launch_bounds__(LN_LW * 64) void k_lmm_sdc_lanes(const LaneDesc* __
 	const LaneSlab S = slabs[slab];
 	// the block's share of the windows
 	const int wBeg = (int) ((int64_t) nWin * part / nParts), wEnd = (int) ((int64_t) nWin * (part + 1) / nParts);
-	for(int k = tid; k < S.dictLen; k += blockDim.x) dictL[k] = dictAll[S.dictOff + k];
+	for(int k0 = tid; k0 < S.dictLen; k0 += 8 * blockDim.x) { // eight loads in flight per thread
+		double v[8];
+#pragma unroll
+		for(int j = 0; j < 8; j++) v[j] = dictAll[S.dictOff + min(k0 + j * (int) blockDim.x, S.dictLen - 1)];
+#pragma unroll
+		for(int j = 0; j < 8; j++)
+			if(k0 + j * (int) blockDim.x < S.dictLen) dictL[k0 + j * (int) blockDim.x] = v[j];
+	}
 	for(int k = tid; k < LN_TAGS; k += blockDim.x) {
 		accS[k] = 0.0;
 		descS[k] = descPk[S.l0 + min(k, S.n - 1)];
@@ -271,7 +278,7 @@ __global__ __launch_bounds__(LN_LW * 64) void k_lmm_sdc_lanes(const LaneDesc* __
 	double yreg[LN_WIN / 64]; // Y of the window whose first unit was requested last
 	auto request_rows = [&](Ahead& A) {
 #pragma unroll
-		for(int j = 0; j < LN_LK; j++) A.buf[j] = *(base + (int64_t) min(A.c0 + j, A.c1 - 1) * w);
+		for(int j = 0; j < LN_LK; j++) A.buf[j] = __builtin_nontemporal_load(base + (int64_t) min(A.c0 + j, A.c1 - 1) * w);
 	};
 	auto request_window = [&](Ahead& A, int win) { // win < wEnd: the window's first unit
 		A.win = win; A.first = true;

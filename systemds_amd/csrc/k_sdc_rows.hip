@@ -11,12 +11,15 @@
 // values in a register - no atomics, no output tile, no barrier behind the table load.
 //
 // Layout: rows are cut into quarters of RW_Q = 256; inside a quarter the rows are sorted by their number of
-// entries (perm holds the quarter's rows in that order) and cut into 4 slices of 64; a slice stores its entries
-// in groups of four per row (8 bytes), the 64 rows of a group side by side (512 bytes, one coalesced load per
-// wave), as many groups as its longest row needs; shorter rows are padded with the position of a 0.0 behind the
-// tables. A row's entries are sorted by position, so that its sum does not depend on the order in which the lists
-// were walked. A wave takes a quarter: it sums its four slices, puts the sums back into row order through a
-// 2 KB buffer of its own in LDS and writes 256 consecutive rows.
+// entries and dealt to the 64 lanes four at a time, long rows with short ones (the rows at places i, 127 - i,
+// 128 + i and 255 - i of that order go to lane i), so that the lanes' lists are of nearly one length. A lane's list
+// is its four rows' entries one after the other in groups of two (4 bytes; an odd row ends on the position of a 0.0
+// behind the tables, a row without entries is one such group); bit 15 of a group marks a row's last group; the
+// groups of the 64 lanes lie side by side (256 bytes, one coalesced load per wave), as many as the longest lane
+// needs. perm holds, per lane, the four rows' places in the quarter. A row's entries are sorted by position, so that
+// its sum does not depend on the order in which the lists were walked. A wave takes a quarter: a lane sums along its
+// list, puts a sum into row order through a 2 KB buffer of the wave in LDS where a row ends, and the wave writes
+// 256 consecutive rows.
 #include "../../include/cla_hip.h"
 #include "cla_device.hpp"
 #include <algorithm>
@@ -25,38 +28,39 @@
 namespace cla {
 
 constexpr int RW_WIN = SDC_TILE;   // rows per window (the conversion starts from the row-tile index)
-constexpr int RW_SL = RW_WIN / 64; // slices per window
 constexpr int RW_KR = 40;          // most entries of a row (the conversion's staging area in LDS)
 constexpr int RW_Q = 256;          // rows per quarter: the unit of sorting and of a wave's work
-constexpr int RW_QS = RW_Q / 64;   // slices per quarter
+constexpr int RW_QW = RW_WIN / RW_Q; // quarters per window
+constexpr int RW_F = RW_Q / 64;    // rows per lane and quarter
 constexpr int RW_WAVES = 16;       // waves per block
 constexpr int RW_THREADS = RW_WAVES * 64;
-// entry groups of a quarter's slices that a lane requests a quarter ahead (the first slice holds the longest rows)
-__device__ constexpr int RW_PFS[RW_QS] = {6, 4, 3, 3};
-constexpr int RW_PFN = 6 + 4 + 3 + 3;
+constexpr int RW_PF = 24;          // groups of a quarter that a lane requests a quarter ahead
 constexpr int RW_TBL_MAX = 16000;  // table entries of all listed groups in LDS (125 KB, next to 2 KB per wave)
-static_assert(RW_WIN == 1024 && RW_Q == 256 /* (a row's place in its quarter is a byte) */, "a conversion block sorts the four quarters of a window");
+constexpr uint32_t RW_LAST = 0x8000u; // a row's last group
+static_assert(RW_WIN == 1024 && RW_Q == 256 && RW_F == 4 && RW_TBL_MAX < (int) RW_LAST,
+	"a conversion block sorts the four quarters of a window; a row's place in its quarter is a byte; bit 15 of a position is free");
 
-typedef uint16_t u16x4 __attribute__((ext_vector_type(4)));
 constexpr int RB_THREADS = 1024;   // threads of a conversion block (one window)
 
-// block = window. FILL == false: the window's size in entry groups into winSize. FILL == true: headers, perm, data.
+// block = window. FILL == false: the window's size in groups into winSize. FILL == true: headers, perm, data.
 template <bool FILL>
 __global__ __launch_bounds__(RB_THREADS) void k_rows_build(const DGroup* __restrict__ groups, const int32_t* __restrict__ list,
 	const int32_t* __restrict__ gBase, int nL, int64_t nRows, uint32_t zeroIdx, uint32_t* __restrict__ winSize,
-	const uint64_t* __restrict__ winOff, uint2* __restrict__ hdr, uint8_t* __restrict__ perm, u16x4* __restrict__ data,
+	const uint64_t* __restrict__ winOff, uint2* __restrict__ hdr, uint8_t* __restrict__ perm, uint32_t* __restrict__ data,
 	int* __restrict__ overflow) {
 	extern __shared__ uint32_t smemU[];
 	uint32_t* cnt = smemU;                        // RW_WIN
 	uint32_t* hist = cnt + RW_WIN;                // per quarter 64 (RW_KR + 1 used): rows per count, then first position per count
-	uint32_t* sl = hist + 256;                     // RW_SL + 1: entry groups per slice, then their prefix sums
-	uint16_t* rowOf = (uint16_t*) (sl + 32);      // RW_WIN: row at sorted position
+	uint32_t* kG = hist + 256;                     // RW_QW + 1: groups per quarter, then their prefix sums
+	uint8_t* gcnt = (uint8_t*) (kG + 32);          // RW_WIN: groups of the row at (quarter, lane, turn)
+	uint16_t* rowOf = (uint16_t*) (gcnt + RW_WIN); // RW_WIN: row at sorted position
 	uint16_t* stage = rowOf + RW_WIN;             // RW_WIN x RW_KR
 	const int tid = threadIdx.x;
 	const int win = blockIdx.x;
 	const int64_t r0 = (int64_t) win * RW_WIN;
 	for(int k = tid; k < RW_WIN; k += RB_THREADS) cnt[k] = 0;
 	if(tid < 256) hist[tid] = 0;
+	if(tid < 32) kG[tid] = 0;
 	__syncthreads();
 	// a wave walks a group's part of the window at a time (256 offsets per step, decoded with a prefix sum over the wave)
 	for(int l = tid >> 6; l < nL; l += RB_THREADS / 64) {
@@ -78,7 +82,7 @@ __global__ __launch_bounds__(RB_THREADS) void k_rows_build(const DGroup* __restr
 	}
 	if(over) *overflow = 1; // a row with more entries than the staging area holds: the caller drops the row lists
 	__syncthreads();
-	if(tid < RW_WIN / RW_Q) {
+	if(tid < RW_QW) {
 		uint32_t pos = tid * RW_Q;
 		for(int c = RW_KR; c >= 0; c--) {
 			const uint32_t n = hist[tid * 64 + c];
@@ -89,51 +93,58 @@ __global__ __launch_bounds__(RB_THREADS) void k_rows_build(const DGroup* __restr
 	__syncthreads();
 	for(int k = tid; k < RW_WIN; k += RB_THREADS) rowOf[atomicAdd(&hist[(k / RW_Q) * 64 + min(cnt[k], (uint32_t) RW_KR)], 1u)] = (uint16_t) k;
 	__syncthreads();
-	if(tid < RW_SL) sl[tid] = (min(cnt[rowOf[tid * 64]], (uint32_t) RW_KR) + 3) / 4; // the slice's first row is its longest
+	// thread = sorted position p: quarter, place s in the quarter's order -> (lane, turn)
+	const int p = tid, qt = p / RW_Q, s = p % RW_Q;
+	const int turn = s >> 6, lane = (turn & 1) ? 63 - (s & 63) : (s & 63);
+	const int r = rowOf[p];
+	const int c = (int) min(cnt[r], (uint32_t) RW_KR);
+	const int gr = max(1, (c + 1) / 2);
+	gcnt[(qt * 64 + lane) * RW_F + turn] = (uint8_t) gr;
 	__syncthreads();
-	if(tid == 0) {
-		uint32_t pos = 0;
-		for(int j = 0; j < RW_SL; j++) {
-			const uint32_t n = sl[j];
-			sl[j] = pos;
-			pos += n;
-		}
-		sl[RW_SL] = pos;
-		if(!FILL) winSize[win] = pos;
+	int before = 0, all = 0;
+#pragma unroll
+	for(int k = 0; k < RW_F; k++) {
+		const int g = gcnt[(qt * 64 + lane) * RW_F + k];
+		before += k < turn ? g : 0;
+		all += g;
 	}
-	if(!FILL) return;
+	if(turn == 0) atomicMax(&kG[qt], (uint32_t) all);
 	__syncthreads();
-	const uint64_t base = winOff[win];
-	if(tid < RW_SL) hdr[(size_t) win * RW_SL + tid] = make_uint2((uint32_t) (base + sl[tid]), sl[tid + 1] - sl[tid]);
-	for(int p = tid; p < RW_WIN; p += RB_THREADS) {
-		const int r = rowOf[p], j = p >> 6, lane = p & 63;
-		perm[(size_t) win * RW_WIN + p] = (uint8_t) (r % RW_Q); // (position p lies in the quarter of its row)
-		uint16_t* e = stage + r * RW_KR;
-		const int c = (int) min(cnt[r], (uint32_t) RW_KR);
-		for(int a = 1; a < c; a++) { // ascending positions
-			const uint16_t x = e[a];
-			int z = a - 1;
-			for(; z >= 0 && e[z] > x; z--) e[z + 1] = e[z];
-			e[z + 1] = x;
-		}
-		const int k4 = (int) (sl[j + 1] - sl[j]);
-		u16x4* dst = data + (base + sl[j]) * 64 + lane;
-		for(int q = 0; q < k4; q++) {
-			u16x4 v;
-			v.x = 4 * q + 0 < c ? e[4 * q + 0] : (uint16_t) zeroIdx;
-			v.y = 4 * q + 1 < c ? e[4 * q + 1] : (uint16_t) zeroIdx;
-			v.z = 4 * q + 2 < c ? e[4 * q + 2] : (uint16_t) zeroIdx;
-			v.w = 4 * q + 3 < c ? e[4 * q + 3] : (uint16_t) zeroIdx;
-			dst[(size_t) q * 64] = v;
-		}
+	const uint32_t mine = kG[qt];
+	uint32_t first = 0, total = 0;
+#pragma unroll
+	for(int k = 0; k < RW_QW; k++) {
+		first += k < qt ? kG[k] : 0;
+		total += kG[k];
 	}
+	if(!FILL) {
+		if(tid == 0) winSize[win] = total;
+		return;
+	}
+	const uint64_t base = winOff[win] + first;
+	if(s == 0) hdr[(size_t) win * RW_QW + qt] = make_uint2((uint32_t) base, mine);
+	perm[(((size_t) win * RW_QW + qt) * 64 + lane) * RW_F + turn] = (uint8_t) (r % RW_Q); // (position p lies in the quarter of its row)
+	uint16_t* e = stage + r * RW_KR;
+	for(int a = 1; a < c; a++) { // ascending positions
+		const uint16_t x = e[a];
+		int z = a - 1;
+		for(; z >= 0 && e[z] > x; z--) e[z + 1] = e[z];
+		e[z + 1] = x;
+	}
+	uint32_t* dst = data + (base + before) * 64 + lane;
+	for(int q = 0; q < gr; q++) {
+		const uint32_t lo = 2 * q < c ? e[2 * q] : zeroIdx, hi = 2 * q + 1 < c ? e[2 * q + 1] : zeroIdx;
+		dst[(size_t) q * 64] = lo | hi << 16 | (q == gr - 1 ? RW_LAST : 0u);
+	}
+	if(turn == RW_F - 1)
+		for(uint32_t q = (uint32_t) all; q < mine; q++) data[(base + q) * 64 + lane] = zeroIdx | zeroIdx << 16;
 }
 
-// block = 16 waves, all tables in LDS; a wave takes quarters in turn, a lane owns a row of each of their slices.
+// block = 16 waves, all tables in LDS; a wave takes quarters in turn, a lane owns four rows of each.
 // ACC == false: a row starts from constRow (or zero); ACC == true: from what other groups already wrote.
 template <bool ACC>
 __global__ __launch_bounds__(RW_THREADS) void k_rmm_sdc_rows(const int32_t* __restrict__ tblIndex, int nTbl,
-	const uint2* __restrict__ hdr, const uint8_t* __restrict__ perm, const u16x4* __restrict__ data,
+	const uint2* __restrict__ hdr, const uint32_t* __restrict__ perm, const uint32_t* __restrict__ data,
 	const double* __restrict__ T, int constRow, double* __restrict__ out, int64_t nRows, int nQuarters,
 	unsigned long long* __restrict__ nnz) {
 	extern __shared__ double smemD[];
@@ -141,75 +152,97 @@ __global__ __launch_bounds__(RW_THREADS) void k_rmm_sdc_rows(const int32_t* __re
 	const int tid = threadIdx.x, lane = tid & 63;
 	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 	double* back = smemD + (nTbl + 2) / 2 * 2 + wave * RW_Q; // this wave's sums in row order
-	for(int k = tid; k < nTbl; k += RW_THREADS) tbl[k] = T[tblIndex[k]];
+	{ // all of a thread's table values requested before the first is stored (two dependent loads each)
+		constexpr int TPT = (RW_TBL_MAX + RW_THREADS - 1) / RW_THREADS;
+		int32_t ti[TPT];
+		double tv[TPT];
+#pragma unroll
+		for(int j = 0; j < TPT; j++) ti[j] = tblIndex[min(j * RW_THREADS + tid, nTbl - 1)];
+#pragma unroll
+		for(int j = 0; j < TPT; j++) tv[j] = T[ti[j]];
+#pragma unroll
+		for(int j = 0; j < TPT; j++)
+			if(j * RW_THREADS + tid < nTbl) tbl[j * RW_THREADS + tid] = tv[j];
+	}
 	if(tid == 0) tbl[nTbl] = 0.0;
 	const double init = !ACC && constRow >= 0 ? T[constRow] : 0.0;
 	__syncthreads();
 	int cntNz = 0;
-	// Requested a quarter ahead (two register sets take turns): the first entry groups of its slices, the lane's
-	// rows, the start values; two quarters ahead: the slices' headers. The work on a set is straight-line code.
+	// Requested a quarter ahead (two register sets take turns): the first groups of its lists, the lane's rows, the
+	// start values; two quarters ahead: the quarter's header. The work on a set is straight-line code.
 	struct Ahead {
-		u16x4 v[RW_PFN];
-		uint2 h[RW_QS];
-		uint8_t p[RW_QS];
-		double start[RW_QS];
+		uint32_t v[RW_PF];
+		uint2 h;
+		uint32_t p;
+		double start[RW_F];
 	};
-	struct Hdr { uint2 h[RW_QS]; };
-	auto header = [&](int qt) {
-		Hdr H;
-		const uint2* hp = hdr + (size_t) min(qt, nQuarters - 1) * RW_QS;
+	// (a vector load although the address is uniform: a scalar load is counted with the LDS reads, whose waits would
+	// then wait for it too)
+	int vzero = 0;
+	asm volatile("" : "+v"(vzero));
+	auto header = [&](int qt) { return hdr[min(qt, nQuarters - 1) + vzero]; };
+	auto request = [&](Ahead& A, int qt, const uint2 h) { // qt < nQuarters
+		A.h = make_uint2((uint32_t) __builtin_amdgcn_readfirstlane((int) h.x), (uint32_t) __builtin_amdgcn_readfirstlane((int) h.y));
+		const uint32_t* src = data + (size_t) A.h.x * 64 + lane;
+		const int kq = (int) A.h.y; // (at least four groups: a row has one)
 #pragma unroll
-		for(int j = 0; j < RW_QS; j++) H.h[j] = hp[j];
-		return H;
-	};
-	auto request = [&](Ahead& A, int qt, const Hdr& H) { // qt < nQuarters
-		int o = 0;
+		for(int q = 0; q < RW_PF; q++) A.v[q] = __builtin_nontemporal_load(src + (size_t) min(q, kq - 1) * 64);
+		A.p = perm[(size_t) qt * 64 + lane];
 #pragma unroll
-		for(int j = 0; j < RW_QS; j++) {
-			A.h[j] = H.h[j];
-			const u16x4* src = data + (size_t) H.h[j].x * 64 + lane;
-			const int k4 = (int) H.h[j].y;
-#pragma unroll
-			for(int q = 0; q < RW_PFS[j]; q++) A.v[o + q] = src[(size_t) min(q, max(k4 - 1, 0)) * 64]; // (a group of slack lies behind the last slice)
-			o += RW_PFS[j];
-			A.p[j] = perm[(size_t) qt * RW_Q + j * 64 + lane];
+		for(int j = 0; j < RW_F; j++) {
 			A.start[j] = init;
 			if(ACC) A.start[j] = out[min((int64_t) qt * RW_Q + j * 64 + lane, nRows - 1)]; // (a template parameter: a load under a run-time branch is waited for at the branch's end)
 		}
 	};
 	const int step = gridDim.x * RW_WAVES;
-	auto work = [&](Ahead& A, Ahead& B, int qt, Hdr& hNext) { // A holds the requests of `qt`, hNext the headers of qt + step
+	auto work = [&](Ahead& A, Ahead& B, int qt, uint2& hNext) { // A holds the requests of `qt`, hNext the header of qt + step
 		request(B, min(qt + step, nQuarters - 1), hNext);
 		hNext = header(qt + 2 * step);
-		int o = 0;
+		const int kq = (int) A.h.y;
+		uint32_t pw = A.p;
+		double acc = 0.0;
+		auto close = [&](uint32_t e) { // a group with bit 15 set ends the row at hand
+			if(e & RW_LAST) {
+				back[pw & 0xffu] = acc;
+				acc = 0.0;
+				pw >>= 8;
+			}
+		};
+		const uint32_t none = (uint32_t) nTbl * 0x00010001u; // a group of two 0.0
+		// four groups' table values requested before the first is added (a row's end is a branch: the compiler does not
+		// move LDS reads across it)
 #pragma unroll
-		for(int j = 0; j < RW_QS; j++) {
-			const int k4 = (int) A.h[j].y;
-			double acc = 0.0;
+		for(int q0 = 0; q0 < RW_PF; q0 += 4) {
+			if(q0 < kq) {
+				uint32_t e[4];
+				double a[4], b2[4];
 #pragma unroll
-			for(int q = 0; q < RW_PFS[j]; q++) {
-				if(q < k4) {
-					const u16x4 e = A.v[o + q];
-					const double a = tbl[e.x], b2 = tbl[e.y], c = tbl[e.z], d = tbl[e.w];
-					acc = (((acc + a) + b2) + c) + d;
+				for(int j = 0; j < 4; j++) {
+					e[j] = q0 + j < kq ? A.v[q0 + j] : none;
+					a[j] = tbl[e[j] & (RW_LAST - 1)];
+					b2[j] = tbl[e[j] >> 16];
+				}
+#pragma unroll
+				for(int j = 0; j < 4; j++) {
+					acc = (acc + a[j]) + b2[j];
+					close(e[j]);
 				}
 			}
-			const u16x4* src = data + (size_t) A.h[j].x * 64 + lane;
-			for(int q = RW_PFS[j]; q < k4; q++) {
-				const u16x4 e = src[(size_t) q * 64];
-				acc = (((acc + tbl[e.x]) + tbl[e.y]) + tbl[e.z]) + tbl[e.w];
-			}
-			o += RW_PFS[j];
-			back[A.p[j]] = acc;
+		}
+		const uint32_t* src = data + (size_t) A.h.x * 64 + lane;
+		for(int q = RW_PF; q < kq; q++) {
+			const uint32_t e = src[(size_t) q * 64];
+			acc = (acc + tbl[e & (RW_LAST - 1)]) + tbl[e >> 16];
+			close(e);
 		}
 		__builtin_amdgcn_wave_barrier(); // LDS serves a wave's accesses in order: the reads below see the sums
 #pragma unroll
-		for(int j = 0; j < RW_QS; j++) {
+		for(int j = 0; j < RW_F; j++) {
 			const int64_t r = (int64_t) qt * RW_Q + j * 64 + lane;
 			const double res = A.start[j] + back[j * 64 + lane];
 			if(r < nRows) {
 				cntNz += res != 0.0;
-				out[r] = res;
+				__builtin_nontemporal_store(res, &out[r]);
 			}
 		}
 		__builtin_amdgcn_wave_barrier();
@@ -218,7 +251,7 @@ __global__ __launch_bounds__(RW_THREADS) void k_rmm_sdc_rows(const int32_t* __re
 	if(q0 < nQuarters) {
 		Ahead A, B;
 		request(A, q0, header(q0));
-		Hdr hNext = header(q0 + step);
+		uint2 hNext = header(q0 + step);
 		for(int qt = q0; qt < nQuarters; qt += 2 * step) {
 			work(A, B, qt, hNext);
 			if(qt + step < nQuarters) work(B, A, qt + step, hNext);
@@ -253,7 +286,7 @@ static int rows_plan(cla_block* b) {
 	}
 	hipStream_t st = b->stream;
 	const size_t idxBytes = (sizeof(int32_t) * (size_t) nTbl + 15) / 16 * 16, listBytes = (sizeof(int32_t) * 2 * (size_t) nL + 15) / 16 * 16;
-	const size_t sizeBytes = (sizeof(uint64_t) * (size_t) nWin + 15) / 16 * 16, hdrBytes = sizeof(uint2) * (size_t) nWin * RW_SL;
+	const size_t sizeBytes = (sizeof(uint64_t) * (size_t) nWin + 15) / 16 * 16, hdrBytes = sizeof(uint2) * (size_t) nWin * RW_QW;
 	const size_t permBytes = sizeof(uint8_t) * (size_t) nWin * RW_WIN;
 	char* meta = nullptr;
 	CLA_HIP(hipMalloc((void**) &meta, idxBytes + listBytes + sizeBytes + hdrBytes + permBytes + 16));
@@ -269,7 +302,7 @@ static int rows_plan(cla_block* b) {
 	CLA_HIP(hipMemcpyAsync(dList, list.data(), sizeof(int32_t) * (size_t) nL, hipMemcpyHostToDevice, st));
 	CLA_HIP(hipMemcpyAsync(dBase, gBase.data(), sizeof(int32_t) * (size_t) nL, hipMemcpyHostToDevice, st));
 	CLA_HIP(hipMemsetAsync(dOver, 0, sizeof(int), st));
-	const size_t lds = sizeof(uint32_t) * (RW_WIN + 256 + 32) + sizeof(uint16_t) * ((size_t) RW_WIN + (size_t) RW_WIN * RW_KR);
+	const size_t lds = sizeof(uint32_t) * (RW_WIN + 256 + 32) + RW_WIN + sizeof(uint16_t) * ((size_t) RW_WIN + (size_t) RW_WIN * RW_KR);
 	CLA_HIP(allow_full_lds((const void*) k_rows_build<false>));
 	CLA_HIP(allow_full_lds((const void*) k_rows_build<true>));
 	hipLaunchKernelGGL(k_rows_build<false>, dim3(nWin), dim3(RB_THREADS), lds, st, b->dGroups, dList, dBase, nL, b->nRows, (uint32_t) nTbl,
@@ -288,16 +321,16 @@ static int rows_plan(cla_block* b) {
 		total += sizes[w];
 	}
 	if(total > 0xfffffff0ull) return 0; // (headers hold 32-bit group offsets)
-	const size_t dataBytes = (size_t) (total + 1) * 64 * sizeof(u16x4);
+	const size_t dataBytes = (size_t) (total + 1) * 64 * sizeof(uint32_t);
 	size_t freeB = 0, totalB = 0;
 	CLA_HIP(hipMemGetInfo(&freeB, &totalB));
 	if(dataBytes + ((size_t) 1 << 30) > freeB) return 0;
 	CLA_HIP(hipMalloc((void**) &b->dRowsData, dataBytes));
 	b->derivedBytes += (int64_t) (idxBytes + listBytes + sizeBytes + hdrBytes + permBytes + dataBytes);
-	CLA_HIP(hipMemsetAsync((char*) b->dRowsData + dataBytes - 64 * sizeof(u16x4), 0, 64 * sizeof(u16x4), st));
+	CLA_HIP(hipMemsetAsync((char*) b->dRowsData + dataBytes - 64 * sizeof(uint32_t), 0, 64 * sizeof(uint32_t), st));
 	CLA_HIP(hipMemcpyAsync(dOff, offs.data(), sizeof(uint64_t) * (size_t) nWin, hipMemcpyHostToDevice, st));
 	hipLaunchKernelGGL(k_rows_build<true>, dim3(nWin), dim3(RB_THREADS), lds, st, b->dGroups, dList, dBase, nL, b->nRows, (uint32_t) nTbl,
-		nullptr, dOff, dHdr, dPerm, (u16x4*) b->dRowsData, dOver);
+		nullptr, dOff, dHdr, dPerm, (uint32_t*) b->dRowsData, dOver);
 	CLA_HIP(hipGetLastError());
 	CLA_HIP(hipStreamSynchronize(st)); // `offs` goes out of scope
 	b->rowsTbl = nTbl;
@@ -323,7 +356,7 @@ int launch_rmm_sdc_rows(cla_block* b, int constRow, int accumulate, double* dOut
 	auto go = [&](auto kernel) {
 		CLA_HIP(allow_full_lds((const void*) kernel));
 		hipLaunchKernelGGL(kernel, dim3(grid), dim3(RW_THREADS), lds, b->stream, (const int32_t*) meta, b->rowsTbl,
-			(const uint2*) (meta + b->rowsOff[0]), (const uint8_t*) (meta + b->rowsOff[1]), (const u16x4*) b->dRowsData,
+			(const uint2*) (meta + b->rowsOff[0]), (const uint32_t*) (meta + b->rowsOff[1]), (const uint32_t*) b->dRowsData,
 			(const double*) b->dTables, constRow, dOut, b->nRows, nQuarters, dNnz);
 		return 0;
 	};
