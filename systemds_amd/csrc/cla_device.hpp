@@ -65,6 +65,38 @@ __device__ __forceinline__ void count_add(unsigned long long* counter, int local
 	if((threadIdx.x & (WAVE - 1)) == 0 && s != 0) atomicAdd(counter, (unsigned long long) s);
 }
 
+// Tail of a left multiply whose kernel is the only one of the call: every block comes here behind its last add into
+// out; the last one to arrive counts the non-zeros of out[0 .. n) into *nnz and leaves *done at zero for the next
+// launch (the same is what a kernel of its own behind this one would do; done == nullptr: no tail).
+__device__ __forceinline__ void lmm_tail(unsigned* done, unsigned nBlocks, const double* out, int n, unsigned long long* nnz) {
+	if(done == nullptr) return;
+	__shared__ unsigned ticketS;
+	__shared__ int partS[16];
+	// this thread's adds have been acknowledged before the block takes its ticket (the adds, the ticket and the reads
+	// below are all performed at device scope, past the caches that the chip's parts do not share: no cache has to be
+	// written back or invalidated, which a fence would do)
+	asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+	__syncthreads();
+	if(threadIdx.x == 0) ticketS = atomicAdd(done, 1u);
+	__syncthreads();
+	if(ticketS != nBlocks - 1) return;
+	int cnt = 0;
+	for(int i = threadIdx.x; i < n; i += blockDim.x) {
+		// (read where the other blocks' adds were performed, not from a cache of this CU)
+		const unsigned long long bits = __hip_atomic_load((const unsigned long long*) out + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+		cnt += (bits << 1) != 0ull; // != 0.0 (a NaN counts, a negative zero does not)
+	}
+	cnt = wave_sum_i32(cnt);
+	if((threadIdx.x & (WAVE - 1)) == 0) partS[threadIdx.x >> 6] = cnt;
+	__syncthreads();
+	if(threadIdx.x == 0) {
+		int s = 0;
+		for(unsigned w = 0; w < (blockDim.x + WAVE - 1) / WAVE; w++) s += partS[w];
+		*nnz = (unsigned long long) s;
+		*done = 0;
+	}
+}
+
 // Largest j in [0, nRuns) with runStart[j] <= row (runStart[0] == 0).
 __device__ __forceinline__ int rle_find(const int32_t* __restrict__ runStart, int nRuns, int32_t row) {
 	int lo = 0, hi = nRuns - 1;

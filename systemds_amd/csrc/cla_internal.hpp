@@ -193,8 +193,12 @@ struct cla_block {
 	void* dRowsData = nullptr;       // the listed groups' entries as row lists, built on first use
 	int rowsState = 0, rowsTbl = 0;  // 0 not planned yet, 1 ready, -1 the lists do not fit; table entries of all listed groups
 	size_t rowsOff[2] = {0, 0};
+	size_t rowsColOff = 0;           // the table entries' columns inside dRowsMeta
+	bool rowsFusable = false;        // the row-list kernel can make its tables itself (single-column lists only, nothing else in the block)
 	bool sdcPackFailed = false;
 	bool dictNonFinite = false;      // some dictionary holds an infinity or a NaN (set at finalize): the left multiply then sums Y per tuple first, as the reference does
+	bool lmmTailWanted = false;      // left multiply: a kernel that serves the whole block may count the result's non-zeros itself (no constants to add)
+	bool lmmTailDone = false;        // ... and one has: no finishing kernel behind it
 	bool preUsed = false;            // left multiply: some kernel of the call wrote pre-aggregates (k_lmm_post has work)
 	uint32_t* dSdcPacked = nullptr;  // all listed groups' entries as (code << 16 | row inside its 4096-row tile), built on first use
 	int sdcPlanGroup = -2;
@@ -246,8 +250,11 @@ int launch_lmm_u8(cla_block* b, const double* dY, int p, double* dPre);
 int launch_lmm_u8_dot(cla_block* b, const double* dY, int p, double* dOut);
 int launch_lmm_sdc_tiles(cla_block* b, const double* dY, int p, double* dPre, int onlyGroup, double* dOut);
 int launch_lmm_sdc_lanes(cla_block* b, const double* dY, int p, double* dOut);
+int sdc_plan_all(cla_block* b); // the list of the block's SDCZeros groups with entries (b->sdcList)
 int launch_rmm_sdc_lanes(cla_block* b, int constRow, int accumulate, double* dOut, unsigned long long* dNnz);
-int launch_rmm_sdc_rows(cla_block* b, int constRow, int accumulate, double* dOut, unsigned long long* dNnz);
+int launch_rmm_sdc_rows(cla_block* b, int constRow, int accumulate, double* dOut, unsigned long long* dNnz, const double* dU = nullptr,
+	unsigned long long* nnzNext = nullptr);
+bool rows_fusable(cla_block* b);
 int launch_rmm_sdc_tiles(cla_block* b, int q, int constRow, int accumulate, double* dOut, unsigned long long* dNnz);
 int launch_tsmm_decode(cla_block* b, double* dOut);
 int launch_tsmm_direct(cla_block* b, double* dOut);

@@ -324,13 +324,30 @@ int launch_lmm(cla_block* b, const double* dY, int p, double* dOut, unsigned lon
 	if(rc) return rc;
 	double* dPre = b->dTables;
 	double* dRs = b->dTables + (size_t) p * b->totalVals;
-	CLA_HIP(hipMemsetAsync(dPre, 0, sizeof(double) * ((size_t) p * b->totalVals + (size_t) p), st));
 	CLA_HIP(hipMemsetAsync(dOut, 0, sizeof(double) * (size_t) p * b->nCols, st));
-	CLA_HIP(hipMemsetAsync(dNnz, 0, sizeof(unsigned long long), st));
-	// single-column DDC groups on byte codes: contributions go straight into dOut
+	// Blocks that one kernel serves whole (byte-code DDC groups of one column; SDCZeros lists only) and that have no
+	// constants to add: that kernel also counts the result's non-zeros, and nothing else runs.
 	b->preUsed = false;
-	const int dot = nRows > 0 ? launch_lmm_u8_dot(b, dY, p, dOut) : 1;
+	b->lmmTailWanted = !b->hasConst && dNnz == b->dCounters && (int64_t) p * b->nCols < ((int64_t) 1 << 30);
+	b->lmmTailDone = false;
+	int dot = nRows > 0 ? launch_lmm_u8_dot(b, dY, p, dOut) : 1;
 	if(dot < 0) return dot;
+	if(dot != 0 && nRows > 0 && b->lmmTailWanted && b->opt.sdcLanes && !b->dictNonFinite && b->hasSdc && !b->hasUnc && !b->hasRle) {
+		bool onlyLists = true;
+		for(int g = 0; g < nG && onlyLists; g++) onlyLists = b->groups[g].d.type == G_SDCZ && b->groups[g].d.nOffsets > 0;
+		if(onlyLists) {
+			if((rc = sdc_plan_all(b))) return rc;
+			const int r = launch_lmm_sdc_lanes(b, dY, p, dOut);
+			if(r < 0) return r;
+		}
+	}
+	b->lmmTailWanted = false;
+	if(b->lmmTailDone) {
+		CLA_HIP(hipGetLastError());
+		return 0;
+	}
+	CLA_HIP(hipMemsetAsync(dPre, 0, sizeof(double) * ((size_t) p * b->totalVals + (size_t) p), st));
+	CLA_HIP(hipMemsetAsync(dNnz, 0, sizeof(unsigned long long), st));
 	if(dot != 0 && (rc = run_preagg(b, dY, p, dPre, -1, dOut))) return rc;
 
 	int64_t rowsPerBlock = 256 * 1024;

@@ -184,7 +184,7 @@ __device__ __forceinline__ void u8_dot(const CodeVec<1, RPT> (&cv)[NB], const ch
 template <int PER, int NB, int LB, int LN>
 __global__ __launch_bounds__(LD_THREADS, 4) void k_lmm_u8_dot(const uint8_t* __restrict__ arena, size_t arenaStride, int nGroups,
 	const double* __restrict__ dictPad, const int32_t* __restrict__ col0, const double* __restrict__ Y, int64_t nRows,
-	double* __restrict__ out, int nCols) {
+	double* __restrict__ out, int nCols, unsigned* __restrict__ done, unsigned long long* __restrict__ nnz) {
 	static_assert(PER % (2 * NB) == 0, "a slab holds whole ping/pong turns");
 	extern __shared__ double smem[];
 	double* tbl = smem;                 // PER * 256: dictionaries of the current slab
@@ -290,6 +290,7 @@ __global__ __launch_bounds__(LD_THREADS, 4) void k_lmm_u8_dot(const uint8_t* __r
 		for(int k = 0; k < LD_SLOTS; k++) v += slots[g * LD_SLOTS + k];
 		if(v != 0.0) unsafeAtomicAdd(&out[(size_t) blockIdx.y * nCols + col0[g]], v);
 	}
+	lmm_tail(done, gridDim.x * gridDim.y, out, (int) gridDim.y * nCols, nnz);
 }
 
 // All groups DDC with byte codes in one arena and one column each: the dictionaries at a fixed stride of
@@ -336,8 +337,10 @@ int launch_lmm_u8_dot(cla_block* b, const double* dY, int p, double* dOut) {
 	Prof pf(b, "k_lmm_u8_dot", (long) grid * p, LD_THREADS, (long) lds, algo);
 	auto kern = k_lmm_u8_dot<PER, 5, 4, 2>;
 	CLA_HIP(allow_full_lds((const void*) kern));
+	const bool tail = b->lmmTailWanted; // (this kernel serves every group of the block)
 	hipLaunchKernelGGL(kern, dim3(grid, p), dim3(LD_THREADS), lds, b->stream, b->dArena, b->arenaStride, nG, b->dDictPad, dCol0, dY,
-		b->nRows, dOut, b->nCols);
+		b->nRows, dOut, b->nCols, tail ? (unsigned*) (b->dCounters + 6) : nullptr, b->dCounters);
+	b->lmmTailDone = tail;
 	CLA_HIP(hipGetLastError());
 	return 0;
 }

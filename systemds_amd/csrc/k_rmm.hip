@@ -579,6 +579,18 @@ int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned lon
 		b->nnzSlot = b->nnzRot;
 		dNnz = b->dCounters + b->nnzSlot;
 	}
+	// Blocks of single-column SDCZeros lists only: the row-list kernel makes its tables from the dictionaries and
+	// counts likewise into a counter that the call before has cleared: the only launch.
+	if(q == 1 && !squares && !noAlloc && !u8Path && b->opt.sdcRows && nRows > 0 && dNnz == b->dCounters && rows_fusable(b)) {
+		b->nnzSlot = b->nnzRot;
+		const int r = launch_rmm_sdc_rows(b, -1, 0, dOut, b->dCounters + b->nnzSlot, dB, b->dCounters + (b->nnzRot % 3 + 1));
+		if(r < 0) return r;
+		if(r == 0) {
+			b->nnzRot = b->nnzRot % 3 + 1;
+			return 0;
+		}
+		b->nnzSlot = 0;
+	}
 	// K1 (also clears the non-zero counter)
 	if(!fused || b->hasConst) {
 		const int nK1 = fused ? 0 : nG; // fused: the constants' row only

@@ -229,7 +229,7 @@ __device__ __forceinline__ void ln_lmm_chunk(const u32x4 v, const double* yt, co
 __global__ __launch_bounds__(LN_LW * 64) void k_lmm_sdc_lanes(const LaneDesc* __restrict__ desc,
 	const LaneSlab* __restrict__ slabs, int nSlabs, const double* __restrict__ dictAll, const uint32_t* __restrict__ descPk,
 	int dictLds, const uint32_t* __restrict__ chunkStart, const u32x4* __restrict__ data, const double* __restrict__ Y,
-	int64_t nRows, int nWin, double* __restrict__ out, int nCols) {
+	int64_t nRows, int nWin, double* __restrict__ out, int nCols, unsigned* __restrict__ done, unsigned long long* __restrict__ nnz) {
 	extern __shared__ double smem[];
 	const int tid = threadIdx.x, lane = tid & 63, nWaves = blockDim.x >> 6;
 	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6); // (uniform: the chunk starts below come by scalar loads)
@@ -346,6 +346,7 @@ __global__ __launch_bounds__(LN_LW * 64) void k_lmm_sdc_lanes(const LaneDesc* __
 	if(live && sum.tag < (uint32_t) LN_TAGS) unsafeAtomicAdd(&accS[sum.tag], (sum.acc[0] + sum.acc[1]) + (sum.acc[2] + sum.acc[3]));
 	__syncthreads();
 	for(int k = tid; k < S.n; k += blockDim.x) unsafeAtomicAdd(&out[(size_t) blockIdx.y * nCols + desc[S.l0 + k].col0], accS[k]);
+	lmm_tail(done, gridDim.x * gridDim.y, out, (int) gridDim.y * nCols, nnz);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -644,11 +645,15 @@ int launch_lmm_sdc_lanes(cla_block* b, const double* dY, int p, double* dOut) {
 	char* meta = (char*) b->dLaneMeta;
 	double algo = (double) b->nRows * 8 * p;
 	for(int g : b->sdcList) algo += (double) p * ((double) b->groups[g].d.nDeltas * b->groups[g].d.deltaWidth + (double) b->groups[g].d.nOffsets);
+	// (the block's only groups are the listed ones: this kernel's sums are the whole result)
+	const bool tail = b->lmmTailWanted && b->sdcList.size() == b->groups.size();
 	Prof pf(b, "k_lmm_sdc_lanes", (long) parts * nS * p, waves * 64, (long) lds, algo);
 	CLA_HIP(allow_full_lds((const void*) k_lmm_sdc_lanes));
 	hipLaunchKernelGGL(k_lmm_sdc_lanes, dim3((unsigned) (parts * nS), p), dim3(waves * 64), lds, b->stream, (const LaneDesc*) meta,
 		(const LaneSlab*) (meta + b->laneOff[0]), nS, (const double*) (meta + b->laneOff[1]), (const uint32_t*) (meta + b->laneOff[3]),
-		b->laneDictLds, (const uint32_t*) (meta + b->laneOff[4]), (const u32x4*) b->dLaneData, dY, b->nRows, nWin, dOut, b->nCols);
+		b->laneDictLds, (const uint32_t*) (meta + b->laneOff[4]), (const u32x4*) b->dLaneData, dY, b->nRows, nWin, dOut, b->nCols,
+		tail ? (unsigned*) (b->dCounters + 6) : nullptr, b->dCounters);
+	b->lmmTailDone = tail;
 	CLA_HIP(hipGetLastError());
 	return 0;
 }

@@ -142,11 +142,15 @@ __global__ __launch_bounds__(RB_THREADS) void k_rows_build(const DGroup* __restr
 
 // block = 16 waves, all tables in LDS; a wave takes quarters in turn, a lane owns four rows of each.
 // ACC == false: a row starts from constRow (or zero); ACC == true: from what other groups already wrote.
-template <bool ACC>
+// FUSE (blocks of single-column lists only, nothing to add): the kernel makes the tables itself, T being the block's
+// dictionaries and u the vector: table value = dictionary value * u[column]; block 0 clears *nnzNext, the counter of
+// the next call, so that no other kernel runs in a call.
+template <bool ACC, bool FUSE>
 __global__ __launch_bounds__(RW_THREADS) void k_rmm_sdc_rows(const int32_t* __restrict__ tblIndex, int nTbl,
 	const uint2* __restrict__ hdr, const uint32_t* __restrict__ perm, const uint32_t* __restrict__ data,
 	const double* __restrict__ T, int constRow, double* __restrict__ out, int64_t nRows, int nQuarters,
-	unsigned long long* __restrict__ nnz) {
+	unsigned long long* __restrict__ nnz, const int32_t* __restrict__ tblCol, const double* __restrict__ u,
+	unsigned long long* __restrict__ nnzNext) {
 	extern __shared__ double smemD[];
 	double* tbl = smemD;                 // nTbl values and a 0.0
 	const int tid = threadIdx.x, lane = tid & 63;
@@ -160,11 +164,19 @@ __global__ __launch_bounds__(RW_THREADS) void k_rmm_sdc_rows(const int32_t* __re
 		for(int j = 0; j < TPT; j++) ti[j] = tblIndex[min(j * RW_THREADS + tid, nTbl - 1)];
 #pragma unroll
 		for(int j = 0; j < TPT; j++) tv[j] = T[ti[j]];
+		if(FUSE) {
+			double uv[TPT];
+#pragma unroll
+			for(int j = 0; j < TPT; j++) uv[j] = u[tblCol[min(j * RW_THREADS + tid, nTbl - 1)]];
+#pragma unroll
+			for(int j = 0; j < TPT; j++) tv[j] = __dmul_rn(tv[j], uv[j]);
+		}
 #pragma unroll
 		for(int j = 0; j < TPT; j++)
 			if(j * RW_THREADS + tid < nTbl) tbl[j * RW_THREADS + tid] = tv[j];
 	}
 	if(tid == 0) tbl[nTbl] = 0.0;
+	if(FUSE && blockIdx.x == 0 && tid == 0) *nnzNext = 0;
 	const double init = !ACC && constRow >= 0 ? T[constRow] : 0.0;
 	__syncthreads();
 	int cntNz = 0;
@@ -279,13 +291,20 @@ static int rows_plan(cla_block* b) {
 	if(nTbl > RW_TBL_MAX || nTbl >= 65535) return 0; // an entry is a 16-bit position; all tables sit in LDS
 	if(entries > (double) b->nRows * (RW_KR / 2)) return 0; // dense lists: rows too long for the staging area
 	if(sizeof(double) * ((size_t) nTbl + 2 + (size_t) RW_WAVES * RW_Q) > (size_t) std::min(g_ldsPerBlock, 160 * 1024)) return 0;
-	std::vector<int32_t> tblIndex(nTbl);
+	std::vector<int32_t> tblIndex(nTbl), tblCol(nTbl);
+	// (fusable: the listed groups are all of the block and have one column each, so that a group's dictionary sits in
+	// the block's dictionary buffer where its table sits in the table buffer)
+	bool fusable = (size_t) nL == b->groups.size() && !b->hasConst && b->dAllDict != nullptr;
 	for(int l = 0; l < nL; l++) {
 		const DGroup& G = b->groups[list[l]].d;
-		for(int k = 0; k < G.nVals; k++) tblIndex[gBase[l] + k] = G.tblOff + k;
+		fusable = fusable && G.nColG == 1 && G.dict == b->dAllDict + G.tblOff;
+		for(int k = 0; k < G.nVals; k++) {
+			tblIndex[gBase[l] + k] = G.tblOff + k;
+			tblCol[gBase[l] + k] = b->groups[list[l]].cols[0];
+		}
 	}
 	hipStream_t st = b->stream;
-	const size_t idxBytes = (sizeof(int32_t) * (size_t) nTbl + 15) / 16 * 16, listBytes = (sizeof(int32_t) * 2 * (size_t) nL + 15) / 16 * 16;
+	const size_t idxBytes = 2 * ((sizeof(int32_t) * (size_t) nTbl + 15) / 16 * 16), listBytes = (sizeof(int32_t) * 2 * (size_t) nL + 15) / 16 * 16;
 	const size_t sizeBytes = (sizeof(uint64_t) * (size_t) nWin + 15) / 16 * 16, hdrBytes = sizeof(uint2) * (size_t) nWin * RW_QW;
 	const size_t permBytes = sizeof(uint8_t) * (size_t) nWin * RW_WIN;
 	char* meta = nullptr;
@@ -299,6 +318,7 @@ static int rows_plan(cla_block* b) {
 	uint8_t* dPerm = (uint8_t*) (meta + idxBytes + listBytes + sizeBytes + hdrBytes);
 	int* dOver = (int*) (meta + idxBytes + listBytes + sizeBytes + hdrBytes + permBytes);
 	CLA_HIP(hipMemcpyAsync(dIdx, tblIndex.data(), sizeof(int32_t) * (size_t) nTbl, hipMemcpyHostToDevice, st));
+	CLA_HIP(hipMemcpyAsync((char*) dIdx + idxBytes / 2, tblCol.data(), sizeof(int32_t) * (size_t) nTbl, hipMemcpyHostToDevice, st));
 	CLA_HIP(hipMemcpyAsync(dList, list.data(), sizeof(int32_t) * (size_t) nL, hipMemcpyHostToDevice, st));
 	CLA_HIP(hipMemcpyAsync(dBase, gBase.data(), sizeof(int32_t) * (size_t) nL, hipMemcpyHostToDevice, st));
 	CLA_HIP(hipMemsetAsync(dOver, 0, sizeof(int), st));
@@ -336,16 +356,20 @@ static int rows_plan(cla_block* b) {
 	b->rowsTbl = nTbl;
 	b->rowsOff[0] = idxBytes + listBytes + sizeBytes;
 	b->rowsOff[1] = idxBytes + listBytes + sizeBytes + hdrBytes;
+	b->rowsColOff = idxBytes / 2;
+	b->rowsFusable = fusable;
 	b->rowsState = 1;
 	return 0;
 }
 
 // X %*% u of all listed groups (tables in b->dTables). Returns 1 when the lists do not fit (tables beyond LDS or
-// 16-bit positions, rows with too many entries), 0 when done.
-int launch_rmm_sdc_rows(cla_block* b, int constRow, int accumulate, double* dOut, unsigned long long* dNnz) {
+// 16-bit positions, rows with too many entries), 0 when done. dU != nullptr: the kernel makes the tables itself
+// (rows_fusable said it can) and clears *nnzNext.
+int launch_rmm_sdc_rows(cla_block* b, int constRow, int accumulate, double* dOut, unsigned long long* dNnz, const double* dU,
+	unsigned long long* nnzNext) {
 	int rc = rows_plan(b);
 	if(rc) return rc;
-	if(b->rowsState != 1) return 1;
+	if(b->rowsState != 1 || (dU != nullptr && !b->rowsFusable)) return 1;
 	const int nQuarters = (int) ((b->nRows + RW_Q - 1) / RW_Q);
 	const size_t lds = sizeof(double) * ((size_t) (b->rowsTbl + 2) / 2 * 2 + (size_t) RW_WAVES * RW_Q);
 	const unsigned grid = (unsigned) std::min((nQuarters + RW_WAVES - 1) / RW_WAVES, g_numCU);
@@ -357,12 +381,23 @@ int launch_rmm_sdc_rows(cla_block* b, int constRow, int accumulate, double* dOut
 		CLA_HIP(allow_full_lds((const void*) kernel));
 		hipLaunchKernelGGL(kernel, dim3(grid), dim3(RW_THREADS), lds, b->stream, (const int32_t*) meta, b->rowsTbl,
 			(const uint2*) (meta + b->rowsOff[0]), (const uint32_t*) (meta + b->rowsOff[1]), (const uint32_t*) b->dRowsData,
-			(const double*) b->dTables, constRow, dOut, b->nRows, nQuarters, dNnz);
+			dU ? (const double*) b->dAllDict : (const double*) b->dTables, constRow, dOut, b->nRows, nQuarters, dNnz,
+			(const int32_t*) (meta + b->rowsColOff), dU, nnzNext);
 		return 0;
 	};
-	if((rc = accumulate ? go(k_rmm_sdc_rows<true>) : go(k_rmm_sdc_rows<false>))) return rc;
+	if((rc = dU ? go(k_rmm_sdc_rows<false, true>) : accumulate ? go(k_rmm_sdc_rows<true, false>) : go(k_rmm_sdc_rows<false, false>))) return rc;
 	CLA_HIP(hipGetLastError());
 	return 0;
+}
+
+// Whether X %*% u of this block can run as the one kernel above with tables of its own (builds the row lists on
+// first use).
+bool rows_fusable(cla_block* b) {
+	if(b->hasConst || b->hasUnc || b->hasRle || !b->hasSdc || b->nRows == 0) return false;
+	for(auto& g : b->groups)
+		if(g.d.type != G_SDCZ || g.d.nOffsets <= 0 || g.d.nColG != 1) return false;
+	if(sdc_plan_all(b) != 0 || rows_plan(b) != 0) return false;
+	return b->rowsState == 1 && b->rowsFusable;
 }
 
 } // namespace cla

@@ -487,6 +487,11 @@ static int sdc_plan(cla_block* b, int onlyGroup, int32_t** dList, int32_t** dBin
 	return 0;
 }
 
+int sdc_plan_all(cla_block* b) {
+	int32_t *dList = nullptr, *dBinOff = nullptr;
+	return sdc_plan(b, -1, &dList, &dBinOff);
+}
+
 // Returns 1 if some SDC group cannot use the tile kernel (caller falls back), 0 when done.
 int launch_lmm_sdc_tiles(cla_block* b, const double* dY, int p, double* dPre, int onlyGroup, double* dOut) {
 	int32_t *dList = nullptr, *dBinOff = nullptr;
