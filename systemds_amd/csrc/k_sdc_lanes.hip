@@ -238,7 +238,12 @@ __global__ __launch_bounds__(LN_LW * 64) void k_lmm_sdc_lanes(const LaneDesc* __
 	uint32_t* descS = (uint32_t*) (accS + LN_TAGS);            // per group: dictionary offset | spare code << 16 (LN_TAGS)
 	int32_t* nextS = (int32_t*) (descS + LN_TAGS);             // the block's next window (2 slots: 8 bytes)
 	double* yt = (double*) (nextS + 2) + wave * LN_YT;         // this wave's Y window
-	const int slab = blockIdx.x % nSlabs, part = blockIdx.x / nSlabs, nParts = gridDim.x / nSlabs;
+	// Blocks go round the 8 XCDs by their index. The slabs of a share of the windows read the same part of Y: they sit 8
+	// block indices apart, on one XCD and at work at the same time, so that its L2 fetches that part of Y once.
+	const int nParts = gridDim.x / nSlabs;
+	const int period = 8 * nSlabs, grp = blockIdx.x / period, in = blockIdx.x % period;
+	const int inLast = nParts - grp * 8 < 8 ? nParts - grp * 8 : 8; // shares of the last, partial period
+	const int slab = in / inLast, part = grp * 8 + in % inLast;
 	const LaneSlab S = slabs[slab];
 	// the block's share of the windows
 	const int wBeg = (int) ((int64_t) nWin * part / nParts), wEnd = (int) ((int64_t) nWin * (part + 1) / nParts);
