@@ -62,6 +62,18 @@ public final class ClaHipNative {
 
 	public static native int setOption(long h, String key, int value);
 
+	/** Frees every format the library derived from the block since finalizeBlock; the next call that wants one builds it again. */
+	public static native int dropDerived(long h);
+
+	/** Product bits of prepare. */
+	public static final int PRODUCT_RMM = 1, PRODUCT_LMM = 2, PRODUCT_TSMM = 4;
+
+	/** Builds now what the first call of the named products would build (nColB / nRowY: the widths of the operands to come). */
+	public static native int prepare(long h, int products, int nColB, int nRowY);
+
+	/** Bytes of device memory held by the derived formats. */
+	public static native long derivedBytes(long h);
+
 	// ---- drivers (compress/lib/CLALibRightMultBy, CLALibLeftMultBy, CLALibTSMM, CLALibMMChain, ...)
 	public static native long rmm(long h, double[] B, int nColB, double[] out);
 

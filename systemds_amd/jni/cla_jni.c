@@ -135,6 +135,15 @@ JNIEXPORT jint JNICALL FN(setOption)(JNIEnv* env, jclass c, jlong h, jstring key
 	return rc;
 }
 
+JNIEXPORT jint JNICALL FN(dropDerived)(JNIEnv* env, jclass c, jlong h) { (void) env; (void) c; return cla_block_drop_derived(H(h)); }
+
+JNIEXPORT jint JNICALL FN(prepare)(JNIEnv* env, jclass c, jlong h, jint products, jint nColB, jint nRowY) {
+	(void) env; (void) c;
+	return cla_block_prepare(H(h), (uint32_t) products, nColB, nRowY);
+}
+
+JNIEXPORT jlong JNICALL FN(derivedBytes)(JNIEnv* env, jclass c, jlong h) { (void) env; (void) c; return cla_block_derived_bytes(H(h)); }
+
 /* one input array, one output array */
 JNIEXPORT jlong JNICALL FN(rmm)(JNIEnv* env, jclass c, jlong h, jdoubleArray B, jint nColB, jdoubleArray out) {
 	(void) c;
