@@ -304,3 +304,35 @@ def test_many_rows_of_y_in_chunks_of_columns(cla, ora, shape, p):
     assert_matches_truth(out2, Y, D, what=f"Y %*% X in column chunks, {shape}, {p} rows, second call")
     assert_matches_truth(bins, Y, D, what=f"Y %*% X, {shape}, {p} rows, bin kernels")
     assert nnz == np.count_nonzero(out) and nnz2 == np.count_nonzero(out2) and nnz_b == np.count_nonzero(bins)
+
+
+def test_repeated_calls_count_their_own_non_zeros(cla, ora):
+    """The kernels that serve a whole block count the result's non-zeros themselves (the last workgroup to finish
+    does and leaves its ticket counter at zero): calls in a row with different numbers of rows of Y, also queued
+    without a wait between them, each report their own count."""
+    from devmem import DevBuf
+    from systemds_amd import synth
+    n_rows, n_cols = 60000, 24
+    rng = np.random.default_rng(77)
+    specs = [synth.GroupSpec("ddc", np.array([c], np.int32), np.where(rng.random((40, 1)) < 0.3, 0.0, rng.standard_normal((40, 1))),
+                             rng.integers(0, 40, n_rows).astype(np.uint8)) for c in range(n_cols)]
+    blk = cla.build_block(n_rows, n_cols, specs)
+    Ys = [rng.standard_normal((p, n_rows)) * (rng.random((p, 1)) < 0.7) for p in (1, 3, 2, 5, 1)]
+    names = set()
+    for rep in range(4):
+        for Y in Ys:
+            out, nnz = blk.lmm(Y)
+            assert nnz == np.count_nonzero(out)
+            names |= {k["name"] for k in blk.stats()["kernels"]}
+    assert "k_lmm_u8_dot" in names and "k_lmm_finish" not in names, names
+    # queued back to back on the block's stream: the last call's count is the one reported
+    dY = [DevBuf.from_numpy(Y) for Y in Ys]
+    dO = [DevBuf(Y.shape[0] * n_cols * 8) for Y in Ys]
+    for Y, y, o in zip(Ys, dY, dO):
+        blk.lmm_dev_async(y.ptr, Y.shape[0], o.ptr)
+    last = blk.nnz()
+    outs = [o.to_numpy((Y.shape[0], n_cols)) for o, Y in zip(dO, Ys)]
+    assert last == np.count_nonzero(outs[-1])
+    for got, Y in zip(outs, Ys):
+        assert np.array_equal(got != 0, blk.lmm(Y)[0] != 0)
+    blk.close()

@@ -88,8 +88,9 @@ def test_every_kernel_choice_against_the_decompressed_product(cla, ora, n_rows, 
             assert_close(out, D, u, f"{mode}: X %*% u")
             assert nnz == np.count_nonzero(out)
             for p in (1, 3):
-                out, _ = blk.lmm(Y[:p])
+                out, nnz = blk.lmm(Y[:p])
                 assert_close(out, Y[:p], D, f"{mode}: t(v) %*% X, {p} rows")
+                assert nnz == np.count_nonzero(out), f"{mode}: non-zeros of t(v) %*% X, {p} rows"
             w = rng.standard_normal((n_rows, 1))
             out, _ = blk.mmchain(u, w, 1)
             Xu, _ = truth(D, u)
