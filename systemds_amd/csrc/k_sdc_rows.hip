@@ -32,7 +32,7 @@ constexpr int RW_KR = 40;          // most entries of a row (the conversion's st
 constexpr int RW_Q = 256;          // rows per quarter: the unit of sorting and of a wave's work
 constexpr int RW_QW = RW_WIN / RW_Q; // quarters per window
 constexpr int RW_F = RW_Q / 64;    // rows per lane and quarter
-constexpr int RW_WAVES = 16;       // waves per block
+constexpr int RW_WAVES = 8;        // waves per block (C4: 0.110 / 0.095 / 0.086 / 0.088 / 0.097 ms with 4 / 6 / 8 / 12 / 16)
 constexpr int RW_THREADS = RW_WAVES * 64;
 constexpr int RW_PF = 24;          // groups of a quarter that a lane requests a quarter ahead
 constexpr int RW_TBL_MAX = 16000;  // table entries of all listed groups in LDS (125 KB, next to 2 KB per wave)
