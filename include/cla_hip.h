@@ -124,6 +124,11 @@ int cla_block_set_stream(cla_handle h, void* hipStream);
  *                   columns by chunk (sub-blocks kept with the block); single-column byte-code blocks only from 13 rows of Y
  *                   on (the kernel reports non-finite values of Y and the host looks, i.e. waits for the stream once per call;
  *                   such a Y takes the bin kernels)
+ *   ddc_reorder     1 / 0 (read by cla_block_finalize): the block's copy of a DDC group with two- or four-byte codes and a
+ *                   dictionary of 16 KiB or more is renumbered by descending count of the tuples (codes in place, dictionary
+ *                   rows alike), so that the tuples most rows refer to share cache lines. The reference numbers tuples by
+ *                   first appearance (CG/ColGroupFactory.java:682-703); no product depends on the numbering, and cla_counts,
+ *                   cla_cooc and cla_preagg answer in the caller's numbering either way
  * Blocks derived from this one (overlapping results, joint blocks) inherit the values at the time of the call
  * that uses them. Returns 0, or -CLA_ERR_INVALID for an unknown key or value. */
 int cla_block_set_option(cla_handle h, const char* key, int32_t value);

@@ -527,6 +527,7 @@ static int finalize_groups(cla_block* b) {
 				set_error("group %zu holds a code >= its number of dictionary entries (%d)", gi, G.nVals);
 				return -CLA_ERR_INVALID;
 			}
+			if(b->opt.ddcReorder && (rc = reorder_ddc_by_count(b, (int) gi))) return rc;
 		}
 		if(G.type == G_SDCZ) {
 			if(!g.def.empty()) {
@@ -711,6 +712,7 @@ int cla_block_set_option(cla_handle b, const char* key, int32_t value) {
 		{"sdc_lanes", &Options::sdcLanes, 0, 1},
 		{"sdc_rows", &Options::sdcRows, 0, 1},
 		{"lmm_joint", &Options::lmmJoint, 0, 1},
+		{"ddc_reorder", &Options::ddcReorder, 0, 1},
 	};
 	for(const Entry& e : table)
 		if(strcmp(e.name, key) == 0) {
@@ -1091,6 +1093,7 @@ static cla_block* make_joint(cla_block* left, cla_block* right) {
 			g.cols = pg.cols;
 			for(int& col : g.cols) col += shift;
 			g.dict = pg.dict;
+			g.codeOrder = pg.codeOrder;
 			g.bytes = 0;
 			if(upload(g, g.cols.data(), sizeof(int32_t) * g.cols.size(), (const void**) &g.d.cols) ||
 				(!g.dict.empty() && upload_dict(g))) {
@@ -1175,6 +1178,7 @@ static cla_block* make_sub(cla_block* b, const Chunk& A, const Chunk& B, bool cr
 				colMap.push_back(pg.cols[j]);
 			}
 			g.dict = pg.dict;
+			g.codeOrder = pg.codeOrder;
 			g.bytes = 0;
 			if(upload(g, g.cols.data(), sizeof(int32_t) * g.cols.size(), (const void**) &g.d.cols) ||
 				(!g.dict.empty() && upload_dict(g))) {
@@ -1666,6 +1670,7 @@ cla_handle cla_rmm_overlapping(cla_handle b, const double* B, int32_t nColB) {
 		g.cols = cols;
 		g.d.nColG = q;
 		g.dict.assign(T.begin() + (size_t) P.tblOff * q, T.begin() + (size_t) (P.tblOff + P.nVals) * q);
+		g.codeOrder = pg.codeOrder;
 		g.bytes = 0;
 		if(upload(g, cols.data(), sizeof(int32_t) * (size_t) q, (const void**) &g.d.cols) || upload_dict(g)) { cla_block_free(c); return nullptr; }
 		g.bytes = pg.bytes; // what a kernel streams for this group
@@ -1777,6 +1782,15 @@ int cla_cooc(cla_handle b, int32_t gA, int32_t gB, int64_t* out) {
 	if((rc = launch_cooc(b, gA, gB, (unsigned long long*) b->dScratch))) return rc;
 	CLA_HIP(hipMemcpyAsync(out, b->dScratch, n * sizeof(int64_t), hipMemcpyDeviceToHost, b->stream));
 	CLA_HIP(hipStreamSynchronize(b->stream));
+	// back to the caller's numbering of the tuples
+	const std::vector<int32_t>&oA = b->groups[gA].codeOrder, &oB = b->groups[gB].codeOrder;
+	if(!oA.empty() || !oB.empty()) {
+		const size_t nA = (size_t) b->groups[gA].d.nVals, nB = (size_t) b->groups[gB].d.nVals;
+		std::vector<int64_t> t(out, out + n);
+		for(size_t i = 0; i < nA; i++)
+			for(size_t j = 0; j < nB; j++)
+				out[(oA.empty() ? i : (size_t) oA[i]) * nB + (oB.empty() ? j : (size_t) oB[j])] = t[i * nB + j];
+	}
 	return 0;
 	CLA_CATCH_CODE(int)
 }
@@ -1796,6 +1810,15 @@ int cla_preagg(cla_handle b, int32_t group, const double* Y, int32_t nRowY, doub
 	if((rc = launch_preagg(b, group, b->dStageIn, nRowY, b->dStageOut))) return rc;
 	CLA_HIP(hipMemcpyAsync(preAgg, b->dStageOut, nOut * sizeof(double), hipMemcpyDeviceToHost, b->stream));
 	CLA_HIP(hipStreamSynchronize(b->stream));
+	const std::vector<int32_t>& order = b->groups[group].codeOrder;
+	if(!order.empty()) { // back to the caller's numbering of the tuples
+		std::vector<double> t((size_t) nVals);
+		for(int r = 0; r < nRowY; r++) {
+			double* row = preAgg + (size_t) r * nVals;
+			std::copy(row, row + nVals, t.begin());
+			for(int k = 0; k < nVals; k++) row[order[k]] = t[k];
+		}
+	}
 	return 0;
 	CLA_CATCH_CODE(int)
 }
@@ -1812,6 +1835,11 @@ int cla_counts(cla_handle b, int32_t group, int32_t* counts) {
 	if((rc = launch_counts(b, group, (int32_t*) b->dScratch))) return rc;
 	CLA_HIP(hipMemcpyAsync(counts, b->dScratch, sizeof(int32_t) * (size_t) nVals, hipMemcpyDeviceToHost, b->stream));
 	CLA_HIP(hipStreamSynchronize(b->stream));
+	const std::vector<int32_t>& order = b->groups[group].codeOrder;
+	if(!order.empty()) { // back to the caller's numbering of the tuples
+		std::vector<int32_t> t(counts, counts + nVals);
+		for(int k = 0; k < nVals; k++) counts[order[k]] = t[k];
+	}
 	return 0;
 	CLA_CATCH_CODE(int)
 }

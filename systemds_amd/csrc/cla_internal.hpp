@@ -57,6 +57,7 @@ struct HostGroup {
 	std::vector<int32_t> cols;
 	std::vector<double> dict;       // host copy of the (morphed) dictionary
 	std::vector<double> def;        // SDC default tuple (empty => none)
+	std::vector<int32_t> codeOrder; // renumbered by count at finalize: the caller's code of each code held here (empty => unchanged)
 	std::vector<void*> owned;       // device allocations owned by this group
 	int64_t bytes = 0;              // HBM bytes of the compressed representation
 };
@@ -80,6 +81,7 @@ struct Options {
 	int sdcPacked = 1;      // packed SDCZeros lists for the mat-vecs
 	int sdcLanes = 1;       // SDCZeros mat-vecs on lane-major lists, one lane per group
 	int sdcRows = 1;        // SDCZeros right mat-vec on row lists, one lane per row
+	int ddcReorder = 1;     // finalize renumbers the tuples of large DDC dictionaries by descending count (0: the caller's numbering is kept)
 };
 
 struct KernelStat {
@@ -238,6 +240,7 @@ extern int g_numCU;
 // ---- launchers implemented in the kernel translation units ----
 int launch_validate_codes(cla_block* b, const void* codes, int width, int64_t n, int nVals, int* ok);
 int launch_counts(cla_block* b, int group, int32_t* dCounts);
+int reorder_ddc_by_count(cla_block* b, int group);
 int launch_sdc_build(cla_block* b, HostGroup& g);
 int launch_rmm(cla_block* b, const double* dB, int q, double* dOut, unsigned long long* dNnz, int squares = 0,
 	double* ws = nullptr, size_t wsDoubles = 0);

@@ -124,6 +124,80 @@ int launch_counts(cla_block* b, int group, int32_t* dCounts) {
 }
 
 // ---------------------------------------------------------------------------
+// Dictionary order by count. A DDC group with a dictionary beyond the first-level cache is looked up
+// in global memory by the decode kernels; with skewed codes most lookups go to few tuples, and those
+// share cache lines when they sit next to each other. The reference numbers tuples by first appearance
+// (ColGroupFactory.java:682-703 through ACountHashMap.java:92-111), which puts frequent tuples first
+// only roughly; here the block's own copy is renumbered by descending count at finalize: the codes in
+// place, the dictionary rows alike. No product depends on the numbering (sums run over rows and
+// columns, never over codes); the entry points that return arrays indexed by code (counts,
+// co-occurrence, pre-aggregate) map their result back through HostGroup::codeOrder.
+// ---------------------------------------------------------------------------
+template <int W>
+__global__ __launch_bounds__(256) void k_recode(void* codes, int64_t n, const uint32_t* __restrict__ lut) {
+	constexpr int PER = 16 / W;
+	const int64_t nVec = n / PER;
+	u32x4* vec = (u32x4*) codes;
+	for(int64_t i = (int64_t) blockIdx.x * blockDim.x + threadIdx.x; i < nVec; i += (int64_t) gridDim.x * blockDim.x) {
+		u32x4 v = vec[i];
+#pragma unroll
+		for(int k = 0; k < 4; k++) {
+			if(W == 2) v[k] = lut[v[k] & 0xffffu] | (lut[v[k] >> 16] << 16);
+			else v[k] = lut[v[k]];
+		}
+		vec[i] = v;
+	}
+	if(blockIdx.x == 0 && threadIdx.x < (int) (n - nVec * PER)) {
+		const int64_t i = nVec * PER + threadIdx.x;
+		if(W == 2) ((uint16_t*) codes)[i] = (uint16_t) lut[((const uint16_t*) codes)[i]];
+		else ((uint32_t*) codes)[i] = lut[((const uint32_t*) codes)[i]];
+	}
+}
+
+int reorder_ddc_by_count(cla_block* b, int group) {
+	HostGroup& g = b->groups[group];
+	DGroup& G = g.d;
+	const int nVals = G.nVals;
+	const int64_t n = b->nRows;
+	// byte codes: at most 256 tuples, which the kernels hold in LDS or find in the first-level cache anyway
+	if(G.type != G_DDC || (G.codeWidth != 2 && G.codeWidth != 4)) return 0;
+	if((size_t) nVals * G.nColG * sizeof(double) < 16 * 1024 || n < 16 * (int64_t) nVals) return 0;
+	int rc = ensure_scratch(b, sizeof(int32_t) * 2 * (size_t) nVals);
+	if(rc) return rc;
+	int32_t* dCounts = (int32_t*) b->dScratch;
+	uint32_t* dLut = (uint32_t*) (dCounts + nVals);
+	if((rc = launch_counts(b, group, dCounts))) return rc;
+	std::vector<int32_t> counts(nVals);
+	CLA_HIP(hipMemcpyAsync(counts.data(), dCounts, sizeof(int32_t) * (size_t) nVals, hipMemcpyDeviceToHost, b->stream));
+	CLA_HIP(hipStreamSynchronize(b->stream));
+	std::vector<int32_t> order(nVals); // new code -> old code
+	for(int k = 0; k < nVals; k++) order[k] = k;
+	std::stable_sort(order.begin(), order.end(), [&](int32_t x, int32_t y) { return counts[x] > counts[y]; });
+	bool identity = true;
+	for(int k = 0; k < nVals; k++) identity &= order[k] == k;
+	if(identity) return 0;
+	std::vector<uint32_t> lut(nVals);
+	for(int k = 0; k < nVals; k++) lut[order[k]] = (uint32_t) k;
+	CLA_HIP(hipMemcpyAsync(dLut, lut.data(), sizeof(uint32_t) * (size_t) nVals, hipMemcpyHostToDevice, b->stream));
+	const int64_t blocks = std::max<int64_t>(1, (n * G.codeWidth / 16 + 256 * 4 - 1) / (256 * 4));
+	const unsigned grid = (unsigned) std::min<int64_t>(blocks, (int64_t) g_numCU * 16);
+	void* codes = const_cast<void*>(G.codes);
+	Prof pf(b, "k_recode", grid, 256, 0, 2.0 * (double) n * G.codeWidth);
+	if(G.codeWidth == 2) hipLaunchKernelGGL(k_recode<2>, dim3(grid), dim3(256), 0, b->stream, codes, n, dLut);
+	else hipLaunchKernelGGL(k_recode<4>, dim3(grid), dim3(256), 0, b->stream, codes, n, dLut);
+	CLA_HIP(hipGetLastError());
+	const size_t w = (size_t) G.nColG;
+	std::vector<double> nd(g.dict.size());
+	for(int k = 0; k < nVals; k++) std::copy(g.dict.begin() + order[k] * w, g.dict.begin() + (order[k] + 1) * w, nd.begin() + k * w);
+	g.dict.swap(nd);
+	CLA_HIP(hipMemcpyAsync(const_cast<double*>(G.dict), g.dict.data(), sizeof(double) * g.dict.size(), hipMemcpyHostToDevice,
+		b->stream));
+	CLA_HIP(hipStreamSynchronize(b->stream));
+	g.codeOrder.swap(order);
+	return 0;
+}
+
+// ---------------------------------------------------------------------------
 // Offset-list acceleration structures (device twin of AOffset's skip list).
 // ---------------------------------------------------------------------------
 // per chunk of SDC_CK entries: (sum of row increments, number of emitted rows)
