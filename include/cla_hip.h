@@ -124,6 +124,10 @@ int cla_block_set_stream(cla_handle h, void* hipStream);
  *                   columns by chunk (sub-blocks kept with the block); single-column byte-code blocks only from 13 rows of Y
  *                   on (the kernel reports non-finite values of Y and the host looks, i.e. waits for the stream once per call;
  *                   such a Y takes the bin kernels)
+ *   tsmm_one_kernel 1 / 0: t(X) %*% X of a whole block of at most 64 columns on the decoded Gram kernels as the call's only
+ *                   kernel (its blocks add into an accumulator kept with the block, nCols x nCols doubles; the last block
+ *                   to finish writes the output, mirrored, and the count of its non-zeros and clears the accumulator)
+ *                   instead of a fill of the output in front of the kernel and a mirror-and-count kernel behind it
  *   ddc_reorder     1 / 0 (read by cla_block_finalize): the block's copy of a DDC group with two- or four-byte codes and a
  *                   dictionary of 16 KiB or more is renumbered by descending count of the tuples (codes in place, dictionary
  *                   rows alike), so that the tuples most rows refer to share cache lines. The reference numbers tuples by

@@ -105,6 +105,14 @@ int ensure_scratch(cla_block* b, size_t bytes) {
 	return 0;
 }
 
+int ensure_gram_acc(cla_block* b) {
+	if(b->dGramAcc != nullptr) return 0;
+	const size_t bytes = sizeof(double) * std::max<size_t>((size_t) b->nCols * b->nCols, 1);
+	CLA_HIP(hipMalloc((void**) &b->dGramAcc, bytes));
+	CLA_HIP(hipMemset(b->dGramAcc, 0, bytes));
+	return 0;
+}
+
 static int ensure_stage(double** p, size_t* cap, size_t nDoubles) {
 	if(nDoubles <= *cap) return 0;
 	if(*p) CLA_HIP(hipFree(*p));
@@ -327,6 +335,7 @@ void cla_block_free(cla_handle b) {
 	for(uint8_t* p : b->expCodes)
 		if(p) (void) hipFree(p);
 	if(b->dCounters) (void) hipFree(b->dCounters);
+	if(b->dGramAcc) (void) hipFree(b->dGramAcc);
 	if(b->hCounters) (void) hipHostFree(b->hCounters);
 	if(b->ownStream && b->stream) (void) hipStreamDestroy(b->stream);
 	delete b;
@@ -713,6 +722,7 @@ int cla_block_set_option(cla_handle b, const char* key, int32_t value) {
 		{"sdc_rows", &Options::sdcRows, 0, 1},
 		{"lmm_joint", &Options::lmmJoint, 0, 1},
 		{"ddc_reorder", &Options::ddcReorder, 0, 1},
+		{"tsmm_one_kernel", &Options::tsmmOneKernel, 0, 1},
 	};
 	for(const Entry& e : table)
 		if(strcmp(e.name, key) == 0) {

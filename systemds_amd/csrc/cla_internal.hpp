@@ -81,6 +81,7 @@ struct Options {
 	int sdcPacked = 1;      // packed SDCZeros lists for the mat-vecs
 	int sdcLanes = 1;       // SDCZeros mat-vecs on lane-major lists, one lane per group
 	int sdcRows = 1;        // SDCZeros right mat-vec on row lists, one lane per row
+	int tsmmOneKernel = 1;  // decoded Gram matrix of a whole block as the call's only kernel (0: a fill in front, k_tsmm_finish behind)
 	int ddcReorder = 1;     // finalize renumbers the tuples of large DDC dictionaries by descending count (0: the caller's numbering is kept)
 };
 
@@ -205,7 +206,8 @@ struct cla_block {
 	uint32_t* dSdcPacked = nullptr;  // all listed groups' entries as (code << 16 | row inside its 4096-row tile), built on first use
 	int sdcPlanGroup = -2;
 	std::vector<int32_t> sdcList, sdcBinOff;
-	unsigned long long* dCounters = nullptr;   // 8 x u64
+	unsigned long long* dCounters = nullptr;   // 8 x u64: 0 - 3 non-zero counts, 6 and 7 ticket counters of the left multiply's and the Gram kernels' tails
+	double* dGramAcc = nullptr;      // nCols x nCols, zero between calls: where the blocks of a one-kernel t(X) %*% X add (gram_tail)
 	unsigned long long* hCounters = nullptr;   // pinned
 
 	std::vector<cla::KernelStat> lastStats;
@@ -259,8 +261,9 @@ int launch_rmm_sdc_rows(cla_block* b, int constRow, int accumulate, double* dOut
 	unsigned long long* nnzNext = nullptr);
 bool rows_fusable(cla_block* b);
 int launch_rmm_sdc_tiles(cla_block* b, int q, int constRow, int accumulate, double* dOut, unsigned long long* dNnz);
-int launch_tsmm_decode(cla_block* b, double* dOut);
-int launch_tsmm_direct(cla_block* b, double* dOut);
+int launch_tsmm_decode(cla_block* b, double* dOut, unsigned long long* dNnz = nullptr);
+int launch_tsmm_direct(cla_block* b, double* dOut, unsigned long long* dNnz = nullptr);
+int ensure_gram_acc(cla_block* b); // the zeroed nCols x nCols accumulator of the one-kernel t(X) %*% X (a workspace kept with the block)
 int ensure_expanded(cla_block* b);
 int launch_rmm_decode(cla_block* b, const double* dB, int q, const double* dConstRow, double* dOut,
 	unsigned long long* dNnz);

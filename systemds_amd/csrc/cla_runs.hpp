@@ -146,6 +146,46 @@ struct RunCursors {
 	}
 };
 
+// Tail of a t(X) %*% X whose kernel is the only one of the call. The blocks have added their tiles' upper triangles
+// into acc (nCols x nCols, all zero when the kernel starts); every block comes here behind its last add, and the last one
+// to arrive copies acc to out, mirrored, counts out's non-zeros into *nnz and leaves acc and *done at zero for the next
+// launch: what a fill of out in front of the kernel and a kernel of its own behind it would do. `lds`: 17 words of the
+// block's LDS that nobody else uses any more (no static LDS here: the Gram kernels address theirs from offset zero).
+__device__ __forceinline__ void gram_tail(unsigned* done, unsigned nBlocks, double* acc, double* out, int nCols, unsigned long long* nnz,
+	unsigned* lds) {
+	unsigned& gramTicketS = lds[0];
+	int* const gramPartS = (int*) lds + 1;
+	// this thread's adds have been acknowledged before the block takes its ticket (the adds, the ticket and the reads
+	// below are all performed at device scope, past the caches that the chip's parts do not share)
+	asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+	__syncthreads();
+	if(threadIdx.x == 0) gramTicketS = atomicAdd(done, 1u);
+	__syncthreads();
+	if(gramTicketS != nBlocks - 1) return;
+	int cnt = 0;
+	for(int idx = threadIdx.x; idx < nCols * nCols; idx += blockDim.x) {
+		const int i = idx / nCols, j = idx - i * nCols;
+		if(j < i) continue;
+		unsigned long long* cell = (unsigned long long*) acc + idx;
+		const unsigned long long bits = __hip_atomic_load(cell, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+		__hip_atomic_store(cell, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+		double v;
+		__builtin_memcpy(&v, &bits, 8);
+		out[idx] = v;
+		out[(size_t) j * nCols + i] = v;
+		cnt += v != 0.0 ? (i == j ? 1 : 2) : 0;
+	}
+	cnt = wave_sum_i32(cnt);
+	if((threadIdx.x & (WAVE - 1)) == 0) gramPartS[threadIdx.x >> 6] = cnt;
+	__syncthreads();
+	if(threadIdx.x == 0) {
+		int s = 0;
+		for(unsigned w = 0; w < (blockDim.x + WAVE - 1) / WAVE; w++) s += gramPartS[w];
+		*nnz = (unsigned long long) s;
+		*done = 0;
+	}
+}
+
 int mrt_build(cla_block* b, const std::vector<RunCol>& runs, int sliceRows, Mrt& T);
 void mrt_free(Mrt& T);
 int launch_run_sums(cla_block* b, const std::vector<RunCol>& runs, const Mrt& T, const double* dB, int ld, int q, const double* dConstRow);

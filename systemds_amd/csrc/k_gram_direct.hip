@@ -69,6 +69,9 @@ struct GdrArgs {
 	int64_t nRows;
 	double* out;
 	int nCols;
+	double* acc;               // the call's only kernel: the blocks add here and the last one writes out (gram_tail)
+	unsigned* done;            // its ticket counter (nullptr: the blocks add into out, the caller fills and finishes)
+	unsigned long long* nnz;
 };
 
 struct GdrPlan {
@@ -410,8 +413,9 @@ __global__ __launch_bounds__(GDR_THREADS) void k_tsmm_direct(const GdrArgs A) {
 		const int ci = i < 16 ? (i < A.nV ? A.cols[i].col : -1) : (i - 16 < nR ? A.runs[i - 16].col : -1);
 		const int cj = j < 16 ? (j < A.nV ? A.cols[j].col : -1) : (j - 16 < nR ? A.runs[j - 16].col : -1);
 		if(ci < 0 || cj < 0) continue;
-		unsafeAtomicAdd(&A.out[(size_t) min(ci, cj) * A.nCols + max(ci, cj)], s);
+		unsafeAtomicAdd(&(A.done != nullptr ? A.acc : A.out)[(size_t) min(ci, cj) * A.nCols + max(ci, cj)], s);
 	}
+	if(A.done != nullptr) gram_tail(A.done, gridDim.x, A.acc, A.out, A.nCols, A.nnz, (unsigned*) gramS);
 }
 
 // Which columns of the block are streams, which are followed by run cursors; 1 when the block is not of this shape.
@@ -552,7 +556,7 @@ void gdr_plan_drop(cla_block* b) {
 
 // dOut (nCols x nCols, zeroed) += upper triangle of t(D) %*% D of the decoded rows, constants included. Returns 1
 // when the block is not of this kernel's shape (the caller takes the tile kernel on the matrix cores).
-int launch_tsmm_direct(cla_block* b, double* dOut) {
+int launch_tsmm_direct(cla_block* b, double* dOut, unsigned long long* dNnz) {
 	if(!b->opt.tsmmDirect || b->crossSplit > 0 || b->crossBlocks > 0) return 1;
 	if(b->gdrPlan == nullptr) {
 		int rc = ensure_expanded(b);
@@ -565,6 +569,12 @@ int launch_tsmm_direct(cla_block* b, double* dOut) {
 	if(b->gdrPlan->rc) return b->gdrPlan->rc;
 	GdrArgs A = b->gdrPlan->A;
 	A.out = dOut;
+	A.acc = nullptr; A.done = nullptr; A.nnz = nullptr;
+	if(dNnz != nullptr) {
+		const int rc = ensure_gram_acc(b);
+		if(rc) return rc;
+		A.acc = b->dGramAcc; A.done = (unsigned*) (b->dCounters + 7); A.nnz = dNnz;
+	}
 	const size_t lds = b->gdrPlan->lds;
 	const int nChunks = (int) ((b->nRows + GDR_CH - 1) / GDR_CH);
 	const unsigned grid = (unsigned) std::max(1, std::min((nChunks + GDR_WAVES - 1) / GDR_WAVES, g_numCU * (lds <= 76 * 1024 ? 2 : 1)));

@@ -88,6 +88,8 @@ struct DecArgs {
 	int64_t nRows;
 	unsigned long long* nnz;
 	int nCols;
+	double* acc;                       // t(X) %*% X as the call's only kernel: the blocks add here and the last one writes out (gram_tail)
+	unsigned* done;                    // its ticket counter (nullptr: the blocks add into out, the caller fills and finishes)
 };
 
 typedef double f64x4 __attribute__((ext_vector_type(4)));
@@ -714,10 +716,12 @@ __device__ __forceinline__ void decode_body(const DecArgs& A) {
 			}
 		}
 		__syncthreads();
+		double* const dst = A.done != nullptr ? A.acc : A.out;
 		for(int i = tid; i < NP * NP; i += DEC_THREADS) {
 			const int r = i / NP, c = i - r * NP;
-			if(r <= c && c < A.nCols && stage[i] != 0.0) unsafeAtomicAdd(&A.out[(size_t) r * A.nCols + c], stage[i]);
+			if(r <= c && c < A.nCols && stage[i] != 0.0) unsafeAtomicAdd(&dst[(size_t) r * A.nCols + c], stage[i]);
 		}
+		if(A.done != nullptr) gram_tail(A.done, gridDim.x, A.acc, A.out, A.nCols, A.nnz, (unsigned*) stage);
 		return;
 	}
 	count_add(A.nnz, cnt);
@@ -949,6 +953,7 @@ static int dec_build_plan(cla_block* b, bool gram, int q, int rpl, DecLaunch& L,
 	A.nGroups = nG; A.nCopies = (int) copies.size(); A.nChunks = nChunks; A.nColD = nColD;
 	A.valDoubles = (int) valD; A.bDoubles = (int) bD; A.stageDoubles = (int) stageD; A.slotBytes = (int) slotB;
 	A.B = nullptr; A.q = q; A.ld = q; A.constRow = nullptr; A.Y = nullptr; A.P = 0; A.badY = nullptr; A.out = nullptr; A.nRows = b->nRows; A.nnz = nullptr; A.nCols = nCols;
+	A.acc = nullptr; A.done = nullptr;
 	const int nTiles = (int) ((b->nRows + DEC_TILE - 1) / DEC_TILE);
 	const int blocksPerCU = L.lds <= 76 * 1024 ? 2 : 1;
 	L.grid = (unsigned) std::min(nTiles, g_numCU * blocksPerCU);
@@ -1531,11 +1536,14 @@ int launch_lmm_decode(cla_block* b, const double* dY, int p, double* dOut, unsig
 
 // dOut (nCols x nCols, zeroed) += upper triangle of t(D) %*% D of the decoded rows, constants
 // included. Returns 1 when the block is not eligible (more than 64 columns, LDS plan too large).
-int launch_tsmm_decode(cla_block* b, double* dOut) {
+// dNnz != nullptr: the kernel is the call's only one (dOut need not be zero; it is written whole, mirrored, and its
+// non-zeros are counted into *dNnz by the last block, gram_tail), else the caller has zeroed dOut, mirrors and counts.
+int launch_tsmm_decode(cla_block* b, double* dOut, unsigned long long* dNnz) {
 	const int nCols = b->nCols;
 	if(b->groups.empty() || b->nRows == 0 || nCols > 64) return 1;
+	if(dNnz != nullptr && (b->crossBlocks > 0 || b->crossSplit > 0)) return 1; // (only a part of the Gram matrix is wanted: no one-kernel form)
 	{
-		const int rc = launch_tsmm_direct(b, dOut);
+		const int rc = launch_tsmm_direct(b, dOut, dNnz);
 		if(rc != 1) return rc;
 	}
 	const int NB = (nCols + 15) / 16;
@@ -1548,6 +1556,10 @@ int launch_tsmm_decode(cla_block* b, double* dOut) {
 	int rc = gram_prepare(b, L, flat);
 	if(rc) return rc;
 	L.A.out = dOut;
+	if(dNnz != nullptr) {
+		if((rc = ensure_gram_acc(b))) return rc;
+		L.A.acc = b->dGramAcc; L.A.done = (unsigned*) (b->dCounters + 7); L.A.nnz = dNnz;
+	}
 	Prof pf(b, "k_tsmm_decode", L.grid, DEC_THREADS, (long) L.lds, (double) b->device_bytes_cached);
 	// a last column block of at most 4 columns: its rows on the 4 x 4 x 4 matrix instruction
 	const bool narrow = XB == 0 && NB >= 2 && nCols - 16 * (NB - 1) <= 4 && b->opt.tsmmNarrow;

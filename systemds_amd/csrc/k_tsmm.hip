@@ -588,16 +588,23 @@ int launch_tsmm(cla_block* b, double* dOut, unsigned long long* dNnz) {
 	const int64_t nRows = b->nRows;
 	hipStream_t st = b->stream;
 	clear_stats(b);
-	CLA_HIP(hipMemsetAsync(dOut, 0, sizeof(double) * (size_t) nCols * nCols, st));
-	CLA_HIP(hipMemsetAsync(dNnz, 0, sizeof(unsigned long long), st));
+	auto clear = [&]() -> int {
+		CLA_HIP(hipMemsetAsync(dOut, 0, sizeof(double) * (size_t) nCols * nCols, st));
+		CLA_HIP(hipMemsetAsync(dNnz, 0, sizeof(unsigned long long), st));
+		return 0;
+	};
 	// Overlapping column groups (the result of an overlapping right multiply): every compressed form here
 	// assumes one group per column, and such blocks typically hold more groups than columns, where the
 	// reference decompresses as well (CLALibTSMM.java:73-77).
 	{
+		int rc0;
 		std::vector<char> seen((size_t) nCols, 0);
 		for(auto& g : b->groups)
 			for(int c : g.cols) {
-				if(seen[c]) return launch_tsmm_decompressed(b, dOut, dNnz, "overlapping column groups");
+				if(seen[c]) {
+					if((rc0 = clear())) return rc0;
+					return launch_tsmm_decompressed(b, dOut, dNnz, "overlapping column groups");
+				}
 				seen[c] = 1;
 			}
 	}
@@ -633,6 +640,16 @@ int launch_tsmm(cla_block* b, double* dOut, unsigned long long* dNnz) {
 	// More than 64 columns: the decoded Gram matrices of pairs of 32-column chunks (about 1.4 ms per pair of
 	// chunks on 10M rows) against one pass per pair of groups (3-16 us each): chunks when there are a hundred
 	// times more pairs of groups than pairs of chunks, or when there is no per-pair form.
+	// The decoded Gram matrix of a whole block of at most 64 columns as the call's only kernel: its blocks add into an
+	// accumulator kept with the block, and the last one to finish writes the output (both triangles) and the count of
+	// its non-zeros and clears the accumulator again: no fill in front of the kernel, no kernel behind it.
+	bool decodeTried = false;
+	if(dense && nCols <= 64 && split == 0 && b->crossBlocks == 0 && nRows > 0 && b->opt.tsmmMfma && b->opt.tsmmOneKernel) {
+		decodeTried = true;
+		rc = launch_tsmm_decode(b, dOut, dNnz);
+		if(rc <= 0) return rc;
+	}
+	if((rc = clear())) return rc;
 	const int64_t mAll = (nCols + 31) / 32, mLeft = split > 0 ? std::max<int64_t>(1, mAll / 2) : 0;
 	const int64_t nJoints = split > 0 ? mLeft * std::max<int64_t>(1, mAll - mLeft) : mAll * (mAll - 1) / 2;
 	const bool chunkCheaper = !forcePairs && pairsFit && nPairs >= 100 * nJoints;
@@ -656,7 +673,7 @@ int launch_tsmm(cla_block* b, double* dOut, unsigned long long* dNnz) {
 	if(dense) {
 		// t(D) %*% D of the decoded rows, constants included (no correction layer needed)
 		const bool noMfma = !b->opt.tsmmMfma;
-		rc = (noMfma || nRows == 0) ? 1 : launch_tsmm_decode(b, dOut);
+		rc = (noMfma || nRows == 0 || decodeTried) ? 1 : launch_tsmm_decode(b, dOut);
 		if(rc < 0) return rc;
 		if(rc == 0) {
 			Prof pf(b, "k_tsmm_finish", 1, 256, 0, 0);

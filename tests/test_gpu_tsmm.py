@@ -186,3 +186,60 @@ def test_decoded_gram_with_a_narrow_last_column_block(cla, ora, n_cols, big_dict
             specs.append(synth.GroupSpec("ddc", np.array([c], np.int32), rng.standard_normal((16, 1)), codes))
             c += 1
     check_tsmm(cla, ora, specs, n_rows, n_cols, f"{n_cols} columns, narrow {narrow}", {"tsmm_route": 2, "tsmm_narrow": narrow})
+
+
+@pytest.mark.parametrize("shape", ["decode", "direct"])
+def test_decoded_gram_is_one_kernel_per_call(cla, ora, shape):
+    """A block of at most 64 columns that the decoded Gram kernels take runs as one kernel per call: the blocks add
+    into an accumulator kept with the block and the last one writes the output, mirrored, counts its non-zeros and
+    clears the accumulator (no fill of the output in front, no k_tsmm_finish behind). Repeated and queued calls
+    into outputs that hold garbage must all give the first call's result and count, also with other products
+    between them."""
+    import devmem
+    from systemds_amd import synth
+    if shape == "decode":
+        c = synth.config3(scale=100)
+        specs, n_rows, n_cols = c["groups"], c["n_rows"], c["n_cols"]
+        kernel = "k_tsmm_decode"
+    else:
+        from test_gpu_gram_direct import stream_block
+        n_rows = 70003
+        specs, n_cols = stream_block(21, n_rows)
+        kernel = "k_tsmm_direct"
+    D = ora.np_decompress(specs, n_rows, n_cols)
+    scale = np.abs(D).T @ np.abs(D)
+    blk = cla.build_block(n_rows, n_cols, specs)
+    try:
+        first, nnz = blk.tsmm()
+        blk.profile(True)
+        blk.tsmm()
+        names = [k["name"] for k in blk.stats()["kernels"]]
+        blk.profile(False)
+        assert names == [kernel], names
+        # the same kernel between a fill of the output and k_tsmm_finish (option tsmm_one_kernel 0): the same matrix
+        blk.set_option("tsmm_one_kernel", 0)
+        blk.profile(True)
+        plain, pnnz = blk.tsmm()
+        names = [k["name"] for k in blk.stats()["kernels"]]
+        blk.profile(False)
+        blk.set_option("tsmm_one_kernel", 1)
+        assert names == [kernel, "k_tsmm_finish"], names
+        assert pnnz == nnz
+        assert_fp64_close(plain, first, scale, what=f"{shape}: with and without the tail")
+        outs = [devmem.DevBuf.from_numpy(np.full((n_cols, n_cols), np.nan)) for _ in range(3)]
+        rng = np.random.default_rng(3)
+        blk.tsmm_dev_async(outs[0].ptr)
+        blk.tsmm_dev_async(outs[1].ptr)
+        blk.rmm(rng.standard_normal((n_cols, 2)))
+        blk.lmm(rng.standard_normal((1, n_rows)))
+        assert blk.tsmm_dev(outs[2].ptr) == nnz
+        for o in outs:
+            again = o.to_numpy((n_cols, n_cols))
+            assert np.array_equal(again, again.T)
+            assert_fp64_close(again, first, scale, what=f"{shape}: repeated call")
+            assert np.count_nonzero(again) == nnz
+            o.free()
+    finally:
+        blk.close()
+    assert_matches_truth(first, D.T, D, what=f"{shape}: one kernel per call")
+    assert nnz == np.count_nonzero(first)
