@@ -68,20 +68,36 @@ def cpu_row(fn, n_rows, what):
             "sample": f"{what}: the full workload ({n_rows} rows), median of 3 passes, {sec:.3f} s per pass"}
 
 
+DEVICE_WARMUP_MS = 300.0  # set from --device-warmup-ms
+
+
 def time_async(blk, launch, reps, warm=2):
     """Wall time per call of `launch` (queues the driver's kernels without waiting) over `reps` calls bracketed
-    by device synchronisation, and the per-kernel HIP-event times of one more call."""
+    by device synchronisation, and the per-kernel HIP-event times of five more calls. Like the headline, a row is
+    timed behind an untimed device warm-up (calls of the same product for --device-warmup-ms: the host work between
+    two rows - generating and uploading the next configuration, the CPU legs - leaves the device idle for seconds, and
+    its first milliseconds of load run at transient clocks); the figure without it is returned as well."""
     import torch
+
+    def train():
+        blk.nnz()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            launch()
+        blk.nnz()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / reps * 1e3
+
     for _ in range(warm):
         launch()
-    blk.nnz()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(reps):
-        launch()
-    blk.nnz()
-    torch.cuda.synchronize()
-    ms = (time.perf_counter() - t0) / reps * 1e3
+    cold_ms = train()
+    t_w = time.perf_counter()
+    while time.perf_counter() - t_w < DEVICE_WARMUP_MS * 1e-3:
+        for _ in range(max(1, reps // 2)):
+            launch()
+        blk.nnz()
+    ms = train()
     # per-kernel HIP-event times: the median over five profiled calls of each kernel's summed time in a call
     blk.profile(True)
     calls = []
@@ -97,7 +113,7 @@ def time_async(blk, launch, reps, warm=2):
     blk.profile(False)
     agg = {name: {"ms": statistics.median(c[name]["ms"] for c in calls if name in c), "launches": calls[-1][name]["launches"]}
            for name in calls[-1]}
-    return ms, agg
+    return ms, agg, cold_ms
 
 
 def extra_row(blk, launch, n_rows, algo_bytes, flops=0.0, reps=10, prepare=None):
@@ -126,13 +142,13 @@ def extra_row(blk, launch, n_rows, algo_bytes, flops=0.0, reps=10, prepare=None)
         launch()
         blk.nnz()
         prep["first_call_after_prepare_ms"] = round((time.perf_counter() - t0) * 1e3, 3)
-    ms, ks = time_async(blk, launch, reps)
+    ms, ks, cold_ms = time_async(blk, launch, reps)
     kname = max(ks, key=lambda k: ks[k]["ms"])
     kms = ks[kname]["ms"]
     ksum = sum(v["ms"] for v in ks.values())
     hbm_floor_ms = algo_bytes / (HBM_PEAK_GBS * 1e9) * 1e3
     mfma_floor_ms = flops / (MFMA_F64_PEAK_TF * 1e12) * 1e3
-    row = {"ms": round(ms, 5), "first_call_ms": round(first_ms, 3), "rows_per_s": n_rows / (ms * 1e-3),
+    row = {"ms": round(ms, 5), "cold_ms": round(cold_ms, 5), "first_call_ms": round(first_ms, 3), "rows_per_s": n_rows / (ms * 1e-3),
            "kernel": kname, "kernel_ms": round(kms, 5), "kernels": {k: round(v["ms"], 5) for k, v in ks.items()},
            "kernels_ms": round(ksum, 5), "algo_bytes": algo_bytes, "algo_GBs": algo_bytes / (ksum * 1e-3) / 1e9,
            "frac_hbm": algo_bytes / (ksum * 1e-3) / 1e9 / HBM_PEAK_GBS,
@@ -256,6 +272,8 @@ def main():
                     help="also run a plain 1 GiB device copy (torch) so that a rocprofv3 --pmc run can scale "
                          "FETCH_SIZE / WRITE_SIZE against a kernel of known traffic")
     args = ap.parse_args()
+    global DEVICE_WARMUP_MS
+    DEVICE_WARMUP_MS = args.device_warmup_ms
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (the path shards by rows, each GPU taking a row range of every group); "
               f"--gpus {args.gpus} is not supported", file=sys.stderr)
