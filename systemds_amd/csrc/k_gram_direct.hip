@@ -10,11 +10,13 @@
 //   V x V   lane-private sums acc[i][j] += x_i x_j (NV (NV + 1) / 2 multiply-adds per row on the vector unit,
 //           whose fp64 rate equals the matrix unit's and which computes neither padding nor the lower triangle),
 //           reduced over the lanes once at the end of the range;
-//   R x V   a run-length column is constant between two run ends, so  sum_r v_a x_c = sum_segments v_a(seg) T_c(seg)
-//           with T_c the sum of x_c over a segment: lanes keep T_c, and where some column's run ends the
-//           wave reduces T over its lanes (through LDS), adds v_a T_c for every run-length column a and
-//           starts a new segment;
-//   R x R   likewise with the segment's row count in place of T_c.
+//   R x V   a run-length column is constant between two run ends; by summation by parts
+//             sum_r v_a x_c = v_a(now) U_c(now) + sum over a's run ends of (v_a before - v_a behind) U_c(at that row)
+//           with U_c the running sum of x_c: lanes keep U_c of their own rows, and where column a's run ends only
+//           that column's sums take U_c times the step of v_a (the lanes fold their twelve U_c eight to one first,
+//           so that the sums are two registers per run-length column, kept in accumulation registers); no sum over
+//           the wave's lanes before the end of its range;
+//   R x R   likewise with the row count in place of U_c.
 // No value of a run-length column is ever looked up per row, and no one-code-per-row copy of it is read.
 //
 // The streams reach the wave through a ring of three chunks of 128 rows in LDS, filled by global -> LDS loads
@@ -32,12 +34,10 @@ constexpr int GDR_THREADS = 256;
 constexpr int GDR_WAVES = GDR_THREADS / 64;
 constexpr int GDR_VMAX = 12;                 // varying columns
 constexpr int GDR_NP = 16 + RC_MAX;          // block tile: index < 16 varying column, 16 + a run-length column a
-constexpr int GDR_RED = 65;                  // doubles per column in the lane transposition (odd: few bank conflicts on the way back)
-constexpr int GDR_REDC = 6;                  // columns per pass of the transposition
-constexpr int GDR_SV = GDR_VMAX + RC_MAX;    // entries of a segment's vector: T of the varying columns, then value x rows of the run-length columns
-constexpr int GDR_WDOUBLES = 64 + 32 + GDR_REDC * GDR_RED + 24 + RC_MAX; // per wave: window values, window ends, transposition, segment vector, run-length values
+constexpr int GDR_WDOUBLES = 64 + 32 + RC_MAX * RC_MAX; // per wave: window values, window ends, the R x R sums
 constexpr int GDR_CH = 128;                  // rows per chunk of the wave's stream ring (2 slices of 64 rows)
 constexpr int GDR_NBUF = 4;                  // ring buffers per wave: one being read, three in flight
+constexpr int GDR_REBASE = 128;             // chunks between two rebases of the run-length columns' running sums (a power of two)
 constexpr int GDR_NI = 8;                    // at most this many 1 KB pieces per chunk and wave (8 KB per ring buffer)
 
 struct GdrCol {            // 24 bytes
@@ -128,9 +128,7 @@ __global__ __launch_bounds__(GDR_THREADS) void k_tsmm_direct(const GdrArgs A) {
 	double* const wbase = gramS + GDR_NP * GDR_NP + wave * GDR_WDOUBLES;
 	double* const winVal = wbase;
 	int32_t* const winEnd = (int32_t*) (wbase + 64);
-	double* const red = wbase + 96;
-	double* const svS = red + GDR_REDC * GDR_RED;   // GDR_SV (24 reserved): the closing segment's vector
-	double* const vvS = svS + 24;                   // RC_MAX: the run-length columns' values on the closing segment
+	double* const rrS = wbase + 96;                 // RC_MAX x RC_MAX: cell (a, b) = the steps of v_a v_b at a's run ends, written by cursor lane b
 	// the wave's ring: GDR_NBUF buffers of ringBytes behind everything else
 	const uint32_t ringBytes = (uint32_t) A.ringBytes;
 	const uint32_t ring0 = (uint32_t) ((A.valDoubles + GDR_NP * GDR_NP + GDR_WAVES * GDR_WDOUBLES) * 8) + (uint32_t) wave * GDR_NBUF * ringBytes;
@@ -142,7 +140,6 @@ __global__ __launch_bounds__(GDR_THREADS) void k_tsmm_direct(const GdrArgs A) {
 		for(int t = tid; t < D.fill; t += GDR_THREADS) smem[D.off + t] = D.add + (t < D.n ? src[(size_t) t * D.nC + D.h] : 0.0);
 	}
 	for(int i = tid; i < GDR_NP * GDR_NP; i += GDR_THREADS) gramS[i] = 0.0;
-	if(lane < 24 + RC_MAX) svS[lane] = 0.0; // (entries of columns the block does not have stay zero)
 	__syncthreads();
 
 	const int32_t nRows = (int32_t) A.nRows;
@@ -225,16 +222,44 @@ __global__ __launch_bounds__(GDR_THREADS) void k_tsmm_direct(const GdrArgs A) {
 
 		RunCursors rc;
 		rc.start(A.runs, nR, winEnd, winVal, ch0 * GDR_CH, lane);
-		int32_t segStart = ch0 * GDR_CH;
 		int32_t eNext = HASR ? rc.next_end() : RC_NEVER;
 
-		// Where a run ends: T of all lanes summed per column, through LDS, GDR_REDC columns per pass: the eight lanes of
-		// group g = lane / 8 (groups 0, 1, 3 .. 6; group 2 is the cursor lanes) sum eight lanes' values each and meet
-		// through three moves inside their half row. The sums go to LDS as the segment's vector s next to the
-		// run-length columns' values v; then lane (a, cs) adds v_a s_c for its columns c = cs, cs + 8, cs + 16 into
-		// registers. T restarts.
-		double G[3] = {0.0, 0.0, 0.0};
-		auto dpp_f64 = [](double v, auto ctrlTag) {
+		// Run-length columns by summation by parts. With U_c(l) the sum of x_c over lane l's rows since the last rebase
+		// and v_a constant between two run ends,  sum_rows v_a x_c = v_a(now) U_c(now) + sum over a's run ends of
+		// (v_a before - v_a behind) U_c(at the end):  where column a's run ends the lanes add U_c times the step of v_a
+		// into sums H[a][c] of their own, which are summed over the lanes once, at the end of the wave's range. R x R likewise with the row count in place of U_c (products v_a v_b, kept by
+		// the cursor lanes in LDS: cell (a, b) holds the steps at a's run ends, written by cursor lane b). A rebase
+		// (every GDR_REBASE chunks and at the end) adds v_a(now) U_c and restarts U and the row count, so that the
+		// terms stay of the size of a few hundred rows' sums.
+		// H is kept folded: where a run ends the lanes of every group of eight fold their twelve U_c into one value per
+		// lane (lane k of the group ends up with the group's sum of column k in fold0 and of column 8 + k % 4 in fold1:
+		// three exchange steps that halve the number of values a lane holds), so H is two values per run-length column
+		// and lane instead of twelve; the groups of eight are summed once, at the end of the wave's range.
+		static_assert(NV <= 12, "two folded registers hold twelve columns");
+		// H is touched where a run ends and nowhere else: it is pinned to accumulation registers (a lone wave per SIMD
+		// has 256 of them next to its vector registers, and this kernel runs no matrix instruction) and moved to a
+		// vector register and back around each multiply-add, so that it never competes with the row loop's sums.
+		int Hr[HASR ? RC_MAX : 1][4]; // H0 low, H0 high, H1 low, H1 high
+#pragma unroll
+		for(int a = 0; a < (HASR ? RC_MAX : 1); a++)
+#pragma unroll
+			for(int k = 0; k < 4; k++) asm volatile("v_accvgpr_write_b32 %0, 0" : "=a"(Hr[a][k]));
+		auto h_get = [&](int lo, int hi) __attribute__((always_inline)) {
+			int p[2];
+			asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(p[0]) : "a"(lo));
+			asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(p[1]) : "a"(hi));
+			double r;
+			__builtin_memcpy(&r, p, 8);
+			return r;
+		};
+		auto h_put = [&](int& lo, int& hi, double v) __attribute__((always_inline)) {
+			int p[2];
+			__builtin_memcpy(p, &v, 8);
+			asm volatile("v_accvgpr_write_b32 %0, %1" : "=a"(lo) : "v"(p[0]));
+			asm volatile("v_accvgpr_write_b32 %0, %1" : "=a"(hi) : "v"(p[1]));
+		};
+		const bool fb0 = (lane & 1) != 0, fb1 = (lane & 2) != 0, fb2 = (lane & 4) != 0;
+		auto dpp_f64 = [](double v, auto ctrlTag) __attribute__((always_inline)) {
 			constexpr int ctrl = decltype(ctrlTag)::value;
 			int p[2];
 			__builtin_memcpy(p, &v, 8);
@@ -244,40 +269,115 @@ __global__ __launch_bounds__(GDR_THREADS) void k_tsmm_direct(const GdrArgs A) {
 			__builtin_memcpy(&r, p, 8);
 			return r;
 		};
-		auto flush = [&](int32_t upTo) {
-			const double nseg = (double) (upTo - segStart);
-			segStart = upTo;
-			const int g = lane >> 3, k8 = lane & 7;
-			const int cp = g < 2 ? g : g - 1; // column of the pass that group g sums (groups 2 and 7: none)
-			const bool vlane = g != 2 && g != 7;
+		auto xchg1 = [&](double v) __attribute__((always_inline)) { return dpp_f64(v, std::integral_constant<int, 0xB1>()); }; // lane ^ 1
+		auto xchg2 = [&](double v) __attribute__((always_inline)) { return dpp_f64(v, std::integral_constant<int, 0x4E>()); }; // lane ^ 2
+		auto xchg4 = [&](double v) __attribute__((always_inline)) { // lane ^ 4: banks 0 and 2 from the bank above, 1 and 3 from the bank below
+			int p[2];
+			__builtin_memcpy(p, &v, 8);
 #pragma unroll
-			for(int p0 = 0; p0 < NV; p0 += GDR_REDC) {
-#pragma unroll
-				for(int c = p0; c < p0 + GDR_REDC && c < NV; c++) red[(c - p0) * GDR_RED + lane] = T[c];
-				wave_lds_sync();
-				// (all eight reads requested before the first sum: one wait instead of one per read)
-				double rv[8];
-#pragma unroll
-				for(int j = 0; j < 8; j++) rv[j] = red[(vlane ? cp : 0) * GDR_RED + k8 * 8 + j];
-				__builtin_amdgcn_sched_barrier(0);
-				double sp = ((rv[0] + rv[1]) + (rv[2] + rv[3])) + ((rv[4] + rv[5]) + (rv[6] + rv[7]));
-				if(!(vlane && p0 + cp < NV)) sp = 0.0;
-				sp += dpp_f64(sp, std::integral_constant<int, 0xB1>());  // quad_perm [1, 0, 3, 2]
-				sp += dpp_f64(sp, std::integral_constant<int, 0x4E>());  // quad_perm [2, 3, 0, 1]
-				sp += dpp_f64(sp, std::integral_constant<int, 0x141>()); // row_half_mirror
-				if(vlane && k8 == 0 && p0 + cp < NV) svS[p0 + cp] = sp;
-				wave_lds_sync();
+			for(int h = 0; h < 2; h++) {
+				int r = __builtin_amdgcn_update_dpp(0, p[h], 0x104, 0xf, 0x5, false); // row_shl:4
+				p[h] = __builtin_amdgcn_update_dpp(r, p[h], 0x114, 0xf, 0xA, false);   // row_shr:4
 			}
-			if(lane >= RC_LANE0 && lane < RC_LANE0 + nR) {
-				svS[GDR_VMAX + lane - RC_LANE0] = rc.val * nseg;
-				vvS[lane - RC_LANE0] = rc.val;
-			}
-			wave_lds_sync();
-			const double va = vvS[k8];
+			double r;
+			__builtin_memcpy(&r, p, 8);
+			return r;
+		};
+		// fold0 / fold1 of T as it stands
+		auto fold = [&](double& f0, double& f1) __attribute__((always_inline)) {
+			double w[4], u[2];
 #pragma unroll
-			for(int t = 0; t < 3; t++)
-				if(g + 8 * t < GDR_SV) G[t] = __builtin_fma(va, svS[g + 8 * t], G[t]);
-			wave_lds_sync();
+			for(int j = 0; j < 4; j++) {
+				const double lo = 2 * j < NV ? T[2 * j < NV ? 2 * j : 0] : 0.0, hi = 2 * j + 1 < NV ? T[2 * j + 1 < NV ? 2 * j + 1 : 0] : 0.0;
+				w[j] = (fb0 ? hi : lo) + xchg1(fb0 ? lo : hi);
+			}
+#pragma unroll
+			for(int i = 0; i < 2; i++) u[i] = (fb1 ? w[2 * i + 1] : w[2 * i]) + xchg2(fb1 ? w[2 * i] : w[2 * i + 1]);
+			f0 = (fb2 ? u[1] : u[0]) + xchg4(fb2 ? u[0] : u[1]);
+			f1 = 0.0;
+			if(NV > 8) {
+				double w1[2];
+#pragma unroll
+				for(int j = 0; j < 2; j++) {
+					const double lo = 8 + 2 * j < NV ? T[8 + 2 * j < NV ? 8 + 2 * j : 0] : 0.0, hi = 9 + 2 * j < NV ? T[9 + 2 * j < NV ? 9 + 2 * j : 0] : 0.0;
+					w1[j] = (fb0 ? hi : lo) + xchg1(fb0 ? lo : hi);
+				}
+				const double u1 = (fb1 ? w1[1] : w1[0]) + xchg2(fb1 ? w1[0] : w1[1]);
+				const double t1 = u1 + xchg4(u1); // (lanes k and k ^ 4 hold the same column: one of them keeps it)
+				f1 = fb2 ? 0.0 : t1;
+			}
+		};
+		rrS[lane] = 0.0;
+		wave_lds_sync();
+		int32_t base = ch0 * GDR_CH;
+		auto bcast_f64 = [](double v, int src) {
+			int p[2];
+			__builtin_memcpy(p, &v, 8);
+			p[0] = __builtin_amdgcn_readlane(p[0], src);
+			p[1] = __builtin_amdgcn_readlane(p[1], src);
+			double r;
+			__builtin_memcpy(&r, p, 8);
+			return r;
+		};
+		auto add_h = [&](auto aTag, double f0, double f1, double f) __attribute__((always_inline)) {
+			constexpr int a = decltype(aTag)::value;
+			if(a < (HASR ? RC_MAX : 1)) {
+				h_put(Hr[a][0], Hr[a][1], __builtin_fma(f0, f, h_get(Hr[a][0], Hr[a][1])));
+				if(NV > 8) h_put(Hr[a][2], Hr[a][3], __builtin_fma(f1, f, h_get(Hr[a][2], Hr[a][3])));
+			}
+		};
+		// the runs that end at row e (T holds the rows in front of e): their columns move on, H and the R x R cells take the steps
+		auto event = [&](int32_t e) __attribute__((always_inline)) {
+			const double vOldL = rc.val;
+			const unsigned long long mine = __ballot(rc.end == e); // (cursor lanes only)
+			rc.advance(e, lane);
+			const double vNewL = rc.val;
+			const double dvl = vOldL - vNewL, svl = vOldL + vNewL;
+			const double nrel = (double) (e - base);
+			const int bL = lane - RC_LANE0;
+			const bool mineL = ((mine >> lane) & 1ull) != 0;
+			unsigned mm = (unsigned) (mine >> RC_LANE0) & ((1u << RC_MAX) - 1u);
+			double f0, f1;
+			fold(f0, f1);
+			while(mm != 0) {
+				const int a = __builtin_ctz(mm);
+				mm &= mm - 1;
+				const double dv = bcast_f64(dvl, RC_LANE0 + a);
+				switch(a) {
+					case 0: add_h(std::integral_constant<int, 0>(), f0, f1, dv); break;
+					case 1: add_h(std::integral_constant<int, 1>(), f0, f1, dv); break;
+					case 2: add_h(std::integral_constant<int, 2>(), f0, f1, dv); break;
+					case 3: add_h(std::integral_constant<int, 3>(), f0, f1, dv); break;
+					case 4: add_h(std::integral_constant<int, 4>(), f0, f1, dv); break;
+					case 5: add_h(std::integral_constant<int, 5>(), f0, f1, dv); break;
+					case 6: add_h(std::integral_constant<int, 6>(), f0, f1, dv); break;
+					default: add_h(std::integral_constant<int, 7>(), f0, f1, dv); break;
+				}
+				// v_a v_b steps by (v_a - v_a') v_b, with v_b already moved on where b < a ends here too; b = a: v_a^2 - v_a'^2
+				if(bL >= 0 && bL < nR) {
+					const double f = bL == a ? svl : (mineL && bL < a ? vNewL : vOldL);
+					rrS[a * RC_MAX + bL] += nrel * dv * f;
+				}
+			}
+		};
+		auto rebase = [&](int32_t upTo) __attribute__((always_inline)) {
+			const double nrel = (double) (upTo - base);
+			base = upTo;
+			const int bL = lane - RC_LANE0;
+			double f0, f1;
+			fold(f0, f1);
+			auto one = [&](auto aTag) __attribute__((always_inline)) {
+				constexpr int a = decltype(aTag)::value;
+				if(a < nR) { // (uniform)
+					const double va = rc.value(a);
+					add_h(aTag, f0, f1, va);
+					if(bL >= a && bL < nR) rrS[a * RC_MAX + bL] += nrel * va * rc.val; // (every pair a <= b once)
+				}
+			};
+			one(std::integral_constant<int, 0>()); one(std::integral_constant<int, 1>());
+			one(std::integral_constant<int, 2>()); one(std::integral_constant<int, 3>());
+			one(std::integral_constant<int, 4>()); one(std::integral_constant<int, 5>());
+			one(std::integral_constant<int, 6>()); one(std::integral_constant<int, 7>());
 #pragma unroll
 			for(int c = 0; c < NV; c++) T[c] = 0.0;
 		};
@@ -300,7 +400,7 @@ __global__ __launch_bounds__(GDR_THREADS) void k_tsmm_direct(const GdrArgs A) {
 		};
 
 		// one slice: s0 its first row, kTag its place in the chunk, guard: rows behind the end of the matrix count as zeros
-		auto slice = [&](auto kTag, int32_t s0, uint32_t boff, bool guard) {
+		auto slice = [&](auto kTag, int32_t s0, uint32_t boff, bool guard) __attribute__((always_inline)) {
 			constexpr int k = decltype(kTag)::value;
 			const int32_t row = s0 + lane;
 			__builtin_amdgcn_sched_barrier(0); // (slices one after the other: interleaved, their values do not fit the registers next to the sums)
@@ -326,7 +426,7 @@ __global__ __launch_bounds__(GDR_THREADS) void k_tsmm_direct(const GdrArgs A) {
 #pragma unroll
 				for(int j = i; j < NV; j++, t++) acc[t] = __builtin_fma(x[i], x[j], acc[t]);
 			if(!HASR) {}
-			else if(eNext >= s0 + 64) {
+			else if(__builtin_expect(eNext >= s0 + 64, 1)) {
 #pragma unroll
 				for(int c = 0; c < NV; c++) T[c] += x[c];
 			}
@@ -337,9 +437,8 @@ __global__ __launch_bounds__(GDR_THREADS) void k_tsmm_direct(const GdrArgs A) {
 					const bool m = row >= from && row < eNext;
 #pragma unroll
 					for(int c = 0; c < NV; c++) T[c] += m ? x[c] : 0.0;
-					flush(eNext);
+					event(eNext);
 					from = eNext;
-					rc.advance(eNext, lane);
 					eNext = rc.next_end();
 				}
 				const bool m = row >= from;
@@ -370,6 +469,7 @@ __global__ __launch_bounds__(GDR_THREADS) void k_tsmm_direct(const GdrArgs A) {
 			codes(std::integral_constant<int, 0>(), boff);
 			slice(std::integral_constant<int, 0>(), c0, boff, false);
 			slice(std::integral_constant<int, 1>(), c0 + 64, boff, false);
+			if(HASR && __builtin_expect(((ch - ch0) & (GDR_REBASE - 1)) == GDR_REBASE - 1, 0)) rebase(c0 + GDR_CH);
 			buf = buf + 1 == GDR_NBUF ? 0 : buf + 1;
 		}
 		if(chFull < ch1) { // the last, partly filled chunk of the matrix
@@ -380,7 +480,7 @@ __global__ __launch_bounds__(GDR_THREADS) void k_tsmm_direct(const GdrArgs A) {
 			slice(std::integral_constant<int, 0>(), c0, boff, true);
 			if(c0 + 64 < nRows) slice(std::integral_constant<int, 1>(), c0 + 64, boff, true);
 		}
-		if(HASR) flush(min(ch1 * GDR_CH, nRows));
+		if(HASR) rebase(min(ch1 * GDR_CH, nRows));
 
 		// the wave's sums into the block's tile
 		{
@@ -393,14 +493,21 @@ __global__ __launch_bounds__(GDR_THREADS) void k_tsmm_direct(const GdrArgs A) {
 					if(lane == 0 && s != 0.0) unsafeAtomicAdd(&gramS[i * GDR_NP + j], s);
 				}
 			if(HASR) {
-				// lane (a, cs): v_a s_c summed over the segments for c = cs, cs + 8, cs + 16 (c < GDR_VMAX: varying column c)
-				const int a = lane & 7, cs = lane >> 3;
+				// lane k of every group of eight: its group's share of column k (and of column 8 + k % 4 where k < 4)
 #pragma unroll
-				for(int tt = 0; tt < 3; tt++) {
-					const int c = cs + 8 * tt;
-					if(a >= nR || c >= GDR_SV) continue;
-					if(c < GDR_VMAX) { if(c < NV) unsafeAtomicAdd(&gramS[c * GDR_NP + 16 + a], G[tt]); }
-					else if(c - GDR_VMAX >= a && c - GDR_VMAX < nR) unsafeAtomicAdd(&gramS[(16 + a) * GDR_NP + 16 + c - GDR_VMAX], G[tt]);
+				for(int a = 0; a < RC_MAX; a++) {
+					if(a >= nR) continue; // (uniform)
+					const int c0 = lane & 7, c1 = 8 + (lane & 3);
+					const double h0 = h_get(Hr[a][0], Hr[a][1]), h1 = h_get(Hr[a][2], Hr[a][3]);
+					if(c0 < NV && h0 != 0.0) unsafeAtomicAdd(&gramS[c0 * GDR_NP + 16 + a], h0);
+					if((lane & 4) == 0 && c1 < NV && h1 != 0.0) unsafeAtomicAdd(&gramS[c1 * GDR_NP + 16 + a], h1);
+				}
+				// lane 8 a + b2: cell (a, b2) of the upper triangle = the steps at a's run ends + those at b2's
+				wave_lds_sync();
+				const int a = lane >> 3, b2 = lane & 7;
+				if(a <= b2 && b2 < nR) {
+					const double sr = a == b2 ? rrS[a * RC_MAX + a] : rrS[a * RC_MAX + b2] + rrS[b2 * RC_MAX + a];
+					if(sr != 0.0) unsafeAtomicAdd(&gramS[(16 + a) * GDR_NP + 16 + b2], sr);
 				}
 			}
 		}
