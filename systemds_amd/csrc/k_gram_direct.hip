@@ -25,6 +25,7 @@
 #include "../../include/cla_hip.h"
 #include "cla_runs.hpp"
 #include <algorithm>
+#include <cmath>
 #include <cstring>
 #include <vector>
 
@@ -455,7 +456,11 @@ __global__ __launch_bounds__(GDR_THREADS) void k_tsmm_direct(const GdrArgs A) {
 		for(int d = 1; d < GDR_NBUF - 1; d++) inF[d - 1] = ch0 + d < ch1 ? dma(ch0 + d, d) : 0;
 		int buf = 0;
 		const int chFull = min(ch1, nRows / GDR_CH); // (only the matrix's last chunk can be partly filled: a loop of its own keeps this one free of branches)
-		for(int ch = ch0; ch < chFull; ch++) {
+		// (the rebase sits between two runs of the chunk loop, not inside it: code at the loop's own depth, however rarely
+		// taken, costs the loop registers)
+		for(int chB = ch0; chB < chFull; chB += GDR_REBASE) {
+		const int chE = min(chB + GDR_REBASE, chFull);
+		for(int ch = chB; ch < chE; ch++) {
 			const uint32_t boff = (uint32_t) buf * ringBytes;
 			const int32_t c0 = ch * GDR_CH;
 			int keep = 0;
@@ -469,8 +474,9 @@ __global__ __launch_bounds__(GDR_THREADS) void k_tsmm_direct(const GdrArgs A) {
 			codes(std::integral_constant<int, 0>(), boff);
 			slice(std::integral_constant<int, 0>(), c0, boff, false);
 			slice(std::integral_constant<int, 1>(), c0 + 64, boff, false);
-			if(HASR && __builtin_expect(((ch - ch0) & (GDR_REBASE - 1)) == GDR_REBASE - 1, 0)) rebase(c0 + GDR_CH);
 			buf = buf + 1 == GDR_NBUF ? 0 : buf + 1;
+		}
+		if(HASR) rebase(chE * GDR_CH);
 		}
 		if(chFull < ch1) { // the last, partly filled chunk of the matrix
 			const uint32_t boff = (uint32_t) buf * ringBytes;
@@ -588,6 +594,12 @@ static int gdr_build_plan(cla_block* b, GdrPlan& P) {
 	}
 	// (columns that no group holds row data for are constants: the tile kernel and the pair kernels serve them)
 	if(covered != b->nCols) return 0;
+	// Summation by parts multiplies sums of earlier rows by the step of a run-length value: with an infinite or NaN value
+	// among the dictionaries that is no longer the product of the rows' own cells (0 x inf where every row's product is
+	// finite). Such blocks take the tile kernel, which forms every row's cells.
+	bool nonFinite = b->dictNonFinite;
+	for(const RunCol& R : runs) nonFinite |= !std::isfinite(R.add);
+	if(nonFinite && !runs.empty()) return 0;
 	std::vector<GdrCol> all;
 	std::vector<GdrStream> streams;
 	int pieces = 0;

@@ -127,6 +127,33 @@ def test_blocks_outside_the_kernels_shape(cla, ora):
     assert_fp64_close(a, b, ora.abs_matmul(D.T, D), what="direct vs tiles")
 
 
+def test_non_finite_run_length_values_take_the_tile_kernel(cla, ora):
+    """The run-following kernel handles run-length columns by summation by parts (sums of earlier rows times the step
+    of a run-length value), which is the rows' own products only for finite values: a block with an infinite or NaN
+    dictionary value next to run-length columns takes the tile kernel, whose cells are the per-row products
+    (infinite and NaN cells where the decompressed product has them)."""
+    n_rows = 20011
+    specs, n_cols = stream_block(31, n_rows)
+    rle = next(s for s in specs if s.type == "rle")
+    rle.dict[1, 0] = np.inf
+    blk = cla.build_block(n_rows, n_cols, specs)
+    out, nnz = blk.tsmm()
+    names = {k["name"] for k in blk.stats()["kernels"]}
+    blk.close()
+    assert "k_tsmm_direct" not in names and "k_tsmm_decode" in names, names
+    D = ora.np_decompress(specs, n_rows, n_cols)
+    with np.errstate(invalid="ignore", over="ignore"):
+        truth = D.T @ D
+    fin = np.isfinite(truth)
+    assert np.array_equal(np.isnan(out), np.isnan(truth))
+    assert np.array_equal(np.isinf(out), np.isinf(truth)) and np.array_equal(out[np.isinf(truth)], truth[np.isinf(truth)])
+    scale = ora.abs_matmul(np.where(np.isfinite(D), D, 0.0).T, np.where(np.isfinite(D), D, 0.0))
+    with np.errstate(invalid="ignore"):
+        err = np.abs(out - truth)
+    assert np.all(err[fin] <= 1e-12 * scale[fin] + 1e-300)
+    assert nnz == np.count_nonzero(out)
+
+
 def test_long_runs_keep_no_expanded_copy(cla):
     """A run-length group whose runs are long gets no one-code-per-row copy: the block's derived bytes stay far below
     one byte per row and group."""
