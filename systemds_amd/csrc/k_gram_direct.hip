@@ -129,7 +129,7 @@ __global__ __launch_bounds__(GDR_THREADS) void k_tsmm_direct(const GdrArgs A) {
 	double* const wbase = gramS + GDR_NP * GDR_NP + wave * GDR_WDOUBLES;
 	double* const winVal = wbase;
 	int32_t* const winEnd = (int32_t*) (wbase + 64);
-	double* const rrS = wbase + 96;                 // RC_MAX x RC_MAX: cell (a, b) = the steps of v_a v_b at a's run ends, written by cursor lane b
+	double* const rrS = wbase + 96;                 // RC_MAX x RC_MAX: where the cursor lanes put their R x R sums at the end (cell (a, b) by cursor lane b)
 	// the wave's ring: GDR_NBUF buffers of ringBytes behind everything else
 	const uint32_t ringBytes = (uint32_t) A.ringBytes;
 	const uint32_t ring0 = (uint32_t) ((A.valDoubles + GDR_NP * GDR_NP + GDR_WAVES * GDR_WDOUBLES) * 8) + (uint32_t) wave * GDR_NBUF * ringBytes;
@@ -228,8 +228,9 @@ __global__ __launch_bounds__(GDR_THREADS) void k_tsmm_direct(const GdrArgs A) {
 		// Run-length columns by summation by parts. With U_c(l) the sum of x_c over lane l's rows since the last rebase
 		// and v_a constant between two run ends,  sum_rows v_a x_c = v_a(now) U_c(now) + sum over a's run ends of
 		// (v_a before - v_a behind) U_c(at the end):  where column a's run ends the lanes add U_c times the step of v_a
-		// into sums H[a][c] of their own, which are summed over the lanes once, at the end of the wave's range. R x R likewise with the row count in place of U_c (products v_a v_b, kept by
-		// the cursor lanes in LDS: cell (a, b) holds the steps at a's run ends, written by cursor lane b). A rebase
+		// into sums H[a][c] of their own, which are summed over the lanes once, at the end of the wave's range. R x R
+		// likewise with the row count in place of U_c (products v_a v_b: cursor lane b keeps cell (a, b), the steps at
+		// a's run ends). A rebase
 		// (every GDR_REBASE chunks and at the end) adds v_a(now) U_c and restarts U and the row count, so that the
 		// terms stay of the size of a few hundred rows' sums.
 		// H is kept folded: where a run ends the lanes of every group of eight fold their twelve U_c into one value per
@@ -240,11 +241,11 @@ __global__ __launch_bounds__(GDR_THREADS) void k_tsmm_direct(const GdrArgs A) {
 		// H is touched where a run ends and nowhere else: it is pinned to accumulation registers (a lone wave per SIMD
 		// has 256 of them next to its vector registers, and this kernel runs no matrix instruction) and moved to a
 		// vector register and back around each multiply-add, so that it never competes with the row loop's sums.
-		int Hr[HASR ? RC_MAX : 1][4]; // H0 low, H0 high, H1 low, H1 high
+		int Hr[HASR ? RC_MAX : 1][6]; // H0 low, H0 high, H1 low, H1 high; cursor lane b: the R x R cell (a, b) low, high
 #pragma unroll
 		for(int a = 0; a < (HASR ? RC_MAX : 1); a++)
 #pragma unroll
-			for(int k = 0; k < 4; k++) asm volatile("v_accvgpr_write_b32 %0, 0" : "=a"(Hr[a][k]));
+			for(int k = 0; k < 6; k++) asm volatile("v_accvgpr_write_b32 %0, 0" : "=a"(Hr[a][k]));
 		auto h_get = [&](int lo, int hi) __attribute__((always_inline)) {
 			int p[2];
 			asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(p[0]) : "a"(lo));
@@ -284,12 +285,12 @@ __global__ __launch_bounds__(GDR_THREADS) void k_tsmm_direct(const GdrArgs A) {
 			__builtin_memcpy(&r, p, 8);
 			return r;
 		};
-		// fold0 / fold1 of T as it stands
-		auto fold = [&](double& f0, double& f1) __attribute__((always_inline)) {
+		// fold0 / fold1 of the running sums el(c), c < NV
+		auto fold = [&](double& f0, double& f1, auto el) __attribute__((always_inline)) {
 			double w[4], u[2];
 #pragma unroll
 			for(int j = 0; j < 4; j++) {
-				const double lo = 2 * j < NV ? T[2 * j < NV ? 2 * j : 0] : 0.0, hi = 2 * j + 1 < NV ? T[2 * j + 1 < NV ? 2 * j + 1 : 0] : 0.0;
+				const double lo = 2 * j < NV ? el(2 * j < NV ? 2 * j : 0) : 0.0, hi = 2 * j + 1 < NV ? el(2 * j + 1 < NV ? 2 * j + 1 : 0) : 0.0;
 				w[j] = (fb0 ? hi : lo) + xchg1(fb0 ? lo : hi);
 			}
 #pragma unroll
@@ -300,7 +301,7 @@ __global__ __launch_bounds__(GDR_THREADS) void k_tsmm_direct(const GdrArgs A) {
 				double w1[2];
 #pragma unroll
 				for(int j = 0; j < 2; j++) {
-					const double lo = 8 + 2 * j < NV ? T[8 + 2 * j < NV ? 8 + 2 * j : 0] : 0.0, hi = 9 + 2 * j < NV ? T[9 + 2 * j < NV ? 9 + 2 * j : 0] : 0.0;
+					const double lo = 8 + 2 * j < NV ? el(8 + 2 * j < NV ? 8 + 2 * j : 0) : 0.0, hi = 9 + 2 * j < NV ? el(9 + 2 * j < NV ? 9 + 2 * j : 0) : 0.0;
 					w1[j] = (fb0 ? hi : lo) + xchg1(fb0 ? lo : hi);
 				}
 				const double u1 = (fb1 ? w1[1] : w1[0]) + xchg2(fb1 ? w1[0] : w1[1]);
@@ -308,8 +309,6 @@ __global__ __launch_bounds__(GDR_THREADS) void k_tsmm_direct(const GdrArgs A) {
 				f1 = fb2 ? 0.0 : t1;
 			}
 		};
-		rrS[lane] = 0.0;
-		wave_lds_sync();
 		int32_t base = ch0 * GDR_CH;
 		auto bcast_f64 = [](double v, int src) {
 			int p[2];
@@ -320,15 +319,17 @@ __global__ __launch_bounds__(GDR_THREADS) void k_tsmm_direct(const GdrArgs A) {
 			__builtin_memcpy(&r, p, 8);
 			return r;
 		};
-		auto add_h = [&](auto aTag, double f0, double f1, double f) __attribute__((always_inline)) {
+		auto add_h = [&](auto aTag, double f0, double f1, double f, double rr) __attribute__((always_inline)) {
 			constexpr int a = decltype(aTag)::value;
 			if(a < (HASR ? RC_MAX : 1)) {
 				h_put(Hr[a][0], Hr[a][1], __builtin_fma(f0, f, h_get(Hr[a][0], Hr[a][1])));
 				if(NV > 8) h_put(Hr[a][2], Hr[a][3], __builtin_fma(f1, f, h_get(Hr[a][2], Hr[a][3])));
+				h_put(Hr[a][4], Hr[a][5], h_get(Hr[a][4], Hr[a][5]) + rr);
 			}
 		};
-		// the runs that end at row e (T holds the rows in front of e): their columns move on, H and the R x R cells take the steps
-		auto event = [&](int32_t e) __attribute__((always_inline)) {
+		// the runs that end at row e (el(c): the running sums with the rows in front of e): their columns move on, H and the
+		// R x R cells take the steps
+		auto event = [&](int32_t e, auto el) __attribute__((always_inline)) {
 			const double vOldL = rc.val;
 			const unsigned long long mine = __ballot(rc.end == e); // (cursor lanes only)
 			rc.advance(e, lane);
@@ -339,25 +340,23 @@ __global__ __launch_bounds__(GDR_THREADS) void k_tsmm_direct(const GdrArgs A) {
 			const bool mineL = ((mine >> lane) & 1ull) != 0;
 			unsigned mm = (unsigned) (mine >> RC_LANE0) & ((1u << RC_MAX) - 1u);
 			double f0, f1;
-			fold(f0, f1);
+			fold(f0, f1, el);
 			while(mm != 0) {
 				const int a = __builtin_ctz(mm);
 				mm &= mm - 1;
 				const double dv = bcast_f64(dvl, RC_LANE0 + a);
-				switch(a) {
-					case 0: add_h(std::integral_constant<int, 0>(), f0, f1, dv); break;
-					case 1: add_h(std::integral_constant<int, 1>(), f0, f1, dv); break;
-					case 2: add_h(std::integral_constant<int, 2>(), f0, f1, dv); break;
-					case 3: add_h(std::integral_constant<int, 3>(), f0, f1, dv); break;
-					case 4: add_h(std::integral_constant<int, 4>(), f0, f1, dv); break;
-					case 5: add_h(std::integral_constant<int, 5>(), f0, f1, dv); break;
-					case 6: add_h(std::integral_constant<int, 6>(), f0, f1, dv); break;
-					default: add_h(std::integral_constant<int, 7>(), f0, f1, dv); break;
-				}
 				// v_a v_b steps by (v_a - v_a') v_b, with v_b already moved on where b < a ends here too; b = a: v_a^2 - v_a'^2
-				if(bL >= 0 && bL < nR) {
-					const double f = bL == a ? svl : (mineL && bL < a ? vNewL : vOldL);
-					rrS[a * RC_MAX + bL] += nrel * dv * f;
+				const double fr = bL == a ? svl : (mineL && bL < a ? vNewL : vOldL);
+				const double rr = bL >= 0 && bL < nR ? nrel * dv * fr : 0.0;
+				switch(a) {
+					case 0: add_h(std::integral_constant<int, 0>(), f0, f1, dv, rr); break;
+					case 1: add_h(std::integral_constant<int, 1>(), f0, f1, dv, rr); break;
+					case 2: add_h(std::integral_constant<int, 2>(), f0, f1, dv, rr); break;
+					case 3: add_h(std::integral_constant<int, 3>(), f0, f1, dv, rr); break;
+					case 4: add_h(std::integral_constant<int, 4>(), f0, f1, dv, rr); break;
+					case 5: add_h(std::integral_constant<int, 5>(), f0, f1, dv, rr); break;
+					case 6: add_h(std::integral_constant<int, 6>(), f0, f1, dv, rr); break;
+					default: add_h(std::integral_constant<int, 7>(), f0, f1, dv, rr); break;
 				}
 			}
 		};
@@ -366,13 +365,12 @@ __global__ __launch_bounds__(GDR_THREADS) void k_tsmm_direct(const GdrArgs A) {
 			base = upTo;
 			const int bL = lane - RC_LANE0;
 			double f0, f1;
-			fold(f0, f1);
+			fold(f0, f1, [&](int c) __attribute__((always_inline)) { return T[c]; });
 			auto one = [&](auto aTag) __attribute__((always_inline)) {
 				constexpr int a = decltype(aTag)::value;
 				if(a < nR) { // (uniform)
 					const double va = rc.value(a);
-					add_h(aTag, f0, f1, va);
-					if(bL >= a && bL < nR) rrS[a * RC_MAX + bL] += nrel * va * rc.val; // (every pair a <= b once)
+					add_h(aTag, f0, f1, va, bL >= a && bL < nR ? nrel * va * rc.val : 0.0); // (every pair a <= b once)
 				}
 			};
 			one(std::integral_constant<int, 0>()); one(std::integral_constant<int, 1>());
@@ -432,19 +430,14 @@ __global__ __launch_bounds__(GDR_THREADS) void k_tsmm_direct(const GdrArgs A) {
 				for(int c = 0; c < NV; c++) T[c] += x[c];
 			}
 			else {
-				// runs end inside the slice: rows in front of each end go to the segment it closes
-				int32_t from = s0;
+				// runs end inside the slice: a run end sees the running sums with the slice's rows in front of it
 				while(eNext < s0 + 64) {
-					const bool m = row >= from && row < eNext;
-#pragma unroll
-					for(int c = 0; c < NV; c++) T[c] += m ? x[c] : 0.0;
-					event(eNext);
-					from = eNext;
+					const bool m = row < eNext;
+					event(eNext, [&](int c) __attribute__((always_inline)) { return T[c] + (m ? x[c] : 0.0); });
 					eNext = rc.next_end();
 				}
-				const bool m = row >= from;
 #pragma unroll
-				for(int c = 0; c < NV; c++) T[c] += m ? x[c] : 0.0;
+				for(int c = 0; c < NV; c++) T[c] += x[c];
 			}
 		};
 
@@ -509,6 +502,14 @@ __global__ __launch_bounds__(GDR_THREADS) void k_tsmm_direct(const GdrArgs A) {
 					if((lane & 4) == 0 && c1 < NV && h1 != 0.0) unsafeAtomicAdd(&gramS[c1 * GDR_NP + 16 + a], h1);
 				}
 				// lane 8 a + b2: cell (a, b2) of the upper triangle = the steps at a's run ends + those at b2's
+				{
+					const int bL = lane - RC_LANE0;
+#pragma unroll
+					for(int a = 0; a < RC_MAX; a++) {
+						const double r = h_get(Hr[a][4], Hr[a][5]);
+						if(bL >= 0 && bL < RC_MAX) rrS[a * RC_MAX + bL] = r;
+					}
+				}
 				wave_lds_sync();
 				const int a = lane >> 3, b2 = lane & 7;
 				if(a <= b2 && b2 < nR) {
